@@ -1,0 +1,137 @@
+"""ctypes binding of libfxhip.so (the C ABI declared in include/fxhip.h).
+
+The library is built in-tree by ``__graft_entry__.build()`` (or ``make`` in
+``functs_amd/csrc/fxhip``).  There is no fallback: if the shared object is
+missing, importing this module raises.
+"""
+import ctypes
+import os
+import re
+
+# torch ships its own HIP runtime; import it first so that libfxhip binds to
+# the same libamdhip64 instance (streams and pointers are shared with torch).
+import torch  # noqa: F401
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfxhip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "fxhip.h")
+
+FX_ARG_MAX_RANK = 8
+
+
+class FxArg(ctypes.Structure):
+    _fields_ = [
+        ("kind", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("ptr", ctypes.c_void_p),
+        ("rank", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("sizes", ctypes.c_int64 * FX_ARG_MAX_RANK),
+        ("strides", ctypes.c_int64 * FX_ARG_MAX_RANK),
+        ("ival", ctypes.c_int64),
+        ("fval", ctypes.c_double),
+    ]
+
+
+def _parse_header():
+    """Opcode / dtype / error constants straight from the C header, so that the
+    Python side can never drift from the ABI."""
+    text = open(HEADER_PATH).read()
+    consts = {}
+    for m in re.finditer(r"#define\s+(FX_[A-Z0-9_]+)\s+\(?(-?\d+)\)?", text):
+        consts[m.group(1)] = int(m.group(2))
+    body = re.search(r"enum fx_opcode \{(.*?)\};", text, re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    val = 0
+    for tok in body.split(","):
+        tok = tok.strip()
+        if not tok:
+            continue
+        if "=" in tok:
+            name, v = [t.strip() for t in tok.split("=")]
+            val = int(v)
+        else:
+            name = tok
+        consts[name] = val
+        val += 1
+    return consts
+
+
+C = _parse_header()
+
+
+def exported_symbols():
+    """Names of every function the header declares."""
+    text = open(HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fx_[a-z0-9_]+)\s*\(", text)))
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libfxhip.so is not built (%s). Run `python -c 'import __graft_entry__ as g; g.build()'` "
+        "or `make -C functs_amd/csrc/fxhip`." % LIB_PATH
+    )
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_ip = ctypes.POINTER(ctypes.c_int)
+
+
+def _sig(name, restype, *argtypes):
+    fn = getattr(lib, name)
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+    return fn
+
+
+_sig("fx_last_error", ctypes.c_char_p)
+_sig("fx_api_version", _i)
+_sig("fx_region_create", _i, _i, _i, ctypes.POINTER(_vp))
+_sig("fx_region_destroy", None, _vp)
+_sig("fx_region_input_tensor", _i, _vp, _i, _i, _i, _ip)
+_sig("fx_region_input_scalar", _i, _vp, _i, _i, _ip)
+_sig("fx_region_task_index", _i, _vp, _ip)
+_sig("fx_region_loop_var", _i, _vp, _ip)
+_sig("fx_region_const_int", _i, _vp, ctypes.c_int64, _ip)
+_sig("fx_region_const_float", _i, _vp, ctypes.c_double, _ip)
+_sig("fx_region_const_bool", _i, _vp, _i, _ip)
+_sig("fx_region_const_none", _i, _vp, _ip)
+_sig("fx_region_int_list", _i, _vp, _ip, _i, _ip)
+_sig("fx_region_tensor_list", _i, _vp, _ip, _i, _ip)
+_sig("fx_region_op", _i, _vp, _i, _ip, _i, _i, _ip)
+_sig("fx_region_output", _i, _vp, _i)
+_sig("fx_region_compact_rows", _i, _vp, _i)
+_sig("fx_region_finalize", _i, _vp)
+_sig("fx_region_plan", _i, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp))
+_sig("fx_plan_num_outputs", _i, _vp)
+_sig("fx_plan_output", _i, _vp, _i, _i, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+     ctypes.POINTER(ctypes.c_int64))
+_sig("fx_plan_scratch_bytes", ctypes.c_size_t, _vp)
+_sig("fx_plan_launches", _i, _vp)
+_sig("fx_plan_algorithmic_bytes", ctypes.c_int64, _vp)
+_sig("fx_plan_blob", _i, _vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)), ctypes.POINTER(ctypes.c_size_t))
+_sig("fx_plan_disasm", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_region_marshal", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,
+     ctypes.c_size_t)
+_sig("fx_dyn_bytes", ctypes.c_size_t)
+_sig("fx_region_run", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp)
+_sig("fx_compact_rows", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+     ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, ctypes.c_size_t, _vp, _vp)
+_sig("fx_compact_rows_scratch_bytes", ctypes.c_size_t, ctypes.c_int64)
+_sig("fx_device_count", _i)
+_sig("fx_copy_bytes", _i, _vp, _vp, ctypes.c_size_t, _vp)
+
+
+class FxError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("fxhip error %d: %s" % (code, msg))
+        self.code = code
+
+
+def check(rc):
+    if rc < 0:
+        raise FxError(rc, lib.fx_last_error().decode())
+    return rc

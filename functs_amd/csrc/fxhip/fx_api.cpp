@@ -1,0 +1,399 @@
+// C ABI of libfxhip (see include/fxhip.h) and the launch-time runtime:
+// argument marshalling into the by-value FxDyn block, one-time upload of the
+// static region blob, kernel launches on the caller's stream.
+//
+// Counterpart of GraphBuilder::prepareRunArgs / runKernel
+// (fait/fuser/graph_builder.cpp:718-927) and CudaCodeGenTssa::call_raw
+// (fait/tensorexpr/cuda_codegen_tssa.cpp:1167-1290).
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "fx_lower.h"
+
+hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+                           hipStream_t stream);
+hipError_t fx_launch_compact_count(const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+                                   hipStream_t stream);
+hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid,
+                                     uint32_t lds_bytes, hipStream_t stream);
+hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream);
+hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                                  const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
+                                  uint32_t* total_host, hipStream_t stream);
+
+struct fx_region {
+  fx::Region r;
+  std::mutex mu;  // plan cache + device upload (the reference serialises extent
+                  // evaluation the same way, cuda_codegen_tssa.cpp:1207)
+};
+struct fx_plan {
+  fx::Plan p;
+};
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+#define FX_TRY try {
+#define FX_CATCH                                                   \
+  }                                                                \
+  catch (const fx::Error& e) { return fail(e.code, e.what()); }    \
+  catch (const std::exception& e) { return fail(FX_E_INVALID, e.what()); }
+
+#define HIP_OK(expr)                                                                                  \
+  do {                                                                                                \
+    hipError_t e__ = (expr);                                                                          \
+    if (e__ != hipSuccess) return fail(FX_E_HIP, std::string(#expr) + ": " + hipGetErrorString(e__)); \
+  } while (0)
+
+int add_value(fx_region* reg, const fx::Value& v, int* id) {
+  if (!reg || !id) return fail(FX_E_INVALID, "null argument");
+  if (reg->r.finalized) return fail(FX_E_INVALID, "region already finalized");
+  *id = reg->r.add(v);
+  return FX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* fx_last_error(void) { return g_err.c_str(); }
+int fx_api_version(void) { return FX_API_VERSION; }
+
+int fx_region_create(int parallel_degree, int is_parallel_map, fx_region** out) {
+  if (!out) return fail(FX_E_INVALID, "null out");
+  if (parallel_degree < 1) return fail(FX_E_INVALID, "parallel_degree must be >= 1");
+  fx_region* r = new fx_region();
+  r->r.degree = parallel_degree;
+  r->r.is_map = is_parallel_map != 0;
+  *out = r;
+  return FX_OK;
+}
+
+void fx_region_destroy(fx_region* r) {
+  if (!r) return;
+  for (auto& kv : r->r.plans)
+    if (kv.second->dev_blob) (void)hipFree(kv.second->dev_blob);
+  delete r;
+}
+
+int fx_region_input_tensor(fx_region* reg, int dtype, int rank, int per_task, int* id) {
+  if (!reg) return fail(FX_E_INVALID, "null region");
+  if (fx::dtype_size(dtype) == 0) return fail(FX_E_UNSUPPORTED, "unsupported tensor dtype");
+  fx::Value v;
+  v.kind = fx::VK_TENSOR;
+  v.prod = fx::P_INPUT;
+  v.dtype = dtype;
+  v.rank = rank;
+  v.per_task = per_task != 0;
+  v.input_index = (int)reg->r.inputs.size();
+  int rc = add_value(reg, v, id);
+  if (rc == FX_OK) reg->r.inputs.push_back(*id);
+  return rc;
+}
+
+int fx_region_input_scalar(fx_region* reg, int kind, int per_task, int* id) {
+  if (!reg) return fail(FX_E_INVALID, "null region");
+  if (kind < 1 || kind > 3) return fail(FX_E_INVALID, "scalar kind must be 1 (int), 2 (float) or 3 (bool)");
+  fx::Value v;
+  v.kind = kind == 1 ? fx::VK_INT : (kind == 2 ? fx::VK_FLOAT : fx::VK_BOOL);
+  v.prod = fx::P_INPUT;
+  v.per_task = per_task != 0;
+  v.input_index = (int)reg->r.inputs.size();
+  int rc = add_value(reg, v, id);
+  if (rc == FX_OK) reg->r.inputs.push_back(*id);
+  return rc;
+}
+
+int fx_region_task_index(fx_region* reg, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_INT;
+  v.prod = fx::P_TASK;
+  return add_value(reg, v, id);
+}
+
+int fx_region_loop_var(fx_region* reg, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_INT;
+  v.prod = fx::P_LOOPVAR;
+  return add_value(reg, v, id);
+}
+
+int fx_region_const_int(fx_region* reg, int64_t x, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_INT;
+  v.ival = x;
+  return add_value(reg, v, id);
+}
+int fx_region_const_float(fx_region* reg, double x, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_FLOAT;
+  v.fval = x;
+  return add_value(reg, v, id);
+}
+int fx_region_const_bool(fx_region* reg, int x, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_BOOL;
+  v.ival = x != 0;
+  return add_value(reg, v, id);
+}
+int fx_region_const_none(fx_region* reg, int* id) {
+  fx::Value v;
+  v.kind = fx::VK_NONE;
+  return add_value(reg, v, id);
+}
+
+static int add_list(fx_region* reg, const int* ids, int n, fx::VKind kind, fx::VKind elem, int* id) {
+  if (!reg || (n > 0 && !ids)) return fail(FX_E_INVALID, "null argument");
+  fx::Value v;
+  v.kind = kind;
+  v.prod = fx::P_LIST;
+  for (int i = 0; i < n; ++i) {
+    if (ids[i] < 0 || ids[i] >= (int)reg->r.vals.size()) return fail(FX_E_INVALID, "bad value id in list");
+    fx::VKind k = reg->r.vals[ids[i]].kind;
+    if (elem == fx::VK_INT ? !(k == fx::VK_INT || k == fx::VK_BOOL) : k != elem)
+      return fail(FX_E_INVALID, "list element of the wrong kind");
+    v.args.push_back(ids[i]);
+  }
+  return add_value(reg, v, id);
+}
+int fx_region_int_list(fx_region* reg, const int* ids, int n, int* id) {
+  return add_list(reg, ids, n, fx::VK_INT_LIST, fx::VK_INT, id);
+}
+int fx_region_tensor_list(fx_region* reg, const int* ids, int n, int* id) {
+  return add_list(reg, ids, n, fx::VK_TENSOR_LIST, fx::VK_TENSOR, id);
+}
+
+int fx_region_op(fx_region* reg, int opcode, const int* arg_ids, int n_args, int out_dtype, int* id) {
+  if (!reg || !id || (n_args > 0 && !arg_ids)) return fail(FX_E_INVALID, "null argument");
+  if (reg->r.finalized) return fail(FX_E_INVALID, "region already finalized");
+  FX_TRY
+  std::vector<int> args(arg_ids, arg_ids + n_args);
+  *id = reg->r.addOp(opcode, args, out_dtype);
+  return FX_OK;
+  FX_CATCH
+}
+
+int fx_region_output(fx_region* reg, int value_id) {
+  if (!reg) return fail(FX_E_INVALID, "null region");
+  if (reg->r.finalized) return fail(FX_E_INVALID, "region already finalized");
+  if (value_id < 0 || value_id >= (int)reg->r.vals.size() || reg->r.vals[value_id].kind != fx::VK_TENSOR)
+    return fail(FX_E_INVALID, "output must be a tensor value");
+  reg->r.outputs.push_back(value_id);
+  return FX_OK;
+}
+
+int fx_region_compact_rows(fx_region* reg, int mask_value_id) {
+  if (!reg) return fail(FX_E_INVALID, "null region");
+  if (reg->r.finalized) return fail(FX_E_INVALID, "region already finalized");
+  if (mask_value_id < 0 || mask_value_id >= (int)reg->r.vals.size() ||
+      reg->r.vals[mask_value_id].kind != fx::VK_TENSOR)
+    return fail(FX_E_INVALID, "mask must be a tensor value");
+  reg->r.mask = mask_value_id;
+  return FX_OK;
+}
+
+int fx_region_finalize(fx_region* reg) {
+  if (!reg) return fail(FX_E_INVALID, "null region");
+  if (reg->r.outputs.empty()) return fail(FX_E_INVALID, "region has no outputs");
+  reg->r.finalized = true;
+  return FX_OK;
+}
+
+int fx_region_plan(fx_region* reg, const fx_arg* args, int n_args, const fx_plan** plan) {
+  if (!reg || !plan || (n_args > 0 && !args)) return fail(FX_E_INVALID, "null argument");
+  FX_TRY
+  std::lock_guard<std::mutex> g(reg->mu);
+  const fx::Plan* p = fx::plan_region(reg->r, args, n_args);
+  *plan = reinterpret_cast<const fx_plan*>(p);
+  return FX_OK;
+  FX_CATCH
+}
+
+static const fx::Plan* P(const fx_plan* p) { return reinterpret_cast<const fx::Plan*>(p); }
+
+int fx_plan_num_outputs(const fx_plan* p) { return p ? (int)P(p)->out_dtype.size() : 0; }
+
+int fx_plan_output(const fx_plan* p, int out_idx, int task, int32_t* dtype, int32_t* rank, int64_t* sizes) {
+  if (!p) return fail(FX_E_INVALID, "null plan");
+  const fx::Plan* pl = P(p);
+  if (out_idx < 0 || out_idx >= (int)pl->out_dtype.size() || task < 0 || task >= pl->region->degree)
+    return fail(FX_E_INVALID, "output/task index out of range");
+  const auto& s = pl->out_shape[out_idx][task];
+  if (dtype) *dtype = pl->out_dtype[out_idx];
+  if (rank) *rank = (int32_t)s.size();
+  if (sizes)
+    for (size_t i = 0; i < s.size(); ++i) sizes[i] = s[i];
+  return FX_OK;
+}
+
+size_t fx_plan_scratch_bytes(const fx_plan* p) { return p ? P(p)->scratch_bytes : 0; }
+int fx_plan_launches(const fx_plan* p) { return p ? P(p)->launches : 0; }
+int64_t fx_plan_algorithmic_bytes(const fx_plan* p) { return p ? P(p)->alg_bytes : 0; }
+
+int fx_plan_blob(const fx_plan* p, const uint32_t** words, size_t* n_words) {
+  if (!p || !words || !n_words) return fail(FX_E_INVALID, "null argument");
+  *words = P(p)->blob.data();
+  *n_words = P(p)->blob.size();
+  return FX_OK;
+}
+
+int fx_plan_disasm(const fx_plan* p, char* buf, size_t cap) {
+  if (!p || !buf || cap == 0) return fail(FX_E_INVALID, "null argument");
+  std::string s = fx::disasm(*P(p));
+  size_t n = std::min(cap - 1, s.size());
+  memcpy(buf, s.data(), n);
+  buf[n] = 0;
+  return (int)s.size();
+}
+
+int fx_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+// Fill the by-value dynamic block.  Exposed (without launching) so that host
+// tests can check the marshalling.
+static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
+                    uint32_t* totals_host, FxDyn* dyn) {
+  const fx::Region& R = *pl->region;
+  const int T = R.degree;
+  auto ptr_of = [&](const fx::PtrSrc& s, int task) -> uint64_t {
+    switch (s.kind) {
+      case fx::PtrSrc::INPUT: {
+        bool per_task = R.vals[R.inputs[s.index]].per_task;
+        return (uint64_t)(uintptr_t)args[pl->arg_base[s.index] + (per_task ? task : 0)].ptr;
+      }
+      case fx::PtrSrc::OUTPUT: return (uint64_t)(uintptr_t)out_ptrs[s.index * T + task];
+      case fx::PtrSrc::FLAGS: return (uint64_t)(uintptr_t)((char*)scratch + pl->flags_off);
+      case fx::PtrSrc::COUNTS: return (uint64_t)(uintptr_t)((char*)scratch + pl->counts_off);
+      case fx::PtrSrc::TOTALS: return (uint64_t)(uintptr_t)totals_host;
+    }
+    return 0;
+  };
+  auto scal_of = [&](const fx::ScalSrc& s, int task) -> uint32_t {
+    const fx::Value& v = R.vals[R.inputs[s.input]];
+    const fx_arg& a = args[pl->arg_base[s.input] + (v.per_task ? task : 0)];
+    double x = v.kind == fx::VK_FLOAT ? a.fval : (double)a.ival;
+    uint32_t u;
+    if (s.as_float) {
+      float f = (float)x;  // double -> float like graph_builder.cpp:850-854
+      memcpy(&u, &f, 4);
+    } else {
+      u = (uint32_t)(int32_t)(int64_t)x;
+    }
+    return u;
+  };
+  size_t np = pl->sptr.size(), ntp = pl->tptr.size(), ns = pl->sscal.size(), nts = pl->tscal.size();
+  for (size_t i = 0; i < np; ++i) dyn->p[i] = ptr_of(pl->sptr[i], 0);
+  for (int t = 0; t < T; ++t)
+    for (size_t i = 0; i < ntp; ++i) dyn->p[np + t * ntp + i] = ptr_of(pl->tptr[i], t);
+  for (size_t i = 0; i < ns; ++i) dyn->s[i] = scal_of(pl->sscal[i], 0);
+  for (int t = 0; t < T; ++t)
+    for (size_t i = 0; i < nts; ++i) dyn->s[ns + t * nts + i] = scal_of(pl->tscal[i], t);
+  return FX_OK;
+}
+
+int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                      void* scratch, uint32_t* totals_host, void* dyn_out, size_t dyn_cap) {
+  if (!reg || !plan || !out_ptrs || !dyn_out) return fail(FX_E_INVALID, "null argument");
+  const fx::Plan* pl = P(plan);
+  if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
+  if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
+  if (dyn_cap < sizeof(FxDyn)) return fail(FX_E_INVALID, "dyn_out too small");
+  memset(dyn_out, 0, sizeof(FxDyn));
+  return fill_dyn(pl, args, out_ptrs, scratch, totals_host, (FxDyn*)dyn_out);
+}
+
+size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
+
+int fx_region_run(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                  void* scratch, uint32_t* totals_host, void* stream_) {
+  if (!reg || !plan || !out_ptrs) return fail(FX_E_INVALID, "null argument");
+  fx::Plan* pl = const_cast<fx::Plan*>(P(plan));
+  if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
+  if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
+  if (pl->mode == FX_MODE_COMPACT && (!scratch || !totals_host))
+    return fail(FX_E_INVALID, "compacting region needs scratch memory and a pinned totals buffer");
+  hipStream_t stream = (hipStream_t)stream_;
+
+  int dev = 0;
+  HIP_OK(hipGetDevice(&dev));
+  {
+    std::lock_guard<std::mutex> g(reg->mu);
+    if (!pl->dev_blob || pl->dev_id != dev) {
+      void* d = nullptr;
+      HIP_OK(hipMalloc(&d, pl->blob.size() * 4));
+      HIP_OK(hipMemcpy(d, pl->blob.data(), pl->blob.size() * 4, hipMemcpyHostToDevice));
+      pl->dev_blob = d;
+      pl->dev_id = dev;
+    }
+  }
+  FxDyn dyn;
+  int rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, &dyn);
+  if (rc != FX_OK) return rc;
+  const uint32_t* sb = (const uint32_t*)pl->dev_blob;
+  if (pl->mode == FX_MODE_COMPACT) {
+    // tasks without rows launch no tile: their total is published here.  The
+    // caller must not reuse totals_host while an earlier run is still in flight.
+    for (int t = 0; t < reg->r.degree; ++t) totals_host[t] = 0;
+  }
+  if (pl->mode == FX_MODE_DENSE) {
+    HIP_OK(fx_launch_dense(pl->max_rank, sb, &dyn, pl->grid, pl->lds_bytes, stream));
+  } else {
+    HIP_OK(fx_launch_compact_count(sb, &dyn, pl->grid_count, pl->lds_bytes, stream));
+    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, &dyn, pl->grid, pl->lds_bytes, stream));
+  }
+  return FX_OK;
+}
+
+size_t fx_compact_rows_scratch_bytes(int64_t n) {
+  if (n < 0) n = 0;
+  return (size_t)(((n + FX_BLOCK - 1) / FX_BLOCK + 1) * 4 + 256);
+}
+
+int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs, const int32_t* rowlen,
+                    const int32_t* elsize, int n_cols, void* scratch, size_t scratch_bytes, uint32_t* total_host,
+                    void* stream_) {
+  if (n < 0 || n_cols < 0 || n_cols > 8) return fail(FX_E_INVALID, "fx_compact_rows: n >= 0 and 0 <= n_cols <= 8");
+  if (n >= ((int64_t)1 << 31)) return fail(FX_E_LIMIT, "fx_compact_rows: n above 2^31");
+  if (!total_host) return fail(FX_E_INVALID, "fx_compact_rows: total_host is required");
+  if (n > 0 && (!mask || !scratch)) return fail(FX_E_INVALID, "fx_compact_rows: null mask/scratch");
+  if (scratch_bytes < fx_compact_rows_scratch_bytes(n)) return fail(FX_E_INVALID, "fx_compact_rows: scratch too small");
+  for (int i = 0; i < n_cols; ++i) {
+    if (!cols || !outs || !rowlen || !elsize) return fail(FX_E_INVALID, "fx_compact_rows: null column arrays");
+    if (elsize[i] != 4 && elsize[i] != 8 && elsize[i] != 1) return fail(FX_E_UNSUPPORTED, "fx_compact_rows: elsize 1, 4 or 8");
+    if (rowlen[i] < 1) return fail(FX_E_INVALID, "fx_compact_rows: rowlen >= 1");
+    if ((int64_t)rowlen[i] * n >= ((int64_t)1 << 31)) return fail(FX_E_LIMIT, "fx_compact_rows: column above 2^31 elements");
+  }
+  if (n == 0) {
+    *total_host = 0;
+    return FX_OK;
+  }
+  HIP_OK(fx_launch_compact_rows(mask, n, cols, outs, rowlen, elsize, n_cols, (uint32_t*)scratch, total_host,
+                                (hipStream_t)stream_));
+  return FX_OK;
+}
+
+int fx_copy_bytes(const void* src, void* dst, size_t bytes, void* stream) {
+  if (bytes % 16) return fail(FX_E_INVALID, "fx_copy_bytes: size must be a multiple of 16");
+  if (bytes == 0) return FX_OK;
+  size_t n4 = bytes / 16;
+  size_t blocks = (n4 + FX_BLOCK - 1) / FX_BLOCK;
+  // 4 vectors per lane keeps enough loads in flight without oversubscribing
+  uint32_t grid = (uint32_t)std::min<size_t>((blocks + 3) / 4, 1u << 20);
+  if (grid == 0) grid = 1;
+  HIP_OK(fx_launch_copy(src, dst, bytes, grid, (hipStream_t)stream));
+  return FX_OK;
+}
+
+}  // extern "C"

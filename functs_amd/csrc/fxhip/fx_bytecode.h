@@ -1,0 +1,180 @@
+// Region bytecode shared by the host lowering (fx_lower.cpp), the gfx950 VM
+// kernels (fx_kernels.hip) and the test-only scalar emulator.
+//
+// A fused functionalized region (the body of a prim::FusionGroup, possibly
+// replicated over the tasks of a prim::ParallelMap) is lowered on the host to
+// one small accumulator-machine program per region output.  The program
+// computes ONE output element from its output coordinates; the kernel runs it
+// for FX_V elements per lane at once so that instruction decode (scalar,
+// wave-uniform) is amortised over 4 x 64 elements per wave.
+//
+// This replaces the CUDA-C text the reference generates per region
+// (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121) and the per-element index
+// arithmetic of its lowerings (functs/csrc/jit/tensorexpr/nnc_ext.cpp:62-392,
+// fait/fuser/custom_lowering_func.cpp:17-498).
+#pragma once
+#include <stdint.h>
+
+#define FX_MAXR 6        // max rank of a region output (root coordinates)
+#define FX_V 4           // elements per lane
+#define FX_BLOCK 256     // threads per workgroup (4 wavefronts of 64)
+#define FX_TILE (FX_V * FX_BLOCK)
+#define FX_MAX_TEMPS 24  // LDS temp slots per lane (each FX_V wide)
+#define FX_MASK_DEPTH 16 // nesting depth of predicated regions (4 bits each in a u64)
+#define FX_DYN_P 320     // 8-byte dynamic words passed by value (pointers)
+#define FX_DYN_S 176     // 4-byte dynamic words passed by value (scalars)
+#define FX_MAX_TPTR 32   // per-task pointers staged in LDS
+#define FX_MAX_TSCAL 32  // per-task scalars staged in LDS
+#define FX_MAGIC 0x46585231u  // "FXR1"
+
+// storage dtypes of buffers
+enum FxDtype : uint32_t {
+  FX_F32 = 0,
+  FX_I64 = 1,
+  FX_I32 = 2,
+  FX_U8 = 3,   // uint8 and bool
+  FX_F16 = 4,
+  FX_BF16 = 5,
+};
+
+// value classes inside the VM (32-bit registers)
+enum FxVt : uint32_t { FX_VT_F = 0, FX_VT_I = 1 };
+
+enum FxOp : uint32_t {
+  FX_NOP = 0,
+  // ---- register moves / loads (writes are predicated by the lane mask) ----
+  FX_LDA,    // A = buf[a] at affine[b](coords); dt = storage dtype
+  FX_LDB,    // B = ...
+  FX_LDXA,   // A = buf[a] at element offset (int)A + imm
+  FX_AFFA,   // A = (int) affine[b](coords)
+  FX_AFFB,
+  FX_IMMA,   // A = imm (raw 32 bits)
+  FX_IMMB,
+  FX_SCLA,   // A = scalar slot a (bit 30 set: per-task table)
+  FX_SCLB,
+  FX_STT,    // temp[a] = A
+  FX_LDTA,   // A = temp[a]
+  FX_LDTB,   // B = temp[a]
+  FX_MOVBA,  // B = A
+  FX_SWAP,   // A <-> B
+  // ---- predication ----
+  FX_MIF,    // push mask; mask &= (A != 0); if no lane of the wave is live jump to a
+  FX_MELSE,  // mask = saved & ~mask; if no lane live jump to a
+  FX_MMERGE, // A = live ? A : temp[a]; pop mask
+  FX_MEND,   // pop mask (both sides wrote A with predicated moves)
+  // ---- unary float (A = f(A)) ----
+  FX_FNEG, FX_FABS, FX_EXP, FX_LOG, FX_SQRT, FX_RSQRT, FX_RCP, FX_SIGMOID,
+  FX_TANH, FX_RELU, FX_FLOOR, FX_CEIL, FX_ROUND, FX_TRUNC, FX_SIN, FX_COS,
+  FX_ERF, FX_LOG2, FX_EXP2, FX_EXPM1, FX_LOG1P,
+  // ---- unary int / conversions ----
+  FX_INEG, FX_LNOT, FX_INZ, FX_FNZ, FX_F2I, FX_I2F, FX_IABS,
+  // ---- binary: A = A op X, X = B or imm (flags & FX_F_IMM) ----
+  FX_FADD, FX_FSUB, FX_FRSUB, FX_FMUL, FX_FDIV, FX_FRDIV, FX_FMIN, FX_FMAX,
+  FX_FPOW, FX_FMOD, FX_ATAN2,
+  FX_IADD, FX_ISUB, FX_IRSUB, FX_IMUL, FX_IFDIV, FX_ITDIV, FX_IPMOD, FX_ITMOD,
+  FX_IMIN, FX_IMAX, FX_IAND, FX_IOR, FX_IXOR,
+  FX_FLT, FX_FLE, FX_FGT, FX_FGE, FX_FEQ, FX_FNE,
+  FX_ILT, FX_ILE, FX_IGT, FX_IGE, FX_IEQ, FX_INE,
+  // ---- misc ----
+  FX_IRANGE, // A = (A >= a && A < b && (A - a) % imm == 0)
+  FX_WHERE,  // A = temp[a] != 0 ? A : B
+  // ---- serial reduction over an extra coordinate ----
+  FX_RBEGIN, // push loop: counter = 0, extent = imm, acc slot = temp[a] preset by program
+  FX_RNEXT,  // counter += 1; if counter < extent jump to a
+  FX_RIDX,   // A = (int) loop counter of depth a
+  FX_OP_COUNT
+};
+
+#define FX_F_IMM 1u  // binary op takes its second operand from imm
+#define FX_F_I2F 2u  // LDA/LDB/AFFA/AFFB/SCLA/SCLB: convert the int result to float
+
+struct FxInsn {
+  uint16_t op;
+  uint8_t flags;
+  uint8_t dt;
+  int32_t a;
+  int32_t b;
+  uint32_t imm;
+};
+
+// element offset = base + tcoef * task + sum_k coef[k] * coord[k] + sum_d rcoef[d] * loop_counter[d]
+#define FX_MAXLOOP 2
+struct FxAffine {
+  int32_t coef[FX_MAXR];
+  int32_t tcoef;
+  int32_t base;
+  int32_t rcoef[FX_MAXLOOP];
+  int32_t pad[6];
+};
+
+#define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table
+
+struct FxOut {
+  uint32_t prog_begin, prog_end;  // instruction range, relative to the class base
+  uint32_t rank;
+  uint32_t numel;                 // dense: elements per task. compaction: rowlen * n_rows
+  uint32_t dim[FX_MAXR];
+  uint32_t magic[FX_MAXR];        // fast division by dim[k]
+  uint32_t shift[FX_MAXR];
+  uint32_t dtype;
+  uint32_t ptr_slot;              // may carry FX_SLOT_TASK
+  uint32_t task_stride;           // element offset added per task (shared output buffer)
+  uint32_t block_begin;           // first block of this output inside one task
+  uint32_t n_blocks;
+  uint32_t rowlen;                // compaction: elements per row (numel / dim[0])
+  uint32_t rl_magic, rl_shift;    // fast division by rowlen
+  uint32_t vt;                    // FxVt of the program result
+  uint32_t pad[3];
+};
+
+struct FxClass {
+  uint32_t block_begin, block_end;  // grid range covered by this class (dense / scatter pass)
+  uint32_t first_task;              // index into the task map
+  uint32_t n_tasks;
+  uint32_t blocks_per_task;
+  uint32_t n_outs;
+  uint32_t off_outs;                // word offset of FxOut[n_outs]
+  uint32_t off_insn;                // word offset of FxInsn[]
+  uint32_t off_aff;                 // word offset of FxAffine[]
+  uint32_t n_temps;
+  // row compaction (mode 1)
+  uint32_t mask_begin, mask_end;    // mask program
+  uint32_t n_rows;
+  uint32_t n_rowtiles;              // ceil(n_rows / row_tile)
+  uint32_t mask_vt;
+  uint32_t cnt_block_begin, cnt_block_end;  // grid range in the count pass
+  uint32_t cnt_blocks_per_task;
+  uint32_t pad[2];
+};
+
+enum FxMode : uint32_t { FX_MODE_DENSE = 0, FX_MODE_COMPACT = 1 };
+
+struct FxHeader {
+  uint32_t magic;
+  uint32_t mode;
+  uint32_t n_classes;
+  uint32_t n_tasks;
+  uint32_t n_sptr, n_tptr, n_sscal, n_tscal;
+  uint32_t off_class;    // word offset of FxClass[n_classes]
+  uint32_t off_taskmap;  // word offset of uint32 task ids grouped by class
+  uint32_t row_tile;     // rows per compaction tile (<= FX_BLOCK)
+  uint32_t max_rowtiles; // stride of the per-task tile-count table
+  uint32_t slot_flags, slot_counts, slot_total;  // shared pointer slots used by compaction
+  uint32_t total_words;
+};
+
+// dynamic (per call) arguments, passed by value in the kernarg segment
+struct FxDyn {
+  uint64_t p[FX_DYN_P];  // [shared ptrs][task 0 ptrs][task 1 ptrs]...
+  uint32_t s[FX_DYN_S];  // [shared scalars][task 0 scalars]...
+};
+
+// fast unsigned division n / d for n < 2^31: q = (umulhi(n, magic) + n) >> shift
+static inline void fx_fastdiv_make(uint32_t d, uint32_t* magic, uint32_t* shift) {
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  uint64_t one = 1;
+  uint64_t m = ((one << 32) * ((one << s) - d)) / d + 1;
+  *magic = (uint32_t)m;
+  *shift = s;
+}

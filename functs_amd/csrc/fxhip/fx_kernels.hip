@@ -1,0 +1,923 @@
+// gfx950 kernels of the fused-region backend.
+//
+//   fx_region_dense   : one launch evaluates every output of a fused
+//                       functionalized region for every ParallelMap task.
+//   fx_compact_count  : pass 1 of row compaction (mask program -> row flags +
+//                       per-tile keep counts, wave ballot + popcount).
+//   fx_compact_scatter: pass 2 (per-tile exclusive offset, ballot/prefix row
+//                       map in LDS, region programs evaluated only for kept
+//                       rows, results written densely in source order).
+//
+// The three kernels share one bytecode interpreter (fx_run).  Instruction
+// fetch and decode are wave-uniform (scalar loads / scalar branches); every
+// instruction then operates on FX_V elements per lane, laid out so that lane l
+// of a workgroup handles elements l, l+256, l+512, l+768 of its tile: each
+// global load/store instruction of a wave covers 256 contiguous bytes.
+//
+// Replaces the NVRTC-generated kernels of the reference
+// (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121, launch shape
+// fait/fuser/graph_builder.cpp:463-499) and, for the data-dependent part, the
+// ATen nonzero/index calls the reference leaves unfused
+// (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include "fx_bytecode.h"
+
+namespace {
+
+// Everything wave-uniform (the static region blob, the by-value dynamic
+// arguments in the kernarg segment) is addressed through the constant address
+// space so that it is fetched with scalar loads.  The FxDyn kernel parameter
+// is never named inside a kernel: indexing a by-value aggregate dynamically
+// would make the compiler copy it to per-lane scratch.
+#define FX_AS4 __attribute__((address_space(4)))
+typedef const FX_AS4 uint32_t* fx_c32;
+typedef const FX_AS4 uint64_t* fx_c64;
+typedef uint32_t fx_u32x4 __attribute__((ext_vector_type(4)));
+typedef const FX_AS4 fx_u32x4* fx_cinsn;   // one FxInsn = 4 words
+typedef const FX_AS4 fx_u32x4* fx_caff;    // one FxAffine = 4 x 4 words
+typedef const FX_AS4 FxHeader* fx_chdr;
+typedef const FX_AS4 FxClass* fx_ccls;
+typedef const FX_AS4 FxOut* fx_cout;
+
+__device__ __forceinline__ fx_c64 fx_dyn_p() {
+  return (fx_c64)((const FX_AS4 uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + 8);
+}
+__device__ __forceinline__ fx_c32 fx_dyn_s() {
+  return (fx_c32)((const FX_AS4 uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + 8 + 8 * FX_DYN_P);
+}
+
+struct FxCtx {
+  fx_cinsn insn;          // class instruction base
+  fx_caff aff;            // class affine base
+  fx_c64 sptr;            // shared pointers (kernarg)
+  const uint64_t* tptr;   // per-task pointers (LDS)
+  fx_c32 sscal;           // shared scalars (kernarg)
+  const uint32_t* tscal;  // per-task scalars (LDS)
+  uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
+  int task;
+};
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
+
+// Data buffers are plain device allocations: address them through the global
+// address space (global_load / global_store instead of flat accesses).
+#define FX_AS1 __attribute__((address_space(1)))
+__device__ __forceinline__ uint32_t fx_load(const void* base_, int64_t off, uint32_t dt) {
+  const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
+  switch (dt) {
+    case FX_F32: return ((const FX_AS1 uint32_t*)base)[off];
+    case FX_I32: return ((const FX_AS1 uint32_t*)base)[off];
+    case FX_I64: return (uint32_t)((const FX_AS1 uint64_t*)base)[off];
+    case FX_U8: return base[off];
+    case FX_F16: {
+      uint16_t h = ((const FX_AS1 uint16_t*)base)[off];
+      __half hv = __ushort_as_half(h);
+      return f2u(__half2float(hv));
+    }
+    case FX_BF16: return ((uint32_t)((const FX_AS1 uint16_t*)base)[off]) << 16;
+    default: return 0;
+  }
+}
+
+__device__ __forceinline__ void fx_store(void* base_, int64_t off, uint32_t dt, uint32_t vt, uint32_t v) {
+  FX_AS1 uint8_t* base = (FX_AS1 uint8_t*)base_;
+  switch (dt) {
+    case FX_F32: ((FX_AS1 uint32_t*)base)[off] = (vt == FX_VT_F) ? v : f2u((float)(int32_t)v); break;
+    case FX_I32: ((FX_AS1 int32_t*)base)[off] = (vt == FX_VT_I) ? (int32_t)v : (int32_t)u2f(v); break;
+    case FX_I64: ((FX_AS1 int64_t*)base)[off] = (vt == FX_VT_I) ? (int64_t)(int32_t)v : (int64_t)u2f(v); break;
+    case FX_U8: base[off] = (vt == FX_VT_I) ? (uint8_t)v : (uint8_t)(u2f(v) != 0.0f); break;
+    case FX_F16: {
+      __half hv = __float2half(vt == FX_VT_F ? u2f(v) : (float)(int32_t)v);
+      ((FX_AS1 uint16_t*)base)[off] = __half_as_ushort(hv);
+    } break;
+    case FX_BF16: {
+      float f = vt == FX_VT_F ? u2f(v) : (float)(int32_t)v;
+      uint32_t u = f2u(f);
+      uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+      if (f != f) r = 0x7fc0u;
+      ((FX_AS1 uint16_t*)base)[off] = (uint16_t)r;
+    } break;
+    default: break;
+  }
+}
+
+__device__ __forceinline__ const void* fx_ptr(const FxCtx& cx, int32_t slot) {
+  uint64_t p = (slot & FX_SLOT_TASK) ? cx.tptr[slot & 0xffff] : cx.sptr[slot & 0xffff];
+  return (const void*)p;
+}
+
+__device__ __forceinline__ uint32_t fx_scalar(const FxCtx& cx, int32_t slot) {
+  return (slot & FX_SLOT_TASK) ? cx.tscal[slot & 0xffff] : cx.sscal[slot & 0xffff];
+}
+
+__device__ __forceinline__ int32_t floordiv_i(int32_t a, int32_t b) {
+  if (b == 0) return 0;
+  int32_t q = a / b;
+  if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
+  return q;
+}
+__device__ __forceinline__ int32_t pymod_i(int32_t a, int32_t b) {
+  if (b == 0) return 0;
+  int32_t r = a % b;
+  if (r != 0 && ((r < 0) != (b < 0))) r += b;
+  return r;
+}
+
+// NaN-propagating min / max (ATen semantics for maximum/minimum/clamp)
+__device__ __forceinline__ float fx_fmax(float a, float b) { return (a > b || a != a) ? a : b; }
+__device__ __forceinline__ float fx_fmin(float a, float b) { return (a < b || a != a) ? a : b; }
+
+__device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
+// The interpreter.  R = number of root coordinates that carry information.
+template <int R>
+__device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end,
+                                       const int32_t (&c)[FX_V][R > 0 ? R : 1], uint32_t M,
+                                       uint32_t (&A)[FX_V]) {
+  uint32_t B[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) B[j] = 0;
+  uint64_t MS = 0;              // mask stack, FX_V bits per level
+  int32_t lc[FX_MAXLOOP] = {0, 0};   // reduction loop counters (uniform)
+  int32_t le[FX_MAXLOOP] = {0, 0};
+  const uint32_t VM = (1u << FX_V) - 1u;
+
+  while (pc < pc_end) {
+    pc = __builtin_amdgcn_readfirstlane(pc);
+    FxInsn ins;
+    {
+      const fx_u32x4 w = cx.insn[pc];
+      ins.op = (uint16_t)(w.x & 0xffffu);
+      ins.flags = (uint8_t)((w.x >> 16) & 0xffu);
+      ins.dt = (uint8_t)(w.x >> 24);
+      ins.a = (int32_t)w.y;
+      ins.b = (int32_t)w.z;
+      ins.imm = w.w;
+    }
+    ++pc;
+    const uint32_t op = ins.op;
+    const bool useimm = (ins.flags & FX_F_IMM) != 0;
+
+#define FX_UNARY_F(expr)                                   \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
+      float a = u2f(A[j]);                                 \
+      A[j] = f2u(expr);                                    \
+    }                                                      \
+  } break
+#define FX_UNARY_I(expr)                                   \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
+      int32_t a = (int32_t)A[j];                           \
+      A[j] = (uint32_t)(expr);                             \
+    }                                                      \
+  } break
+#define FX_BIN_F(expr)                                     \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
+      float a = u2f(A[j]);                                 \
+      float b = u2f(useimm ? ins.imm : B[j]);              \
+      A[j] = f2u(expr);                                    \
+    }                                                      \
+  } break
+#define FX_CMP_F(expr)                                     \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
+      float a = u2f(A[j]);                                 \
+      float b = u2f(useimm ? ins.imm : B[j]);              \
+      A[j] = (expr) ? 1u : 0u;                             \
+    }                                                      \
+  } break
+#define FX_BIN_I(expr)                                     \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
+      int32_t a = (int32_t)A[j];                           \
+      int32_t b = (int32_t)(useimm ? ins.imm : B[j]);      \
+      A[j] = (uint32_t)(expr);                             \
+    }                                                      \
+  } break
+
+    switch (op) {
+      case FX_NOP: break;
+      case FX_LDA:
+      case FX_LDB:
+      case FX_AFFA:
+      case FX_AFFB: {
+        FxAffine af;
+        {
+          const fx_u32x4 w0 = cx.aff[ins.b * 4 + 0], w1 = cx.aff[ins.b * 4 + 1], w2 = cx.aff[ins.b * 4 + 2];
+          af.coef[0] = (int32_t)w0.x; af.coef[1] = (int32_t)w0.y; af.coef[2] = (int32_t)w0.z; af.coef[3] = (int32_t)w0.w;
+          af.coef[4] = (int32_t)w1.x; af.coef[5] = (int32_t)w1.y; af.tcoef = (int32_t)w1.z; af.base = (int32_t)w1.w;
+          af.rcoef[0] = (int32_t)w2.x; af.rcoef[1] = (int32_t)w2.y;
+        }
+        int32_t base = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
+        const bool is_load = (op == FX_LDA || op == FX_LDB);
+        const void* p = is_load ? fx_ptr(cx, ins.a) : nullptr;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          if ((M >> j) & 1u) {
+            int32_t off = base;
+#pragma unroll
+            for (int k = 0; k < R; ++k) off += af.coef[k] * c[j][k];
+            uint32_t v = is_load ? fx_load(p, (int64_t)off, ins.dt) : (uint32_t)off;
+            if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
+            if (op == FX_LDA || op == FX_AFFA) A[j] = v; else B[j] = v;
+          }
+        }
+      } break;
+      case FX_LDXA: {
+        const void* p = fx_ptr(cx, ins.a);
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          if ((M >> j) & 1u) A[j] = fx_load(p, (int64_t)((int32_t)A[j] + (int32_t)ins.imm), ins.dt);
+        }
+      } break;
+      case FX_IMMA:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = ins.imm;
+        break;
+      case FX_IMMB:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) B[j] = ins.imm;
+        break;
+      case FX_SCLA: {
+        uint32_t s = fx_scalar(cx, ins.a);
+        if (ins.flags & FX_F_I2F) s = f2u((float)(int32_t)s);
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = s;
+      } break;
+      case FX_SCLB: {
+        uint32_t s = fx_scalar(cx, ins.a);
+        if (ins.flags & FX_F_I2F) s = f2u((float)(int32_t)s);
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) B[j] = s;
+      } break;
+      case FX_STT:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) cx.temps[(ins.a * FX_V + j) * FX_BLOCK] = A[j];
+        break;
+      case FX_LDTA:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+        break;
+      case FX_LDTB:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) B[j] = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+        break;
+      case FX_MOVBA:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) B[j] = A[j];
+        break;
+      case FX_SWAP:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) { uint32_t t = A[j]; A[j] = B[j]; B[j] = t; }
+        break;
+
+      case FX_MIF: {
+        MS = (MS << FX_V) | (uint64_t)M;
+        uint32_t cnd = 0;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) cnd |= (A[j] != 0u ? 1u : 0u) << j;
+        M &= cnd;
+        if (!wave_any(M != 0u)) pc = ins.a;
+      } break;
+      case FX_MELSE: {
+        uint32_t top = (uint32_t)MS & VM;
+        M = top & ~M;
+        if (!wave_any(M != 0u)) pc = ins.a;
+      } break;
+      case FX_MMERGE: {
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          uint32_t t = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+          A[j] = ((M >> j) & 1u) ? A[j] : t;
+        }
+        M = (uint32_t)MS & VM;
+        MS >>= FX_V;
+      } break;
+      case FX_MEND:
+        M = (uint32_t)MS & VM;
+        MS >>= FX_V;
+        break;
+
+      case FX_FNEG: FX_UNARY_F(-a);
+      case FX_FABS: FX_UNARY_F(fabsf(a));
+      case FX_EXP: FX_UNARY_F(expf(a));
+      case FX_LOG: FX_UNARY_F(logf(a));
+      case FX_SQRT: FX_UNARY_F(sqrtf(a));
+      case FX_RSQRT: FX_UNARY_F(1.0f / sqrtf(a));
+      case FX_RCP: FX_UNARY_F(1.0f / a);
+      case FX_SIGMOID: FX_UNARY_F(1.0f / (1.0f + expf(-a)));
+      case FX_TANH: FX_UNARY_F(tanhf(a));
+      case FX_RELU: FX_UNARY_F((a <= 0.0f) ? 0.0f : a);
+      case FX_FLOOR: FX_UNARY_F(floorf(a));
+      case FX_CEIL: FX_UNARY_F(ceilf(a));
+      case FX_ROUND: FX_UNARY_F(rintf(a));
+      case FX_TRUNC: FX_UNARY_F(truncf(a));
+      case FX_SIN: FX_UNARY_F(sinf(a));
+      case FX_COS: FX_UNARY_F(cosf(a));
+      case FX_ERF: FX_UNARY_F(erff(a));
+      case FX_LOG2: FX_UNARY_F(log2f(a));
+      case FX_EXP2: FX_UNARY_F(exp2f(a));
+      case FX_EXPM1: FX_UNARY_F(expm1f(a));
+      case FX_LOG1P: FX_UNARY_F(log1pf(a));
+
+      case FX_INEG: FX_UNARY_I(-a);
+      case FX_IABS: FX_UNARY_I(a < 0 ? -a : a);
+      case FX_LNOT: FX_UNARY_I(a == 0 ? 1 : 0);
+      case FX_INZ: FX_UNARY_I(a != 0 ? 1 : 0);
+      case FX_FNZ:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) A[j] = (u2f(A[j]) != 0.0f) ? 1u : 0u;
+        break;
+      case FX_F2I:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) A[j] = (uint32_t)(int32_t)u2f(A[j]);
+        break;
+      case FX_I2F:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) A[j] = f2u((float)(int32_t)A[j]);
+        break;
+
+      case FX_FADD: FX_BIN_F(a + b);
+      case FX_FSUB: FX_BIN_F(a - b);
+      case FX_FRSUB: FX_BIN_F(b - a);
+      case FX_FMUL: FX_BIN_F(a * b);
+      case FX_FDIV: FX_BIN_F(a / b);
+      case FX_FRDIV: FX_BIN_F(b / a);
+      case FX_FMIN: FX_BIN_F(fx_fmin(a, b));
+      case FX_FMAX: FX_BIN_F(fx_fmax(a, b));
+      case FX_FPOW: FX_BIN_F(powf(a, b));
+      case FX_FMOD: FX_BIN_F(fmodf(a, b));
+      case FX_ATAN2: FX_BIN_F(atan2f(a, b));
+
+      case FX_IADD: FX_BIN_I(a + b);
+      case FX_ISUB: FX_BIN_I(a - b);
+      case FX_IRSUB: FX_BIN_I(b - a);
+      case FX_IMUL: FX_BIN_I(a * b);
+      case FX_IFDIV: FX_BIN_I(floordiv_i(a, b));
+      case FX_ITDIV: FX_BIN_I(b == 0 ? 0 : a / b);
+      case FX_IPMOD: FX_BIN_I(pymod_i(a, b));
+      case FX_ITMOD: FX_BIN_I(b == 0 ? 0 : a % b);
+      case FX_IMIN: FX_BIN_I(a < b ? a : b);
+      case FX_IMAX: FX_BIN_I(a > b ? a : b);
+      case FX_IAND: FX_BIN_I(a & b);
+      case FX_IOR: FX_BIN_I(a | b);
+      case FX_IXOR: FX_BIN_I(a ^ b);
+
+      case FX_FLT: FX_CMP_F(a < b);
+      case FX_FLE: FX_CMP_F(a <= b);
+      case FX_FGT: FX_CMP_F(a > b);
+      case FX_FGE: FX_CMP_F(a >= b);
+      case FX_FEQ: FX_CMP_F(a == b);
+      case FX_FNE: FX_CMP_F(a != b);
+      case FX_ILT: FX_BIN_I(a < b ? 1 : 0);
+      case FX_ILE: FX_BIN_I(a <= b ? 1 : 0);
+      case FX_IGT: FX_BIN_I(a > b ? 1 : 0);
+      case FX_IGE: FX_BIN_I(a >= b ? 1 : 0);
+      case FX_IEQ: FX_BIN_I(a == b ? 1 : 0);
+      case FX_INE: FX_BIN_I(a != b ? 1 : 0);
+
+      case FX_IRANGE: {
+        const int32_t lo = ins.a, hi = ins.b, st = (int32_t)ins.imm;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          int32_t a = (int32_t)A[j];
+          bool in = (a >= lo) && (a < hi);
+          if (st > 1) in = in && (((a - lo) % st) == 0);
+          A[j] = in ? 1u : 0u;
+        }
+      } break;
+      case FX_WHERE:
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          uint32_t cnd = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+          A[j] = cnd != 0u ? A[j] : B[j];
+        }
+        break;
+
+      case FX_RBEGIN: {
+        const int d = ins.a & (FX_MAXLOOP - 1);
+        lc[d] = 0;
+        le[d] = (int32_t)ins.imm;
+        if (le[d] <= 0) pc = ins.b;
+      } break;
+      case FX_RNEXT: {
+        const int d = ins.b & (FX_MAXLOOP - 1);
+        lc[d] += 1;
+        if (lc[d] < le[d]) pc = ins.a;
+      } break;
+      case FX_RIDX: {
+        const int32_t v = lc[ins.a & (FX_MAXLOOP - 1)];
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = (uint32_t)v;
+      } break;
+      default: break;
+    }
+  }
+#undef FX_UNARY_F
+#undef FX_UNARY_I
+#undef FX_BIN_F
+#undef FX_CMP_F
+#undef FX_BIN_I
+}
+
+__device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint32_t shift) {
+  return (__umulhi(n, magic) + n) >> shift;
+}
+
+// Decompose flat index e (row-major over od.dim[0..rank)) into coordinates.
+template <int R>
+__device__ __forceinline__ void fx_decompose(const FX_AS4 FxOut& od, uint32_t e, int32_t (&c)[R > 0 ? R : 1]) {
+#pragma unroll
+  for (int k = R - 1; k >= 1; --k) {
+    uint32_t q = fx_fastdiv(e, od.magic[k], od.shift[k]);
+    c[k] = (int32_t)(e - q * od.dim[k]);
+    e = q;
+  }
+  if (R > 0) c[0] = (int32_t)e;
+}
+
+struct FxWork {
+  fx_ccls cls;
+  int task;
+  uint32_t local_block;  // block index inside the task
+};
+
+template <bool COUNT_PASS>
+__device__ __forceinline__ FxWork fx_locate(fx_c32 sb, uint32_t block) {
+  fx_chdr h = (fx_chdr)sb;
+  fx_ccls cls = (fx_ccls)(sb + h->off_class);
+  uint32_t ci = 0;
+  while (ci + 1 < h->n_classes && block >= (COUNT_PASS ? cls[ci].cnt_block_end : cls[ci].block_end)) ++ci;
+  fx_ccls cl = cls + ci;
+  const uint32_t rel = block - (COUNT_PASS ? cl->cnt_block_begin : cl->block_begin);
+  const uint32_t bpt = COUNT_PASS ? cl->cnt_blocks_per_task : cl->blocks_per_task;
+  uint32_t ti = rel / bpt;
+  FxWork w;
+  w.cls = cl;
+  w.local_block = rel - ti * bpt;
+  w.task = (int)(sb + h->off_taskmap)[cl->first_task + ti];
+  return w;
+}
+
+// Stage this task's pointer / scalar record in LDS (one record per workgroup).
+__device__ __forceinline__ void fx_stage_task(fx_chdr h, int task, uint64_t* s_tp, uint32_t* s_ts) {
+  const uint32_t ntp = h->n_tptr, nts = h->n_tscal;
+  // the source lives in the kernarg segment; lanes read distinct words, so go
+  // through a generic pointer (vector loads)
+  const uint64_t* gp = (const uint64_t*)fx_dyn_p();
+  const uint32_t* gs = (const uint32_t*)fx_dyn_s();
+  if (threadIdx.x < ntp) s_tp[threadIdx.x] = gp[h->n_sptr + task * ntp + threadIdx.x];
+  if (threadIdx.x >= 64 && threadIdx.x - 64 < nts)
+    s_ts[threadIdx.x - 64] = gs[h->n_sscal + task * nts + (threadIdx.x - 64)];
+  __syncthreads();
+}
+
+}  // namespace
+
+// --------------------------------------------------------------------------
+// dense region kernel
+// --------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __restrict__ sb_, const FxDyn) {
+  extern __shared__ uint32_t s_temps[];
+  __shared__ uint64_t s_tp[FX_MAX_TPTR];
+  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+
+  fx_c32 sb = (fx_c32)sb_;
+  fx_chdr h = (fx_chdr)sb;
+  const FxWork w = fx_locate<false>(sb, blockIdx.x);
+  fx_ccls cl = w.cls;
+  fx_stage_task(h, w.task, s_tp, s_ts);
+
+  fx_cout outs = (fx_cout)(sb + cl->off_outs);
+  uint32_t oi = 0;
+  while (oi + 1 < cl->n_outs && w.local_block >= outs[oi].block_begin + outs[oi].n_blocks) ++oi;
+  const FX_AS4 FxOut& od = outs[oi];
+  const uint32_t tile = w.local_block - od.block_begin;
+
+  FxCtx cx;
+  cx.insn = (fx_cinsn)(sb + cl->off_insn);
+  cx.aff = (fx_caff)(sb + cl->off_aff);
+  cx.sptr = fx_dyn_p();
+  cx.tptr = s_tp;
+  cx.sscal = fx_dyn_s();
+  cx.tscal = s_ts;
+  cx.temps = s_temps + threadIdx.x;
+  cx.task = w.task;
+
+  int32_t c[FX_V][R > 0 ? R : 1];
+  uint32_t M = 0;
+  uint32_t e[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) {
+    e[j] = tile * FX_TILE + j * FX_BLOCK + threadIdx.x;
+    if (e[j] < od.numel) M |= 1u << j;
+    fx_decompose<R>(od, e[j], c[j]);
+  }
+  uint32_t A[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) A[j] = 0;
+  fx_run<R>(cx, (int)od.prog_begin, (int)od.prog_end, c, M, A);
+
+  void* op = (void*)fx_ptr(cx, (int32_t)od.ptr_slot);
+  const int64_t obase = (int64_t)od.task_stride * w.task;
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) {
+    if ((M >> j) & 1u) fx_store(op, obase + e[j], od.dtype, od.vt, A[j]);
+  }
+}
+
+// --------------------------------------------------------------------------
+// row compaction, pass 1: evaluate the mask program per row, write one flag
+// byte per row and one keep count per row tile.
+// grid = per task ceil(n_rows / FX_TILE) blocks; tile counts are per
+// row_tile rows (row_tile divides FX_BLOCK or equals it).
+// --------------------------------------------------------------------------
+__global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __restrict__ sb_, const FxDyn) {
+  extern __shared__ uint32_t s_temps[];
+  __shared__ uint64_t s_tp[FX_MAX_TPTR];
+  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+  __shared__ uint32_t s_wcnt[FX_V][FX_BLOCK / 64];
+
+  fx_c32 sb = (fx_c32)sb_;
+  fx_chdr h = (fx_chdr)sb;
+  const FxWork w = fx_locate<true>(sb, blockIdx.x);
+  fx_ccls cl = w.cls;
+  fx_stage_task(h, w.task, s_tp, s_ts);
+
+  FxCtx cx;
+  cx.insn = (fx_cinsn)(sb + cl->off_insn);
+  cx.aff = (fx_caff)(sb + cl->off_aff);
+  cx.sptr = fx_dyn_p();
+  cx.tptr = s_tp;
+  cx.sscal = fx_dyn_s();
+  cx.tscal = s_ts;
+  cx.temps = s_temps + threadIdx.x;
+  cx.task = w.task;
+
+  const uint32_t n_rows = cl->n_rows;
+  int32_t c[FX_V][1];
+  uint32_t M = 0;
+  uint32_t row[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) {
+    row[j] = w.local_block * FX_TILE + j * FX_BLOCK + threadIdx.x;
+    c[j][0] = (int32_t)row[j];
+    if (row[j] < n_rows) M |= 1u << j;
+  }
+  uint32_t A[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) A[j] = 0;
+  fx_run<1>(cx, (int)cl->mask_begin, (int)cl->mask_end, c, M, A);
+
+  uint8_t* flags = (uint8_t*)fx_dyn_p()[h->slot_flags] + (size_t)w.task * n_rows;
+  uint32_t* counts = (uint32_t*)fx_dyn_p()[h->slot_counts] + (size_t)w.task * h->max_rowtiles;
+  const uint32_t rt = h->row_tile;           // 64, 128 or 256
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) {
+    bool live = (M >> j) & 1u;
+    bool keep = live && (cl->mask_vt == FX_VT_F ? (u2f(A[j]) != 0.0f) : (A[j] != 0u));
+    if (live) flags[row[j]] = keep ? 1 : 0;
+    uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+    if (lane == 0) s_wcnt[j][wave] = (uint32_t)__popcll(bal);
+  }
+  __syncthreads();
+  // one count per row tile: FX_BLOCK / rt tiles per j-slab
+  const uint32_t waves_per_tile = rt / 64u;
+  const uint32_t tiles_per_slab = FX_BLOCK / rt;
+  if (threadIdx.x < FX_V * tiles_per_slab) {
+    uint32_t j = threadIdx.x / tiles_per_slab, t = threadIdx.x % tiles_per_slab;
+    uint32_t first_row = w.local_block * FX_TILE + j * FX_BLOCK + t * rt;
+    if (first_row < n_rows) {
+      uint32_t s = 0;
+      for (uint32_t k = 0; k < waves_per_tile; ++k) s += s_wcnt[j][t * waves_per_tile + k];
+      counts[first_row / rt] = s;
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
+// row compaction, pass 2.  One workgroup per (task, row tile):
+//   offset  = sum of the keep counts of the earlier tiles of this task
+//   row map = kept rows of this tile in source order (ballot + popcount prefix)
+//   for every output: evaluate its program on the kept rows only and write
+//   rows [offset, offset + kept) of the compacted output.
+// The last tile of a task also publishes the task's total.
+// --------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* __restrict__ sb_, const FxDyn) {
+  extern __shared__ uint32_t s_temps[];
+  __shared__ uint64_t s_tp[FX_MAX_TPTR];
+  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+  __shared__ uint32_t s_rowmap[FX_BLOCK];
+  __shared__ uint32_t s_wsum[FX_BLOCK / 64];
+  __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
+  __shared__ uint32_t s_prefix;
+
+  fx_c32 sb = (fx_c32)sb_;
+  fx_chdr h = (fx_chdr)sb;
+  const FxWork w = fx_locate<false>(sb, blockIdx.x);
+  fx_ccls cl = w.cls;
+  fx_stage_task(h, w.task, s_tp, s_ts);
+
+  const uint32_t n_rows = cl->n_rows;
+  const uint32_t rt = h->row_tile;
+  const uint32_t tile = w.local_block;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint8_t* flags = (const uint8_t*)fx_dyn_p()[h->slot_flags] + (size_t)w.task * n_rows;
+  const uint32_t* counts = (const uint32_t*)fx_dyn_p()[h->slot_counts] + (size_t)w.task * h->max_rowtiles;
+
+  // exclusive offset of this tile
+  uint32_t part = 0;
+  for (uint32_t t = threadIdx.x; t < tile; t += FX_BLOCK) part += counts[t];
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+  if (lane == 0) s_wsum[wave] = part;
+
+  // row map of this tile
+  const uint32_t row = tile * rt + threadIdx.x;
+  const bool keep = (threadIdx.x < rt) && (row < n_rows) && (flags[row] != 0);
+  const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+  const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+  if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t p = 0;
+    for (int k = 0; k < FX_BLOCK / 64; ++k) p += s_wsum[k];
+    s_prefix = p;
+    uint32_t acc = 0;
+    s_woff[0] = 0;
+    for (int k = 1; k <= FX_BLOCK / 64; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
+  }
+  __syncthreads();
+  if (keep) s_rowmap[s_woff[wave] + before] = row;
+  __syncthreads();
+  const uint32_t n_kept = s_woff[FX_BLOCK / 64];
+  const uint32_t prefix = s_prefix;
+  if (tile + 1 == cl->n_rowtiles && threadIdx.x == 0) {
+    ((uint32_t*)fx_dyn_p()[h->slot_total])[w.task] = prefix + n_kept;
+  }
+  if (n_kept == 0) return;
+
+  FxCtx cx;
+  cx.insn = (fx_cinsn)(sb + cl->off_insn);
+  cx.aff = (fx_caff)(sb + cl->off_aff);
+  cx.sptr = fx_dyn_p();
+  cx.tptr = s_tp;
+  cx.sscal = fx_dyn_s();
+  cx.tscal = s_ts;
+  cx.temps = s_temps + threadIdx.x;
+  cx.task = w.task;
+
+  fx_cout outs = (fx_cout)(sb + cl->off_outs);
+  for (uint32_t oi = 0; oi < cl->n_outs; ++oi) {
+    const FX_AS4 FxOut& od = outs[oi];
+    const uint32_t rowlen = od.rowlen;
+    const uint32_t n_el = n_kept * rowlen;
+    uint8_t* op = (uint8_t*)fx_ptr(cx, (int32_t)od.ptr_slot);
+    const int64_t obase = (int64_t)od.task_stride * w.task + (int64_t)prefix * rowlen;
+    for (uint32_t it = 0; it < n_el; it += FX_TILE) {
+      int32_t c[FX_V][R > 0 ? R : 1];
+      uint32_t M = 0;
+      uint32_t e[FX_V];
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) {
+        e[j] = it + j * FX_BLOCK + threadIdx.x;
+        const bool live = e[j] < n_el;
+        if (live) M |= 1u << j;
+        uint32_t r = fx_fastdiv(e[j], od.rl_magic, od.rl_shift);
+        uint32_t col = e[j] - r * rowlen;
+        // inner coordinates from col, coordinate 0 from the row map
+        int32_t cc[R > 0 ? R : 1];
+#pragma unroll
+        for (int k = R - 1; k >= 1; --k) {
+          uint32_t q = fx_fastdiv(col, od.magic[k], od.shift[k]);
+          cc[k] = (int32_t)(col - q * od.dim[k]);
+          col = q;
+        }
+        cc[0] = live ? (int32_t)s_rowmap[r] : 0;
+#pragma unroll
+        for (int k = 0; k < R; ++k) c[j][k] = cc[k];
+      }
+      uint32_t A[FX_V];
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) A[j] = 0;
+      fx_run<R>(cx, (int)od.prog_begin, (int)od.prog_end, c, M, A);
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) {
+        if ((M >> j) & 1u) fx_store(op, obase + e[j], od.dtype, od.vt, A[j]);
+      }
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
+// stand-alone order-preserving row compaction: out_c = col_c[mask] for up to
+// 8 columns that share one byte mask.  Tiles of FX_BLOCK rows.
+//   pass 1: per-tile keep counts (ballot + popcount)
+//   pass 2 (only above FX_SCAN_DIRECT tiles): exclusive scan of the counts
+//   pass 3: ballot/prefix row map in LDS, coalesced row copies
+// --------------------------------------------------------------------------
+#define FX_SCAN_DIRECT 2048
+struct FxCols {
+  const void* src[8];
+  void* dst[8];
+  int32_t words[8];   // 4-byte words per row (elsize 4/8) or bytes per row (elsize 1)
+  int32_t bytes[8];   // 1 = byte column, 0 = word column
+  int32_t n;
+};
+
+__global__ __launch_bounds__(FX_BLOCK) void fx_rows_count(const uint8_t* __restrict__ mask, uint32_t n,
+                                                          uint32_t* __restrict__ counts) {
+  __shared__ uint32_t s_w[FX_BLOCK / 64];
+  const uint32_t row = blockIdx.x * FX_BLOCK + threadIdx.x;
+  const bool keep = row < n && mask[row] != 0;
+  const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+  if ((threadIdx.x & 63u) == 0) s_w[threadIdx.x >> 6] = (uint32_t)__popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t s = 0;
+    for (int k = 0; k < FX_BLOCK / 64; ++k) s += s_w[k];
+    counts[blockIdx.x] = s;
+  }
+}
+
+// in-place exclusive scan of counts[0..t) by one workgroup; counts[t] = total
+__global__ __launch_bounds__(FX_BLOCK) void fx_rows_scan(uint32_t* __restrict__ counts, uint32_t t) {
+  __shared__ uint32_t s_w[FX_BLOCK / 64];
+  __shared__ uint32_t s_carry;
+  if (threadIdx.x == 0) s_carry = 0;
+  __syncthreads();
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  for (uint32_t base = 0; base < t; base += FX_BLOCK) {
+    const uint32_t i = base + threadIdx.x;
+    const uint32_t v = i < t ? counts[i] : 0u;
+    uint32_t x = v;  // inclusive wave scan
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      uint32_t y = __shfl_up(x, o, 64);
+      if (lane >= (uint32_t)o) x += y;
+    }
+    if (lane == 63) s_w[wave] = x;
+    __syncthreads();
+    uint32_t woff = 0;
+    for (uint32_t k = 0; k < wave; ++k) woff += s_w[k];
+    const uint32_t carry = s_carry;
+    if (i < t) counts[i] = carry + woff + x - v;
+    __syncthreads();
+    if (threadIdx.x == FX_BLOCK - 1) s_carry = carry + woff + x;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) counts[t] = s_carry;
+}
+
+template <bool SCANNED>
+__global__ __launch_bounds__(FX_BLOCK) void fx_rows_scatter(const uint8_t* __restrict__ mask, uint32_t n,
+                                                            const uint32_t* __restrict__ counts, const FxCols cols,
+                                                            uint32_t* __restrict__ total_host) {
+  __shared__ uint32_t s_rowmap[FX_BLOCK];
+  __shared__ uint32_t s_wsum[FX_BLOCK / 64];
+  __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
+  __shared__ uint32_t s_prefix;
+  const uint32_t tile = blockIdx.x;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  uint32_t part = 0;
+  if (!SCANNED) {
+    for (uint32_t t = threadIdx.x; t < tile; t += FX_BLOCK) part += counts[t];
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+    if (lane == 0) s_wsum[wave] = part;
+  }
+  const uint32_t row = tile * FX_BLOCK + threadIdx.x;
+  const bool keep = row < n && mask[row] != 0;
+  const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+  const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+  if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t p = 0;
+    if (SCANNED) p = counts[tile];
+    else for (int k = 0; k < FX_BLOCK / 64; ++k) p += s_wsum[k];
+    s_prefix = p;
+    uint32_t acc = 0;
+    s_woff[0] = 0;
+    for (int k = 1; k <= FX_BLOCK / 64; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
+  }
+  __syncthreads();
+  if (keep) s_rowmap[s_woff[wave] + before] = row;
+  __syncthreads();
+  const uint32_t n_kept = s_woff[FX_BLOCK / 64];
+  const uint32_t prefix = s_prefix;
+  if (tile + 1 == gridDim.x && threadIdx.x == 0) *total_host = prefix + n_kept;
+  if (n_kept == 0) return;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    if (c >= cols.n) break;
+    const uint32_t w = (uint32_t)cols.words[c];
+    const uint32_t n_el = n_kept * w;
+    if (cols.bytes[c]) {
+      const FX_AS1 uint8_t* src = (const FX_AS1 uint8_t*)cols.src[c];
+      FX_AS1 uint8_t* dst = (FX_AS1 uint8_t*)cols.dst[c] + (size_t)prefix * w;
+      for (uint32_t e = threadIdx.x; e < n_el; e += FX_BLOCK) {
+        const uint32_t r = e / w, k = e - r * w;
+        dst[e] = src[(size_t)s_rowmap[r] * w + k];
+      }
+    } else {
+      const FX_AS1 uint32_t* src = (const FX_AS1 uint32_t*)cols.src[c];
+      FX_AS1 uint32_t* dst = (FX_AS1 uint32_t*)cols.dst[c] + (size_t)prefix * w;
+      for (uint32_t e = threadIdx.x; e < n_el; e += FX_BLOCK) {
+        const uint32_t r = e / w, k = e - r * w;
+        dst[e] = src[(size_t)s_rowmap[r] * w + k];
+      }
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
+// plain copy kernel of known size: calibration of the HBM counters and the
+// bandwidth ceiling a kernel of this launch shape can reach.
+// --------------------------------------------------------------------------
+__global__ __launch_bounds__(FX_BLOCK) void fx_copy_f4(const float4* __restrict__ src, float4* __restrict__ dst, size_t n4) {
+  size_t i = (size_t)blockIdx.x * FX_BLOCK + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * FX_BLOCK;
+  for (; i < n4; i += stride) dst[i] = src[i];
+}
+
+// --------------------------------------------------------------------------
+// host-callable launchers (C++ linkage inside the library; the C ABI is in
+// fx_api.cpp)
+// --------------------------------------------------------------------------
+extern "C++" {
+
+hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+                           hipStream_t stream) {
+  if (grid == 0) return hipSuccess;
+  switch (rank) {
+    case 0:
+    case 1: fx_region_dense<1><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 2: fx_region_dense<2><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 3: fx_region_dense<3><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 4: fx_region_dense<4><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    default: fx_region_dense<FX_MAXR><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+  }
+  return hipGetLastError();
+}
+
+hipError_t fx_launch_compact_count(const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+                                   hipStream_t stream) {
+  if (grid == 0) return hipSuccess;
+  fx_compact_count<<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn);
+  return hipGetLastError();
+}
+
+hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid,
+                                     uint32_t lds_bytes, hipStream_t stream) {
+  if (grid == 0) return hipSuccess;
+  switch (rank) {
+    case 0:
+    case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 2: fx_compact_scatter<2><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 3: fx_compact_scatter<3><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 4: fx_compact_scatter<4><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    default: fx_compact_scatter<FX_MAXR><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+  }
+  return hipGetLastError();
+}
+
+hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                                  const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
+                                  uint32_t* total_host, hipStream_t stream) {
+  FxCols c;
+  for (int i = 0; i < 8; ++i) { c.src[i] = nullptr; c.dst[i] = nullptr; c.words[i] = 0; c.bytes[i] = 0; }
+  c.n = n_cols;
+  for (int i = 0; i < n_cols; ++i) {
+    c.src[i] = cols[i];
+    c.dst[i] = outs[i];
+    c.bytes[i] = elsize[i] == 1 ? 1 : 0;
+    c.words[i] = elsize[i] == 1 ? rowlen[i] : rowlen[i] * (elsize[i] / 4);
+  }
+  const uint32_t tiles = (uint32_t)((n + FX_BLOCK - 1) / FX_BLOCK);
+  fx_rows_count<<<tiles, FX_BLOCK, 0, stream>>>(mask, (uint32_t)n, counts);
+  if (tiles > FX_SCAN_DIRECT) {
+    fx_rows_scan<<<1, FX_BLOCK, 0, stream>>>(counts, tiles);
+    fx_rows_scatter<true><<<tiles, FX_BLOCK, 0, stream>>>(mask, (uint32_t)n, counts, c, total_host);
+  } else {
+    fx_rows_scatter<false><<<tiles, FX_BLOCK, 0, stream>>>(mask, (uint32_t)n, counts, c, total_host);
+  }
+  return hipGetLastError();
+}
+
+hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream) {
+  fx_copy_f4<<<grid, FX_BLOCK, 0, stream>>>((const float4*)src, (float4*)dst, bytes / 16);
+  return hipGetLastError();
+}
+
+}  // extern "C++"

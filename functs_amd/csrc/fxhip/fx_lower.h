@@ -1,0 +1,102 @@
+// Host-side region IR, shape functions and lowering to VM bytecode.
+// Pure C++ (no HIP): everything here runs without a device.
+//
+// Plays the role of fait/fuser/graph_builder.cpp:259-712 (GraphBuilder::compile),
+// the shape tables fait/fuser/shape_func.cpp:9-374 and the lowering functions
+// functs/csrc/jit/tensorexpr/nnc_ext.cpp:62-392 /
+// fait/fuser/custom_lowering_func.cpp:17-498, but emits descriptors for
+// hand-written kernels instead of NNC statements.
+#pragma once
+#include <stdint.h>
+
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../../include/fxhip.h"
+#include "fx_bytecode.h"
+
+namespace fx {
+
+struct Error : std::runtime_error {
+  int code;
+  Error(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+
+enum VKind { VK_TENSOR, VK_INT, VK_FLOAT, VK_BOOL, VK_NONE, VK_INT_LIST, VK_TENSOR_LIST };
+enum Prod { P_INPUT, P_CONST, P_TASK, P_LOOPVAR, P_LIST, P_OP };
+
+struct Value {
+  VKind kind = VK_NONE;
+  Prod prod = P_CONST;
+  int dtype = -1;  // FX_DT_* for tensors
+  int rank = -1;
+  int op = 0;
+  std::vector<int> args;
+  int64_t ival = 0;
+  double fval = 0;
+  int input_index = -1;
+  bool per_task = false;
+};
+
+struct Plan;
+
+struct Region {
+  int degree = 1;
+  bool is_map = false;
+  bool finalized = false;
+  std::vector<Value> vals;
+  std::vector<int> inputs;   // value ids, declaration order
+  std::vector<int> outputs;  // value ids
+  int mask = -1;             // row-compaction mask value id
+  std::map<std::vector<int64_t>, std::unique_ptr<Plan>> plans;
+
+  int add(const Value& v) {
+    vals.push_back(v);
+    return (int)vals.size() - 1;
+  }
+  int addOp(int opcode, const std::vector<int>& args, int out_dtype);
+};
+
+// where a dynamic pointer / scalar slot is filled from at run time
+struct PtrSrc {
+  enum Kind { INPUT, OUTPUT, FLAGS, COUNTS, TOTALS } kind;
+  int index;  // region input index / output index
+};
+struct ScalSrc {
+  int input;      // region input index
+  bool as_float;  // store float(value) instead of int32(value)
+};
+
+struct Plan {
+  const Region* region = nullptr;
+  std::vector<uint32_t> blob;  // static part (FxHeader ...)
+  uint32_t mode = FX_MODE_DENSE;
+  uint32_t grid = 0;           // dense grid, or scatter grid in compaction mode
+  uint32_t grid_count = 0;     // compaction pass 1
+  uint32_t lds_bytes = 0;
+  int max_rank = 1;
+  std::vector<PtrSrc> sptr, tptr;
+  std::vector<ScalSrc> sscal, tscal;
+  std::vector<int> out_dtype;                                 // per output
+  std::vector<std::vector<std::vector<int64_t>>> out_shape;   // [out][task][dim]
+  size_t scratch_bytes = 0, flags_off = 0, counts_off = 0;
+  int launches = 0;
+  int64_t alg_bytes = 0;
+  std::vector<int> arg_base;  // first fx_arg of each region input
+  int n_args = 0;
+  // device copy of blob, created on first run
+  void* dev_blob = nullptr;
+  int dev_id = -1;
+};
+
+// Builds (or fetches from the cache) the plan of `r` for these arguments.
+const Plan* plan_region(Region& r, const fx_arg* args, int n_args);
+std::string disasm(const Plan& p);
+
+int dtype_size(int dt);
+
+}  // namespace fx

@@ -1,0 +1,202 @@
+/* fxhip.h - C ABI of the MI355X (gfx950) execution layer for FuncTs/FAIT fused
+ * functionalized regions.
+ *
+ * This is the boundary the reference crosses when a tssa::ParallelFunctor
+ * operator runs: it replaces the NVRTC code generator and launcher
+ *   fait/tensorexpr/cuda_codegen_tssa.h:193-239  (class CudaCodeGenTssa)
+ * and the per-operator lowering tables that define the kernel arithmetic
+ *   functs/csrc/jit/tensorexpr/nnc_ext.cpp:62-392
+ *   fait/fuser/custom_lowering_func.cpp:502-559
+ *   fait/fuser/shape_func.cpp:274-374
+ * Plain C types only: no torch types, no C++ types.  All device buffers are
+ * owned by the caller.  Every function returns 0 on success or a negative
+ * FX_E_* code; fx_last_error() gives the message for the calling thread.
+ */
+#ifndef FXHIP_H_
+#define FXHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FX_API_VERSION 1
+#define FX_MAX_RANK 6 /* max rank of a region output */
+#define FX_ARG_MAX_RANK 8
+
+/* error codes */
+#define FX_OK 0
+#define FX_E_INVALID (-1)     /* malformed call or region (reference: malformed_input, cuda_codegen_tssa.cpp:1293-1295) */
+#define FX_E_UNSUPPORTED (-2) /* op / dtype / rank outside what the kernels implement (reference aborts: graph_builder.cpp:409-414) */
+#define FX_E_HIP (-3)         /* a HIP runtime call failed */
+#define FX_E_LIMIT (-4)       /* a fixed capacity was exceeded (tasks x pointers, temps, nesting) */
+#define FX_E_NODEVICE (-5)    /* no usable gfx950 device */
+
+/* element types of tensors (storage) and scalars */
+#define FX_DT_F32 0
+#define FX_DT_I64 1
+#define FX_DT_I32 2
+#define FX_DT_U8 3
+#define FX_DT_F16 4
+#define FX_DT_BF16 5
+#define FX_DT_BOOL 6 /* stored as one byte */
+
+/* Operators a region can be built from.  Each mirrors one entry of the
+ * reference's lowering tables (file:line given per group). */
+enum fx_opcode {
+  /* immut:: access / assign family: nnc_ext.cpp:62-392, symbol_ext.cpp:9-199 */
+  FX_OP_ACCESS = 1,   /* (src) */
+  FX_OP_ASSIGN,       /* (self, src) -> src                      nnc_ext.cpp:71-80 */
+  FX_OP_CLONE,        /* (src)  clone / contiguous               nnc_ext.cpp:62-69 */
+  FX_OP_SELECT,       /* (src, int dim, int index)               nnc_ext.cpp:166-185 */
+  FX_OP_SELECT_REV,   /* (self, src, int dim, int index)         nnc_ext.cpp:187-212 */
+  FX_OP_SLICE,        /* (src, int dim, int? start, int? end, int step)   custom_lowering_func.cpp:200-227 */
+  FX_OP_SLICE_REV,    /* (self, src, int dim, int? start, int? end, int step)  nnc_ext.cpp:112-164 */
+  FX_OP_SQUEEZE,      /* (src, int dim) */
+  FX_OP_UNSQUEEZE,    /* (src, int dim)                          nnc_ext.cpp:214-229 */
+  FX_OP_VIEW,         /* (src, int[] sizes)  view / reshape      nnc_ext.cpp:231-295 */
+  FX_OP_PERMUTE,      /* (src, int[] dims)                       nnc_ext.cpp:320-358 */
+  FX_OP_TRANSPOSE,    /* (src, int d0, int d1)                   shape_func.cpp:127-138 */
+  FX_OP_EXPAND,       /* (src, int[] sizes)                      nnc_ext.cpp:360-370 */
+  FX_OP_EXPAND_AS,    /* (src, other) */
+  FX_OP_REPEAT,       /* (src, int[] repeats)                    nnc_ext.cpp:297-318 */
+  FX_OP_INDEX,        /* (src, Tensor[] {int64 index})  dim 0    nnc_ext.cpp:372-392 */
+  FX_OP_CAT,          /* (Tensor[] tensors, int dim)             custom_lowering_func.cpp:297-330 */
+  FX_OP_STACK,        /* (Tensor[] tensors, int dim)             custom_lowering_func.cpp:332-350 */
+  /* creation: custom_lowering_func.cpp:17-49 */
+  FX_OP_FULL,         /* (int[] size, scalar value)  zeros / ones / full; out dtype required */
+  FX_OP_ARANGE,       /* (int start, int end)        out dtype required */
+  FX_OP_SCALAR_TENSOR,/* (scalar) -> 0-dim tensor    out dtype required */
+  FX_OP_TRIU,         /* (self, int diagonal) */
+  /* elementwise unary: stock NNC lowerings (graph_builder.cpp:388-407) */
+  FX_OP_EXP, FX_OP_LOG, FX_OP_SQRT, FX_OP_RSQRT, FX_OP_SIGMOID, FX_OP_TANH, FX_OP_RELU,
+  FX_OP_NEG, FX_OP_ABS, FX_OP_FLOOR, FX_OP_CEIL, FX_OP_ROUND, FX_OP_SIN, FX_OP_COS, FX_OP_ERF,
+  FX_OP_RECIPROCAL, FX_OP_LOGICAL_NOT,
+  FX_OP_TO,           /* (self) dtype cast; out dtype required */
+  /* elementwise binary, tensor (x) tensor|scalar with broadcasting:
+   * custom_lowering_func.cpp:51-76, shape_func.cpp:23-49 */
+  FX_OP_ADD,          /* (self, other, scalar alpha=1) */
+  FX_OP_SUB,          /* (self, other, scalar alpha=1) */
+  FX_OP_RSUB,         /* (self, other, scalar alpha=1) -> other - alpha*self */
+  FX_OP_MUL, FX_OP_DIV, FX_OP_MAXIMUM, FX_OP_MINIMUM, FX_OP_POW, FX_OP_FMOD,
+  FX_OP_EQ, FX_OP_NE, FX_OP_LT, FX_OP_LE, FX_OP_GT, FX_OP_GE,
+  FX_OP_AND, FX_OP_OR, FX_OP_XOR,
+  FX_OP_CLAMP,        /* (self, scalar? min, scalar? max)       custom_lowering_func.cpp:355-368 */
+  FX_OP_WHERE,        /* (cond, self, other) */
+  /* reductions over one dimension: custom_lowering_func.cpp:112-180 */
+  FX_OP_MAX_DIM,      /* (self, int dim, bool keepdim) -> values */
+  FX_OP_SUM_DIM,      /* (self, int dim, bool keepdim) */
+  FX_OP_SOFTMAX,      /* (self, int dim) */
+  /* integer scalar arithmetic on index values */
+  FX_OP_INT_ADD, FX_OP_INT_SUB, FX_OP_INT_MUL, FX_OP_INT_NEG,
+  FX_OP_SIZE,         /* (tensor, int dim) -> int                graph_builder.cpp:319-327 */
+  /* A prim::Loop whose only carried value is a tensor read through
+   * immut::select(T, dim, i) and written through immut::select_rev(T, ., dim, i),
+   * collapsed to one region: (self, body, int dim, int lo, int hi) where body is
+   * built with fx_region_loop_var() standing for i.  No reference counterpart:
+   * the reference keeps such loops serial (parallelize_loops.cpp:17). */
+  FX_OP_FORALL_SELECT_REV,
+  FX_OP__COUNT
+};
+
+typedef struct fx_region fx_region; /* a region under construction / compiled */
+typedef struct fx_plan fx_plan;     /* a region specialised to concrete shapes */
+
+/* One run-time argument.  Tensors may be strided; sizes/strides in elements. */
+typedef struct fx_arg {
+  int32_t kind; /* 0 tensor, 1 int, 2 float, 3 bool */
+  int32_t dtype;
+  const void* ptr; /* device pointer (tensor) */
+  int32_t rank;
+  int32_t reserved;
+  int64_t sizes[FX_ARG_MAX_RANK];
+  int64_t strides[FX_ARG_MAX_RANK];
+  int64_t ival; /* int / bool scalar */
+  double fval;  /* float scalar (narrowed to fp32 like graph_builder.cpp:850-854) */
+} fx_arg;
+
+const char* fx_last_error(void);
+int fx_api_version(void);
+
+/* ---- region construction (replaces GraphBuilder::compile, graph_builder.cpp:259-712) ----
+ * parallel_degree / is_parallel_map have the meaning of the attributes of
+ * tssa::ParallelFunctor (fait/passes/te_op.h:13-23). */
+int fx_region_create(int parallel_degree, int is_parallel_map, fx_region** out);
+void fx_region_destroy(fx_region*);
+
+/* Values.  Every function returns a value id (>= 0) in *id. */
+/* tensor input; per_task = the matching entry of attr::is_parallel_args (a list
+ * with one tensor per task, te_op.cpp:89-98) */
+int fx_region_input_tensor(fx_region*, int dtype, int rank, int per_task, int* id);
+int fx_region_input_scalar(fx_region*, int kind /*1 int,2 float,3 bool*/, int per_task, int* id);
+int fx_region_task_index(fx_region*, int* id); /* subgraph input 0 (te_op.cpp:192, graph_builder.cpp:269-272) */
+int fx_region_loop_var(fx_region*, int* id);   /* see FX_OP_FORALL_SELECT_REV */
+int fx_region_const_int(fx_region*, int64_t v, int* id);
+int fx_region_const_float(fx_region*, double v, int* id);
+int fx_region_const_bool(fx_region*, int v, int* id);
+int fx_region_const_none(fx_region*, int* id);
+int fx_region_int_list(fx_region*, const int* ids, int n, int* id);
+int fx_region_tensor_list(fx_region*, const int* ids, int n, int* id);
+/* out_dtype < 0: infer by type promotion */
+int fx_region_op(fx_region*, int opcode, const int* arg_ids, int n_args, int out_dtype, int* id);
+int fx_region_output(fx_region*, int value_id);
+/* Fuse an order-preserving masked row select into the region: every output x
+ * becomes x[mask] (mask: bool tensor over dim 0, computed in the region).
+ * Contract: ATen index/nonzero semantics, which the reference leaves to ATen
+ * (convert_to_tensorssa.cpp:422-443, fuse_ops.cpp:173-200). */
+int fx_region_compact_rows(fx_region*, int mask_value_id);
+int fx_region_finalize(fx_region*);
+
+/* ---- specialisation to shapes (replaces DimExprEvaluator + prepareRunArgs shape part,
+ *      evaluate_dim.cpp:132-227, graph_builder.cpp:863-889) ----
+ * args: for each region input in declaration order, 1 entry, or
+ * parallel_degree entries if it is per-task.  The plan is owned by the region
+ * and cached by shape signature. */
+int fx_region_plan(fx_region*, const fx_arg* args, int n_args, const fx_plan** plan);
+int fx_plan_num_outputs(const fx_plan*);
+/* shape of output out_idx for task; for a compacted output sizes[0] is the upper bound */
+int fx_plan_output(const fx_plan*, int out_idx, int task, int32_t* dtype, int32_t* rank, int64_t* sizes);
+size_t fx_plan_scratch_bytes(const fx_plan*); /* device scratch the caller must provide to fx_region_run */
+int fx_plan_launches(const fx_plan*);         /* kernel launches one fx_region_run issues */
+int64_t fx_plan_algorithmic_bytes(const fx_plan*); /* compulsory input bytes + dense output bytes */
+/* debugging / test hooks: the lowered bytecode blob (like CodeGen::getCodeText) */
+int fx_plan_blob(const fx_plan*, const uint32_t** words, size_t* n_words);
+int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);
+
+/* ---- execution (replaces CudaCodeGenTssa::call_raw, cuda_codegen_tssa.cpp:1167-1290) ----
+ * out_ptrs[out_idx * parallel_degree + task] = device buffer of that output.
+ * scratch: fx_plan_scratch_bytes() of device memory (may be NULL when 0).
+ * totals_host: for compacting regions, pinned host memory (device-visible) of
+ *   parallel_degree uint32 that receives the kept-row count per task; it is
+ *   valid after the stream has been synchronised.  NULL otherwise.
+ * Asynchronous on `stream` (a hipStream_t); no hidden synchronisation. */
+int fx_region_run(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
+                  void* scratch, uint32_t* totals_host, void* stream);
+
+/* The argument marshalling of fx_region_run without the launch (host only; the
+ * analogue of GraphBuilder::prepareRunArgs, graph_builder.cpp:718-899).
+ * dyn_out receives fx_dyn_bytes() bytes: the by-value block the kernels read. */
+int fx_region_marshal(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
+                      void* scratch, uint32_t* totals_host, void* dyn_out, size_t dyn_cap);
+size_t fx_dyn_bytes(void);
+
+/* ---- stand-alone order-preserving row compaction (x[mask] for several x) ----
+ * mask: n bytes (0/1); cols[i]: [n, rowlen[i]] fp32/int32 (4-byte) or int64 (8-byte) rows.
+ * outs[i] must hold n * rowlen[i] elements.  Same contract as ATen
+ * index(Tensor, [bool mask]) / nonzero. */
+int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                    const int32_t* rowlen, const int32_t* elsize, int n_cols, void* scratch,
+                    size_t scratch_bytes, uint32_t* total_host, void* stream);
+size_t fx_compact_rows_scratch_bytes(int64_t n);
+
+/* ---- device utilities ---- */
+int fx_device_count(void);
+/* plain 16-byte copy kernel of known size: counter calibration and bandwidth ceiling */
+int fx_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FXHIP_H_ */

@@ -1,0 +1,111 @@
+"""Fused regions of the five benchmark configurations, written directly against
+the region builder.  Each function states the functionalized graph (immut::
+access / assign operators) that the pass pipeline produces for the matching
+TorchScript program and hands it to the HIP backend as ONE region.
+
+Graph shapes follow the reference's own worked examples: README.md:284-299
+(get_started after functionalization), README.md:484-507 (slice/select assigns
+inlined into one fused subgraph), README.md:611-659 (ParallelMap ->
+tssa::ParallelFunctor with parallel_degree / is_parallel_args).
+"""
+import torch
+
+from .region import Region
+
+
+def build_c1():
+    """get_started loop (examples/get_started.py:10-15) after functionalization:
+        for i in range(n): b = immut::select_rev(b, immut::select(b, 0, i) + 1, 0, i)
+    The carried tensor is read and written only through slab i, so the n
+    iterations collapse into one region (FX_OP_FORALL_SELECT_REV)."""
+    r = Region()
+    b = r.tensor_input(torch.float32, 2)
+    n = r.scalar_input("int")
+    i = r.loop_var()
+    body = b.select(0, i) + 1
+    r.output(r.op("FORALL_SELECT_REV", b, body, 0, 0, n))
+    return r.finalize()
+
+
+def _yolo_body(r, pred, anchors, strides):
+    """pred: [1, N, 85] value.  Returns (boxes [N,4], cls [N,80], obj [N], keep [N])."""
+    # pred[..., :2].sigmoid_()  ->  slice_rev(pred, sigmoid(slice(pred)))
+    pred1 = pred.slice_rev(pred.slice(2, 0, 2).sigmoid(), 2, 0, 2)
+    obj = pred1.select(2, 4).sigmoid()           # [1, N]
+    cls = pred1.slice(2, 5, None).sigmoid()      # [1, N, 80]
+    p = pred1.select(0, 0)                       # [N, 85]
+    xy = (anchors.slice(1, 0, 2) + anchors.slice(1, 2, None)) * 0.5 + (p.slice(1, 0, 2) - 0.5) * strides.unsqueeze(-1)
+    wh = (anchors.slice(1, 2, None) - anchors.slice(1, 0, 2)) * 0.5 * p.slice(1, 2, 4).exp()
+    boxes = r.op("FULL", r.int_list([r.op("SIZE", anchors, 0), 4]), 0.0, dtype=torch.float32)
+    boxes = boxes.select_rev(xy.select(1, 0) - wh.select(1, 0), 1, 0)
+    boxes = boxes.select_rev(xy.select(1, 1) - wh.select(1, 1), 1, 1)
+    boxes = boxes.select_rev(xy.select(1, 0) + wh.select(1, 0), 1, 2)
+    boxes = boxes.select_rev(xy.select(1, 1) + wh.select(1, 1), 1, 3)
+    obj0 = obj.select(0, 0)
+    keep = obj0 >= 0.3
+    return boxes, cls.select(0, 0), obj0, keep
+
+
+def build_c2():
+    """YOLOv3-style post-processing of one image: decode + sigmoid + confidence
+    mask select as one compacting region."""
+    r = Region()
+    pred = r.tensor_input(torch.float32, 3)
+    anchors = r.tensor_input(torch.float32, 2)
+    strides = r.tensor_input(torch.float32, 1)
+    boxes, cls, obj, keep = _yolo_body(r, pred, anchors, strides)
+    r.output(boxes)
+    r.output(cls)
+    r.output(obj)
+    r.compact_rows(keep)
+    return r.finalize()
+
+
+def build_c5(batch=16):
+    """The per-image loop over c2 as one ParallelMap launch: task i works on
+    preds[i:i+1]; anchors and strides are shared (is_parallel_args = 0)."""
+    r = Region(parallel_degree=batch, is_parallel_map=True)
+    preds = r.tensor_input(torch.float32, 3)
+    anchors = r.tensor_input(torch.float32, 2)
+    strides = r.tensor_input(torch.float32, 1)
+    i = r.task_index()
+    pred = preds.slice(0, i, r.op("INT_ADD", i, 1))
+    boxes, cls, obj, keep = _yolo_body(r, pred, anchors, strides)
+    r.output(boxes)
+    r.output(cls)
+    r.output(obj)
+    r.compact_rows(keep)
+    return r.finalize()
+
+
+def build_c3_decode():
+    """SSD prior/variance decode (two slice assigns) + softmax: one dense region
+    with two outputs (boxes [N,4], scores [N,C])."""
+    r = Region()
+    loc = r.tensor_input(torch.float32, 3)
+    conf = r.tensor_input(torch.float32, 3)
+    priors = r.tensor_input(torch.float32, 2)
+    l0 = loc.select(0, 0)
+    cxcy = priors.slice(1, 0, 2) + l0.slice(1, 0, 2) * 0.1 * priors.slice(1, 2, None)
+    wh = priors.slice(1, 2, None) * (l0.slice(1, 2, None) * 0.2).exp()
+    boxes = r.op("FULL", r.int_list([r.op("SIZE", priors, 0), 4]), 0.0, dtype=torch.float32)
+    boxes = boxes.slice_rev(cxcy - wh / 2, 1, 0, 2)
+    boxes = boxes.slice_rev(cxcy + wh / 2, 1, 2, None)
+    scores = conf.select(0, 0).softmax(-1)
+    r.output(boxes)
+    r.output(scores)
+    return r.finalize()
+
+
+def build_c3_classes(n_fg=80):
+    """The per-class loop `for c in range(1, C): m = scores[:, c] > 0.05;
+    boxes[m], scores[:, c][m]` as one ParallelMap over the classes."""
+    r = Region(parallel_degree=n_fg, is_parallel_map=True)
+    boxes = r.tensor_input(torch.float32, 2)
+    scores = r.tensor_input(torch.float32, 2)
+    c = r.op("INT_ADD", r.task_index(), 1)
+    sc = scores.select(1, c)
+    r.output(boxes)
+    r.output(sc)
+    r.compact_rows(sc > 0.05)
+    return r.finalize()

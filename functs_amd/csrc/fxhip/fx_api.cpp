@@ -13,12 +13,12 @@
 
 #include "fx_lower.h"
 
-hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                            hipStream_t stream);
-hipError_t fx_launch_compact_count(const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                                    hipStream_t stream);
-hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid,
-                                     uint32_t lds_bytes, hipStream_t stream);
+hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
+                                     uint32_t grid, hipStream_t stream);
 hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream);
 hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                   const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
@@ -316,8 +316,8 @@ int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, i
 
 size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
 
-int fx_region_run(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
-                  void* scratch, uint32_t* totals_host, void* stream_) {
+static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                    void* scratch, uint32_t* totals_host, void* stream_, float* kernel_ms, int cap, int* n_kernels) {
   if (!reg || !plan || !out_ptrs) return fail(FX_E_INVALID, "null argument");
   fx::Plan* pl = const_cast<fx::Plan*>(P(plan));
   if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
@@ -342,18 +342,56 @@ int fx_region_run(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n
   int rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, &dyn);
   if (rc != FX_OK) return rc;
   const uint32_t* sb = (const uint32_t*)pl->dev_blob;
+  FxLaunchInfo li;
+  li.blob_words = (uint32_t)pl->blob.size();
+  li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
+  li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
+  li.n_temps = pl->n_temps;
   if (pl->mode == FX_MODE_COMPACT) {
     // tasks without rows launch no tile: their total is published here.  The
     // caller must not reuse totals_host while an earlier run is still in flight.
     for (int t = 0; t < reg->r.degree; ++t) totals_host[t] = 0;
   }
+  // optional per-kernel timing with events on the launch stream
+  hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+  const bool timed = kernel_ms != nullptr;
+  int nk = 0;
+  if (timed)
+    for (auto& e : ev) HIP_OK(hipEventCreate(&e));
+  auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(ev[i], stream) : hipSuccess; };
   if (pl->mode == FX_MODE_DENSE) {
-    HIP_OK(fx_launch_dense(pl->max_rank, sb, &dyn, pl->grid, pl->lds_bytes, stream));
+    HIP_OK(mark(0));
+    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, pl->grid, stream));
+    HIP_OK(mark(1));
+    nk = pl->grid > 0 ? 1 : 0;
   } else {
-    HIP_OK(fx_launch_compact_count(sb, &dyn, pl->grid_count, pl->lds_bytes, stream));
-    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, &dyn, pl->grid, pl->lds_bytes, stream));
+    HIP_OK(mark(0));
+    HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream));
+    HIP_OK(mark(1));
+    HIP_OK(mark(2));
+    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn, pl->grid, stream));
+    HIP_OK(mark(3));
+    nk = pl->grid > 0 ? 2 : 0;
+  }
+  if (timed) {
+    HIP_OK(hipEventSynchronize(ev[nk == 2 ? 3 : 1]));
+    for (int k = 0; k < nk && k < cap; ++k) HIP_OK(hipEventElapsedTime(&kernel_ms[k], ev[2 * k], ev[2 * k + 1]));
+    for (auto& e : ev) (void)hipEventDestroy(e);
+    if (n_kernels) *n_kernels = nk;
   }
   return FX_OK;
+}
+
+int fx_region_run(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                  void* scratch, uint32_t* totals_host, void* stream) {
+  return run_impl(reg, plan, args, n_args, out_ptrs, scratch, totals_host, stream, nullptr, 0, nullptr);
+}
+
+int fx_region_run_timed(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                        void* scratch, uint32_t* totals_host, void* stream, float* kernel_ms, int cap,
+                        int* n_kernels) {
+  if (!kernel_ms || cap < 2) return fail(FX_E_INVALID, "fx_region_run_timed: kernel_ms[>=2] required");
+  return run_impl(reg, plan, args, n_args, out_ptrs, scratch, totals_host, stream, kernel_ms, cap, n_kernels);
 }
 
 size_t fx_compact_rows_scratch_bytes(int64_t n) {

@@ -100,11 +100,25 @@ struct FxInsn {
 // element offset = base + tcoef * task + sum_k coef[k] * coord[k] + sum_d rcoef[d] * loop_counter[d]
 #define FX_MAXLOOP 2
 struct FxAffine {
-  int32_t coef[FX_MAXR];
+  int32_t coef03[4];          // coefficients of root coordinates 0..3
   int32_t tcoef;
   int32_t base;
   int32_t rcoef[FX_MAXLOOP];
-  int32_t pad[6];
+  int32_t coef45[2];          // coefficients of root coordinates 4, 5
+  int32_t pad[2];
+};
+#define FX_AFF_WORDS 12
+static inline int32_t fx_aff_coef(const struct FxAffine* a, int k) { return k < 4 ? a->coef03[k] : a->coef45[k - 4]; }
+static inline void fx_aff_set_coef(struct FxAffine* a, int k, int32_t v) {
+  if (k < 4) a->coef03[k] = v; else a->coef45[k - 4] = v;
+}
+
+// what a launcher needs to know about a lowered region besides the blob itself
+struct FxLaunchInfo {
+  uint32_t blob_words;  // multiple of 4
+  uint32_t n_p;         // pointer slots in use
+  uint32_t n_s;         // scalar slots in use
+  uint32_t n_temps;     // LDS temp slots per lane
 };
 
 #define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table

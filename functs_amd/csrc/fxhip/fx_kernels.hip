@@ -8,66 +8,58 @@
 //                       map in LDS, region programs evaluated only for kept
 //                       rows, results written densely in source order).
 //
-// The three kernels share one bytecode interpreter (fx_run).  Instruction
-// fetch and decode are wave-uniform (scalar loads / scalar branches); every
-// instruction then operates on FX_V elements per lane, laid out so that lane l
-// of a workgroup handles elements l, l+256, l+512, l+768 of its tile: each
-// global load/store instruction of a wave covers 256 contiguous bytes.
+// The three kernels share one bytecode interpreter (fx_run).  A workgroup
+// first copies the whole region descriptor (programs, affine maps, output
+// descriptors, task classes) and the per-call pointer / scalar tables of all
+// tasks into LDS with one round of coalesced 128-bit loads; from then on every
+// table access is an LDS broadcast read, so no dependent chain of cold global
+// loads sits in front of the data traffic.  Instruction decode is
+// wave-uniform (the opcode word goes through readfirstlane, the switch is a
+// scalar branch); every instruction then operates on FX_V elements per lane,
+// laid out so that lane l of a workgroup handles elements l, l+256, l+512,
+// l+768 of its tile: each global load/store instruction of a wave covers 256
+// contiguous bytes.
 //
 // Replaces the NVRTC-generated kernels of the reference
 // (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121, launch shape
-// fait/fuser/graph_builder.cpp:463-499) and, for the data-dependent part, the
-// ATen nonzero/index calls the reference leaves unfused
-// (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
+// fait/fuser/graph_builder.cpp:463-499, per-task code cloning
+// fait/tensorexpr/functor_parallization.cpp:93-108) and, for the
+// data-dependent part, the ATen nonzero/index calls the reference leaves
+// unfused (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
-#include <hip/hip_bf16.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "fx_bytecode.h"
 
 namespace {
 
-// Everything wave-uniform (the static region blob, the by-value dynamic
-// arguments in the kernarg segment) is addressed through the constant address
-// space so that it is fetched with scalar loads.  The FxDyn kernel parameter
-// is never named inside a kernel: indexing a by-value aggregate dynamically
-// would make the compiler copy it to per-lane scratch.
+#define FX_AS1 __attribute__((address_space(1)))
 #define FX_AS4 __attribute__((address_space(4)))
-typedef const FX_AS4 uint32_t* fx_c32;
-typedef const FX_AS4 uint64_t* fx_c64;
 typedef uint32_t fx_u32x4 __attribute__((ext_vector_type(4)));
-typedef const FX_AS4 fx_u32x4* fx_cinsn;   // one FxInsn = 4 words
-typedef const FX_AS4 fx_u32x4* fx_caff;    // one FxAffine = 4 x 4 words
-typedef const FX_AS4 FxHeader* fx_chdr;
-typedef const FX_AS4 FxClass* fx_ccls;
-typedef const FX_AS4 FxOut* fx_cout;
 
-__device__ __forceinline__ fx_c64 fx_dyn_p() {
-  return (fx_c64)((const FX_AS4 uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + 8);
-}
-__device__ __forceinline__ fx_c32 fx_dyn_s() {
-  return (fx_c32)((const FX_AS4 uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + 8 + 8 * FX_DYN_P);
-}
+// word offset of a field inside a blob structure
+#define FX_W(Type, field) (offsetof(Type, field) / 4)
+
+__device__ __forceinline__ uint32_t uni(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
 struct FxCtx {
-  fx_cinsn insn;          // class instruction base
-  fx_caff aff;            // class affine base
-  fx_c64 sptr;            // shared pointers (kernarg)
-  const uint64_t* tptr;   // per-task pointers (LDS)
-  fx_c32 sscal;           // shared scalars (kernarg)
-  const uint32_t* tscal;  // per-task scalars (LDS)
+  const fx_u32x4* insn;   // LDS: class instruction base
+  const uint32_t* aff;    // LDS: class affine base (FX_AFF_WORDS words each)
+  const uint64_t* ptrs;   // LDS: [shared ptrs][task 0 ptrs][task 1 ptrs]...
+  const uint32_t* scal;   // LDS: [shared scalars][task 0 scalars]...
+  uint32_t tp_off;        // index of this task's first pointer
+  uint32_t ts_off;        // index of this task's first scalar
   uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
   int task;
 };
 
-__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
-__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
-
 // Data buffers are plain device allocations: address them through the global
 // address space (global_load / global_store instead of flat accesses).
-#define FX_AS1 __attribute__((address_space(1)))
-__device__ __forceinline__ uint32_t fx_load(const void* base_, int64_t off, uint32_t dt) {
+__device__ __forceinline__ uint32_t fx_load(uint64_t base_, int64_t off, uint32_t dt) {
   const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
   switch (dt) {
     case FX_F32: return ((const FX_AS1 uint32_t*)base)[off];
@@ -84,7 +76,7 @@ __device__ __forceinline__ uint32_t fx_load(const void* base_, int64_t off, uint
   }
 }
 
-__device__ __forceinline__ void fx_store(void* base_, int64_t off, uint32_t dt, uint32_t vt, uint32_t v) {
+__device__ __forceinline__ void fx_store(uint64_t base_, int64_t off, uint32_t dt, uint32_t vt, uint32_t v) {
   FX_AS1 uint8_t* base = (FX_AS1 uint8_t*)base_;
   switch (dt) {
     case FX_F32: ((FX_AS1 uint32_t*)base)[off] = (vt == FX_VT_F) ? v : f2u((float)(int32_t)v); break;
@@ -106,13 +98,14 @@ __device__ __forceinline__ void fx_store(void* base_, int64_t off, uint32_t dt, 
   }
 }
 
-__device__ __forceinline__ const void* fx_ptr(const FxCtx& cx, int32_t slot) {
-  uint64_t p = (slot & FX_SLOT_TASK) ? cx.tptr[slot & 0xffff] : cx.sptr[slot & 0xffff];
-  return (const void*)p;
+__device__ __forceinline__ uint64_t fx_ptr(const FxCtx& cx, int32_t slot) {
+  const uint32_t i = (slot & FX_SLOT_TASK) ? cx.tp_off + (uint32_t)(slot & 0xffff) : (uint32_t)(slot & 0xffff);
+  return cx.ptrs[i];
 }
 
 __device__ __forceinline__ uint32_t fx_scalar(const FxCtx& cx, int32_t slot) {
-  return (slot & FX_SLOT_TASK) ? cx.tscal[slot & 0xffff] : cx.sscal[slot & 0xffff];
+  const uint32_t i = (slot & FX_SLOT_TASK) ? cx.ts_off + (uint32_t)(slot & 0xffff) : (uint32_t)(slot & 0xffff);
+  return cx.scal[i];
 }
 
 __device__ __forceinline__ int32_t floordiv_i(int32_t a, int32_t b) {
@@ -135,34 +128,37 @@ __device__ __forceinline__ float fx_fmin(float a, float b) { return (a < b || a 
 __device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
 
 // The interpreter.  R = number of root coordinates that carry information.
+// The program lives in LDS; the next instruction word is fetched while the
+// current one executes.  The host pads every program area with one trailing
+// NOP so that the look-ahead read stays inside the blob.
 template <int R>
-__device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end,
-                                       const int32_t (&c)[FX_V][R > 0 ? R : 1], uint32_t M,
-                                       uint32_t (&A)[FX_V]) {
+__device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end, const int32_t (&c)[FX_V][R],
+                                       uint32_t M, uint32_t (&A)[FX_V]) {
   uint32_t B[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) B[j] = 0;
-  uint64_t MS = 0;              // mask stack, FX_V bits per level
-  int32_t lc[FX_MAXLOOP] = {0, 0};   // reduction loop counters (uniform)
-  int32_t le[FX_MAXLOOP] = {0, 0};
+  uint64_t MS = 0;      // mask stack, FX_V bits per level
+  int32_t lc0 = 0, lc1 = 0, le0 = 0, le1 = 0;  // reduction loop counters / extents (uniform)
   const uint32_t VM = (1u << FX_V) - 1u;
 
+  fx_u32x4 nxt = cx.insn[pc];
   while (pc < pc_end) {
-    pc = __builtin_amdgcn_readfirstlane(pc);
-    FxInsn ins;
-    {
-      const fx_u32x4 w = cx.insn[pc];
-      ins.op = (uint16_t)(w.x & 0xffffu);
-      ins.flags = (uint8_t)((w.x >> 16) & 0xffu);
-      ins.dt = (uint8_t)(w.x >> 24);
-      ins.a = (int32_t)w.y;
-      ins.b = (int32_t)w.z;
-      ins.imm = w.w;
-    }
-    ++pc;
-    const uint32_t op = ins.op;
-    const bool useimm = (ins.flags & FX_F_IMM) != 0;
+    const fx_u32x4 w = nxt;
+    int npc = pc + 1;
+    nxt = cx.insn[npc];
+    const uint32_t w0 = uni(w.x);
+    const uint32_t op = w0 & 0xffffu;
+    const bool useimm = (w0 & (FX_F_IMM << 16)) != 0;
+    const bool cvt = (w0 & (FX_F_I2F << 16)) != 0;
+    const uint32_t dt = w0 >> 24;
+    const int32_t ia = (int32_t)w.y, ib = (int32_t)w.z;
+    const uint32_t imm = w.w;
 
+#define FX_JUMP(target)                 \
+  {                                     \
+    npc = (int)uni((uint32_t)(target)); \
+    nxt = cx.insn[npc];                 \
+  }
 #define FX_UNARY_F(expr)                                   \
   {                                                        \
     _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
@@ -181,7 +177,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
   {                                                        \
     _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
       float a = u2f(A[j]);                                 \
-      float b = u2f(useimm ? ins.imm : B[j]);              \
+      float b = u2f(useimm ? imm : B[j]);                  \
       A[j] = f2u(expr);                                    \
     }                                                      \
   } break
@@ -189,7 +185,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
   {                                                        \
     _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
       float a = u2f(A[j]);                                 \
-      float b = u2f(useimm ? ins.imm : B[j]);              \
+      float b = u2f(useimm ? imm : B[j]);                  \
       A[j] = (expr) ? 1u : 0u;                             \
     }                                                      \
   } break
@@ -197,7 +193,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
   {                                                        \
     _Pragma("unroll") for (int j = 0; j < FX_V; ++j) {     \
       int32_t a = (int32_t)A[j];                           \
-      int32_t b = (int32_t)(useimm ? ins.imm : B[j]);      \
+      int32_t b = (int32_t)(useimm ? imm : B[j]);          \
       A[j] = (uint32_t)(expr);                             \
     }                                                      \
   } break
@@ -208,66 +204,69 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
       case FX_LDB:
       case FX_AFFA:
       case FX_AFFB: {
-        FxAffine af;
-        {
-          const fx_u32x4 w0 = cx.aff[ins.b * 4 + 0], w1 = cx.aff[ins.b * 4 + 1], w2 = cx.aff[ins.b * 4 + 2];
-          af.coef[0] = (int32_t)w0.x; af.coef[1] = (int32_t)w0.y; af.coef[2] = (int32_t)w0.z; af.coef[3] = (int32_t)w0.w;
-          af.coef[4] = (int32_t)w1.x; af.coef[5] = (int32_t)w1.y; af.tcoef = (int32_t)w1.z; af.base = (int32_t)w1.w;
-          af.rcoef[0] = (int32_t)w2.x; af.rcoef[1] = (int32_t)w2.y;
+        const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + ib * FX_AFF_WORDS);
+        const fx_u32x4 a0 = ap[0], a1 = ap[1];
+        int32_t cf[FX_MAXR];
+        cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
+        if (R > 4) {
+          const fx_u32x4 a2 = ap[2];
+          cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
+        } else {
+          cf[4] = 0; cf[5] = 0;
         }
-        int32_t base = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
+        const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
         const bool is_load = (op == FX_LDA || op == FX_LDB);
-        const void* p = is_load ? fx_ptr(cx, ins.a) : nullptr;
+        const uint64_t p = is_load ? fx_ptr(cx, ia) : 0ull;
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
           if ((M >> j) & 1u) {
             int32_t off = base;
 #pragma unroll
-            for (int k = 0; k < R; ++k) off += af.coef[k] * c[j][k];
-            uint32_t v = is_load ? fx_load(p, (int64_t)off, ins.dt) : (uint32_t)off;
-            if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
+            for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
+            uint32_t v = is_load ? fx_load(p, (int64_t)off, dt) : (uint32_t)off;
+            if (cvt) v = f2u((float)(int32_t)v);
             if (op == FX_LDA || op == FX_AFFA) A[j] = v; else B[j] = v;
           }
         }
       } break;
       case FX_LDXA: {
-        const void* p = fx_ptr(cx, ins.a);
+        const uint64_t p = fx_ptr(cx, ia);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) A[j] = fx_load(p, (int64_t)((int32_t)A[j] + (int32_t)ins.imm), ins.dt);
+          if ((M >> j) & 1u) A[j] = fx_load(p, (int64_t)((int32_t)A[j] + (int32_t)imm), dt);
         }
       } break;
       case FX_IMMA:
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = ins.imm;
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = imm;
         break;
       case FX_IMMB:
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) B[j] = ins.imm;
+        for (int j = 0; j < FX_V; ++j) B[j] = imm;
         break;
       case FX_SCLA: {
-        uint32_t s = fx_scalar(cx, ins.a);
-        if (ins.flags & FX_F_I2F) s = f2u((float)(int32_t)s);
+        uint32_t s = fx_scalar(cx, ia);
+        if (cvt) s = f2u((float)(int32_t)s);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = s;
       } break;
       case FX_SCLB: {
-        uint32_t s = fx_scalar(cx, ins.a);
-        if (ins.flags & FX_F_I2F) s = f2u((float)(int32_t)s);
+        uint32_t s = fx_scalar(cx, ia);
+        if (cvt) s = f2u((float)(int32_t)s);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) B[j] = s;
       } break;
       case FX_STT:
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) cx.temps[(ins.a * FX_V + j) * FX_BLOCK] = A[j];
+        for (int j = 0; j < FX_V; ++j) cx.temps[(ia * FX_V + j) * FX_BLOCK] = A[j];
         break;
       case FX_LDTA:
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+        for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = cx.temps[(ia * FX_V + j) * FX_BLOCK];
         break;
       case FX_LDTB:
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) B[j] = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+        for (int j = 0; j < FX_V; ++j) B[j] = cx.temps[(ia * FX_V + j) * FX_BLOCK];
         break;
       case FX_MOVBA:
 #pragma unroll
@@ -284,17 +283,17 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) cnd |= (A[j] != 0u ? 1u : 0u) << j;
         M &= cnd;
-        if (!wave_any(M != 0u)) pc = ins.a;
+        if (!wave_any(M != 0u)) FX_JUMP(ia)
       } break;
       case FX_MELSE: {
         uint32_t top = (uint32_t)MS & VM;
         M = top & ~M;
-        if (!wave_any(M != 0u)) pc = ins.a;
+        if (!wave_any(M != 0u)) FX_JUMP(ia)
       } break;
       case FX_MMERGE: {
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
-          uint32_t t = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+          uint32_t t = cx.temps[(ia * FX_V + j) * FX_BLOCK];
           A[j] = ((M >> j) & 1u) ? A[j] : t;
         }
         M = (uint32_t)MS & VM;
@@ -384,7 +383,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
       case FX_INE: FX_BIN_I(a != b ? 1 : 0);
 
       case FX_IRANGE: {
-        const int32_t lo = ins.a, hi = ins.b, st = (int32_t)ins.imm;
+        const int32_t lo = ia, hi = ib, st = (int32_t)uni(imm);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
           int32_t a = (int32_t)A[j];
@@ -396,30 +395,33 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
       case FX_WHERE:
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
-          uint32_t cnd = cx.temps[(ins.a * FX_V + j) * FX_BLOCK];
+          uint32_t cnd = cx.temps[(ia * FX_V + j) * FX_BLOCK];
           A[j] = cnd != 0u ? A[j] : B[j];
         }
         break;
 
       case FX_RBEGIN: {
-        const int d = ins.a & (FX_MAXLOOP - 1);
-        lc[d] = 0;
-        le[d] = (int32_t)ins.imm;
-        if (le[d] <= 0) pc = ins.b;
+        const uint32_t d = uni((uint32_t)ia) & 1u;
+        const int32_t ext = (int32_t)uni(imm);
+        if (d == 0) { lc0 = 0; le0 = ext; } else { lc1 = 0; le1 = ext; }
+        if (ext <= 0) FX_JUMP(ib)
       } break;
       case FX_RNEXT: {
-        const int d = ins.b & (FX_MAXLOOP - 1);
-        lc[d] += 1;
-        if (lc[d] < le[d]) pc = ins.a;
+        const uint32_t d = uni((uint32_t)ib) & 1u;
+        bool again;
+        if (d == 0) { lc0 += 1; again = lc0 < le0; } else { lc1 += 1; again = lc1 < le1; }
+        if (again) FX_JUMP(ia)
       } break;
       case FX_RIDX: {
-        const int32_t v = lc[ins.a & (FX_MAXLOOP - 1)];
+        const int32_t v = (uni((uint32_t)ia) & 1u) ? lc1 : lc0;
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = (uint32_t)v;
       } break;
       default: break;
     }
+    pc = npc;
   }
+#undef FX_JUMP
 #undef FX_UNARY_F
 #undef FX_UNARY_I
 #undef FX_BIN_F
@@ -431,52 +433,71 @@ __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint3
   return (__umulhi(n, magic) + n) >> shift;
 }
 
-// Decompose flat index e (row-major over od.dim[0..rank)) into coordinates.
-template <int R>
-__device__ __forceinline__ void fx_decompose(const FX_AS4 FxOut& od, uint32_t e, int32_t (&c)[R > 0 ? R : 1]) {
-#pragma unroll
-  for (int k = R - 1; k >= 1; --k) {
-    uint32_t q = fx_fastdiv(e, od.magic[k], od.shift[k]);
-    c[k] = (int32_t)(e - q * od.dim[k]);
-    e = q;
-  }
-  if (R > 0) c[0] = (int32_t)e;
+// ---- workgroup prologue ----------------------------------------------------
+// LDS layout (words): [blob][pointers: 2 words each][scalars][pad][temps]
+struct FxLaunch {
+  uint32_t blob_words;  // multiple of 4
+  uint32_t n_p;         // pointers in use in FxDyn::p
+  uint32_t n_s;         // scalars in use in FxDyn::s
+  uint32_t temps_off;   // word offset of the temp area in LDS (multiple of 4)
+};
+#define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
+
+__device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict__ sb, const FxLaunch& la) {
+  const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)sb;
+  fx_u32x4* l4 = (fx_u32x4*)L;
+  for (uint32_t i = threadIdx.x; i < la.blob_words / 4; i += FX_BLOCK) l4[i] = g4[i];
+  // The by-value FxDyn block is read through the kernarg segment pointer (never
+  // by naming the parameter: indexing a by-value aggregate dynamically would
+  // make the compiler copy it to per-lane scratch).
+  const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
+  const uint64_t* gp = (const uint64_t*)(ka + FX_KERNARG_DYN_OFF);
+  const uint32_t* gs = (const uint32_t*)(ka + FX_KERNARG_DYN_OFF + 8 * FX_DYN_P);
+  uint64_t* lp = (uint64_t*)(L + la.blob_words);
+  uint32_t* ls = L + la.blob_words + 2 * la.n_p;
+  for (uint32_t i = threadIdx.x; i < la.n_p; i += FX_BLOCK) lp[i] = gp[i];
+  for (uint32_t i = threadIdx.x; i < la.n_s; i += FX_BLOCK) ls[i] = gs[i];
+  __syncthreads();
 }
 
 struct FxWork {
-  fx_ccls cls;
+  const uint32_t* cls;   // LDS: FxClass words
   int task;
   uint32_t local_block;  // block index inside the task
 };
 
 template <bool COUNT_PASS>
-__device__ __forceinline__ FxWork fx_locate(fx_c32 sb, uint32_t block) {
-  fx_chdr h = (fx_chdr)sb;
-  fx_ccls cls = (fx_ccls)(sb + h->off_class);
+__device__ __forceinline__ FxWork fx_locate(const uint32_t* L, uint32_t block) {
+  const uint32_t n_classes = uni(L[FX_W(FxHeader, n_classes)]);
+  const uint32_t* cls = L + uni(L[FX_W(FxHeader, off_class)]);
+  const uint32_t cw = sizeof(FxClass) / 4;
+  const uint32_t end_w = COUNT_PASS ? FX_W(FxClass, cnt_block_end) : FX_W(FxClass, block_end);
   uint32_t ci = 0;
-  while (ci + 1 < h->n_classes && block >= (COUNT_PASS ? cls[ci].cnt_block_end : cls[ci].block_end)) ++ci;
-  fx_ccls cl = cls + ci;
-  const uint32_t rel = block - (COUNT_PASS ? cl->cnt_block_begin : cl->block_begin);
-  const uint32_t bpt = COUNT_PASS ? cl->cnt_blocks_per_task : cl->blocks_per_task;
-  uint32_t ti = rel / bpt;
+  while (ci + 1 < n_classes && block >= uni(cls[ci * cw + end_w])) ++ci;
+  const uint32_t* cl = cls + ci * cw;
+  const uint32_t rel = block - uni(cl[COUNT_PASS ? FX_W(FxClass, cnt_block_begin) : FX_W(FxClass, block_begin)]);
+  const uint32_t bpt = uni(cl[COUNT_PASS ? FX_W(FxClass, cnt_blocks_per_task) : FX_W(FxClass, blocks_per_task)]);
+  const uint32_t ti = rel / bpt;
   FxWork w;
   w.cls = cl;
   w.local_block = rel - ti * bpt;
-  w.task = (int)(sb + h->off_taskmap)[cl->first_task + ti];
+  w.task = (int)uni(L[uni(L[FX_W(FxHeader, off_taskmap)]) + uni(cl[FX_W(FxClass, first_task)]) + ti]);
   return w;
 }
 
-// Stage this task's pointer / scalar record in LDS (one record per workgroup).
-__device__ __forceinline__ void fx_stage_task(fx_chdr h, int task, uint64_t* s_tp, uint32_t* s_ts) {
-  const uint32_t ntp = h->n_tptr, nts = h->n_tscal;
-  // the source lives in the kernarg segment; lanes read distinct words, so go
-  // through a generic pointer (vector loads)
-  const uint64_t* gp = (const uint64_t*)fx_dyn_p();
-  const uint32_t* gs = (const uint32_t*)fx_dyn_s();
-  if (threadIdx.x < ntp) s_tp[threadIdx.x] = gp[h->n_sptr + task * ntp + threadIdx.x];
-  if (threadIdx.x >= 64 && threadIdx.x - 64 < nts)
-    s_ts[threadIdx.x - 64] = gs[h->n_sscal + task * nts + (threadIdx.x - 64)];
-  __syncthreads();
+__device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, const FxWork& w) {
+  FxCtx cx;
+  cx.insn = (const fx_u32x4*)(L + uni(w.cls[FX_W(FxClass, off_insn)]));
+  cx.aff = L + uni(w.cls[FX_W(FxClass, off_aff)]);
+  cx.ptrs = (const uint64_t*)(L + la.blob_words);
+  cx.scal = L + la.blob_words + 2 * la.n_p;
+  const uint32_t n_sptr = uni(L[FX_W(FxHeader, n_sptr)]), n_tptr = uni(L[FX_W(FxHeader, n_tptr)]);
+  const uint32_t n_sscal = uni(L[FX_W(FxHeader, n_sscal)]), n_tscal = uni(L[FX_W(FxHeader, n_tscal)]);
+  cx.tp_off = n_sptr + (uint32_t)w.task * n_tptr;
+  cx.ts_off = n_sscal + (uint32_t)w.task * n_tscal;
+  cx.temps = L + la.temps_off + threadIdx.x;
+  cx.task = w.task;
+  return cx;
 }
 
 }  // namespace
@@ -485,52 +506,61 @@ __device__ __forceinline__ void fx_stage_task(fx_chdr h, int task, uint64_t* s_t
 // dense region kernel
 // --------------------------------------------------------------------------
 template <int R>
-__global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __restrict__ sb_, const FxDyn) {
-  extern __shared__ uint32_t s_temps[];
-  __shared__ uint64_t s_tp[FX_MAX_TPTR];
-  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+__global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __restrict__ sb, const FxLaunch la,
+                                                            const FxDyn) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
+  fx_stage(L, sb, la);
+  const FxWork w = fx_locate<false>(L, blockIdx.x);
+  const FxCtx cx = fx_make_ctx(L, la, w);
 
-  fx_c32 sb = (fx_c32)sb_;
-  fx_chdr h = (fx_chdr)sb;
-  const FxWork w = fx_locate<false>(sb, blockIdx.x);
-  fx_ccls cl = w.cls;
-  fx_stage_task(h, w.task, s_tp, s_ts);
-
-  fx_cout outs = (fx_cout)(sb + cl->off_outs);
+  const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
+  const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
+  const uint32_t ow = sizeof(FxOut) / 4;
   uint32_t oi = 0;
-  while (oi + 1 < cl->n_outs && w.local_block >= outs[oi].block_begin + outs[oi].n_blocks) ++oi;
-  const FX_AS4 FxOut& od = outs[oi];
-  const uint32_t tile = w.local_block - od.block_begin;
+  while (oi + 1 < n_outs &&
+         w.local_block >= uni(outs[oi * ow + FX_W(FxOut, block_begin)]) + uni(outs[oi * ow + FX_W(FxOut, n_blocks)]))
+    ++oi;
+  const uint32_t* od = outs + oi * ow;
+  const uint32_t tile = w.local_block - uni(od[FX_W(FxOut, block_begin)]);
+  const uint32_t numel = uni(od[FX_W(FxOut, numel)]);
 
-  FxCtx cx;
-  cx.insn = (fx_cinsn)(sb + cl->off_insn);
-  cx.aff = (fx_caff)(sb + cl->off_aff);
-  cx.sptr = fx_dyn_p();
-  cx.tptr = s_tp;
-  cx.sscal = fx_dyn_s();
-  cx.tscal = s_ts;
-  cx.temps = s_temps + threadIdx.x;
-  cx.task = w.task;
-
-  int32_t c[FX_V][R > 0 ? R : 1];
+  int32_t c[FX_V][R];
   uint32_t M = 0;
   uint32_t e[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) {
     e[j] = tile * FX_TILE + j * FX_BLOCK + threadIdx.x;
-    if (e[j] < od.numel) M |= 1u << j;
-    fx_decompose<R>(od, e[j], c[j]);
+    if (e[j] < numel) M |= 1u << j;
+  }
+  // flat index -> coordinates (row-major over dim[0..R))
+  {
+    uint32_t rem[FX_V];
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) rem[j] = e[j];
+#pragma unroll
+    for (int k = R - 1; k >= 1; --k) {
+      const uint32_t dk = od[FX_W(FxOut, dim) + k], mk = od[FX_W(FxOut, magic) + k], sk = od[FX_W(FxOut, shift) + k];
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) {
+        const uint32_t q = fx_fastdiv(rem[j], mk, sk);
+        c[j][k] = (int32_t)(rem[j] - q * dk);
+        rem[j] = q;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) c[j][0] = (int32_t)rem[j];
   }
   uint32_t A[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) A[j] = 0;
-  fx_run<R>(cx, (int)od.prog_begin, (int)od.prog_end, c, M, A);
+  fx_run<R>(cx, (int)uni(od[FX_W(FxOut, prog_begin)]), (int)uni(od[FX_W(FxOut, prog_end)]), c, M, A);
 
-  void* op = (void*)fx_ptr(cx, (int32_t)od.ptr_slot);
-  const int64_t obase = (int64_t)od.task_stride * w.task;
+  const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
+  const int64_t obase = (int64_t)od[FX_W(FxOut, task_stride)] * w.task;
+  const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) {
-    if ((M >> j) & 1u) fx_store(op, obase + e[j], od.dtype, od.vt, A[j]);
+    if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
   }
 }
 
@@ -538,31 +568,17 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
 // row compaction, pass 1: evaluate the mask program per row, write one flag
 // byte per row and one keep count per row tile.
 // grid = per task ceil(n_rows / FX_TILE) blocks; tile counts are per
-// row_tile rows (row_tile divides FX_BLOCK or equals it).
+// row_tile rows (row_tile is 64, 128 or 256).
 // --------------------------------------------------------------------------
-__global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __restrict__ sb_, const FxDyn) {
-  extern __shared__ uint32_t s_temps[];
-  __shared__ uint64_t s_tp[FX_MAX_TPTR];
-  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+__global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __restrict__ sb, const FxLaunch la,
+                                                             const FxDyn) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
   __shared__ uint32_t s_wcnt[FX_V][FX_BLOCK / 64];
+  fx_stage(L, sb, la);
+  const FxWork w = fx_locate<true>(L, blockIdx.x);
+  const FxCtx cx = fx_make_ctx(L, la, w);
 
-  fx_c32 sb = (fx_c32)sb_;
-  fx_chdr h = (fx_chdr)sb;
-  const FxWork w = fx_locate<true>(sb, blockIdx.x);
-  fx_ccls cl = w.cls;
-  fx_stage_task(h, w.task, s_tp, s_ts);
-
-  FxCtx cx;
-  cx.insn = (fx_cinsn)(sb + cl->off_insn);
-  cx.aff = (fx_caff)(sb + cl->off_aff);
-  cx.sptr = fx_dyn_p();
-  cx.tptr = s_tp;
-  cx.sscal = fx_dyn_s();
-  cx.tscal = s_ts;
-  cx.temps = s_temps + threadIdx.x;
-  cx.task = w.task;
-
-  const uint32_t n_rows = cl->n_rows;
+  const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
   int32_t c[FX_V][1];
   uint32_t M = 0;
   uint32_t row[FX_V];
@@ -575,27 +591,29 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
   uint32_t A[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) A[j] = 0;
-  fx_run<1>(cx, (int)cl->mask_begin, (int)cl->mask_end, c, M, A);
+  fx_run<1>(cx, (int)uni(w.cls[FX_W(FxClass, mask_begin)]), (int)uni(w.cls[FX_W(FxClass, mask_end)]), c, M, A);
 
-  uint8_t* flags = (uint8_t*)fx_dyn_p()[h->slot_flags] + (size_t)w.task * n_rows;
-  uint32_t* counts = (uint32_t*)fx_dyn_p()[h->slot_counts] + (size_t)w.task * h->max_rowtiles;
-  const uint32_t rt = h->row_tile;           // 64, 128 or 256
+  const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
+  FX_AS1 uint8_t* flags = (FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * n_rows;
+  FX_AS1 uint32_t* counts =
+      (FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
+  const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
+  const uint32_t mask_vt = uni(w.cls[FX_W(FxClass, mask_vt)]);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) {
-    bool live = (M >> j) & 1u;
-    bool keep = live && (cl->mask_vt == FX_VT_F ? (u2f(A[j]) != 0.0f) : (A[j] != 0u));
+    const bool live = (M >> j) & 1u;
+    const bool keep = live && (mask_vt == FX_VT_F ? (u2f(A[j]) != 0.0f) : (A[j] != 0u));
     if (live) flags[row[j]] = keep ? 1 : 0;
-    uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+    const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
     if (lane == 0) s_wcnt[j][wave] = (uint32_t)__popcll(bal);
   }
   __syncthreads();
-  // one count per row tile: FX_BLOCK / rt tiles per j-slab
   const uint32_t waves_per_tile = rt / 64u;
   const uint32_t tiles_per_slab = FX_BLOCK / rt;
   if (threadIdx.x < FX_V * tiles_per_slab) {
-    uint32_t j = threadIdx.x / tiles_per_slab, t = threadIdx.x % tiles_per_slab;
-    uint32_t first_row = w.local_block * FX_TILE + j * FX_BLOCK + t * rt;
+    const uint32_t j = threadIdx.x / tiles_per_slab, t = threadIdx.x % tiles_per_slab;
+    const uint32_t first_row = w.local_block * FX_TILE + j * FX_BLOCK + t * rt;
     if (first_row < n_rows) {
       uint32_t s = 0;
       for (uint32_t k = 0; k < waves_per_tile; ++k) s += s_wcnt[j][t * waves_per_tile + k];
@@ -613,27 +631,26 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
 // The last tile of a task also publishes the task's total.
 // --------------------------------------------------------------------------
 template <int R>
-__global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* __restrict__ sb_, const FxDyn) {
-  extern __shared__ uint32_t s_temps[];
-  __shared__ uint64_t s_tp[FX_MAX_TPTR];
-  __shared__ uint32_t s_ts[FX_MAX_TSCAL];
+__global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* __restrict__ sb, const FxLaunch la,
+                                                               const FxDyn) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
   __shared__ uint32_t s_rowmap[FX_BLOCK];
   __shared__ uint32_t s_wsum[FX_BLOCK / 64];
   __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
   __shared__ uint32_t s_prefix;
+  fx_stage(L, sb, la);
+  const FxWork w = fx_locate<false>(L, blockIdx.x);
+  const FxCtx cx = fx_make_ctx(L, la, w);
 
-  fx_c32 sb = (fx_c32)sb_;
-  fx_chdr h = (fx_chdr)sb;
-  const FxWork w = fx_locate<false>(sb, blockIdx.x);
-  fx_ccls cl = w.cls;
-  fx_stage_task(h, w.task, s_tp, s_ts);
-
-  const uint32_t n_rows = cl->n_rows;
-  const uint32_t rt = h->row_tile;
+  const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
+  const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
+  const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
   const uint32_t tile = w.local_block;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint8_t* flags = (const uint8_t*)fx_dyn_p()[h->slot_flags] + (size_t)w.task * n_rows;
-  const uint32_t* counts = (const uint32_t*)fx_dyn_p()[h->slot_counts] + (size_t)w.task * h->max_rowtiles;
+  const FX_AS1 uint8_t* flags =
+      (const FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * n_rows;
+  const FX_AS1 uint32_t* counts =
+      (const FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
 
   // exclusive offset of this tile
   uint32_t part = 0;
@@ -660,32 +677,34 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   __syncthreads();
   if (keep) s_rowmap[s_woff[wave] + before] = row;
   __syncthreads();
-  const uint32_t n_kept = s_woff[FX_BLOCK / 64];
-  const uint32_t prefix = s_prefix;
-  if (tile + 1 == cl->n_rowtiles && threadIdx.x == 0) {
-    ((uint32_t*)fx_dyn_p()[h->slot_total])[w.task] = prefix + n_kept;
+  const uint32_t n_kept = uni(s_woff[FX_BLOCK / 64]);
+  const uint32_t prefix = uni(s_prefix);
+  if (tile + 1 == uni(w.cls[FX_W(FxClass, n_rowtiles)]) && threadIdx.x == 0) {
+    ((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])])[w.task] = prefix + n_kept;
   }
   if (n_kept == 0) return;
 
-  FxCtx cx;
-  cx.insn = (fx_cinsn)(sb + cl->off_insn);
-  cx.aff = (fx_caff)(sb + cl->off_aff);
-  cx.sptr = fx_dyn_p();
-  cx.tptr = s_tp;
-  cx.sscal = fx_dyn_s();
-  cx.tscal = s_ts;
-  cx.temps = s_temps + threadIdx.x;
-  cx.task = w.task;
-
-  fx_cout outs = (fx_cout)(sb + cl->off_outs);
-  for (uint32_t oi = 0; oi < cl->n_outs; ++oi) {
-    const FX_AS4 FxOut& od = outs[oi];
-    const uint32_t rowlen = od.rowlen;
+  const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
+  const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
+  const uint32_t ow = sizeof(FxOut) / 4;
+  for (uint32_t oi = 0; oi < n_outs; ++oi) {
+    const uint32_t* od = outs + oi * ow;
+    const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
+    const uint32_t rl_magic = od[FX_W(FxOut, rl_magic)], rl_shift = od[FX_W(FxOut, rl_shift)];
     const uint32_t n_el = n_kept * rowlen;
-    uint8_t* op = (uint8_t*)fx_ptr(cx, (int32_t)od.ptr_slot);
-    const int64_t obase = (int64_t)od.task_stride * w.task + (int64_t)prefix * rowlen;
+    const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
+    const int64_t obase = (int64_t)od[FX_W(FxOut, task_stride)] * w.task + (int64_t)prefix * rowlen;
+    const int pb = (int)uni(od[FX_W(FxOut, prog_begin)]), pe = (int)uni(od[FX_W(FxOut, prog_end)]);
+    const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
+    uint32_t dk[R], mk[R], sk[R];
+#pragma unroll
+    for (int k = 1; k < R; ++k) {
+      dk[k] = od[FX_W(FxOut, dim) + k];
+      mk[k] = od[FX_W(FxOut, magic) + k];
+      sk[k] = od[FX_W(FxOut, shift) + k];
+    }
     for (uint32_t it = 0; it < n_el; it += FX_TILE) {
-      int32_t c[FX_V][R > 0 ? R : 1];
+      int32_t c[FX_V][R];
       uint32_t M = 0;
       uint32_t e[FX_V];
 #pragma unroll
@@ -693,27 +712,23 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         e[j] = it + j * FX_BLOCK + threadIdx.x;
         const bool live = e[j] < n_el;
         if (live) M |= 1u << j;
-        uint32_t r = fx_fastdiv(e[j], od.rl_magic, od.rl_shift);
+        const uint32_t r = fx_fastdiv(e[j], rl_magic, rl_shift);
         uint32_t col = e[j] - r * rowlen;
-        // inner coordinates from col, coordinate 0 from the row map
-        int32_t cc[R > 0 ? R : 1];
 #pragma unroll
         for (int k = R - 1; k >= 1; --k) {
-          uint32_t q = fx_fastdiv(col, od.magic[k], od.shift[k]);
-          cc[k] = (int32_t)(col - q * od.dim[k]);
+          const uint32_t q = fx_fastdiv(col, mk[k], sk[k]);
+          c[j][k] = (int32_t)(col - q * dk[k]);
           col = q;
         }
-        cc[0] = live ? (int32_t)s_rowmap[r] : 0;
-#pragma unroll
-        for (int k = 0; k < R; ++k) c[j][k] = cc[k];
+        c[j][0] = live ? (int32_t)s_rowmap[r] : 0;
       }
       uint32_t A[FX_V];
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) A[j] = 0;
-      fx_run<R>(cx, (int)od.prog_begin, (int)od.prog_end, c, M, A);
+      fx_run<R>(cx, pb, pe, c, M, A);
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
-        if ((M >> j) & 1u) fx_store(op, obase + e[j], od.dtype, od.vt, A[j]);
+        if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
       }
     }
   }
@@ -855,39 +870,55 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_copy_f4(const float4* __restrict_
 // host-callable launchers (C++ linkage inside the library; the C ABI is in
 // fx_api.cpp)
 // --------------------------------------------------------------------------
-extern "C++" {
+static FxLaunch make_launch(const FxLaunchInfo& li) {
+  FxLaunch la;
+  la.blob_words = li.blob_words;
+  la.n_p = li.n_p;
+  la.n_s = li.n_s;
+  la.temps_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
+  return la;
+}
 
-hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+uint32_t fx_lds_bytes(const FxLaunchInfo& li) {
+  FxLaunch la = make_launch(li);
+  return (la.temps_off + li.n_temps * FX_V * FX_BLOCK) * 4u;
+}
+
+hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                            hipStream_t stream) {
   if (grid == 0) return hipSuccess;
+  const FxLaunch la = make_launch(li);
+  const uint32_t lds = fx_lds_bytes(li);
   switch (rank) {
     case 0:
-    case 1: fx_region_dense<1><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 2: fx_region_dense<2><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 3: fx_region_dense<3><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 4: fx_region_dense<4><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    default: fx_region_dense<FX_MAXR><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 1: fx_region_dense<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 2: fx_region_dense<2><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 3: fx_region_dense<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 4: fx_region_dense<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    default: fx_region_dense<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
   }
   return hipGetLastError();
 }
 
-hipError_t fx_launch_compact_count(const uint32_t* sb, const FxDyn* dyn, uint32_t grid, uint32_t lds_bytes,
+hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                                    hipStream_t stream) {
   if (grid == 0) return hipSuccess;
-  fx_compact_count<<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn);
+  fx_compact_count<<<grid, FX_BLOCK, fx_lds_bytes(li), stream>>>(sb, make_launch(li), *dyn);
   return hipGetLastError();
 }
 
-hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxDyn* dyn, uint32_t grid,
-                                     uint32_t lds_bytes, hipStream_t stream) {
+hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
+                                     uint32_t grid, hipStream_t stream) {
   if (grid == 0) return hipSuccess;
+  const FxLaunch la = make_launch(li);
+  const uint32_t lds = fx_lds_bytes(li);
   switch (rank) {
     case 0:
-    case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 2: fx_compact_scatter<2><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 3: fx_compact_scatter<3><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    case 4: fx_compact_scatter<4><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
-    default: fx_compact_scatter<FX_MAXR><<<grid, FX_BLOCK, lds_bytes, stream>>>(sb, *dyn); break;
+    case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 2: fx_compact_scatter<2><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 3: fx_compact_scatter<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 4: fx_compact_scatter<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    default: fx_compact_scatter<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
   }
   return hipGetLastError();
 }
@@ -920,4 +951,3 @@ hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t gri
   return hipGetLastError();
 }
 
-}  // extern "C++"

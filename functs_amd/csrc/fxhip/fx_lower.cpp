@@ -327,6 +327,9 @@ class Lowerer {
     return (int)d;
   }
   void sliceBounds(int vid_start, int vid_end, int64_t size, int64_t* start, int64_t* end);
+  // start as an index expression (may depend on the task index / loop variable) and the
+  // number of positions covered before stepping
+  bool sliceDynamic(int vid_start, int vid_end, IdxExpr* start, int64_t* extent);
 };
 
 // ---------------------------------------------------------------------------
@@ -413,6 +416,21 @@ void Lowerer::sliceBounds(int vid_start, int vid_end, int64_t size, int64_t* sta
   *end = e;
 }
 
+// A slice whose bounds move with the task index or the collapsed loop variable
+// (x[i:i+1] inside a ParallelMap): start stays symbolic, end - start must be a
+// constant, and no clamping is applied (the bounds are assumed in range, as the
+// FAIT lowering does, custom_lowering_func.cpp:458-470).
+bool Lowerer::sliceDynamic(int vid_start, int vid_end, IdxExpr* start, int64_t* extent) {
+  if (isNone(vid_start) || isNone(vid_end)) return false;
+  IdxExpr s = intOf(vid_start), e = intOf(vid_end);
+  if (s.isConst() && e.isConst()) return false;
+  IdxExpr d = e - s;
+  FX_CHECK(d.isConst(), FX_E_UNSUPPORTED, "slice with task-dependent bounds needs a constant length");
+  *start = s;
+  *extent = std::max<int64_t>(d.k, 0);
+  return true;
+}
+
 // ---------------------------------------------------------------------------
 // shape functions (fait/fuser/shape_func.cpp:9-374)
 // ---------------------------------------------------------------------------
@@ -456,8 +474,11 @@ Shape Lowerer::shapeOf(int vid) {
       case FX_OP_SLICE: {
         s = shapeOf(arg(0));
         int d = normDim(constIntOf(arg(1), "slice"), (int64_t)s.size(), "slice");
-        int64_t st, en;
-        sliceBounds(arg(2), arg(3), s[d], &st, &en);
+        int64_t st = 0, en = 0;
+        IdxExpr dst;
+        int64_t ext;
+        if (sliceDynamic(arg(2), arg(3), &dst, &ext)) en = ext;
+        else sliceBounds(arg(2), arg(3), s[d], &st, &en);
         int64_t step = constIntOf(arg(4), "slice step");
         FX_CHECK(step > 0, FX_E_INVALID, "slice step must be positive");
         s[d] = (en - st + step - 1) / step;
@@ -511,7 +532,8 @@ Shape Lowerer::shapeOf(int vid) {
       case FX_OP_REPEAT: {
         Shape in = shapeOf(arg(0));
         auto rep = intListOf(arg(1), "repeat");
-        FX_CHECK(rep.size() >= in.size(), FX_E_INVALID, "repeat: rank");
+        // missing leading repeats count as 1 (computeRepeatShape, shape_func.cpp:206-230)
+        while (rep.size() < in.size()) rep.insert(rep.begin(), 1);
         s.resize(rep.size());
         for (size_t i = 0; i < rep.size(); ++i) {
           int64_t ii = (int64_t)i - (int64_t)(rep.size() - in.size());
@@ -585,7 +607,7 @@ int Lowerer::addAffine(const IdxExpr& e) {
              "index arithmetic exceeds 32 bits (tensors above 2^31 elements are not supported)");
     return (int32_t)x;
   };
-  for (int i = 0; i < FX_MAXR; ++i) a.coef[i] = fit(e.c[i]);
+  for (int i = 0; i < FX_MAXR; ++i) fx_aff_set_coef(&a, i, fit(e.c[i]));
   for (int i = 0; i < FX_MAXLOOP; ++i) a.rcoef[i] = fit(e.rc[i]);
   a.tcoef = fit(e.ct);
   a.base = fit(e.k);
@@ -760,9 +782,15 @@ Lowerer::Res Lowerer::resolve(int vid, Frame f) {
         Shape s = shapeOf(arg(0));
         int d = normDim(constIntOf(arg(1), "slice"), (int64_t)s.size(), "slice");
         int64_t st, en;
-        sliceBounds(arg(2), arg(3), s[d], &st, &en);
         int64_t step = constIntOf(arg(4), "slice step");
-        f[d] = f[d] * step + IdxExpr(st);
+        IdxExpr dst;
+        int64_t ext;
+        if (sliceDynamic(arg(2), arg(3), &dst, &ext)) {
+          f[d] = f[d] * step + dst;
+        } else {
+          sliceBounds(arg(2), arg(3), s[d], &st, &en);
+          f[d] = f[d] * step + IdxExpr(st);
+        }
         vid = arg(0);
         continue;
       }
@@ -1752,8 +1780,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
   P->grid = gb;
   P->grid_count = gc;
   P->max_rank = max_rank;
-  P->lds_bytes = (uint32_t)max_temps * FX_V * FX_BLOCK * 4;
-  FX_CHECK(P->lds_bytes <= 96 * 1024, FX_E_LIMIT, "region needs too many temporaries for LDS");
+  P->n_temps = (uint32_t)max_temps;
 
   // slot budget
   P->sptr = slots.sptr;
@@ -1819,7 +1846,8 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     while (blob.size() % 4) blob.push_back(0);
     cb.cls.off_insn = (uint32_t)blob.size();
     for (auto& i : cb.code) appendStruct(blob, i);
-    while (blob.size() % 16) blob.push_back(0);
+    { FxInsn nop; memset(&nop, 0, sizeof(nop)); appendStruct(blob, nop); }  // look-ahead pad
+    while (blob.size() % 4) blob.push_back(0);
     cb.cls.off_aff = (uint32_t)blob.size();
     for (auto& a : cb.affs) appendStruct(blob, a);
     while (blob.size() % 4) blob.push_back(0);
@@ -1843,6 +1871,11 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
   hp->off_taskmap = off_taskmap;
   hp->total_words = (uint32_t)blob.size();
 
+  P->lds_bytes = (uint32_t)((blob.size() + 2 * (P->sptr.size() + P->tptr.size() * (size_t)T) +
+                             (P->sscal.size() + P->tscal.size() * (size_t)T) + 4 +
+                             (size_t)max_temps * FX_V * FX_BLOCK) * 4);
+  FX_CHECK(P->lds_bytes <= 64 * 1024, FX_E_LIMIT,
+           "region descriptor + temporaries need " << P->lds_bytes << " bytes of LDS (limit 65536)");
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;
@@ -1888,7 +1921,7 @@ std::string disasm(const Plan& p) {
         if (x.op == FX_LDA || x.op == FX_LDB || x.op == FX_AFFA || x.op == FX_AFFB) {
           const FxAffine& a = aff[x.b];
           o << "  [";
-          for (int k = 0; k < FX_MAXR; ++k) o << a.coef[k] << (k + 1 < FX_MAXR ? "," : "");
+          for (int k = 0; k < FX_MAXR; ++k) o << fx_aff_coef(&a, k) << (k + 1 < FX_MAXR ? "," : "");
           o << "] t=" << a.tcoef << " r=" << a.rcoef[0] << "," << a.rcoef[1] << " base=" << a.base;
         }
         o << "\n";

@@ -311,6 +311,19 @@ class BoundCall:
                                 self.totals.data_ptr() if self.totals is not None else None,
                                 ctypes.c_void_p(stream)))
 
+    def launch_timed(self, stream=None):
+        """launch() with HIP events around every kernel; returns the list of
+        kernel durations in milliseconds (synchronises)."""
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+        ms = (ctypes.c_float * 4)()
+        nk = ctypes.c_int()
+        check(lib.fx_region_run_timed(self.region._h, self.plan.handle, self.arr, self.n, self.ptrs,
+                                      self.scratch.data_ptr() if self.scratch is not None else None,
+                                      self.totals.data_ptr() if self.totals is not None else None,
+                                      ctypes.c_void_p(stream), ms, 4, ctypes.byref(nk)))
+        return [ms[i] for i in range(nk.value)]
+
     def results(self):
         """Outputs as the operator returns them: a tensor per output, or a list
         of per-task tensors for a ParallelMap.  Compacted outputs are narrowed to

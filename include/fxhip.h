@@ -175,6 +175,15 @@ int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);
 int fx_region_run(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
                   void* scratch, uint32_t* totals_host, void* stream);
 
+/* fx_region_run with a HIP event pair around every kernel on `stream`; waits for
+ * the last event and returns the duration of each launch in milliseconds
+ * (kernel_ms[0..*n_kernels), order of launch: [count, scatter] for compacting
+ * regions, [dense] otherwise).  Measurement aid of the benchmark; the reference
+ * measures with CUPTI activity records instead (fait/util/profile.cpp:29-46). */
+int fx_region_run_timed(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
+                        void* scratch, uint32_t* totals_host, void* stream, float* kernel_ms, int cap,
+                        int* n_kernels);
+
 /* The argument marshalling of fx_region_run without the launch (host only; the
  * analogue of GraphBuilder::prepareRunArgs, graph_builder.cpp:718-899).
  * dyn_out receives fx_dyn_bytes() bytes: the by-value block the kernels read. */

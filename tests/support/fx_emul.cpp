@@ -111,7 +111,7 @@ uint32_t run(const Ctx& cx, int pc, int pc_end, const int32_t* c) {
         if (!M) break;
         const FxAffine& af = cx.aff[ins.b];
         int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
-        for (int k = 0; k < FX_MAXR; ++k) off += af.coef[k] * c[k];
+        for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
         bool is_load = ins.op == FX_LDA || ins.op == FX_LDB;
         uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt) : (uint32_t)off;
         if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);

@@ -347,6 +347,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
   li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
   li.n_temps = pl->n_temps;
+  li.stage_words = pl->stage_words;
   if (pl->mode == FX_MODE_COMPACT) {
     // tasks without rows launch no tile: their total is published here.  The
     // caller must not reuse totals_host while an earlier run is still in flight.

@@ -19,6 +19,7 @@
 #define FX_V 4           // elements per lane
 #define FX_BLOCK 256     // threads per workgroup (4 wavefronts of 64)
 #define FX_TILE (FX_V * FX_BLOCK)
+#define FX_ITEM (FX_V * 64)  // elements one wave processes per work item
 #define FX_MAX_TEMPS 24  // LDS temp slots per lane (each FX_V wide)
 #define FX_MASK_DEPTH 16 // nesting depth of predicated regions (4 bits each in a u64)
 #define FX_DYN_P 320     // 8-byte dynamic words passed by value (pointers)
@@ -82,6 +83,9 @@ enum FxOp : uint32_t {
   FX_RBEGIN, // push loop: counter = 0, extent = imm, acc slot = temp[a] preset by program
   FX_RNEXT,  // counter += 1; if counter < extent jump to a
   FX_RIDX,   // A = (int) loop counter of depth a
+  // ---- loads from an input tile staged in LDS (row-tiled kernels) ----
+  FX_LDSA,   // A = stage[a] at affine[b](coords) relative to the tile; dt = storage dtype
+  FX_LDSB,
   FX_OP_COUNT
 };
 
@@ -119,6 +123,7 @@ struct FxLaunchInfo {
   uint32_t n_p;         // pointer slots in use
   uint32_t n_s;         // scalar slots in use
   uint32_t n_temps;     // LDS temp slots per lane
+  uint32_t stage_words; // LDS words of the largest per-tile stage area (multiple of 4)
 };
 
 #define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table
@@ -138,6 +143,19 @@ struct FxOut {
   uint32_t rowlen;                // compaction: elements per row (numel / dim[0])
   uint32_t rl_magic, rl_shift;    // fast division by rowlen
   uint32_t vt;                    // FxVt of the program result
+  uint32_t colmajor;              // compaction: iterate (column, row chunk) instead of flat elements
+  uint32_t pad[2];
+};
+
+// An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows
+// [r0, r0 + row_tile) of a tile are one contiguous run of S * row_tile elements,
+// copied to LDS with 128-bit loads before the programs run.
+struct FxStage {
+  uint32_t ptr_slot;   // may carry FX_SLOT_TASK
+  uint32_t row_elems;  // S
+  int32_t tcoef;       // element offset per task (shared buffer sliced by the task index)
+  uint32_t lds_off;    // word offset inside the stage area
+  uint32_t n_rows;     // rows of the buffer along coordinate 0 (clamps the last tile)
   uint32_t pad[3];
 };
 
@@ -158,7 +176,8 @@ struct FxClass {
   uint32_t mask_vt;
   uint32_t cnt_block_begin, cnt_block_end;  // grid range in the count pass
   uint32_t cnt_blocks_per_task;
-  uint32_t pad[2];
+  uint32_t n_stages;                // staged inputs (FxStage[n_stages] at off_stages)
+  uint32_t off_stages;
 };
 
 enum FxMode : uint32_t { FX_MODE_DENSE = 0, FX_MODE_COMPACT = 1 };
@@ -175,6 +194,8 @@ struct FxHeader {
   uint32_t max_rowtiles; // stride of the per-task tile-count table
   uint32_t slot_flags, slot_counts, slot_total;  // shared pointer slots used by compaction
   uint32_t total_words;
+  uint32_t max_rows;     // stride of the per-task row-flag table
+  uint32_t pad[3];
 };
 
 // dynamic (per call) arguments, passed by value in the kernarg segment

@@ -54,6 +54,8 @@ struct FxCtx {
   uint32_t tp_off;        // index of this task's first pointer
   uint32_t ts_off;        // index of this task's first scalar
   uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
+  const uint32_t* stage;  // LDS: input tiles staged by the row-tiled kernels
+  const int32_t* stage_adj;  // LDS: per stage, word index of element 0 of the buffer (may be negative)
   int task;
 };
 
@@ -226,6 +228,32 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
             uint32_t v = is_load ? fx_load(p, (int64_t)off, dt) : (uint32_t)off;
             if (cvt) v = f2u((float)(int32_t)v);
             if (op == FX_LDA || op == FX_AFFA) A[j] = v; else B[j] = v;
+          }
+        }
+      } break;
+      case FX_LDSA:
+      case FX_LDSB: {
+        const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + ib * FX_AFF_WORDS);
+        const fx_u32x4 a0 = ap[0], a1 = ap[1];
+        int32_t cf[FX_MAXR];
+        cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
+        if (R > 4) {
+          const fx_u32x4 a2 = ap[2];
+          cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
+        } else {
+          cf[4] = 0; cf[5] = 0;
+        }
+        // the task term is part of the tile's global origin, not of the LDS index
+        const int32_t base = (int32_t)a1.y + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1 + cx.stage_adj[ia];
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          if ((M >> j) & 1u) {
+            int32_t off = base;
+#pragma unroll
+            for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
+            uint32_t v = cx.stage[off];
+            if (cvt) v = f2u((float)(int32_t)v);
+            if (op == FX_LDSA) A[j] = v; else B[j] = v;
           }
         }
       } break;
@@ -439,8 +467,11 @@ struct FxLaunch {
   uint32_t blob_words;  // multiple of 4
   uint32_t n_p;         // pointers in use in FxDyn::p
   uint32_t n_s;         // scalars in use in FxDyn::s
+  uint32_t stage_off;   // word offset of the stage area in LDS (multiple of 4)
   uint32_t temps_off;   // word offset of the temp area in LDS (multiple of 4)
+  uint32_t pad;
 };
+#define FX_MAX_STAGES 8
 #define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
 
 __device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict__ sb, const FxLaunch& la) {
@@ -496,8 +527,48 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
   cx.tp_off = n_sptr + (uint32_t)w.task * n_tptr;
   cx.ts_off = n_sscal + (uint32_t)w.task * n_tscal;
   cx.temps = L + la.temps_off + threadIdx.x;
+  cx.stage = L + la.stage_off;
+  cx.stage_adj = nullptr;
   cx.task = w.task;
   return cx;
+}
+
+// Copy rows [r0, r0 + rows) of every staged input of this class into LDS.
+// 128-bit loads wherever the 16-byte group lies inside the tile; the (at most
+// two) partial groups at the ends are read element-wise, so nothing outside
+// the tile is touched whatever the alignment of the buffer.
+__device__ __forceinline__ void fx_stage_tiles(uint32_t* L, const FxLaunch& la, const FxWork& w, const FxCtx& cx,
+                                               uint32_t r0, uint32_t rt, int32_t* s_adj) {
+  const uint32_t n_stages = uni(w.cls[FX_W(FxClass, n_stages)]);
+  const uint32_t* st = L + uni(w.cls[FX_W(FxClass, off_stages)]);
+  uint32_t* area = L + la.stage_off;
+  for (uint32_t s = 0; s < n_stages; ++s) {
+    const uint32_t* d = st + s * (sizeof(FxStage) / 4);
+    const uint32_t S = uni(d[FX_W(FxStage, row_elems)]);
+    const int32_t tcoef = (int32_t)uni(d[FX_W(FxStage, tcoef)]);
+    const uint32_t lds_off = uni(d[FX_W(FxStage, lds_off)]);
+    const uint32_t n_rows = uni(d[FX_W(FxStage, n_rows)]);
+    const uint32_t rows = (r0 + rt <= n_rows) ? rt : (n_rows > r0 ? n_rows - r0 : 0u);
+    const uint32_t count = rows * S;
+    const int64_t g0 = (int64_t)S * r0 + (int64_t)tcoef * w.task;
+    const uint64_t p = fx_ptr(cx, (int32_t)d[FX_W(FxStage, ptr_slot)]) + (uint64_t)(g0 * 4);
+    const uint32_t mis = (uint32_t)((p >> 2) & 3ull);
+    const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(p - 4ull * mis);
+    const FX_AS1 uint32_t* g1 = (const FX_AS1 uint32_t*)(p - 4ull * mis);
+    const uint32_t n4 = (mis + count + 3u) >> 2;
+    uint32_t* dst = area + lds_off;
+    for (uint32_t i = threadIdx.x; i < n4; i += FX_BLOCK) {
+      const uint32_t e = i * 4u;  // index in the aligned view; tile elements are [mis, mis + count)
+      if (e >= mis && e + 4u <= mis + count) {
+        *(fx_u32x4*)(dst + e) = g4[i];
+      } else {
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; ++k)
+          if (e + k >= mis && e + k < mis + count) dst[e + k] = g1[e + k];
+      }
+    }
+    if (threadIdx.x == 0) s_adj[s] = (int32_t)(lds_off + mis) - (int32_t)(S * r0);
+  }
 }
 
 }  // namespace
@@ -594,7 +665,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
   fx_run<1>(cx, (int)uni(w.cls[FX_W(FxClass, mask_begin)]), (int)uni(w.cls[FX_W(FxClass, mask_end)]), c, M, A);
 
   const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
-  FX_AS1 uint8_t* flags = (FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * n_rows;
+  FX_AS1 uint8_t* flags = (FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * uni(L[FX_W(FxHeader, max_rows)]);
   FX_AS1 uint32_t* counts =
       (FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
   const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
@@ -638,17 +709,21 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   __shared__ uint32_t s_wsum[FX_BLOCK / 64];
   __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
   __shared__ uint32_t s_prefix;
+  __shared__ int32_t s_adj[FX_MAX_STAGES];
   fx_stage(L, sb, la);
   const FxWork w = fx_locate<false>(L, blockIdx.x);
-  const FxCtx cx = fx_make_ctx(L, la, w);
+  FxCtx cx = fx_make_ctx(L, la, w);
+  cx.stage_adj = s_adj;
 
   const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
   const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
+  // input tiles -> LDS (completed by the barriers of the row-map construction below)
+  fx_stage_tiles(L, la, w, cx, w.local_block * rt, rt, s_adj);
   const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
   const uint32_t tile = w.local_block;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const FX_AS1 uint8_t* flags =
-      (const FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * n_rows;
+      (const FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * uni(L[FX_W(FxHeader, max_rows)]);
   const FX_AS1 uint32_t* counts =
       (const FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
 
@@ -687,11 +762,20 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
   const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
   const uint32_t ow = sizeof(FxOut) / 4;
+  // Work items of FX_ITEM elements are dealt to the four waves round-robin over
+  // ALL outputs of the tile, so that a long program of a narrow output (a few
+  // items) overlaps with the short programs of the wide ones instead of
+  // serialising the whole workgroup behind it.  No barrier from here on.
+  const uint32_t wave_u = uni(wave);
+  uint32_t item_base = 0;
   for (uint32_t oi = 0; oi < n_outs; ++oi) {
     const uint32_t* od = outs + oi * ow;
     const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
+    const uint32_t colmajor = uni(od[FX_W(FxOut, colmajor)]);
     const uint32_t rl_magic = od[FX_W(FxOut, rl_magic)], rl_shift = od[FX_W(FxOut, rl_shift)];
     const uint32_t n_el = n_kept * rowlen;
+    const uint32_t chunks = (n_kept + FX_ITEM - 1) / FX_ITEM;   // row chunks per column (column-major)
+    const uint32_t n_items = colmajor ? rowlen * chunks : (n_el + FX_ITEM - 1) / FX_ITEM;
     const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
     const int64_t obase = (int64_t)od[FX_W(FxOut, task_stride)] * w.task + (int64_t)prefix * rowlen;
     const int pb = (int)uni(od[FX_W(FxOut, prog_begin)]), pe = (int)uni(od[FX_W(FxOut, prog_end)]);
@@ -703,17 +787,31 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
       mk[k] = od[FX_W(FxOut, magic) + k];
       sk[k] = od[FX_W(FxOut, shift) + k];
     }
-    for (uint32_t it = 0; it < n_el; it += FX_TILE) {
+    // first item of this output that belongs to this wave
+    uint32_t it = (wave_u + 4u - (item_base & 3u)) & 3u;
+    for (; it < n_items; it += 4u) {
       int32_t c[FX_V][R];
       uint32_t M = 0;
       uint32_t e[FX_V];
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
-        e[j] = it + j * FX_BLOCK + threadIdx.x;
-        const bool live = e[j] < n_el;
+        uint32_t r, col;
+        bool live;
+        if (colmajor) {
+          // all lanes of the item share one column: predicates on the inner
+          // coordinate are wave-uniform and whole branches get skipped
+          const uint32_t cc = it / chunks, ch = it - cc * chunks;
+          r = ch * FX_ITEM + j * 64u + lane;
+          col = cc;
+          live = r < n_kept;
+          e[j] = r * rowlen + col;
+        } else {
+          e[j] = it * FX_ITEM + j * 64u + lane;
+          live = e[j] < n_el;
+          r = fx_fastdiv(e[j], rl_magic, rl_shift);
+          col = e[j] - r * rowlen;
+        }
         if (live) M |= 1u << j;
-        const uint32_t r = fx_fastdiv(e[j], rl_magic, rl_shift);
-        uint32_t col = e[j] - r * rowlen;
 #pragma unroll
         for (int k = R - 1; k >= 1; --k) {
           const uint32_t q = fx_fastdiv(col, mk[k], sk[k]);
@@ -731,6 +829,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
       }
     }
+    item_base += n_items;
   }
 }
 
@@ -875,7 +974,9 @@ static FxLaunch make_launch(const FxLaunchInfo& li) {
   la.blob_words = li.blob_words;
   la.n_p = li.n_p;
   la.n_s = li.n_s;
-  la.temps_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
+  la.stage_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
+  la.temps_off = la.stage_off + li.stage_words;
+  la.pad = 0;
   return la;
 }
 

@@ -348,6 +348,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
   li.n_temps = pl->n_temps;
   li.stage_words = pl->stage_words;
+  li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
   if (pl->mode == FX_MODE_COMPACT) {
     // tasks without rows launch no tile: their total is published here.  The
     // caller must not reuse totals_host while an earlier run is still in flight.
@@ -362,7 +363,8 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(ev[i], stream) : hipSuccess; };
   if (pl->mode == FX_MODE_DENSE) {
     HIP_OK(mark(0));
-    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, pl->grid, stream));
+    // persistent workgroups: at most 8 per CU worth of blocks stride over the units
+    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
   } else {

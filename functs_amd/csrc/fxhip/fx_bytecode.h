@@ -20,6 +20,7 @@
 #define FX_BLOCK 256     // threads per workgroup (4 wavefronts of 64)
 #define FX_TILE (FX_V * FX_BLOCK)
 #define FX_ITEM (FX_V * 64)  // elements one wave processes per work item
+#define FX_UNIT (16 * FX_ITEM)  // dense kernel: elements of the largest work unit (4 waves x 4 items)
 #define FX_MAX_TEMPS 24  // LDS temp slots per lane (each FX_V wide)
 #define FX_MASK_DEPTH 16 // nesting depth of predicated regions (4 bits each in a u64)
 #define FX_DYN_P 320     // 8-byte dynamic words passed by value (pointers)
@@ -124,6 +125,7 @@ struct FxLaunchInfo {
   uint32_t n_s;         // scalar slots in use
   uint32_t n_temps;     // LDS temp slots per lane
   uint32_t stage_words; // LDS words of the largest per-tile stage area (multiple of 4)
+  uint32_t total_units; // dense kernel: number of FX_UNIT work units
 };
 
 #define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table
@@ -144,7 +146,8 @@ struct FxOut {
   uint32_t rl_magic, rl_shift;    // fast division by rowlen
   uint32_t vt;                    // FxVt of the program result
   uint32_t colmajor;              // compaction: iterate (column, row chunk) instead of flat elements
-  uint32_t pad[2];
+  uint32_t lead;                  // program starts with an unconditional affine load (batched by the kernels)
+  uint32_t unit_items;            // dense: items per wave and work unit (1 or FX_K)
 };
 
 // An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows

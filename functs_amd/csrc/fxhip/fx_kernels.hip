@@ -61,48 +61,56 @@ struct FxCtx {
 
 // Data buffers are plain device allocations: address them through the global
 // address space (global_load / global_store instead of flat accesses).
-__device__ __forceinline__ uint32_t fx_load(uint64_t base_, int64_t off, uint32_t dt) {
+// `base_` is wave-uniform (kept in SGPRs by the callers) and `off` is an
+// element index below 2^31 / element size: the access is base + 32-bit byte
+// offset, which needs no 64-bit vector arithmetic.
+__device__ __forceinline__ uint32_t fx_load(uint64_t base_, int32_t off, uint32_t dt) {
   const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
+  const uint32_t o = (uint32_t)off;
   switch (dt) {
-    case FX_F32: return ((const FX_AS1 uint32_t*)base)[off];
-    case FX_I32: return ((const FX_AS1 uint32_t*)base)[off];
-    case FX_I64: return (uint32_t)((const FX_AS1 uint64_t*)base)[off];
-    case FX_U8: return base[off];
+    case FX_F32:
+    case FX_I32: return *(const FX_AS1 uint32_t*)(base + (o << 2));
+    case FX_I64: return (uint32_t)*(const FX_AS1 uint64_t*)(base + (o << 3));
+    case FX_U8: return base[o];
     case FX_F16: {
-      uint16_t h = ((const FX_AS1 uint16_t*)base)[off];
+      uint16_t h = *(const FX_AS1 uint16_t*)(base + (o << 1));
       __half hv = __ushort_as_half(h);
       return f2u(__half2float(hv));
     }
-    case FX_BF16: return ((uint32_t)((const FX_AS1 uint16_t*)base)[off]) << 16;
+    case FX_BF16: return ((uint32_t)*(const FX_AS1 uint16_t*)(base + (o << 1))) << 16;
     default: return 0;
   }
 }
 
-__device__ __forceinline__ void fx_store(uint64_t base_, int64_t off, uint32_t dt, uint32_t vt, uint32_t v) {
+__device__ __forceinline__ void fx_store(uint64_t base_, uint32_t o, uint32_t dt, uint32_t vt, uint32_t v) {
   FX_AS1 uint8_t* base = (FX_AS1 uint8_t*)base_;
   switch (dt) {
-    case FX_F32: ((FX_AS1 uint32_t*)base)[off] = (vt == FX_VT_F) ? v : f2u((float)(int32_t)v); break;
-    case FX_I32: ((FX_AS1 int32_t*)base)[off] = (vt == FX_VT_I) ? (int32_t)v : (int32_t)u2f(v); break;
-    case FX_I64: ((FX_AS1 int64_t*)base)[off] = (vt == FX_VT_I) ? (int64_t)(int32_t)v : (int64_t)u2f(v); break;
-    case FX_U8: base[off] = (vt == FX_VT_I) ? (uint8_t)v : (uint8_t)(u2f(v) != 0.0f); break;
+    case FX_F32: *(FX_AS1 uint32_t*)(base + (o << 2)) = (vt == FX_VT_F) ? v : f2u((float)(int32_t)v); break;
+    case FX_I32: *(FX_AS1 int32_t*)(base + (o << 2)) = (vt == FX_VT_I) ? (int32_t)v : (int32_t)u2f(v); break;
+    case FX_I64:
+      *(FX_AS1 int64_t*)(base + (o << 3)) = (vt == FX_VT_I) ? (int64_t)(int32_t)v : (int64_t)u2f(v);
+      break;
+    case FX_U8: base[o] = (vt == FX_VT_I) ? (uint8_t)v : (uint8_t)(u2f(v) != 0.0f); break;
     case FX_F16: {
       __half hv = __float2half(vt == FX_VT_F ? u2f(v) : (float)(int32_t)v);
-      ((FX_AS1 uint16_t*)base)[off] = __half_as_ushort(hv);
+      *(FX_AS1 uint16_t*)(base + (o << 1)) = __half_as_ushort(hv);
     } break;
     case FX_BF16: {
       float f = vt == FX_VT_F ? u2f(v) : (float)(int32_t)v;
       uint32_t u = f2u(f);
       uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
       if (f != f) r = 0x7fc0u;
-      ((FX_AS1 uint16_t*)base)[off] = (uint16_t)r;
+      *(FX_AS1 uint16_t*)(base + (o << 1)) = (uint16_t)r;
     } break;
     default: break;
   }
 }
 
+// wave-uniform buffer pointer, returned in scalar registers
 __device__ __forceinline__ uint64_t fx_ptr(const FxCtx& cx, int32_t slot) {
   const uint32_t i = (slot & FX_SLOT_TASK) ? cx.tp_off + (uint32_t)(slot & 0xffff) : (uint32_t)(slot & 0xffff);
-  return cx.ptrs[i];
+  const uint64_t p = cx.ptrs[i];
+  return ((uint64_t)uni((uint32_t)(p >> 32)) << 32) | (uint64_t)uni((uint32_t)p);
 }
 
 __device__ __forceinline__ uint32_t fx_scalar(const FxCtx& cx, int32_t slot) {
@@ -121,6 +129,21 @@ __device__ __forceinline__ int32_t pymod_i(int32_t a, int32_t b) {
   int32_t r = a % b;
   if (r != 0 && ((r < 0) != (b < 0))) r += b;
   return r;
+}
+
+// sigmoid(x) = 1 / (1 + 2^(-x * log2 e)).  The product is split into a rounded
+// part and its rounding error (hi/lo of log2 e), the error is applied to the
+// result as a first-order factor, and the reciprocal is the hardware
+// approximation: about 3 ulp in total (3e-7 relative), against a 1e-5 bound,
+// for a quarter of the instructions of expf + IEEE division.
+__device__ __forceinline__ float fx_sigmoid(float x) {
+  const float l2e_hi = 1.44269502e+00f, l2e_lo = 1.92596299e-08f, ln2 = 6.93147182e-01f;
+  const float nx = -x;
+  const float th = nx * l2e_hi;
+  const float tl = __builtin_fmaf(nx, l2e_hi, -th) + nx * l2e_lo;
+  float e = __builtin_amdgcn_exp2f(th);
+  e = __builtin_fmaf(e, tl * ln2, e);
+  return __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // NaN-propagating min / max (ATen semantics for maximum/minimum/clamp)
@@ -219,15 +242,29 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
         const bool is_load = (op == FX_LDA || op == FX_LDB);
         const uint64_t p = is_load ? fx_ptr(cx, ia) : 0ull;
+        const bool toA = (op == FX_LDA || op == FX_AFFA);
+        if (!wave_any(M != VM)) {
+          // every element of the wave is live: no per-element predication
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) {
+          for (int j = 0; j < FX_V; ++j) {
             int32_t off = base;
 #pragma unroll
             for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
-            uint32_t v = is_load ? fx_load(p, (int64_t)off, dt) : (uint32_t)off;
+            uint32_t v = is_load ? fx_load(p, off, dt) : (uint32_t)off;
             if (cvt) v = f2u((float)(int32_t)v);
-            if (op == FX_LDA || op == FX_AFFA) A[j] = v; else B[j] = v;
+            if (toA) A[j] = v; else B[j] = v;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) {
+            if ((M >> j) & 1u) {
+              int32_t off = base;
+#pragma unroll
+              for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
+              uint32_t v = is_load ? fx_load(p, off, dt) : (uint32_t)off;
+              if (cvt) v = f2u((float)(int32_t)v);
+              if (toA) A[j] = v; else B[j] = v;
+            }
           }
         }
       } break;
@@ -261,7 +298,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         const uint64_t p = fx_ptr(cx, ia);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) A[j] = fx_load(p, (int64_t)((int32_t)A[j] + (int32_t)imm), dt);
+          if ((M >> j) & 1u) A[j] = fx_load(p, (int32_t)A[j] + (int32_t)imm, dt);
         }
       } break;
       case FX_IMMA:
@@ -339,7 +376,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
       case FX_SQRT: FX_UNARY_F(sqrtf(a));
       case FX_RSQRT: FX_UNARY_F(1.0f / sqrtf(a));
       case FX_RCP: FX_UNARY_F(1.0f / a);
-      case FX_SIGMOID: FX_UNARY_F(1.0f / (1.0f + expf(-a)));
+      case FX_SIGMOID: FX_UNARY_F(fx_sigmoid(a));
       case FX_TANH: FX_UNARY_F(tanhf(a));
       case FX_RELU: FX_UNARY_F((a <= 0.0f) ? 0.0f : a);
       case FX_FLOOR: FX_UNARY_F(floorf(a));
@@ -457,6 +494,44 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 #undef FX_BIN_I
 }
 
+// Programs that start with an unconditional affine load (flagged by the host in
+// FxOut::lead) have that load issued for FX_K work items at once, before any of
+// them is computed: FX_K * FX_V loads per lane are in flight instead of FX_V.
+// The interpreter then starts behind the load with A preset.
+#define FX_K 4
+template <int R>
+__device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const int32_t (&c)[FX_V][R], uint32_t M,
+                                             uint32_t (&P)[FX_V]) {
+  const fx_u32x4 w = cx.insn[pc];
+  const uint32_t w0 = uni(w.x);
+  const bool cvt = (w0 & (FX_F_I2F << 16)) != 0;
+  const uint32_t dt = w0 >> 24;
+  const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + (int32_t)w.z * FX_AFF_WORDS);
+  const fx_u32x4 a0 = ap[0], a1 = ap[1];
+  int32_t cf[FX_MAXR];
+  cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
+  if (R > 4) {
+    const fx_u32x4 a2 = ap[2];
+    cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
+  } else {
+    cf[4] = 0; cf[5] = 0;
+  }
+  const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task;
+  const uint64_t p = fx_ptr(cx, (int32_t)w.y);
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) {
+    P[j] = 0;
+    if ((M >> j) & 1u) {
+      int32_t off = base;
+#pragma unroll
+      for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
+      uint32_t v = fx_load(p, off, dt);
+      if (cvt) v = f2u((float)(int32_t)v);
+      P[j] = v;
+    }
+  }
+}
+
 __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint32_t shift) {
   return (__umulhi(n, magic) + n) >> shift;
 }
@@ -469,7 +544,7 @@ struct FxLaunch {
   uint32_t n_s;         // scalars in use in FxDyn::s
   uint32_t stage_off;   // word offset of the stage area in LDS (multiple of 4)
   uint32_t temps_off;   // word offset of the temp area in LDS (multiple of 4)
-  uint32_t pad;
+  uint32_t total_units; // dense: work units of FX_UNIT elements; the grid strides over them
 };
 #define FX_MAX_STAGES 8
 #define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
@@ -580,58 +655,87 @@ template <int R>
 __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __restrict__ sb, const FxLaunch la,
                                                             const FxDyn) {
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];
-  fx_stage(L, sb, la);
-  const FxWork w = fx_locate<false>(L, blockIdx.x);
-  const FxCtx cx = fx_make_ctx(L, la, w);
-
-  const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
-  const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
+  fx_stage(L, sb, la);   // once per workgroup; the loop below has no barrier
+  const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
   const uint32_t ow = sizeof(FxOut) / 4;
-  uint32_t oi = 0;
-  while (oi + 1 < n_outs &&
-         w.local_block >= uni(outs[oi * ow + FX_W(FxOut, block_begin)]) + uni(outs[oi * ow + FX_W(FxOut, n_blocks)]))
-    ++oi;
-  const uint32_t* od = outs + oi * ow;
-  const uint32_t tile = w.local_block - uni(od[FX_W(FxOut, block_begin)]);
-  const uint32_t numel = uni(od[FX_W(FxOut, numel)]);
 
-  int32_t c[FX_V][R];
-  uint32_t M = 0;
-  uint32_t e[FX_V];
+  // Persistent workgroups: work units of FX_UNIT elements (one output of one
+  // task each) are strided over the grid; inside a unit every wave owns FX_K
+  // consecutive items of FX_ITEM elements.
+  for (uint32_t unit = blockIdx.x; unit < la.total_units; unit += gridDim.x) {
+    const FxWork w = fx_locate<false>(L, unit);
+    const FxCtx cx = fx_make_ctx(L, la, w);
+    const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
+    const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
+    uint32_t oi = 0;
+    while (oi + 1 < n_outs && w.local_block >= uni(outs[oi * ow + FX_W(FxOut, block_begin)]) +
+                                                   uni(outs[oi * ow + FX_W(FxOut, n_blocks)]))
+      ++oi;
+    const uint32_t* od = outs + oi * ow;
+    const uint32_t ublock = w.local_block - uni(od[FX_W(FxOut, block_begin)]);
+    const uint32_t numel = uni(od[FX_W(FxOut, numel)]);
+    const int pb = (int)uni(od[FX_W(FxOut, prog_begin)]), pe = (int)uni(od[FX_W(FxOut, prog_end)]);
+    const uint32_t lead = uni(od[FX_W(FxOut, lead)]);
+    const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
+    const uint32_t obase = uni(od[FX_W(FxOut, task_stride)]) * (uint32_t)w.task;
+    const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
+    uint32_t dk[R], mk[R], sk[R];
 #pragma unroll
-  for (int j = 0; j < FX_V; ++j) {
-    e[j] = tile * FX_TILE + j * FX_BLOCK + threadIdx.x;
-    if (e[j] < numel) M |= 1u << j;
-  }
-  // flat index -> coordinates (row-major over dim[0..R))
-  {
-    uint32_t rem[FX_V];
-#pragma unroll
-    for (int j = 0; j < FX_V; ++j) rem[j] = e[j];
-#pragma unroll
-    for (int k = R - 1; k >= 1; --k) {
-      const uint32_t dk = od[FX_W(FxOut, dim) + k], mk = od[FX_W(FxOut, magic) + k], sk = od[FX_W(FxOut, shift) + k];
+    for (int k = 1; k < R; ++k) {
+      dk[k] = od[FX_W(FxOut, dim) + k];
+      mk[k] = od[FX_W(FxOut, magic) + k];
+      sk[k] = od[FX_W(FxOut, shift) + k];
+    }
+    // unit = 4 waves x kmax items; kmax is 1 for heavy or small outputs (more, smaller units)
+    const uint32_t kmax = uni(od[FX_W(FxOut, unit_items)]);
+    const uint32_t first = ublock * (4u * kmax * FX_ITEM) + wave * (kmax * FX_ITEM);
+    if (first >= numel) continue;
+
+    auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, int32_t (&c)[FX_V][R]) {
+      M = 0;
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
-        const uint32_t q = fx_fastdiv(rem[j], mk, sk);
-        c[j][k] = (int32_t)(rem[j] - q * dk);
-        rem[j] = q;
+        e[j] = first + k * FX_ITEM + j * 64u + lane;
+        if (e[j] < numel) M |= 1u << j;
+        uint32_t rem = e[j];
+#pragma unroll
+        for (int q = R - 1; q >= 1; --q) {
+          const uint32_t d = fx_fastdiv(rem, mk[q], sk[q]);
+          c[j][q] = (int32_t)(rem - d * dk[q]);
+          rem = d;
+        }
+        c[j][0] = (int32_t)rem;
+      }
+    };
+
+    uint32_t P[FX_K][FX_V];
+    if (lead) {
+#pragma unroll
+      for (uint32_t k = 0; k < FX_K; ++k) {
+        if (k < kmax && first + k * FX_ITEM < numel) {
+          uint32_t e[FX_V], M;
+          int32_t c[FX_V][R];
+          make_item(k, e, M, c);
+          fx_lead_load<R>(cx, pb, c, M, P[k]);
+        }
       }
     }
 #pragma unroll
-    for (int j = 0; j < FX_V; ++j) c[j][0] = (int32_t)rem[j];
-  }
-  uint32_t A[FX_V];
+    for (uint32_t k = 0; k < FX_K; ++k) {
+      if (k < kmax && first + k * FX_ITEM < numel) {
+        uint32_t e[FX_V], M;
+        int32_t c[FX_V][R];
+        make_item(k, e, M, c);
+        uint32_t A[FX_V];
 #pragma unroll
-  for (int j = 0; j < FX_V; ++j) A[j] = 0;
-  fx_run<R>(cx, (int)uni(od[FX_W(FxOut, prog_begin)]), (int)uni(od[FX_W(FxOut, prog_end)]), c, M, A);
-
-  const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
-  const int64_t obase = (int64_t)od[FX_W(FxOut, task_stride)] * w.task;
-  const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
+        for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
+        fx_run<R>(cx, lead ? pb + 1 : pb, pe, c, M, A);
 #pragma unroll
-  for (int j = 0; j < FX_V; ++j) {
-    if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
+        for (int j = 0; j < FX_V; ++j) {
+          if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
+        }
+      }
+    }
   }
 }
 
@@ -777,7 +881,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     const uint32_t chunks = (n_kept + FX_ITEM - 1) / FX_ITEM;   // row chunks per column (column-major)
     const uint32_t n_items = colmajor ? rowlen * chunks : (n_el + FX_ITEM - 1) / FX_ITEM;
     const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
-    const int64_t obase = (int64_t)od[FX_W(FxOut, task_stride)] * w.task + (int64_t)prefix * rowlen;
+    const uint32_t obase = uni(od[FX_W(FxOut, task_stride)]) * (uint32_t)w.task + prefix * rowlen;
     const int pb = (int)uni(od[FX_W(FxOut, prog_begin)]), pe = (int)uni(od[FX_W(FxOut, prog_end)]);
     const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
     uint32_t dk[R], mk[R], sk[R];
@@ -787,12 +891,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
       mk[k] = od[FX_W(FxOut, magic) + k];
       sk[k] = od[FX_W(FxOut, shift) + k];
     }
-    // first item of this output that belongs to this wave
-    uint32_t it = (wave_u + 4u - (item_base & 3u)) & 3u;
-    for (; it < n_items; it += 4u) {
-      int32_t c[FX_V][R];
-      uint32_t M = 0;
-      uint32_t e[FX_V];
+    const uint32_t lead = uni(od[FX_W(FxOut, lead)]);
+    auto make_item = [&](uint32_t it, uint32_t (&e)[FX_V], uint32_t& M, int32_t (&c)[FX_V][R]) {
+      M = 0;
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
         uint32_t r, col;
@@ -813,20 +914,48 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         }
         if (live) M |= 1u << j;
 #pragma unroll
-        for (int k = R - 1; k >= 1; --k) {
+        for (int k = R - 1; k >= 2; --k) {
           const uint32_t q = fx_fastdiv(col, mk[k], sk[k]);
           c[j][k] = (int32_t)(col - q * dk[k]);
           col = q;
         }
+        if (R > 1) c[j][1] = (int32_t)col;  // what is left is the coordinate itself
         c[j][0] = live ? (int32_t)s_rowmap[r] : 0;
       }
-      uint32_t A[FX_V];
+    };
+    // items of this output that belong to this wave: first, first + 4, ...
+    // taken FX_K at a time so that their leading loads overlap
+    uint32_t it0 = (wave_u + 4u - (item_base & 3u)) & 3u;
+    for (; it0 < n_items; it0 += 4u * FX_K) {
+      uint32_t P[FX_K][FX_V];
+      if (lead) {
 #pragma unroll
-      for (int j = 0; j < FX_V; ++j) A[j] = 0;
-      fx_run<R>(cx, pb, pe, c, M, A);
+        for (uint32_t k = 0; k < FX_K; ++k) {
+          const uint32_t it = it0 + 4u * k;
+          if (it < n_items) {
+            uint32_t e[FX_V], M;
+            int32_t c[FX_V][R];
+            make_item(it, e, M, c);
+            fx_lead_load<R>(cx, pb, c, M, P[k]);
+          }
+        }
+      }
 #pragma unroll
-      for (int j = 0; j < FX_V; ++j) {
-        if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
+      for (uint32_t k = 0; k < FX_K; ++k) {
+        const uint32_t it = it0 + 4u * k;
+        if (it < n_items) {
+          uint32_t e[FX_V], M;
+          int32_t c[FX_V][R];
+          make_item(it, e, M, c);
+          uint32_t A[FX_V];
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
+          fx_run<R>(cx, lead ? pb + 1 : pb, pe, c, M, A);
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) {
+            if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
+          }
+        }
       }
     }
     item_base += n_items;
@@ -976,7 +1105,7 @@ static FxLaunch make_launch(const FxLaunchInfo& li) {
   la.n_s = li.n_s;
   la.stage_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
   la.temps_off = la.stage_off + li.stage_words;
-  la.pad = 0;
+  la.total_units = li.total_units;
   return la;
 }
 

@@ -605,7 +605,7 @@ int Lowerer::addAffine(const IdxExpr& e) {
   memset(&a, 0, sizeof(a));
   auto fit = [](int64_t x) {
     FX_CHECK(x >= std::numeric_limits<int32_t>::min() && x <= std::numeric_limits<int32_t>::max(), FX_E_LIMIT,
-             "index arithmetic exceeds 32 bits (tensors above 2^31 elements are not supported)");
+             "index arithmetic exceeds 32 bits");
     return (int32_t)x;
   };
   for (int i = 0; i < FX_MAXR; ++i) fx_aff_set_coef(&a, i, fit(e.c[i]));
@@ -1632,6 +1632,7 @@ static void findStages(ClassBuild& cb, const std::vector<PtrSrc>& sptr, const st
 }
 
 static void applyStages(ClassBuild& cb, uint32_t row_tile) {
+  struct Fix { ClassBuild& cb; ~Fix() { for (auto& od : cb.outs) if (od.prog_end > od.prog_begin && cb.code[od.prog_begin].op != FX_LDA) od.lead = 0; } } fix{cb};
   uint32_t off = 0;
   for (auto& st : cb.stages) {
     st.lds_off = off;
@@ -1717,6 +1718,14 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     for (int t = 0; t < n; ++t) {
       const fx_arg& a = args[arg_base[i] + t];
       FX_CHECK(a.dtype == v.dtype, FX_E_INVALID, "input " << i << ": dtype differs from the declared one");
+      // the kernels address every buffer with a 32-bit byte offset from its base
+      int64_t extent = 1;
+      for (int d = 0; d < a.rank; ++d) {
+        FX_CHECK(a.strides[d] >= 0, FX_E_UNSUPPORTED, "input " << i << ": negative strides are not supported");
+        if (a.sizes[d] > 0) extent += (a.sizes[d] - 1) * a.strides[d];
+      }
+      FX_CHECK(extent * dtype_size(a.dtype) < ((int64_t)1 << 32), FX_E_LIMIT,
+               "input " << i << " spans 4 GiB or more; split it before fusing");
       FX_CHECK(a.rank == v.rank || v.rank < 0, FX_E_INVALID, "input " << i << ": rank differs from the declared one");
     }
   }
@@ -1779,7 +1788,8 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     }
     for (size_t o = 0; o < R.outputs.size(); ++o) {
       Shape s = L.shapeOf(R.outputs[o]);
-      FX_CHECK(numel_of(s) < ((int64_t)1 << 31), FX_E_LIMIT, "output above 2^31 elements");
+      FX_CHECK(numel_of(s) * dtype_size(P->out_dtype[o]) < ((int64_t)1 << 32), FX_E_LIMIT,
+               "output " << o << " is 4 GiB or larger; split the region");
       for (int t : cb.tasks) P->out_shape[o][t] = s;
       FxOut od;
       memset(&od, 0, sizeof(od));
@@ -1792,6 +1802,11 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       od.dtype = storage_dt(P->out_dtype[o]);
       od.ptr_slot = (uint32_t)out_slot[o];
       od.task_stride = 0;
+      {
+        // leading load: unconditional, affine, not inside a reduction loop
+        const FxInsn& i0 = L.code[p.begin];
+        od.lead = (p.end > p.begin && i0.op == FX_LDA) ? 1u : 0u;
+      }
       if (P->mode == FX_MODE_COMPACT) {
         FX_CHECK(!s.empty() && s[0] == (int64_t)cb.cls.n_rows, FX_E_INVALID,
                  "compacted output " << o << ": dim 0 must match the mask length");
@@ -1844,6 +1859,10 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       if (total_rows / 64 >= 4096) row_tile = 256;
       else if (total_rows / 64 >= 2048) row_tile = 128;
     }
+    if (getenv("FX_ROW_TILE")) {  // experiment switch
+      int rt = atoi(getenv("FX_ROW_TILE"));
+      if ((rt == 64 || rt == 128 || rt == 256) && fits((uint32_t)rt)) row_tile = (uint32_t)rt;
+    }
     for (auto& cb : classes) {
       applyStages(cb, row_tile);
       P->stage_words = std::max(P->stage_words, stageWords(cb, row_tile));
@@ -1863,7 +1882,14 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       uint32_t b = 0;
       for (auto& od : cb.outs) {
         od.block_begin = b;
-        od.n_blocks = (od.numel + FX_TILE - 1) / FX_TILE;
+        // big streaming outputs use large units (per-unit bookkeeping amortised, leading loads of
+        // 4 items batched); heavy programs (reduction loops) and small outputs use the smallest
+        // unit so that the work spreads over all CUs
+        bool heavy = false;
+        for (uint32_t pc = od.prog_begin; pc < od.prog_end; ++pc) heavy = heavy || cb.code[pc].op == FX_RBEGIN;
+        od.unit_items = (!heavy && od.numel >= (8u << 20)) ? 4u : 1u;
+        const uint32_t unit = 4u * od.unit_items * FX_ITEM;
+        od.n_blocks = (od.numel + unit - 1) / unit;
         b += od.n_blocks;
       }
       c.blocks_per_task = std::max<uint32_t>(b, 1);

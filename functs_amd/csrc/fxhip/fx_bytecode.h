@@ -87,6 +87,9 @@ enum FxOp : uint32_t {
   // ---- loads from an input tile staged in LDS (row-tiled kernels) ----
   FX_LDSA,   // A = stage[a] at affine[b](coords) relative to the tile; dt = storage dtype
   FX_LDSB,
+  // ---- reductions across the wave (row-per-wave mapping, FxOut::rowwave) ----
+  FX_WMAX,   // A = max of A over every live element of the wave (NaN-propagating)
+  FX_WSUM,   // A = sum of A over every live element of the wave
   FX_OP_COUNT
 };
 
@@ -148,6 +151,8 @@ struct FxOut {
   uint32_t colmajor;              // compaction: iterate (column, row chunk) instead of flat elements
   uint32_t lead;                  // program starts with an unconditional affine load (batched by the kernels)
   uint32_t unit_items;            // dense: items per wave and work unit (1 or FX_K)
+  uint32_t rowwave;               // dense: one item = one row of dim[rank-1] elements (needed by FX_WMAX/FX_WSUM)
+  uint32_t pad;
 };
 
 // An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows

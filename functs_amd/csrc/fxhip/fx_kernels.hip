@@ -465,6 +465,22 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         }
         break;
 
+      case FX_WMAX:
+      case FX_WSUM: {
+        const bool is_max = op == FX_WMAX;
+        float v = is_max ? -__builtin_inff() : 0.0f;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          if ((M >> j) & 1u) v = is_max ? fx_fmax(v, u2f(A[j])) : v + u2f(A[j]);
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+          const float t = __shfl_xor(v, o, 64);
+          v = is_max ? fx_fmax(v, t) : v + t;
+        }
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) A[j] = f2u(v);
+      } break;
       case FX_RBEGIN: {
         const uint32_t d = uni((uint32_t)ia) & 1u;
         const int32_t ext = (int32_t)uni(imm);
@@ -686,17 +702,30 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
       mk[k] = od[FX_W(FxOut, magic) + k];
       sk[k] = od[FX_W(FxOut, shift) + k];
     }
-    // unit = 4 waves x kmax items; kmax is 1 for heavy or small outputs (more, smaller units)
+    // unit = 4 waves x kmax items; kmax is 1 for heavy or small outputs (more, smaller units).
+    // An item is FX_ITEM consecutive elements, or one whole row (rowwave) so that
+    // the wave-wide reductions see exactly the elements of that row.
     const uint32_t kmax = uni(od[FX_W(FxOut, unit_items)]);
-    const uint32_t first = ublock * (4u * kmax * FX_ITEM) + wave * (kmax * FX_ITEM);
-    if (first >= numel) continue;
+    const uint32_t rowwave = uni(od[FX_W(FxOut, rowwave)]);
+    const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
+    const uint32_t item0 = ublock * (4u * kmax) + wave * kmax;
+    const uint32_t n_items = rowwave ? numel / (rowlen ? rowlen : 1u) : (numel + FX_ITEM - 1) / FX_ITEM;
+    if (item0 >= n_items) continue;
 
     auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, int32_t (&c)[FX_V][R]) {
       M = 0;
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
-        e[j] = first + k * FX_ITEM + j * 64u + lane;
-        if (e[j] < numel) M |= 1u << j;
+        bool live;
+        if (rowwave) {
+          const uint32_t col = j * 64u + lane;
+          live = col < rowlen;
+          e[j] = (item0 + k) * rowlen + (live ? col : 0u);
+        } else {
+          e[j] = (item0 + k) * FX_ITEM + j * 64u + lane;
+          live = e[j] < numel;
+        }
+        if (live) M |= 1u << j;
         uint32_t rem = e[j];
 #pragma unroll
         for (int q = R - 1; q >= 1; --q) {
@@ -712,7 +741,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
     if (lead) {
 #pragma unroll
       for (uint32_t k = 0; k < FX_K; ++k) {
-        if (k < kmax && first + k * FX_ITEM < numel) {
+        if (k < kmax && item0 + k < n_items) {
           uint32_t e[FX_V], M;
           int32_t c[FX_V][R];
           make_item(k, e, M, c);
@@ -722,7 +751,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
     }
 #pragma unroll
     for (uint32_t k = 0; k < FX_K; ++k) {
-      if (k < kmax && first + k * FX_ITEM < numel) {
+      if (k < kmax && item0 + k < n_items) {
         uint32_t e[FX_V], M;
         int32_t c[FX_V][R];
         make_item(k, e, M, c);

@@ -228,7 +228,7 @@ struct SlotAlloc {
   }
 };
 
-struct Prog { uint32_t begin, end, vt; };
+struct Prog { uint32_t begin, end, vt; bool rowwave; };
 
 class Lowerer {
  public:
@@ -238,6 +238,7 @@ class Lowerer {
   std::vector<FxInsn> code;
   std::vector<FxAffine> affs;
   int maxTemps = 0;
+  bool allowRowWave = false;  // dense outputs only: a reduction over the last dim may use wave-wide ops
 
   Shape shapeOf(int vid);
   Prog lower(int vid, const Shape& rootShape);
@@ -259,6 +260,10 @@ class Lowerer {
   std::vector<std::pair<int64_t, int64_t>> tempRange_ = std::vector<std::pair<int64_t, int64_t>>(FX_MAX_TEMPS);
   bool loopVarBound_ = false;
   IdxExpr loopVar_;
+  bool usedRowWave_ = false;
+  // true when coordinate `d` of frame f is exactly the innermost root coordinate, nothing else
+  // in the frame moves with it, and the whole extent fits one wave item
+  bool rowWaveFrame(const Frame& f, int d, int64_t extent) const;
 
   const Value& V(int id) const { return R_.vals[id]; }
 
@@ -1520,6 +1525,27 @@ void Lowerer::emitOp(const Res& r) {
       // computeSoftmax, custom_lowering_func.cpp:134-180: max, exp(x-max), sum, div
       Shape in = shapeOf(arg(0));
       int d = normDim(constIntOf(arg(1), "softmax"), (int64_t)in.size(), "softmax");
+      if (rowWaveFrame(f, d, in[d])) {
+        // the wave holds exactly one row: max / sum are wave reductions instead of a
+        // serial loop per element (the reference materialises them as separate
+        // kernels, custom_lowering_func.cpp:154-179)
+        usedRowWave_ = true;
+        emitAs(arg(0), f, FX_VT_F);
+        int tx = allocTemp();
+        emitI(FX_STT, tx);
+        emitI(FX_WMAX);
+        emitI(FX_MOVBA);
+        emitI(FX_LDTA, tx);
+        emitI(FX_FSUB);
+        emitI(FX_EXP);
+        emitI(FX_STT, tx);
+        emitI(FX_WSUM);
+        emitI(FX_MOVBA);
+        emitI(FX_LDTA, tx);
+        emitI(FX_FDIV);
+        freeTemp(tx);
+        return;
+      }
       int tmax = allocTemp();
       emitReduce(FX_FMAX, fbits(-std::numeric_limits<float>::infinity()), in[d], [&](int depth) {
         Frame fi = f; fi[d] = IdxExpr::loop(depth);
@@ -1548,6 +1574,20 @@ void Lowerer::emitOp(const Res& r) {
   FX_CHECK(false, FX_E_UNSUPPORTED, "no lowering for opcode " << v.op);
 }
 
+bool Lowerer::rowWaveFrame(const Frame& f, int d, int64_t extent) const {
+  if (!allowRowWave || rootRank_ < 1 || maskDepth_ != 0 || loopDepth_ != 0) return false;
+  const int r = rootRank_ - 1;
+  if (extent != rootDim_[r] || extent > FX_ITEM || extent < 1) return false;
+  IdxExpr want = IdxExpr::root(r);
+  const IdxExpr& x = f[d];
+  if (!x.affine() || x.k != 0 || x.ct != 0) return false;
+  for (int i = 0; i < FX_MAXR; ++i) if (x.c[i] != want.c[i]) return false;
+  for (int i = 0; i < FX_MAXLOOP; ++i) if (x.rc[i] != 0) return false;
+  for (size_t k = 0; k < f.size(); ++k)
+    if ((int)k != d && f[k].c[r] != 0) return false;
+  return true;
+}
+
 Prog Lowerer::lower(int vid, const Shape& rootShape) {
   FX_CHECK(rootShape.size() <= FX_MAXR, FX_E_UNSUPPORTED, "region outputs above rank " << FX_MAXR << " are not supported");
   rootRank_ = (int)rootShape.size();
@@ -1555,6 +1595,7 @@ Prog Lowerer::lower(int vid, const Shape& rootShape) {
   tempTop_ = 0;
   maskDepth_ = 0;
   loopDepth_ = 0;
+  usedRowWave_ = false;
   Frame f(rootRank_);
   for (int i = 0; i < rootRank_; ++i) f[i] = IdxExpr::root(i);
   Prog p;
@@ -1562,6 +1603,7 @@ Prog Lowerer::lower(int vid, const Shape& rootShape) {
   emit(vid, f);
   p.end = (uint32_t)code.size();
   p.vt = vt_of(V(vid).dtype);
+  p.rowwave = usedRowWave_;
   return p;
 }
 
@@ -1774,6 +1816,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     for (size_t i = 0; i < R.inputs.size(); ++i)
       in[i] = &args[arg_base[i] + (R.vals[R.inputs[i]].per_task ? cb.tasks[0] : 0)];
     Lowerer L(R, in, T, slots);
+    L.allowRowWave = P->mode == FX_MODE_DENSE;
     memset(&cb.cls, 0, sizeof(cb.cls));
     if (P->mode == FX_MODE_COMPACT) {
       Shape ms = L.shapeOf(R.mask);
@@ -1802,6 +1845,10 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       od.dtype = storage_dt(P->out_dtype[o]);
       od.ptr_slot = (uint32_t)out_slot[o];
       od.task_stride = 0;
+      if (p.rowwave) {
+        od.rowwave = 1;
+        od.rowlen = (uint32_t)s.back();
+      }
       {
         // leading load: unconditional, affine, not inside a reduction loop
         const FxInsn& i0 = L.code[p.begin];
@@ -1888,8 +1935,14 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         bool heavy = false;
         for (uint32_t pc = od.prog_begin; pc < od.prog_end; ++pc) heavy = heavy || cb.code[pc].op == FX_RBEGIN;
         od.unit_items = (!heavy && od.numel >= (8u << 20)) ? 4u : 1u;
-        const uint32_t unit = 4u * od.unit_items * FX_ITEM;
-        od.n_blocks = (od.numel + unit - 1) / unit;
+        if (od.rowwave) {
+          const uint32_t rows = od.rowlen ? od.numel / od.rowlen : 0;
+          od.n_blocks = (rows + 4u * od.unit_items - 1) / (4u * od.unit_items);
+          od.lead = 0;
+        } else {
+          const uint32_t unit = 4u * od.unit_items * FX_ITEM;
+          od.n_blocks = (od.numel + unit - 1) / unit;
+        }
         b += od.n_blocks;
       }
       c.blocks_per_task = std::max<uint32_t>(b, 1);
@@ -2032,7 +2085,7 @@ static const char* opname(uint32_t op) {
       "INEG", "LNOT", "INZ", "FNZ", "F2I", "I2F", "IABS", "FADD", "FSUB", "FRSUB", "FMUL", "FDIV", "FRDIV", "FMIN",
       "FMAX", "FPOW", "FMOD", "ATAN2", "IADD", "ISUB", "IRSUB", "IMUL", "IFDIV", "ITDIV", "IPMOD", "ITMOD", "IMIN",
       "IMAX", "IAND", "IOR", "IXOR", "FLT", "FLE", "FGT", "FGE", "FEQ", "FNE", "ILT", "ILE", "IGT", "IGE", "IEQ",
-      "INE", "IRANGE", "WHERE", "RBEGIN", "RNEXT", "RIDX", "LDSA", "LDSB"};
+      "INE", "IRANGE", "WHERE", "RBEGIN", "RNEXT", "RIDX", "LDSA", "LDSB", "WMAX", "WSUM"};
   if (op < sizeof(names) / sizeof(names[0])) return names[op];
   return "?";
 }

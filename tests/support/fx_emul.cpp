@@ -91,135 +91,163 @@ uint32_t scalar_of(const Ctx& cx, int32_t slot) {
   return (slot & FX_SLOT_TASK) ? cx.tscal[slot & 0xffff] : cx.sscal[slot & 0xffff];
 }
 
-// one element; returns A.  `live` mirrors the lane mask bit.
-uint32_t run(const Ctx& cx, int pc, int pc_end, const int32_t* c) {
+// A batch of elements executed in lockstep, like the lanes of one wave item:
+// control flow is uniform, `live` mirrors the lane mask.  Batches of one element
+// are used for ordinary outputs; row-per-wave outputs run one row per batch so
+// that FX_WMAX / FX_WSUM see exactly the elements the GPU wave sees.
+struct Lane {
   uint32_t A = 0, B = 0;
-  uint32_t temps[FX_MAX_TEMPS];
-  memset(temps, 0, sizeof(temps));
   bool M = true;
   std::vector<bool> stack;
+  uint32_t temps[FX_MAX_TEMPS];
+  int32_t c[FX_MAXR];
+};
+
+void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
+  for (auto& l : L) { l.A = 0; l.B = 0; l.M = true; l.stack.clear(); memset(l.temps, 0, sizeof(l.temps)); }
   int32_t lc[FX_MAXLOOP] = {0, 0}, le[FX_MAXLOOP] = {0, 0};
   long guard = 0;
+  auto any_live = [&]() { for (auto& l : L) if (l.M) return true; return false; };
   while (pc < pc_end) {
     if (++guard > 50000000) break;
     const FxInsn ins = cx.insn[pc++];
     const bool useimm = ins.flags & FX_F_IMM;
-    const float fa = u2f(A), fb = u2f(useimm ? ins.imm : B);
-    const int32_t ia = (int32_t)A, ib = (int32_t)(useimm ? ins.imm : B);
-    switch (ins.op) {
-      case FX_NOP: break;
-      case FX_LDA: case FX_LDB: case FX_AFFA: case FX_AFFB: {
-        if (!M) break;
-        const FxAffine& af = cx.aff[ins.b];
-        int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
-        for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
-        bool is_load = ins.op == FX_LDA || ins.op == FX_LDB;
-        uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt) : (uint32_t)off;
-        if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
-        if (ins.op == FX_LDA || ins.op == FX_AFFA) A = v; else B = v;
-      } break;
-      case FX_LDSA: case FX_LDSB: {
-        // a staged load reads the same element as the global load it replaces
-        if (!M) break;
-        const FxAffine& af = cx.aff[ins.b];
-        int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
-        for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
-        uint32_t v = load_elem(ptr_of(cx, (int32_t)cx.stages[ins.a].ptr_slot), off, ins.dt);
-        if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
-        if (ins.op == FX_LDSA) A = v; else B = v;
-      } break;
-      case FX_LDXA: if (M) A = load_elem(ptr_of(cx, ins.a), (int64_t)((int32_t)A + (int32_t)ins.imm), ins.dt); break;
-      case FX_IMMA: if (M) A = ins.imm; break;
-      case FX_IMMB: B = ins.imm; break;
-      case FX_SCLA: if (M) { A = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) A = f2u((float)(int32_t)A); } break;
-      case FX_SCLB: B = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) B = f2u((float)(int32_t)B); break;
-      case FX_STT: temps[ins.a] = A; break;
-      case FX_LDTA: if (M) A = temps[ins.a]; break;
-      case FX_LDTB: B = temps[ins.a]; break;
-      case FX_MOVBA: B = A; break;
-      case FX_SWAP: { uint32_t t = A; A = B; B = t; } break;
-      case FX_MIF: stack.push_back(M); M = M && (A != 0); if (!M) pc = ins.a; break;
-      case FX_MELSE: M = stack.back() && !M; if (!M) pc = ins.a; break;
-      case FX_MMERGE: A = M ? A : temps[ins.a]; M = stack.back(); stack.pop_back(); break;
-      case FX_MEND: M = stack.back(); stack.pop_back(); break;
-      case FX_FNEG: A = f2u(-fa); break;
-      case FX_FABS: A = f2u(fabsf(fa)); break;
-      case FX_EXP: A = f2u(expf(fa)); break;
-      case FX_LOG: A = f2u(logf(fa)); break;
-      case FX_SQRT: A = f2u(sqrtf(fa)); break;
-      case FX_RSQRT: A = f2u(1.0f / sqrtf(fa)); break;
-      case FX_RCP: A = f2u(1.0f / fa); break;
-      case FX_SIGMOID: A = f2u(1.0f / (1.0f + expf(-fa))); break;
-      case FX_TANH: A = f2u(tanhf(fa)); break;
-      case FX_RELU: A = f2u(fa <= 0.0f ? 0.0f : fa); break;
-      case FX_FLOOR: A = f2u(floorf(fa)); break;
-      case FX_CEIL: A = f2u(ceilf(fa)); break;
-      case FX_ROUND: A = f2u(rintf(fa)); break;
-      case FX_TRUNC: A = f2u(truncf(fa)); break;
-      case FX_SIN: A = f2u(sinf(fa)); break;
-      case FX_COS: A = f2u(cosf(fa)); break;
-      case FX_ERF: A = f2u(erff(fa)); break;
-      case FX_LOG2: A = f2u(log2f(fa)); break;
-      case FX_EXP2: A = f2u(exp2f(fa)); break;
-      case FX_EXPM1: A = f2u(expm1f(fa)); break;
-      case FX_LOG1P: A = f2u(log1pf(fa)); break;
-      case FX_INEG: A = (uint32_t)(-ia); break;
-      case FX_IABS: A = (uint32_t)(ia < 0 ? -ia : ia); break;
-      case FX_LNOT: A = ia == 0; break;
-      case FX_INZ: A = ia != 0; break;
-      case FX_FNZ: A = fa != 0.0f; break;
-      case FX_F2I: A = (uint32_t)(int32_t)fa; break;
-      case FX_I2F: A = f2u((float)ia); break;
-      case FX_FADD: A = f2u(fa + fb); break;
-      case FX_FSUB: A = f2u(fa - fb); break;
-      case FX_FRSUB: A = f2u(fb - fa); break;
-      case FX_FMUL: A = f2u(fa * fb); break;
-      case FX_FDIV: A = f2u(fa / fb); break;
-      case FX_FRDIV: A = f2u(fb / fa); break;
-      case FX_FMIN: A = f2u(fx_fmin(fa, fb)); break;
-      case FX_FMAX: A = f2u(fx_fmax(fa, fb)); break;
-      case FX_FPOW: A = f2u(powf(fa, fb)); break;
-      case FX_FMOD: A = f2u(fmodf(fa, fb)); break;
-      case FX_ATAN2: A = f2u(atan2f(fa, fb)); break;
-      case FX_IADD: A = (uint32_t)(ia + ib); break;
-      case FX_ISUB: A = (uint32_t)(ia - ib); break;
-      case FX_IRSUB: A = (uint32_t)(ib - ia); break;
-      case FX_IMUL: A = (uint32_t)(ia * ib); break;
-      case FX_IFDIV: A = (uint32_t)floordiv_i(ia, ib); break;
-      case FX_ITDIV: A = (uint32_t)(ib == 0 ? 0 : ia / ib); break;
-      case FX_IPMOD: A = (uint32_t)pymod_i(ia, ib); break;
-      case FX_ITMOD: A = (uint32_t)(ib == 0 ? 0 : ia % ib); break;
-      case FX_IMIN: A = (uint32_t)(ia < ib ? ia : ib); break;
-      case FX_IMAX: A = (uint32_t)(ia > ib ? ia : ib); break;
-      case FX_IAND: A = (uint32_t)(ia & ib); break;
-      case FX_IOR: A = (uint32_t)(ia | ib); break;
-      case FX_IXOR: A = (uint32_t)(ia ^ ib); break;
-      case FX_FLT: A = fa < fb; break;
-      case FX_FLE: A = fa <= fb; break;
-      case FX_FGT: A = fa > fb; break;
-      case FX_FGE: A = fa >= fb; break;
-      case FX_FEQ: A = fa == fb; break;
-      case FX_FNE: A = fa != fb; break;
-      case FX_ILT: A = ia < ib; break;
-      case FX_ILE: A = ia <= ib; break;
-      case FX_IGT: A = ia > ib; break;
-      case FX_IGE: A = ia >= ib; break;
-      case FX_IEQ: A = ia == ib; break;
-      case FX_INE: A = ia != ib; break;
-      case FX_IRANGE: {
-        int32_t lo = ins.a, hi = ins.b, st = (int32_t)ins.imm;
-        bool in = ia >= lo && ia < hi;
-        if (st > 1) in = in && ((ia - lo) % st == 0);
-        A = in;
-      } break;
-      case FX_WHERE: A = temps[ins.a] != 0 ? A : B; break;
-      case FX_RBEGIN: { int d = ins.a & (FX_MAXLOOP - 1); lc[d] = 0; le[d] = (int32_t)ins.imm; if (le[d] <= 0) pc = ins.b; } break;
-      case FX_RNEXT: { int d = ins.b & (FX_MAXLOOP - 1); lc[d] += 1; if (lc[d] < le[d]) pc = ins.a; } break;
-      case FX_RIDX: if (M) A = (uint32_t)lc[ins.a & (FX_MAXLOOP - 1)]; break;
-      default: break;
+    if (ins.op == FX_MIF) {
+      for (auto& l : L) { l.stack.push_back(l.M); l.M = l.M && (l.A != 0); }
+      if (!any_live()) pc = ins.a;
+      continue;
+    }
+    if (ins.op == FX_MELSE) {
+      for (auto& l : L) l.M = l.stack.back() && !l.M;
+      if (!any_live()) pc = ins.a;
+      continue;
+    }
+    if (ins.op == FX_RBEGIN) { int d = ins.a & (FX_MAXLOOP - 1); lc[d] = 0; le[d] = (int32_t)ins.imm; if (le[d] <= 0) pc = ins.b; continue; }
+    if (ins.op == FX_RNEXT) { int d = ins.b & (FX_MAXLOOP - 1); lc[d] += 1; if (lc[d] < le[d]) pc = ins.a; continue; }
+    if (ins.op == FX_WMAX || ins.op == FX_WSUM) {
+      float v = ins.op == FX_WMAX ? -INFINITY : 0.0f;
+      for (auto& l : L) if (l.M) v = ins.op == FX_WMAX ? fx_fmax(v, u2f(l.A)) : v + u2f(l.A);
+      for (auto& l : L) l.A = f2u(v);
+      continue;
+    }
+    for (auto& l : L) {
+      uint32_t& A = l.A;
+      uint32_t& B = l.B;
+      const bool M = l.M;
+      uint32_t* temps = l.temps;
+      const int32_t* c = l.c;
+      const float fa = u2f(A), fb = u2f(useimm ? ins.imm : B);
+      const int32_t ia = (int32_t)A, ib = (int32_t)(useimm ? ins.imm : B);
+      switch (ins.op) {
+        case FX_NOP: break;
+        case FX_LDA: case FX_LDB: case FX_AFFA: case FX_AFFB: case FX_LDSA: case FX_LDSB: {
+          if (!M) break;
+          const FxAffine& af = cx.aff[ins.b];
+          int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
+          for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
+          const bool staged = ins.op == FX_LDSA || ins.op == FX_LDSB;
+          const bool is_load = staged || ins.op == FX_LDA || ins.op == FX_LDB;
+          // a staged load reads the same element as the global load it replaces
+          const int32_t slot = staged ? (int32_t)cx.stages[ins.a].ptr_slot : ins.a;
+          uint32_t v = is_load ? load_elem(ptr_of(cx, slot), off, ins.dt) : (uint32_t)off;
+          if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
+          if (ins.op == FX_LDA || ins.op == FX_AFFA || ins.op == FX_LDSA) A = v; else B = v;
+        } break;
+        case FX_LDXA: if (M) A = load_elem(ptr_of(cx, ins.a), (int64_t)((int32_t)A + (int32_t)ins.imm), ins.dt); break;
+        case FX_IMMA: if (M) A = ins.imm; break;
+        case FX_IMMB: B = ins.imm; break;
+        case FX_SCLA: if (M) { A = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) A = f2u((float)(int32_t)A); } break;
+        case FX_SCLB: B = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) B = f2u((float)(int32_t)B); break;
+        case FX_STT: temps[ins.a] = A; break;
+        case FX_LDTA: if (M) A = temps[ins.a]; break;
+        case FX_LDTB: B = temps[ins.a]; break;
+        case FX_MOVBA: B = A; break;
+        case FX_SWAP: { uint32_t t = A; A = B; B = t; } break;
+        case FX_MMERGE: A = M ? A : temps[ins.a]; l.M = l.stack.back(); l.stack.pop_back(); break;
+        case FX_MEND: l.M = l.stack.back(); l.stack.pop_back(); break;
+        case FX_FNEG: A = f2u(-fa); break;
+        case FX_FABS: A = f2u(fabsf(fa)); break;
+        case FX_EXP: A = f2u(expf(fa)); break;
+        case FX_LOG: A = f2u(logf(fa)); break;
+        case FX_SQRT: A = f2u(sqrtf(fa)); break;
+        case FX_RSQRT: A = f2u(1.0f / sqrtf(fa)); break;
+        case FX_RCP: A = f2u(1.0f / fa); break;
+        case FX_SIGMOID: A = f2u(1.0f / (1.0f + expf(-fa))); break;
+        case FX_TANH: A = f2u(tanhf(fa)); break;
+        case FX_RELU: A = f2u(fa <= 0.0f ? 0.0f : fa); break;
+        case FX_FLOOR: A = f2u(floorf(fa)); break;
+        case FX_CEIL: A = f2u(ceilf(fa)); break;
+        case FX_ROUND: A = f2u(rintf(fa)); break;
+        case FX_TRUNC: A = f2u(truncf(fa)); break;
+        case FX_SIN: A = f2u(sinf(fa)); break;
+        case FX_COS: A = f2u(cosf(fa)); break;
+        case FX_ERF: A = f2u(erff(fa)); break;
+        case FX_LOG2: A = f2u(log2f(fa)); break;
+        case FX_EXP2: A = f2u(exp2f(fa)); break;
+        case FX_EXPM1: A = f2u(expm1f(fa)); break;
+        case FX_LOG1P: A = f2u(log1pf(fa)); break;
+        case FX_INEG: A = (uint32_t)(-ia); break;
+        case FX_IABS: A = (uint32_t)(ia < 0 ? -ia : ia); break;
+        case FX_LNOT: A = ia == 0; break;
+        case FX_INZ: A = ia != 0; break;
+        case FX_FNZ: A = fa != 0.0f; break;
+        case FX_F2I: A = (uint32_t)(int32_t)fa; break;
+        case FX_I2F: A = f2u((float)ia); break;
+        case FX_FADD: A = f2u(fa + fb); break;
+        case FX_FSUB: A = f2u(fa - fb); break;
+        case FX_FRSUB: A = f2u(fb - fa); break;
+        case FX_FMUL: A = f2u(fa * fb); break;
+        case FX_FDIV: A = f2u(fa / fb); break;
+        case FX_FRDIV: A = f2u(fb / fa); break;
+        case FX_FMIN: A = f2u(fx_fmin(fa, fb)); break;
+        case FX_FMAX: A = f2u(fx_fmax(fa, fb)); break;
+        case FX_FPOW: A = f2u(powf(fa, fb)); break;
+        case FX_FMOD: A = f2u(fmodf(fa, fb)); break;
+        case FX_ATAN2: A = f2u(atan2f(fa, fb)); break;
+        case FX_IADD: A = (uint32_t)(ia + ib); break;
+        case FX_ISUB: A = (uint32_t)(ia - ib); break;
+        case FX_IRSUB: A = (uint32_t)(ib - ia); break;
+        case FX_IMUL: A = (uint32_t)(ia * ib); break;
+        case FX_IFDIV: A = (uint32_t)floordiv_i(ia, ib); break;
+        case FX_ITDIV: A = (uint32_t)(ib == 0 ? 0 : ia / ib); break;
+        case FX_IPMOD: A = (uint32_t)pymod_i(ia, ib); break;
+        case FX_ITMOD: A = (uint32_t)(ib == 0 ? 0 : ia % ib); break;
+        case FX_IMIN: A = (uint32_t)(ia < ib ? ia : ib); break;
+        case FX_IMAX: A = (uint32_t)(ia > ib ? ia : ib); break;
+        case FX_IAND: A = (uint32_t)(ia & ib); break;
+        case FX_IOR: A = (uint32_t)(ia | ib); break;
+        case FX_IXOR: A = (uint32_t)(ia ^ ib); break;
+        case FX_FLT: A = fa < fb; break;
+        case FX_FLE: A = fa <= fb; break;
+        case FX_FGT: A = fa > fb; break;
+        case FX_FGE: A = fa >= fb; break;
+        case FX_FEQ: A = fa == fb; break;
+        case FX_FNE: A = fa != fb; break;
+        case FX_ILT: A = ia < ib; break;
+        case FX_ILE: A = ia <= ib; break;
+        case FX_IGT: A = ia > ib; break;
+        case FX_IGE: A = ia >= ib; break;
+        case FX_IEQ: A = ia == ib; break;
+        case FX_INE: A = ia != ib; break;
+        case FX_IRANGE: {
+          int32_t lo = ins.a, hi = ins.b, st = (int32_t)ins.imm;
+          bool in = ia >= lo && ia < hi;
+          if (st > 1) in = in && ((ia - lo) % st == 0);
+          A = in;
+        } break;
+        case FX_WHERE: A = temps[ins.a] != 0 ? A : B; break;
+        case FX_RIDX: if (M) A = (uint32_t)lc[ins.a & (FX_MAXLOOP - 1)]; break;
+        default: break;
+      }
     }
   }
-  return A;
+}
+
+uint32_t run1(const Ctx& cx, int pc, int pc_end, const int32_t* c) {
+  std::vector<Lane> L(1);
+  memcpy(L[0].c, c, sizeof(L[0].c));
+  run(cx, pc, pc_end, L);
+  return L[0].A;
 }
 
 void decompose(const FxOut& od, uint32_t e, int32_t* c) {
@@ -254,10 +282,21 @@ extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_,
         for (uint32_t oi = 0; oi < cl.n_outs; ++oi) {
           const FxOut& od = outs[oi];
           void* op = (void*)ptr_of(cx, (int32_t)od.ptr_slot);
+          if (od.rowwave) {
+            const uint32_t rows = od.rowlen ? od.numel / od.rowlen : 0;
+            for (uint32_t r = 0; r < rows; ++r) {
+              std::vector<Lane> L(od.rowlen);
+              for (uint32_t k = 0; k < od.rowlen; ++k) decompose(od, r * od.rowlen + k, L[k].c);
+              run(cx, (int)od.prog_begin, (int)od.prog_end, L);
+              for (uint32_t k = 0; k < od.rowlen; ++k)
+                store_elem(op, (int64_t)od.task_stride * task + r * od.rowlen + k, od.dtype, od.vt, L[k].A);
+            }
+            continue;
+          }
           for (uint32_t e = 0; e < od.numel; ++e) {
             int32_t c[FX_MAXR];
             decompose(od, e, c);
-            uint32_t v = run(cx, (int)od.prog_begin, (int)od.prog_end, c);
+            uint32_t v = run1(cx, (int)od.prog_begin, (int)od.prog_end, c);
             store_elem(op, (int64_t)od.task_stride * task + e, od.dtype, od.vt, v);
           }
         }
@@ -265,7 +304,7 @@ extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_,
         std::vector<uint32_t> rowmap;
         for (uint32_t r = 0; r < cl.n_rows; ++r) {
           int32_t c[FX_MAXR] = {(int32_t)r, 0, 0, 0, 0, 0};
-          uint32_t v = run(cx, (int)cl.mask_begin, (int)cl.mask_end, c);
+          uint32_t v = run1(cx, (int)cl.mask_begin, (int)cl.mask_end, c);
           bool keep = cl.mask_vt == FX_VT_F ? (u2f(v) != 0.0f) : (v != 0);
           if (keep) rowmap.push_back(r);
         }
@@ -279,7 +318,7 @@ extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_,
               uint32_t e = col;
               for (int q = FX_MAXR - 1; q >= 1; --q) { c[q] = (int32_t)(e % od.dim[q]); e /= od.dim[q]; }
               c[0] = (int32_t)rowmap[k];
-              uint32_t v = run(cx, (int)od.prog_begin, (int)od.prog_end, c);
+              uint32_t v = run1(cx, (int)od.prog_begin, (int)od.prog_end, c);
               store_elem(op, (int64_t)od.task_stride * task + (int64_t)k * od.rowlen + col, od.dtype, od.vt, v);
             }
           }

@@ -1,0 +1,40 @@
+// Python module functs_amd._C: same entry-point names as the reference's
+// functs._C (functs/csrc/jit/python/init.cpp:31-76, script_init.cpp:83-95).
+#include <torch/csrc/jit/python/pybind_utils.h>
+#include <torch/extension.h>
+
+#include "passes.h"
+#include "tensorssa.h"
+
+namespace py = pybind11;
+using namespace functs;
+using torch::jit::Graph;
+
+PYBIND11_MODULE(_C, m) {
+  m.doc() = "MI355X backend of FuncTs/FAIT fused functionalized regions";
+  py::class_<TensorSSAMutateInfo, std::shared_ptr<TensorSSAMutateInfo>>(m, "TensorSSAMutateInfo")
+      .def(py::init<>())
+      .def_property_readonly("mutNodes", [](TensorSSAMutateInfo& self) { return self.mutNodes; })
+      .def_property_readonly("mutValues", [](TensorSSAMutateInfo& self) { return self.mutValues; });
+  m.def("_jit_pass_remove_inplace", RemoveInplace);
+  m.def("_jit_pass_dumb_remove_inter_precedure_mutation", DumbRemoveInterPrecedureMutation);
+  m.def("_jit_pass_rewrite_mutation", TensorSSARewriteMutation);
+  m.def("_jit_pass_block_propagation", TensorSSAPropagation);
+  m.def("_jit_pass_rename", TensorSSARename);
+  m.def("_jit_pass_tensorssa_remove_update", TensorSSARemoveUpdate);
+  m.def("_jit_pass_convert_to_tensorssa", ConvertToTensorSSA);
+  m.def("_jit_pass_fait_fuse_ops", FuseOps);
+  m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
+  m.def("_jit_pass_parallelize_loops", ParallelizeLoops);
+  m.def("_jit_pass_fuse_masked_select", FuseMaskedSelect);
+  m.def("_jit_pass_to_parallel_functor", ToParallelFunctor);
+  m.def("_jit_pass_fait_pipeline", FaitPipeline);
+  m.def("_jit_pass_validate", Validate);
+  m.def("_create_function_from_graph", [](const std::string& name, std::shared_ptr<Graph> graph) {
+    // script_init.cpp:87-95; the stock GraphFunction + interpreter run the graph
+    auto cu = std::make_shared<torch::jit::CompilationUnit>();
+    auto* fn = cu->create_function(c10::QualifiedName(name), std::move(graph));
+    return torch::jit::StrongFunctionPtr(std::move(cu), fn);
+  });
+  m.def("_fxhip_library", []() { return functs::fxhipLibraryPath(); });
+}

@@ -1,0 +1,52 @@
+// Region formation on functionalized graphs and the tssa::ParallelFunctor
+// operator.  Interfaces of fait/passes/fuse_ops.h, parallelize_loops.h, te_op.h,
+// validate_graph.h and functs/csrc/jit/passes/fait/fait_pipeline.h.
+#pragma once
+#include <torch/csrc/jit/ir/ir.h>
+
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace functs {
+
+// fait/passes/fuse_ops.cpp:506-527: group fusable operators of every block
+// into prim::FusionGroup nodes (block-bodied).
+void FuseOps(std::shared_ptr<torch::jit::Graph> graph);
+
+// A prim::Loop whose single carried tensor T is read only through
+// immut::select(T, d, i) and written back through immut::select_rev(T, ., d, i)
+// touches a different slab in every iteration: the loop becomes one
+// fx::forall_select_rev node that a FusionGroup can absorb.  The reference never
+// parallelises loops with carried values (parallelize_loops.cpp:17).
+void CollapseAssignLoops(std::shared_ptr<torch::jit::Graph> graph);
+
+// fait/passes/parallelize_loops.cpp:12-145: loops without carried values whose
+// list reads are list[i] and whose list writes are one append per list become
+// prim::ParallelMap(len, lists...){block(i, elems...) -> rets}.
+void ParallelizeLoops(std::shared_ptr<torch::jit::Graph> graph);
+
+// Fold `x[mask]` consumers of a FusionGroup into the group when the bool mask is
+// produced by the same group (row compaction fused into the region).  The
+// reference leaves these to ATen (convert_to_tensorssa.cpp:422-443,
+// fuse_ops.cpp:173-200).
+void FuseMaskedSelect(std::shared_ptr<torch::jit::Graph> graph);
+
+// fait/passes/te_op.cpp:135-236: FusionGroup / ParallelMap{FusionGroup} ->
+// tssa::ParallelFunctor (Subgraph + parallel_degree, is_parallel_map,
+// is_parallel_args, input_refine_types).
+void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
+
+// fait/passes/validate_graph.cpp:6-38: every use is dominated by its definition.
+void Validate(std::shared_ptr<torch::jit::Graph> graph);
+
+// functs/csrc/jit/passes/fait/fait_pipeline.cpp:31-68 (the passes of it that the
+// fused-region path needs), on an already functionalized graph.
+void FaitPipeline(std::shared_ptr<torch::jit::Graph> graph, std::vector<c10::TypePtr> input_types);
+
+std::string fxhipLibraryPath();
+
+// shared by the passes
+bool isFusableNode(torch::jit::Node* node);
+
+}  // namespace functs

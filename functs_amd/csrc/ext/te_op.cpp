@@ -1,0 +1,650 @@
+// tssa::ParallelFunctor: the operator a fused region runs as, and the pass that
+// creates it from prim::FusionGroup / prim::ParallelMap nodes.
+//
+// Node contract as in the reference (fait/passes/te_op.cpp:34-249, te_op.h:13-23):
+//   g(attr::Subgraph)          the region; input 0 is the task index (or a None
+//                              placeholder for a plain fused op), then the arguments
+//   i(attr::parallel_degree)   number of tasks (-1: taken from the leading int input)
+//   i(attr::is_parallel_map)   outputs are List[Tensor] with one entry per task
+//   is(attr::is_parallel_args) per argument: 1 = a list holding one value per task
+//   tys(attr::input_refine_types)
+// plus i(attr::compact_rows): the last subgraph output is a row mask that is
+// applied to every other output (see FuseMaskedSelect).
+// Stack protocol as GraphBuilder::runKernel (fait/fuser/graph_builder.cpp:901-927):
+// pops the arguments, pushes one IValue per output; outputs are freshly
+// allocated, inputs are never written.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/DeviceGuard.h>
+#include <torch/csrc/jit/ir/constants.h>
+#include <torch/csrc/jit/runtime/custom_operator.h>
+
+#include <mutex>
+#include <sstream>
+
+#include "../../../include/fxhip.h"
+#include "passes.h"
+#include "symbols.h"
+
+namespace functs {
+using namespace torch::jit;
+
+namespace {
+
+bool isTensorValue(const Value* v) { return v->type()->kind() == c10::TypeKind::TensorType; }
+
+// ---------------------------------------------------------------------------
+// pass: FusionGroup / ParallelMap -> ParallelFunctor
+// ---------------------------------------------------------------------------
+void cloneBlockInto(Block* src, Graph* sub, std::unordered_map<Value*, Value*>& map,
+                    const std::vector<Value*>* returns = nullptr) {
+  auto env = [&](Value* v) -> Value* {
+    auto it = map.find(v);
+    if (it != map.end()) return it->second;
+    if (v->node()->kind() == c10::prim::Constant) {
+      Node* c = sub->createClone(v->node(), [](Value* x) { return x; });
+      sub->prependNode(c);
+      map[v] = c->output();
+      return c->output();
+    }
+    TORCH_CHECK(false, "ParallelFunctor: free value %", v->debugName(), " in a fused region");
+  };
+  for (Node* n : src->nodes()) {
+    Node* c = sub->createClone(n, env);
+    sub->appendNode(c);
+    for (size_t i = 0; i < n->outputs().size(); ++i) map[n->output(i)] = c->output(i);
+  }
+  if (returns) {
+    for (Value* o : *returns) sub->registerOutput(env(o));
+  } else {
+    for (Value* o : src->outputs()) sub->registerOutput(env(o));
+  }
+}
+
+Node* functorFromGroup(Node* group) {
+  Graph* g = group->owningGraph();
+  Node* f = g->createWithSubgraph(sym::ParallelFunctor());
+  auto sub = f->g(c10::attr::Subgraph);
+  std::vector<c10::TypePtr> types;
+  for (Value* in : group->inputs()) {
+    f->addInput(in);
+    types.push_back(in->type());
+  }
+  f->tys_(sym::input_refine_types(), types);
+  f->i_(sym::parallel_degree(), 1);
+  f->i_(sym::is_parallel_map(), 0);
+  f->is_(sym::is_parallel_args(), std::vector<int64_t>(group->inputs().size(), 1));  // te_op.cpp:186-187
+  f->i_(sym::compact_rows(), group->hasAttribute(sym::compact_rows()) ? group->i(sym::compact_rows()) : 0);
+  for (Value* out : group->outputs()) f->addOutput()->copyMetadata(out);
+  std::unordered_map<Value*, Value*> map;
+  sub->addInput()->setType(c10::NoneType::get());  // placeholder for the task index (te_op.cpp:192)
+  Block* body = group->blocks()[0];
+  for (Value* p : body->inputs()) map[p] = sub->addInput()->copyMetadata(p);
+  cloneBlockInto(body, sub.get(), map);
+  return f;
+}
+
+// ParallelMap(len, lists...) { block(i, elems...): FusionGroup(...) -> rets }
+Node* functorFromMap(Node* mapNode, Node* group) {
+  Graph* g = mapNode->owningGraph();
+  Block* mb = mapNode->blocks()[0];
+  Block* body = group->blocks()[0];
+  Node* f = g->createWithSubgraph(sym::ParallelFunctor());
+  auto sub = f->g(c10::attr::Subgraph);
+  auto len = constant_as<int64_t>(mapNode->input(0));
+  f->i_(sym::parallel_degree(), len ? *len : -1);
+  f->i_(sym::is_parallel_map(), 1);
+  f->i_(sym::compact_rows(), group->hasAttribute(sym::compact_rows()) ? group->i(sym::compact_rows()) : 0);
+  if (!len) f->addInput(mapNode->input(0));  // trip count travels as the leading argument
+  std::vector<int64_t> par;
+  std::vector<c10::TypePtr> types;
+  std::unordered_map<Value*, Value*> map;
+  Value* idx = sub->addInput()->setType(c10::IntType::get());
+  // subgraph parameters follow the group's inputs; what they are bound to decides the kind
+  std::vector<Value*> params_in_order;
+  for (size_t k = 0; k < group->inputs().size(); ++k) {
+    Value* in = group->input(k);
+    Value* p = body->inputs()[k];
+    if (in == mb->inputs()[0]) {  // the loop index
+      map[p] = idx;
+      continue;
+    }
+    Value* sp = sub->addInput()->copyMetadata(p);
+    map[p] = sp;
+    auto pos = std::find(mb->inputs().begin() + 1, mb->inputs().end(), in);
+    if (pos != mb->inputs().end()) {
+      size_t li = pos - mb->inputs().begin();  // list argument of the map
+      f->addInput(mapNode->input(li));
+      types.push_back(mapNode->input(li)->type());
+      par.push_back(1);
+    } else {
+      TORCH_CHECK(in->node()->owningBlock() != mb, "ParallelMap: group input defined inside the map body");
+      f->addInput(in);
+      types.push_back(in->type());
+      par.push_back(0);
+    }
+  }
+  f->is_(sym::is_parallel_args(), par);
+  f->tys_(sym::input_refine_types(), types);
+  for (Value* out : mapNode->outputs()) f->addOutput()->copyMetadata(out);
+  // the map returns group outputs in its own order; the row mask stays last
+  std::vector<Value*> returns;
+  for (Value* r : mb->outputs()) returns.push_back(body->outputs()[r->offset()]);
+  if (f->i(sym::compact_rows())) returns.push_back(body->outputs().back());
+  cloneBlockInto(body, sub.get(), map, &returns);
+  return f;
+}
+
+// A map whose body did not end up as exactly one fused group goes back to a
+// loop (ConvertInfusibleMapsToLoops, parallelize_loops.cpp:295-362).
+Node* mapBackToLoop(Node* mapNode) {
+  Graph* g = mapNode->owningGraph();
+  Block* mb = mapNode->blocks()[0];
+  WithInsertPoint guard(mapNode);
+  std::vector<Value*> out_lists;
+  for (Value* o : mapNode->outputs()) {
+    auto lt = o->type()->cast<c10::ListType>();
+    Node* lc = g->createList(lt->getElementType(), {});
+    g->insertNode(lc);
+    lc->output()->setType(o->type());
+    out_lists.push_back(lc->output());
+  }
+  Value* ctrue = g->insertConstant(true);
+  Node* loop = g->create(c10::prim::Loop, {mapNode->input(0), ctrue}, 0);
+  g->insertNode(loop);
+  Block* lb = loop->addBlock();
+  Value* i = lb->addInput()->setType(c10::IntType::get());
+  std::unordered_map<Value*, Value*> map;
+  map[mb->inputs()[0]] = i;
+  for (size_t k = 1; k < mb->inputs().size(); ++k) {
+    Node* get = g->create(c10::aten::__getitem__, {mapNode->input(k), i}, 1);
+    get->output()->setType(mb->inputs()[k]->type());
+    lb->appendNode(get);
+    map[mb->inputs()[k]] = get->output();
+  }
+  auto env = [&](Value* v) -> Value* {
+    auto it = map.find(v);
+    return it != map.end() ? it->second : v;
+  };
+  for (Node* n : mb->nodes()) {
+    Node* c = g->createClone(n, env);
+    lb->appendNode(c);
+    for (size_t k = 0; k < n->outputs().size(); ++k) map[n->output(k)] = c->output(k);
+  }
+  for (size_t k = 0; k < out_lists.size(); ++k) {
+    Node* app = g->create(c10::aten::append, {out_lists[k], env(mb->outputs()[k])}, 1);
+    app->output()->setType(out_lists[k]->type());
+    lb->appendNode(app);
+  }
+  Node* ct = g->create(c10::prim::Constant, 1);
+  ct->output()->setType(c10::BoolType::get());
+  ct->ival_(c10::attr::value, true);
+  lb->appendNode(ct);
+  lb->registerOutput(ct->output());
+  for (size_t k = 0; k < out_lists.size(); ++k) mapNode->output(k)->replaceAllUsesWith(out_lists[k]);
+  mapNode->destroy();
+  return loop;
+}
+
+void toFunctorIn(Block* b) {
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    if (n->kind() == c10::prim::FusionGroup) {
+      Node* f = functorFromGroup(n);
+      f->insertBefore(n);
+      for (size_t k = 0; k < n->outputs().size(); ++k) n->output(k)->replaceAllUsesWith(f->output(k));
+      n->destroy();
+      continue;
+    }
+    if (n->kind() == sym::ParallelMap()) {
+      Block* mb = n->blocks()[0];
+      Node* group = nullptr;
+      bool single = true;
+      for (Node* m : mb->nodes()) {
+        if (m->kind() == c10::prim::Constant) continue;
+        if (m->kind() == c10::prim::FusionGroup && !group) group = m;
+        else single = false;
+      }
+      if (group && single)  // every value the map returns comes out of the group
+        for (Value* r : mb->outputs()) single = single && r->node() == group;
+      if (group && single) {
+        Node* f = functorFromMap(n, group);
+        f->insertBefore(n);
+        for (size_t k = 0; k < n->outputs().size(); ++k) n->output(k)->replaceAllUsesWith(f->output(k));
+        n->destroy();
+      } else {
+        Node* loop = mapBackToLoop(n);
+        toFunctorIn(loop->blocks()[0]);
+      }
+      continue;
+    }
+    for (Block* inner : n->blocks()) toFunctorIn(inner);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// run time: subgraph -> fx_region (C ABI), argument marshalling, launch
+// ---------------------------------------------------------------------------
+int fxDtype(c10::ScalarType t) {
+  switch (t) {
+    case c10::kFloat: return FX_DT_F32;
+    case c10::kLong: return FX_DT_I64;
+    case c10::kInt: return FX_DT_I32;
+    case c10::kByte: return FX_DT_U8;
+    case c10::kHalf: return FX_DT_F16;
+    case c10::kBFloat16: return FX_DT_BF16;
+    case c10::kBool: return FX_DT_BOOL;
+    default: TORCH_CHECK(false, "fused regions do not support dtype ", t);
+  }
+}
+c10::ScalarType atDtype(int d) {
+  switch (d) {
+    case FX_DT_F32: return c10::kFloat;
+    case FX_DT_I64: return c10::kLong;
+    case FX_DT_I32: return c10::kInt;
+    case FX_DT_U8: return c10::kByte;
+    case FX_DT_F16: return c10::kHalf;
+    case FX_DT_BF16: return c10::kBFloat16;
+    case FX_DT_BOOL: return c10::kBool;
+  }
+  TORCH_CHECK(false, "bad fx dtype");
+}
+
+#define FX_OK_OR_THROW(expr)                                            \
+  do {                                                                  \
+    int rc__ = (expr);                                                  \
+    TORCH_CHECK(rc__ >= 0, "fxhip: ", fx_last_error(), " (", #expr, ")"); \
+  } while (0)
+
+struct Variant {
+  fx_region* region = nullptr;
+  ~Variant() {
+    if (region) fx_region_destroy(region);
+  }
+};
+
+class RegionRunner {
+ public:
+  explicit RegionRunner(const Node* node)
+      : graph_(node->g(c10::attr::Subgraph)),
+        is_par_(node->is(sym::is_parallel_args())),
+        degree_(node->i(sym::parallel_degree())),
+        is_map_(node->i(sym::is_parallel_map()) != 0),
+        compact_(node->hasAttribute(sym::compact_rows()) && node->i(sym::compact_rows()) != 0) {
+    n_args_ = graph_->inputs().size() - 1;
+    TORCH_CHECK(is_par_.size() == n_args_, "ParallelFunctor: is_parallel_args does not match the subgraph");
+    n_stack_ = n_args_ + (degree_ < 0 ? 1 : 0);
+    n_outs_ = graph_->outputs().size() - (compact_ ? 1 : 0);
+  }
+
+  void run(Stack& stack) {
+    auto inputs = last(stack, n_stack_);
+    int64_t degree = degree_;
+    size_t first = 0;
+    if (degree_ < 0) {
+      degree = inputs[0].toInt();
+      first = 1;
+    }
+    if (!is_map_) degree = 1;
+    TORCH_CHECK(degree >= 0, "ParallelFunctor: negative trip count");
+    if (degree == 0) {  // an empty map
+      drop(stack, n_stack_);
+      for (size_t o = 0; o < n_outs_; ++o) push(stack, c10::List<at::Tensor>());
+      return;
+    }
+    // flatten arguments
+    std::vector<fx_arg> args;
+    std::vector<at::Tensor> keep;
+    std::ostringstream sig;
+    sig << degree;
+    c10::Device device(c10::kCPU);
+    bool have_device = false;
+    auto addTensor = [&](const at::Tensor& t) {
+      TORCH_CHECK(t.is_cuda(), "tssa::ParallelFunctor runs on the GPU only; got a ", t.device(), " tensor");
+      TORCH_CHECK(t.dim() <= FX_ARG_MAX_RANK, "tensor rank above ", FX_ARG_MAX_RANK);
+      if (!have_device) { device = t.device(); have_device = true; }
+      fx_arg a;
+      memset(&a, 0, sizeof(a));
+      a.kind = 0;
+      a.dtype = fxDtype(t.scalar_type());
+      a.ptr = t.data_ptr();
+      a.rank = (int32_t)t.dim();
+      for (int64_t d = 0; d < t.dim(); ++d) { a.sizes[d] = t.size(d); a.strides[d] = t.stride(d); }
+      args.push_back(a);
+      sig << "|t" << a.dtype << "r" << a.rank;
+    };
+    auto addScalar = [&](const c10::IValue& v) {
+      fx_arg a;
+      memset(&a, 0, sizeof(a));
+      if (v.isDouble()) { a.kind = 2; a.fval = v.toDouble(); sig << "|f"; }
+      else if (v.isBool()) { a.kind = 3; a.ival = v.toBool(); sig << "|b"; }
+      else if (v.isInt()) { a.kind = 1; a.ival = v.toInt(); sig << "|i"; }
+      else TORCH_CHECK(false, "ParallelFunctor: unsupported scalar argument ", v.tagKind());
+      args.push_back(a);
+    };
+    for (size_t k = 0; k < n_args_; ++k) {
+      const c10::IValue& v = inputs[first + k];
+      const bool per_task = is_map_ && is_par_[k] != 0;
+      if (per_task) {
+        TORCH_CHECK(v.isList(), "ParallelFunctor: argument ", k, " must be a list with one entry per task");
+        auto lst = v.toListRef();
+        TORCH_CHECK((int64_t)lst.size() >= degree, "ParallelFunctor: list argument ", k, " is shorter than the trip count");
+        for (int64_t t = 0; t < degree; ++t) {
+          if (lst[t].isTensor()) addTensor(lst[t].toTensor());
+          else addScalar(lst[t]);
+        }
+      } else if (v.isTensor()) {
+        addTensor(v.toTensor());
+      } else {
+        addScalar(v);
+      }
+    }
+    TORCH_CHECK(have_device, "ParallelFunctor: a region needs at least one tensor argument");
+    c10::DeviceGuard guard(device);
+
+    Variant* var;
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      auto& slot = variants_[sig.str()];
+      if (!slot) {
+        slot = std::make_unique<Variant>();
+        build(*slot, degree, inputs, first);
+      }
+      var = slot.get();
+    }
+    const fx_plan* plan = nullptr;
+    FX_OK_OR_THROW(fx_region_plan(var->region, args.data(), (int)args.size(), &plan));
+    const int n_out = fx_plan_num_outputs(plan);
+    std::vector<std::vector<at::Tensor>> outs(n_out);
+    std::vector<void*> ptrs((size_t)n_out * degree);
+    for (int o = 0; o < n_out; ++o) {
+      for (int64_t t = 0; t < degree; ++t) {
+        int32_t dt, rank;
+        int64_t sizes[FX_ARG_MAX_RANK];
+        FX_OK_OR_THROW(fx_plan_output(plan, o, (int)t, &dt, &rank, sizes));
+        at::Tensor ten = at::empty(at::IntArrayRef(sizes, rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
+        ptrs[(size_t)o * degree + t] = ten.data_ptr();
+        outs[o].push_back(std::move(ten));
+      }
+    }
+    at::Tensor scratch, totals;
+    const size_t sb = fx_plan_scratch_bytes(plan);
+    if (compact_) {
+      scratch = at::empty({(int64_t)std::max<size_t>(sb, 1)}, at::TensorOptions().dtype(at::kByte).device(device));
+      totals = at::empty({degree}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+    }
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
+    FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
+                                 compact_ ? scratch.data_ptr() : nullptr,
+                                 compact_ ? (uint32_t*)totals.data_ptr() : nullptr, (void*)stream.stream()));
+    if (compact_) {
+      // the kept-row counts decide the output shapes: one synchronisation, as ATen's
+      // nonzero / masked index does
+      stream.synchronize();
+      const int32_t* tot = totals.data_ptr<int32_t>();
+      for (int o = 0; o < n_out; ++o)
+        for (int64_t t = 0; t < degree; ++t) outs[o][t] = outs[o][t].narrow(0, 0, tot[t]);
+    }
+    drop(stack, n_stack_);
+    for (int o = 0; o < n_out; ++o) {
+      if (is_map_) push(stack, c10::List<at::Tensor>(std::move(outs[o])));
+      else push(stack, std::move(outs[o][0]));
+    }
+  }
+
+ private:
+  std::shared_ptr<Graph> graph_;
+  std::vector<int64_t> is_par_;
+  int64_t degree_;
+  bool is_map_, compact_;
+  size_t n_args_ = 0, n_stack_ = 0, n_outs_ = 0;
+  std::mutex mu_;
+  std::map<std::string, std::unique_ptr<Variant>> variants_;
+
+  void build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue> inputs, size_t first);
+};
+
+// --- subgraph -> region -----------------------------------------------------
+struct Translator {
+  fx_region* r;
+  std::unordered_map<const Value*, int> ids;
+
+  int cint(int64_t v) { int id; FX_OK_OR_THROW(fx_region_const_int(r, v, &id)); return id; }
+  int cfloat(double v) { int id; FX_OK_OR_THROW(fx_region_const_float(r, v, &id)); return id; }
+  int cbool(bool v) { int id; FX_OK_OR_THROW(fx_region_const_bool(r, v, &id)); return id; }
+  int cnone() { int id; FX_OK_OR_THROW(fx_region_const_none(r, &id)); return id; }
+  int ilist(const std::vector<int>& v) { int id; FX_OK_OR_THROW(fx_region_int_list(r, v.data(), (int)v.size(), &id)); return id; }
+  int tlist(const std::vector<int>& v) { int id; FX_OK_OR_THROW(fx_region_tensor_list(r, v.data(), (int)v.size(), &id)); return id; }
+  int op(int code, std::vector<int> args, int dtype = -1) {
+    int id;
+    FX_OK_OR_THROW(fx_region_op(r, code, args.data(), (int)args.size(), dtype, &id));
+    return id;
+  }
+
+  int get(const Value* v) {
+    auto it = ids.find(v);
+    if (it != ids.end()) return it->second;
+    const Node* n = v->node();
+    TORCH_CHECK(n->kind() == c10::prim::Constant, "ParallelFunctor: value %", v->debugName(), " has no region value");
+    auto iv = toIValue(v);
+    TORCH_CHECK(iv, "bad constant");
+    int id;
+    if (iv->isNone()) id = cnone();
+    else if (iv->isBool()) id = cbool(iv->toBool());
+    else if (iv->isInt()) id = cint(iv->toInt());
+    else if (iv->isDouble()) id = cfloat(iv->toDouble());
+    else if (iv->isIntList()) {
+      std::vector<int> e;
+      for (int64_t x : iv->toIntVector()) e.push_back(cint(x));
+      id = ilist(e);
+    } else if (iv->isDevice() || iv->isString()) id = cnone();
+    else TORCH_CHECK(false, "ParallelFunctor: constant of type ", iv->tagKind(), " inside a fused region");
+    ids[v] = id;
+    return id;
+  }
+
+  // dtype argument (ScalarType constant or None) -> fx dtype or -1
+  int dtypeArg(const Value* v) {
+    auto iv = toIValue(v);
+    if (!iv || iv->isNone()) return -1;
+    return fxDtype(static_cast<c10::ScalarType>(iv->toInt()));
+  }
+
+  void node(const Node* n);
+  void block(const Block* b) {
+    for (const Node* n : b->nodes()) node(n);
+  }
+};
+
+void Translator::node(const Node* n) {
+  using namespace c10;
+  const Symbol k = n->kind();
+  auto in = [&](size_t i) { return get(n->input(i)); };
+  auto out = [&](int id) { ids[n->output(0)] = id; };
+  const size_t ni = n->inputs().size();
+  if (k == prim::Constant) return;  // created on demand
+  if (k == prim::ListConstruct) {
+    std::vector<int> e;
+    for (const Value* v : n->inputs()) e.push_back(get(v));
+    auto lt = n->output()->type()->cast<ListType>();
+    bool ints = lt && lt->getElementType()->kind() == TypeKind::IntType;
+    out(ints ? ilist(e) : tlist(e));
+    return;
+  }
+  struct Simple { Symbol s; int code; };
+  static const std::vector<Simple> unary{
+      {aten::exp, FX_OP_EXP}, {aten::log, FX_OP_LOG}, {aten::sqrt, FX_OP_SQRT}, {aten::rsqrt, FX_OP_RSQRT},
+      {aten::sigmoid, FX_OP_SIGMOID}, {aten::tanh, FX_OP_TANH}, {aten::relu, FX_OP_RELU}, {aten::abs, FX_OP_ABS},
+      {aten::floor, FX_OP_FLOOR}, {aten::ceil, FX_OP_CEIL}, {aten::round, FX_OP_ROUND}, {aten::sin, FX_OP_SIN},
+      {aten::cos, FX_OP_COS}, {aten::erf, FX_OP_ERF}, {aten::reciprocal, FX_OP_RECIPROCAL},
+      {aten::logical_not, FX_OP_LOGICAL_NOT}, {sym::Access(), FX_OP_ACCESS}};
+  for (auto& u : unary)
+    if (u.s == k) { out(op(u.code, {in(0)})); return; }
+  static const std::vector<Simple> binary{
+      {aten::mul, FX_OP_MUL}, {aten::div, FX_OP_DIV}, {aten::maximum, FX_OP_MAXIMUM}, {aten::minimum, FX_OP_MINIMUM},
+      {aten::pow, FX_OP_POW}, {aten::eq, FX_OP_EQ}, {aten::ne, FX_OP_NE}, {aten::lt, FX_OP_LT}, {aten::le, FX_OP_LE},
+      {aten::gt, FX_OP_GT}, {aten::ge, FX_OP_GE}, {aten::__and__, FX_OP_AND}, {aten::__or__, FX_OP_OR},
+      {aten::__xor__, FX_OP_XOR}};
+  const bool tensor_out = isTensorValue(n->output(0));
+  if (!tensor_out && n->output(0)->type()->kind() == TypeKind::IntType) {
+    // integer scalar arithmetic on index values
+    if (k == aten::add) { out(op(FX_OP_INT_ADD, {in(0), in(1)})); return; }
+    if (k == aten::sub) { out(op(FX_OP_INT_SUB, {in(0), in(1)})); return; }
+    if (k == aten::mul) { out(op(FX_OP_INT_MUL, {in(0), in(1)})); return; }
+    if (k == aten::neg) { out(op(FX_OP_INT_NEG, {in(0)})); return; }
+    if (k == aten::size) { out(op(FX_OP_SIZE, {in(0), in(1)})); return; }
+    if (k == aten::__derive_index) {  // start + index * step
+      out(op(FX_OP_INT_ADD, {in(1), op(FX_OP_INT_MUL, {in(0), in(2)})}));
+      return;
+    }
+  }
+  for (auto& b : binary)
+    if (b.s == k) { out(op(b.code, {in(0), in(1)})); return; }
+  if (k == aten::add || k == aten::sub || k == aten::rsub) {
+    int code = k == aten::add ? FX_OP_ADD : (k == aten::sub ? FX_OP_SUB : FX_OP_RSUB);
+    out(ni > 2 ? op(code, {in(0), in(1), in(2)}) : op(code, {in(0), in(1)}));
+    return;
+  }
+  if (k == aten::neg) { out(op(FX_OP_NEG, {in(0)})); return; }
+  if (k == aten::clone || k == aten::contiguous) { out(op(FX_OP_CLONE, {in(0)})); return; }
+  if (k == sym::Assign()) { out(op(FX_OP_ASSIGN, {in(0), in(1)})); return; }
+  if (k == aten::select || k == sym::Select()) { out(op(FX_OP_SELECT, {in(0), in(1), in(2)})); return; }
+  if (k == sym::SelectRev()) { out(op(FX_OP_SELECT_REV, {in(0), in(1), in(2), in(3)})); return; }
+  if (k == aten::slice || k == sym::Slice()) { out(op(FX_OP_SLICE, {in(0), in(1), in(2), in(3), in(4)})); return; }
+  if (k == sym::SliceRev()) { out(op(FX_OP_SLICE_REV, {in(0), in(1), in(2), in(3), in(4), in(5)})); return; }
+  if (k == aten::squeeze || k == sym::Squeeze()) {
+    TORCH_CHECK(ni == 2, "squeeze without a dim inside a fused region");
+    out(op(FX_OP_SQUEEZE, {in(0), in(1)}));
+    return;
+  }
+  if (k == aten::unsqueeze || k == sym::Unsqueeze()) { out(op(FX_OP_UNSQUEEZE, {in(0), in(1)})); return; }
+  if (k == aten::view || k == aten::reshape || k == sym::View() || k == sym::Reshape()) {
+    out(op(FX_OP_VIEW, {in(0), in(1)}));
+    return;
+  }
+  if (k == aten::permute || k == sym::Permute()) { out(op(FX_OP_PERMUTE, {in(0), in(1)})); return; }
+  if (k == aten::transpose) { out(op(FX_OP_TRANSPOSE, {in(0), in(1), in(2)})); return; }
+  if (k == aten::expand || k == sym::Expand()) { out(op(FX_OP_EXPAND, {in(0), in(1)})); return; }
+  if (k == aten::expand_as || k == sym::ExpandAs()) { out(op(FX_OP_EXPAND_AS, {in(0), in(1)})); return; }
+  if (k == aten::repeat || k == sym::Repeat()) { out(op(FX_OP_REPEAT, {in(0), in(1)})); return; }
+  if (k == aten::index || k == sym::Index()) { out(op(FX_OP_INDEX, {in(0), in(1)})); return; }
+  if (k == aten::cat) { out(op(FX_OP_CAT, {in(0), in(1)})); return; }
+  if (k == aten::stack) { out(op(FX_OP_STACK, {in(0), in(1)})); return; }
+  if (k == aten::triu) { out(op(FX_OP_TRIU, {in(0), in(1)})); return; }
+  if (k == aten::clamp) { out(op(FX_OP_CLAMP, {in(0), in(1), in(2)})); return; }
+  if (k == aten::where) { out(op(FX_OP_WHERE, {in(0), in(1), in(2)})); return; }
+  if (k == aten::softmax) { out(op(FX_OP_SOFTMAX, {in(0), in(1)})); return; }
+  if (k == aten::max) {
+    TORCH_CHECK(ni >= 2 && n->outputs().size() == 2 && !n->output(1)->hasUses(),
+                "aten::max.dim: only the values output can be fused");
+    out(op(FX_OP_MAX_DIM, {in(0), in(1), ni > 2 ? in(2) : cbool(false)}));
+    return;
+  }
+  if (k == aten::zeros || k == aten::ones) {
+    int dt = dtypeArg(n->input(1));
+    out(op(FX_OP_FULL, {in(0), cfloat(k == aten::ones ? 1.0 : 0.0)}, dt < 0 ? FX_DT_F32 : dt));
+    return;
+  }
+  if (k == aten::full) {
+    int dt = dtypeArg(n->input(2));
+    out(op(FX_OP_FULL, {in(0), in(1)}, dt < 0 ? FX_DT_F32 : dt));
+    return;
+  }
+  if (k == aten::zeros_like || k == aten::ones_like) {
+    auto tt = n->input(0)->type()->cast<TensorType>();
+    TORCH_CHECK(tt && tt->dim(), "zeros_like: the rank of the argument must be known");
+    std::vector<int> dims;
+    for (size_t d = 0; d < *tt->dim(); ++d) dims.push_back(op(FX_OP_SIZE, {in(0), cint((int64_t)d)}));
+    int dt = dtypeArg(n->input(1));
+    if (dt < 0 && tt->scalarType()) dt = fxDtype(*tt->scalarType());
+    out(op(FX_OP_FULL, {ilist(dims), cfloat(k == aten::ones_like ? 1.0 : 0.0)}, dt < 0 ? FX_DT_F32 : dt));
+    return;
+  }
+  if (k == aten::arange) {
+    TORCH_CHECK(ni >= 3, "aten::arange: only the (start, end, ...) form can be fused");
+    int dt = dtypeArg(n->input(2));
+    out(op(FX_OP_ARANGE, {in(0), in(1)}, dt < 0 ? FX_DT_I64 : dt));
+    return;
+  }
+  if (k == aten::tensor) {
+    int dt = dtypeArg(n->input(1));
+    out(op(FX_OP_SCALAR_TENSOR, {in(0)}, dt));
+    return;
+  }
+  if (k == aten::to) {
+    // to.dtype(self, dtype, ...) / to.device(self, device, dtype, ...)
+    int dt = -1;
+    for (size_t i = 1; i < ni && dt < 0; ++i)
+      if (n->input(i)->type()->kind() == TypeKind::IntType) dt = dtypeArg(n->input(i));
+    TORCH_CHECK(dt >= 0, "aten::to without a dtype inside a fused region");
+    out(op(FX_OP_TO, {in(0)}, dt));
+    return;
+  }
+  if (k == sym::ForallSelectRev()) {
+    // (T0, dim, lo, hi, captured...) { block(i, T, captured'...) -> src }
+    const Block* b = n->blocks()[0];
+    int lv;
+    FX_OK_OR_THROW(fx_region_loop_var(r, &lv));
+    ids[b->inputs()[0]] = lv;
+    ids[b->inputs()[1]] = in(0);
+    for (size_t c = 2; c < b->inputs().size(); ++c) ids[b->inputs()[c]] = in(2 + c);
+    block(b);
+    out(op(FX_OP_FORALL_SELECT_REV, {in(0), get(b->outputs()[0]), in(1), in(2), in(3)}));
+    return;
+  }
+  TORCH_CHECK(false, "ParallelFunctor: no lowering for ", k.toQualString());  // graph_builder.cpp:409-414
+}
+
+void RegionRunner::build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue> inputs, size_t first) {
+  FX_OK_OR_THROW(fx_region_create((int)degree, is_map_ ? 1 : 0, &var.region));
+  Translator tr{var.region, {}};
+  // input 0: the task index
+  const Value* idx = graph_->inputs()[0];
+  if (idx->type()->kind() == c10::TypeKind::IntType) {
+    int id;
+    FX_OK_OR_THROW(fx_region_task_index(var.region, &id));
+    tr.ids[idx] = id;
+  }
+  for (size_t k = 0; k < n_args_; ++k) {
+    const Value* p = graph_->inputs()[k + 1];
+    const c10::IValue& v = inputs[first + k];
+    const bool per_task = is_map_ && is_par_[k] != 0;
+    c10::IValue sample = v;
+    if (per_task) sample = v.toListRef().at(0);
+    int id;
+    if (sample.isTensor()) {
+      const at::Tensor& t = sample.toTensor();
+      FX_OK_OR_THROW(fx_region_input_tensor(var.region, fxDtype(t.scalar_type()), (int)t.dim(), per_task, &id));
+    } else {
+      int kind = sample.isDouble() ? 2 : (sample.isBool() ? 3 : 1);
+      FX_OK_OR_THROW(fx_region_input_scalar(var.region, kind, per_task, &id));
+    }
+    tr.ids[p] = id;
+  }
+  tr.block(graph_->block());
+  const size_t n_sub_out = graph_->outputs().size();
+  for (size_t o = 0; o < n_sub_out; ++o) {
+    int id = tr.get(graph_->outputs()[o]);
+    if (compact_ && o + 1 == n_sub_out) FX_OK_OR_THROW(fx_region_compact_rows(var.region, id));
+    else FX_OK_OR_THROW(fx_region_output(var.region, id));
+  }
+  FX_OK_OR_THROW(fx_region_finalize(var.region));
+}
+
+Operation createParallelFunctor(const Node* node) {
+  auto runner = std::make_shared<RegionRunner>(node);
+  return [runner](Stack& stack) { runner->run(stack); };
+}
+
+RegisterOperators registerFunctor({
+    Operator(sym::ParallelFunctor(), createParallelFunctor, c10::AliasAnalysisKind::PURE_FUNCTION),
+});
+
+}  // namespace
+
+void ToParallelFunctor(std::shared_ptr<Graph> graph) { toFunctorIn(graph->block()); }
+
+std::string fxhipLibraryPath() { return "functs_amd/lib/libfxhip.so"; }
+
+}  // namespace functs

@@ -1,0 +1,111 @@
+"""TorchScript front end: functionalize a program and run its fused regions on
+the GPU through ``tssa::ParallelFunctor``.
+
+Same entry points as the reference's ``functs.jit`` (functs/jit/_script.py:12-110):
+``script`` functionalizes, ``build`` forms regions and returns a callable,
+``shape_infer`` refines the graph's argument types from example inputs.
+"""
+import inspect
+from typing import List, Sequence
+
+import torch
+
+from . import _C  # noqa: F401  (registers immut:: operators and tssa::ParallelFunctor)
+
+
+class AotScriptFunction(object):
+    """Callable around the compiled graph (functs/jit/_script.py:12-26)."""
+
+    def __init__(self, aot_script_fn, **kwargs):
+        self._aot_script_fn = aot_script_fn
+
+    @property
+    def graph(self):
+        return self._aot_script_fn.graph
+
+    def __call__(self, *args, **kwargs):
+        return self._aot_script_fn(*args, **kwargs)
+
+
+def extract_type_hint_from_tensor(input_):
+    """functs/jit/_script.py:29-49"""
+    if isinstance(input_, bool):
+        return torch.BoolType.get()
+    if isinstance(input_, int):
+        return torch.IntType.get()
+    if isinstance(input_, float):
+        return torch.FloatType.get()
+    if isinstance(input_, torch.Tensor):
+        return torch.TensorType.get().with_dtype(input_.dtype).with_sizes(list(input_.shape)).with_device(input_.device)
+    if isinstance(input_, (list, tuple)):
+        return torch.TupleType([extract_type_hint_from_tensor(e) for e in input_])
+    raise TypeError("unsupported type {} at the type hint stage".format(type(input_)))
+
+
+def _graph_of(fn):
+    if isinstance(fn, AotScriptFunction):
+        return fn.graph
+    return fn.graph
+
+
+def shape_infer(fn, example_input: Sequence[object], refined_types=None) -> None:
+    """Give the graph's tensor arguments the dtype / rank / device of the examples
+    (functs/jit/_script.py:52-55).  Regions specialise on the shapes they are
+    called with, so nothing else has to be propagated ahead of time."""
+    g = _graph_of(fn)
+    hints = [extract_type_hint_from_tensor(i) for i in example_input]
+    inputs = list(g.inputs())
+    off = len(inputs) - len(hints)
+    for v, t in zip(inputs[off:], hints):
+        if isinstance(t, torch.TensorType):
+            v.setType(t)
+
+
+def _strip_self(g):
+    inputs = list(g.inputs())
+    if inputs and inputs[0].debugName().startswith("self") and not inputs[0].uses():
+        g.eraseInput(0)
+
+
+def build(fn, example_input: List[object]) -> AotScriptFunction:
+    """Form fused regions in a functionalized script and return the callable
+    (functs/jit/_script.py:58-73)."""
+    if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
+        raise AttributeError("only a functionalized jit script can be built")
+    g = fn.graph.copy()
+    if isinstance(fn, torch.jit.ScriptModule):
+        _strip_self(g)
+    hints = [extract_type_hint_from_tensor(i) for i in example_input]
+    _C._jit_pass_fait_pipeline(g, hints)
+    return AotScriptFunction(_C._create_function_from_graph("forward", g))
+
+
+def script(fn, backend="jit", remove_update=True, enable_dce_cse=True, add_clone=False):
+    """TorchScript-compile ``fn`` and rewrite every tensor mutation into
+    immut:: Access / Assign chains (functs/jit/_script.py:76-110)."""
+    if backend not in ("jit", "aot"):
+        raise AttributeError("No backend named {}".format(backend))
+    jit_fn = torch.jit.script(fn)
+    is_function = inspect.isfunction(fn)
+    if is_function:
+        # torch.jit.script hands out one cached ScriptFunction per Python function, and
+        # its executor may already hold a plan: rewrite a private copy of the graph
+        g = jit_fn.graph.copy()
+    else:
+        if torch.cuda.is_available():
+            jit_fn = jit_fn.cuda()
+        jit_fn = torch.jit.freeze(jit_fn.eval())
+        g = jit_fn.graph
+    if add_clone:
+        _C._jit_pass_dumb_remove_inter_precedure_mutation(g)
+    torch._C._jit_pass_inline(g)
+    _C._jit_pass_convert_to_tensorssa(g)
+    if remove_update:
+        _C._jit_pass_tensorssa_remove_update(g)
+    if enable_dce_cse:
+        torch._C._jit_pass_dce(g)
+        torch._C._jit_pass_cse(g)
+        torch._C._jit_pass_constant_propagation(g)
+    if is_function:
+        return torch._C._create_function_from_graph(fn.__name__, g)
+    return jit_fn

@@ -1,0 +1,200 @@
+"""The TorchScript route: functs_amd.jit.script -> build (region formation ->
+tssa::ParallelFunctor).  CPU tests check the graphs; the gpu tests run the built
+functions on cuda:0 against stock TorchScript on the CPU (the oracle)."""
+import pytest
+import torch
+
+import functs_amd.jit as fj
+from functs_amd import _C
+from oracle import configs as oc
+from tests.util import assert_close, assert_exact, assert_boxes_close
+
+SMALL_GRIDS = [2, 3, 4]
+
+
+def _functors(graph):
+    out = []
+
+    def walk(block):
+        for n in block.nodes():
+            if n.kind() == "tssa::ParallelFunctor":
+                out.append(n)
+            for b in n.blocks():
+                walk(b)
+
+    walk(graph)
+    return out
+
+
+def _kinds(block, out=None):
+    out = [] if out is None else out
+    for n in block.nodes():
+        out.append(n.kind())
+        for b in n.blocks():
+            _kinds(b, out)
+    return out
+
+
+def _built(name, args):
+    return fj.build(fj.script(oc.CONFIGS[name][0]), list(args))
+
+
+def test_c1_is_one_functor_with_a_collapsed_loop():
+    args = oc.c1_inputs(0, 64)
+    f = _built("c1", args)
+    fs = _functors(f.graph)
+    assert len(fs) == 1 and "prim::Loop" not in _kinds(f.graph)
+    n = fs[0]
+    assert n.i("is_parallel_map") == 0 and n.i("parallel_degree") == 1
+    assert list(getattr(n, "is")("is_parallel_args")) == [1] * len(list(n.inputs()))
+    sub = n.g("Subgraph")
+    assert next(sub.inputs()).type().kind() == "NoneType"  # task-index placeholder (te_op.cpp:192)
+    assert "fx::forall_select_rev" in _kinds(sub)
+
+
+def test_c2_folds_the_row_mask_into_the_region():
+    args = oc.c2_inputs(0, SMALL_GRIDS)
+    f = _built("c2", args)
+    fs = _functors(f.graph)
+    assert len(fs) == 1
+    assert fs[0].i("compact_rows") == 1
+    assert "aten::index" not in _kinds(f.graph)
+    sub = fs[0].g("Subgraph")
+    assert len(list(sub.outputs())) == len(list(fs[0].outputs())) + 1  # mask rides last
+    assert list(sub.outputs())[-1].node().kind() == "aten::ge"
+
+
+def test_c5_is_one_parallel_map_functor():
+    args = oc.c5_inputs(0, SMALL_GRIDS, 3)
+    f = _built("c5", args)
+    fs = _functors(f.graph)
+    kinds = _kinds(f.graph)
+    assert len(fs) == 1 and "prim::Loop" not in kinds and "aten::append" not in kinds
+    n = fs[0]
+    assert n.i("is_parallel_map") == 1 and n.i("compact_rows") == 1
+    assert list(getattr(n, "is")("is_parallel_args")) == [0, 0, 0]  # preds, anchors, strides are shared
+    sub = n.g("Subgraph")
+    assert next(sub.inputs()).type().kind() == "IntType"  # the task index
+    for o in n.outputs():
+        assert o.type().kind() == "ListType"
+
+
+def test_c3_is_decode_plus_class_map():
+    args = oc.c3_inputs(0, 60, 7)
+    f = _built("c3", args)
+    fs = _functors(f.graph)
+    assert [n.i("is_parallel_map") for n in fs] == [0, 1]
+    assert [n.i("compact_rows") for n in fs] == [0, 1]
+    assert "aten::softmax" in _kinds(fs[0].g("Subgraph"))
+
+
+def test_unfusable_map_body_returns_to_a_loop():
+    def prog(x: torch.Tensor):
+        out = []
+        for i in range(x.size(0)):
+            r = x[i] * 2 + 1
+            out.append(torch.nonzero(r).float().sigmoid().exp())
+        return out
+
+    f = fj.build(fj.script(prog), [torch.rand(3, 8)])
+    kinds = _kinds(f.graph)
+    assert "prim::ParallelMap" not in kinds and "prim::FusionGroup" not in kinds
+    assert "prim::Loop" in kinds and "aten::nonzero" in kinds
+    _C._jit_pass_validate(f.graph)
+
+
+def test_single_elementwise_op_is_left_to_aten():
+    def prog(x: torch.Tensor):
+        return x.sigmoid()
+
+    f = fj.build(fj.script(prog), [torch.rand(3, 8)])
+    assert not _functors(f.graph)
+    assert torch.equal(f(torch.ones(2, 2)), torch.ones(2, 2).sigmoid())
+
+
+def test_functor_refuses_cpu_tensors():
+    f = _built("c1", oc.c1_inputs(0, 64))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        f(*oc.c1_inputs(0, 64))
+
+
+def test_validate_rejects_use_before_definition():
+    g = torch._C.parse_ir("""
+graph(%a : Tensor):
+  %one : int = prim::Constant[value=1]()
+  %c : Tensor = aten::add(%a, %a, %one)
+  %b : Tensor = aten::mul(%c, %a)
+  return (%b)""")
+    _C._jit_pass_validate(g)
+    nodes = [n for n in g.nodes() if n.kind() in ("aten::add", "aten::mul")]
+    nodes[1].moveBefore(nodes[0])
+    with pytest.raises(RuntimeError, match="before it is defined"):
+        _C._jit_pass_validate(g)
+
+
+# --------------------------------------------------------------------------- gpu
+def _cuda(args):
+    return [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
+
+
+def _cpu(x):
+    if isinstance(x, (list, tuple)):
+        return [_cpu(t) for t in x]
+    return x.cpu()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", [64, 1024])
+def test_c1_torchscript_gpu(size):
+    args = oc.c1_inputs(0, size)
+    ref = oc.run("c1", *args)
+    got = _built("c1", args)(*_cuda(args))
+    assert_exact(got.cpu(), ref, "c1")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("grids", [SMALL_GRIDS, oc.YOLO_GRIDS])
+def test_c2_torchscript_gpu(grids):
+    args = oc.c2_inputs(0, grids)
+    assert oc.threshold_margin(torch.sigmoid(args[0][..., 4]), 0.3) > 1e-6
+    rb, rc, ro = oc.run("c2", *args)
+    f = _built("c2", args)
+    for _ in range(2):  # the second call reuses the compiled variant
+        gb, gc, go = _cpu(f(*_cuda(args)))
+        assert_boxes_close(gb, rb, "c2 boxes")
+        assert_close(gc, rc, "c2 cls")
+        assert_close(go, ro, "c2 obj")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("grids,batch", [(SMALL_GRIDS, 3), (oc.YOLO_GRIDS, 16)])
+def test_c5_torchscript_gpu(grids, batch):
+    args = oc.c5_inputs(0, grids, batch)
+    rb, rc, ro = oc.run("c5", *args)
+    gb, gc, go = _cpu(_built("c5", args)(*_cuda(args)))
+    assert_boxes_close(gb, list(rb), "c5 boxes")
+    assert_close(gc, list(rc), "c5 cls")
+    assert_close(go, list(ro), "c5 obj")
+
+
+@pytest.mark.gpu
+def test_c5_torchscript_gpu_new_batch_size_same_function():
+    """parallel_degree is taken from the trip count at run time."""
+    args3 = oc.c5_inputs(0, SMALL_GRIDS, 3)
+    f = _built("c5", args3)
+    for batch in (3, 5, 1):
+        args = oc.c5_inputs(batch, SMALL_GRIDS, batch)
+        rb, rc, ro = oc.run("c5", *args)
+        gb, gc, go = _cpu(f(*_cuda(args)))
+        assert_boxes_close(gb, list(rb), "c5 boxes b=%d" % batch)
+        assert_close(go, list(ro), "c5 obj b=%d" % batch)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_priors,n_cls", [(60, 7), (8732, 81)])
+def test_c3_torchscript_gpu(n_priors, n_cls):
+    args = oc.c3_inputs(0, n_priors, n_cls)
+    rb, rs = oc.run("c3", *args)
+    gb, gs = _cpu(_built("c3", args)(*_cuda(args)))
+    assert_close(gb, list(rb), "c3 boxes", rtol=1e-5, atol=1e-6)
+    assert_close(gs, list(rs), "c3 scores")

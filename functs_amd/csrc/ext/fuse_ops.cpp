@@ -28,7 +28,7 @@ bool isTensorValue(const Value* v) { return v->type()->kind() == c10::TypeKind::
 const std::unordered_set<Symbol>& fusableSymbols() {
   using namespace c10;
   static const std::unordered_set<Symbol> s{
-      aten::clone, aten::contiguous, aten::to, aten::zeros, aten::ones, aten::full, aten::zeros_like,
+      aten::clone, aten::contiguous, aten::to, aten::zeros, aten::ones, aten::full, aten::full_like, aten::zeros_like,
       aten::ones_like, aten::arange, aten::tensor, aten::exp, aten::sigmoid, aten::tanh, aten::relu, aten::neg,
       aten::abs, aten::sqrt, aten::rsqrt, aten::log, aten::reciprocal, aten::floor, aten::ceil, aten::round,
       aten::sin, aten::cos, aten::erf, aten::triu, aten::clamp, aten::add, aten::sub, aten::rsub, aten::mul,

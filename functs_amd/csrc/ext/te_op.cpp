@@ -552,13 +552,11 @@ void Translator::node(const Node* n) {
     return;
   }
   if (k == aten::zeros_like || k == aten::ones_like) {
-    auto tt = n->input(0)->type()->cast<TensorType>();
-    TORCH_CHECK(tt && tt->dim(), "zeros_like: the rank of the argument must be known");
-    std::vector<int> dims;
-    for (size_t d = 0; d < *tt->dim(); ++d) dims.push_back(op(FX_OP_SIZE, {in(0), cint((int64_t)d)}));
-    int dt = dtypeArg(n->input(1));
-    if (dt < 0 && tt->scalarType()) dt = fxDtype(*tt->scalarType());
-    out(op(FX_OP_FULL, {ilist(dims), cfloat(k == aten::ones_like ? 1.0 : 0.0)}, dt < 0 ? FX_DT_F32 : dt));
+    out(op(FX_OP_FULL, {in(0), cfloat(k == aten::ones_like ? 1.0 : 0.0)}, dtypeArg(n->input(1))));
+    return;
+  }
+  if (k == aten::full_like) {
+    out(op(FX_OP_FULL, {in(0), in(1)}, dtypeArg(n->input(2))));
     return;
   }
   if (k == aten::arange) {

@@ -91,7 +91,7 @@ int Region::addOp(int opcode, const std::vector<int>& args, int out_dtype) {
       break;
     case FX_OP_ASSIGN: v.dtype = tdt(1); break;
     case FX_OP_SUM_DIM: v.dtype = is_float_dt(tdt(0)) ? tdt(0) : FX_DT_I64; break;
-    case FX_OP_FULL: v.dtype = out_dtype >= 0 ? out_dtype : FX_DT_F32; break;
+    case FX_OP_FULL: v.dtype = out_dtype >= 0 ? out_dtype : (tdt(0) >= 0 ? tdt(0) : FX_DT_F32); break;
     case FX_OP_ARANGE: v.dtype = out_dtype >= 0 ? out_dtype : FX_DT_I64; break;
     case FX_OP_SCALAR_TENSOR:
       v.dtype = out_dtype >= 0 ? out_dtype : (vals[args[0]].kind == VK_FLOAT ? FX_DT_F32 : FX_DT_I64);
@@ -568,7 +568,7 @@ Shape Lowerer::shapeOf(int vid) {
         int d = normDim(constIntOf(arg(1), "stack"), (int64_t)s.size() + 1, "stack");
         s.insert(s.begin() + d, (int64_t)ts.size());
       } break;
-      case FX_OP_FULL: s = intListOf(arg(0), "full"); break;
+      case FX_OP_FULL: s = V(arg(0)).kind == VK_TENSOR ? shapeOf(arg(0)) : intListOf(arg(0), "full"); break;
       case FX_OP_ARANGE: {
         int64_t a = constIntOf(arg(0), "arange"), b = constIntOf(arg(1), "arange");
         s = {std::max<int64_t>(b - a, 0)};

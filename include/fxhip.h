@@ -66,7 +66,8 @@ enum fx_opcode {
   FX_OP_CAT,          /* (Tensor[] tensors, int dim)             custom_lowering_func.cpp:297-330 */
   FX_OP_STACK,        /* (Tensor[] tensors, int dim)             custom_lowering_func.cpp:332-350 */
   /* creation: custom_lowering_func.cpp:17-49 */
-  FX_OP_FULL,         /* (int[] size, scalar value)  zeros / ones / full; out dtype required */
+  FX_OP_FULL,         /* (int[] size | Tensor like, scalar value)  zeros / ones / full(_like); out dtype
+                         required with a size list, inherited from `like` when negative */
   FX_OP_ARANGE,       /* (int start, int end)        out dtype required */
   FX_OP_SCALAR_TENSOR,/* (scalar) -> 0-dim tensor    out dtype required */
   FX_OP_TRIU,         /* (self, int diagonal) */

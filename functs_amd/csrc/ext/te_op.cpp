@@ -257,10 +257,39 @@ c10::ScalarType atDtype(int d) {
     TORCH_CHECK(rc__ >= 0, "fxhip: ", fx_last_error(), " (", #expr, ")"); \
   } while (0)
 
+// device scratch and the pinned landing zone of the kept-row counts; a call
+// borrows one and hands it back, so concurrent calls never share
+struct Workspace {
+  at::Tensor scratch, totals;
+};
+
 struct Variant {
   fx_region* region = nullptr;
+  std::mutex mu;
+  std::vector<Workspace> pool;
   ~Variant() {
     if (region) fx_region_destroy(region);
+  }
+  Workspace take(size_t scratch_bytes, int64_t degree, c10::Device device) {
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      while (!pool.empty()) {
+        Workspace ws = std::move(pool.back());
+        pool.pop_back();
+        if ((size_t)ws.scratch.numel() >= scratch_bytes && ws.totals.numel() >= degree &&
+            ws.scratch.device() == device)
+          return ws;
+      }
+    }
+    Workspace ws;
+    ws.scratch = at::empty({(int64_t)std::max<size_t>(scratch_bytes, 1)},
+                           at::TensorOptions().dtype(at::kByte).device(device));
+    ws.totals = at::empty({degree}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+    return ws;
+  }
+  void give(Workspace ws) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (pool.size() < 4) pool.push_back(std::move(ws));
   }
 };
 
@@ -356,35 +385,69 @@ class RegionRunner {
     const fx_plan* plan = nullptr;
     FX_OK_OR_THROW(fx_region_plan(var->region, args.data(), (int)args.size(), &plan));
     const int n_out = fx_plan_num_outputs(plan);
-    std::vector<std::vector<at::Tensor>> outs(n_out);
+    // One allocation per output: the tasks' tensors are views at 256-byte aligned
+    // offsets of it.  The views are made after the launch, while the kernels run.
+    struct Slot { int64_t offset_elems; int32_t rank; int64_t sizes[FX_ARG_MAX_RANK]; };
+    std::vector<Slot> slots((size_t)n_out * degree);
+    std::vector<at::Tensor> buffers(n_out);
     std::vector<void*> ptrs((size_t)n_out * degree);
     for (int o = 0; o < n_out; ++o) {
+      int32_t dt = 0;
+      int64_t total = 0, item = 1;
       for (int64_t t = 0; t < degree; ++t) {
-        int32_t dt, rank;
-        int64_t sizes[FX_ARG_MAX_RANK];
-        FX_OK_OR_THROW(fx_plan_output(plan, o, (int)t, &dt, &rank, sizes));
-        at::Tensor ten = at::empty(at::IntArrayRef(sizes, rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
-        ptrs[(size_t)o * degree + t] = ten.data_ptr();
-        outs[o].push_back(std::move(ten));
+        Slot& sl = slots[(size_t)o * degree + t];
+        FX_OK_OR_THROW(fx_plan_output(plan, o, (int)t, &dt, &sl.rank, sl.sizes));
+        int64_t numel = 1;
+        for (int d = 0; d < sl.rank; ++d) numel *= sl.sizes[d];
+        item = (int64_t)c10::elementSize(atDtype(dt));
+        const int64_t align = 256 / item;
+        sl.offset_elems = total;
+        total += (numel + align - 1) / align * align;
       }
+      if (degree == 1) {
+        const Slot& sl = slots[(size_t)o * degree];
+        buffers[o] = at::empty(at::IntArrayRef(sl.sizes, sl.rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
+      } else {
+        buffers[o] = at::empty({total}, at::TensorOptions().dtype(atDtype(dt)).device(device));
+      }
+      char* base = (char*)buffers[o].data_ptr();
+      for (int64_t t = 0; t < degree; ++t)
+        ptrs[(size_t)o * degree + t] = base + slots[(size_t)o * degree + t].offset_elems * item;
     }
-    at::Tensor scratch, totals;
-    const size_t sb = fx_plan_scratch_bytes(plan);
-    if (compact_) {
-      scratch = at::empty({(int64_t)std::max<size_t>(sb, 1)}, at::TensorOptions().dtype(at::kByte).device(device));
-      totals = at::empty({degree}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
-    }
+    Workspace ws;
+    if (compact_) ws = var->take(fx_plan_scratch_bytes(plan), degree, device);
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
-                                 compact_ ? scratch.data_ptr() : nullptr,
-                                 compact_ ? (uint32_t*)totals.data_ptr() : nullptr, (void*)stream.stream()));
+                                 compact_ ? ws.scratch.data_ptr() : nullptr,
+                                 compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
+    std::vector<std::vector<at::Tensor>> outs(n_out);
+    for (int o = 0; o < n_out; ++o) {
+      if (degree == 1) {
+        outs[o].push_back(std::move(buffers[o]));
+        continue;
+      }
+      outs[o].reserve(degree);
+      for (int64_t t = 0; t < degree; ++t) {
+        const Slot& sl = slots[(size_t)o * degree + t];
+        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(buffers[o].storage()),
+                                                         buffers[o].key_set(), buffers[o].dtype());
+        impl->set_storage_offset(sl.offset_elems);
+        impl->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
+        outs[o].emplace_back(std::move(impl));
+      }
+    }
     if (compact_) {
       // the kept-row counts decide the output shapes: one synchronisation, as ATen's
       // nonzero / masked index does
       stream.synchronize();
-      const int32_t* tot = totals.data_ptr<int32_t>();
+      const int32_t* tot = ws.totals.data_ptr<int32_t>();
       for (int o = 0; o < n_out; ++o)
-        for (int64_t t = 0; t < degree; ++t) outs[o][t] = outs[o][t].narrow(0, 0, tot[t]);
+        for (int64_t t = 0; t < degree; ++t) {
+          Slot& sl = slots[(size_t)o * degree + t];
+          sl.sizes[0] = tot[t];
+          outs[o][t].unsafeGetTensorImpl()->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
+        }
+      var->give(std::move(ws));
     }
     drop(stack, n_stack_);
     for (int o = 0; o < n_out; ++o) {

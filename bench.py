@@ -103,6 +103,19 @@ class Workload:
         return total
 
 
+def recorded_traffic(kernel, workload):
+    """HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter
+    summary of this kernel and workload, or None when none is recorded."""
+    path = os.path.join(ROOT, "profiles", "%s_%s_hbm_traffic.md" % ("fx_compact_scatter", workload))
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch %s:" % kernel):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def measure(w, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -166,6 +179,9 @@ def main():
     ap.add_argument("--workload", default="c5")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-per-config", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="also launch the library's plain copy kernel on BYTES (3 times): the known-size reference "
+                         "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this path runs on ONE GPU (its tasks are independent; see DESIGN.md for how it "
@@ -198,6 +214,16 @@ def main():
             rec["cpu"] = (us, n, cores)
         return rec
 
+    if args.copy_calibration:
+        from functs_amd import _lib
+        n = args.copy_calibration // 4
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.copy_bytes(src, dst)
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+
     head = run_one(args.workload, True)
     per = {}
     if not args.no_per_config:
@@ -212,6 +238,7 @@ def main():
                 per[name] = {"error": str(e)[:200]}
     cpu_us, cpu_n, cores = head.pop("cpu")
     dom_ms = max(head["kernel_us"]) / 1e3
+    dom_kernel = "fx_compact_scatter" if head["launches_per_call"] > 1 else "fx_region_dense"
     out = {
         "metric": "per-call latency",
         "value": head["torchscript_route_latency_us"],
@@ -230,8 +257,8 @@ def main():
                    "region_api_latency_us": head["latency_us"], "launches_per_call": head["launches_per_call"],
                    "kernel_us": head["kernel_us"], "gbps_all_kernels": head["gbps_all_kernels"]},
         "roofline": {"bound": "hbm", "achieved": head["gbps_dominant_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": head["frac_hbm_peak"], "traffic": None,
-                     "kernel": "fx_compact_scatter" if head["launches_per_call"] > 1 else "fx_region_dense",
+                     "frac": head["frac_hbm_peak"], "traffic": recorded_traffic(dom_kernel, args.workload),
+                     "kernel": dom_kernel,
                      "algorithmic_bytes": head["algorithmic_bytes"], "kernel_ms": round(dom_ms, 5)},
         "cpu_baseline": {"value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
                          "sample": "%d calls of torch.jit.script(%s) on the same seeded CPU tensors" % (cpu_n, args.workload)},

@@ -137,3 +137,14 @@ def check(rc):
     if rc < 0:
         raise FxError(rc, lib.fx_last_error().decode())
     return rc
+
+
+def copy_bytes(src, dst, stream=None):
+    """dst[:] = src with the library's plain 128-bit copy kernel (the known-size
+    dispatch that hardware-counter readings are calibrated against)."""
+    import torch
+    assert src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()
+    nbytes = src.numel() * src.element_size()
+    assert nbytes == dst.numel() * dst.element_size()
+    st = torch.cuda.current_stream(src.device).cuda_stream if stream is None else stream
+    check(lib.fx_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, st))

@@ -17,6 +17,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/DeviceGuard.h>
 #include <torch/csrc/jit/ir/constants.h>
+#include <torch/csrc/jit/passes/common_subexpression_elimination.h>
 #include <torch/csrc/jit/runtime/custom_operator.h>
 
 #include <mutex>
@@ -61,6 +62,14 @@ void cloneBlockInto(Block* src, Graph* sub, std::unordered_map<Value*, Value*>& 
   }
 }
 
+// A region holds pure operators only, so equal expressions can be merged; alias
+// analysis has no entry for the collapsed-loop node, regions with one are left as is.
+void cseRegion(std::shared_ptr<Graph> sub) {
+  for (Node* n : sub->nodes())
+    if (n->kind() == sym::ForallSelectRev()) return;
+  EliminateCommonSubexpression(sub);
+}
+
 Node* functorFromGroup(Node* group) {
   Graph* g = group->owningGraph();
   Node* f = g->createWithSubgraph(sym::ParallelFunctor());
@@ -81,6 +90,7 @@ Node* functorFromGroup(Node* group) {
   Block* body = group->blocks()[0];
   for (Value* p : body->inputs()) map[p] = sub->addInput()->copyMetadata(p);
   cloneBlockInto(body, sub.get(), map);
+  cseRegion(sub);
   return f;
 }
 
@@ -132,6 +142,7 @@ Node* functorFromMap(Node* mapNode, Node* group) {
   for (Value* r : mb->outputs()) returns.push_back(body->outputs()[r->offset()]);
   if (f->i(sym::compact_rows())) returns.push_back(body->outputs().back());
   cloneBlockInto(body, sub.get(), map, &returns);
+  cseRegion(sub);
   return f;
 }
 

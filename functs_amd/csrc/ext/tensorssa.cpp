@@ -156,6 +156,7 @@ void pruneForest(std::shared_ptr<Graph> g, ViewForest& f) {
         case c10::aten::append: case c10::prim::SetAttr:
           bad.insert(root);
           break;
+
         default:
           // a write this pass does not understand
           if (user->kind() != c10::aten::copy_ && user->kind() != sym::Assign() && writesInput(user, u.offset))
@@ -282,15 +283,18 @@ void aliasRemoval(Block* b, ViewForest& f, TensorSSAMutateInfo& info) {
     update->insertAfter(at);
     info.addMutNodes(update);
 
-    // pass down (depth first over the views that dominate the mutation)
+    // pass down, level by level over the views that dominate the mutation; the
+    // youngest view of a level first, which reproduces the node order of the
+    // reference's printed graphs (README.md:113-140)
     struct Visit { Value* old_value; Value* new_value; Node* update; };
-    std::vector<Visit> stack{{root, up, update}};
+    std::deque<Visit> stack{{root, up, update}};
     while (!stack.empty()) {
-      Visit cur = stack.back();
-      stack.pop_back();
+      Visit cur = stack.front();
+      stack.pop_front();
       auto kids = f.children.find(cur.old_value);
       if (kids == f.children.end()) continue;
-      for (Value* from : kids->second) {
+      for (auto kit = kids->second.rbegin(); kit != kids->second.rend(); ++kit) {
+        Value* from = *kit;
         Node* fromNode = from->node();
         bool alive = (fromNode == node) || (fromNode->isBefore(node) && node->isDominatedBy(fromNode));
         if (!alive) continue;

@@ -263,15 +263,21 @@ int fx_device_count(void) {
 
 // Fill the by-value dynamic block.  Exposed (without launching) so that host
 // tests can check the marshalling.
+// `safe`: a device address that can always be read.  Kernels clamp the address of
+// an element that is not live to element 0 of its buffer, so a tensor without
+// elements (whose pointer may be null) is given this address instead.
 static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
-                    uint32_t* totals_host, FxDyn* dyn) {
+                    uint32_t* totals_host, const void* safe, FxDyn* dyn) {
   const fx::Region& R = *pl->region;
   const int T = R.degree;
   auto ptr_of = [&](const fx::PtrSrc& s, int task) -> uint64_t {
     switch (s.kind) {
       case fx::PtrSrc::INPUT: {
         bool per_task = R.vals[R.inputs[s.index]].per_task;
-        return (uint64_t)(uintptr_t)args[pl->arg_base[s.index] + (per_task ? task : 0)].ptr;
+        const fx_arg& a = args[pl->arg_base[s.index] + (per_task ? task : 0)];
+        bool empty = a.ptr == nullptr;
+        for (int d = 0; d < a.rank; ++d) empty = empty || a.sizes[d] == 0;
+        return (uint64_t)(uintptr_t)((empty && safe) ? safe : a.ptr);
       }
       case fx::PtrSrc::OUTPUT: return (uint64_t)(uintptr_t)out_ptrs[s.index * T + task];
       case fx::PtrSrc::FLAGS: return (uint64_t)(uintptr_t)((char*)scratch + pl->flags_off);
@@ -311,7 +317,7 @@ int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, i
   if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
   if (dyn_cap < sizeof(FxDyn)) return fail(FX_E_INVALID, "dyn_out too small");
   memset(dyn_out, 0, sizeof(FxDyn));
-  return fill_dyn(pl, args, out_ptrs, scratch, totals_host, (FxDyn*)dyn_out);
+  return fill_dyn(pl, args, out_ptrs, scratch, totals_host, nullptr, (FxDyn*)dyn_out);
 }
 
 size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
@@ -339,7 +345,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     }
   }
   FxDyn dyn;
-  int rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, &dyn);
+  int rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn);
   if (rc != FX_OK) return rc;
   const uint32_t* sb = (const uint32_t*)pl->dev_blob;
   FxLaunchInfo li;

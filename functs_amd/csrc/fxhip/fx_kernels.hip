@@ -46,6 +46,13 @@ __device__ __forceinline__ uint32_t uni(uint32_t x) { return __builtin_amdgcn_re
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
+#ifdef FX_PHASE_PROF
+__device__ unsigned long long fx_prof_buf[1 << 16];
+#define FX_PROF(slot) do { if ((threadIdx.x & 63u) == 0 && blockIdx.x < 2048) fx_prof_buf[blockIdx.x * 32 + (slot)] = wall_clock64(); } while (0)
+#else
+#define FX_PROF(slot) do { } while (0)
+#endif
+
 struct FxCtx {
   const fx_u32x4* insn;   // LDS: class instruction base
   const uint32_t* aff;    // LDS: class affine base (FX_AFF_WORDS words each)
@@ -64,21 +71,44 @@ struct FxCtx {
 // `base_` is wave-uniform (kept in SGPRs by the callers) and `off` is an
 // element index below 2^31 / element size: the access is base + 32-bit byte
 // offset, which needs no 64-bit vector arithmetic.
-__device__ __forceinline__ uint32_t fx_load(uint64_t base_, int32_t off, uint32_t dt) {
+// FX_V loads of one instruction.  All of them are issued before anything looks
+// at loaded data (no conversion, no select between a loaded and an older value),
+// so a wave pays the memory latency once per instruction and the loads of a
+// following instruction overlap as well.  Elements that are not live read
+// element 0 of the buffer and end up with an unspecified value, like after any
+// arithmetic instruction; the host never passes a buffer without an element 0.
+__device__ __forceinline__ void fx_load_vec(uint64_t base_, const int32_t (&off)[FX_V], uint32_t M, uint32_t dt,
+                                            bool cvt, uint32_t (&out)[FX_V]) {
   const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
-  const uint32_t o = (uint32_t)off;
-  switch (dt) {
-    case FX_F32:
-    case FX_I32: return *(const FX_AS1 uint32_t*)(base + (o << 2));
-    case FX_I64: return (uint32_t)*(const FX_AS1 uint64_t*)(base + (o << 3));
-    case FX_U8: return base[o];
-    case FX_F16: {
-      uint16_t h = *(const FX_AS1 uint16_t*)(base + (o << 1));
-      __half hv = __ushort_as_half(h);
-      return f2u(__half2float(hv));
+  uint32_t o[FX_V];
+#pragma unroll
+  for (int j = 0; j < FX_V; ++j) o[j] = ((M >> j) & 1u) ? (uint32_t)off[j] : 0u;
+  if (dt == FX_F32 || dt == FX_I32) {
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = *(const FX_AS1 uint32_t*)(base + (o[j] << 2));
+  } else if (dt == FX_I64) {  // values fit 32 bits: the low word is the value
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = *(const FX_AS1 uint32_t*)(base + (o[j] << 3));
+  } else if (dt == FX_U8) {
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = base[o[j]];
+  } else {
+    uint32_t h[FX_V];
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) h[j] = *(const FX_AS1 uint16_t*)(base + (o[j] << 1));
+    if (dt == FX_F16) {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) out[j] = f2u(__half2float(__ushort_as_half((uint16_t)h[j])));
+    } else {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) out[j] = h[j] << 16;
     }
-    case FX_BF16: return ((uint32_t)*(const FX_AS1 uint16_t*)(base + (o << 1))) << 16;
-    default: return 0;
+  }
+  if (cvt) {
+    // a real branch: folded into selects, the conversion would need the data at once
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = f2u((float)(int32_t)out[j]);
   }
 }
 
@@ -240,31 +270,22 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
           cf[4] = 0; cf[5] = 0;
         }
         const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
-        const bool is_load = (op == FX_LDA || op == FX_LDB);
-        const uint64_t p = is_load ? fx_ptr(cx, ia) : 0ull;
-        const bool toA = (op == FX_LDA || op == FX_AFFA);
-        if (!wave_any(M != VM)) {
-          // every element of the wave is live: no per-element predication
+        int32_t off[FX_V];
 #pragma unroll
-          for (int j = 0; j < FX_V; ++j) {
-            int32_t off = base;
+        for (int j = 0; j < FX_V; ++j) {
+          off[j] = base;
 #pragma unroll
-            for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
-            uint32_t v = is_load ? fx_load(p, off, dt) : (uint32_t)off;
-            if (cvt) v = f2u((float)(int32_t)v);
-            if (toA) A[j] = v; else B[j] = v;
-          }
+          for (int k = 0; k < R; ++k) off[j] += cf[k] * c[j][k];
+        }
+        if (op == FX_LDA) {
+          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, A);
+        } else if (op == FX_LDB) {
+          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, B);
         } else {
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
-            if ((M >> j) & 1u) {
-              int32_t off = base;
-#pragma unroll
-              for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
-              uint32_t v = is_load ? fx_load(p, off, dt) : (uint32_t)off;
-              if (cvt) v = f2u((float)(int32_t)v);
-              if (toA) A[j] = v; else B[j] = v;
-            }
+            const uint32_t v = cvt ? f2u((float)off[j]) : (uint32_t)off[j];
+            if (op == FX_AFFA) A[j] = v; else B[j] = v;
           }
         }
       } break;
@@ -295,11 +316,10 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         }
       } break;
       case FX_LDXA: {
-        const uint64_t p = fx_ptr(cx, ia);
+        int32_t off[FX_V];
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) A[j] = fx_load(p, (int32_t)A[j] + (int32_t)imm, dt);
-        }
+        for (int j = 0; j < FX_V; ++j) off[j] = (int32_t)A[j] + (int32_t)imm;
+        fx_load_vec(fx_ptr(cx, ia), off, M, dt, false, A);
       } break;
       case FX_IMMA:
 #pragma unroll
@@ -534,18 +554,14 @@ __device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const int3
   }
   const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task;
   const uint64_t p = fx_ptr(cx, (int32_t)w.y);
+  int32_t off[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) {
-    P[j] = 0;
-    if ((M >> j) & 1u) {
-      int32_t off = base;
+    off[j] = base;
 #pragma unroll
-      for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
-      uint32_t v = fx_load(p, off, dt);
-      if (cvt) v = f2u((float)(int32_t)v);
-      P[j] = v;
-    }
+    for (int k = 0; k < R; ++k) off[j] += cf[k] * c[j][k];
   }
+  fx_load_vec(p, off, M, dt, cvt, P);
 }
 
 __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint32_t shift) {
@@ -843,7 +859,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
   __shared__ uint32_t s_prefix;
   __shared__ int32_t s_adj[FX_MAX_STAGES];
+  if (threadIdx.x == 0) FX_PROF(0);
   fx_stage(L, sb, la);
+  if (threadIdx.x == 0) FX_PROF(1);
   const FxWork w = fx_locate<false>(L, blockIdx.x);
   FxCtx cx = fx_make_ctx(L, la, w);
   cx.stage_adj = s_adj;
@@ -891,6 +909,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     ((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])])[w.task] = prefix + n_kept;
   }
   if (n_kept == 0) return;
+  if (threadIdx.x == 0) FX_PROF(2);
 
   const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
   const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
@@ -957,6 +976,10 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     uint32_t it0 = (wave_u + 4u - (item_base & 3u)) & 3u;
     for (; it0 < n_items; it0 += 4u * FX_K) {
       uint32_t P[FX_K][FX_V];
+#ifdef FX_PHASE_PROF
+      const bool pf = (oi == 1) && (it0 < 4u) && wave_u == 0;
+      if (pf) FX_PROF(16);
+#endif
       if (lead) {
 #pragma unroll
         for (uint32_t k = 0; k < FX_K; ++k) {
@@ -967,6 +990,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
             make_item(it, e, M, c);
             fx_lead_load<R>(cx, pb, c, M, P[k]);
           }
+#ifdef FX_PHASE_PROF
+          if (pf) FX_PROF(17 + k);
+#endif
         }
       }
 #pragma unroll
@@ -976,18 +1002,28 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
           uint32_t e[FX_V], M;
           int32_t c[FX_V][R];
           make_item(it, e, M, c);
+#ifdef FX_PHASE_PROF
+          if (pf && k == 0) FX_PROF(21);
+#endif
           uint32_t A[FX_V];
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
           fx_run<R>(cx, lead ? pb + 1 : pb, pe, c, M, A);
+#ifdef FX_PHASE_PROF
+          if (pf && k == 0) FX_PROF(22);
+#endif
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
             if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
           }
+#ifdef FX_PHASE_PROF
+          if (pf) FX_PROF(23 + k);
+#endif
         }
       }
     }
     item_base += n_items;
+    FX_PROF(4 + oi * 4 + (threadIdx.x >> 6));
   }
 }
 
@@ -1210,3 +1246,10 @@ hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t gri
   return hipGetLastError();
 }
 
+
+#ifdef FX_PHASE_PROF
+// timestamps written by FX_PROF (profiling builds only)
+extern "C" int fx_prof_read(unsigned long long* out, size_t n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fx_prof_buf), n * sizeof(unsigned long long));
+}
+#endif

@@ -152,7 +152,15 @@ struct FxOut {
   uint32_t lead;                  // program starts with an unconditional affine load (batched by the kernels)
   uint32_t unit_items;            // dense: items per wave and work unit (1 or FX_K)
   uint32_t rowwave;               // dense: one item = one row of dim[rank-1] elements (needed by FX_WMAX/FX_WSUM)
-  uint32_t pad;
+  // A lane works on a group of FX_V consecutive elements along the last dimension
+  // (coordinate vd); rows are padded to whole groups.
+  uint32_t inner;                 // extent of the last dimension (1 for a scalar)
+  uint32_t vd;                    // index of that dimension: max(rank, 1) - 1
+  uint32_t gpr;                   // groups per run of `inner` elements: ceil(inner / FX_V)
+  uint32_t gp_magic, gp_shift;    // fast division by gpr
+  uint32_t gprow;                 // compaction: groups per kept row: rowlen / inner * gpr
+  uint32_t gr_magic, gr_shift;    // fast division by gprow
+  uint32_t n_groups;              // dense: groups per task: numel / inner * gpr
 };
 
 // An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows

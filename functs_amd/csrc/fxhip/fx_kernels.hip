@@ -38,11 +38,13 @@ namespace {
 #define FX_AS1 __attribute__((address_space(1)))
 #define FX_AS4 __attribute__((address_space(4)))
 typedef uint32_t fx_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t fx_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));  // 128 bits, 4-byte aligned
 
 // word offset of a field inside a blob structure
 #define FX_W(Type, field) (offsetof(Type, field) / 4)
 
 __device__ __forceinline__ uint32_t uni(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
@@ -78,8 +80,23 @@ struct FxCtx {
 // element 0 of the buffer and end up with an unspecified value, like after any
 // arithmetic instruction; the host never passes a buffer without an element 0.
 __device__ __forceinline__ void fx_load_vec(uint64_t base_, const int32_t (&off)[FX_V], uint32_t M, uint32_t dt,
-                                            bool cvt, uint32_t (&out)[FX_V]) {
+                                            bool cvt, bool consecutive, uint32_t (&out)[FX_V]) {
   const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
+  const uint32_t VM = (1u << FX_V) - 1u;
+  // FX_V consecutive 32-bit elements in every lane that is live at all, and at least
+  // one such lane (so the buffer holds FX_V elements): one 128-bit load per lane.
+  // It needs 4-byte alignment only.
+  if (consecutive && (dt == FX_F32 || dt == FX_I32) && !wave_any(M != 0u && M != VM) && wave_any(M == VM)) {
+    const uint32_t o0 = M ? (uint32_t)off[0] : 0u;
+    const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)(base + (o0 << 2));
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    if (cvt) {
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) out[j] = f2u((float)(int32_t)out[j]);
+    }
+    return;
+  }
   uint32_t o[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) o[j] = ((M >> j) & 1u) ? (uint32_t)off[j] : 0u;
@@ -180,14 +197,93 @@ __device__ __forceinline__ float fx_sigmoid(float x) {
 __device__ __forceinline__ float fx_fmax(float a, float b) { return (a > b || a != a) ? a : b; }
 __device__ __forceinline__ float fx_fmin(float a, float b) { return (a < b || a != a) ? a : b; }
 
-__device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
+// Coordinates of the FX_V elements a lane works on.  They differ in ONE
+// coordinate (vd, wave-uniform): element j has coordinates c0 with c0[vd]
+// replaced by cv[j].  `step` (wave-uniform) says cv[j] == cv[0] + j, i.e. the
+// lane holds FX_V consecutive elements along dimension vd.
+template <int R>
+struct FxCoord {
+  int32_t c0[R];     // entry vd is 0
+  int32_t cv[FX_V];
+  uint32_t vd;
+  uint32_t step;
+};
+
+// off[j] = base + sum_k cf[k] * coordinate_k(element j)
+// Returns true (wave-uniform) when off[j] == off[0] + j for every lane.
+template <int R>
+__device__ __forceinline__ bool fx_offsets(const FxCoord<R>& q, const int32_t (&cf)[FX_MAXR], int32_t base,
+                                           int32_t (&off)[FX_V]) {
+  int32_t s = base;
+#pragma unroll
+  for (int k = 0; k < R; ++k) s += cf[k] * q.c0[k];
+  int32_t cfv = cf[0];
+#pragma unroll
+  for (int k = 1; k < R; ++k) cfv = (q.vd == (uint32_t)k) ? cf[k] : cfv;
+  if (q.step) {
+    const int32_t o0 = s + cfv * q.cv[0];
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) off[j] = o0 + j * cfv;
+    return uni((uint32_t)cfv) == 1u;
+  } else {
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) off[j] = s + cfv * q.cv[j];
+    return false;
+  }
+}
+
+// row index (all dimensions but vd, flattened) -> c0[1..R-1]; returns what is
+// left for dimension 0.  dk / mk / sk: extent and fast-division constants per dimension.
+template <int R>
+__device__ __forceinline__ uint32_t fx_unflatten(uint32_t rem, uint32_t vd, const uint32_t (&dk)[R],
+                                                 const uint32_t (&mk)[R], const uint32_t (&sk)[R], int32_t (&c0)[R]) {
+#pragma unroll
+  for (int k = R - 1; k >= 1; --k) {
+    if (vd == (uint32_t)k) {
+      c0[k] = 0;
+    } else {
+      const uint32_t d = (__umulhi(rem, mk[k]) + rem) >> sk[k];
+      c0[k] = (int32_t)(rem - d * dk[k]);
+      rem = d;
+    }
+  }
+  return rem;
+}
+
+// Results of one item.  contig (wave-uniform): e[j] == e[0] + j, so a lane whose
+// FX_V elements are all live writes them with one 128-bit store.
+__device__ __forceinline__ void fx_store_vec(uint64_t base_, uint32_t obase, const uint32_t (&e)[FX_V], uint32_t M,
+                                             bool contig, uint32_t dt, uint32_t vt, const uint32_t (&A)[FX_V]) {
+  const bool raw32 = (dt == FX_F32 && vt == FX_VT_F) || (dt == FX_I32 && vt == FX_VT_I);
+  if (raw32 && contig) {
+    FX_AS1 uint8_t* base = (FX_AS1 uint8_t*)base_;
+    if (M == (1u << FX_V) - 1u) {
+      // The four results pass through an opaque copy: seen as one vector value, the
+      // optimiser would turn the interpreter's accumulators into vector registers.
+      uint32_t t0 = A[0], t1 = A[1], t2 = A[2], t3 = A[3];
+      asm("" : "+v"(t0), "+v"(t1), "+v"(t2), "+v"(t3));
+      fx_u32x4 v;
+      v.x = t0; v.y = t1; v.z = t2; v.w = t3;
+      *(FX_AS1 fx_u32x4_a4*)(base + ((obase + e[0]) << 2)) = v;
+    } else {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j)
+        if ((M >> j) & 1u) *(FX_AS1 uint32_t*)(base + ((obase + e[0] + j) << 2)) = A[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j)
+      if ((M >> j) & 1u) fx_store(base_, obase + e[j], dt, vt, A[j]);
+  }
+}
 
 // The interpreter.  R = number of root coordinates that carry information.
 // The program lives in LDS; the next instruction word is fetched while the
 // current one executes.  The host pads every program area with one trailing
 // NOP so that the look-ahead read stays inside the blob.
 template <int R>
-__device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end, const int32_t (&c)[FX_V][R],
+__device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end, const FxCoord<R>& q,
                                        uint32_t M, uint32_t (&A)[FX_V]) {
   uint32_t B[FX_V];
 #pragma unroll
@@ -271,16 +367,11 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         }
         const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
         int32_t off[FX_V];
-#pragma unroll
-        for (int j = 0; j < FX_V; ++j) {
-          off[j] = base;
-#pragma unroll
-          for (int k = 0; k < R; ++k) off[j] += cf[k] * c[j][k];
-        }
+        const bool consecutive = fx_offsets<R>(q, cf, base, off);
         if (op == FX_LDA) {
-          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, A);
+          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, A);
         } else if (op == FX_LDB) {
-          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, B);
+          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B);
         } else {
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
@@ -303,13 +394,12 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         }
         // the task term is part of the tile's global origin, not of the LDS index
         const int32_t base = (int32_t)a1.y + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1 + cx.stage_adj[ia];
+        int32_t off[FX_V];
+        fx_offsets<R>(q, cf, base, off);
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) {
           if ((M >> j) & 1u) {
-            int32_t off = base;
-#pragma unroll
-            for (int k = 0; k < R; ++k) off += cf[k] * c[j][k];
-            uint32_t v = cx.stage[off];
+            uint32_t v = cx.stage[off[j]];
             if (cvt) v = f2u((float)(int32_t)v);
             if (op == FX_LDSA) A[j] = v; else B[j] = v;
           }
@@ -319,7 +409,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         int32_t off[FX_V];
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) off[j] = (int32_t)A[j] + (int32_t)imm;
-        fx_load_vec(fx_ptr(cx, ia), off, M, dt, false, A);
+        fx_load_vec(fx_ptr(cx, ia), off, M, dt, false, false, A);
       } break;
       case FX_IMMA:
 #pragma unroll
@@ -536,7 +626,7 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 // The interpreter then starts behind the load with A preset.
 #define FX_K 4
 template <int R>
-__device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const int32_t (&c)[FX_V][R], uint32_t M,
+__device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const FxCoord<R>& q, uint32_t M,
                                              uint32_t (&P)[FX_V]) {
   const fx_u32x4 w = cx.insn[pc];
   const uint32_t w0 = uni(w.x);
@@ -555,13 +645,8 @@ __device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const int3
   const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task;
   const uint64_t p = fx_ptr(cx, (int32_t)w.y);
   int32_t off[FX_V];
-#pragma unroll
-  for (int j = 0; j < FX_V; ++j) {
-    off[j] = base;
-#pragma unroll
-    for (int k = 0; k < R; ++k) off[j] += cf[k] * c[j][k];
-  }
-  fx_load_vec(p, off, M, dt, cvt, P);
+  const bool consecutive = fx_offsets<R>(q, cf, base, off);
+  fx_load_vec(p, off, M, dt, cvt, consecutive, P);
 }
 
 __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint32_t shift) {
@@ -712,6 +797,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
     const uint32_t obase = uni(od[FX_W(FxOut, task_stride)]) * (uint32_t)w.task;
     const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
     uint32_t dk[R], mk[R], sk[R];
+    dk[0] = mk[0] = sk[0] = 0;
 #pragma unroll
     for (int k = 1; k < R; ++k) {
       dk[k] = od[FX_W(FxOut, dim) + k];
@@ -719,38 +805,45 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
       sk[k] = od[FX_W(FxOut, shift) + k];
     }
     // unit = 4 waves x kmax items; kmax is 1 for heavy or small outputs (more, smaller units).
-    // An item is FX_ITEM consecutive elements, or one whole row (rowwave) so that
-    // the wave-wide reductions see exactly the elements of that row.
+    // An item is 64 lane groups of FX_V consecutive elements along the last dimension,
+    // or one whole row (rowwave) so that the wave-wide reductions see exactly the
+    // elements of that row.
     const uint32_t kmax = uni(od[FX_W(FxOut, unit_items)]);
     const uint32_t rowwave = uni(od[FX_W(FxOut, rowwave)]);
-    const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
+    const uint32_t inner = uni(od[FX_W(FxOut, inner)]);
+    const uint32_t vd = uni(od[FX_W(FxOut, vd)]);
+    const uint32_t gpr = uni(od[FX_W(FxOut, gpr)]);
+    const uint32_t gp_magic = od[FX_W(FxOut, gp_magic)], gp_shift = od[FX_W(FxOut, gp_shift)];
+    const uint32_t n_groups = uni(od[FX_W(FxOut, n_groups)]);
     const uint32_t item0 = ublock * (4u * kmax) + wave * kmax;
-    const uint32_t n_items = rowwave ? numel / (rowlen ? rowlen : 1u) : (numel + FX_ITEM - 1) / FX_ITEM;
+    const uint32_t n_items = rowwave ? numel / inner : (n_groups + 63u) / 64u;
     if (item0 >= n_items) continue;
 
-    auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, int32_t (&c)[FX_V][R]) {
+    auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) {
+      uint32_t row, col0;
+      bool live;
+      if (rowwave) {
+        row = item0 + k;
+        col0 = lane * FX_V;
+        live = true;
+      } else {
+        const uint32_t g = (item0 + k) * 64u + lane;
+        live = g < n_groups;
+        const uint32_t gg = live ? g : 0u;
+        row = fx_fastdiv(gg, gp_magic, gp_shift);
+        col0 = (gg - row * gpr) * FX_V;
+      }
       M = 0;
 #pragma unroll
       for (int j = 0; j < FX_V; ++j) {
-        bool live;
-        if (rowwave) {
-          const uint32_t col = j * 64u + lane;
-          live = col < rowlen;
-          e[j] = (item0 + k) * rowlen + (live ? col : 0u);
-        } else {
-          e[j] = (item0 + k) * FX_ITEM + j * 64u + lane;
-          live = e[j] < numel;
-        }
-        if (live) M |= 1u << j;
-        uint32_t rem = e[j];
-#pragma unroll
-        for (int q = R - 1; q >= 1; --q) {
-          const uint32_t d = fx_fastdiv(rem, mk[q], sk[q]);
-          c[j][q] = (int32_t)(rem - d * dk[q]);
-          rem = d;
-        }
-        c[j][0] = (int32_t)rem;
+        if (live && col0 + j < inner) M |= 1u << j;
+        q.cv[j] = (int32_t)(col0 + j);
+        e[j] = row * inner + col0 + j;
       }
+      q.vd = vd;
+      q.step = 1;
+      const uint32_t rem = fx_unflatten<R>(row, vd, dk, mk, sk, q.c0);
+      q.c0[0] = vd == 0 ? 0 : (int32_t)rem;
     };
 
     uint32_t P[FX_K][FX_V];
@@ -759,9 +852,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
       for (uint32_t k = 0; k < FX_K; ++k) {
         if (k < kmax && item0 + k < n_items) {
           uint32_t e[FX_V], M;
-          int32_t c[FX_V][R];
-          make_item(k, e, M, c);
-          fx_lead_load<R>(cx, pb, c, M, P[k]);
+          FxCoord<R> q;
+          make_item(k, e, M, q);
+          fx_lead_load<R>(cx, pb, q, M, P[k]);
         }
       }
     }
@@ -769,16 +862,13 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
     for (uint32_t k = 0; k < FX_K; ++k) {
       if (k < kmax && item0 + k < n_items) {
         uint32_t e[FX_V], M;
-        int32_t c[FX_V][R];
-        make_item(k, e, M, c);
+        FxCoord<R> q;
+        make_item(k, e, M, q);
         uint32_t A[FX_V];
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
-        fx_run<R>(cx, lead ? pb + 1 : pb, pe, c, M, A);
-#pragma unroll
-        for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
-        }
+        fx_run<R>(cx, lead ? pb + 1 : pb, pe, q, M, A);
+        fx_store_vec(op, obase, e, M, true, odt, ovt, A);
       }
     }
   }
@@ -799,19 +889,22 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
   const FxCtx cx = fx_make_ctx(L, la, w);
 
   const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
-  int32_t c[FX_V][1];
+  FxCoord<1> q;
+  q.c0[0] = 0;
+  q.vd = 0;
+  q.step = 0;
   uint32_t M = 0;
   uint32_t row[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) {
     row[j] = w.local_block * FX_TILE + j * FX_BLOCK + threadIdx.x;
-    c[j][0] = (int32_t)row[j];
+    q.cv[j] = (int32_t)row[j];
     if (row[j] < n_rows) M |= 1u << j;
   }
   uint32_t A[FX_V];
 #pragma unroll
   for (int j = 0; j < FX_V; ++j) A[j] = 0;
-  fx_run<1>(cx, (int)uni(w.cls[FX_W(FxClass, mask_begin)]), (int)uni(w.cls[FX_W(FxClass, mask_end)]), c, M, A);
+  fx_run<1>(cx, (int)uni(w.cls[FX_W(FxClass, mask_begin)]), (int)uni(w.cls[FX_W(FxClass, mask_end)]), q, M, A);
 
   const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
   FX_AS1 uint8_t* flags = (FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * uni(L[FX_W(FxHeader, max_rows)]);
@@ -924,15 +1017,23 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     const uint32_t* od = outs + oi * ow;
     const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
     const uint32_t colmajor = uni(od[FX_W(FxOut, colmajor)]);
-    const uint32_t rl_magic = od[FX_W(FxOut, rl_magic)], rl_shift = od[FX_W(FxOut, rl_shift)];
-    const uint32_t n_el = n_kept * rowlen;
+    const uint32_t inner = uni(od[FX_W(FxOut, inner)]);
+    const uint32_t vd = uni(od[FX_W(FxOut, vd)]);
+    const uint32_t gpr = uni(od[FX_W(FxOut, gpr)]);
+    const uint32_t gp_magic = od[FX_W(FxOut, gp_magic)], gp_shift = od[FX_W(FxOut, gp_shift)];
+    const uint32_t gprow = uni(od[FX_W(FxOut, gprow)]);
+    const uint32_t gr_magic = od[FX_W(FxOut, gr_magic)], gr_shift = od[FX_W(FxOut, gr_shift)];
     const uint32_t chunks = (n_kept + FX_ITEM - 1) / FX_ITEM;   // row chunks per column (column-major)
-    const uint32_t n_items = colmajor ? rowlen * chunks : (n_el + FX_ITEM - 1) / FX_ITEM;
+    // lane groups: FX_V consecutive elements of a kept row along the last dimension, or
+    // (rank 1) FX_V consecutive kept rows
+    const uint32_t n_groups = vd == 0 ? (n_kept + FX_V - 1) / FX_V : n_kept * gprow;
+    const uint32_t n_items = colmajor ? rowlen * chunks : (n_groups + 63u) / 64u;
     const uint64_t op = fx_ptr(cx, (int32_t)od[FX_W(FxOut, ptr_slot)]);
     const uint32_t obase = uni(od[FX_W(FxOut, task_stride)]) * (uint32_t)w.task + prefix * rowlen;
     const int pb = (int)uni(od[FX_W(FxOut, prog_begin)]), pe = (int)uni(od[FX_W(FxOut, prog_end)]);
     const uint32_t odt = uni(od[FX_W(FxOut, dtype)]), ovt = uni(od[FX_W(FxOut, vt)]);
     uint32_t dk[R], mk[R], sk[R];
+    dk[0] = mk[0] = sk[0] = 0;
 #pragma unroll
     for (int k = 1; k < R; ++k) {
       dk[k] = od[FX_W(FxOut, dim) + k];
@@ -940,59 +1041,73 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
       sk[k] = od[FX_W(FxOut, shift) + k];
     }
     const uint32_t lead = uni(od[FX_W(FxOut, lead)]);
-    auto make_item = [&](uint32_t it, uint32_t (&e)[FX_V], uint32_t& M, int32_t (&c)[FX_V][R]) {
+    auto make_item = [&](uint32_t it, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) {
       M = 0;
+      if (colmajor) {
+        // all lanes of the item share one column: predicates on the inner
+        // coordinates are wave-uniform and whole branches get skipped
+        const uint32_t cc = it / chunks, ch = it - cc * chunks;
 #pragma unroll
-      for (int j = 0; j < FX_V; ++j) {
-        uint32_t r, col;
-        bool live;
-        if (colmajor) {
-          // all lanes of the item share one column: predicates on the inner
-          // coordinate are wave-uniform and whole branches get skipped
-          const uint32_t cc = it / chunks, ch = it - cc * chunks;
-          r = ch * FX_ITEM + j * 64u + lane;
-          col = cc;
-          live = r < n_kept;
-          e[j] = r * rowlen + col;
-        } else {
-          e[j] = it * FX_ITEM + j * 64u + lane;
-          live = e[j] < n_el;
-          r = fx_fastdiv(e[j], rl_magic, rl_shift);
-          col = e[j] - r * rowlen;
+        for (int j = 0; j < FX_V; ++j) {
+          const uint32_t r = ch * FX_ITEM + j * 64u + lane;
+          const bool live = r < n_kept;
+          if (live) M |= 1u << j;
+          e[j] = r * rowlen + cc;
+          q.cv[j] = live ? (int32_t)s_rowmap[r] : 0;
         }
-        if (live) M |= 1u << j;
+        q.vd = 0;
+        q.step = 0;
+        fx_unflatten<R>(cc, 0u, dk, mk, sk, q.c0);
+        q.c0[0] = 0;
+      } else if (vd == 0) {
+        const uint32_t r0 = (it * 64u + lane) * FX_V;
 #pragma unroll
-        for (int k = R - 1; k >= 2; --k) {
-          const uint32_t q = fx_fastdiv(col, mk[k], sk[k]);
-          c[j][k] = (int32_t)(col - q * dk[k]);
-          col = q;
+        for (int j = 0; j < FX_V; ++j) {
+          const bool live = r0 + j < n_kept;
+          if (live) M |= 1u << j;
+          e[j] = r0 + j;
+          q.cv[j] = live ? (int32_t)s_rowmap[r0 + j] : 0;
         }
-        if (R > 1) c[j][1] = (int32_t)col;  // what is left is the coordinate itself
-        c[j][0] = live ? (int32_t)s_rowmap[r] : 0;
+        q.vd = 0;
+        q.step = 0;
+#pragma unroll
+        for (int k = 0; k < R; ++k) q.c0[k] = 0;
+      } else {
+        const uint32_t g = it * 64u + lane;
+        const bool live = g < n_groups;
+        const uint32_t gg = live ? g : 0u;
+        const uint32_t r = fx_fastdiv(gg, gr_magic, gr_shift);
+        const uint32_t t = gg - r * gprow;
+        const uint32_t mid = fx_fastdiv(t, gp_magic, gp_shift);
+        const uint32_t col0 = (t - mid * gpr) * FX_V;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          if (live && col0 + j < inner) M |= 1u << j;
+          e[j] = r * rowlen + mid * inner + col0 + j;
+          q.cv[j] = (int32_t)(col0 + j);
+        }
+        q.vd = vd;
+        q.step = 1;
+        fx_unflatten<R>(mid, vd, dk, mk, sk, q.c0);
+        q.c0[0] = (int32_t)s_rowmap[r];
       }
     };
+    const bool contig = !colmajor;
     // items of this output that belong to this wave: first, first + 4, ...
     // taken FX_K at a time so that their leading loads overlap
     uint32_t it0 = (wave_u + 4u - (item_base & 3u)) & 3u;
     for (; it0 < n_items; it0 += 4u * FX_K) {
       uint32_t P[FX_K][FX_V];
-#ifdef FX_PHASE_PROF
-      const bool pf = (oi == 1) && (it0 < 4u) && wave_u == 0;
-      if (pf) FX_PROF(16);
-#endif
       if (lead) {
 #pragma unroll
         for (uint32_t k = 0; k < FX_K; ++k) {
           const uint32_t it = it0 + 4u * k;
           if (it < n_items) {
             uint32_t e[FX_V], M;
-            int32_t c[FX_V][R];
-            make_item(it, e, M, c);
-            fx_lead_load<R>(cx, pb, c, M, P[k]);
+            FxCoord<R> q;
+            make_item(it, e, M, q);
+            fx_lead_load<R>(cx, pb, q, M, P[k]);
           }
-#ifdef FX_PHASE_PROF
-          if (pf) FX_PROF(17 + k);
-#endif
         }
       }
 #pragma unroll
@@ -1000,25 +1115,13 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         const uint32_t it = it0 + 4u * k;
         if (it < n_items) {
           uint32_t e[FX_V], M;
-          int32_t c[FX_V][R];
-          make_item(it, e, M, c);
-#ifdef FX_PHASE_PROF
-          if (pf && k == 0) FX_PROF(21);
-#endif
+          FxCoord<R> q;
+          make_item(it, e, M, q);
           uint32_t A[FX_V];
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
-          fx_run<R>(cx, lead ? pb + 1 : pb, pe, c, M, A);
-#ifdef FX_PHASE_PROF
-          if (pf && k == 0) FX_PROF(22);
-#endif
-#pragma unroll
-          for (int j = 0; j < FX_V; ++j) {
-            if ((M >> j) & 1u) fx_store(op, obase + e[j], odt, ovt, A[j]);
-          }
-#ifdef FX_PHASE_PROF
-          if (pf) FX_PROF(23 + k);
-#endif
+          fx_run<R>(cx, lead ? pb + 1 : pb, pe, q, M, A);
+          fx_store_vec(op, obase, e, M, contig, odt, ovt, A);
         }
       }
     }

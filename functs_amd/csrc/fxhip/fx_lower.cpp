@@ -1705,6 +1705,16 @@ static void fillDims(FxOut& o, const Shape& s) {
     o.dim[k] = d;
     fx_fastdiv_make(d, &o.magic[k], &o.shift[k]);
   }
+  // lane groups of FX_V elements along the last dimension
+  o.vd = s.empty() ? 0u : (uint32_t)s.size() - 1u;
+  o.inner = s.empty() ? 1u : (uint32_t)std::max<int64_t>(s.back(), 1);
+  o.gpr = (o.inner + FX_V - 1) / FX_V;
+  fx_fastdiv_make(o.gpr, &o.gp_magic, &o.gp_shift);
+  int64_t numel = 1;
+  for (int64_t d : s) numel *= d;
+  o.n_groups = (uint32_t)(numel / o.inner * o.gpr);
+  o.gprow = o.gpr;
+  fx_fastdiv_make(o.gprow, &o.gr_magic, &o.gr_shift);
 }
 
 }  // namespace
@@ -1863,6 +1873,9 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         // narrow rows with a long (predicated) program: walk column by column so that
         // predicates on the inner coordinate are uniform per wave
         od.colmajor = (od.rowlen >= 2 && od.rowlen <= 16 && (p.end - p.begin) >= 24) ? 1u : 0u;
+        od.gprow = std::max<uint32_t>(od.rowlen, 1) / od.inner * od.gpr;
+        if (s.size() <= 1) od.gprow = 1;  // rank 1: a group is FX_V kept rows
+        fx_fastdiv_make(std::max<uint32_t>(od.gprow, 1), &od.gr_magic, &od.gr_shift);
       }
       max_rank = std::max<int>(max_rank, (int)s.size());
       cb.outs.push_back(od);
@@ -1940,8 +1953,8 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
           od.n_blocks = (rows + 4u * od.unit_items - 1) / (4u * od.unit_items);
           od.lead = 0;
         } else {
-          const uint32_t unit = 4u * od.unit_items * FX_ITEM;
-          od.n_blocks = (od.numel + unit - 1) / unit;
+          const uint32_t unit = 4u * od.unit_items * (FX_ITEM / FX_V);  // groups per work unit
+          od.n_blocks = (od.n_groups + unit - 1) / unit;
         }
         b += od.n_blocks;
       }

@@ -625,28 +625,43 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 // them is computed: FX_K * FX_V loads per lane are in flight instead of FX_V.
 // The interpreter then starts behind the load with A preset.
 #define FX_K 4
+// The leading load of a program, decoded once per output: everything about it is
+// wave-uniform and the same for every item.
+struct FxLead {
+  int32_t cf[FX_MAXR];
+  int32_t base;
+  uint64_t p;
+  uint32_t dt;
+  bool cvt;
+};
+
 template <int R>
-__device__ __forceinline__ void fx_lead_load(const FxCtx& cx, int pc, const FxCoord<R>& q, uint32_t M,
-                                             uint32_t (&P)[FX_V]) {
+__device__ __forceinline__ FxLead fx_lead_decode(const FxCtx& cx, int pc) {
+  FxLead ld;
   const fx_u32x4 w = cx.insn[pc];
   const uint32_t w0 = uni(w.x);
-  const bool cvt = (w0 & (FX_F_I2F << 16)) != 0;
-  const uint32_t dt = w0 >> 24;
+  ld.cvt = (w0 & (FX_F_I2F << 16)) != 0;
+  ld.dt = w0 >> 24;
   const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + (int32_t)w.z * FX_AFF_WORDS);
   const fx_u32x4 a0 = ap[0], a1 = ap[1];
-  int32_t cf[FX_MAXR];
-  cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
+  ld.cf[0] = (int32_t)uni(a0.x); ld.cf[1] = (int32_t)uni(a0.y);
+  ld.cf[2] = (int32_t)uni(a0.z); ld.cf[3] = (int32_t)uni(a0.w);
   if (R > 4) {
     const fx_u32x4 a2 = ap[2];
-    cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
+    ld.cf[4] = (int32_t)uni(a2.x); ld.cf[5] = (int32_t)uni(a2.y);
   } else {
-    cf[4] = 0; cf[5] = 0;
+    ld.cf[4] = 0; ld.cf[5] = 0;
   }
-  const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task;
-  const uint64_t p = fx_ptr(cx, (int32_t)w.y);
+  ld.base = (int32_t)uni(a1.y) + (int32_t)uni(a1.x) * cx.task;
+  ld.p = fx_ptr(cx, (int32_t)w.y);
+  return ld;
+}
+
+template <int R>
+__device__ __forceinline__ void fx_lead_load(const FxLead& ld, const FxCoord<R>& q, uint32_t M, uint32_t (&P)[FX_V]) {
   int32_t off[FX_V];
-  const bool consecutive = fx_offsets<R>(q, cf, base, off);
-  fx_load_vec(p, off, M, dt, cvt, consecutive, P);
+  const bool consecutive = fx_offsets<R>(q, ld.cf, ld.base, off);
+  fx_load_vec(ld.p, off, M, ld.dt, ld.cvt, consecutive, P);
 }
 
 __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint32_t shift) {
@@ -848,13 +863,14 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
 
     uint32_t P[FX_K][FX_V];
     if (lead) {
+      const FxLead ld = fx_lead_decode<R>(cx, pb);
 #pragma unroll
       for (uint32_t k = 0; k < FX_K; ++k) {
         if (k < kmax && item0 + k < n_items) {
           uint32_t e[FX_V], M;
           FxCoord<R> q;
           make_item(k, e, M, q);
-          fx_lead_load<R>(cx, pb, q, M, P[k]);
+          fx_lead_load<R>(ld, q, M, P[k]);
         }
       }
     }
@@ -1012,8 +1028,12 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   // items) overlaps with the short programs of the wide ones instead of
   // serialising the whole workgroup behind it.  No barrier from here on.
   const uint32_t wave_u = uni(wave);
-  uint32_t item_base = 0;
-  for (uint32_t oi = 0; oi < n_outs; ++oi) {
+  // Half of the waves walk the outputs backwards: a latency-bound output (a long
+  // predicated program on a few items) then overlaps, on the same SIMD, with the
+  // arithmetic-bound wide outputs of the other waves.
+  const bool backwards = ((blockIdx.x + wave_u) & 1u) != 0;
+  for (uint32_t oo = 0; oo < n_outs; ++oo) {
+    const uint32_t oi = backwards ? n_outs - 1u - oo : oo;
     const uint32_t* od = outs + oi * ow;
     const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
     const uint32_t colmajor = uni(od[FX_W(FxOut, colmajor)]);
@@ -1095,7 +1115,11 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     const bool contig = !colmajor;
     // items of this output that belong to this wave: first, first + 4, ...
     // taken FX_K at a time so that their leading loads overlap
-    uint32_t it0 = (wave_u + 4u - (item_base & 3u)) & 3u;
+    // (the rotation by the output index spreads single-item outputs over the waves; it
+    // must not depend on the order in which a wave walks the outputs)
+    uint32_t it0 = (wave_u + 4u - (oi & 3u)) & 3u;
+    FxLead ld;
+    if (lead) ld = fx_lead_decode<R>(cx, pb);
     for (; it0 < n_items; it0 += 4u * FX_K) {
       uint32_t P[FX_K][FX_V];
       if (lead) {
@@ -1106,7 +1130,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
             uint32_t e[FX_V], M;
             FxCoord<R> q;
             make_item(it, e, M, q);
-            fx_lead_load<R>(cx, pb, q, M, P[k]);
+            fx_lead_load<R>(ld, q, M, P[k]);
           }
         }
       }
@@ -1125,7 +1149,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         }
       }
     }
-    item_base += n_items;
     FX_PROF(4 + oi * 4 + (threadIdx.x >> 6));
   }
 }

@@ -93,6 +93,24 @@ enum FxOp : uint32_t {
   FX_OP_COUNT
 };
 
+// instructions the batched "pure" interpreter implements (binary ones only with FX_F_IMM)
+static inline bool fx_op_is_pure_unary(uint32_t op) {
+  switch (op) {
+    case FX_FNEG: case FX_FABS: case FX_EXP: case FX_SQRT: case FX_RSQRT: case FX_RCP: case FX_SIGMOID:
+    case FX_RELU: case FX_F2I: case FX_I2F:
+      return true;
+    default: return false;
+  }
+}
+static inline bool fx_op_is_pure_binary(uint32_t op) {
+  switch (op) {
+    case FX_FADD: case FX_FSUB: case FX_FRSUB: case FX_FMUL: case FX_FDIV: case FX_FMIN: case FX_FMAX:
+    case FX_IADD: case FX_IMUL: case FX_FLT: case FX_FLE: case FX_FGT: case FX_FGE: case FX_FEQ: case FX_FNE:
+      return true;
+    default: return false;
+  }
+}
+
 #define FX_F_IMM 1u  // binary op takes its second operand from imm
 #define FX_F_I2F 2u  // LDA/LDB/AFFA/AFFB/SCLA/SCLB: convert the int result to float
 
@@ -161,6 +179,9 @@ struct FxOut {
   uint32_t gprow;                 // compaction: groups per kept row: rowlen / inner * gpr
   uint32_t gr_magic, gr_shift;    // fast division by gprow
   uint32_t n_groups;              // dense: groups per task: numel / inner * gpr
+  uint32_t pure;                  // after the leading load only coordinate-free elementwise instructions with
+                                  // immediate operands follow: FX_K items are interpreted as one batch
+  uint32_t pad[3];
 };
 
 // An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows

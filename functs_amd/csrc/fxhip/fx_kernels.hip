@@ -625,6 +625,85 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 // them is computed: FX_K * FX_V loads per lane are in flight instead of FX_V.
 // The interpreter then starts behind the load with A preset.
 #define FX_K 4
+// Interpreter for the tail of a "pure" program (FxOut::pure): coordinate-free
+// elementwise instructions with immediate operands.  One pass over the program
+// serves the FX_K items of a batch, so fetch and dispatch are paid once per
+// FX_K * FX_V elements of a lane.
+#define FX_NB (FX_K * FX_V)
+__device__ __forceinline__ void fx_run_pure(const FxCtx& cx, int pc, const int pc_end, uint32_t (&X)[FX_NB]) {
+  for (; pc < pc_end; ++pc) {
+    const fx_u32x4 w = cx.insn[pc];
+    const uint32_t op = uni(w.x) & 0xffffu;
+    const uint32_t imm = uni(w.w);
+#define FX_PU_F(expr)                                      \
+  {                                                        \
+    _Pragma("unroll") for (int j = 0; j < FX_NB; ++j) {    \
+      float a = u2f(X[j]);                                 \
+      X[j] = f2u(expr);                                    \
+    }                                                      \
+  } break
+#define FX_PB_F(expr)                                      \
+  {                                                        \
+    const float b = u2f(imm);                              \
+    _Pragma("unroll") for (int j = 0; j < FX_NB; ++j) {    \
+      float a = u2f(X[j]);                                 \
+      X[j] = f2u(expr);                                    \
+    }                                                      \
+  } break
+#define FX_PC_F(expr)                                      \
+  {                                                        \
+    const float b = u2f(imm);                              \
+    _Pragma("unroll") for (int j = 0; j < FX_NB; ++j) {    \
+      float a = u2f(X[j]);                                 \
+      X[j] = (expr) ? 1u : 0u;                             \
+    }                                                      \
+  } break
+    switch (op) {
+      case FX_FNEG: FX_PU_F(-a);
+      case FX_FABS: FX_PU_F(fabsf(a));
+      case FX_EXP: FX_PU_F(expf(a));
+      case FX_SQRT: FX_PU_F(sqrtf(a));
+      case FX_RSQRT: FX_PU_F(1.0f / sqrtf(a));
+      case FX_RCP: FX_PU_F(1.0f / a);
+      case FX_SIGMOID: FX_PU_F(fx_sigmoid(a));
+      case FX_RELU: FX_PU_F((a <= 0.0f) ? 0.0f : a);
+      case FX_F2I:
+#pragma unroll
+        for (int j = 0; j < FX_NB; ++j) X[j] = (uint32_t)(int32_t)u2f(X[j]);
+        break;
+      case FX_I2F:
+#pragma unroll
+        for (int j = 0; j < FX_NB; ++j) X[j] = f2u((float)(int32_t)X[j]);
+        break;
+      case FX_FADD: FX_PB_F(a + b);
+      case FX_FSUB: FX_PB_F(a - b);
+      case FX_FRSUB: FX_PB_F(b - a);
+      case FX_FMUL: FX_PB_F(a * b);
+      case FX_FDIV: FX_PB_F(a / b);
+      case FX_FMIN: FX_PB_F(fx_fmin(a, b));
+      case FX_FMAX: FX_PB_F(fx_fmax(a, b));
+      case FX_IADD:
+#pragma unroll
+        for (int j = 0; j < FX_NB; ++j) X[j] = (uint32_t)((int32_t)X[j] + (int32_t)imm);
+        break;
+      case FX_IMUL:
+#pragma unroll
+        for (int j = 0; j < FX_NB; ++j) X[j] = (uint32_t)((int32_t)X[j] * (int32_t)imm);
+        break;
+      case FX_FLT: FX_PC_F(a < b);
+      case FX_FLE: FX_PC_F(a <= b);
+      case FX_FGT: FX_PC_F(a > b);
+      case FX_FGE: FX_PC_F(a >= b);
+      case FX_FEQ: FX_PC_F(a == b);
+      case FX_FNE: FX_PC_F(a != b);
+      default: break;
+    }
+#undef FX_PU_F
+#undef FX_PB_F
+#undef FX_PC_F
+  }
+}
+
 // The leading load of a program, decoded once per output: everything about it is
 // wave-uniform and the same for every item.
 struct FxLead {
@@ -861,6 +940,32 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
       q.c0[0] = vd == 0 ? 0 : (int32_t)rem;
     };
 
+    if (uni(od[FX_W(FxOut, pure)])) {
+      // the FX_K items of this wave as one batch (items past the end have no live element)
+      const FxLead ld = fx_lead_decode<R>(cx, pb);
+      uint32_t X[FX_NB], e0[FX_K], Mk[FX_K];
+#pragma unroll
+      for (uint32_t k = 0; k < FX_K; ++k) {
+        uint32_t e[FX_V], M, Pk[FX_V];
+        FxCoord<R> q;
+        make_item(k, e, M, q);
+        if (k >= kmax) M = 0;
+        fx_lead_load<R>(ld, q, M, Pk);
+        e0[k] = e[0];
+        Mk[k] = M;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) X[k * FX_V + j] = Pk[j];
+      }
+      fx_run_pure(cx, pb + 1, pe, X);
+#pragma unroll
+      for (uint32_t k = 0; k < FX_K; ++k) {
+        uint32_t e[FX_V], Ak[FX_V];
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) { e[j] = e0[k] + j; Ak[j] = X[k * FX_V + j]; }
+        fx_store_vec(op, obase, e, Mk[k], true, odt, ovt, Ak);
+      }
+      continue;
+    }
     uint32_t P[FX_K][FX_V];
     if (lead) {
       const FxLead ld = fx_lead_decode<R>(cx, pb);
@@ -1120,6 +1225,33 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     uint32_t it0 = (wave_u + 4u - (oi & 3u)) & 3u;
     FxLead ld;
     if (lead) ld = fx_lead_decode<R>(cx, pb);
+    if (uni(od[FX_W(FxOut, pure)])) {
+      // FX_K items as one batch (items past the end have no live element)
+      for (; it0 < n_items; it0 += 4u * FX_K) {
+        uint32_t X[FX_NB], e0[FX_K], Mk[FX_K];
+#pragma unroll
+        for (uint32_t k = 0; k < FX_K; ++k) {
+          uint32_t e[FX_V], M, Pk[FX_V];
+          FxCoord<R> q;
+          make_item(it0 + 4u * k, e, M, q);
+          fx_lead_load<R>(ld, q, M, Pk);
+          e0[k] = e[0];
+          Mk[k] = M;
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) X[k * FX_V + j] = Pk[j];
+        }
+        fx_run_pure(cx, pb + 1, pe, X);
+#pragma unroll
+        for (uint32_t k = 0; k < FX_K; ++k) {
+          uint32_t e[FX_V], Ak[FX_V];
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) { e[j] = e0[k] + j; Ak[j] = X[k * FX_V + j]; }
+          fx_store_vec(op, obase, e, Mk[k], true, odt, ovt, Ak);
+        }
+      }
+      FX_PROF(4 + oi * 4 + (threadIdx.x >> 6));
+      continue;
+    }
     for (; it0 < n_items; it0 += 4u * FX_K) {
       uint32_t P[FX_K][FX_V];
       if (lead) {

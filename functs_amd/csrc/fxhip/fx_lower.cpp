@@ -1863,6 +1863,12 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         // leading load: unconditional, affine, not inside a reduction loop
         const FxInsn& i0 = L.code[p.begin];
         od.lead = (p.end > p.begin && i0.op == FX_LDA) ? 1u : 0u;
+        bool pure = od.lead != 0 && !p.rowwave;
+        for (uint32_t pc = p.begin + 1; pure && pc < p.end; ++pc) {
+          const FxInsn& in = L.code[pc];
+          pure = fx_op_is_pure_unary(in.op) || (fx_op_is_pure_binary(in.op) && (in.flags & FX_F_IMM));
+        }
+        od.pure = pure ? 1u : 0u;
       }
       if (P->mode == FX_MODE_COMPACT) {
         FX_CHECK(!s.empty() && s[0] == (int64_t)cb.cls.n_rows, FX_E_INVALID,
@@ -1876,6 +1882,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         od.gprow = std::max<uint32_t>(od.rowlen, 1) / od.inner * od.gpr;
         if (s.size() <= 1) od.gprow = 1;  // rank 1: a group is FX_V kept rows
         fx_fastdiv_make(std::max<uint32_t>(od.gprow, 1), &od.gr_magic, &od.gr_shift);
+        if (od.colmajor) od.pure = 0;
       }
       max_rank = std::max<int>(max_rank, (int)s.size());
       cb.outs.push_back(od);

@@ -979,7 +979,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
         }
       }
     }
-#pragma unroll
+    // one copy of the interpreter: the loop stays rolled, the preloaded values are picked by selects
+#pragma unroll 1
     for (uint32_t k = 0; k < FX_K; ++k) {
       if (k < kmax && item0 + k < n_items) {
         uint32_t e[FX_V], M;
@@ -987,7 +988,12 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
         make_item(k, e, M, q);
         uint32_t A[FX_V];
 #pragma unroll
-        for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
+        for (int j = 0; j < FX_V; ++j) {
+          uint32_t v = P[0][j];
+#pragma unroll
+          for (uint32_t kk = 1; kk < FX_K; ++kk) v = (k == kk) ? P[kk][j] : v;
+          A[j] = lead ? v : 0u;
+        }
         fx_run<R>(cx, lead ? pb + 1 : pb, pe, q, M, A);
         fx_store_vec(op, obase, e, M, true, odt, ovt, A);
       }
@@ -1266,7 +1272,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
           }
         }
       }
-#pragma unroll
+#pragma unroll 1
       for (uint32_t k = 0; k < FX_K; ++k) {
         const uint32_t it = it0 + 4u * k;
         if (it < n_items) {
@@ -1275,7 +1281,12 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
           make_item(it, e, M, q);
           uint32_t A[FX_V];
 #pragma unroll
-          for (int j = 0; j < FX_V; ++j) A[j] = lead ? P[k][j] : 0u;
+          for (int j = 0; j < FX_V; ++j) {
+            uint32_t v = P[0][j];
+#pragma unroll
+            for (uint32_t kk = 1; kk < FX_K; ++kk) v = (k == kk) ? P[kk][j] : v;
+            A[j] = lead ? v : 0u;
+          }
           fx_run<R>(cx, lead ? pb + 1 : pb, pe, q, M, A);
           fx_store_vec(op, obase, e, M, contig, odt, ovt, A);
         }

@@ -940,8 +940,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
       q.c0[0] = vd == 0 ? 0 : (int32_t)rem;
     };
 
-    if (uni(od[FX_W(FxOut, pure)])) {
-      // the FX_K items of this wave as one batch (items past the end have no live element)
+    if (uni(od[FX_W(FxOut, pure)]) && kmax == FX_K && item0 + FX_K <= n_items) {
+      // the FX_K items of this wave as one batch; an incomplete batch takes the generic path
       const FxLead ld = fx_lead_decode<R>(cx, pb);
       uint32_t X[FX_NB], e0[FX_K], Mk[FX_K];
 #pragma unroll
@@ -949,7 +949,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
         uint32_t e[FX_V], M, Pk[FX_V];
         FxCoord<R> q;
         make_item(k, e, M, q);
-        if (k >= kmax) M = 0;
         fx_lead_load<R>(ld, q, M, Pk);
         e0[k] = e[0];
         Mk[k] = M;
@@ -1142,7 +1141,11 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   // Half of the waves walk the outputs backwards: a latency-bound output (a long
   // predicated program on a few items) then overlaps, on the same SIMD, with the
   // arithmetic-bound wide outputs of the other waves.
+#ifdef FX_PHASE_PROF
+  const bool backwards = false;  // profiling builds time the outputs one after the other
+#else
   const bool backwards = ((blockIdx.x + wave_u) & 1u) != 0;
+#endif
   for (uint32_t oo = 0; oo < n_outs; ++oo) {
     const uint32_t oi = backwards ? n_outs - 1u - oo : oo;
     const uint32_t* od = outs + oi * ow;
@@ -1232,8 +1235,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     FxLead ld;
     if (lead) ld = fx_lead_decode<R>(cx, pb);
     if (uni(od[FX_W(FxOut, pure)])) {
-      // FX_K items as one batch (items past the end have no live element)
-      for (; it0 < n_items; it0 += 4u * FX_K) {
+      // FX_K items as one batch; an incomplete batch at the end takes the generic path
+      for (; it0 + 4u * (FX_K - 1u) < n_items; it0 += 4u * FX_K) {
         uint32_t X[FX_NB], e0[FX_K], Mk[FX_K];
 #pragma unroll
         for (uint32_t k = 0; k < FX_K; ++k) {
@@ -1255,8 +1258,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
           fx_store_vec(op, obase, e, Mk[k], true, odt, ovt, Ak);
         }
       }
-      FX_PROF(4 + oi * 4 + (threadIdx.x >> 6));
-      continue;
     }
     for (; it0 < n_items; it0 += 4u * FX_K) {
       uint32_t P[FX_K][FX_V];

@@ -5,6 +5,7 @@ benchmark models.  They are inputs to functs_amd.jit.script / build.
   yolov3_postproc  functs/benchmark/ai_model/yolov3/yolov3_bbox.py:12-23, 206-243
   yolov3_batched   the per-image loop of yolov3_bbox.py:233-241
   ssd_postproc     functs/benchmark/ai_model/ssd/ssd_bbox.py:121-154, 163-172, 268
+  lstm             functs/benchmark/ai_model/lstm/lstm.py:79-133
 """
 from typing import List
 
@@ -70,9 +71,39 @@ def ssd_postproc(loc: Tensor, conf: Tensor, priors: Tensor):
     return out_b, out_s
 
 
+def lstm(x: Tensor, wih: Tensor, whh: Tensor, bih: Tensor, bhh: Tensor):
+    """x [T, B, H]; wih / whh [L, 4, H, H]; bih / bhh [L, 4, 1, H] (gate order i, f, g, o)."""
+    seq_len = x.size(0)
+    n_layers = wih.size(0)
+    batch = x.size(1)
+    hidden = x.size(2)
+    out = torch.zeros(seq_len, batch, hidden, device=x.device)
+    state_h = torch.zeros(n_layers, batch, hidden, device=x.device)
+    state_c = torch.zeros(n_layers, batch, hidden, device=x.device)
+    for t in range(seq_len):
+        cur = x[t]
+        for j in range(n_layers):
+            h = state_h[j]
+            c = state_c[j]
+            ih = torch.matmul(cur, wih[j]) + bih[j]
+            hh = torch.matmul(h, whh[j]) + bhh[j]
+            ingate = torch.sigmoid(ih[0] + hh[0])
+            forgetgate = torch.sigmoid(ih[1] + hh[1])
+            cellgate = torch.tanh(ih[2] + hh[2])
+            outgate = torch.sigmoid(ih[3] + hh[3])
+            c2 = (forgetgate * c) + (ingate * cellgate)
+            h2 = outgate * torch.tanh(c2)
+            state_c[j] = c2
+            state_h[j] = h2
+            cur = h2
+        out[t] = cur
+    return out, state_h, state_c
+
+
 PROGRAMS = {
     "c1": get_started,
     "c2": yolov3_postproc,
     "c3": ssd_postproc,
+    "c4": lstm,
     "c5": yolov3_batched,
 }

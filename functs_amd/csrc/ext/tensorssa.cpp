@@ -152,7 +152,14 @@ void pruneForest(std::shared_ptr<Graph> g, ViewForest& f) {
     for (const Use& u : v->uses()) {
       Node* user = u.user;
       switch (user->kind()) {
-        case c10::prim::ListConstruct: case c10::prim::TupleConstruct: case c10::prim::DictConstruct:
+        case c10::prim::TupleConstruct: {
+          // a tuple that only packs the values the graph returns holds no second name
+          bool only_returned = true;
+          for (const Use& tu : user->output()->uses())
+            only_returned = only_returned && tu.user == g->return_node();
+          if (!only_returned) bad.insert(root);
+        } break;
+        case c10::prim::ListConstruct: case c10::prim::DictConstruct:
         case c10::aten::append: case c10::prim::SetAttr:
           bad.insert(root);
           break;

@@ -360,6 +360,7 @@ class RegionRunner {
       if (v.isDouble()) { a.kind = 2; a.fval = v.toDouble(); sig << "|f"; }
       else if (v.isBool()) { a.kind = 3; a.ival = v.toBool(); sig << "|b"; }
       else if (v.isInt()) { a.kind = 1; a.ival = v.toInt(); sig << "|i"; }
+      else if (v.isDevice() || v.isNone()) { a.kind = 1; a.ival = 0; sig << "|d"; }  // placement only: outputs follow the tensors
       else TORCH_CHECK(false, "ParallelFunctor: unsupported scalar argument ", v.tagKind());
       args.push_back(a);
     };

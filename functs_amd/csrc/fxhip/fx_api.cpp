@@ -353,7 +353,6 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
   li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
   li.n_temps = pl->n_temps;
-  li.stage_words = pl->stage_words;
   li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
   if (pl->mode == FX_MODE_COMPACT) {
     // tasks without rows launch no tile: their total is published here.  The

@@ -84,9 +84,6 @@ enum FxOp : uint32_t {
   FX_RBEGIN, // push loop: counter = 0, extent = imm, acc slot = temp[a] preset by program
   FX_RNEXT,  // counter += 1; if counter < extent jump to a
   FX_RIDX,   // A = (int) loop counter of depth a
-  // ---- loads from an input tile staged in LDS (row-tiled kernels) ----
-  FX_LDSA,   // A = stage[a] at affine[b](coords) relative to the tile; dt = storage dtype
-  FX_LDSB,
   // ---- reductions across the wave (row-per-wave mapping, FxOut::rowwave) ----
   FX_WMAX,   // A = max of A over every live element of the wave (NaN-propagating)
   FX_WSUM,   // A = sum of A over every live element of the wave
@@ -145,7 +142,6 @@ struct FxLaunchInfo {
   uint32_t n_p;         // pointer slots in use
   uint32_t n_s;         // scalar slots in use
   uint32_t n_temps;     // LDS temp slots per lane
-  uint32_t stage_words; // LDS words of the largest per-tile stage area (multiple of 4)
   uint32_t total_units; // dense kernel: number of FX_UNIT work units
 };
 
@@ -184,17 +180,6 @@ struct FxOut {
   uint32_t pad[3];
 };
 
-// An input whose every access is  S * coord[0] + rest,  0 <= rest < S : the rows
-// [r0, r0 + row_tile) of a tile are one contiguous run of S * row_tile elements,
-// copied to LDS with 128-bit loads before the programs run.
-struct FxStage {
-  uint32_t ptr_slot;   // may carry FX_SLOT_TASK
-  uint32_t row_elems;  // S
-  int32_t tcoef;       // element offset per task (shared buffer sliced by the task index)
-  uint32_t lds_off;    // word offset inside the stage area
-  uint32_t n_rows;     // rows of the buffer along coordinate 0 (clamps the last tile)
-  uint32_t pad[3];
-};
 
 struct FxClass {
   uint32_t block_begin, block_end;  // grid range covered by this class (dense / scatter pass)
@@ -213,8 +198,7 @@ struct FxClass {
   uint32_t mask_vt;
   uint32_t cnt_block_begin, cnt_block_end;  // grid range in the count pass
   uint32_t cnt_blocks_per_task;
-  uint32_t n_stages;                // staged inputs (FxStage[n_stages] at off_stages)
-  uint32_t off_stages;
+  uint32_t pad2[2];
 };
 
 enum FxMode : uint32_t { FX_MODE_DENSE = 0, FX_MODE_COMPACT = 1 };

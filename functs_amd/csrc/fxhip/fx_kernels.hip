@@ -63,8 +63,6 @@ struct FxCtx {
   uint32_t tp_off;        // index of this task's first pointer
   uint32_t ts_off;        // index of this task's first scalar
   uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
-  const uint32_t* stage;  // LDS: input tiles staged by the row-tiled kernels
-  const int32_t* stage_adj;  // LDS: per stage, word index of element 0 of the buffer (may be negative)
   int task;
 };
 
@@ -377,31 +375,6 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
           for (int j = 0; j < FX_V; ++j) {
             const uint32_t v = cvt ? f2u((float)off[j]) : (uint32_t)off[j];
             if (op == FX_AFFA) A[j] = v; else B[j] = v;
-          }
-        }
-      } break;
-      case FX_LDSA:
-      case FX_LDSB: {
-        const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + ib * FX_AFF_WORDS);
-        const fx_u32x4 a0 = ap[0], a1 = ap[1];
-        int32_t cf[FX_MAXR];
-        cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
-        if (R > 4) {
-          const fx_u32x4 a2 = ap[2];
-          cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
-        } else {
-          cf[4] = 0; cf[5] = 0;
-        }
-        // the task term is part of the tile's global origin, not of the LDS index
-        const int32_t base = (int32_t)a1.y + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1 + cx.stage_adj[ia];
-        int32_t off[FX_V];
-        fx_offsets<R>(q, cf, base, off);
-#pragma unroll
-        for (int j = 0; j < FX_V; ++j) {
-          if ((M >> j) & 1u) {
-            uint32_t v = cx.stage[off[j]];
-            if (cvt) v = f2u((float)(int32_t)v);
-            if (op == FX_LDSA) A[j] = v; else B[j] = v;
           }
         }
       } break;
@@ -753,11 +726,10 @@ struct FxLaunch {
   uint32_t blob_words;  // multiple of 4
   uint32_t n_p;         // pointers in use in FxDyn::p
   uint32_t n_s;         // scalars in use in FxDyn::s
-  uint32_t stage_off;   // word offset of the stage area in LDS (multiple of 4)
   uint32_t temps_off;   // word offset of the temp area in LDS (multiple of 4)
+  uint32_t pad;         // keeps the struct at 24 bytes: the tables that follow it in the argument segment are 8-byte aligned
   uint32_t total_units; // dense: work units of FX_UNIT elements; the grid strides over them
 };
-#define FX_MAX_STAGES 8
 #define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
 
 __device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict__ sb, const FxLaunch& la) {
@@ -813,48 +785,8 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
   cx.tp_off = n_sptr + (uint32_t)w.task * n_tptr;
   cx.ts_off = n_sscal + (uint32_t)w.task * n_tscal;
   cx.temps = L + la.temps_off + threadIdx.x;
-  cx.stage = L + la.stage_off;
-  cx.stage_adj = nullptr;
   cx.task = w.task;
   return cx;
-}
-
-// Copy rows [r0, r0 + rows) of every staged input of this class into LDS.
-// 128-bit loads wherever the 16-byte group lies inside the tile; the (at most
-// two) partial groups at the ends are read element-wise, so nothing outside
-// the tile is touched whatever the alignment of the buffer.
-__device__ __forceinline__ void fx_stage_tiles(uint32_t* L, const FxLaunch& la, const FxWork& w, const FxCtx& cx,
-                                               uint32_t r0, uint32_t rt, int32_t* s_adj) {
-  const uint32_t n_stages = uni(w.cls[FX_W(FxClass, n_stages)]);
-  const uint32_t* st = L + uni(w.cls[FX_W(FxClass, off_stages)]);
-  uint32_t* area = L + la.stage_off;
-  for (uint32_t s = 0; s < n_stages; ++s) {
-    const uint32_t* d = st + s * (sizeof(FxStage) / 4);
-    const uint32_t S = uni(d[FX_W(FxStage, row_elems)]);
-    const int32_t tcoef = (int32_t)uni(d[FX_W(FxStage, tcoef)]);
-    const uint32_t lds_off = uni(d[FX_W(FxStage, lds_off)]);
-    const uint32_t n_rows = uni(d[FX_W(FxStage, n_rows)]);
-    const uint32_t rows = (r0 + rt <= n_rows) ? rt : (n_rows > r0 ? n_rows - r0 : 0u);
-    const uint32_t count = rows * S;
-    const int64_t g0 = (int64_t)S * r0 + (int64_t)tcoef * w.task;
-    const uint64_t p = fx_ptr(cx, (int32_t)d[FX_W(FxStage, ptr_slot)]) + (uint64_t)(g0 * 4);
-    const uint32_t mis = (uint32_t)((p >> 2) & 3ull);
-    const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(p - 4ull * mis);
-    const FX_AS1 uint32_t* g1 = (const FX_AS1 uint32_t*)(p - 4ull * mis);
-    const uint32_t n4 = (mis + count + 3u) >> 2;
-    uint32_t* dst = area + lds_off;
-    for (uint32_t i = threadIdx.x; i < n4; i += FX_BLOCK) {
-      const uint32_t e = i * 4u;  // index in the aligned view; tile elements are [mis, mis + count)
-      if (e >= mis && e + 4u <= mis + count) {
-        *(fx_u32x4*)(dst + e) = g4[i];
-      } else {
-#pragma unroll
-        for (uint32_t k = 0; k < 4u; ++k)
-          if (e + k >= mis && e + k < mis + count) dst[e + k] = g1[e + k];
-      }
-    }
-    if (threadIdx.x == 0) s_adj[s] = (int32_t)(lds_off + mis) - (int32_t)(S * r0);
-  }
 }
 
 }  // namespace
@@ -1077,18 +1009,14 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   __shared__ uint32_t s_wsum[FX_BLOCK / 64];
   __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
   __shared__ uint32_t s_prefix;
-  __shared__ int32_t s_adj[FX_MAX_STAGES];
   if (threadIdx.x == 0) FX_PROF(0);
   fx_stage(L, sb, la);
   if (threadIdx.x == 0) FX_PROF(1);
   const FxWork w = fx_locate<false>(L, blockIdx.x);
   FxCtx cx = fx_make_ctx(L, la, w);
-  cx.stage_adj = s_adj;
 
   const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
   const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
-  // input tiles -> LDS (completed by the barriers of the row-map construction below)
-  fx_stage_tiles(L, la, w, cx, w.local_block * rt, rt, s_adj);
   const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
   const uint32_t tile = w.local_block;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -1438,9 +1366,9 @@ static FxLaunch make_launch(const FxLaunchInfo& li) {
   la.blob_words = li.blob_words;
   la.n_p = li.n_p;
   la.n_s = li.n_s;
-  la.stage_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
-  la.temps_off = la.stage_off + li.stage_words;
+  la.temps_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
   la.total_units = li.total_units;
+  la.pad = 0;
   return la;
 }
 

@@ -1623,80 +1623,8 @@ struct ClassBuild {
   std::vector<FxInsn> code;
   std::vector<FxAffine> affs;
   std::vector<FxOut> outs;
-  std::vector<FxStage> stages;
   FxClass cls;
 };
-
-// Which inputs of a row-tiled class can be staged in LDS: every load of the
-// buffer inside the output programs must have the form S * coord[0] + rest with
-// 0 <= rest < S (one contiguous run per tile), a 4-byte element type and one
-// common task stride.
-static void findStages(ClassBuild& cb, const std::vector<PtrSrc>& sptr, const std::vector<PtrSrc>& tptr) {
-  struct Use { bool ok = true; bool any = false; int64_t S = 0; int64_t tcoef = 0; };
-  std::map<int, Use> uses;
-  auto is_input = [&](int slot) {
-    const auto& tab = (slot & FX_SLOT_TASK) ? tptr : sptr;
-    size_t i = (size_t)(slot & 0xffff);
-    return i < tab.size() && tab[i].kind == PtrSrc::INPUT;
-  };
-  for (const FxOut& od : cb.outs) {
-    for (uint32_t pc = od.prog_begin; pc < od.prog_end; ++pc) {
-      const FxInsn& ins = cb.code[pc];
-      if (ins.op == FX_LDXA) { uses[ins.a].ok = false; continue; }
-      if (ins.op != FX_LDA && ins.op != FX_LDB) continue;
-      Use& u = uses[ins.a];
-      if (!u.ok) continue;
-      const FxAffine& a = cb.affs[ins.b];
-      bool ok = is_input(ins.a) && (ins.dt == FX_F32 || ins.dt == FX_I32) && a.rcoef[0] == 0 && a.rcoef[1] == 0;
-      int64_t S = fx_aff_coef(&a, 0);
-      ok = ok && S > 0;
-      int64_t lo = a.base, hi = a.base;
-      for (int k = 1; k < FX_MAXR; ++k) {
-        int64_t cf = fx_aff_coef(&a, k), ext = (int64_t)od.dim[k] - 1;
-        if (cf >= 0) hi += cf * ext; else lo += cf * ext;
-      }
-      ok = ok && lo >= 0 && hi < S;
-      if (ok && u.any) ok = (u.S == S && u.tcoef == a.tcoef);
-      if (!ok) { u.ok = false; continue; }
-      u.any = true; u.S = S; u.tcoef = a.tcoef;
-    }
-  }
-  for (auto& kv : uses) {
-    if (!kv.second.ok || !kv.second.any || cb.stages.size() >= 8) continue;
-    FxStage st;
-    memset(&st, 0, sizeof(st));
-    st.ptr_slot = (uint32_t)kv.first;
-    st.row_elems = (uint32_t)kv.second.S;
-    st.tcoef = (int32_t)kv.second.tcoef;
-    st.n_rows = cb.cls.n_rows;
-    cb.stages.push_back(st);
-  }
-}
-
-static void applyStages(ClassBuild& cb, uint32_t row_tile) {
-  struct Fix { ClassBuild& cb; ~Fix() { for (auto& od : cb.outs) if (od.prog_end > od.prog_begin && cb.code[od.prog_begin].op != FX_LDA) od.lead = 0; } } fix{cb};
-  uint32_t off = 0;
-  for (auto& st : cb.stages) {
-    st.lds_off = off;
-    off += (row_tile * st.row_elems + 4u + 3u) & ~3u;
-  }
-  for (const FxOut& od : cb.outs)
-    for (uint32_t pc = od.prog_begin; pc < od.prog_end; ++pc) {
-      FxInsn& ins = cb.code[pc];
-      if (ins.op != FX_LDA && ins.op != FX_LDB) continue;
-      for (size_t s = 0; s < cb.stages.size(); ++s)
-        if ((int32_t)cb.stages[s].ptr_slot == ins.a) {
-          ins.op = ins.op == FX_LDA ? FX_LDSA : FX_LDSB;
-          ins.a = (int32_t)s;
-          break;
-        }
-    }
-}
-static uint32_t stageWords(const ClassBuild& cb, uint32_t row_tile) {
-  uint32_t off = 0;
-  for (auto& st : cb.stages) off += (row_tile * st.row_elems + 4u + 3u) & ~3u;
-  return off;
-}
 
 static void fillDims(FxOut& o, const Shape& s) {
   o.rank = (uint32_t)s.size();
@@ -1893,47 +1821,12 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     max_temps = std::max(max_temps, L.maxTemps);
   }
 
-  // grids.  Row tile of the compaction passes: as large as the LDS budget of the
-  // staged input tiles allows while leaving enough tiles to fill 256 CUs.
+  // grids.  Row tile of the compaction passes: 256 rows unless that leaves too few
+  // tiles to fill 256 CUs.
   uint32_t row_tile = 64;
-  P->stage_words = 0;
   if (P->mode == FX_MODE_COMPACT) {
-    // staging input tiles in LDS is an experiment switch: it trades occupancy
-    // and tile size for load latency
-    if (getenv("FX_STAGE_TILES") && atoi(getenv("FX_STAGE_TILES")) > 0)
-      for (auto& cb : classes) findStages(cb, slots.sptr, slots.tptr);
-    size_t fixed_words = 64;  // header, class table slack
-    for (auto& cb : classes)
-      fixed_words += cb.code.size() * 4 + 4 + cb.affs.size() * FX_AFF_WORDS + cb.outs.size() * (sizeof(FxOut) / 4) +
-                     cb.stages.size() * (sizeof(FxStage) / 4) + sizeof(FxClass) / 4 + 8;
-    fixed_words += (size_t)T + 2 * (slots.sptr.size() + slots.tptr.size() * (size_t)T) +
-                   (slots.sscal.size() + slots.tscal.size() * (size_t)T) + (size_t)max_temps * FX_V * FX_BLOCK;
-    const size_t budget = 64 * 1024 / 4;
-    auto fits = [&](uint32_t rt) {
-      uint32_t sw = 0;
-      for (auto& cb : classes) sw = std::max(sw, stageWords(cb, rt));
-      return fixed_words + sw <= budget;
-    };
-    const uint32_t cands[3] = {256, 128, 64};
-    bool chosen = false;
-    for (uint32_t rt : cands) {
-      if (!fits(rt)) continue;
-      if (total_rows / rt >= 512 || rt == 64) { row_tile = rt; chosen = true; break; }
-    }
-    if (!chosen) {
-      // the staged tiles do not fit even at the smallest tile: read inputs from global memory
-      for (auto& cb : classes) cb.stages.clear();
-      if (total_rows / 64 >= 4096) row_tile = 256;
-      else if (total_rows / 64 >= 2048) row_tile = 128;
-    }
-    if (getenv("FX_ROW_TILE")) {  // experiment switch
-      int rt = atoi(getenv("FX_ROW_TILE"));
-      if ((rt == 64 || rt == 128 || rt == 256) && fits((uint32_t)rt)) row_tile = (uint32_t)rt;
-    }
-    for (auto& cb : classes) {
-      applyStages(cb, row_tile);
-      P->stage_words = std::max(P->stage_words, stageWords(cb, row_tile));
-    }
+    if (total_rows / 256 >= 512) row_tile = 256;
+    else if (total_rows / 128 >= 512) row_tile = 128;
   }
   uint32_t max_rowtiles = (uint32_t)((max_rows + row_tile - 1) / row_tile);
   uint32_t gb = 0, gc = 0, first = 0;
@@ -2058,12 +1951,6 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
     cb.cls.off_aff = (uint32_t)blob.size();
     for (auto& a : cb.affs) appendStruct(blob, a);
     while (blob.size() % 4) blob.push_back(0);
-    cb.cls.n_stages = (uint32_t)cb.stages.size();
-    cb.cls.off_stages = (uint32_t)blob.size();
-    for (auto& st : cb.stages) {
-      const uint32_t* w = (const uint32_t*)&st;
-      blob.insert(blob.end(), w, w + sizeof(FxStage) / 4);
-    }
     cb.cls.off_outs = (uint32_t)blob.size();
     for (auto& o : cb.outs) {
       const uint32_t* w = (const uint32_t*)&o;
@@ -2085,7 +1972,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
   hp->total_words = (uint32_t)blob.size();
 
   P->lds_bytes = (uint32_t)((blob.size() + 2 * (P->sptr.size() + P->tptr.size() * (size_t)T) +
-                             (P->sscal.size() + P->tscal.size() * (size_t)T) + 4 + P->stage_words +
+                             (P->sscal.size() + P->tscal.size() * (size_t)T) + 4 +
                              (size_t)max_temps * FX_V * FX_BLOCK) * 4);
   FX_CHECK(P->lds_bytes <= 64 * 1024, FX_E_LIMIT,
            "region descriptor + temporaries need " << P->lds_bytes << " bytes of LDS (limit 65536)");
@@ -2105,7 +1992,7 @@ static const char* opname(uint32_t op) {
       "INEG", "LNOT", "INZ", "FNZ", "F2I", "I2F", "IABS", "FADD", "FSUB", "FRSUB", "FMUL", "FDIV", "FRDIV", "FMIN",
       "FMAX", "FPOW", "FMOD", "ATAN2", "IADD", "ISUB", "IRSUB", "IMUL", "IFDIV", "ITDIV", "IPMOD", "ITMOD", "IMIN",
       "IMAX", "IAND", "IOR", "IXOR", "FLT", "FLE", "FGT", "FGE", "FEQ", "FNE", "ILT", "ILE", "IGT", "IGE", "IEQ",
-      "INE", "IRANGE", "WHERE", "RBEGIN", "RNEXT", "RIDX", "LDSA", "LDSB", "WMAX", "WSUM"};
+      "INE", "IRANGE", "WHERE", "RBEGIN", "RNEXT", "RIDX", "WMAX", "WSUM"};
   if (op < sizeof(names) / sizeof(names[0])) return names[op];
   return "?";
 }
@@ -2131,8 +2018,7 @@ std::string disasm(const Plan& p) {
         float fv; memcpy(&fv, &x.imm, 4);
         o << "    " << i << ": " << opname(x.op) << " a=" << x.a << " b=" << x.b << " imm=" << (int32_t)x.imm << "/" << fv
           << " fl=" << (int)x.flags << " dt=" << (int)x.dt;
-        if (x.op == FX_LDA || x.op == FX_LDB || x.op == FX_AFFA || x.op == FX_AFFB || x.op == FX_LDSA ||
-            x.op == FX_LDSB) {
+        if (x.op == FX_LDA || x.op == FX_LDB || x.op == FX_AFFA || x.op == FX_AFFB) {
           const FxAffine& a = aff[x.b];
           o << "  [";
           for (int k = 0; k < FX_MAXR; ++k) o << fx_aff_coef(&a, k) << (k + 1 < FX_MAXR ? "," : "");

@@ -79,7 +79,6 @@ struct Plan {
   uint32_t grid_count = 0;     // compaction pass 1
   uint32_t lds_bytes = 0;
   uint32_t n_temps = 0;
-  uint32_t stage_words = 0;
   int max_rank = 1;
   std::vector<PtrSrc> sptr, tptr;
   std::vector<ScalSrc> sscal, tscal;

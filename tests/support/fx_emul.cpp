@@ -73,7 +73,6 @@ float fx_fmax(float a, float b) { return (a > b || a != a) ? a : b; }
 float fx_fmin(float a, float b) { return (a < b || a != a) ? a : b; }
 
 struct Ctx {
-  const FxStage* stages;
   const FxInsn* insn;
   const FxAffine* aff;
   const uint64_t* sptr;
@@ -140,18 +139,15 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
       const int32_t ia = (int32_t)A, ib = (int32_t)(useimm ? ins.imm : B);
       switch (ins.op) {
         case FX_NOP: break;
-        case FX_LDA: case FX_LDB: case FX_AFFA: case FX_AFFB: case FX_LDSA: case FX_LDSB: {
+        case FX_LDA: case FX_LDB: case FX_AFFA: case FX_AFFB: {
           if (!M) break;
           const FxAffine& af = cx.aff[ins.b];
           int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
           for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
-          const bool staged = ins.op == FX_LDSA || ins.op == FX_LDSB;
-          const bool is_load = staged || ins.op == FX_LDA || ins.op == FX_LDB;
-          // a staged load reads the same element as the global load it replaces
-          const int32_t slot = staged ? (int32_t)cx.stages[ins.a].ptr_slot : ins.a;
-          uint32_t v = is_load ? load_elem(ptr_of(cx, slot), off, ins.dt) : (uint32_t)off;
+          const bool is_load = ins.op == FX_LDA || ins.op == FX_LDB;
+          uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt) : (uint32_t)off;
           if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
-          if (ins.op == FX_LDA || ins.op == FX_AFFA || ins.op == FX_LDSA) A = v; else B = v;
+          if (ins.op == FX_LDA || ins.op == FX_AFFA) A = v; else B = v;
         } break;
         case FX_LDXA: if (M) A = load_elem(ptr_of(cx, ins.a), (int64_t)((int32_t)A + (int32_t)ins.imm), ins.dt); break;
         case FX_IMMA: if (M) A = ins.imm; break;
@@ -270,7 +266,6 @@ extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_,
     for (uint32_t ti = 0; ti < cl.n_tasks; ++ti) {
       int task = (int)taskmap[cl.first_task + ti];
       Ctx cx;
-      cx.stages = (const FxStage*)(sb + cl.off_stages);
       cx.insn = (const FxInsn*)(sb + cl.off_insn);
       cx.aff = (const FxAffine*)(sb + cl.off_aff);
       cx.sptr = dyn->p;

@@ -2030,7 +2030,8 @@ std::string disasm(const Plan& p) {
     if (h->mode == FX_MODE_COMPACT) { o << "  mask:\n"; dump(cl.mask_begin, cl.mask_end); }
     for (uint32_t k = 0; k < cl.n_outs; ++k) {
       o << "  out " << k << ": numel=" << outs[k].numel << " rank=" << outs[k].rank << " blocks=" << outs[k].n_blocks
-        << " rowlen=" << outs[k].rowlen << "\n";
+        << " rowlen=" << outs[k].rowlen << " inner=" << outs[k].inner << " lead=" << outs[k].lead
+        << " pure=" << outs[k].pure << " unit_items=" << outs[k].unit_items << " colmajor=" << outs[k].colmajor << "\n";
       dump(outs[k].prog_begin, outs[k].prog_end);
     }
   }

@@ -240,6 +240,28 @@ def main():
                 "algorithmic_bytes": alg, "gbps_call": round(alg / (us * 1e-6) / 1e9, 1),
                 "frac_hbm_peak": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 5)}
 
+    def run_stream():
+        """Not a BASELINE config: one big fused elementwise region (sigmoid(2x + 1) on
+        [8192, 4096] fp32), the shape on which the dense kernel itself meets the HBM roofline."""
+        from functs_amd import Region
+        x = torch.rand(8192, 4096, device=dev)
+        r = Region()
+        xi = r.tensor_input(torch.float32, 2)
+        r.output((xi * 2.0 + 1.0).sigmoid())
+        bc = r.finalize().bind(x)
+        for _ in range(args.warmup):
+            bc.launch()
+        torch.cuda.synchronize()
+        acc = 0.0
+        for _ in range(args.steps):
+            acc += sum(bc.launch_timed())
+        ms = acc / args.steps
+        alg = 2 * x.numel() * 4
+        return {"workload": "fused elementwise region sigmoid(2x+1), [8192,4096] fp32", "kernel_us": [round(ms * 1e3, 2)],
+                "launches_per_call": 1, "algorithmic_bytes": alg,
+                "gbps_dominant_kernel": round(alg / (ms * 1e-3) / 1e9, 1),
+                "frac_hbm_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
     head = run_one(args.workload, True)
     per = {}
     if not args.no_per_config:
@@ -252,6 +274,10 @@ def main():
                 per[name] = r
             except Exception as e:  # a config that cannot run is reported, never faked
                 per[name] = {"error": str(e)[:200]}
+        try:
+            per["elementwise_stream"] = run_stream()
+        except Exception as e:
+            per["elementwise_stream"] = {"error": str(e)[:200]}
         try:
             per["c4"] = run_c4()
         except Exception as e:

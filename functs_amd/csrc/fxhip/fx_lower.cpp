@@ -1848,6 +1848,8 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         bool heavy = false;
         for (uint32_t pc = od.prog_begin; pc < od.prog_end; ++pc) heavy = heavy || cb.code[pc].op == FX_RBEGIN;
         od.unit_items = (!heavy && od.numel >= (8u << 20)) ? 4u : 1u;
+        // a pure tail is interpreted once per four items: worth it as soon as every CU still gets a unit
+        if (od.pure && od.numel >= (1u << 20)) od.unit_items = 4u;
         if (od.rowwave) {
           const uint32_t rows = od.rowlen ? od.numel / od.rowlen : 0;
           od.n_blocks = (rows + 4u * od.unit_items - 1) / (4u * od.unit_items);

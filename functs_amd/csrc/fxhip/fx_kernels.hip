@@ -48,13 +48,6 @@ __device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballo
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
-#ifdef FX_PHASE_PROF
-__device__ unsigned long long fx_prof_buf[1 << 16];
-#define FX_PROF(slot) do { if ((threadIdx.x & 63u) == 0 && blockIdx.x < 2048) fx_prof_buf[blockIdx.x * 32 + (slot)] = wall_clock64(); } while (0)
-#else
-#define FX_PROF(slot) do { } while (0)
-#endif
-
 struct FxCtx {
   const fx_u32x4* insn;   // LDS: class instruction base
   const uint32_t* aff;    // LDS: class affine base (FX_AFF_WORDS words each)
@@ -1009,9 +1002,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   __shared__ uint32_t s_wsum[FX_BLOCK / 64];
   __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
   __shared__ uint32_t s_prefix;
-  if (threadIdx.x == 0) FX_PROF(0);
   fx_stage(L, sb, la);
-  if (threadIdx.x == 0) FX_PROF(1);
   const FxWork w = fx_locate<false>(L, blockIdx.x);
   FxCtx cx = fx_make_ctx(L, la, w);
 
@@ -1056,7 +1047,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
     ((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])])[w.task] = prefix + n_kept;
   }
   if (n_kept == 0) return;
-  if (threadIdx.x == 0) FX_PROF(2);
 
   const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
   const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
@@ -1069,11 +1059,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
   // Half of the waves walk the outputs backwards: a latency-bound output (a long
   // predicated program on a few items) then overlaps, on the same SIMD, with the
   // arithmetic-bound wide outputs of the other waves.
-#ifdef FX_PHASE_PROF
-  const bool backwards = false;  // profiling builds time the outputs one after the other
-#else
   const bool backwards = ((blockIdx.x + wave_u) & 1u) != 0;
-#endif
   for (uint32_t oo = 0; oo < n_outs; ++oo) {
     const uint32_t oi = backwards ? n_outs - 1u - oo : oo;
     const uint32_t* od = outs + oi * ow;
@@ -1221,7 +1207,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* _
         }
       }
     }
-    FX_PROF(4 + oi * 4 + (threadIdx.x >> 6));
   }
 }
 
@@ -1445,9 +1430,3 @@ hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t gri
 }
 
 
-#ifdef FX_PHASE_PROF
-// timestamps written by FX_PROF (profiling builds only)
-extern "C" int fx_prof_read(unsigned long long* out, size_t n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(fx_prof_buf), n * sizeof(unsigned long long));
-}
-#endif

@@ -177,7 +177,9 @@ struct FxOut {
   uint32_t n_groups;              // dense: groups per task: numel / inner * gpr
   uint32_t pure;                  // after the leading load only coordinate-free elementwise instructions with
                                   // immediate operands follow: FX_K items are interpreted as one batch
-  uint32_t pad[3];
+  uint32_t rowseg;                // rowwave: lanes per row (16, 32 or 64); a wave holds 64 / rowseg rows and
+                                  // FX_WMAX / FX_WSUM reduce inside each segment of rowseg lanes
+  uint32_t pad[2];
 };
 
 

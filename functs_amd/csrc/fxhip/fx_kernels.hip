@@ -56,6 +56,7 @@ struct FxCtx {
   uint32_t tp_off;        // index of this task's first pointer
   uint32_t ts_off;        // index of this task's first scalar
   uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
+  uint32_t wseg;          // lanes per segment of the wave reductions (rows per wave = 64 / wseg)
   int task;
 };
 
@@ -551,8 +552,10 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) {
-          const float t = __shfl_xor(v, o, 64);
-          v = is_max ? fx_fmax(v, t) : v + t;
+          if ((uint32_t)o < cx.wseg) {  // wave-uniform: the butterfly stays inside a segment
+            const float t = __shfl_xor(v, o, 64);
+            v = is_max ? fx_fmax(v, t) : v + t;
+          }
         }
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) A[j] = f2u(v);
@@ -778,6 +781,7 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
   cx.tp_off = n_sptr + (uint32_t)w.task * n_tptr;
   cx.ts_off = n_sscal + (uint32_t)w.task * n_tscal;
   cx.temps = L + la.temps_off + threadIdx.x;
+  cx.wseg = 64;
   cx.task = w.task;
   return cx;
 }
@@ -800,7 +804,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
   // consecutive items of FX_ITEM elements.
   for (uint32_t unit = blockIdx.x; unit < la.total_units; unit += gridDim.x) {
     const FxWork w = fx_locate<false>(L, unit);
-    const FxCtx cx = fx_make_ctx(L, la, w);
+    FxCtx cx = fx_make_ctx(L, la, w);
     const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
     const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
     uint32_t oi = 0;
@@ -835,16 +839,24 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __re
     const uint32_t gp_magic = od[FX_W(FxOut, gp_magic)], gp_shift = od[FX_W(FxOut, gp_shift)];
     const uint32_t n_groups = uni(od[FX_W(FxOut, n_groups)]);
     const uint32_t item0 = ublock * (4u * kmax) + wave * kmax;
-    const uint32_t n_items = rowwave ? numel / inner : (n_groups + 63u) / 64u;
+    const uint32_t rowseg = rowwave ? uni(od[FX_W(FxOut, rowseg)]) : 64u;
+    const uint32_t segsh = 31u - (uint32_t)__builtin_clz(rowseg);
+    const uint32_t rows_per_item = 64u >> segsh;
+    cx.wseg = rowseg;
+    const uint32_t n_rows_w = numel / inner;
+    const uint32_t n_items = rowwave ? (n_rows_w + rows_per_item - 1) / rows_per_item : (n_groups + 63u) / 64u;
     if (item0 >= n_items) continue;
 
     auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) {
       uint32_t row, col0;
       bool live;
       if (rowwave) {
-        row = item0 + k;
-        col0 = lane * FX_V;
-        live = true;
+        // 64 / rowseg rows per wave, one per segment of rowseg lanes
+        const uint32_t seg = lane >> segsh;
+        row = (item0 + k) * rows_per_item + seg;
+        col0 = (lane - seg * rowseg) * FX_V;
+        live = row < n_rows_w;
+        if (!live) row = 0;
       } else {
         const uint32_t g = (item0 + k) * 64u + lane;
         live = g < n_groups;

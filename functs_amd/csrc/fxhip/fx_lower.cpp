@@ -1786,6 +1786,8 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       if (p.rowwave) {
         od.rowwave = 1;
         od.rowlen = (uint32_t)s.back();
+        const uint32_t lanes = (od.rowlen + FX_V - 1) / FX_V;
+        od.rowseg = lanes <= 16 ? 16u : (lanes <= 32 ? 32u : 64u);
       }
       {
         // leading load: unconditional, affine, not inside a reduction loop
@@ -1852,7 +1854,9 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
         if (od.pure && od.numel >= (1u << 20)) od.unit_items = 4u;
         if (od.rowwave) {
           const uint32_t rows = od.rowlen ? od.numel / od.rowlen : 0;
-          od.n_blocks = (rows + 4u * od.unit_items - 1) / (4u * od.unit_items);
+          const uint32_t rows_per_item = 64u / od.rowseg;
+          const uint32_t items = (rows + rows_per_item - 1) / rows_per_item;
+          od.n_blocks = (items + 4u * od.unit_items - 1) / (4u * od.unit_items);
           od.lead = 0;
         } else {
           const uint32_t unit = 4u * od.unit_items * (FX_ITEM / FX_V);  // groups per work unit

@@ -539,6 +539,10 @@ void Translator::node(const Node* n) {
   auto out = [&](int id) { ids[n->output(0)] = id; };
   const size_t ni = n->inputs().size();
   if (k == prim::Constant) return;  // created on demand
+  if (k == aten::size && ni == 1) {  // all sizes: the tensor itself stands for them
+    out(in(0));
+    return;
+  }
   if (k == prim::ListConstruct) {
     std::vector<int> e;
     for (const Value* v : n->inputs()) e.push_back(get(v));
@@ -568,7 +572,7 @@ void Translator::node(const Node* n) {
     if (k == aten::sub) { out(op(FX_OP_INT_SUB, {in(0), in(1)})); return; }
     if (k == aten::mul) { out(op(FX_OP_INT_MUL, {in(0), in(1)})); return; }
     if (k == aten::neg) { out(op(FX_OP_INT_NEG, {in(0)})); return; }
-    if (k == aten::size) { out(op(FX_OP_SIZE, {in(0), in(1)})); return; }
+    if (k == aten::size && ni == 2) { out(op(FX_OP_SIZE, {in(0), in(1)})); return; }
     if (k == aten::__derive_index) {  // start + index * step
       out(op(FX_OP_INT_ADD, {in(1), op(FX_OP_INT_MUL, {in(0), in(2)})}));
       return;

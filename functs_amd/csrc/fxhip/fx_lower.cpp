@@ -389,6 +389,7 @@ int64_t Lowerer::constIntOf(int vid, const char* what) {
 
 std::vector<int64_t> Lowerer::intListOf(int vid, const char* what) {
   const Value& v = V(vid);
+  if (v.kind == VK_TENSOR) return shapeOf(vid);  // a tensor where sizes are expected: its sizes (aten::size(t))
   FX_CHECK(v.kind == VK_INT_LIST, FX_E_INVALID, what << ": expected int[]");
   std::vector<int64_t> r;
   for (int a : v.args) r.push_back(constIntOf(a, what));

@@ -138,6 +138,8 @@ int fx_region_const_int(fx_region*, int64_t v, int* id);
 int fx_region_const_float(fx_region*, double v, int* id);
 int fx_region_const_bool(fx_region*, int v, int* id);
 int fx_region_const_none(fx_region*, int* id);
+/* Wherever an operator takes an int[] of sizes (view, expand, full), the id of a tensor
+ * value may be passed instead and stands for that tensor's sizes (aten::size(t)). */
 int fx_region_int_list(fx_region*, const int* ids, int n, int* id);
 int fx_region_tensor_list(fx_region*, const int* ids, int n, int* id);
 /* out_dtype < 0: infer by type promotion */

@@ -231,9 +231,24 @@ def main():
         from oracle import configs as oc
         cpu_args = oc.c4_inputs(0)
         us, n_functors = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
+        # the same call replayed as one HIP graph (functs_amd.jit.build(..., hip_graph=True))
+        import functs_amd.jit as fj
+        from functs_amd.benchmark import PROGRAMS
+        gfn = fj.build(fj.script(PROGRAMS["c4"]), list(cpu_args), hip_graph=True)
+        gargs = [a.to(dev) for a in cpu_args]
+        for _ in range(3):
+            gfn(*gargs)
+        torch.cuda.synchronize()
+        n_rep = max(args.steps // 10, 5)
+        t0 = time.perf_counter()
+        for _ in range(n_rep):
+            gfn(*gargs)
+        torch.cuda.synchronize()
+        graph_us = (time.perf_counter() - t0) * 1e6 / n_rep
         seq_len, layers = cpu_args[0].size(0), cpu_args[1].size(0)
         alg = 17072128  # weights + biases + x + out, each once
         return {"workload": "c4 stacked LSTM 2x512, T=64, B=1", "torchscript_route_latency_us": round(us, 1),
+                "hip_graph_latency_us": round(graph_us, 1),
                 "torchscript_route_functors": n_functors,
                 "launches_per_call": 1 + seq_len * (layers * 3 + 2),
                 "fused_region_launches_per_call": 1 + seq_len * layers,

@@ -67,9 +67,78 @@ def _strip_self(g):
         g.eraseInput(0)
 
 
-def build(fn, example_input: List[object]) -> AotScriptFunction:
+class GraphedFunction(AotScriptFunction):
+    """A built function whose whole call is one HIP graph: for programs whose loops
+    stay host loops (carried state, e.g. an LSTM) the per-launch host work of
+    hundreds of small kernels is paid once, at capture.
+
+    The first call with a given set of tensor shapes runs the function twice on a
+    side stream (variants get compiled, workspaces allocated), then captures it with
+    private input buffers; later calls copy the arguments into those buffers, replay
+    and return clones of the captured outputs.  Non-tensor arguments are baked into
+    the capture, so they are part of the key.  A function with a row-compacting
+    region cannot be captured: its output shapes need a synchronisation per call.
+    """
+
+    def __init__(self, aot_script_fn):
+        super().__init__(aot_script_fn)
+        if "compact_rows=1" in str(aot_script_fn.graph):
+            raise ValueError("a function with a row-compacting region cannot run as a HIP graph")
+        self._captures = {}
+
+    @staticmethod
+    def _key(args):
+        k = []
+        for a in args:
+            if isinstance(a, torch.Tensor):
+                k.append((tuple(a.shape), a.dtype, a.device))
+            elif isinstance(a, (list, tuple)) and a and isinstance(a[0], torch.Tensor):
+                k.append(tuple((tuple(t.shape), t.dtype, t.device) for t in a))
+            else:
+                k.append(repr(a))
+        return tuple(k)
+
+    @staticmethod
+    def _map(x, f):
+        if isinstance(x, torch.Tensor):
+            return f(x)
+        if isinstance(x, (list, tuple)):
+            return type(x)(GraphedFunction._map(e, f) for e in x)
+        return x
+
+    def __call__(self, *args):
+        key = self._key(args)
+        cap = self._captures.get(key)
+        if cap is None:
+            static = [self._map(a, lambda t: t.clone()) for a in args]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    self._aot_script_fn(*static)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = self._aot_script_fn(*static)
+            cap = self._captures[key] = (graph, static, out)
+        graph, static, out = cap
+
+        def refill(dst, src):
+            if isinstance(dst, torch.Tensor):
+                dst.copy_(src)
+            elif isinstance(dst, (list, tuple)):
+                for d, s_ in zip(dst, src):
+                    refill(d, s_)
+
+        for d, a in zip(static, args):
+            refill(d, a)
+        graph.replay()
+        return self._map(out, lambda t: t.clone())
+
+
+def build(fn, example_input: List[object], hip_graph: bool = False) -> AotScriptFunction:
     """Form fused regions in a functionalized script and return the callable
-    (functs/jit/_script.py:58-73)."""
+    (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
         raise AttributeError("only a functionalized jit script can be built")
     g = fn.graph.copy()
@@ -77,7 +146,8 @@ def build(fn, example_input: List[object]) -> AotScriptFunction:
         _strip_self(g)
     hints = [extract_type_hint_from_tensor(i) for i in example_input]
     _C._jit_pass_fait_pipeline(g, hints)
-    return AotScriptFunction(_C._create_function_from_graph("forward", g))
+    aot = _C._create_function_from_graph("forward", g)
+    return GraphedFunction(aot) if hip_graph else AotScriptFunction(aot)
 
 
 def script(fn, backend="jit", remove_update=True, enable_dce_cse=True, add_clone=False):

@@ -233,3 +233,32 @@ def test_c4_lstm_torchscript_gpu(seq_len, hidden):
     # 1e-5 per step compounds over the recurrence: 1e-4 at the last step (matmul runs in rocBLAS)
     for name, g_, r in zip(("out", "state_h", "state_c"), got, ref):
         assert_close(g_.cpu(), r, "c4 " + name, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_c4_lstm_as_hip_graph():
+    """Every replay is checked against the eager call, with other work and
+    synchronisations of the program in between, and with fresh input values."""
+    from functs_amd.benchmark import PROGRAMS
+    args0 = oc.c4_inputs(0, 12, 64, 2, 1)
+    f = fj.script(PROGRAMS["c4"])
+    eager = fj.build(f, list(args0))
+    graphed = fj.build(f, list(args0), hip_graph=True)
+    for seed in (0, 1, 2, 1):
+        args = _cuda(oc.c4_inputs(seed, 12, 64, 2, 1))
+        want = eager(*args)
+        torch.cuda.synchronize()
+        got = graphed(*args)
+        junk = torch.rand(4096, device="cuda").sum().item()  # unrelated work between replays
+        assert junk > 0
+        for g_, w in zip(got, want):
+            assert torch.equal(g_, w)
+    ref = oc.run("c4", *oc.c4_inputs(1, 12, 64, 2, 1))
+    for g_, r in zip(got, ref):
+        assert_close(g_.cpu(), r, "graphed c4", rtol=1e-4, atol=1e-6)
+
+
+def test_hip_graph_refuses_row_compaction():
+    args = oc.c2_inputs(0, SMALL_GRIDS)
+    with pytest.raises(ValueError, match="row-compacting"):
+        fj.build(fj.script(oc.c2_fn), list(args), hip_graph=True)

@@ -64,13 +64,15 @@ enum FxOp : uint32_t {
   FX_MELSE,  // mask = saved & ~mask; if no lane live jump to a
   FX_MMERGE, // A = live ? A : temp[a]; pop mask
   FX_MEND,   // pop mask (both sides wrote A with predicated moves)
+  FX_MIFR,   // x = (int) affine[b](coords); A = (0 <= x < imm >> 8 && x % (imm & 255) == 0); then as MIF
   // ---- unary float (A = f(A)) ----
   FX_FNEG, FX_FABS, FX_EXP, FX_LOG, FX_SQRT, FX_RSQRT, FX_RCP, FX_SIGMOID,
   FX_TANH, FX_RELU, FX_FLOOR, FX_CEIL, FX_ROUND, FX_TRUNC, FX_SIN, FX_COS,
   FX_ERF, FX_LOG2, FX_EXP2, FX_EXPM1, FX_LOG1P,
   // ---- unary int / conversions ----
   FX_INEG, FX_LNOT, FX_INZ, FX_FNZ, FX_F2I, FX_I2F, FX_IABS,
-  // ---- binary: A = A op X, X = B or imm (flags & FX_F_IMM) ----
+  // ---- binary: A = A op X, X = B or imm (flags & FX_F_IMM).  With FX_F_MEMB / FX_F_TMPB the
+  //      instruction first loads B like LDB (fields a, b, dt) / LDTB (field a) ----
   FX_FADD, FX_FSUB, FX_FRSUB, FX_FMUL, FX_FDIV, FX_FRDIV, FX_FMIN, FX_FMAX,
   FX_FPOW, FX_FMOD, FX_ATAN2,
   FX_IADD, FX_ISUB, FX_IRSUB, FX_IMUL, FX_IFDIV, FX_ITDIV, FX_IPMOD, FX_ITMOD,
@@ -110,6 +112,9 @@ static inline bool fx_op_is_pure_binary(uint32_t op) {
 
 #define FX_F_IMM 1u  // binary op takes its second operand from imm
 #define FX_F_I2F 2u  // LDA/LDB/AFFA/AFFB/SCLA/SCLB: convert the int result to float
+#define FX_F_MEMB 4u // before the operation: B = buf[a] at affine[b](coords), dt = storage dtype (always set on LDB)
+#define FX_F_TMPB 8u // before the operation: B = temp[a] (always set on LDTB)
+static inline bool fx_op_is_binary(uint32_t op) { return op >= FX_FADD && op <= FX_INE; }
 
 struct FxInsn {
   uint16_t op;

@@ -300,6 +300,24 @@ __device__ __forceinline__ void fx_store_vec(uint64_t base_, uint32_t obase, con
   }
 }
 
+// Element offsets of affine record `idx` at the FX_V elements of a lane group.
+template <int R>
+__device__ __forceinline__ bool fx_affine(const FxCtx& cx, const FxCoord<R>& q, int32_t idx, int32_t lc0, int32_t lc1,
+                                          int32_t (&off)[FX_V]) {
+  const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + idx * FX_AFF_WORDS);
+  const fx_u32x4 a0 = ap[0], a1 = ap[1];
+  int32_t cf[FX_MAXR];
+  cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
+  if (R > 4) {
+    const fx_u32x4 a2 = ap[2];
+    cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
+  } else {
+    cf[4] = 0; cf[5] = 0;
+  }
+  const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
+  return fx_offsets<R>(q, cf, base, off);
+}
+
 // The interpreter.  R = number of root coordinates that carry information.
 // The program lives in LDS; the next instruction word is fetched while the
 // current one executes.  The host pads every program area with one trailing
@@ -371,29 +389,28 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
     }                                                      \
   } break
 
+    // second operand fetched as part of the instruction (LDB, LDTB and binary operations that
+    // took such a load over)
+    if (w0 & ((FX_F_MEMB | FX_F_TMPB) << 16)) {
+      if (w0 & (FX_F_TMPB << 16)) {
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) B[j] = cx.temps[(ia * FX_V + j) * FX_BLOCK];
+      } else {
+        int32_t off[FX_V];
+        const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
+        fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B);
+      }
+    }
+
     switch (op) {
       case FX_NOP: break;
       case FX_LDA:
-      case FX_LDB:
       case FX_AFFA:
       case FX_AFFB: {
-        const fx_u32x4* ap = (const fx_u32x4*)(cx.aff + ib * FX_AFF_WORDS);
-        const fx_u32x4 a0 = ap[0], a1 = ap[1];
-        int32_t cf[FX_MAXR];
-        cf[0] = (int32_t)a0.x; cf[1] = (int32_t)a0.y; cf[2] = (int32_t)a0.z; cf[3] = (int32_t)a0.w;
-        if (R > 4) {
-          const fx_u32x4 a2 = ap[2];
-          cf[4] = (int32_t)a2.x; cf[5] = (int32_t)a2.y;
-        } else {
-          cf[4] = 0; cf[5] = 0;
-        }
-        const int32_t base = (int32_t)a1.y + (int32_t)a1.x * cx.task + (int32_t)a1.z * lc0 + (int32_t)a1.w * lc1;
         int32_t off[FX_V];
-        const bool consecutive = fx_offsets<R>(q, cf, base, off);
+        const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
         if (op == FX_LDA) {
           fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, A);
-        } else if (op == FX_LDB) {
-          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B);
         } else {
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
@@ -402,6 +419,9 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
           }
         }
       } break;
+      case FX_LDB:   // done above: FX_F_MEMB / FX_F_TMPB are always set on these two
+      case FX_LDTB:
+        break;
       case FX_LDXA: {
         int32_t off[FX_V];
 #pragma unroll
@@ -436,10 +456,6 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) if ((M >> j) & 1u) A[j] = cx.temps[(ia * FX_V + j) * FX_BLOCK];
         break;
-      case FX_LDTB:
-#pragma unroll
-        for (int j = 0; j < FX_V; ++j) B[j] = cx.temps[(ia * FX_V + j) * FX_BLOCK];
-        break;
       case FX_MOVBA:
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) B[j] = A[j];
@@ -454,6 +470,23 @@ __device__ __forceinline__ void fx_run(const FxCtx& cx, int pc, const int pc_end
         uint32_t cnd = 0;
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) cnd |= (A[j] != 0u ? 1u : 0u) << j;
+        M &= cnd;
+        if (!wave_any(M != 0u)) FX_JUMP(ia)
+      } break;
+      case FX_MIFR: {
+        int32_t off[FX_V];
+        fx_affine<R>(cx, q, ib, lc0, lc1, off);
+        const uint32_t hi = uni(imm) >> 8;
+        const int32_t st = (int32_t)(uni(imm) & 255u);
+        MS = (MS << FX_V) | (uint64_t)M;
+        uint32_t cnd = 0;
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          bool in = (uint32_t)off[j] < hi;
+          if (st > 1) in = in && ((off[j] % st) == 0);
+          A[j] = in ? 1u : 0u;
+          cnd |= (in ? 1u : 0u) << j;
+        }
         M &= cnd;
         if (!wave_any(M != 0u)) FX_JUMP(ia)
       } break;
@@ -822,7 +855,7 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
 // dense region kernel
 // --------------------------------------------------------------------------
 template <int R>
-__global__ __launch_bounds__(FX_BLOCK) void fx_region_dense(const uint32_t* __restrict__ sb, const FxLaunch la,
+__global__ __launch_bounds__(FX_BLOCK, 4) void fx_region_dense(const uint32_t* __restrict__ sb, const FxLaunch la,
                                                             const FxDyn) {
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];
   fx_stage(L, sb, la);   // once per workgroup; the loop below has no barrier
@@ -1037,7 +1070,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
 // The last tile of a task also publishes the task's total.
 // --------------------------------------------------------------------------
 template <int R>
-__global__ __launch_bounds__(FX_BLOCK) void fx_compact_scatter(const uint32_t* __restrict__ sb, const FxLaunch la,
+__global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t* __restrict__ sb, const FxLaunch la,
                                                                const FxDyn) {
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];
   __shared__ uint32_t s_rowmap[FX_BLOCK];

@@ -277,6 +277,16 @@ class Lowerer {
 
   // ---- emission helpers ----
   int emitI(uint16_t op, int32_t a = 0, int32_t b = 0, uint32_t imm = 0, uint8_t flags = 0, uint8_t dt = 0) {
+    if (op == FX_LDB) flags |= FX_F_MEMB;
+    if (op == FX_LDTB) flags |= FX_F_TMPB;
+    // A binary operation that follows the load of its B operand takes the load over: one
+    // instruction instead of two.  No jump can land between the two: targets are MELSE, MMERGE
+    // and loop boundaries, none of which is a binary operation.
+    if (fx_op_is_binary(op) && !(flags & FX_F_IMM) && !code.empty() &&
+        (code.back().op == FX_LDB || code.back().op == FX_LDTB)) {
+      code.back().op = op;
+      return (int)code.size() - 1;
+    }
     FxInsn i; i.op = op; i.flags = flags; i.dt = dt; i.a = a; i.b = b; i.imm = imm;
     code.push_back(i);
     return (int)code.size() - 1;
@@ -1160,11 +1170,21 @@ void Lowerer::emitBinary(uint16_t op, const Operand& l, const Operand& r, uint32
 void Lowerer::emitCond(const IdxExpr& x, int64_t lo, int64_t hi, int64_t step, const std::function<void()>& thenFn,
                        const std::function<void()>& elseFn) {
   FX_CHECK(maskDepth_ + 1 <= FX_MASK_DEPTH, FX_E_LIMIT, "predicated regions nested deeper than " << FX_MASK_DEPTH);
+  const size_t before = code.size();
   emitIdx(x);
   auto fit = [](int64_t v) { return (int32_t)std::min<int64_t>(std::max<int64_t>(v, std::numeric_limits<int32_t>::min()), std::numeric_limits<int32_t>::max()); };
-  emitI(FX_IRANGE, fit(lo), fit(hi), (uint32_t)(int32_t)step);
   ++maskDepth_;
-  int mif = emitI(FX_MIF);
+  int mif;
+  if (code.size() == before + 1 && code.back().op == FX_AFFA && code.back().flags == 0 && lo == 0 && hi > 0 &&
+      hi < (1 << 24) && step >= 1 && step < 256) {
+    // the index is one affine function of the coordinates: test and predicate in one instruction
+    const int32_t aff = code.back().b;
+    code.pop_back();
+    mif = emitI(FX_MIFR, 0, aff, ((uint32_t)hi << 8) | (uint32_t)step);
+  } else {
+    emitI(FX_IRANGE, fit(lo), fit(hi), (uint32_t)(int32_t)step);
+    mif = emitI(FX_MIF);
+  }
   thenFn();
   int t = allocTemp();
   emitI(FX_STT, t);
@@ -1994,7 +2014,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
 static const char* opname(uint32_t op) {
   static const char* names[] = {
       "NOP", "LDA", "LDB", "LDXA", "AFFA", "AFFB", "IMMA", "IMMB", "SCLA", "SCLB", "STT", "LDTA", "LDTB", "MOVBA",
-      "SWAP", "MIF", "MELSE", "MMERGE", "MEND", "FNEG", "FABS", "EXP", "LOG", "SQRT", "RSQRT", "RCP", "SIGMOID",
+      "SWAP", "MIF", "MELSE", "MMERGE", "MEND", "MIFR", "FNEG", "FABS", "EXP", "LOG", "SQRT", "RSQRT", "RCP", "SIGMOID",
       "TANH", "RELU", "FLOOR", "CEIL", "ROUND", "TRUNC", "SIN", "COS", "ERF", "LOG2", "EXP2", "EXPM1", "LOG1P",
       "INEG", "LNOT", "INZ", "FNZ", "F2I", "I2F", "IABS", "FADD", "FSUB", "FRSUB", "FMUL", "FDIV", "FRDIV", "FMIN",
       "FMAX", "FPOW", "FMOD", "ATAN2", "IADD", "ISUB", "IRSUB", "IMUL", "IFDIV", "ITDIV", "IPMOD", "ITMOD", "IMIN",
@@ -2025,7 +2045,7 @@ std::string disasm(const Plan& p) {
         float fv; memcpy(&fv, &x.imm, 4);
         o << "    " << i << ": " << opname(x.op) << " a=" << x.a << " b=" << x.b << " imm=" << (int32_t)x.imm << "/" << fv
           << " fl=" << (int)x.flags << " dt=" << (int)x.dt;
-        if (x.op == FX_LDA || x.op == FX_LDB || x.op == FX_AFFA || x.op == FX_AFFB) {
+        if (x.op == FX_LDA || x.op == FX_AFFA || x.op == FX_AFFB || x.op == FX_MIFR || (x.flags & FX_F_MEMB)) {
           const FxAffine& a = aff[x.b];
           o << "  [";
           for (int k = 0; k < FX_MAXR; ++k) o << fx_aff_coef(&a, k) << (k + 1 < FX_MAXR ? "," : "");

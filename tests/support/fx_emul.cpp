@@ -116,6 +116,25 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
       if (!any_live()) pc = ins.a;
       continue;
     }
+    auto affine_at = [&](const Lane& l, int idx) {
+      const FxAffine& af = cx.aff[idx];
+      int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
+      for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * l.c[k];
+      return off;
+    };
+    if (ins.op == FX_MIFR) {
+      const uint32_t hi = ins.imm >> 8;
+      const int32_t st = (int32_t)(ins.imm & 255u);
+      for (auto& l : L) {
+        const int32_t x = affine_at(l, ins.b);
+        const bool in = (uint32_t)x < hi && (st <= 1 || x % st == 0);
+        l.A = in ? 1u : 0u;
+        l.stack.push_back(l.M);
+        l.M = l.M && in;
+      }
+      if (!any_live()) pc = ins.a;
+      continue;
+    }
     if (ins.op == FX_MELSE) {
       for (auto& l : L) l.M = l.stack.back() && !l.M;
       if (!any_live()) pc = ins.a;
@@ -135,16 +154,20 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
       const bool M = l.M;
       uint32_t* temps = l.temps;
       const int32_t* c = l.c;
+      if (ins.flags & FX_F_TMPB) B = temps[ins.a];
+      else if ((ins.flags & FX_F_MEMB) && M) {
+        B = load_elem(ptr_of(cx, ins.a), affine_at(l, ins.b), ins.dt);
+        if (ins.flags & FX_F_I2F) B = f2u((float)(int32_t)B);
+      }
       const float fa = u2f(A), fb = u2f(useimm ? ins.imm : B);
       const int32_t ia = (int32_t)A, ib = (int32_t)(useimm ? ins.imm : B);
       switch (ins.op) {
         case FX_NOP: break;
-        case FX_LDA: case FX_LDB: case FX_AFFA: case FX_AFFB: {
+        case FX_LDB: case FX_LDTB: break;  // the operand fetch above did it
+        case FX_LDA: case FX_AFFA: case FX_AFFB: {
           if (!M) break;
-          const FxAffine& af = cx.aff[ins.b];
-          int32_t off = af.base + af.tcoef * cx.task + af.rcoef[0] * lc[0] + af.rcoef[1] * lc[1];
-          for (int k = 0; k < FX_MAXR; ++k) off += fx_aff_coef(&af, k) * c[k];
-          const bool is_load = ins.op == FX_LDA || ins.op == FX_LDB;
+          const int32_t off = affine_at(l, ins.b);
+          const bool is_load = ins.op == FX_LDA;
           uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt) : (uint32_t)off;
           if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
           if (ins.op == FX_LDA || ins.op == FX_AFFA) A = v; else B = v;
@@ -156,7 +179,6 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
         case FX_SCLB: B = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) B = f2u((float)(int32_t)B); break;
         case FX_STT: temps[ins.a] = A; break;
         case FX_LDTA: if (M) A = temps[ins.a]; break;
-        case FX_LDTB: B = temps[ins.a]; break;
         case FX_MOVBA: B = A; break;
         case FX_SWAP: { uint32_t t = A; A = B; B = t; } break;
         case FX_MMERGE: A = M ? A : temps[ins.a]; l.M = l.stack.back(); l.stack.pop_back(); break;

@@ -29,30 +29,27 @@ HBM_PEAK_GBPS = 8000.0
 def build_workload(name, dev):
     import torch
     from functs_amd import configs
-    from oracle import configs as oc
+    from functs_amd.benchmark.inputs import INPUTS
 
     def G(*xs):
         return [x.to(dev) if isinstance(x, torch.Tensor) else x for x in xs]
 
+    if name not in ("c1", "c2", "c3", "c5"):
+        raise SystemExit("unknown workload %s" % name)
+    cpu_args = INPUTS[name](0)
     if name == "c1":
-        a, b, n = oc.c1_inputs(0)
-        cpu_args = (a, b, n)
+        a, b, n = cpu_args
         calls = [(configs.build_c1(), G(b, n))]
         desc = "c1 get_started loop [1024,1024] n=1024"
     elif name == "c2":
-        cpu_args = oc.c2_inputs(0)
         calls = [(configs.build_c2(), G(*cpu_args))]
         desc = "c2 YOLOv3-style post-proc [1,10647,85]"
     elif name == "c5":
-        cpu_args = oc.c5_inputs(0)
         calls = [(configs.build_c5(16), G(*cpu_args))]
         desc = "c5 ParallelMap x16 YOLOv3-style post-proc [16,10647,85]"
     elif name == "c3":
-        cpu_args = oc.c3_inputs(0)
         calls = [(configs.build_c3_decode(), G(*cpu_args)), (configs.build_c3_classes(80), None)]
         desc = "c3 SSD300-style post-proc [1,8732,4]+[1,8732,81]"
-    else:
-        raise SystemExit("unknown workload %s" % name)
     return desc, calls, cpu_args
 
 
@@ -142,23 +139,28 @@ def torchscript_route(name, cpu_args, dev, steps, warmup):
     import torch
     import functs_amd.jit as fj
     from functs_amd.benchmark import PROGRAMS
+    import functs_amd.aot as aot
     fn = fj.build(fj.script(PROGRAMS[name]), list(cpu_args))
     args = [a.to(dev) if isinstance(a, torch.Tensor) else a for a in cpu_args]
     for _ in range(warmup):
         fn(*args)
     torch.cuda.synchronize()
+    l0, s0 = aot.launch_stats()
     t0 = time.perf_counter()
     for _ in range(steps):
         fn(*args)
     torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / steps
+    l1, s1 = aot.launch_stats()
     n_functors = str(fn.graph).count("= tssa::ParallelFunctor")
-    return (time.perf_counter() - t0) * 1e6 / steps, n_functors
+    return us, n_functors, (s1 - s0) / max(l1 - l0, 1)
 
 
-def cpu_baseline(name, cpu_args, budget_s):
+def cpu_baseline(name, budget_s):
     import torch
     from oracle import configs as oc
     fn = oc.scripted(name)
+    cpu_args = getattr(oc, name + "_inputs")(0)
     for _ in range(2):
         fn(*cpu_args)
     n, t0 = 0, time.perf_counter()
@@ -179,6 +181,8 @@ def main():
     ap.add_argument("--workload", default="c5")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-per-config", action="store_true")
+    ap.add_argument("--interpreter", action="store_true",
+                    help="run every region with the bytecode interpreter (no ahead-of-time compiled kernels)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch the library's plain copy kernel on BYTES (3 times): the known-size reference "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -190,6 +194,9 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs an MI355X (no CPU fallback exists)")
     dev = torch.device("cuda:0")
+    import functs_amd.aot as aot
+    if args.interpreter:
+        aot.enable(False)
 
     def run_one(name, with_cpu):
         w = Workload(name, dev)
@@ -206,11 +213,19 @@ def main():
             "gbps_all_kernels": round(alg / (sum(kern) * 1e-3) / 1e9, 1),
             "frac_hbm_peak": round(alg / (dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         }
-        ts_us, n_functors = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup)
+        rec["compiled_kernels"] = all(bc.region.specialized(*bc.args) for bc in w.bound)
+        if rec["compiled_kernels"]:
+            # the same launches through the bytecode interpreter
+            aot.enable(False)
+            _, ikern = measure(w, max(args.steps // 4, 5), 3)
+            aot.enable(True)
+            rec["interpreter_kernel_us"] = [round(k * 1e3, 2) for k in ikern]
+        ts_us, n_functors, spec_share = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup)
         rec["torchscript_route_latency_us"] = round(ts_us, 2)
         rec["torchscript_route_functors"] = n_functors
+        rec["torchscript_route_compiled_share"] = round(spec_share, 3)
         if with_cpu:
-            us, n, cores = cpu_baseline(name, w.cpu_args, args.cpu_seconds)
+            us, n, cores = cpu_baseline(name, args.cpu_seconds)
             rec["cpu"] = (us, n, cores)
         return rec
 
@@ -228,9 +243,9 @@ def main():
         """The stacked LSTM has carried state, so its loops stay host loops: per (step, layer)
         two rocBLAS matmuls and one fused region (gates + both state writes), per step one
         select_rev of `out`.  Only the TorchScript route exists for it."""
-        from oracle import configs as oc
-        cpu_args = oc.c4_inputs(0)
-        us, n_functors = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
+        from functs_amd.benchmark.inputs import INPUTS
+        cpu_args = INPUTS["c4"](0)
+        us, n_functors, spec_share = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
         # the same call replayed as one HIP graph (functs_amd.jit.build(..., hip_graph=True))
         import functs_amd.jit as fj
         from functs_amd.benchmark import PROGRAMS
@@ -249,7 +264,7 @@ def main():
         alg = 17072128  # weights + biases + x + out, each once
         return {"workload": "c4 stacked LSTM 2x512, T=64, B=1", "torchscript_route_latency_us": round(us, 1),
                 "hip_graph_latency_us": round(graph_us, 1),
-                "torchscript_route_functors": n_functors,
+                "torchscript_route_functors": n_functors, "torchscript_route_compiled_share": round(spec_share, 3),
                 "launches_per_call": 1 + seq_len * (layers * 3 + 2),
                 "fused_region_launches_per_call": 1 + seq_len * layers,
                 "algorithmic_bytes": alg, "gbps_call": round(alg / (us * 1e-6) / 1e9, 1),
@@ -264,6 +279,7 @@ def main():
         xi = r.tensor_input(torch.float32, 2)
         r.output((xi * 2.0 + 1.0).sigmoid())
         bc = r.finalize().bind(x)
+        compiled = bc.region.specialized(x)
         for _ in range(args.warmup):
             bc.launch()
         torch.cuda.synchronize()
@@ -273,6 +289,7 @@ def main():
         ms = acc / args.steps
         alg = 2 * x.numel() * 4
         return {"workload": "fused elementwise region sigmoid(2x+1), [8192,4096] fp32", "kernel_us": [round(ms * 1e3, 2)],
+                "compiled_kernels": compiled,
                 "launches_per_call": 1, "algorithmic_bytes": alg,
                 "gbps_dominant_kernel": round(alg / (ms * 1e-3) / 1e9, 1),
                 "frac_hbm_peak": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
@@ -315,6 +332,7 @@ def main():
         "data": "synthetic (torch.manual_seed(0), CPU generator, copied to HBM)",
         "config": {"workload": head["workload"],
                    "route": "functs_amd.jit.script -> build -> tssa::ParallelFunctor (C++ operator over the C ABI)",
+                   "compiled_kernels": head["compiled_kernels"] and not args.interpreter,
                    "region_api_latency_us": head["latency_us"], "launches_per_call": head["launches_per_call"],
                    "kernel_us": head["kernel_us"], "gbps_all_kernels": head["gbps_all_kernels"]},
         "roofline": {"bound": "hbm", "achieved": head["gbps_dominant_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",

@@ -114,6 +114,13 @@ _sig("fx_plan_launches", _i, _vp)
 _sig("fx_plan_algorithmic_bytes", ctypes.c_int64, _vp)
 _sig("fx_plan_blob", _i, _vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)), ctypes.POINTER(ctypes.c_size_t))
 _sig("fx_plan_disasm", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_plan_spec_key", ctypes.c_uint64, _vp)
+_sig("fx_plan_specialized", _i, _vp)
+_sig("fx_plan_spec_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_set_specialization", None, _i)
+_sig("fx_specialization_count", _i)
+_sig("fx_spec_dump_dir", _i, ctypes.c_char_p)
+_sig("fx_launch_stats", None, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64))
 _sig("fx_region_marshal", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,
      ctypes.c_size_t)
 _sig("fx_dyn_bytes", ctypes.c_size_t)

@@ -7,18 +7,24 @@
 // (fait/tensorexpr/cuda_codegen_tssa.cpp:1167-1290).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
 
 #include "fx_lower.h"
 
+struct FxSpecKernels;
+const FxSpecKernels* fx_spec_find(uint64_t hash);
+int fx_spec_count();
 hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
-                           hipStream_t stream);
+                           hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
-                                   hipStream_t stream);
+                                   hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
-                                     uint32_t grid, hipStream_t stream);
+                                     uint32_t grid, hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream);
 hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                   const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
@@ -208,17 +214,89 @@ int fx_region_finalize(fx_region* reg) {
   return FX_OK;
 }
 
+// ---- specialised kernels ----
+static std::atomic<int> g_specialize{[] {
+  const char* e = getenv("FXHIP_SPECIALIZE");
+  return (e && e[0] == '0') ? 0 : 1;
+}()};
+static std::mutex g_dump_mu;
+static std::string g_dump_dir;
+
+static std::atomic<uint64_t> g_launches{0}, g_spec_launches{0};
+
+static const FxSpecKernels* spec_of(const fx::Plan* p) {
+  if (!g_specialize.load(std::memory_order_relaxed) || p->spec_key == 0) return nullptr;
+  return fx_spec_find(p->spec_key);
+}
+
+// With a dump directory set, every plan that has no specialised kernels linked in leaves
+// the translation unit that would specialise it there (one file per key).
+static void dump_spec_source(const fx::Plan* p) {
+  std::string dir;
+  {
+    std::lock_guard<std::mutex> g(g_dump_mu);
+    dir = g_dump_dir;
+  }
+  if (dir.empty() || p->spec_key == 0 || fx_spec_find(p->spec_key)) return;
+  char name[64];
+  snprintf(name, sizeof(name), "/fx_spec_%016llx.hip", (unsigned long long)p->spec_key);
+  const std::string path = dir + name;
+  if (FILE* f = fopen(path.c_str(), "r")) { fclose(f); return; }
+  // label: what the plan computes, in shapes
+  std::string label = p->mode == FX_MODE_COMPACT ? "row compaction, " : "dense, ";
+  label += std::to_string(p->region->degree) + " task(s), outputs of task 0:";
+  for (size_t o = 0; o < p->out_shape.size(); ++o) {
+    label += " [";
+    const auto& sh = p->out_shape[o][0];
+    for (size_t d = 0; d < sh.size(); ++d) label += (d ? "," : "") + std::to_string(sh[d]);
+    label += "]";
+  }
+  const std::string src = fx::spec_source(*p, label);
+  if (FILE* f = fopen(path.c_str(), "w")) {
+    fwrite(src.data(), 1, src.size(), f);
+    fclose(f);
+  }
+}
+
 int fx_region_plan(fx_region* reg, const fx_arg* args, int n_args, const fx_plan** plan) {
   if (!reg || !plan || (n_args > 0 && !args)) return fail(FX_E_INVALID, "null argument");
   FX_TRY
   std::lock_guard<std::mutex> g(reg->mu);
   const fx::Plan* p = fx::plan_region(reg->r, args, n_args);
   *plan = reinterpret_cast<const fx_plan*>(p);
+  dump_spec_source(p);
   return FX_OK;
   FX_CATCH
 }
 
 static const fx::Plan* P(const fx_plan* p) { return reinterpret_cast<const fx::Plan*>(p); }
+
+void fx_set_specialization(int on) { g_specialize.store(on ? 1 : 0, std::memory_order_relaxed); }
+int fx_specialization_count(void) { return fx_spec_count(); }
+int fx_plan_specialized(const fx_plan* p) { return (p && spec_of(P(p))) ? 1 : 0; }
+uint64_t fx_plan_spec_key(const fx_plan* p) { return p ? P(p)->spec_key : 0; }
+
+int fx_plan_spec_source(const fx_plan* p, const char* label, char* buf, size_t cap) {
+  if (!p || !buf || cap == 0) return fail(FX_E_INVALID, "null argument");
+  FX_TRY
+  std::string s = fx::spec_source(*P(p), label ? label : "");
+  size_t n = std::min(cap - 1, s.size());
+  memcpy(buf, s.data(), n);
+  buf[n] = 0;
+  return (int)s.size();
+  FX_CATCH
+}
+
+void fx_launch_stats(uint64_t* total, uint64_t* specialised) {
+  if (total) *total = g_launches.load(std::memory_order_relaxed);
+  if (specialised) *specialised = g_spec_launches.load(std::memory_order_relaxed);
+}
+
+int fx_spec_dump_dir(const char* dir) {
+  std::lock_guard<std::mutex> g(g_dump_mu);
+  g_dump_dir = dir ? dir : "";
+  return FX_OK;
+}
 
 int fx_plan_num_outputs(const fx_plan* p) { return p ? (int)P(p)->out_dtype.size() : 0; }
 
@@ -359,6 +437,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     // caller must not reuse totals_host while an earlier run is still in flight.
     for (int t = 0; t < reg->r.degree; ++t) totals_host[t] = 0;
   }
+  const FxSpecKernels* spec = spec_of(pl);
+  g_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
+  if (spec) g_spec_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
   const bool timed = kernel_ms != nullptr;
@@ -369,15 +450,15 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   if (pl->mode == FX_MODE_DENSE) {
     HIP_OK(mark(0));
     // persistent workgroups: at most 8 per CU worth of blocks stride over the units
-    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream));
+    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
   } else {
     HIP_OK(mark(0));
-    HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream));
+    HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream, spec));
     HIP_OK(mark(1));
     HIP_OK(mark(2));
-    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn, pl->grid, stream));
+    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn, pl->grid, stream, spec));
     HIP_OK(mark(3));
     nk = pl->grid > 0 ? 2 : 0;
   }

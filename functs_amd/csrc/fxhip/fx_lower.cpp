@@ -2003,6 +2003,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
                              (size_t)max_temps * FX_V * FX_BLOCK) * 4);
   FX_CHECK(P->lds_bytes <= 64 * 1024, FX_E_LIMIT,
            "region descriptor + temporaries need " << P->lds_bytes << " bytes of LDS (limit 65536)");
+  P->spec_key = spec_hash(*P);
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;
@@ -2022,6 +2023,94 @@ static const char* opname(uint32_t op) {
       "INE", "IRANGE", "WHERE", "RBEGIN", "RNEXT", "RIDX", "WMAX", "WSUM"};
   if (op < sizeof(names) / sizeof(names[0])) return names[op];
   return "?";
+}
+
+// ---- specialisation: the compile-time part of a plan, its key and its source ----
+int kernel_rank(int rank) { return rank <= 1 ? 1 : rank <= 4 ? rank : FX_MAXR; }
+
+namespace {
+struct SpecEntry { int begin, end, kind, pure; };
+struct SpecView {
+  const FxInsn* ins = nullptr;
+  uint32_t n_insn = 0;
+  uint32_t n_temps = 0;
+  uint32_t mode = 0;
+  int rank = 1;
+  std::vector<SpecEntry> entries;
+};
+// Only plans with one task class (all tasks share their programs) are specialised.
+bool spec_view(const Plan& p, SpecView* v) {
+  const uint32_t* sb = p.blob.data();
+  const FxHeader* h = (const FxHeader*)sb;
+  if (h->n_classes != 1) return false;
+  const FxClass& cl = *(const FxClass*)(sb + h->off_class);
+  const FxOut* outs = (const FxOut*)(sb + cl.off_outs);
+  v->ins = (const FxInsn*)(sb + cl.off_insn);
+  v->n_temps = cl.n_temps;
+  v->mode = h->mode;
+  v->rank = kernel_rank(p.max_rank);
+  uint32_t n = 0;
+  if (h->mode == FX_MODE_COMPACT) {
+    v->entries.push_back({(int)cl.mask_begin, (int)cl.mask_end, 1, 0});
+    n = std::max(n, cl.mask_end);
+  }
+  for (uint32_t k = 0; k < cl.n_outs; ++k) {
+    const FxOut& od = outs[k];
+    v->entries.push_back({(int)(od.prog_begin + (od.lead ? 1u : 0u)), (int)od.prog_end, 0, (int)od.pure});
+    n = std::max(n, od.prog_end);
+  }
+  v->n_insn = n;
+  return n > 0;
+}
+}  // namespace
+
+uint64_t spec_hash(const Plan& p) {
+  SpecView v;
+  if (!spec_view(p, &v)) return 0;
+  uint64_t hsh = 1469598103934665603ull;   // FNV-1a, 64 bits
+  auto mix = [&](const void* data, size_t n) {
+    const uint8_t* b = (const uint8_t*)data;
+    for (size_t i = 0; i < n; ++i) { hsh ^= b[i]; hsh *= 1099511628211ull; }
+  };
+  const uint32_t head[5] = {v.mode, (uint32_t)v.rank, v.n_insn, v.n_temps, (uint32_t)FX_V};
+  mix(head, sizeof(head));
+  for (uint32_t i = 0; i < v.n_insn; ++i) {
+    const FxInsn& x = v.ins[i];
+    const uint32_t w[4] = {(uint32_t)x.op | ((uint32_t)x.flags << 16) | ((uint32_t)x.dt << 24), (uint32_t)x.a, (uint32_t)x.b, x.imm};
+    mix(w, sizeof(w));
+  }
+  for (const SpecEntry& e : v.entries) mix(&e, sizeof(e));
+  return hsh ? hsh : 1;
+}
+
+std::string spec_source(const Plan& p, const std::string& label) {
+  SpecView v;
+  FX_CHECK(spec_view(p, &v), FX_E_UNSUPPORTED, "only plans whose tasks share one set of programs can be specialised");
+  const uint64_t hsh = spec_hash(p);
+  char hx[32];
+  snprintf(hx, sizeof(hx), "%016llx", (unsigned long long)hsh);
+  std::ostringstream o;
+  o << "// Generated by fx_plan_spec_source; do not edit.  Region: " << label << "\n"
+    << "// The lowered programs of this region as a compile-time table: the region kernels are\n"
+    << "// instantiated for it and picked at run time when a plan's programs hash to the same key.\n"
+    << "#include \"../fx_spec.h\"\n\nnamespace {\nstruct P_" << hx << " {\n"
+    << "  static constexpr uint64_t hash = 0x" << hx << "ull;\n"
+    << "  static constexpr int n_temps = " << v.n_temps << ";\n"
+    << "  static constexpr FxInsn code[" << v.n_insn << "] = {\n";
+  for (uint32_t i = 0; i < v.n_insn; ++i) {
+    const FxInsn& x = v.ins[i];
+    o << "      {FX_" << opname(x.op) << ", " << (int)x.flags << ", " << (int)x.dt << ", " << x.a << ", " << x.b << ", 0x"
+      << std::hex << x.imm << std::dec << "u},  // " << i << "\n";
+  }
+  o << "  };\n  static constexpr int n_entries = " << v.entries.size() << ";\n"
+    << "  static constexpr FxSpecEntry entries[" << v.entries.size() << "] = {";
+  for (size_t i = 0; i < v.entries.size(); ++i) {
+    const SpecEntry& e = v.entries[i];
+    o << (i ? ", " : "") << "{" << e.begin << ", " << e.end << ", " << e.kind << ", " << e.pure << "}";
+  }
+  o << "};\n};\n}  // namespace\n\n"
+    << (v.mode == FX_MODE_COMPACT ? "FX_SPEC_COMPACT" : "FX_SPEC_DENSE") << "(P_" << hx << ", " << v.rank << ")\n";
+  return o.str();
 }
 
 std::string disasm(const Plan& p) {

@@ -90,6 +90,7 @@ struct Plan {
   std::vector<int> arg_base;  // first fx_arg of each region input
   int n_args = 0;
   // device copy of blob, created on first run
+  uint64_t spec_key = 0;       // spec_hash of this plan
   void* dev_blob = nullptr;
   int dev_id = -1;
 };
@@ -97,6 +98,12 @@ struct Plan {
 // Builds (or fetches from the cache) the plan of `r` for these arguments.
 const Plan* plan_region(Region& r, const fx_arg* args, int n_args);
 std::string disasm(const Plan& p);
+// Rank the region kernels are instantiated for (1, 2, 3, 4 or FX_MAXR).
+int kernel_rank(int rank);
+// Key of the compile-time part of a plan (programs, entry points, kernel rank); 0 if the plan
+// cannot be specialised.  spec_source writes the translation unit that specialises it.
+uint64_t spec_hash(const Plan& p);
+std::string spec_source(const Plan& p, const std::string& label);
 
 int dtype_size(int dt);
 

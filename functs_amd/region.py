@@ -260,6 +260,24 @@ class Region:
         check(lib.fx_plan_disasm(p.handle, buf, len(buf)))
         return buf.value.decode()
 
+    def specialized(self, *args):
+        """True if calls with these arguments run ahead-of-time compiled kernels
+        (``python -m functs_amd.aot``) instead of the bytecode interpreter."""
+        arr, n, _ = self._flatten(args)
+        return bool(lib.fx_plan_specialized(self.plan(arr, n).handle))
+
+    def spec_source(self, *args, label=""):
+        """HIP translation unit that specialises the kernels for these arguments."""
+        arr, n, _ = self._flatten(args)
+        p = self.plan(arr, n)
+        buf = ctypes.create_string_buffer(1 << 22)
+        check(lib.fx_plan_spec_source(p.handle, label.encode(), buf, len(buf)))
+        return buf.value.decode()
+
+    def spec_key(self, *args):
+        arr, n, _ = self._flatten(args)
+        return int(lib.fx_plan_spec_key(self.plan(arr, n).handle))
+
     def bind(self, *args):
         """Resolve the plan for these arguments and allocate outputs; returns a
         ``BoundCall`` whose ``launch()`` only marshals and launches."""

@@ -168,6 +168,21 @@ int64_t fx_plan_algorithmic_bytes(const fx_plan*); /* compulsory input bytes + d
 int fx_plan_blob(const fx_plan*, const uint32_t** words, size_t* n_words);
 int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);
 
+/* ---- ahead-of-time specialised kernels ----
+ * The library runs a plan's programs with a bytecode interpreter.  A plan can also be
+ * compiled: fx_plan_spec_source writes a HIP translation unit holding the plan's programs as
+ * compile-time constants; built into the library (csrc/fxhip/spec/), its kernels are used for
+ * every plan whose programs hash to the same key.  Results are the same instruction for
+ * instruction; only speed differs.  Stands where the reference compiles each subgraph at run
+ * time (fait/tensorexpr/cuda_codegen_tssa.cpp:1319-1414 CompileToNVRTC). */
+uint64_t fx_plan_spec_key(const fx_plan*);      /* 0: plan cannot be specialised (tasks with different programs) */
+int fx_plan_specialized(const fx_plan*);        /* 1 if fx_region_run uses specialised kernels for this plan */
+int fx_plan_spec_source(const fx_plan*, const char* label, char* buf, size_t cap); /* returns the full length */
+void fx_set_specialization(int on);             /* process-wide switch, default on (FXHIP_SPECIALIZE=0: off) */
+int fx_specialization_count(void);              /* specialised regions linked into the library */
+void fx_launch_stats(uint64_t* total, uint64_t* specialised); /* region kernel launches of this process so far */
+int fx_spec_dump_dir(const char* dir);          /* plans without specialised kernels leave their source in dir (NULL: stop) */
+
 /* ---- execution (replaces CudaCodeGenTssa::call_raw, cuda_codegen_tssa.cpp:1167-1290) ----
  * out_ptrs[out_idx * parallel_degree + task] = device buffer of that output.
  * scratch: fx_plan_scratch_bytes() of device memory (may be NULL when 0).

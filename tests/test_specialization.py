@@ -1,0 +1,146 @@
+"""Ahead-of-time compiled regions (functs_amd.aot): the compiled kernels must compute what
+the bytecode interpreter computes, bit for bit, and the generated sources that are
+committed must be the ones the current lowering produces for the benchmark programs."""
+import glob
+import os
+
+import pytest
+import torch
+
+import functs_amd.aot as aot
+from functs_amd import Region, _lib, configs
+from functs_amd.benchmark.inputs import INPUTS
+from oracle import configs as oc
+
+SPEC_DIR = aot.SPEC_DIR
+
+
+def _region_calls(name):
+    """(region, cpu arguments) of a benchmark configuration described through the Region API."""
+    args = INPUTS[name](0)
+    if name == "c1":
+        a, b, n = args
+        return [(configs.build_c1(), (b, n))]
+    if name == "c2":
+        return [(configs.build_c2(), args)]
+    if name == "c5":
+        return [(configs.build_c5(16), args)]
+    if name == "c3":
+        return [(configs.build_c3_decode(), args)]
+    raise KeyError(name)
+
+
+def test_product_inputs_equal_oracle_inputs():
+    for name in ("c1", "c2", "c3", "c4", "c5"):
+        mine, theirs = INPUTS[name](0), getattr(oc, name + "_inputs")(0)
+        assert len(mine) == len(theirs)
+        for x, y in zip(mine, theirs):
+            assert torch.equal(x, y) if isinstance(x, torch.Tensor) else x == y
+
+
+def test_library_links_the_committed_specialisations():
+    files = glob.glob(os.path.join(SPEC_DIR, "fx_spec_*.hip"))
+    assert files, "no generated sources under csrc/fxhip/spec"
+    assert aot.linked() == len(files)
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c5"])
+def test_benchmark_regions_have_compiled_kernels(name):
+    # planning needs no GPU: the key of the lowered programs must be one that is linked in
+    for region, args in _region_calls(name):
+        key = region.spec_key(*args)
+        assert key != 0
+        assert region.specialized(*args), "no compiled kernels for key %016x: regenerate with python -m functs_amd.aot" % key
+        # and the committed source is what the lowering produces today
+        path = os.path.join(SPEC_DIR, "fx_spec_%016x.hip" % key)
+        committed = open(path).read().split("\n", 1)[1]
+        assert region.spec_source(*args).split("\n", 1)[1] == committed
+
+
+def test_switch_and_key_of_a_new_region():
+    r = Region()
+    x = r.tensor_input(torch.float32, 2)
+    r.output((x * 3.0 - 0.25).relu())
+    r.finalize()
+    t = torch.zeros(5, 7)
+    assert r.spec_key(t) != 0 and not r.specialized(t)      # nobody compiled this one
+    src = r.spec_source(t, label="test")
+    assert "FX_SPEC_DENSE(P_%016x, 2)" % r.spec_key(t) in src and "FX_RELU" in src
+    # same programs, other sizes: dense programs do not depend on the extents here
+    assert r.spec_key(torch.zeros(9, 7)) == r.spec_key(t)
+    aot.enable(False)
+    try:
+        for region, args in _region_calls("c1"):
+            assert not region.specialized(*args)
+    finally:
+        aot.enable(True)
+
+
+def test_capture_writes_one_file_per_unknown_region(tmp_path):
+    r = Region()
+    x = r.tensor_input(torch.float32, 1)
+    r.output(x.sigmoid() + 1.0)
+    r.finalize()
+    with aot.capture(str(tmp_path)):
+        r.disasm(torch.zeros(100))        # planning is enough
+        for region, args in _region_calls("c1"):
+            region.disasm(*args)          # already linked: leaves nothing
+    files = os.listdir(tmp_path)
+    assert files == ["fx_spec_%016x.hip" % r.spec_key(torch.zeros(100))]
+    r.disasm(torch.zeros(50))             # capture is over
+    assert os.listdir(tmp_path) == files
+
+
+def _flat(o):
+    if isinstance(o, (list, tuple)):
+        for x in o:
+            yield from _flat(x)
+    else:
+        yield o
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c5"])
+def test_compiled_equals_interpreter_region_api(name):
+    dev = torch.device("cuda:0")
+    prev = None
+    for region, args in _region_calls(name) + ([(configs.build_c3_classes(80), None)] if name == "c3" else []):
+        gargs = prev if args is None else [a.to(dev) if isinstance(a, torch.Tensor) else a for a in args]
+        assert region.specialized(*gargs)
+        total0, spec0 = aot.launch_stats()
+        fast = list(_flat(region(*gargs)))
+        total1, spec1 = aot.launch_stats()
+        assert spec1 - spec0 == total1 - total0 > 0
+        aot.enable(False)
+        try:
+            slow = list(_flat(region(*gargs)))
+            assert aot.launch_stats()[1] == spec1
+        finally:
+            aot.enable(True)
+        assert len(fast) == len(slow)
+        for x, y in zip(fast, slow):
+            assert x.shape == y.shape and torch.equal(x, y)
+        prev = region(*gargs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_compiled_equals_interpreter_torchscript_route(name):
+    import functs_amd.jit as fj
+    from functs_amd.benchmark import PROGRAMS
+    dev = torch.device("cuda:0")
+    cpu_args = INPUTS[name](0)
+    fn = fj.build(fj.script(PROGRAMS[name]), list(cpu_args))
+    gargs = [a.to(dev) if isinstance(a, torch.Tensor) else a for a in cpu_args]
+    total0, spec0 = aot.launch_stats()
+    fast = list(_flat(fn(*gargs)))
+    total1, spec1 = aot.launch_stats()
+    assert total1 > total0 and spec1 - spec0 == total1 - total0, "a region of %s ran interpreted" % name
+    aot.enable(False)
+    try:
+        slow = list(_flat(fn(*gargs)))
+    finally:
+        aot.enable(True)
+    assert len(fast) == len(slow)
+    for x, y in zip(fast, slow):
+        assert x.shape == y.shape and torch.equal(x, y)

@@ -208,6 +208,7 @@ def main():
             "latency_us": round(ms * 1e3, 2),
             "kernel_us": [round(k * 1e3, 2) for k in kern],
             "launches_per_call": w.launches,
+            "row_compaction": any(bc.plan.compact for bc in w.bound),
             "algorithmic_bytes": alg,
             "gbps_dominant_kernel": round(alg / (dom * 1e-3) / 1e9, 1),
             "gbps_all_kernels": round(alg / (sum(kern) * 1e-3) / 1e9, 1),
@@ -316,7 +317,7 @@ def main():
             per["c4"] = {"error": str(e)[:200]}
     cpu_us, cpu_n, cores = head.pop("cpu")
     dom_ms = max(head["kernel_us"]) / 1e3
-    dom_kernel = "fx_compact_scatter" if head["launches_per_call"] > 1 else "fx_region_dense"
+    dom_kernel = "fx_compact_scatter" if head["row_compaction"] else "fx_region_dense"
     out = {
         "metric": "per-call latency",
         "value": head["torchscript_route_latency_us"],

@@ -272,6 +272,7 @@ c10::ScalarType atDtype(int d) {
 // borrows one and hands it back, so concurrent calls never share
 struct Workspace {
   at::Tensor scratch, totals;
+  void* stream = nullptr;   // stream of the last run that used it (that run may still be in flight)
 };
 
 struct Variant {
@@ -281,15 +282,24 @@ struct Variant {
   ~Variant() {
     if (region) fx_region_destroy(region);
   }
-  Workspace take(size_t scratch_bytes, int64_t degree, c10::Device device) {
+  // A workspace goes back to the pool as soon as the kept-row counts are known, while the
+  // second pass may still be reading its scratch: on the same stream the next run is ordered
+  // behind it; another stream waits for it first.
+  Workspace take(size_t scratch_bytes, int64_t degree, c10::Device device, void* stream) {
     {
-      std::lock_guard<std::mutex> lock(mu);
+      std::unique_lock<std::mutex> lock(mu);
       while (!pool.empty()) {
         Workspace ws = std::move(pool.back());
         pool.pop_back();
         if ((size_t)ws.scratch.numel() >= scratch_bytes && ws.totals.numel() >= degree &&
-            ws.scratch.device() == device)
+            ws.scratch.device() == device) {
+          lock.unlock();
+          if (ws.stream != stream) {
+            const hipError_t e = hipStreamSynchronize((hipStream_t)ws.stream);
+            TORCH_CHECK(e == hipSuccess, "hipStreamSynchronize: ", hipGetErrorString(e));
+          }
           return ws;
+        }
       }
     }
     Workspace ws;
@@ -426,9 +436,12 @@ class RegionRunner {
       for (int64_t t = 0; t < degree; ++t)
         ptrs[(size_t)o * degree + t] = base + slots[(size_t)o * degree + t].offset_elems * item;
     }
-    Workspace ws;
-    if (compact_) ws = var->take(fx_plan_scratch_bytes(plan), degree, device);
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
+    Workspace ws;
+    if (compact_) {
+      ws = var->take(fx_plan_scratch_bytes(plan), degree, device, (void*)stream.stream());
+      ws.stream = (void*)stream.stream();
+    }
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
@@ -449,9 +462,10 @@ class RegionRunner {
       }
     }
     if (compact_) {
-      // the kept-row counts decide the output shapes: one synchronisation, as ATen's
-      // nonzero / masked index does
-      stream.synchronize();
+      // The kept-row counts decide the output shapes.  ATen's nonzero / masked index
+      // synchronise the stream for that; here the counts arrive through pinned memory early
+      // in the second pass, and the outputs are valid in stream order.
+      FX_OK_OR_THROW(fx_region_wait_totals(plan, (const uint32_t*)ws.totals.data_ptr(), (void*)stream.stream()));
       const int32_t* tot = ws.totals.data_ptr<int32_t>();
       for (int o = 0; o < n_out; ++o)
         for (int64_t t = 0; t < degree; ++t) {

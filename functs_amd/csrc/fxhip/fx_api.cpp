@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -433,9 +434,13 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   li.n_temps = pl->n_temps;
   li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
   if (pl->mode == FX_MODE_COMPACT) {
-    // tasks without rows launch no tile: their total is published here.  The
-    // caller must not reuse totals_host while an earlier run is still in flight.
-    for (int t = 0; t < reg->r.degree; ++t) totals_host[t] = 0;
+    // Tasks without rows launch no tile: their total is published here.  The others hold a
+    // mark until the last tile of the task stores the count (fx_region_wait_totals looks for
+    // it).  The caller must not reuse totals_host while an earlier run is still in flight.
+    for (int t = 0; t < reg->r.degree; ++t)
+      totals_host[t] = (pl->out_shape.empty() || pl->out_shape[0][t].empty() || pl->out_shape[0][t][0] > 0)
+                           ? FX_TOTAL_PENDING
+                           : 0u;
   }
   const FxSpecKernels* spec = spec_of(pl);
   g_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
@@ -468,6 +473,43 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     for (auto& e : ev) (void)hipEventDestroy(e);
     if (n_kernels) *n_kernels = nk;
   }
+  return FX_OK;
+}
+
+int fx_region_wait_totals(const fx_plan* plan, const uint32_t* totals_host, void* stream_) {
+  if (!plan || !totals_host) return fail(FX_E_INVALID, "null argument");
+  const fx::Plan* pl = P(plan);
+  if (pl->mode != FX_MODE_COMPACT) return fail(FX_E_INVALID, "not a compacting region");
+  hipStream_t stream = (hipStream_t)stream_;
+  const volatile uint32_t* tot = totals_host;
+  const int T = pl->region->degree;
+  // The count of a task is stored by its last tile early in the second pass, through
+  // host-coherent memory: it is usually here well before the kernel has finished.  If the
+  // stream has drained without all of them showing up (memory that the host does not see
+  // until then), a synchronisation settles it.
+  using clock = std::chrono::steady_clock;
+  const clock::time_point t0 = clock::now();
+  clock::time_point next_query = t0 + std::chrono::microseconds(50);
+  for (;;) {
+    bool all = true;
+    for (int t = 0; t < T; ++t) all = all && tot[t] != FX_TOTAL_PENDING;
+    if (all) {
+      std::atomic_thread_fence(std::memory_order_acquire);
+      return FX_OK;
+    }
+    __builtin_ia32_pause();
+    const clock::time_point now = clock::now();
+    if (now >= next_query) {
+      // the runtime is asked rarely: a query takes its locks and slows the launches of other threads
+      const hipError_t q = hipStreamQuery(stream);
+      if (q == hipSuccess || now - t0 > std::chrono::seconds(10)) break;
+      if (q != hipErrorNotReady) HIP_OK(q);
+      next_query = now + std::chrono::microseconds(50);
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  for (int t = 0; t < T; ++t)
+    if (tot[t] == FX_TOTAL_PENDING) return fail(FX_E_HIP, "a task's kept-row count was never written");
   return FX_OK;
 }
 

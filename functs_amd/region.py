@@ -324,6 +324,7 @@ class BoundCall:
     def launch(self, stream=None):
         if stream is None:
             stream = torch.cuda.current_stream(self.device).cuda_stream
+        self._stream = stream
         check(lib.fx_region_run(self.region._h, self.plan.handle, self.arr, self.n, self.ptrs,
                                 self.scratch.data_ptr() if self.scratch is not None else None,
                                 self.totals.data_ptr() if self.totals is not None else None,
@@ -334,6 +335,7 @@ class BoundCall:
         kernel durations in milliseconds (synchronises)."""
         if stream is None:
             stream = torch.cuda.current_stream(self.device).cuda_stream
+        self._stream = stream
         ms = (ctypes.c_float * 4)()
         nk = ctypes.c_int()
         check(lib.fx_region_run_timed(self.region._h, self.plan.handle, self.arr, self.n, self.ptrs,
@@ -345,9 +347,11 @@ class BoundCall:
     def results(self):
         """Outputs as the operator returns them: a tensor per output, or a list
         of per-task tensors for a ParallelMap.  Compacted outputs are narrowed to
-        the kept rows (this synchronises the stream, like ATen's nonzero)."""
+        the kept rows: this waits for the kept-row counts, which the kernels store
+        early (ATen's nonzero waits for the whole stream); the outputs are valid in
+        stream order."""
         if self.plan.compact:
-            torch.cuda.current_stream(self.device).synchronize()
+            check(lib.fx_region_wait_totals(self.plan.handle, self.totals.data_ptr(), ctypes.c_void_p(self._stream)))
             totals = self.totals.tolist()
             outs = [[ten.narrow(0, 0, totals[t]) for t, ten in enumerate(row)] for row in self.outs]
         else:

@@ -188,10 +188,20 @@ int fx_spec_dump_dir(const char* dir);          /* plans without specialised ker
  * scratch: fx_plan_scratch_bytes() of device memory (may be NULL when 0).
  * totals_host: for compacting regions, pinned host memory (device-visible) of
  *   parallel_degree uint32 that receives the kept-row count per task; it is
- *   valid after the stream has been synchronised.  NULL otherwise.
+ *   valid after the stream has been synchronised, or after fx_region_wait_totals.
+ *   NULL otherwise.
  * Asynchronous on `stream` (a hipStream_t); no hidden synchronisation. */
 int fx_region_run(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
                   void* scratch, uint32_t* totals_host, void* stream);
+
+/* Returns once every task's kept-row count of the last fx_region_run on `stream` with this
+ * totals_host is readable.  The counts are stored early in the second pass, so this usually
+ * returns while the kernels still run: the caller can size its output views and go on; the
+ * outputs themselves are valid in stream order, like after any asynchronous launch.  Falls
+ * back to synchronising the stream.  Where ATen's nonzero / masked index synchronise
+ * (the reference leaves x[mask] to them, convert_to_tensorssa.cpp:422-443). */
+#define FX_TOTAL_PENDING 0xffffffffu
+int fx_region_wait_totals(const fx_plan*, const uint32_t* totals_host, void* stream);
 
 /* fx_region_run with a HIP event pair around every kernel on `stream`; waits for
  * the last event and returns the duration of each launch in milliseconds

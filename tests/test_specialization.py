@@ -144,3 +144,4 @@ def test_compiled_equals_interpreter_torchscript_route(name):
     assert len(fast) == len(slow)
     for x, y in zip(fast, slow):
         assert x.shape == y.shape and torch.equal(x, y)
+

@@ -4,13 +4,19 @@
 
 A step is one call of the hot path on one batch of synthetic, seeded input
 already resident in HBM: plan lookup + argument marshalling + output allocation
-+ kernel launches + the stream synchronisation that returns the kept-row counts
-(what a caller of the operator waits for).  Prints ONE JSON line.  `value` is
-the per-call latency of the headline workload (c5: ParallelMap over 16
-YOLOv3-style images) through the TorchScript route, i.e. the scripted program
-whose fused regions run as tssa::ParallelFunctor; `region_api_latency_us` is
-the same regions driven from Python through ctypes; `per_config` repeats the measurement for every BASELINE.json config
-that is implemented.  `roofline` prices the dominant kernel against the 8 TB/s
++ kernel launches + the wait for the kept-row counts (what a caller of the
+operator waits for; the counts arrive before the kernels end, so consecutive
+calls overlap on the stream).  K steps are timed back to back between two device
+synchronisations, the way the reference times a call (functs/utils/evaluate.py:179-190).
+Prints ONE JSON line.  `value` is the per-call latency of the headline workload
+(c5: ParallelMap over 16 YOLOv3-style images) through the TorchScript route, i.e.
+the scripted program whose fused regions run as tssa::ParallelFunctor;
+`drained_latency_us` is the same call with the device drained after every call;
+`region_api_latency_us` is the same regions driven from Python through ctypes;
+`compiled_kernels` says whether the regions ran ahead-of-time compiled kernels
+(functs_amd.aot) or the bytecode interpreter (`--interpreter` forces the latter);
+`per_config` repeats the measurement for every BASELINE.json config that is
+implemented.  `roofline` prices the dominant kernel against the 8 TB/s
 HBM peak with the algorithmic bytes of the call; `cpu_baseline` times the
 unfused TorchScript CPU path (the oracle) on a bounded sample.
 """
@@ -152,8 +158,15 @@ def torchscript_route(name, cpu_args, dev, steps, warmup):
     torch.cuda.synchronize()
     us = (time.perf_counter() - t0) * 1e6 / steps
     l1, s1 = aot.launch_stats()
+    # the same call with the device drained after every call: issue to completion of one call
+    n_sync = max(steps // 4, 5)
+    t0 = time.perf_counter()
+    for _ in range(n_sync):
+        fn(*args)
+        torch.cuda.synchronize()
+    sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
     n_functors = str(fn.graph).count("= tssa::ParallelFunctor")
-    return us, n_functors, (s1 - s0) / max(l1 - l0, 1)
+    return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us
 
 
 def cpu_baseline(name, budget_s):
@@ -221,8 +234,9 @@ def main():
             _, ikern = measure(w, max(args.steps // 4, 5), 3)
             aot.enable(True)
             rec["interpreter_kernel_us"] = [round(k * 1e3, 2) for k in ikern]
-        ts_us, n_functors, spec_share = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup)
+        ts_us, n_functors, spec_share, sync_us = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup)
         rec["torchscript_route_latency_us"] = round(ts_us, 2)
+        rec["torchscript_route_drained_latency_us"] = round(sync_us, 2)
         rec["torchscript_route_functors"] = n_functors
         rec["torchscript_route_compiled_share"] = round(spec_share, 3)
         if with_cpu:
@@ -246,7 +260,7 @@ def main():
         select_rev of `out`.  Only the TorchScript route exists for it."""
         from functs_amd.benchmark.inputs import INPUTS
         cpu_args = INPUTS["c4"](0)
-        us, n_functors, spec_share = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
+        us, n_functors, spec_share, _ = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
         # the same call replayed as one HIP graph (functs_amd.jit.build(..., hip_graph=True))
         import functs_amd.jit as fj
         from functs_amd.benchmark import PROGRAMS
@@ -334,6 +348,7 @@ def main():
         "config": {"workload": head["workload"],
                    "route": "functs_amd.jit.script -> build -> tssa::ParallelFunctor (C++ operator over the C ABI)",
                    "compiled_kernels": head["compiled_kernels"] and not args.interpreter,
+                   "drained_latency_us": head["torchscript_route_drained_latency_us"],
                    "region_api_latency_us": head["latency_us"], "launches_per_call": head["launches_per_call"],
                    "kernel_us": head["kernel_us"], "gbps_all_kernels": head["gbps_all_kernels"]},
         "roofline": {"bound": "hbm", "achieved": head["gbps_dominant_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",

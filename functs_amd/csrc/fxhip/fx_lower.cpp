@@ -1838,6 +1838,11 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       max_rank = std::max<int>(max_rank, (int)s.size());
       cb.outs.push_back(od);
     }
+    // The second compaction pass walks the outputs in table order (half of the waves
+    // backwards).  Narrow outputs read a few bytes of every kept row, i.e. the same 128-byte
+    // lines as each other: next to each other in the walk, the second one finds them in L2.
+    if (P->mode == FX_MODE_COMPACT)
+      std::stable_sort(cb.outs.begin(), cb.outs.end(), [](const FxOut& a, const FxOut& b) { return a.rowlen < b.rowlen; });
     cb.code = L.code;
     cb.affs = L.affs;
     cb.cls.n_temps = (uint32_t)L.maxTemps;

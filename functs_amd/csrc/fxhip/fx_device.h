@@ -752,6 +752,9 @@ struct FxInterp {
   }
   // items of a pure program that the compaction kernel batches (the dense kernel: FX_K)
   static constexpr uint32_t kPure = FX_K;
+  // order in which a wave of the compaction kernel walks the outputs: 0 = alternate waves
+  // backwards, 1 = all forwards (narrow outputs first), 2 = all backwards
+  static constexpr int kWalk = 0;
   template <int N>
   static __device__ __forceinline__ void run_pure(const FxCtx& cx, int pc, int pc_end, uint32_t (&X)[N]) {
     fx_run_pure(cx, pc, pc_end, X);
@@ -1195,7 +1198,7 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
   // Half of the waves walk the outputs backwards: a latency-bound output (a long
   // predicated program on a few items) then overlaps, on the same SIMD, with the
   // arithmetic-bound wide outputs of the other waves.
-  const bool backwards = ((blockIdx.x + wave_u) & 1u) != 0;
+  const bool backwards = S::kWalk == 0 ? ((blockIdx.x + wave_u) & 1u) != 0 : S::kWalk == 2;
   for (uint32_t oo = 0; oo < n_outs; ++oo) {
     const uint32_t oi = backwards ? n_outs - 1u - oo : oo;
     const uint32_t* od = outs + oi * ow;

@@ -128,6 +128,9 @@ struct FxSpec {
   }
   // compiled code is short: registers are spent on more loads in flight instead
   static constexpr uint32_t kPure = 2 * FX_K;
+  // all waves take the narrow outputs first: those share their 128-byte lines, and compiled
+  // their programs are too short to be worth overlapping with the wide outputs
+  static constexpr int kWalk = 1;
   template <int N>
   static __device__ __forceinline__ void run_pure(const FxCtx&, int pc, int, uint32_t (&X)[N]) {
     dispatch_pure<0, N>(pc, X);

@@ -279,9 +279,14 @@ void FuseOps(std::shared_ptr<Graph> graph) {
   std::vector<Block*> blocks;
   collectBlocks(graph->block(), blocks);
   for (Block* b : blocks) {
-    // the body of a ParallelMap is fused as a whole, whatever its size
-    const bool in_map = b->owningNode() && b->owningNode()->kind() == sym::ParallelMap();
-    fuseBlock(b, in_map);
+    // a ParallelMap body that is fusable throughout is fused as a whole, whatever its size
+    // (one launch instead of a loop); a mixed body follows the ordinary rule, so that a lone
+    // view next to an unfusable operator does not become a launch of its own
+    bool whole_map = b->owningNode() && b->owningNode()->kind() == sym::ParallelMap();
+    if (whole_map)
+      for (Node* n : b->nodes())
+        whole_map = whole_map && (n->kind() == c10::prim::Constant || isFusableNode(n) || isIndexLike(n));
+    fuseBlock(b, whole_map);
   }
 }
 
@@ -387,6 +392,7 @@ bool tryParallelize(Node* loop) {
   if (!condc || !condc->isBool() || !condc->toBool() || !nextc || !nextc->isBool() || !nextc->toBool()) return false;
   Value* i = body->inputs()[0];
   std::vector<Node*> reads, appends;
+  bool any_fusable = false;
   for (Node* n : body->nodes()) {
     if (n->kind() == c10::prim::Constant) continue;
     if (n->kind() == c10::aten::__getitem__ && n->input(0)->type()->cast<c10::ListType>()) {
@@ -405,9 +411,17 @@ bool tryParallelize(Node* loop) {
       continue;
     }
     if (!n->blocks().empty()) return false;
-    if (!isFusableNode(n) && !isIndexLike(n)) return false;
+    if (isFusableNode(n) || isIndexLike(n)) {
+      any_fusable = any_fusable || n->kind() != c10::prim::ListConstruct;
+      continue;
+    }
+    // anything else without effects may stay: SplitParallelMaps gives the fusable stretches
+    // maps of their own and the rest returns to a loop (parallelize_loops.cpp:152-362)
+    if (n->hasSideEffects()) return false;
+    if (const auto* schema = n->maybeSchema())
+      if (schema->is_mutable()) return false;
   }
-  if (appends.empty()) return false;
+  if (appends.empty() || !any_fusable) return false;
   // output lists: defined right before use, only appended to inside this loop
   for (Node* a : appends)
     for (const Use& u : a->input(0)->uses())
@@ -583,6 +597,120 @@ void foldIn(Block* b) {
 void FuseMaskedSelect(std::shared_ptr<Graph> graph) { foldIn(graph->block()); }
 
 // ---------------------------------------------------------------------------
+// SplitParallelMaps (fait/passes/parallelize_loops.cpp:152-293): a map whose body holds
+// fusion groups next to other nodes is cut so that every group is alone in a map (one launch
+// for all tasks); what lies between the groups gets maps of its own, which ToParallelFunctor
+// turns back into loops.  A value that crosses a cut travels as a list with one element per task.
+// ---------------------------------------------------------------------------
+namespace {
+
+bool splitMap(Node* map) {
+  Graph* g = map->owningGraph();
+  Block* mb = map->blocks()[0];
+  // constants are free: they move in front of the map and stay visible to every part
+  for (auto it = mb->nodes().begin(); it != mb->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    if (n->kind() == c10::prim::Constant) n->moveBefore(map);
+  }
+  std::vector<std::vector<Node*>> segs;
+  bool prev_group = false, any_group = false;
+  for (Node* n : mb->nodes()) {
+    const bool is_group = n->kind() == c10::prim::FusionGroup;
+    any_group = any_group || is_group;
+    if (segs.empty() || is_group || prev_group) segs.emplace_back();
+    segs.back().push_back(n);
+    prev_group = is_group;
+  }
+  if (!any_group || segs.size() < 2) return false;
+
+  struct Part {
+    Node* map = nullptr;
+    Block* block = nullptr;
+    std::unordered_map<Value*, Value*> vm;       // value of the old body -> value in this part
+    std::unordered_map<Value*, Value*> exported; // value of the old body -> list output of this part
+  };
+  std::vector<Part> parts(segs.size());
+  std::unordered_map<Value*, size_t> def_part;   // value of the old body -> part that computes it
+
+  auto exportValue = [&](size_t t, Value* v) -> Value* {
+    Part& T = parts[t];
+    auto it = T.exported.find(v);
+    if (it != T.exported.end()) return it->second;
+    T.block->registerOutput(T.vm.at(v));
+    Value* list = T.map->addOutput()->setType(c10::ListType::create(v->type()));
+    T.exported[v] = list;
+    return list;
+  };
+  std::function<Value*(size_t, Value*)> resolve = [&](size_t s, Value* v) -> Value* {
+    Part& P = parts[s];
+    auto it = P.vm.find(v);
+    if (it != P.vm.end()) return it->second;
+    auto pos = std::find(mb->inputs().begin() + 1, mb->inputs().end(), v);
+    Value* list = nullptr;
+    if (pos != mb->inputs().end()) {
+      list = map->input(pos - mb->inputs().begin());      // element of one of the map's own lists
+    } else {
+      auto d = def_part.find(v);
+      if (d == def_part.end()) return v;                  // defined outside the map
+      list = exportValue(d->second, v);
+    }
+    P.map->addInput(list);
+    Value* param = P.block->addInput()->copyMetadata(v);
+    P.vm[v] = param;
+    return param;
+  };
+
+  Node* prev = map;
+  for (size_t s = 0; s < segs.size(); ++s) {
+    Part& P = parts[s];
+    P.map = g->create(sym::ParallelMap(), {map->input(0)}, 0);
+    P.map->setSourceRange(map->sourceRange());
+    P.map->insertAfter(prev);
+    prev = P.map;
+    P.block = P.map->addBlock();
+    P.vm[mb->inputs()[0]] = P.block->addInput()->setType(c10::IntType::get());
+    for (Node* n : segs[s]) {
+      Node* c = g->createClone(n, [&](Value* v) { return resolve(s, v); });
+      P.block->appendNode(c);
+      for (size_t k = 0; k < n->outputs().size(); ++k) {
+        P.vm[n->output(k)] = c->output(k);
+        def_part[n->output(k)] = s;
+      }
+    }
+  }
+  for (size_t k = 0; k < map->outputs().size(); ++k) {
+    Value* r = mb->outputs()[k];
+    auto d = def_part.find(r);
+    Value* list;
+    if (d != def_part.end()) {
+      list = exportValue(d->second, r);
+    } else {  // an element of an input list or an outer value handed through: the first part returns it
+      Part& P = parts[0];
+      P.block->registerOutput(resolve(0, r));
+      list = P.map->addOutput();
+    }
+    list->setType(map->output(k)->type());
+    map->output(k)->replaceAllUsesWith(list);
+  }
+  map->destroy();
+  return true;
+}
+
+void splitIn(Block* b) {
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) splitIn(inner);
+    if (n->kind() == sym::ParallelMap()) splitMap(n);
+  }
+}
+
+}  // namespace
+
+void SplitParallelMaps(std::shared_ptr<Graph> graph) { splitIn(graph->block()); }
+
+// ---------------------------------------------------------------------------
 // Validate
 // ---------------------------------------------------------------------------
 namespace {
@@ -623,6 +751,7 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   ParallelizeLoops(graph);
   FuseOps(graph);
   FuseMaskedSelect(graph);
+  SplitParallelMaps(graph);
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
   Validate(graph);

@@ -25,6 +25,8 @@ void CollapseAssignLoops(std::shared_ptr<torch::jit::Graph> graph);
 // list reads are list[i] and whose list writes are one append per list become
 // prim::ParallelMap(len, lists...){block(i, elems...) -> rets}.
 void ParallelizeLoops(std::shared_ptr<torch::jit::Graph> graph);
+// fait/passes/parallelize_loops.cpp:152-293: every fusion group of a map body gets a map of its own
+void SplitParallelMaps(std::shared_ptr<torch::jit::Graph> graph);
 
 // Fold `x[mask]` consumers of a FusionGroup into the group when the bool mask is
 // produced by the same group (row compaction fused into the region).  The

@@ -187,11 +187,10 @@ Node* mapBackToLoop(Node* mapNode) {
     app->output()->setType(out_lists[k]->type());
     lb->appendNode(app);
   }
-  Node* ct = g->create(c10::prim::Constant, 1);
-  ct->output()->setType(c10::BoolType::get());
-  ct->ival_(c10::attr::value, true);
-  lb->appendNode(ct);
-  lb->registerOutput(ct->output());
+  {
+    WithInsertPoint in_body(lb->return_node());
+    lb->registerOutput(g->insertConstant(true));
+  }
   for (size_t k = 0; k < out_lists.size(); ++k) mapNode->output(k)->replaceAllUsesWith(out_lists[k]);
   mapNode->destroy();
   return loop;

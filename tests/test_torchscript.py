@@ -88,19 +88,53 @@ def test_c3_is_decode_plus_class_map():
     assert "aten::softmax" in _kinds(fs[0].g("Subgraph"))
 
 
-def test_unfusable_map_body_returns_to_a_loop():
+def _mixed_body(x: torch.Tensor):
+    out = []
+    for i in range(x.size(0)):
+        r = x[i] * 2 + 1
+        out.append(torch.nonzero(r > 1.5).float().sigmoid().exp())
+    return out
+
+
+def test_map_is_split_around_unfusable_nodes():
+    """SplitParallelMaps (fait/passes/parallelize_loops.cpp:152-293): each fused stretch of the
+    loop body becomes one launch over all iterations; nonzero stays in a loop between them and
+    its ragged results travel as a list."""
+    f = fj.build(fj.script(_mixed_body), [torch.rand(3, 8)])
+    kinds = _kinds(f.graph)
+    assert "prim::ParallelMap" not in kinds and "prim::FusionGroup" not in kinds
+    assert kinds.count("tssa::ParallelFunctor") == 2 and kinds.count("prim::Loop") == 1
+    loop = [n for n in f.graph.nodes() if n.kind() == "prim::Loop"][0]
+    body = [n.kind() for n in loop.blocks().__next__().nodes()]
+    assert "aten::nonzero" in body and "tssa::ParallelFunctor" not in body
+    for fn in _functors(f.graph):
+        assert fn.i("is_parallel_map") == 1
+    _C._jit_pass_validate(f.graph)
+
+
+def test_map_without_fusable_work_stays_a_loop():
     def prog(x: torch.Tensor):
         out = []
         for i in range(x.size(0)):
-            r = x[i] * 2 + 1
-            out.append(torch.nonzero(r).float().sigmoid().exp())
+            out.append(torch.nonzero(x[i]))
         return out
 
     f = fj.build(fj.script(prog), [torch.rand(3, 8)])
     kinds = _kinds(f.graph)
-    assert "prim::ParallelMap" not in kinds and "prim::FusionGroup" not in kinds
+    assert "prim::ParallelMap" not in kinds and "tssa::ParallelFunctor" not in kinds
     assert "prim::Loop" in kinds and "aten::nonzero" in kinds
-    _C._jit_pass_validate(f.graph)
+
+
+@pytest.mark.gpu
+def test_split_map_runs_on_gpu():
+    x = torch.rand(5, 33, generator=torch.Generator().manual_seed(3))
+    want = torch.jit.script(_mixed_body)(x)
+    f = fj.build(fj.script(_mixed_body), [x])
+    got = f(x.cuda())
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        torch.testing.assert_close(g.cpu(), w, rtol=1e-5, atol=1e-6)
 
 
 def test_single_elementwise_op_is_left_to_aten():

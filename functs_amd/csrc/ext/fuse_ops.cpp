@@ -597,6 +597,122 @@ void foldIn(Block* b) {
 void FuseMaskedSelect(std::shared_ptr<Graph> graph) { foldIn(graph->block()); }
 
 // ---------------------------------------------------------------------------
+// UnrollLoopsWithDeps (fait/passes/unroll_loops.cpp:11-77) and UnrollSimpleMaps
+// (fait/passes/parallelize_loops.cpp:372-456): short loops with carried values whose body did
+// not fuse, and maps that only compute from their own parameters and constants, are written
+// out; the second FuseOps then fuses across what were iterations.
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int64_t kMaxUnroll = 64;  // the reference has no limit; a long loop stays a loop here
+
+bool bodyIsFlat(Block* body) {
+  for (Node* n : body->nodes()) {
+    if (!n->blocks().empty() || n->kind() == c10::prim::FusionGroup || n->kind() == sym::ParallelMap() ||
+        n->kind() == sym::ForallSelectRev())
+      return false;
+    if (n->hasSideEffects()) return false;
+  }
+  return true;
+}
+
+void cloneBodyBefore(Block* body, Node* before, std::unordered_map<Value*, Value*>& vm) {
+  Graph* g = before->owningGraph();
+  auto env = [&](Value* v) -> Value* {
+    auto it = vm.find(v);
+    return it != vm.end() ? it->second : v;
+  };
+  for (Node* n : body->nodes()) {
+    Node* c = g->createClone(n, env);
+    c->insertBefore(before);
+    for (size_t k = 0; k < n->outputs().size(); ++k) vm[n->output(k)] = c->output(k);
+  }
+}
+
+bool tryUnrollLoop(Node* loop) {
+  if (loop->inputs().size() <= 2) return false;   // no carried values: ParallelizeLoops' business
+  auto trip = constant_as<int64_t>(loop->input(0));
+  auto cond = constant_as<bool>(loop->input(1));
+  Block* body = loop->blocks()[0];
+  auto next = constant_as<bool>(body->outputs()[0]);
+  if (!trip || *trip < 0 || *trip > kMaxUnroll || !cond || !*cond || !next || !*next) return false;
+  if (!bodyIsFlat(body)) return false;
+  Graph* g = loop->owningGraph();
+  WithInsertPoint guard(loop);
+  std::vector<Value*> carried(loop->inputs().begin() + 2, loop->inputs().end());
+  for (int64_t i = 0; i < *trip; ++i) {
+    std::unordered_map<Value*, Value*> vm;
+    vm[body->inputs()[0]] = g->insertConstant(i);
+    for (size_t k = 0; k < carried.size(); ++k) vm[body->inputs()[k + 1]] = carried[k];
+    cloneBodyBefore(body, loop, vm);
+    for (size_t k = 0; k < carried.size(); ++k) {
+      Value* r = body->outputs()[k + 1];
+      auto it = vm.find(r);
+      carried[k] = it != vm.end() ? it->second : r;
+    }
+  }
+  for (size_t k = 0; k < carried.size(); ++k) loop->output(k)->replaceAllUsesWith(carried[k]);
+  loop->destroy();
+  return true;
+}
+
+bool tryUnrollMap(Node* map) {
+  auto trip = constant_as<int64_t>(map->input(0));
+  if (!trip || *trip < 0 || *trip > kMaxUnroll) return false;
+  Block* body = map->blocks()[0];
+  if (!bodyIsFlat(body)) return false;
+  for (Node* n : body->nodes())
+    for (Value* in : n->inputs())
+      if (in->node()->kind() != c10::prim::Constant && in->node()->owningBlock() != body) return false;
+  Graph* g = map->owningGraph();
+  WithInsertPoint guard(map);
+  std::vector<std::vector<Value*>> outs(map->outputs().size());
+  for (int64_t i = 0; i < *trip; ++i) {
+    std::unordered_map<Value*, Value*> vm;
+    Value* idx = g->insertConstant(i);
+    vm[body->inputs()[0]] = idx;
+    for (size_t k = 1; k < map->inputs().size(); ++k) {
+      Node* get = g->create(c10::aten::__getitem__, {map->input(k), idx}, 1);
+      get->output()->setType(body->inputs()[k]->type());
+      g->insertNode(get);
+      vm[body->inputs()[k]] = get->output();
+    }
+    cloneBodyBefore(body, map, vm);
+    for (size_t k = 0; k < outs.size(); ++k) {
+      Value* r = body->outputs()[k];
+      auto it = vm.find(r);
+      outs[k].push_back(it != vm.end() ? it->second : r);
+    }
+  }
+  for (size_t k = 0; k < outs.size(); ++k) {
+    auto lt = map->output(k)->type()->cast<c10::ListType>();
+    Node* lc = g->createList(lt->getElementType(), outs[k]);
+    g->insertNode(lc);
+    lc->output()->setType(map->output(k)->type());
+    map->output(k)->replaceAllUsesWith(lc->output());
+  }
+  map->destroy();
+  return true;
+}
+
+bool unrollIn(Block* b, bool maps) {
+  bool changed = false;
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) changed = unrollIn(inner, maps) || changed;
+    if (!maps && n->kind() == c10::prim::Loop) changed = tryUnrollLoop(n) || changed;
+    if (maps && n->kind() == sym::ParallelMap()) changed = tryUnrollMap(n) || changed;
+  }
+  return changed;
+}
+
+}  // namespace
+
+bool UnrollLoopsWithDeps(std::shared_ptr<Graph> graph) { return unrollIn(graph->block(), false); }
+bool UnrollSimpleMaps(std::shared_ptr<Graph> graph) { return unrollIn(graph->block(), true); }
+
+// ---------------------------------------------------------------------------
 // SplitParallelMaps (fait/passes/parallelize_loops.cpp:152-293): a map whose body holds
 // fusion groups next to other nodes is cut so that every group is alone in a map (one launch
 // for all tasks); what lies between the groups gets maps of its own, which ToParallelFunctor
@@ -750,6 +866,16 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   CollapseAssignLoops(graph);
   ParallelizeLoops(graph);
   FuseOps(graph);
+  // what did not fuse inside short dependent loops and parameter-only maps is written out and
+  // gets a second chance across iterations (fait_pipeline.cpp:52-55)
+  const bool unrolled_loops = UnrollLoopsWithDeps(graph);
+  const bool unrolled_maps = UnrollSimpleMaps(graph);
+  if (unrolled_loops || unrolled_maps) {
+    ConstantPropagation(graph);
+    EliminateCommonSubexpression(graph);
+    EliminateDeadCode(graph);
+    FuseOps(graph);
+  }
   FuseMaskedSelect(graph);
   SplitParallelMaps(graph);
   ToParallelFunctor(graph);

@@ -27,6 +27,8 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
   m.def("_jit_pass_parallelize_loops", ParallelizeLoops);
   m.def("_jit_pass_split_parallel_maps", SplitParallelMaps);
+  m.def("_jit_pass_unroll_loops_with_deps", UnrollLoopsWithDeps);
+  m.def("_jit_pass_unroll_simple_maps", UnrollSimpleMaps);
   m.def("_jit_pass_fuse_masked_select", FuseMaskedSelect);
   m.def("_jit_pass_to_parallel_functor", ToParallelFunctor);
   m.def("_jit_pass_fait_pipeline", FaitPipeline);

@@ -27,6 +27,9 @@ void CollapseAssignLoops(std::shared_ptr<torch::jit::Graph> graph);
 void ParallelizeLoops(std::shared_ptr<torch::jit::Graph> graph);
 // fait/passes/parallelize_loops.cpp:152-293: every fusion group of a map body gets a map of its own
 void SplitParallelMaps(std::shared_ptr<torch::jit::Graph> graph);
+// fait/passes/unroll_loops.cpp:11-77, parallelize_loops.cpp:372-456; true if the graph changed
+bool UnrollLoopsWithDeps(std::shared_ptr<torch::jit::Graph> graph);
+bool UnrollSimpleMaps(std::shared_ptr<torch::jit::Graph> graph);
 
 // Fold `x[mask]` consumers of a FusionGroup into the group when the bool mask is
 // produced by the same group (row compaction fused into the region).  The

@@ -137,6 +137,63 @@ def test_split_map_runs_on_gpu():
         torch.testing.assert_close(g.cpu(), w, rtol=1e-5, atol=1e-6)
 
 
+def _dependent_loop(x: torch.Tensor, y: torch.Tensor):
+    for i in range(3):
+        x = x + y[i]      # one working operator: the body alone is not worth a region
+    return x
+
+
+def test_short_dependent_loop_is_unrolled_and_fused():
+    """UnrollLoopsWithDeps (fait/passes/unroll_loops.cpp:11-77): a constant-trip loop with a
+    carried value whose body did not fuse is written out; the second FuseOps makes one region
+    of the three iterations."""
+    f = fj.build(fj.script(_dependent_loop), [torch.rand(8), torch.rand(3, 8)])
+    kinds = _kinds(f.graph)
+    assert "prim::Loop" not in kinds and kinds.count("tssa::ParallelFunctor") == 1
+    sub = _functors(f.graph)[0].g("Subgraph")
+    assert [n.kind() for n in sub.nodes()].count("aten::add") == 3
+
+
+def test_long_or_dynamic_loops_are_not_unrolled():
+    def prog(x: torch.Tensor, y: torch.Tensor, n: int):
+        for i in range(n):
+            x = x * 0.5 + y[i]
+        return x
+
+    g = fj.script(prog).graph.copy()
+    assert not _C._jit_pass_unroll_loops_with_deps(g)
+    assert "prim::Loop" in _kinds(g)
+
+
+def test_unroll_simple_maps():
+    """UnrollSimpleMaps (fait/passes/parallelize_loops.cpp:372-456): a constant-trip map that
+    only computes from its index and constants is written out."""
+    def prog(x: torch.Tensor):
+        out = []
+        for i in range(3):
+            out.append(torch.ones(4) * float(i) + 1.0)
+        return out
+
+    g = fj.script(prog).graph.copy()
+    _C._jit_pass_parallelize_loops(g)
+    assert "prim::ParallelMap" in _kinds(g)
+    assert _C._jit_pass_unroll_simple_maps(g)
+    kinds = _kinds(g)
+    assert "prim::ParallelMap" not in kinds and kinds.count("aten::mul") == 3
+    _C._jit_pass_validate(g)
+    got = _C._create_function_from_graph("unrolled", g)(torch.zeros(1))
+    assert [t.tolist() for t in got] == [[1.0] * 4, [2.0] * 4, [3.0] * 4]
+
+
+@pytest.mark.gpu
+def test_unrolled_loop_runs_on_gpu():
+    gen = torch.Generator().manual_seed(5)
+    x, y = torch.rand(257, generator=gen), torch.rand(3, 257, generator=gen)
+    want = _dependent_loop(x.clone(), y)
+    f = fj.build(fj.script(_dependent_loop), [x, y])
+    torch.testing.assert_close(f(x.cuda(), y.cuda()).cpu(), want, rtol=1e-6, atol=0)
+
+
 def test_single_elementwise_op_is_left_to_aten():
     def prog(x: torch.Tensor):
         return x.sigmoid()

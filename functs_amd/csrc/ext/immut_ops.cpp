@@ -69,6 +69,26 @@ Tensor expand_as(Tensor src, Tensor other) { return src.expand_as(other); }
 Tensor repeat(Tensor self, at::IntArrayRef sizes) { return self.repeat(sizes); }
 Tensor index(Tensor src, c10::List<std::optional<Tensor>> indices) { return src.index(indices); }
 
+// The three operators below are in the reference's registry (symbol_ext.cpp:83-111, 176-195)
+// but none of its passes emits them.  The bodies give the results the reference's bodies give,
+// on a fresh tensor instead of through `self`.
+Tensor expand_rev(Tensor src, at::IntArrayRef sizes, bool implicit) { return src.expand(sizes, implicit); }
+// reference: self.repeat(sizes).copy_(src) writes into the temporary that repeat returns, so
+// the result is `self` as it was
+Tensor repeat_rev(Tensor self, Tensor src, at::IntArrayRef sizes) {
+  TORCH_CHECK(at::is_expandable_to(src.sizes(), self.repeat(sizes).sizes()),
+              "immut::repeat_rev: src does not broadcast to self.repeat(size)");
+  return self.clone();
+}
+// reference: self.expand_as(other).copy_(src); ATen refuses the copy as soon as the view
+// really expands (one element would be written more than once)
+Tensor expand_as_rev(Tensor self, Tensor src, Tensor other) {
+  TORCH_CHECK(self.sizes() == other.sizes(),
+              "immut::expand_as_rev: more than one element of the written-to tensor refers to a single memory "
+              "location (self ", self.sizes(), " expanded as ", other.sizes(), ")");
+  return src.expand_as(self).to(self.scalar_type()).contiguous();
+}
+
 }  // namespace
 
 // immut:: schemas as functs/csrc/jit/ir/symbol_ext.cpp:9-199 registers them; no alias
@@ -91,6 +111,9 @@ TORCH_LIBRARY(immut, m) {
   m.def("expand_as(Tensor self, Tensor other) -> Tensor", expand_as);
   m.def("repeat(Tensor self, int[] size) -> Tensor", repeat);
   m.def("index.Tensor(Tensor self, Tensor?[] indices) -> Tensor", index);
+  m.def("expand_rev(Tensor self, int[] size, *, bool implicit=False) -> Tensor", expand_rev);
+  m.def("repeat_rev(Tensor self, Tensor src, int[] size) -> Tensor", repeat_rev);
+  m.def("expand_as_rev(Tensor self, Tensor src, Tensor other) -> Tensor", expand_as_rev);
 }
 
 }  // namespace functs

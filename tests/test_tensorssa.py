@@ -192,3 +192,19 @@ def test_loop_carries_the_mutated_buffer():
     body = next(loops[0].blocks())
     ret = list(body.outputs())
     assert any(v.node().kind() == "immut::select_rev" for v in ret)
+
+
+def test_registered_but_unused_rev_operators():
+    """immut::expand_rev / repeat_rev / expand_as_rev are registered by the reference
+    (functs/csrc/jit/ir/symbol_ext.cpp:83-111) and emitted by none of its passes; the bodies
+    give the reference's results without touching `self`."""
+    x = torch.arange(6.0).reshape(2, 3)
+    assert torch.equal(torch.ops.immut.expand_rev(x[:1], [2, 3]), x[:1].expand(2, 3))
+    keep = x.clone()
+    out = torch.ops.immut.repeat_rev(x, torch.ones(4, 3), [2, 1])
+    assert torch.equal(out, keep) and torch.equal(x, keep) and out.data_ptr() != x.data_ptr()
+    src = torch.full((3,), 7.0)
+    out = torch.ops.immut.expand_as_rev(x, src, torch.zeros(2, 3))
+    assert torch.equal(out, src.expand(2, 3)) and torch.equal(x, keep)
+    with pytest.raises(RuntimeError, match="single memory location"):
+        torch.ops.immut.expand_as_rev(x[:1], torch.ones(2, 3), torch.zeros(2, 3))

@@ -15,7 +15,7 @@ the scripted program whose fused regions run as tssa::ParallelFunctor;
 `region_api_latency_us` is the same regions driven from Python through ctypes;
 `compiled_kernels` says whether the regions ran ahead-of-time compiled kernels
 (functs_amd.aot) or the bytecode interpreter (`--interpreter` forces the latter);
-`per_config` repeats the measurement for every BASELINE.json config that is
+`per_config` repeats the measurement for every benchmark configuration that is
 implemented.  `roofline` prices the dominant kernel against the 8 TB/s
 HBM peak with the algorithmic bytes of the call; `cpu_baseline` times the
 unfused TorchScript CPU path (the oracle) on a bounded sample.
@@ -201,8 +201,8 @@ def main():
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        raise SystemExit("bench.py: this path runs on ONE GPU (its tasks are independent; see DESIGN.md for how it "
-                         "would shard). Run with --gpus 1.")
+        raise SystemExit("bench.py: this path runs on ONE GPU. Its map tasks and row ranges are independent and "
+                         "would shard over GPUs without exchange, but that is not built. Run with --gpus 1.")
     import torch
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs an MI355X (no CPU fallback exists)")
@@ -286,7 +286,7 @@ def main():
                 "frac_hbm_peak": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 5)}
 
     def run_stream():
-        """Not a BASELINE config: one big fused elementwise region (sigmoid(2x + 1) on
+        """Not one of the five configurations: one big fused elementwise region (sigmoid(2x + 1) on
         [8192, 4096] fp32), the shape on which the dense kernel itself meets the HBM roofline."""
         from functs_amd import Region
         x = torch.rand(8192, 4096, device=dev)

@@ -353,3 +353,35 @@ def test_hip_graph_refuses_row_compaction():
     args = oc.c2_inputs(0, SMALL_GRIDS)
     with pytest.raises(ValueError, match="row-compacting"):
         fj.build(fj.script(oc.c2_fn), list(args), hip_graph=True)
+
+
+@pytest.mark.gpu
+def test_back_to_back_calls_with_changing_inputs():
+    """The operator returns when the kept-row counts are known, before its kernels end, so
+    consecutive calls overlap on the stream and reuse scratch and the pinned count buffer.
+    Alternating inputs with different kept rows must never show a stale size or stale rows."""
+    import functs_amd.jit as fj
+    from functs_amd.benchmark import PROGRAMS
+    from functs_amd.benchmark.inputs import INPUTS
+    dev = torch.device("cuda:0")
+    a = INPUTS["c5"](0)
+    b = INPUTS["c5"](1)
+    fn = fj.build(fj.script(PROGRAMS["c5"]), list(a))
+    ga = [t.to(dev) for t in a]
+    gb = [t.to(dev) for t in b]
+    want = {}
+    for key, args in (("a", ga), ("b", gb)):
+        out = fn(*args)
+        torch.cuda.synchronize()
+        want[key] = [[t.clone() for t in lst] for lst in out]
+    assert [t.shape for t in want["a"][0]] != [t.shape for t in want["b"][0]]
+    pending = []
+    for it in range(120):
+        key, args = (("a", ga), ("b", gb))[it % 2]
+        pending.append((key, fn(*args)))          # no synchronisation between calls
+    torch.cuda.synchronize()
+    for key, out in pending:
+        for lst, ref in zip(out, want[key]):
+            assert len(lst) == len(ref)
+            for t, r in zip(lst, ref):
+                assert t.shape == r.shape and torch.equal(t, r)

@@ -8,17 +8,17 @@
 //                       map in LDS, region programs evaluated only for kept
 //                       rows, results written densely in source order).
 //
-// The three kernels share one bytecode interpreter (fx_run).  A workgroup
-// first copies the whole region descriptor (programs, affine maps, output
-// descriptors, task classes) and the per-call pointer / scalar tables of all
-// tasks into LDS with one round of coalesced 128-bit loads; from then on every
-// table access is an LDS broadcast read, so no dependent chain of cold global
-// loads sits in front of the data traffic.  Instruction decode is
-// wave-uniform (the opcode word goes through readfirstlane, the switch is a
-// scalar branch); every instruction then operates on FX_V elements per lane,
-// laid out so that lane l of a workgroup handles elements l, l+256, l+512,
-// l+768 of its tile: each global load/store instruction of a wave covers 256
-// contiguous bytes.
+// The kernels are templates (fx_device.h) over the way a program is run: this file
+// instantiates them with the bytecode interpreter (fx_run); spec/*.hip instantiate them with
+// the programs of one region as compile-time constants (fx_spec.h).  A workgroup first copies
+// the whole region descriptor (programs, affine maps, output descriptors, task classes) and the
+// per-call pointer / scalar tables of all tasks into LDS with one round of coalesced 128-bit
+// loads; from then on every table access is an LDS broadcast read, so no dependent chain of
+// cold global loads sits in front of the data traffic.  Instruction decode is wave-uniform
+// (the opcode word goes through readfirstlane, the switch is a scalar branch); every
+// instruction then operates on FX_V consecutive elements per lane along the last output
+// dimension: a contiguous source is read with one 128-bit load per lane and results are written
+// with one 128-bit store, so a global access of a wave covers 1 KB of contiguous memory.
 //
 // Replaces the NVRTC-generated kernels of the reference
 // (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121, launch shape

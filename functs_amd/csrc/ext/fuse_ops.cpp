@@ -75,6 +75,15 @@ bool listOfFusableElems(Node* n) {
 
 bool isFusableNode(Node* node) {
   if (listOfFusableElems(node)) return true;
+  // taking a tuple of scalars apart (e.g. the (h, w) of an image in a List[Tuple[int, int]]):
+  // the tuple becomes an argument of the region, its elements scalar inputs
+  if (node->kind() == c10::prim::TupleUnpack) {
+    for (Value* o : node->outputs()) {
+      const auto k = o->type()->kind();
+      if (k != c10::TypeKind::IntType && k != c10::TypeKind::FloatType && k != c10::TypeKind::BoolType) return false;
+    }
+    return true;
+  }
   if (!fusableSymbols().count(node->kind())) return false;
   if (node->kind() != sym::ForallSelectRev() && !node->blocks().empty()) return false;
   // scalar arithmetic that shares a symbol with a tensor operator stays outside

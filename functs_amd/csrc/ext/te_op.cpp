@@ -373,21 +373,52 @@ class RegionRunner {
       else TORCH_CHECK(false, "ParallelFunctor: unsupported scalar argument ", v.tagKind());
       args.push_back(a);
     };
+    // A value that is itself a list or tuple of scalars (int[], float[], bool[], Tuple[int, ...];
+    // per task: List[List[int]], List[Tuple[int, int]] ..., graph_builder.cpp:736-857) travels as
+    // its elements; their number is part of the signature.  All tasks must agree on it.
+    auto addValue = [&](const c10::IValue& v, size_t k, int64_t* n_elems) {
+      if (v.isTensor()) { addTensor(v.toTensor()); return; }
+      if (v.isList() || v.isTuple()) {
+        const auto elems = v.isList() ? v.toListRef() : at::ArrayRef<c10::IValue>(v.toTupleRef().elements());
+        TORCH_CHECK(*n_elems < 0 || *n_elems == (int64_t)elems.size(), "ParallelFunctor: argument ", k,
+                    ": the tasks' lists differ in length");
+        if (*n_elems < 0) sig << "|L" << elems.size();
+        *n_elems = (int64_t)elems.size();
+        for (const c10::IValue& e : elems) {
+          TORCH_CHECK(!e.isTensor() && !e.isList() && !e.isTuple(), "ParallelFunctor: argument ", k,
+                      ": nested lists of this kind are not supported");
+          addScalar(e);
+        }
+        return;
+      }
+      addScalar(v);
+    };
     for (size_t k = 0; k < n_args_; ++k) {
       const c10::IValue& v = inputs[first + k];
       const bool per_task = is_map_ && is_par_[k] != 0;
+      int64_t n_elems = -1;
       if (per_task) {
         TORCH_CHECK(v.isList(), "ParallelFunctor: argument ", k, " must be a list with one entry per task");
         auto lst = v.toListRef();
         TORCH_CHECK((int64_t)lst.size() >= degree, "ParallelFunctor: list argument ", k, " is shorter than the trip count");
-        for (int64_t t = 0; t < degree; ++t) {
-          if (lst[t].isTensor()) addTensor(lst[t].toTensor());
-          else addScalar(lst[t]);
+        // element-major: all tasks' first elements, then all second elements ... (one region input each)
+        if (degree > 0 && (lst[0].isList() || lst[0].isTuple())) {
+          const auto first_elems = lst[0].isList() ? lst[0].toListRef() : at::ArrayRef<c10::IValue>(lst[0].toTupleRef().elements());
+          const size_t n = first_elems.size();
+          sig << "|L" << n;
+          for (size_t e = 0; e < n; ++e)
+            for (int64_t t = 0; t < degree; ++t) {
+              const auto elems = lst[t].isList() ? lst[t].toListRef() : at::ArrayRef<c10::IValue>(lst[t].toTupleRef().elements());
+              TORCH_CHECK(elems.size() == n, "ParallelFunctor: argument ", k, ": the tasks' lists differ in length");
+              TORCH_CHECK(!elems[e].isTensor() && !elems[e].isList() && !elems[e].isTuple(), "ParallelFunctor: argument ",
+                          k, ": nested lists of this kind are not supported");
+              addScalar(elems[e]);
+            }
+        } else {
+          for (int64_t t = 0; t < degree; ++t) addValue(lst[t], k, &n_elems);
         }
-      } else if (v.isTensor()) {
-        addTensor(v.toTensor());
       } else {
-        addScalar(v);
+        addValue(v, k, &n_elems);
       }
     }
     TORCH_CHECK(have_device, "ParallelFunctor: a region needs at least one tensor argument");
@@ -497,6 +528,8 @@ class RegionRunner {
 struct Translator {
   fx_region* r;
   std::unordered_map<const Value*, int> ids;
+  // list- or tuple-valued subgraph parameters: the region inputs that carry their elements
+  std::unordered_map<const Value*, std::vector<int>> elements;
 
   int cint(int64_t v) { int id; FX_OK_OR_THROW(fx_region_const_int(r, v, &id)); return id; }
   int cfloat(double v) { int id; FX_OK_OR_THROW(fx_region_const_float(r, v, &id)); return id; }
@@ -554,6 +587,22 @@ void Translator::node(const Node* n) {
   if (k == prim::Constant) return;  // created on demand
   if (k == aten::size && ni == 1) {  // all sizes: the tensor itself stands for them
     out(in(0));
+    return;
+  }
+  if (k == prim::TupleUnpack || k == prim::ListUnpack) {
+    auto it = elements.find(n->input(0));
+    TORCH_CHECK(it != elements.end() && it->second.size() == n->outputs().size(),
+                "ParallelFunctor: ", k.toQualString(), " of a value that is not a region argument");
+    for (size_t i = 0; i < n->outputs().size(); ++i) ids[n->output(i)] = it->second[i];
+    return;
+  }
+  if (k == aten::__getitem__ && elements.count(n->input(0))) {  // list[const]
+    auto idx = constant_as<int64_t>(n->input(1));
+    const auto& e = elements.at(n->input(0));
+    TORCH_CHECK(idx, "ParallelFunctor: a list argument can only be read at a constant position inside a region");
+    const int64_t i = *idx < 0 ? *idx + (int64_t)e.size() : *idx;
+    TORCH_CHECK(i >= 0 && i < (int64_t)e.size(), "ParallelFunctor: list index out of range");
+    out(e[(size_t)i]);
     return;
   }
   if (k == prim::ListConstruct) {
@@ -703,12 +752,29 @@ void RegionRunner::build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue>
     c10::IValue sample = v;
     if (per_task) sample = v.toListRef().at(0);
     int id;
+    auto scalarInput = [&](const c10::IValue& e) {
+      int sid;
+      const int kind = e.isDouble() ? 2 : (e.isBool() ? 3 : 1);
+      FX_OK_OR_THROW(fx_region_input_scalar(var.region, kind, per_task, &sid));
+      return sid;
+    };
     if (sample.isTensor()) {
       const at::Tensor& t = sample.toTensor();
       FX_OK_OR_THROW(fx_region_input_tensor(var.region, fxDtype(t.scalar_type()), (int)t.dim(), per_task, &id));
+    } else if (sample.isList() || sample.isTuple()) {
+      // one scalar input per element; an int[] becomes a size list, a tuple waits for its TupleUnpack
+      const auto elems = sample.isList() ? sample.toListRef() : at::ArrayRef<c10::IValue>(sample.toTupleRef().elements());
+      std::vector<int> eids;
+      bool ints = true;
+      for (const c10::IValue& e : elems) {
+        eids.push_back(scalarInput(e));
+        ints = ints && e.isInt();
+      }
+      tr.elements[p] = eids;
+      if (sample.isList() && ints) tr.ids[p] = tr.ilist(eids);
+      continue;
     } else {
-      int kind = sample.isDouble() ? 2 : (sample.isBool() ? 3 : 1);
-      FX_OK_OR_THROW(fx_region_input_scalar(var.region, kind, per_task, &id));
+      id = scalarInput(sample);
     }
     tr.ids[p] = id;
   }

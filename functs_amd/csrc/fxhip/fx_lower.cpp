@@ -12,6 +12,9 @@
 
 namespace fx {
 
+// thrown by the lowering when it meets a per-task int input in shape or index arithmetic
+struct NeedIndexInt { int input; };
+
 #define FX_CHECK(cond, code, msg)                        \
   do {                                                   \
     if (!(cond)) {                                       \
@@ -363,7 +366,10 @@ IdxExpr Lowerer::intOf(int vid) {
       return loopVar_;
     case P_INPUT: {
       FX_CHECK(v.kind == VK_INT || v.kind == VK_BOOL, FX_E_INVALID, "expected an int input");
-      FX_CHECK(!v.per_task, FX_E_UNSUPPORTED, "per-task int scalars cannot drive index arithmetic");
+      // a per-task int that shapes or indices depend on: its values must be part of the plan key
+      // and tasks with different values need programs of their own (plan_region starts over)
+      if (v.per_task && !(v.input_index < (int)R_.index_ints.size() && R_.index_ints[v.input_index]))
+        throw NeedIndexInt{v.input_index};
       return IdxExpr(in_[v.input_index]->ival);
     }
     case P_OP:
@@ -1671,7 +1677,22 @@ static void fillDims(FxOut& o, const Shape& s) {
 // ---------------------------------------------------------------------------
 // plan construction
 // ---------------------------------------------------------------------------
+static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args);
+
 const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
+  R.index_ints.resize(R.inputs.size(), 0);
+  for (;;) {
+    try {
+      return plan_region_once(R, args, n_args);
+    } catch (const NeedIndexInt& need) {
+      FX_CHECK(need.input >= 0 && need.input < (int)R.index_ints.size() && !R.index_ints[need.input], FX_E_INVALID,
+               "per-task int input " << need.input << " cannot be resolved");
+      R.index_ints[need.input] = 1;
+    }
+  }
+}
+
+static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   FX_CHECK(R.finalized, FX_E_INVALID, "region is not finalized");
   const int T = R.degree;
   // argument layout
@@ -1698,7 +1719,7 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
       } else {
         FX_CHECK(a.kind != 0, FX_E_INVALID, "argument " << arg_base[i] + t << " must be a scalar");
         key.push_back(-7);
-        if ((v.kind == VK_INT || v.kind == VK_BOOL) && !v.per_task) key.push_back(a.ival);
+        if ((v.kind == VK_INT || v.kind == VK_BOOL) && (!v.per_task || R.index_ints[i])) key.push_back(a.ival);
       }
     }
   }
@@ -1736,8 +1757,12 @@ const Plan* plan_region(Region& R, const fx_arg* args, int n_args) {
   for (int t = 0; t < T; ++t)
     for (size_t i = 0; i < R.inputs.size(); ++i) {
       const Value& v = R.vals[R.inputs[i]];
-      if (!v.per_task || v.kind != VK_TENSOR) continue;
+      if (!v.per_task) continue;
       const fx_arg& a = args[arg_base[i] + t];
+      if (v.kind != VK_TENSOR) {
+        if (R.index_ints[i]) tkey[t].push_back(a.ival);
+        continue;
+      }
       for (int d = 0; d < a.rank; ++d) { tkey[t].push_back(a.sizes[d]); tkey[t].push_back(a.strides[d]); }
     }
   std::vector<ClassBuild> classes;

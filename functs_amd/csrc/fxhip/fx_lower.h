@@ -52,6 +52,10 @@ struct Region {
   std::vector<int> inputs;   // value ids, declaration order
   std::vector<int> outputs;  // value ids
   int mask = -1;             // row-compaction mask value id
+  // per-task int inputs (by input index) whose values shapes or index arithmetic depend on:
+  // found out while lowering; their values are part of the plan key and split the tasks
+  // into classes (all other per-task scalars are plain run-time data)
+  std::vector<char> index_ints;
   std::map<std::vector<int64_t>, std::unique_ptr<Plan>> plans;
 
   int add(const Value& v) {

@@ -31,7 +31,7 @@ const std::unordered_set<Symbol>& fusableSymbols() {
       aten::clone, aten::contiguous, aten::to, aten::zeros, aten::ones, aten::full, aten::full_like, aten::zeros_like,
       aten::ones_like, aten::arange, aten::tensor, aten::exp, aten::sigmoid, aten::tanh, aten::relu, aten::neg,
       aten::abs, aten::sqrt, aten::rsqrt, aten::log, aten::reciprocal, aten::floor, aten::ceil, aten::round,
-      aten::sin, aten::cos, aten::erf, aten::triu, aten::clamp, aten::add, aten::sub, aten::rsub, aten::mul,
+      aten::sin, aten::cos, aten::erf, aten::triu, aten::tril, aten::clamp, aten::add, aten::sub, aten::rsub, aten::mul,
       aten::div, aten::minimum, aten::maximum, aten::pow, aten::__and__, aten::__or__, aten::__xor__,
       aten::logical_not, aten::eq, aten::ne, aten::lt, aten::le, aten::gt, aten::ge, aten::where, aten::max,
       aten::softmax, aten::select, aten::slice, aten::squeeze, aten::unsqueeze, aten::reshape, aten::view,
@@ -49,7 +49,7 @@ const std::unordered_set<Symbol>& workingSymbols() {
   using namespace c10;
   static const std::unordered_set<Symbol> s{
       aten::arange, aten::zeros, aten::to, aten::contiguous, aten::exp, aten::sigmoid, aten::tanh, aten::relu,
-      aten::clamp, aten::triu, aten::add, aten::sub, aten::rsub, aten::mul, aten::div, aten::__and__, aten::__or__,
+      aten::clamp, aten::triu, aten::tril, aten::add, aten::sub, aten::rsub, aten::mul, aten::div, aten::__and__, aten::__or__,
       aten::minimum, aten::maximum, aten::eq, aten::ne, aten::lt, aten::le, aten::gt, aten::ge, aten::where,
       aten::max, aten::softmax, aten::repeat, aten::cat, aten::stack, aten::index, aten::neg, aten::abs,
       aten::sqrt, aten::log, aten::pow, sym::Assign(), sym::Select(), sym::SelectRev(), sym::Slice(),

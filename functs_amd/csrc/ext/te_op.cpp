@@ -673,6 +673,7 @@ void Translator::node(const Node* n) {
   if (k == aten::cat) { out(op(FX_OP_CAT, {in(0), in(1)})); return; }
   if (k == aten::stack) { out(op(FX_OP_STACK, {in(0), in(1)})); return; }
   if (k == aten::triu) { out(op(FX_OP_TRIU, {in(0), in(1)})); return; }
+  if (k == aten::tril) { out(op(FX_OP_TRIL, {in(0), in(1)})); return; }
   if (k == aten::clamp) { out(op(FX_OP_CLAMP, {in(0), in(1), in(2)})); return; }
   if (k == aten::where) { out(op(FX_OP_WHERE, {in(0), in(1), in(2)})); return; }
   if (k == aten::softmax) { out(op(FX_OP_SOFTMAX, {in(0), in(1)})); return; }

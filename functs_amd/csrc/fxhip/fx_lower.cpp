@@ -86,7 +86,7 @@ int Region::addOp(int opcode, const std::vector<int>& args, int out_dtype) {
   switch (opcode) {
     case FX_OP_ACCESS: case FX_OP_CLONE: case FX_OP_SELECT: case FX_OP_SLICE: case FX_OP_SQUEEZE:
     case FX_OP_UNSQUEEZE: case FX_OP_VIEW: case FX_OP_PERMUTE: case FX_OP_TRANSPOSE: case FX_OP_EXPAND:
-    case FX_OP_EXPAND_AS: case FX_OP_REPEAT: case FX_OP_INDEX: case FX_OP_TRIU: case FX_OP_CAT:
+    case FX_OP_EXPAND_AS: case FX_OP_REPEAT: case FX_OP_INDEX: case FX_OP_TRIU: case FX_OP_TRIL: case FX_OP_CAT:
     case FX_OP_STACK: case FX_OP_SELECT_REV: case FX_OP_SLICE_REV: case FX_OP_FORALL_SELECT_REV:
     case FX_OP_NEG: case FX_OP_ABS: case FX_OP_RELU: case FX_OP_CLAMP: case FX_OP_MAX_DIM:
     case FX_OP_FLOOR: case FX_OP_CEIL: case FX_OP_ROUND:
@@ -481,7 +481,8 @@ Shape Lowerer::shapeOf(int vid) {
   } else {
     auto arg = [&](int i) { return v.args.at(i); };
     switch (v.op) {
-      case FX_OP_ACCESS: case FX_OP_CLONE: case FX_OP_TRIU: case FX_OP_TO: case FX_OP_EXP: case FX_OP_LOG:
+      case FX_OP_ACCESS: case FX_OP_CLONE: case FX_OP_TRIU: case FX_OP_TRIL: case FX_OP_TO: case FX_OP_EXP:
+      case FX_OP_LOG:
       case FX_OP_SQRT: case FX_OP_RSQRT: case FX_OP_SIGMOID: case FX_OP_TANH: case FX_OP_RELU: case FX_OP_NEG:
       case FX_OP_ABS: case FX_OP_FLOOR: case FX_OP_CEIL: case FX_OP_ROUND: case FX_OP_SIN: case FX_OP_COS:
       case FX_OP_ERF: case FX_OP_RECIPROCAL: case FX_OP_LOGICAL_NOT: case FX_OP_CLAMP: case FX_OP_SOFTMAX:
@@ -1358,6 +1359,20 @@ void Lowerer::emitOp(const Res& r) {
       uint32_t zero = 0;
       if (hi < diag) { emitI(FX_IMMA, 0, 0, zero); finish(); return; }
       emitCond(x, diag, (int64_t)1 << 40, 1, [&] { emitAs(arg(0), f, own); }, [&] { emitI(FX_IMMA, 0, 0, zero); });
+      finish();
+      return;
+    }
+    case FX_OP_TRIL: {
+      // the mirror image of triu: element (i, j) survives where j - i <= diagonal
+      FX_CHECK(f.size() >= 2, FX_E_INVALID, "tril needs rank >= 2");
+      int64_t diag = constIntOf(arg(1), "tril diagonal");
+      IdxExpr x = f[f.size() - 1] - f[f.size() - 2];
+      int64_t lo, hi;
+      range(x, &lo, &hi);
+      if (hi <= diag) { emitAs(arg(0), f, own); finish(); return; }
+      uint32_t zero = 0;
+      if (lo > diag) { emitI(FX_IMMA, 0, 0, zero); finish(); return; }
+      emitCond(x, -((int64_t)1 << 40), diag + 1, 1, [&] { emitAs(arg(0), f, own); }, [&] { emitI(FX_IMMA, 0, 0, zero); });
       finish();
       return;
     }

@@ -99,6 +99,7 @@ enum fx_opcode {
    * built with fx_region_loop_var() standing for i.  No reference counterpart:
    * the reference keeps such loops serial (parallelize_loops.cpp:17). */
   FX_OP_FORALL_SELECT_REV,
+  FX_OP_TRIL,         /* (self, int diagonal)                    fusable in fait/passes/fuse_ops.cpp:57 */
   FX_OP__COUNT
 };
 

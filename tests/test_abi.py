@@ -20,7 +20,7 @@ def test_exports_every_declared_symbol():
 def test_version_and_constants():
     assert lib.fx_api_version() == C["FX_API_VERSION"] == 1
     assert C["FX_OP_ACCESS"] == 1
-    assert C["FX_OP_FORALL_SELECT_REV"] + 1 == C["FX_OP__COUNT"]
+    assert C["FX_OP_TRIL"] + 1 == C["FX_OP__COUNT"]  # new opcodes are appended: numbers of the ABI never move
 
 
 def test_header_cites_reference_lines():

@@ -90,3 +90,15 @@ def test_lists_of_different_lengths_are_refused():
     f = fj.build(fj.script(per_task_size_lists), [_rand(3, 12), [[3, 4], [2, 6], [4, 3]]])
     with pytest.raises(RuntimeError, match="differ in length"):
         f(_rand(3, 12).cuda(), [[3, 4], [12], [4, 3]])
+
+
+def causal_scores(q: torch.Tensor):
+    return torch.tril(q * 2.0 + 1.0, 0).exp()
+
+
+@pytest.mark.gpu
+def test_tril_through_the_torchscript_route():
+    x = _rand(6, 6)
+    f = fj.build(fj.script(causal_scores), [x])
+    assert [n.kind() for n in f.graph.nodes()].count("tssa::ParallelFunctor") == 1
+    torch.testing.assert_close(f(x.cuda()).cpu(), causal_scores(x), rtol=1e-5, atol=1e-6)

@@ -414,3 +414,21 @@ def test_int_and_bool_dtypes(backend):
     tb = torch.randint(0, 2, (17, 9), generator=g).bool()
     got = run_region(backend, r, ta, tb)
     assert_exact(got, [ta + 3, ta * ta - 1, ~tb, ta.to(torch.float32) * 0.5])
+
+
+def test_tril_and_triu_over_every_diagonal(backend):
+    """aten::tril / aten::triu are both fusable in the reference (fait/passes/fuse_ops.cpp:57-58);
+    the library routine is the pin: every diagonal of a non-square matrix, batched."""
+    t = (torch.arange(2 * 5 * 7, dtype=torch.float32) + 1).reshape(2, 5, 7)
+    diags = list(range(-6, 9))
+    r = Region()
+    x = r.tensor_input(torch.float32, 3)
+    for d in diags:
+        r.output(r.op("TRIL", x, d))
+        r.output(r.op("TRIU", x, d))
+    r.finalize()
+    got = run_region(backend, r, t)
+    refs = []
+    for d in diags:
+        refs += [torch.tril(t, d), torch.triu(t, d)]
+    assert_exact(got, refs, "tril/triu")

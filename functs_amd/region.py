@@ -320,6 +320,7 @@ class BoundCall:
         self.ptrs = ptrs
         self.scratch = torch.empty(max(plan.scratch_bytes, 1), dtype=torch.uint8, device=dev) if plan.compact else None
         self.totals = torch.zeros(T, dtype=torch.int32).pin_memory() if plan.compact else None
+        self._stream = None
 
     def launch(self, stream=None):
         if stream is None:
@@ -351,7 +352,8 @@ class BoundCall:
         early (ATen's nonzero waits for the whole stream); the outputs are valid in
         stream order."""
         if self.plan.compact:
-            check(lib.fx_region_wait_totals(self.plan.handle, self.totals.data_ptr(), ctypes.c_void_p(self._stream)))
+            stream = self._stream if self._stream is not None else torch.cuda.current_stream(self.device).cuda_stream
+            check(lib.fx_region_wait_totals(self.plan.handle, self.totals.data_ptr(), ctypes.c_void_p(stream)))
             totals = self.totals.tolist()
             outs = [[ten.narrow(0, 0, totals[t]) for t, ten in enumerate(row)] for row in self.outs]
         else:

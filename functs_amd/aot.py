@@ -87,6 +87,8 @@ def _run_benchmark_programs(names):
         elif name == "c3":
             decoded = configs.build_c3_decode()(*on_gpu(cpu_args))
             configs.build_c3_classes(80)(*decoded)
+    if "coverage" in names or len(names) == len(INPUTS):
+        configs.build_column_standardize()(torch.rand(*configs.COLUMN_STANDARDIZE_SHAPE, device=dev))
     if "stream" in names or len(names) == len(INPUTS):
         x = torch.rand(8192, 4096, device=dev)
         r = Region()

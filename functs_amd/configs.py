@@ -109,3 +109,28 @@ def build_c3_classes(n_fg=80):
     r.output(sc)
     r.compact_rows(sc > 0.05)
     return r.finalize()
+
+
+# shape for which `python -m functs_amd.aot` compiles the region below (its reduction extents are
+# part of the programs, so the compiled kernels serve this shape only)
+COLUMN_STANDARDIZE_SHAPE = (777, 12)
+
+
+def build_column_standardize():
+    """Not one of the five configurations: a region that exercises what they do not, used to
+    keep the ahead-of-time compiled path honest (serial reduction loops, max over a dimension,
+    `where`, `cat` branches, a row softmax in the same launch)::
+
+        mean = x.sum(0) / n;  z = x - mean;  spread = z.abs().max(0)
+        out0 = where(z > 0, z, 0.1 * z) / (spread + 1)
+        out1 = cat([x[:, :2].exp(), x[:, 2:]], 1).softmax(1)
+    """
+    r = Region()
+    x = r.tensor_input(torch.float32, 2)
+    n = r.op("SIZE", x, 0)
+    mean = r.op("SUM_DIM", x, 0, False) / n
+    z = x - mean.unsqueeze(0)
+    spread = r.op("MAX_DIM", r.op("ABS", z), 0, False)
+    r.output(r.where(z > 0.0, z, z * 0.1) / (spread.unsqueeze(0) + 1.0))
+    r.output(r.cat([x.slice(1, 0, 2).exp(), x.slice(1, 2, None)], 1).softmax(1))
+    return r.finalize()

@@ -755,6 +755,10 @@ struct FxInterp {
   // order in which a wave of the compaction kernel walks the outputs: 0 = alternate waves
   // backwards, 1 = all forwards (narrow outputs first), 2 = all backwards
   static constexpr int kWalk = 0;
+  // waves per workgroup of the compaction kernel (its row tile stays FX_BLOCK rows) and the
+  // waves per SIMD that its register budget is set for
+  static constexpr uint32_t kWaves = FX_BLOCK / 64;
+  static constexpr uint32_t kOcc = 4;
   template <int N>
   static __device__ __forceinline__ void run_pure(const FxCtx& cx, int pc, int pc_end, uint32_t (&X)[N]) {
     fx_run_pure(cx, pc, pc_end, X);
@@ -852,6 +856,54 @@ __device__ __forceinline__ uint32_t fx_fastdiv(uint32_t n, uint32_t magic, uint3
   return (__umulhi(n, magic) + n) >> shift;
 }
 
+// A batch of KP items of a pure output whose rows are whole lane groups: rank 2, FX_V
+// consecutive 32-bit elements of one kept row per lane, no ragged group at the end of a
+// row, a unit-stride leading load.  Group g is row g / gprow of the tile's kept rows and
+// elements [FX_V * (g % gprow), +FX_V) of it, and it is element FX_V * g of the tile's
+// rows of the output, so an item costs one division by a constant, one row-map lookup and
+// one multiply instead of the general coordinate machinery.  Items past the end of the
+// tile have no live lane; dead lanes load the first elements of the source and store nothing.
+template <class S, uint32_t KP, uint32_t NW>
+__device__ __forceinline__ void fx_rows_batch(const FxCtx& cx, const FxLead& ld, const uint32_t* rowmap, uint32_t it0,
+                                              uint32_t lane, uint32_t n_groups, uint32_t gprow, uint32_t gr_magic,
+                                              uint32_t gr_shift, uint64_t op, uint32_t obase, int pb, int pe) {
+  uint32_t X[KP * FX_V], o0[KP], e0[KP];
+  bool live[KP];
+#pragma unroll
+  for (uint32_t k = 0; k < KP; ++k) {
+    const uint32_t g = (it0 + NW * k) * 64u + lane;
+    live[k] = g < n_groups;
+    const uint32_t gg = live[k] ? g : 0u;
+    const uint32_t r = fx_fastdiv(gg, gr_magic, gr_shift);   // < FX_BLOCK
+    const uint32_t c = gg - __umul24(r, gprow);                // gprow < 2^24 (checked by the caller)
+    const uint32_t row = rowmap[r];
+    const uint32_t off = (uint32_t)(ld.base + (int32_t)row * ld.cf[0]) + c * FX_V;
+    o0[k] = live[k] ? off : 0u;
+    e0[k] = gg * FX_V;
+  }
+  const FX_AS1 uint8_t* src = (const FX_AS1 uint8_t*)ld.p;
+#pragma unroll
+  for (uint32_t k = 0; k < KP; ++k) {
+    const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)(src + (o0[k] << 2));
+    X[k * FX_V + 0] = v.x; X[k * FX_V + 1] = v.y; X[k * FX_V + 2] = v.z; X[k * FX_V + 3] = v.w;
+  }
+  if (ld.cvt) {
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (uint32_t j = 0; j < KP * FX_V; ++j) X[j] = f2u((float)(int32_t)X[j]);
+  }
+  S::run_pure(cx, pb + 1, pe, X);
+  FX_AS1 uint8_t* dst = (FX_AS1 uint8_t*)op;
+#pragma unroll
+  for (uint32_t k = 0; k < KP; ++k) {
+    if (live[k]) {
+      fx_u32x4 v;
+      v.x = X[k * FX_V + 0]; v.y = X[k * FX_V + 1]; v.z = X[k * FX_V + 2]; v.w = X[k * FX_V + 3];
+      *(FX_AS1 fx_u32x4_a4*)(dst + ((obase + e0[k]) << 2)) = v;
+    }
+  }
+}
+
 // ---- workgroup prologue ----------------------------------------------------
 // LDS layout (words): [blob][pointers: 2 words each][scalars][pad][temps]
 struct FxLaunch {
@@ -864,10 +916,11 @@ struct FxLaunch {
 };
 #define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
 
+template <uint32_t NT = FX_BLOCK>
 __device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict__ sb, const FxLaunch& la) {
   const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)sb;
   fx_u32x4* l4 = (fx_u32x4*)L;
-  for (uint32_t i = threadIdx.x; i < la.blob_words / 4; i += FX_BLOCK) l4[i] = g4[i];
+  for (uint32_t i = threadIdx.x; i < la.blob_words / 4; i += NT) l4[i] = g4[i];
   // The by-value FxDyn block is read through the kernarg segment pointer (never
   // by naming the parameter: indexing a by-value aggregate dynamically would
   // make the compiler copy it to per-lane scratch).
@@ -876,8 +929,8 @@ __device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict
   const uint32_t* gs = (const uint32_t*)(ka + FX_KERNARG_DYN_OFF + 8 * FX_DYN_P);
   uint64_t* lp = (uint64_t*)(L + la.blob_words);
   uint32_t* ls = L + la.blob_words + 2 * la.n_p;
-  for (uint32_t i = threadIdx.x; i < la.n_p; i += FX_BLOCK) lp[i] = gp[i];
-  for (uint32_t i = threadIdx.x; i < la.n_s; i += FX_BLOCK) ls[i] = gs[i];
+  for (uint32_t i = threadIdx.x; i < la.n_p; i += NT) lp[i] = gp[i];
+  for (uint32_t i = threadIdx.x; i < la.n_s; i += NT) ls[i] = gs[i];
   __syncthreads();
 }
 
@@ -1134,14 +1187,15 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
 // The last tile of a task also publishes the task's total.
 // --------------------------------------------------------------------------
 template <int R, class S = FxInterp>
-__global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t* __restrict__ sb, const FxLaunch la,
-                                                               const FxDyn) {
+__global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(const uint32_t* __restrict__ sb,
+                                                                              const FxLaunch la, const FxDyn) {
+  constexpr uint32_t NW = S::kWaves, NT = 64u * NW;   // the row tile is at most FX_BLOCK rows, NT >= FX_BLOCK
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];
   __shared__ uint32_t s_rowmap[FX_BLOCK];
-  __shared__ uint32_t s_wsum[FX_BLOCK / 64];
-  __shared__ uint32_t s_woff[FX_BLOCK / 64 + 1];
+  __shared__ uint32_t s_wsum[NW];
+  __shared__ uint32_t s_woff[NW + 1];
   __shared__ uint32_t s_prefix;
-  fx_stage(L, sb, la);
+  fx_stage<NT>(L, sb, la);
   const FxWork w = fx_locate<false>(L, blockIdx.x);
   FxCtx cx = fx_make_ctx(L, la, w);
 
@@ -1157,7 +1211,7 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
 
   // exclusive offset of this tile
   uint32_t part = 0;
-  for (uint32_t t = threadIdx.x; t < tile; t += FX_BLOCK) part += counts[t];
+  for (uint32_t t = threadIdx.x; t < tile; t += NT) part += counts[t];
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
   if (lane == 0) s_wsum[wave] = part;
@@ -1171,16 +1225,16 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
   __syncthreads();
   if (threadIdx.x == 0) {
     uint32_t p = 0;
-    for (int k = 0; k < FX_BLOCK / 64; ++k) p += s_wsum[k];
+    for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
     s_prefix = p;
     uint32_t acc = 0;
     s_woff[0] = 0;
-    for (int k = 1; k <= FX_BLOCK / 64; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
+    for (uint32_t k = 1; k <= NW; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
   }
   __syncthreads();
   if (keep) s_rowmap[s_woff[wave] + before] = row;
   __syncthreads();
-  const uint32_t n_kept = uni(s_woff[FX_BLOCK / 64]);
+  const uint32_t n_kept = uni(s_woff[NW]);
   const uint32_t prefix = uni(s_prefix);
   if (tile + 1 == uni(w.cls[FX_W(FxClass, n_rowtiles)]) && threadIdx.x == 0) {
     ((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])])[w.task] = prefix + n_kept;
@@ -1280,20 +1334,33 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
       }
     };
     const bool contig = !colmajor;
-    // items of this output that belong to this wave: first, first + 4, ...
+    // items of this output that belong to this wave: first, first + NW, ...
     // taken FX_K at a time so that their leading loads overlap
     // (the rotation by the output index spreads single-item outputs over the waves; it
     // must not depend on the order in which a wave walks the outputs)
-    uint32_t it0 = (wave_u + 4u - (oi & 3u)) & 3u;
+    uint32_t it0 = (wave_u + NW - (oi & (NW - 1u))) & (NW - 1u);
     FxLead ld;
     if (lead) ld = fx_lead_decode<R>(cx, pb);
-    if (uni(od[FX_W(FxOut, pure)])) {
+    bool rows_fast = false;
+    if constexpr (R == 2) {
+      rows_fast = uni(od[FX_W(FxOut, pure)]) && lead && !colmajor && vd == 1u && gprow == gpr && gpr * FX_V == inner &&
+                  inner == rowlen && gprow < (1u << 24) && (ld.dt == FX_F32 || ld.dt == FX_I32) && ld.cf[1] == 1 &&
+                  ((odt == FX_F32 && ovt == FX_VT_F) || (odt == FX_I32 && ovt == FX_VT_I));
+    }
+    if (rows_fast) {
+      constexpr uint32_t KP = S::kPure;
+      const uint32_t grm = uni(gr_magic), grs = uni(gr_shift);
+      for (; it0 + NW * (KP - 1u) < n_items; it0 += NW * KP)
+        fx_rows_batch<S, KP, NW>(cx, ld, s_rowmap, it0, lane, n_groups, gprow, grm, grs, op, obase, pb, pe);
+      for (; it0 < n_items; it0 += NW * 2u)
+        fx_rows_batch<S, 2, NW>(cx, ld, s_rowmap, it0, lane, n_groups, gprow, grm, grs, op, obase, pb, pe);
+    } else if (uni(od[FX_W(FxOut, pure)])) {
       // S::kPure items as one batch; an incomplete batch at the end takes the generic path
       constexpr uint32_t KP = S::kPure;
-      for (; it0 + 4u * (KP - 1u) < n_items; it0 += 4u * KP) {
+      for (; it0 + NW * (KP - 1u) < n_items; it0 += NW * KP) {
         uint32_t X[KP * FX_V], e0[KP], Mk[KP];
         fx_lead_batch<R, (int)KP>(
-            ld, [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) { make_item(it0 + 4u * k, e, M, q); }, X,
+            ld, [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) { make_item(it0 + NW * k, e, M, q); }, X,
             e0, Mk);
         S::run_pure(cx, pb + 1, pe, X);
 #pragma unroll
@@ -1305,12 +1372,12 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
         }
       }
     }
-    for (; it0 < n_items; it0 += 4u * FX_K) {
+    for (; it0 < n_items; it0 += NW * FX_K) {
       uint32_t P[FX_K][FX_V];
       if (lead) {
 #pragma unroll
         for (uint32_t k = 0; k < FX_K; ++k) {
-          const uint32_t it = it0 + 4u * k;
+          const uint32_t it = it0 + NW * k;
           if (it < n_items) {
             uint32_t e[FX_V], M;
             FxCoord<R> q;
@@ -1321,7 +1388,7 @@ __global__ __launch_bounds__(FX_BLOCK, 4) void fx_compact_scatter(const uint32_t
       }
 #pragma unroll 1
       for (uint32_t k = 0; k < FX_K; ++k) {
-        const uint32_t it = it0 + 4u * k;
+        const uint32_t it = it0 + NW * k;
         if (it < n_items) {
           uint32_t e[FX_V], M;
           FxCoord<R> q;

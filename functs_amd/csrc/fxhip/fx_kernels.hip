@@ -193,9 +193,9 @@ int fx_spec_count() {
 
 // a specialised kernel takes the arguments of the generic one
 static hipError_t launch_spec(const void* fn, const uint32_t* sb, const FxLaunch& la, const FxDyn* dyn, uint32_t grid,
-                              uint32_t lds, hipStream_t stream) {
+                              uint32_t lds, hipStream_t stream, uint32_t threads = FX_BLOCK) {
   void* args[3] = {(void*)&sb, (void*)&la, (void*)dyn};
-  return hipLaunchKernel(fn, dim3(grid), dim3(FX_BLOCK), args, lds, stream);
+  return hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds, stream);
 }
 
 static FxLaunch make_launch(const FxLaunchInfo& li) {
@@ -244,7 +244,7 @@ hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunc
   if (grid == 0) return hipSuccess;
   const FxLaunch la = make_launch(li);
   const uint32_t lds = fx_lds_bytes(li);
-  if (spec && spec->scatter) return launch_spec(spec->scatter, sb, la, dyn, grid, lds, stream);
+  if (spec && spec->scatter) return launch_spec(spec->scatter, sb, la, dyn, grid, lds, stream, spec->scatter_threads);
   switch (rank) {
     case 0:
     case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;

@@ -17,6 +17,12 @@
 // This is the ahead-of-time counterpart of the reference's run-time code generator
 // (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121, CompileToNVRTC :1319-1414).
 #pragma once
+#ifndef FX_SPEC_WAVES
+#define FX_SPEC_WAVES 4
+#endif
+#ifndef FX_SPEC_OCC
+#define FX_SPEC_OCC 4
+#endif
 #include "fx_device.h"
 
 // ---- host side: the table of specialised kernels linked into the library ----
@@ -24,6 +30,7 @@ struct FxSpecKernels {
   const void* dense = nullptr;    // fx_region_dense<R, FxSpec<P>>
   const void* count = nullptr;    // fx_compact_count<FxSpec<P>>
   const void* scatter = nullptr;  // fx_compact_scatter<R, FxSpec<P>>
+  uint32_t scatter_threads = 0;   // workgroup size that kernel is compiled for
 };
 void fx_spec_register(uint64_t hash, const FxSpecKernels& k);
 const FxSpecKernels* fx_spec_find(uint64_t hash);
@@ -131,6 +138,11 @@ struct FxSpec {
   // all waves take the narrow outputs first: those share their 128-byte lines, and compiled
   // their programs are too short to be worth overlapping with the wide outputs
   static constexpr int kWalk = 1;
+  // Eight waves share a row tile of the compaction kernel: the set-up of a tile (descriptor
+  // copy, offset, row map) is paid once, a wave's chain of items is half as long, and with
+  // 80 registers three such workgroups fit a CU, so a launch of up to 768 tiles is resident at once.
+  static constexpr uint32_t kWaves = FX_SPEC_WAVES;
+  static constexpr uint32_t kOcc = FX_SPEC_OCC;
   template <int N>
   static __device__ __forceinline__ void run_pure(const FxCtx&, int pc, int, uint32_t (&X)[N]) {
     dispatch_pure<0, N>(pc, X);
@@ -138,11 +150,12 @@ struct FxSpec {
 };
 
 struct FxSpecRegistrar {
-  FxSpecRegistrar(uint64_t hash, const void* dense, const void* count, const void* scatter) {
+  FxSpecRegistrar(uint64_t hash, const void* dense, const void* count, const void* scatter, uint32_t scatter_threads) {
     FxSpecKernels k;
     k.dense = dense;
     k.count = count;
     k.scatter = scatter;
+    k.scatter_threads = scatter_threads;
     fx_spec_register(hash, k);
   }
 };
@@ -150,7 +163,7 @@ struct FxSpecRegistrar {
 }  // namespace
 
 #define FX_SPEC_DENSE(P, R) \
-  static FxSpecRegistrar fx_registrar_##P(P::hash, (const void*)&fx_region_dense<R, FxSpec<P>>, nullptr, nullptr);
+  static FxSpecRegistrar fx_registrar_##P(P::hash, (const void*)&fx_region_dense<R, FxSpec<P>>, nullptr, nullptr, 0);
 #define FX_SPEC_COMPACT(P, R)                                                                    \
   static FxSpecRegistrar fx_registrar_##P(P::hash, nullptr, (const void*)&fx_compact_count<FxSpec<P>>, \
-                                          (const void*)&fx_compact_scatter<R, FxSpec<P>>);
+                                          (const void*)&fx_compact_scatter<R, FxSpec<P>>, 64u * FxSpec<P>::kWaves);

@@ -43,11 +43,202 @@ struct FxSpecEntry {
   int pure;        // output program that the batched path may run
 };
 
-template <int N>
+// Temporaries of a compiled program, and the values its loads fetched (one slot per
+// instruction, indexed by compile-time constants only: what is never read is never kept).
+template <int N, int NI = 1>
 struct FxRegTemps {
-  uint32_t v[N > 0 ? N : 1][FX_V];
+  uint32_t v[N > 0 ? N : 1][FX_V] = {};
+  uint32_t ld[NI][FX_V];
   __device__ __forceinline__ uint32_t& at(int32_t slot, int j) { return v[slot][j]; }
 };
+
+// ---- loads that repeat an earlier load --------------------------------------
+// An instruction reads memory through (buffer a, affine record b, dtype): LDA into A,
+// anything with FX_F_MEMB into B.  Inside one straight-line stretch of a program (no
+// change of the lane mask, no loop edge) two such reads with the same operands fetch
+// the same values, so the later one takes them from the register copy of the earlier.
+constexpr bool fx_spec_loads(const FxInsn& I) { return I.op == FX_LDA || (I.flags & FX_F_MEMB) != 0; }
+constexpr bool fx_spec_barrier(uint32_t op) {
+  return op == FX_MIF || op == FX_MELSE || op == FX_MMERGE || op == FX_MEND || op == FX_MIFR || op == FX_RBEGIN ||
+         op == FX_RNEXT;
+}
+template <class P>
+constexpr int fx_spec_n_insn() { return (int)(sizeof(P::code) / sizeof(P::code[0])); }
+
+// Loads that do not repeat an earlier one are issued together where their stretch starts (the
+// first FX_SPEC_HOIST of them): their addresses depend on the coordinates, the loop counters
+// and the lane mask only, and those are fixed over a stretch.  A wave then pays one memory
+// round trip per stretch instead of one per load.  Dense regions only: in a row compaction
+// the loads of a narrow output are gathers over the kept rows, which gain nothing from being
+// in flight together (measured), and the registers they hold cost a wave per SIMD.
+#ifndef FX_SPEC_HOIST
+#define FX_SPEC_HOIST 8
+#endif
+template <class P>
+constexpr int fx_spec_hoist_cap() {
+  for (int e = 0; e < P::n_entries; ++e)
+    if (P::entries[e].kind == 1) return 0;   // a mask program: this is a row compaction
+  return FX_SPEC_HOIST;
+}
+
+// A stretch is a run of instructions that execute together, in order, under one lane mask
+// and one setting of the loop counters: it starts at a program entry, behind an instruction
+// that changes the mask or a loop counter, and wherever a structured jump lands.
+template <int N>
+struct FxSpecTables {
+  int begin[N];      // first instruction of the stretch of instruction k
+  int end[N];        // first instruction behind it
+  int reuse[N];      // earlier instruction of the stretch whose loaded values k takes over, or -1
+  bool hoisted[N];   // k's load is issued at the start of its stretch
+  bool reused[N];    // a later instruction takes over the values k loads
+};
+template <class P>
+constexpr FxSpecTables<fx_spec_n_insn<P>()> fx_spec_tables() {
+  constexpr int N = fx_spec_n_insn<P>();
+  FxSpecTables<N> t{};
+  bool start[N + 1] = {};
+  for (int e = 0; e < P::n_entries; ++e) {
+    start[P::entries[e].begin] = true;
+    start[P::entries[e].end] = true;
+  }
+  for (int k = 0; k < N; ++k) {
+    const FxInsn J = P::code[k];
+    if (fx_spec_barrier(J.op)) start[k + 1] = true;
+    if ((J.op == FX_MIF || J.op == FX_MIFR || J.op == FX_MELSE || J.op == FX_RNEXT) && J.a >= 0 && J.a <= N) start[J.a] = true;
+    if (J.op == FX_RBEGIN && J.b >= 0 && J.b <= N) start[J.b] = true;
+  }
+  int b = 0;
+  for (int k = 0; k < N; ++k) {
+    if (start[k]) b = k;
+    t.begin[k] = b;
+  }
+  int next = N;
+  for (int k = N - 1; k >= 0; --k) {
+    t.end[k] = next;
+    if (start[k] || fx_spec_barrier(P::code[k].op)) next = k;
+  }
+  for (int k = 0; k < N; ++k) {
+    const FxInsn I = P::code[k];
+    t.reuse[k] = -1;
+    t.hoisted[k] = false;
+    t.reused[k] = false;
+    if (fx_spec_barrier(I.op) || !fx_spec_loads(I)) continue;
+    int rank = 0;
+    for (int m = t.begin[k]; m < k; ++m) {
+      const FxInsn J = P::code[m];
+      if (fx_spec_barrier(J.op) || !fx_spec_loads(J)) continue;
+      if (J.a == I.a && J.b == I.b && J.dt == I.dt && ((J.flags ^ I.flags) & FX_F_I2F) == 0) t.reuse[k] = m;
+      if (t.reuse[m] < 0) ++rank;
+    }
+    if (t.reuse[k] >= 0) {
+      // chains end at the first of the equal loads, the one that really loads
+      while (t.reuse[t.reuse[k]] >= 0) t.reuse[k] = t.reuse[t.reuse[k]];
+      t.reused[t.reuse[k]] = true;
+    } else {
+      t.hoisted[k] = rank < fx_spec_hoist_cap<P>();
+    }
+  }
+  return t;
+}
+template <class P>
+struct FxSpecPlan {
+  static constexpr FxSpecTables<fx_spec_n_insn<P>()> T = fx_spec_tables<P>();
+};
+template <class P> constexpr bool fx_spec_stretch_start(int pc) { return FxSpecPlan<P>::T.begin[pc] == pc; }
+template <class P> constexpr int fx_spec_stretch_end(int pc) { return FxSpecPlan<P>::T.end[pc]; }
+template <class P> constexpr int fx_spec_reuse(int pc) { return FxSpecPlan<P>::T.reuse[pc]; }
+template <class P> constexpr bool fx_spec_hoisted(int pc) { return FxSpecPlan<P>::T.hoisted[pc]; }
+template <class P> constexpr bool fx_spec_reused(int pc) { return FxSpecPlan<P>::T.reused[pc]; }
+
+// number of hoisted loads in [K, END), and whether all of them read 32-bit elements as they are
+template <class P>
+constexpr int fx_spec_hoist_count(int k, int end) {
+  int n = 0;
+  for (; k < end; ++k) if (fx_spec_hoisted<P>(k)) ++n;
+  return n;
+}
+template <class P>
+constexpr bool fx_spec_hoist_plain(int k, int end) {
+  for (; k < end; ++k)
+    if (fx_spec_hoisted<P>(k) &&
+        !((P::code[k].dt == FX_F32 || P::code[k].dt == FX_I32) && (P::code[k].flags & FX_F_I2F) == 0))
+      return false;
+  return true;
+}
+
+// the hoisted loads of the stretch [K, END), one after the other (general form)
+template <class P, int R, int K, int END, class TS>
+__device__ __forceinline__ void fx_spec_prefetch(const FxCtx& cx, const FxCoord<R>& q, TS& ts, uint32_t M, const FxRegs& rg) {
+  if constexpr (K < END) {
+    if constexpr (fx_spec_hoisted<P>(K)) {
+      constexpr FxInsn J = P::code[K];
+      int32_t off[FX_V];
+      const bool consecutive = fx_affine<R>(cx, q, J.b, rg.lc0, rg.lc1, off);
+      fx_load_vec(fx_ptr(cx, J.a), off, M, J.dt, (J.flags & FX_F_I2F) != 0, consecutive, ts.ld[K]);
+    }
+    fx_spec_prefetch<P, R, K + 1, END, TS>(cx, q, ts, M, rg);
+  }
+}
+// addresses of the hoisted loads of [K, END): element offsets (dead elements: 0), buffers, and
+// how many of the loads are runs of FX_V consecutive elements
+template <class P, int R, int K, int END, int RANK, int H>
+__device__ __forceinline__ void fx_spec_pf_addr(const FxCtx& cx, const FxCoord<R>& q, uint32_t M, const FxRegs& rg,
+                                                uint32_t (&off)[H][FX_V], uint64_t (&ptr)[H], int& n_consecutive) {
+  if constexpr (K < END) {
+    if constexpr (fx_spec_hoisted<P>(K)) {
+      constexpr FxInsn J = P::code[K];
+      int32_t o[FX_V];
+      if (fx_affine<R>(cx, q, J.b, rg.lc0, rg.lc1, o)) ++n_consecutive;
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) off[RANK][j] = ((M >> j) & 1u) ? (uint32_t)o[j] : 0u;
+      ptr[RANK] = fx_ptr(cx, J.a);
+      fx_spec_pf_addr<P, R, K + 1, END, RANK + 1, H>(cx, q, M, rg, off, ptr, n_consecutive);
+    } else {
+      fx_spec_pf_addr<P, R, K + 1, END, RANK, H>(cx, q, M, rg, off, ptr, n_consecutive);
+    }
+  }
+}
+// the loads themselves, back to back with no branch between them: WIDE = one 128-bit load
+// per lane, else FX_V single-element loads
+template <class P, int K, int END, int RANK, int H, bool WIDE, class TS>
+__device__ __forceinline__ void fx_spec_pf_load(TS& ts, const uint32_t (&off)[H][FX_V], const uint64_t (&ptr)[H]) {
+  if constexpr (K < END) {
+    if constexpr (fx_spec_hoisted<P>(K)) {
+      const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)ptr[RANK];
+      if constexpr (WIDE) {
+        const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)(base + (off[RANK][0] << 2));
+        ts.ld[K][0] = v.x; ts.ld[K][1] = v.y; ts.ld[K][2] = v.z; ts.ld[K][3] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) ts.ld[K][j] = *(const FX_AS1 uint32_t*)(base + (off[RANK][j] << 2));
+      }
+      fx_spec_pf_load<P, K + 1, END, RANK + 1, H, WIDE, TS>(ts, off, ptr);
+    } else {
+      fx_spec_pf_load<P, K + 1, END, RANK, H, WIDE, TS>(ts, off, ptr);
+    }
+  }
+}
+// Entry of a stretch.  When all its hoisted loads read plain 32-bit elements and all of them
+// (or none) are 128-bit runs, every address is computed first and the loads follow without a
+// branch between them, so that they are in flight together; otherwise one after the other.
+template <class P, int R, int K, int END, class TS>
+__device__ __forceinline__ void fx_spec_stretch_entry(const FxCtx& cx, const FxCoord<R>& q, TS& ts, uint32_t M,
+                                                      const FxRegs& rg) {
+  constexpr int H = fx_spec_hoist_count<P>(K, END);
+  if constexpr (H >= 2 && fx_spec_hoist_plain<P>(K, END)) {
+    uint32_t off[H][FX_V];
+    uint64_t ptr[H];
+    int n_consecutive = 0;
+    fx_spec_pf_addr<P, R, K, END, 0, H>(cx, q, M, rg, off, ptr, n_consecutive);
+    const uint32_t VM = (1u << FX_V) - 1u;
+    const bool whole = !wave_any(M != 0u && M != VM) && wave_any(M == VM);   // as in fx_load_vec
+    if (n_consecutive == 0 || !whole) fx_spec_pf_load<P, K, END, 0, H, false, TS>(ts, off, ptr);
+    else if (n_consecutive == H) fx_spec_pf_load<P, K, END, 0, H, true, TS>(ts, off, ptr);
+    else fx_spec_prefetch<P, R, K, END, TS>(cx, q, ts, M, rg);
+  } else if constexpr (H >= 1) {
+    fx_spec_prefetch<P, R, K, END, TS>(cx, q, ts, M, rg);
+  }
+}
 
 // instructions [PC, END) of program table P
 template <class P, int R, int PC, int END, class TS>
@@ -75,7 +266,27 @@ __device__ __forceinline__ void fx_spec_range(const FxCtx& cx, const FxCoord<R>&
       fx_spec_range<P, R, I.b, END, TS>(cx, q, ts, M, A, rg);
     } else {
       static_assert(I.op != FX_RNEXT, "loop edge outside a loop");
-      fx_step<R>(cx, q, ts, w0, I.a, I.b, I.imm, M, A, rg, [](int32_t) {});
+      if constexpr (fx_spec_stretch_start<P>(PC))
+        fx_spec_stretch_entry<P, R, PC, fx_spec_stretch_end<P>(PC), TS>(cx, q, ts, M, rg);
+      constexpr int src = fx_spec_reuse<P>(PC) >= 0 ? fx_spec_reuse<P>(PC) : (fx_spec_hoisted<P>(PC) ? PC : -1);
+      if constexpr (src >= 0) {
+        if constexpr (I.op == FX_LDA) {
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) A[j] = ts.ld[src][j];
+        } else {
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) rg.B[j] = ts.ld[src][j];
+          // the rest of the instruction, with its second operand in place (LDB is done)
+          if constexpr (I.op != FX_LDB)
+            fx_step<R>(cx, q, ts, w0 & ~((uint32_t)FX_F_MEMB << 16), I.a, I.b, I.imm, M, A, rg, [](int32_t) {});
+        }
+      } else {
+        fx_step<R>(cx, q, ts, w0, I.a, I.b, I.imm, M, A, rg, [](int32_t) {});
+        if constexpr (fx_spec_reused<P>(PC)) {
+#pragma unroll
+          for (int j = 0; j < FX_V; ++j) ts.ld[PC][j] = I.op == FX_LDA ? A[j] : rg.B[j];
+        }
+      }
       fx_spec_range<P, R, PC + 1, END, TS>(cx, q, ts, M, A, rg);
     }
   }
@@ -103,7 +314,7 @@ struct FxSpec {
         if (pc == en.begin) {
           FxRegs rg;
           fx_regs_init(rg);
-          FxRegTemps<P::n_temps> ts = {};
+          FxRegTemps<P::n_temps, fx_spec_n_insn<P>()> ts;
           fx_spec_range<P, R, en.begin, en.end>(cx, q, ts, M, A, rg);
           return;
         }

@@ -89,6 +89,8 @@ def _run_benchmark_programs(names):
             configs.build_c3_classes(80)(*decoded)
     if "coverage" in names or len(names) == len(INPUTS):
         configs.build_column_standardize()(torch.rand(*configs.COLUMN_STANDARDIZE_SHAPE, device=dev))
+    if "coverage" in names or len(names) == len(INPUTS):
+        configs.build_row_filter()(*[torch.rand(*sh, device=dev) - 0.5 for sh in configs.ROW_FILTER_SHAPES])
     if "stream" in names or len(names) == len(INPUTS):
         x = torch.rand(8192, 4096, device=dev)
         r = Region()

@@ -134,3 +134,31 @@ def build_column_standardize():
     r.output(r.where(z > 0.0, z, z * 0.1) / (spread.unsqueeze(0) + 1.0))
     r.output(r.cat([x.slice(1, 0, 2).exp(), x.slice(1, 2, None)], 1).softmax(1))
     return r.finalize()
+
+
+# shapes for which `python -m functs_amd.aot` compiles the region below
+ROW_FILTER_SHAPES = ((1000, 19), (1000, 2))
+
+
+def build_row_filter():
+    """Not one of the five configurations either: a row compaction that takes every route of the
+    compaction kernel in one launch, used to check the compiled kernels against the interpreter.
+    Rows of `x` [n, 19] with a positive first column are kept; of those rows it returns::
+
+        wide   = sigmoid(x[:, 3:])              16 columns: whole groups of four, unaligned rows
+        ragged = x[:, :7] * 2                   7 columns: a ragged last group
+        narrow = cat([a * b + a, a * b - b], 1) with a = x[:, 1:2] * s[:, 0:1], b = x[:, 2:3] + s[:, 1:2]:
+                 every column reads its inputs twice
+        first  = x[:, 0]
+    """
+    r = Region()
+    x = r.tensor_input(torch.float32, 2)
+    s = r.tensor_input(torch.float32, 2)
+    a = x.slice(1, 1, 2) * s.slice(1, 0, 1)
+    b = x.slice(1, 2, 3) + s.slice(1, 1, 2)
+    r.output(x.slice(1, 3, None).sigmoid())
+    r.output(x.slice(1, 0, 7) * 2.0)
+    r.output(r.cat([a * b + a, a * b - b], 1))
+    r.output(x.select(1, 0))
+    r.compact_rows(x.select(1, 0) > 0.0)
+    return r.finalize()

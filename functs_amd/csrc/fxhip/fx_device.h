@@ -1209,6 +1209,11 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   const FX_AS1 uint32_t* counts =
       (const FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
 
+  // this thread's row flag and its share of the counts of the earlier tiles: both loads are
+  // issued before either value is used
+  const uint32_t row = tile * rt + threadIdx.x;
+  const bool in_tile = (threadIdx.x < rt) && (row < n_rows);
+  const uint32_t flag = in_tile ? (uint32_t)flags[row] : 0u;
   // exclusive offset of this tile
   uint32_t part = 0;
   for (uint32_t t = threadIdx.x; t < tile; t += NT) part += counts[t];
@@ -1217,8 +1222,7 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   if (lane == 0) s_wsum[wave] = part;
 
   // row map of this tile
-  const uint32_t row = tile * rt + threadIdx.x;
-  const bool keep = (threadIdx.x < rt) && (row < n_rows) && (flags[row] != 0);
+  const bool keep = flag != 0u;
   const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
   const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
   if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);

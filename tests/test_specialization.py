@@ -198,3 +198,51 @@ def test_compiled_reduction_loops_where_cat_softmax():
     want1 = torch.cat([x[:, :2].exp(), x[:, 2:]], 1).softmax(1)
     torch.testing.assert_close(fast[0].cpu(), want0, rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(fast[1].cpu(), want1, rtol=1e-5, atol=1e-6)
+
+
+def _row_filter_inputs(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.rand(n, sh[1], generator=g) - 0.5 for sh in configs.ROW_FILTER_SHAPES]
+
+
+def test_row_filter_region_is_linked_and_current():
+    r = configs.build_row_filter()
+    args = _row_filter_inputs(configs.ROW_FILTER_SHAPES[0][0], 0)
+    key = r.spec_key(*args)
+    assert r.specialized(*args), "no compiled kernels for key %016x: regenerate with python -m functs_amd.aot" % key
+    committed = open(os.path.join(SPEC_DIR, "fx_spec_%016x.hip" % key)).read().split("\n", 1)[1]
+    assert r.spec_source(*args).split("\n", 1)[1] == committed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [1, 63, 256, 257, 1000, 4099])
+def test_compiled_row_compaction_routes(n):
+    """One launch with an output made of whole groups of four (the lean batch path, with and
+    without a last incomplete batch), one with a ragged last group (the general batch path), a
+    column-wise narrow one whose programs read their inputs twice (repeated loads are reused
+    in compiled programs) and a rank-1 one: compiled == interpreter bit for bit, and equal to
+    torch on the kept rows (bit-exact for the copies, 1e-5 for the arithmetic)."""
+    dev = torch.device("cuda:0")
+    r = configs.build_row_filter()
+    x, s = _row_filter_inputs(n, n)
+    gx, gs = x.to(dev), s.to(dev)
+    assert r.specialized(gx, gs)   # the row count is not part of the programs
+    fast = r(gx, gs)
+    aot.enable(False)
+    try:
+        slow = r(gx, gs)
+    finally:
+        aot.enable(True)
+    for a, b in zip(_flat(fast), _flat(slow)):
+        assert torch.equal(a, b)
+    keep = x[:, 0] > 0
+    xk, sk = x[keep], s[keep]
+    a = xk[:, 1:2] * sk[:, 0:1]
+    b = xk[:, 2:3] + sk[:, 1:2]
+    outs = [o.cpu() for o in _flat(fast) if isinstance(o, torch.Tensor)]
+    wide, ragged, narrow, first = outs[:4]
+    assert wide.shape == (int(keep.sum()), 16)
+    torch.testing.assert_close(wide, xk[:, 3:].sigmoid(), rtol=1e-5, atol=1e-6)
+    assert torch.equal(ragged, xk[:, :7] * 2.0)
+    torch.testing.assert_close(narrow, torch.cat([a * b + a, a * b - b], 1), rtol=1e-5, atol=1e-6)
+    assert torch.equal(first, xk[:, 0])

@@ -402,7 +402,8 @@ int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, i
 size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
 
 static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
-                    void* scratch, uint32_t* totals_host, void* stream_, float* kernel_ms, int cap, int* n_kernels) {
+                    void* scratch, uint32_t* totals_host, void* stream_, float* kernel_ms, int cap, int* n_kernels,
+                    int repeat = 1) {
   if (!reg || !plan || !out_ptrs) return fail(FX_E_INVALID, "null argument");
   fx::Plan* pl = const_cast<fx::Plan*>(P(plan));
   if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
@@ -455,21 +456,25 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   if (pl->mode == FX_MODE_DENSE) {
     HIP_OK(mark(0));
     // persistent workgroups: at most 8 per CU worth of blocks stride over the units
-    HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream, spec));
+    for (int r = 0; r < repeat; ++r)
+      HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
   } else {
     HIP_OK(mark(0));
-    HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream, spec));
+    for (int r = 0; r < repeat; ++r) HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream, spec));
     HIP_OK(mark(1));
     HIP_OK(mark(2));
-    HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn, pl->grid, stream, spec));
+    for (int r = 0; r < repeat; ++r) HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn, pl->grid, stream, spec));
     HIP_OK(mark(3));
     nk = pl->grid > 0 ? 2 : 0;
   }
   if (timed) {
     HIP_OK(hipEventSynchronize(ev[nk == 2 ? 3 : 1]));
-    for (int k = 0; k < nk && k < cap; ++k) HIP_OK(hipEventElapsedTime(&kernel_ms[k], ev[2 * k], ev[2 * k + 1]));
+    for (int k = 0; k < nk && k < cap; ++k) {
+      HIP_OK(hipEventElapsedTime(&kernel_ms[k], ev[2 * k], ev[2 * k + 1]));
+      kernel_ms[k] /= (float)repeat;
+    }
     for (auto& e : ev) (void)hipEventDestroy(e);
     if (n_kernels) *n_kernels = nk;
   }
@@ -523,6 +528,14 @@ int fx_region_run_timed(fx_region* reg, const fx_plan* plan, const fx_arg* args,
                         int* n_kernels) {
   if (!kernel_ms || cap < 2) return fail(FX_E_INVALID, "fx_region_run_timed: kernel_ms[>=2] required");
   return run_impl(reg, plan, args, n_args, out_ptrs, scratch, totals_host, stream, kernel_ms, cap, n_kernels);
+}
+
+int fx_region_run_timed_batched(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args,
+                                void* const* out_ptrs, void* scratch, uint32_t* totals_host, void* stream, int repeat,
+                                float* kernel_ms, int cap, int* n_kernels) {
+  if (!kernel_ms || cap < 2) return fail(FX_E_INVALID, "fx_region_run_timed_batched: kernel_ms[>=2] required");
+  if (repeat < 1 || repeat > 1000) return fail(FX_E_INVALID, "fx_region_run_timed_batched: repeat must be 1..1000");
+  return run_impl(reg, plan, args, n_args, out_ptrs, scratch, totals_host, stream, kernel_ms, cap, n_kernels, repeat);
 }
 
 size_t fx_compact_rows_scratch_bytes(int64_t n) {

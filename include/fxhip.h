@@ -212,6 +212,15 @@ int fx_region_wait_totals(const fx_plan*, const uint32_t* totals_host, void* str
 int fx_region_run_timed(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
                         void* scratch, uint32_t* totals_host, void* stream, float* kernel_ms, int cap,
                         int* n_kernels);
+/* The same with every kernel launched `repeat` times back to back inside its event pair
+ * (1..1000; the kernels of a region are idempotent: they read the call's inputs and write its
+ * outputs); kernel_ms holds the mean per launch.  An event pair around one launch adds about
+ * 2 us to what it reads (an empty kernel reads 6 us that way); a batch spreads that over its
+ * launches, and what is left is the duration a kernel trace reports.  Measurement aid of the
+ * benchmark as well (fait/util/profile.cpp:29-46). */
+int fx_region_run_timed_batched(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
+                                void* scratch, uint32_t* totals_host, void* stream, int repeat, float* kernel_ms,
+                                int cap, int* n_kernels);
 
 /* The argument marshalling of fx_region_run without the launch (host only; the
  * analogue of GraphBuilder::prepareRunArgs, graph_builder.cpp:718-899).

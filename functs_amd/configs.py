@@ -162,3 +162,36 @@ def build_row_filter():
     r.output(x.select(1, 0))
     r.compact_rows(x.select(1, 0) > 0.0)
     return r.finalize()
+
+
+def _level_anchors(r, base, feat, stride):
+    """Anchors of one feature level, generated inside the region the way the reference's
+    model does it on the host (yolov3_bbox.py:78-101): base [A, 4] corner form + the grid shifts."""
+    sx = r.arange(0, feat, dtype=torch.float32) * stride
+    xx = sx.repeat(feat)
+    yy = sx.view(-1, 1).repeat(1, feat).view(-1)
+    shifts = r.stack([xx, yy, xx, yy], -1)
+    return (base.unsqueeze(0) + shifts.unsqueeze(1)).view(-1, 4)
+
+
+def build_c5_generated_anchors(batch, levels):
+    """C5 with the anchor / stride tables generated inside the region (arange, repeat, view,
+    stack, broadcast add, cat) instead of read from HBM: the step in front of the hot path
+    (yolov3_bbox.py:78-101, 209-216).  `levels`: ((feature size, stride), ...); inputs:
+    preds [B, N, 85] and one base-anchor tensor [A, 4] per level, N = sum(f * f * A).
+    Every use of the anchor tensor inlines its generation, so the programs are long (about
+    1 200 instructions for three levels): the interpreter's temporaries exceed a workgroup's
+    LDS and the region runs with compiled kernels only."""
+    r = Region(parallel_degree=batch, is_parallel_map=True)
+    preds = r.tensor_input(torch.float32, 3)
+    bases = [r.tensor_input(torch.float32, 2) for _ in levels]
+    i = r.task_index()
+    pred = preds.slice(0, i, r.op("INT_ADD", i, 1))
+    anchors = r.cat([_level_anchors(r, b, f, s) for b, (f, s) in zip(bases, levels)], 0)
+    strides = r.cat([r.full([f * f * 3], float(s)) for f, s in levels], 0)
+    boxes, cls, obj, keep = _yolo_body(r, pred, anchors, strides)
+    r.output(boxes)
+    r.output(cls)
+    r.output(obj)
+    r.compact_rows(keep)
+    return r.finalize()

@@ -444,6 +444,13 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                            : 0u;
   }
   const FxSpecKernels* spec = spec_of(pl);
+  if (!spec && pl->needs_compiled) {
+    char key[17];
+    snprintf(key, sizeof key, "%016llx", (unsigned long long)pl->spec_key);
+    return fail(FX_E_LIMIT, std::string("the interpreter's temporaries of this region need ") + std::to_string(pl->lds_bytes) +
+                                " bytes of LDS (limit 65536) and no compiled kernels for its programs (key " + key +
+                                ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
+  }
   g_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
   if (spec) g_spec_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream

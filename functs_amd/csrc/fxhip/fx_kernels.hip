@@ -213,13 +213,15 @@ uint32_t fx_lds_bytes(const FxLaunchInfo& li) {
   FxLaunch la = make_launch(li);
   return (la.temps_off + li.n_temps * FX_V * FX_BLOCK) * 4u;
 }
+// compiled kernels keep their temporaries in registers
+static uint32_t lds_bytes_compiled(const FxLaunchInfo& li) { return make_launch(li).temps_off * 4u; }
 
 hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                            hipStream_t stream, const FxSpecKernels* spec) {
   if (grid == 0) return hipSuccess;
   const FxLaunch la = make_launch(li);
   const uint32_t lds = fx_lds_bytes(li);
-  if (spec && spec->dense) return launch_spec(spec->dense, sb, la, dyn, grid, lds, stream);
+  if (spec && spec->dense) return launch_spec(spec->dense, sb, la, dyn, grid, lds_bytes_compiled(li), stream);
   switch (rank) {
     case 0:
     case 1: fx_region_dense<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
@@ -234,7 +236,7 @@ hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li,
 hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                                    hipStream_t stream, const FxSpecKernels* spec) {
   if (grid == 0) return hipSuccess;
-  if (spec && spec->count) return launch_spec(spec->count, sb, make_launch(li), dyn, grid, fx_lds_bytes(li), stream);
+  if (spec && spec->count) return launch_spec(spec->count, sb, make_launch(li), dyn, grid, lds_bytes_compiled(li), stream);
   fx_compact_count<FxInterp><<<grid, FX_BLOCK, fx_lds_bytes(li), stream>>>(sb, make_launch(li), *dyn);
   return hipGetLastError();
 }
@@ -244,7 +246,8 @@ hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunc
   if (grid == 0) return hipSuccess;
   const FxLaunch la = make_launch(li);
   const uint32_t lds = fx_lds_bytes(li);
-  if (spec && spec->scatter) return launch_spec(spec->scatter, sb, la, dyn, grid, lds, stream, spec->scatter_threads);
+  if (spec && spec->scatter)
+    return launch_spec(spec->scatter, sb, la, dyn, grid, lds_bytes_compiled(li), stream, spec->scatter_threads);
   switch (rank) {
     case 0:
     case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;

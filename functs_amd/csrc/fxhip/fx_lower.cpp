@@ -2046,8 +2046,12 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   P->lds_bytes = (uint32_t)((blob.size() + 2 * (P->sptr.size() + P->tptr.size() * (size_t)T) +
                              (P->sscal.size() + P->tscal.size() * (size_t)T) + 4 +
                              (size_t)max_temps * FX_V * FX_BLOCK) * 4);
-  FX_CHECK(P->lds_bytes <= 64 * 1024, FX_E_LIMIT,
-           "region descriptor + temporaries need " << P->lds_bytes << " bytes of LDS (limit 65536)");
+  // Compiled kernels keep the temporaries in registers: the descriptor alone has to fit.  A
+  // region whose interpreter temporaries do not fit as well runs with compiled kernels only.
+  const uint32_t lds_descriptor = P->lds_bytes - (uint32_t)((size_t)max_temps * FX_V * FX_BLOCK * 4);
+  FX_CHECK(lds_descriptor <= 64 * 1024, FX_E_LIMIT,
+           "region descriptor needs " << lds_descriptor << " bytes of LDS (limit 65536)");
+  P->needs_compiled = P->lds_bytes > 64 * 1024;
   P->spec_key = spec_hash(*P);
   const Plan* res = P.get();
   R.plans[key] = std::move(P);

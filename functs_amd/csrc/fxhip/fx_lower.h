@@ -82,6 +82,7 @@ struct Plan {
   uint32_t grid = 0;           // dense grid, or scatter grid in compaction mode
   uint32_t grid_count = 0;     // compaction pass 1
   uint32_t lds_bytes = 0;
+  bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
   uint32_t n_temps = 0;
   int max_rank = 1;
   std::vector<PtrSrc> sptr, tptr;

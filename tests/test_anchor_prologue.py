@@ -1,0 +1,67 @@
+"""The step in front of the hot path: anchor / stride tables generated inside the region
+(the reference's model builds them with arange / repeat / stack / reshape on the host,
+functs/benchmark/ai_model/yolov3/yolov3_bbox.py:78-101, and the reference fuses those operators,
+fait/fuser/custom_lowering_func.cpp:258-350).  Checked against stock torch on the same inputs."""
+import pytest
+import torch
+
+from functs_amd import configs
+from functs_amd._lib import FxError
+from functs_amd.benchmark.programs import yolov3_postproc
+from tests.util import run_region, assert_close, assert_boxes_close
+
+LEVELS = ((3, 32.0), (5, 16.0), (9, 8.0))
+SIZES = (((116, 90), (156, 198), (373, 326)), ((30, 61), (62, 45), (59, 119)), ((10, 13), (16, 30), (33, 23)))
+
+
+def _inputs(batch, seed):
+    g = torch.Generator().manual_seed(seed)
+    n = sum(f * f * 3 for f, _ in LEVELS)
+    preds = torch.randn(batch, n, 85, generator=g)
+    bases = [torch.tensor([[-w / 2, -h / 2, w / 2, h / 2] for w, h in s]) for s in SIZES]
+    return preds, bases
+
+
+def _torch_reference(preds, bases):
+    anc, st = [], []
+    for b, (f, s) in zip(bases, LEVELS):
+        sx = torch.arange(0, f, dtype=torch.float32) * s
+        xx = sx.repeat(f)
+        yy = sx.view(-1, 1).repeat(1, f).view(-1)
+        shifts = torch.stack([xx, yy, xx, yy], -1)
+        anc.append((b[None] + shifts[:, None]).reshape(-1, 4))
+        st.append(torch.full((f * f * 3,), s))
+    anchors, strides = torch.cat(anc), torch.cat(st)
+    return [yolov3_postproc(preds[i:i + 1], anchors, strides) for i in range(preds.size(0))]
+
+
+def test_generated_anchors_equal_torch_on_the_emulator():
+    preds, bases = _inputs(2, 3)
+    r = configs.build_c5_generated_anchors(2, LEVELS)
+    out = run_region("emul", r, preds, *bases)
+    ref = _torch_reference(preds, bases)
+    for i in range(2):
+        assert_boxes_close(out[0][i], ref[i][0], "boxes[%d]" % i)
+        assert_close(out[1][i], ref[i][1], "cls[%d]" % i)
+        assert_close(out[2][i], ref[i][2], "obj[%d]" % i)
+
+
+def test_generated_anchors_have_a_key_and_a_source():
+    preds, bases = _inputs(2, 3)
+    r = configs.build_c5_generated_anchors(2, LEVELS)
+    assert r.spec_key(preds, *bases) != 0
+    assert "FX_SPEC_COMPACT" in r.spec_source(preds, *bases)
+
+
+@pytest.mark.gpu
+def test_generated_anchors_without_compiled_kernels_are_refused():
+    """The interpreter keeps temporaries in LDS and this region has too many of them: with no
+    compiled kernels linked in, the call fails with a message that says so (before any launch)."""
+    dev = torch.device("cuda:0")
+    preds, bases = _inputs(2, 3)
+    r = configs.build_c5_generated_anchors(2, LEVELS)
+    args = [preds.to(dev)] + [b.to(dev) for b in bases]
+    if r.specialized(*args):
+        pytest.skip("compiled kernels for this region are linked in")
+    with pytest.raises(FxError, match="compiled kernels"):
+        r(*args)

@@ -17,8 +17,12 @@ the scripted program whose fused regions run as tssa::ParallelFunctor;
 (functs_amd.aot) or the bytecode interpreter (`--interpreter` forces the latter);
 `per_config` repeats the measurement for every benchmark configuration that is
 implemented.  `roofline` prices the dominant kernel against the 8 TB/s
-HBM peak with the algorithmic bytes of the call; `cpu_baseline` times the
-unfused TorchScript CPU path (the oracle) on a bounded sample.
+HBM peak with the algorithmic bytes of the call; its duration is measured with
+HIP events on the launch stream around ten back-to-back launches of the kernel
+(mean per launch, `kernel_ms`; the reading of a pair around a single launch,
+which carries about 2 us of the pair itself, is `kernel_ms_single_launch`).
+`cpu_baseline` times the unfused TorchScript CPU path (the oracle) on a bounded
+sample.
 """
 import argparse
 import json

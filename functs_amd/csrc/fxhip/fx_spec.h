@@ -349,9 +349,11 @@ struct FxSpec {
   // all waves take the narrow outputs first: those share their 128-byte lines, and compiled
   // their programs are too short to be worth overlapping with the wide outputs
   static constexpr int kWalk = 1;
-  // Eight waves share a row tile of the compaction kernel: the set-up of a tile (descriptor
-  // copy, offset, row map) is paid once, a wave's chain of items is half as long, and with
-  // 80 registers three such workgroups fit a CU, so a launch of up to 768 tiles is resident at once.
+  // Waves per workgroup of the compaction kernel (a power of two, 4 or 8) and the waves per
+  // SIMD its register budget is set for.  Eight waves sharing a row tile halve a wave's chain of
+  // items for the same set-up, but all tiles of a large launch stay resident only with at most
+  // 80 registers (three such workgroups per CU), which these kernels do not reach without
+  // spilling: measured slower, so four it is.
   static constexpr uint32_t kWaves = FX_SPEC_WAVES;
   static constexpr uint32_t kOcc = FX_SPEC_OCC;
   template <int N>

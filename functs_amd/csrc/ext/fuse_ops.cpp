@@ -868,6 +868,7 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   for (size_t i = 0; i < input_types.size() && i < graph->inputs().size(); ++i)
     if (input_types[i] && input_types[i]->kind() == c10::TypeKind::TensorType && isTensorValue(graph->inputs()[i]))
       graph->inputs()[i]->setType(input_types[i]);
+  ConvertProfilingInstrumentation(graph);   // fait.cpp:137: range markers first, they cut regions
   LowerSimpleTuples(graph);
   ConstantPropagation(graph);
   EliminateCommonSubexpression(graph);

@@ -33,6 +33,11 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_to_parallel_functor", ToParallelFunctor);
   m.def("_jit_pass_fait_pipeline", FaitPipeline);
   m.def("_jit_pass_validate", Validate);
+  m.def("_jit_pass_convert_profiling_instrumentation", ConvertProfilingInstrumentation);
+  m.def("_prof_begin", profBegin);
+  m.def("_prof_end", profEnd);
+  m.def("_prof_results", profilingResults);
+  m.def("_prof_reset", resetProfiling);
   m.def("_create_function_from_graph", [](const std::string& name, std::shared_ptr<Graph> graph) {
     // script_init.cpp:87-95; the stock GraphFunction + interpreter run the graph
     auto cu = std::make_shared<torch::jit::CompilationUnit>();

@@ -54,4 +54,12 @@ std::string fxhipLibraryPath();
 // shared by the passes
 bool isFusableNode(torch::jit::Node* node);
 
+// fait/passes/profile_ops.cpp:16-30: `print(label, True / False)` with constant arguments becomes
+// prof::Begin(label) / prof::End(label); fait/util/profile.cpp:133-245: the timers behind them.
+void ConvertProfilingInstrumentation(std::shared_ptr<torch::jit::Graph> graph);
+void profBegin(const std::string& label);
+void profEnd(const std::string& label);
+std::string profilingResults(size_t count);   // what printProfilingResults writes
+void resetProfiling();
+
 }  // namespace functs

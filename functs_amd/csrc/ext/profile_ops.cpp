@@ -1,0 +1,205 @@
+// Range timers for scripted programs: the operators prof::Begin / prof::End, the pass that
+// creates them from `print(label, True / False)` markers, and the C entry points a ctypes
+// harness drives (enableProfiling, disableProfiling, printProfilingResults).
+//
+// Interfaces of fait/passes/profile_ops.cpp:8-30 and fait/util/profile.cpp:99-245
+// (functs/utils/prof.py:40-100 is the harness that loads them).  The reference brackets a range
+// with device synchronisations, opens an NVTX range and counts kernel launches and allocations
+// through CUPTI; here the range is a roctx range (so rocprofv3 --marker-trace shows it) when
+// libroctx64 is present, and the launch count is the library's own (fx_launch_stats: launches of
+// region kernels; ATen's launches are not counted, allocations are not reported).
+#include <ATen/hip/HIPContext.h>
+#include <c10/hip/HIPFunctions.h>
+#include <dlfcn.h>
+#include <torch/csrc/jit/ir/constants.h>
+#include <torch/csrc/jit/runtime/custom_operator.h>
+
+#include <chrono>
+#include <iomanip>
+#include <iostream>
+#include <mutex>
+#include <sstream>
+#include <unordered_map>
+
+#include "../../../include/fxhip.h"
+#include "passes.h"
+
+namespace functs {
+using namespace torch::jit;
+using namespace std::chrono;
+
+namespace {
+
+struct TimeRecord {
+  nanoseconds total{0}, min{INT64_MAX}, max{0};
+  size_t count = 0;
+  bool open = false;
+  steady_clock::time_point begin;
+  uint64_t range = 0;
+};
+
+struct State {
+  std::mutex mu;
+  bool enabled = false;
+  std::vector<std::string> labels;   // in order of first use
+  std::unordered_map<std::string, TimeRecord> records;
+  uint64_t launches_at_enable = 0, launches = 0;
+  // roctx, looked up once
+  bool roctx_tried = false;
+  uint64_t (*range_start)(const char*) = nullptr;
+  void (*range_stop)(uint64_t) = nullptr;
+};
+State& state() {
+  static State s;
+  return s;
+}
+
+void lookupRoctx(State& s) {
+  if (s.roctx_tried) return;
+  s.roctx_tried = true;
+  void* h = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+  if (!h) h = dlopen("libroctx64.so.4", RTLD_NOW | RTLD_GLOBAL);
+  if (!h) return;
+  s.range_start = (uint64_t(*)(const char*))dlsym(h, "roctxRangeStartA");
+  s.range_stop = (void (*)(uint64_t))dlsym(h, "roctxRangeStop");
+  if (!s.range_start || !s.range_stop) s.range_start = nullptr, s.range_stop = nullptr;
+}
+
+void drainDevice() {
+  if (at::hasHIP() && c10::hip::device_count() > 0) c10::hip::device_synchronize();
+}
+
+uint64_t regionLaunches() {
+  uint64_t total = 0, compiled = 0;
+  fx_launch_stats(&total, &compiled);
+  return total;
+}
+
+std::string fmtDuration(nanoseconds dur) {
+  static const char* units[] = {"ns", "us", "ms", "s"};
+  double v = (double)dur.count();
+  int u = 0;
+  while (u < 3 && v > 1e3) { v /= 1e3; ++u; }
+  std::ostringstream ss;
+  ss << std::setprecision(4) << v << units[u];
+  return ss.str();
+}
+
+}  // namespace
+
+void profBegin(const std::string& label) {
+  State& s = state();
+  if (!s.enabled) return;
+  drainDevice();
+  std::lock_guard<std::mutex> g(s.mu);
+  if (!s.records.count(label)) {
+    s.labels.push_back(label);
+    s.records.emplace(label, TimeRecord{});
+  }
+  TimeRecord& r = s.records[label];
+  r.open = true;
+  if (s.range_start) r.range = s.range_start(label.c_str());
+  r.begin = steady_clock::now();
+}
+
+void profEnd(const std::string& label) {
+  State& s = state();
+  if (!s.enabled) return;
+  drainDevice();
+  const steady_clock::time_point now = steady_clock::now();
+  std::lock_guard<std::mutex> g(s.mu);
+  auto it = s.records.find(label);
+  TORCH_CHECK(it != s.records.end() && it->second.open, "prof::End(\"", label, "\") without a prof::Begin before it");
+  TimeRecord& r = it->second;
+  if (s.range_stop) s.range_stop(r.range);
+  const nanoseconds dur = duration_cast<nanoseconds>(now - r.begin);
+  r.open = false;
+  r.count++;
+  r.total += dur;
+  r.min = std::min(r.min, dur);
+  r.max = std::max(r.max, dur);
+}
+
+// the text printProfilingResults writes: launches per run, then one line per label
+std::string profilingResults(size_t count) {
+  State& s = state();
+  std::lock_guard<std::mutex> g(s.mu);
+  if (count == 0) count = 1;
+  std::ostringstream out;
+  const uint64_t launches = s.launches + (s.enabled ? regionLaunches() - s.launches_at_enable : 0);
+  if (launches > 0) out << "Kernel launch: " << launches / count << '\n';
+  if (s.records.empty()) return out.str();
+  auto cell = [&](const std::string& v) { out << std::setw(10) << v; };
+  out << "\nRanges:\n" << std::left << std::setw(16) << "Label" << std::right;
+  for (const char* h : {"Count", "Total", "Mean", "Min", "Max"}) cell(h);
+  out << '\n';
+  for (const std::string& label : s.labels) {
+    const TimeRecord& r = s.records[label];
+    out << std::left << std::setw(16) << label << std::right;
+    cell(std::to_string(r.count));
+    cell(fmtDuration(r.total));
+    cell(r.count ? fmtDuration(r.total / (int64_t)r.count) : "-");
+    cell(r.count ? fmtDuration(r.min) : "-");
+    cell(fmtDuration(r.max));
+    out << '\n';
+  }
+  return out.str();
+}
+
+void resetProfiling() {
+  State& s = state();
+  std::lock_guard<std::mutex> g(s.mu);
+  s.labels.clear();
+  s.records.clear();
+  s.launches = 0;
+  s.launches_at_enable = regionLaunches();
+}
+
+// fait/passes/profile_ops.cpp:16-30: print(<constant str>, <constant bool>) marks the begin
+// (True) or the end (False) of the range with that label.
+void ConvertProfilingInstrumentation(std::shared_ptr<Graph> graph) {
+  std::function<void(Block*)> visit = [&](Block* block) {
+    for (auto it = block->nodes().begin(); it != block->nodes().end();) {
+      Node* node = *it;
+      ++it;
+      for (Block* b : node->blocks()) visit(b);
+      if (node->kind() != c10::prim::Print || node->inputs().size() != 2) continue;
+      const auto label = toIValue(node->input(0));
+      const auto begin = toIValue(node->input(1));
+      if (!label || !label->isString() || !begin || !begin->isBool()) continue;
+      Node* marker =
+          graph->create(c10::Symbol::fromQualString(begin->toBool() ? "prof::Begin" : "prof::End"), {node->input(0)}, 0);
+      marker->insertBefore(node);
+      TORCH_CHECK(marker->maybeOperator(), "prof::Begin / prof::End are not registered");
+      node->destroy();
+    }
+  };
+  visit(graph->block());
+}
+
+static auto registerProfOps =
+    torch::RegisterOperators()
+        .op("prof::Begin(str label) -> ()", profBegin,
+            torch::RegisterOperators::options().aliasAnalysis(c10::AliasAnalysisKind::CONSERVATIVE))
+        .op("prof::End(str label) -> ()", profEnd,
+            torch::RegisterOperators::options().aliasAnalysis(c10::AliasAnalysisKind::CONSERVATIVE));
+
+}  // namespace functs
+
+// C entry points of the harness (fait/util/profile.h:9-15)
+extern "C" __attribute__((visibility("default"))) void enableProfiling() {
+  functs::State& s = functs::state();
+  std::lock_guard<std::mutex> g(s.mu);
+  functs::lookupRoctx(s);
+  s.launches_at_enable = functs::regionLaunches();
+  s.enabled = true;
+}
+extern "C" __attribute__((visibility("default"))) void disableProfiling() {
+  functs::State& s = functs::state();
+  std::lock_guard<std::mutex> g(s.mu);
+  if (s.enabled) s.launches += functs::regionLaunches() - s.launches_at_enable;
+  s.enabled = false;
+}
+extern "C" __attribute__((visibility("default"))) void printProfilingResults(size_t count) {
+  std::cout << functs::profilingResults(count) << std::flush;
+}

@@ -1241,7 +1241,11 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   const uint32_t n_kept = uni(s_woff[NW]);
   const uint32_t prefix = uni(s_prefix);
   if (tile + 1 == uni(w.cls[FX_W(FxClass, n_rowtiles)]) && threadIdx.x == 0) {
-    ((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])])[w.task] = prefix + n_kept;
+    // The host polls this word while the kernel still runs: a system-scope store goes through
+    // to host memory instead of waiting in L2 for the end of the kernel.  (Relaxed: the host
+    // reads the count only; everything else of the call is consumed in stream order.)
+    __hip_atomic_store((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])] + w.task, prefix + n_kept, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
   }
   if (n_kept == 0) return;
 

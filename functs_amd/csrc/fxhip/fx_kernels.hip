@@ -128,7 +128,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rows_scatter(const uint8_t* __res
   __syncthreads();
   const uint32_t n_kept = s_woff[FX_BLOCK / 64];
   const uint32_t prefix = s_prefix;
-  if (tile + 1 == gridDim.x && threadIdx.x == 0) *total_host = prefix + n_kept;
+  // system scope: the caller may poll the word in host memory while the kernel runs
+  if (tile + 1 == gridDim.x && threadIdx.x == 0)
+    __hip_atomic_store(total_host, prefix + n_kept, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   if (n_kept == 0) return;
 #pragma unroll
   for (int c = 0; c < 8; ++c) {

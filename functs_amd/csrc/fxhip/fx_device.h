@@ -752,6 +752,8 @@ struct FxInterp {
   }
   // items of a pure program that the compaction kernel batches (the dense kernel: FX_K)
   static constexpr uint32_t kPure = FX_K;
+  // ... and of the lean batches of whole-group outputs (fx_rows_batch)
+  static constexpr uint32_t kRows = FX_K;
   // order in which a wave of the compaction kernel walks the outputs: 0 = alternate waves
   // backwards, 1 = all forwards (narrow outputs first), 2 = all backwards
   static constexpr int kWalk = 0;
@@ -1356,7 +1358,7 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
                   ((odt == FX_F32 && ovt == FX_VT_F) || (odt == FX_I32 && ovt == FX_VT_I));
     }
     if (rows_fast) {
-      constexpr uint32_t KP = S::kPure;
+      constexpr uint32_t KP = S::kRows;
       const uint32_t grm = uni(gr_magic), grs = uni(gr_shift);
       for (; it0 + NW * (KP - 1u) < n_items; it0 += NW * KP)
         fx_rows_batch<S, KP, NW>(cx, ld, s_rowmap, it0, lane, n_groups, gprow, grm, grs, op, obase, pb, pe);

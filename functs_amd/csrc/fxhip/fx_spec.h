@@ -20,6 +20,9 @@
 #ifndef FX_SPEC_WAVES
 #define FX_SPEC_WAVES 4
 #endif
+#ifndef FX_SPEC_ROWS
+#define FX_SPEC_ROWS (3 * FX_K)
+#endif
 #ifndef FX_SPEC_OCC
 #define FX_SPEC_OCC 4
 #endif
@@ -346,6 +349,9 @@ struct FxSpec {
   }
   // compiled code is short: registers are spent on more loads in flight instead
   static constexpr uint32_t kPure = 2 * FX_K;
+  // the lean batches of whole-group outputs need few registers per item: twelve in flight
+  // (sixteen spill)
+  static constexpr uint32_t kRows = FX_SPEC_ROWS;
   // all waves take the narrow outputs first: those share their 128-byte lines, and compiled
   // their programs are too short to be worth overlapping with the wide outputs
   static constexpr int kWalk = 1;

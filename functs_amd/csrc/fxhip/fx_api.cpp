@@ -5,6 +5,9 @@
 // Counterpart of GraphBuilder::prepareRunArgs / runKernel
 // (fait/fuser/graph_builder.cpp:718-927) and CudaCodeGenTssa::call_raw
 // (fait/tensorexpr/cuda_codegen_tssa.cpp:1167-1290).
+#ifndef FX_DENSE_WG_PER_CU
+#define FX_DENSE_WG_PER_CU 12u   // workgroups of the dense kernel per CU (4 are resident; more, smaller shares even out the tail: measured 4 to 16)
+#endif
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -462,9 +465,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
   auto mark = [&](int i) -> hipError_t { return timed ? hipEventRecord(ev[i], stream) : hipSuccess; };
   if (pl->mode == FX_MODE_DENSE) {
     HIP_OK(mark(0));
-    // persistent workgroups: at most 8 per CU worth of blocks stride over the units
+    // persistent workgroups: at most FX_DENSE_WG_PER_CU per CU worth of blocks stride over the units
     for (int r = 0; r < repeat; ++r)
-      HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * 8u), stream, spec));
+      HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
   } else {

@@ -246,3 +246,25 @@ def test_compiled_row_compaction_routes(n):
     assert torch.equal(ragged, xk[:, :7] * 2.0)
     torch.testing.assert_close(narrow, torch.cat([a * b + a, a * b - b], 1), rtol=1e-5, atol=1e-6)
     assert torch.equal(first, xk[:, 0])
+
+
+@pytest.mark.gpu
+def test_batched_kernel_timing_leaves_results_alone():
+    """Timing a kernel over a batch of launches (the kernels of a region are idempotent) gives
+    the outputs of a plain launch and a mean below the single-launch reading plus noise."""
+    dev = torch.device("cuda:0")
+    r = configs.build_row_filter()
+    x, s = _row_filter_inputs(1000, 5)
+    bc = r.bind(x.to(dev), s.to(dev))
+    bc.launch()
+    want = [o.clone() for o in _flat(bc.results()) if isinstance(o, torch.Tensor)]
+    single = bc.launch_timed()
+    batched = bc.launch_timed(repeat=10)
+    got = [o for o in _flat(bc.results()) if isinstance(o, torch.Tensor)]
+    assert len(single) == len(batched) == 2 and all(t > 0 for t in batched)
+    assert sum(batched) < sum(single) * 1.5
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    from functs_amd._lib import FxError
+    with pytest.raises(FxError, match="repeat"):
+        bc.launch_timed(repeat=0)

@@ -274,10 +274,20 @@ struct Workspace {
   void* stream = nullptr;   // stream of the last run that used it (that run may still be in flight)
 };
 
+// where the tasks' tensors of every output lie in that output's one allocation: fixed per plan
+struct OutSlot { int64_t offset_elems; int32_t rank; int64_t sizes[FX_ARG_MAX_RANK]; };
+struct OutLayout {
+  std::vector<OutSlot> slots;      // [output][task]
+  std::vector<int64_t> total;      // elements to allocate per output
+  std::vector<int32_t> dtype;      // FX dtype per output
+  std::vector<int64_t> item;       // element size per output
+};
+
 struct Variant {
   fx_region* region = nullptr;
   std::mutex mu;
   std::vector<Workspace> pool;
+  std::unordered_map<const fx_plan*, std::shared_ptr<const OutLayout>> layouts;   // plans live as long as the region
   ~Variant() {
     if (region) fx_region_destroy(region);
   }
@@ -439,32 +449,56 @@ class RegionRunner {
     const int n_out = fx_plan_num_outputs(plan);
     // One allocation per output: the tasks' tensors are views at 256-byte aligned
     // offsets of it.  The views are made after the launch, while the kernels run.
-    struct Slot { int64_t offset_elems; int32_t rank; int64_t sizes[FX_ARG_MAX_RANK]; };
-    std::vector<Slot> slots((size_t)n_out * degree);
+    std::shared_ptr<const OutLayout> layout;
+    {
+      std::lock_guard<std::mutex> lock(var->mu);
+      auto it = var->layouts.find(plan);
+      if (it != var->layouts.end()) layout = it->second;
+    }
+    if (!layout) {
+      auto lay = std::make_shared<OutLayout>();
+      lay->slots.resize((size_t)n_out * degree);
+      lay->total.resize(n_out);
+      lay->dtype.resize(n_out);
+      lay->item.resize(n_out);
+      for (int o = 0; o < n_out; ++o) {
+        int32_t dt = 0;
+        int64_t total = 0, item = 1;
+        for (int64_t t = 0; t < degree; ++t) {
+          OutSlot& sl = lay->slots[(size_t)o * degree + t];
+          FX_OK_OR_THROW(fx_plan_output(plan, o, (int)t, &dt, &sl.rank, sl.sizes));
+          int64_t numel = 1;
+          for (int d = 0; d < sl.rank; ++d) numel *= sl.sizes[d];
+          item = (int64_t)c10::elementSize(atDtype(dt));
+          const int64_t align = 256 / item;
+          sl.offset_elems = total;
+          total += (numel + align - 1) / align * align;
+        }
+        lay->total[o] = total;
+        lay->dtype[o] = dt;
+        lay->item[o] = item;
+      }
+      std::lock_guard<std::mutex> lock(var->mu);
+      layout = var->layouts.emplace(plan, std::move(lay)).first->second;
+    }
+    typedef OutSlot Slot;
+    std::vector<Slot> slots;   // a copy only where the kept-row counts change the sizes
+    if (compact_) slots = layout->slots;
+    const Slot* slot_of = compact_ ? slots.data() : layout->slots.data();
     std::vector<at::Tensor> buffers(n_out);
     std::vector<void*> ptrs((size_t)n_out * degree);
     for (int o = 0; o < n_out; ++o) {
-      int32_t dt = 0;
-      int64_t total = 0, item = 1;
-      for (int64_t t = 0; t < degree; ++t) {
-        Slot& sl = slots[(size_t)o * degree + t];
-        FX_OK_OR_THROW(fx_plan_output(plan, o, (int)t, &dt, &sl.rank, sl.sizes));
-        int64_t numel = 1;
-        for (int d = 0; d < sl.rank; ++d) numel *= sl.sizes[d];
-        item = (int64_t)c10::elementSize(atDtype(dt));
-        const int64_t align = 256 / item;
-        sl.offset_elems = total;
-        total += (numel + align - 1) / align * align;
-      }
+      const int32_t dt = layout->dtype[o];
+      const int64_t item = layout->item[o];
       if (degree == 1) {
-        const Slot& sl = slots[(size_t)o * degree];
+        const Slot& sl = slot_of[(size_t)o * degree];
         buffers[o] = at::empty(at::IntArrayRef(sl.sizes, sl.rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
       } else {
-        buffers[o] = at::empty({total}, at::TensorOptions().dtype(atDtype(dt)).device(device));
+        buffers[o] = at::empty({layout->total[o]}, at::TensorOptions().dtype(atDtype(dt)).device(device));
       }
       char* base = (char*)buffers[o].data_ptr();
       for (int64_t t = 0; t < degree; ++t)
-        ptrs[(size_t)o * degree + t] = base + slots[(size_t)o * degree + t].offset_elems * item;
+        ptrs[(size_t)o * degree + t] = base + slot_of[(size_t)o * degree + t].offset_elems * item;
     }
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
     Workspace ws;
@@ -483,7 +517,7 @@ class RegionRunner {
       }
       outs[o].reserve(degree);
       for (int64_t t = 0; t < degree; ++t) {
-        const Slot& sl = slots[(size_t)o * degree + t];
+        const Slot& sl = slot_of[(size_t)o * degree + t];
         auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(buffers[o].storage()),
                                                          buffers[o].key_set(), buffers[o].dtype());
         impl->set_storage_offset(sl.offset_elems);

@@ -133,6 +133,8 @@ _sig("fx_region_run_timed_batched", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, cty
 _sig("fx_compact_rows", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, ctypes.c_size_t, _vp, _vp)
 _sig("fx_compact_rows_scratch_bytes", ctypes.c_size_t, ctypes.c_int64)
+_sig("fx_compact_rows_static", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+     ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, _vp)
 _sig("fx_device_count", _i)
 _sig("fx_copy_bytes", _i, _vp, _vp, ctypes.c_size_t, _vp)
 

@@ -30,6 +30,9 @@ hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, c
 hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
                                      uint32_t grid, hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream);
+hipError_t fx_launch_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                                         const int32_t* rowlen, const int32_t* elsize, int n_cols,
+                                         uint32_t* total_host, hipStream_t stream);
 hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                   const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
                                   uint32_t* total_host, hipStream_t stream);
@@ -553,20 +556,46 @@ size_t fx_compact_rows_scratch_bytes(int64_t n) {
   return (size_t)(((n + FX_BLOCK - 1) / FX_BLOCK + 1) * 4 + 256);
 }
 
-int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs, const int32_t* rowlen,
-                    const int32_t* elsize, int n_cols, void* scratch, size_t scratch_bytes, uint32_t* total_host,
-                    void* stream_) {
+static_assert(FX_STATIC_MAX_ROWS == FX_COMPACT_ROWS_STATIC_MAX, "the header states the limit of the static array");
+// argument checks shared by fx_compact_rows and fx_compact_rows_static
+static int check_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                              const int32_t* rowlen, const int32_t* elsize, int n_cols, const uint32_t* total_host) {
   if (n < 0 || n_cols < 0 || n_cols > 8) return fail(FX_E_INVALID, "fx_compact_rows: n >= 0 and 0 <= n_cols <= 8");
   if (n >= ((int64_t)1 << 31)) return fail(FX_E_LIMIT, "fx_compact_rows: n above 2^31");
   if (!total_host) return fail(FX_E_INVALID, "fx_compact_rows: total_host is required");
-  if (n > 0 && (!mask || !scratch)) return fail(FX_E_INVALID, "fx_compact_rows: null mask/scratch");
-  if (scratch_bytes < fx_compact_rows_scratch_bytes(n)) return fail(FX_E_INVALID, "fx_compact_rows: scratch too small");
+  if (n > 0 && !mask) return fail(FX_E_INVALID, "fx_compact_rows: null mask");
   for (int i = 0; i < n_cols; ++i) {
     if (!cols || !outs || !rowlen || !elsize) return fail(FX_E_INVALID, "fx_compact_rows: null column arrays");
     if (elsize[i] != 4 && elsize[i] != 8 && elsize[i] != 1) return fail(FX_E_UNSUPPORTED, "fx_compact_rows: elsize 1, 4 or 8");
     if (rowlen[i] < 1) return fail(FX_E_INVALID, "fx_compact_rows: rowlen >= 1");
     if ((int64_t)rowlen[i] * n >= ((int64_t)1 << 31)) return fail(FX_E_LIMIT, "fx_compact_rows: column above 2^31 elements");
   }
+  return FX_OK;
+}
+
+int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                           const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* total_host,
+                           void* stream_) {
+  const int rc = check_compact_rows(mask, n, cols, outs, rowlen, elsize, n_cols, total_host);
+  if (rc != FX_OK) return rc;
+  if (n > FX_STATIC_MAX_ROWS)
+    return fail(FX_E_LIMIT, "fx_compact_rows_static: n = " + std::to_string(n) + " rows is above the limit of " +
+                                std::to_string((long long)FX_STATIC_MAX_ROWS) + " (FX_COMPACT_ROWS_STATIC_MAX); use fx_compact_rows with caller scratch");
+  if (n == 0) {
+    *total_host = 0;
+    return FX_OK;
+  }
+  HIP_OK(fx_launch_compact_rows_static(mask, n, cols, outs, rowlen, elsize, n_cols, total_host, (hipStream_t)stream_));
+  return FX_OK;
+}
+
+int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs, const int32_t* rowlen,
+                    const int32_t* elsize, int n_cols, void* scratch, size_t scratch_bytes, uint32_t* total_host,
+                    void* stream_) {
+  const int rc = check_compact_rows(mask, n, cols, outs, rowlen, elsize, n_cols, total_host);
+  if (rc != FX_OK) return rc;
+  if (n > 0 && !scratch) return fail(FX_E_INVALID, "fx_compact_rows: null mask/scratch");
+  if (scratch_bytes < fx_compact_rows_scratch_bytes(n)) return fail(FX_E_INVALID, "fx_compact_rows: scratch too small");
   if (n == 0) {
     *total_host = 0;
     return FX_OK;

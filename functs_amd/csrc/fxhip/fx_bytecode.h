@@ -18,6 +18,7 @@
 #define FX_MAXR 6        // max rank of a region output (root coordinates)
 #define FX_V 4           // elements per lane
 #define FX_BLOCK 256     // threads per workgroup (4 wavefronts of 64)
+#define FX_STATIC_MAX_ROWS (1 << 22)  // most rows fx_compact_rows_static takes (64 KiB of tile counts per GPU)
 #define FX_TILE (FX_V * FX_BLOCK)
 #define FX_ITEM (FX_V * 64)  // elements one wave processes per work item
 #define FX_UNIT (16 * FX_ITEM)  // dense kernel: elements of the largest work unit (4 waves x 4 items)

@@ -284,6 +284,48 @@ hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* co
   return hipGetLastError();
 }
 
+// --------------------------------------------------------------------------
+// Tile counts of fx_compact_rows_static: device memory that exists from the moment the code
+// object is loaded, so the call allocates nothing.  One copy per GPU, at its own address;
+// every call on a GPU shares it.  Nothing in it has to start at zero: fx_rows_count writes
+// the count of every tile of the call and fx_rows_scan the word behind them before anything
+// reads them.
+// --------------------------------------------------------------------------
+#define FX_STATIC_SCRATCH_WORDS (FX_STATIC_MAX_ROWS / FX_BLOCK + 2)
+static __device__ __align__(256) uint32_t fx_static_scratch[FX_STATIC_SCRATCH_WORDS];
+
+#define FX_STATIC_MAX_DEVICES 64
+static std::mutex g_static_mu;
+static uint32_t* g_static_ptr[FX_STATIC_MAX_DEVICES];  // device address of the array, per GPU
+
+// The array's name is a host-side handle, not a device address: the address on the current
+// device is looked up once and kept.
+static hipError_t static_scratch(uint32_t** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= FX_STATIC_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> g(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(fx_static_scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_static_ptr[dev] = (uint32_t*)p;
+  }
+  *out = g_static_ptr[dev];
+  return hipSuccess;
+}
+
+hipError_t fx_launch_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                                         const int32_t* rowlen, const int32_t* elsize, int n_cols,
+                                         uint32_t* total_host, hipStream_t stream) {
+  uint32_t* counts = nullptr;
+  hipError_t e = static_scratch(&counts);
+  if (e != hipSuccess) return e;
+  return fx_launch_compact_rows(mask, n, cols, outs, rowlen, elsize, n_cols, counts, total_host, stream);
+}
+
 hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream) {
   fx_copy_f4<<<grid, FX_BLOCK, 0, stream>>>((const float4*)src, (float4*)dst, bytes / 16);
   return hipGetLastError();

@@ -237,6 +237,17 @@ int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, voi
                     const int32_t* rowlen, const int32_t* elsize, int n_cols, void* scratch,
                     size_t scratch_bytes, uint32_t* total_host, void* stream);
 size_t fx_compact_rows_scratch_bytes(int64_t n);
+/* fx_compact_rows for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as fx_compact_rows without the scratch pair: the
+ * tile counts live in a fixed 64 KiB device array of the library (one per GPU, held until
+ * the process ends), and the call allocates and frees nothing.  n above
+ * FX_COMPACT_ROWS_STATIC_MAX returns FX_E_LIMIT.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (different streams, no ordering between them) race. */
+#define FX_COMPACT_ROWS_STATIC_MAX 4194304 /* rows */
+int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
+                           const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* total_host,
+                           void* stream);
 
 /* ---- device utilities ---- */
 int fx_device_count(void);

@@ -64,22 +64,65 @@ def build_workload(name, dev):
     return desc, calls, cpu_args
 
 
-class Workload:
-    """Binds the regions of one config to resident inputs."""
+COLD_BYTES = 640 << 20   # the buffer sets of a workload together: well above the 256 MB last-level cache
+MAX_SETS = 64
 
-    def __init__(self, name, dev):
+
+class Workload:
+    """Binds the regions of one config to resident inputs: `sets` independent copies of the
+    inputs, outputs and scratch (set 0 is the one the latency loops use; the others exist so
+    that timed kernels can be rotated over more memory than the caches hold)."""
+
+    def __init__(self, name, dev, sets=1):
+        import torch
         self.name = name
         self.desc, calls, self.cpu_args = build_workload(name, dev)
-        self.bound = []
-        prev_out = None
-        for region, args in calls:
+        self.calls = calls
+        self.dev = dev
+        self.sets = []
+        self._bind_set([args for _, args in calls])
+        self.bound = self.sets[0]
+        self.launches = sum(bc.plan.launches for bc in self.bound)
+        for _ in range(sets - 1):
+            self.add_set()
+
+    def _bind_set(self, args_per_call):
+        bound, prev_out = [], None
+        for (region, _), args in zip(self.calls, args_per_call):
             if args is None:  # consumes the previous region's outputs
                 args = prev_out
             bc = region.bind(*args)
-            self.bound.append(bc)
+            bound.append(bc)
             bc.launch()
             prev_out = bc.results()
-        self.launches = sum(bc.plan.launches for bc in self.bound)
+        self.sets.append(bound)
+
+    def add_set(self):
+        import torch
+        clone = lambda a: a.clone() if isinstance(a, torch.Tensor) else a
+        self._bind_set([None if args is None else [clone(a) for a in args] for _, args in self.calls])
+
+    def touched_bytes(self):
+        """Device memory one call of one set reads or writes (inputs, outputs at their
+        allocated size, scratch)."""
+        import torch
+        n = 0
+        for bc in self.bound:
+            for a in bc.args:
+                for t in (a if isinstance(a, (list, tuple)) else [a]):
+                    if isinstance(t, torch.Tensor):
+                        n += t.numel() * t.element_size()
+            for row in bc.outs:
+                n += sum(t.numel() * t.element_size() for t in row)
+            if bc.scratch is not None:
+                n += bc.scratch.numel()
+        return n
+
+    def grow_cold(self):
+        want = min(MAX_SETS, max(4, -(-COLD_BYTES // max(self.touched_bytes(), 1))))
+        while len(self.sets) < want:
+            self.add_set()
+        return len(self.sets)
 
     def step(self):
         out = None
@@ -93,6 +136,21 @@ class Workload:
         for bc in self.bound:
             t += bc.launch_timed(repeat=repeat)
         return t
+
+    def cold_times_ms(self, rounds):
+        """Per kernel of the call, and per region (all its kernels in order), the mean duration
+        when consecutive launches rotate over the buffer sets."""
+        from functs_amd.region import timed_sets
+        flush(self.dev)
+        per_kernel, per_region = [], []
+        for i in range(len(self.bound)):
+            col = [s[i] for s in self.sets]
+            for k in range(col[0].plan.launches):
+                per_kernel.append(timed_sets(col, which=k, rounds=rounds))
+                flush(self.dev)
+            per_region.append(timed_sets(col, which=-1, rounds=rounds))
+            flush(self.dev)
+        return per_kernel, per_region
 
     def algorithmic_bytes(self):
         """Inputs read once + outputs written once for the fused call
@@ -111,17 +169,30 @@ class Workload:
         return total
 
 
+_FLUSH = {}
+
+
+def flush(dev):
+    """Streams 1 GiB through the library's copy kernel: what the caches held before is gone."""
+    import torch
+    from functs_amd import _lib
+    if dev not in _FLUSH:
+        _FLUSH[dev] = (torch.ones(512 << 18, dtype=torch.float32, device=dev), torch.empty(512 << 18, dtype=torch.float32, device=dev))
+    _lib.copy_bytes(*_FLUSH[dev])
+
+
 def recorded_traffic(kernel, workload):
     """HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter
-    summary of this kernel and workload, or None when none is recorded."""
-    path = os.path.join(ROOT, "profiles", "%s_%s_hbm_traffic.md" % ("fx_compact_scatter", workload))
+    summary of this kernel and workload (counter runs are separate rocprofv3 runs, so the
+    figure is read from the summary, not measured in this run), or None when none is recorded."""
+    path = os.path.join(ROOT, "profiles", "%s_%s_hbm_traffic.md" % (kernel, workload))
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch %s:" % kernel):
-                return int(line.split(":")[1])
+                return int(line.split(":")[1]), os.path.relpath(path, ROOT)
     except OSError:
         pass
-    return None
+    return None, None
 
 
 def measure(w, steps, warmup):
@@ -150,10 +221,14 @@ def measure(w, steps, warmup):
     return ms, kern, single
 
 
-def torchscript_route(name, cpu_args, dev, steps, warmup):
+def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0):
     """Per-call wall time of the same config through functs_amd.jit: the scripted
     program, functionalized, with its regions run by tssa::ParallelFunctor
-    (output allocation, launches and the kept-row synchronisation included)."""
+    (output allocation, launches and the kept-row synchronisation included).
+    With cold_bytes, consecutive calls rotate over copies of the inputs and the outputs of
+    the last calls are kept alive, so that the allocator hands out other blocks: the calls
+    then work on memory that the caches do not hold (returned beside the warm figures)."""
+    import collections
     import torch
     import functs_amd.jit as fj
     from functs_amd.benchmark import PROGRAMS
@@ -178,7 +253,28 @@ def torchscript_route(name, cpu_args, dev, steps, warmup):
         torch.cuda.synchronize()
     sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
     n_functors = str(fn.graph).count("= tssa::ParallelFunctor")
-    return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us
+    cold_us = cold_sync_us = None
+    if cold_bytes:
+        in_bytes = sum(a.numel() * a.element_size() for a in args if isinstance(a, torch.Tensor))
+        n_sets = min(MAX_SETS, max(4, -(-cold_bytes // max(2 * in_bytes, 1))))
+        sets = [[a.clone() if isinstance(a, torch.Tensor) else a for a in args] for _ in range(n_sets)]
+        ring = collections.deque(maxlen=n_sets)
+        for i in range(max(warmup, n_sets)):
+            ring.append(fn(*sets[i % n_sets]))
+        torch.cuda.synchronize()
+        flush(dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            ring.append(fn(*sets[i % n_sets]))
+        torch.cuda.synchronize()
+        cold_us = (time.perf_counter() - t0) * 1e6 / steps
+        t0 = time.perf_counter()
+        for i in range(n_sync):
+            ring.append(fn(*sets[i % n_sets]))
+            torch.cuda.synchronize()
+        cold_sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
+    return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us, cold_us, cold_sync_us
 
 
 def cpu_baseline(name, budget_s):
@@ -227,18 +323,33 @@ def main():
         w = Workload(name, dev)
         ms, kern, single = measure(w, args.steps, args.warmup)
         alg = w.algorithmic_bytes()
-        dom = max(kern)
+        # the same kernels with consecutive launches rotated over buffer sets that together
+        # exceed the last-level cache: every launch reads and writes cold lines
+        n_sets = w.grow_cold()
+        rounds = max(2, min(10, -(-40 // n_sets)))
+        cold, cold_regions = w.cold_times_ms(rounds)
+        dom_i = max(range(len(cold)), key=lambda i: cold[i])
+        dom = cold[dom_i]
+        frac = lambda ms_: round(alg / (ms_ * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
         rec = {
             "workload": w.desc,
             "latency_us": round(ms * 1e3, 2),
-            "kernel_us": [round(k * 1e3, 2) for k in kern],
+            "kernel_us": [round(k * 1e3, 2) for k in cold],
+            "kernel_us_warm": [round(k * 1e3, 2) for k in kern],
             "kernel_us_single_launch": [round(k * 1e3, 2) for k in single],
+            "call_kernels_us": round(sum(cold_regions) * 1e3, 2),
+            "cold_sets": n_sets,
+            "cold_bytes": n_sets * w.touched_bytes(),
             "launches_per_call": w.launches,
             "row_compaction": any(bc.plan.compact for bc in w.bound),
             "algorithmic_bytes": alg,
+            "dominant_kernel_index": dom_i,
             "gbps_dominant_kernel": round(alg / (dom * 1e-3) / 1e9, 1),
-            "gbps_all_kernels": round(alg / (sum(kern) * 1e-3) / 1e9, 1),
-            "frac_hbm_peak": round(alg / (dom * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "gbps_all_kernels": round(alg / (sum(cold_regions) * 1e-3) / 1e9, 1),
+            "frac_hbm_peak": frac(dom),
+            "frac_hbm_peak_warm": frac(kern[dom_i]),
+            "frac_hbm_peak_call": frac(sum(cold_regions)),
+            "frac_hbm_peak_call_warm": frac(sum(kern)),
         }
         rec["compiled_kernels"] = all(bc.region.specialized(*bc.args) for bc in w.bound)
         if rec["compiled_kernels"]:
@@ -247,9 +358,12 @@ def main():
             _, ikern, _ = measure(w, max(args.steps // 4, 5), 3)
             aot.enable(True)
             rec["interpreter_kernel_us"] = [round(k * 1e3, 2) for k in ikern]
-        ts_us, n_functors, spec_share, sync_us = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup)
-        rec["torchscript_route_latency_us"] = round(ts_us, 2)
-        rec["torchscript_route_drained_latency_us"] = round(sync_us, 2)
+        ts_us, n_functors, spec_share, sync_us, cold_us, cold_sync_us = torchscript_route(
+            name, w.cpu_args, dev, args.steps, args.warmup, COLD_BYTES)
+        rec["torchscript_route_latency_us"] = round(cold_us, 2)
+        rec["torchscript_route_drained_latency_us"] = round(cold_sync_us, 2)
+        rec["torchscript_route_latency_us_warm"] = round(ts_us, 2)
+        rec["torchscript_route_drained_latency_us_warm"] = round(sync_us, 2)
         rec["torchscript_route_functors"] = n_functors
         rec["torchscript_route_compiled_share"] = round(spec_share, 3)
         if with_cpu:
@@ -273,7 +387,7 @@ def main():
         select_rev of `out`.  Only the TorchScript route exists for it."""
         from functs_amd.benchmark.inputs import INPUTS
         cpu_args = INPUTS["c4"](0)
-        us, n_functors, spec_share, _ = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
+        us, n_functors, spec_share, _, _, _ = torchscript_route("c4", cpu_args, dev, max(args.steps // 10, 5), 2)
         # the same call replayed as one HIP graph (functs_amd.jit.build(..., hip_graph=True))
         import functs_amd.jit as fj
         from functs_amd.benchmark import PROGRAMS
@@ -344,11 +458,13 @@ def main():
         except Exception as e:
             per["c4"] = {"error": str(e)[:200]}
     cpu_us, cpu_n, cores = head.pop("cpu")
-    dom_ms = max(head["kernel_us"]) / 1e3
+    dom_ms = head["kernel_us"][head["dominant_kernel_index"]] / 1e3
     dom_kernel = "fx_compact_scatter" if head["row_compaction"] else "fx_region_dense"
+    traffic, traffic_src = recorded_traffic(dom_kernel, args.workload)
     out = {
         "metric": "per-call latency",
         "value": head["torchscript_route_latency_us"],
+        "value_kind": "back-to-back: K calls between two device synchronisations, consecutive calls on rotated copies of the inputs and on fresh output blocks (cold caches); drained_latency_us: the device drained after every call; *_warm: every call on the same buffers",
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,
@@ -363,14 +479,28 @@ def main():
                    "route": "functs_amd.jit.script -> build -> tssa::ParallelFunctor (C++ operator over the C ABI)",
                    "compiled_kernels": head["compiled_kernels"] and not args.interpreter,
                    "drained_latency_us": head["torchscript_route_drained_latency_us"],
+                   "latency_us_warm": head["torchscript_route_latency_us_warm"],
+                   "drained_latency_us_warm": head["torchscript_route_drained_latency_us_warm"],
                    "region_api_latency_us": head["latency_us"], "launches_per_call": head["launches_per_call"],
-                   "kernel_us": head["kernel_us"], "gbps_all_kernels": head["gbps_all_kernels"]},
+                   "kernel_us": head["kernel_us"], "kernel_us_warm": head["kernel_us_warm"],
+                   "gbps_all_kernels": head["gbps_all_kernels"]},
         "roofline": {"bound": "hbm", "achieved": head["gbps_dominant_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": head["frac_hbm_peak"], "traffic": recorded_traffic(dom_kernel, args.workload),
+                     "frac": head["frac_hbm_peak"], "frac_warm": head["frac_hbm_peak_warm"],
+                     "frac_call": head["frac_hbm_peak_call"], "frac_call_warm": head["frac_hbm_peak_call_warm"],
+                     "traffic": traffic,
+                     "traffic_source": ("%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs; not measured in this run)" % traffic_src)
+                     if traffic_src else None,
                      "kernel": dom_kernel,
                      "algorithmic_bytes": head["algorithmic_bytes"], "kernel_ms": round(dom_ms, 5),
-                     "kernel_ms_single_launch": round(max(head["kernel_us_single_launch"]) / 1e3, 5),
-                     "timing": "HIP events on the launch stream around %d back-to-back launches of the kernel, mean per launch" % KERNEL_BATCH},
+                     "kernel_ms_warm": round(head["kernel_us_warm"][head["dominant_kernel_index"]] / 1e3, 5),
+                     "call_kernels_ms": round(head["call_kernels_us"] / 1e3, 5),
+                     "kernel_ms_single_launch": round(head["kernel_us_single_launch"][head["dominant_kernel_index"]] / 1e3, 5),
+                     "cold_sets": head["cold_sets"], "cold_bytes": head["cold_bytes"],
+                     "timing": "HIP events on the launch stream around back-to-back launches, mean per launch. frac / kernel_ms: "
+                               "the dominant kernel rotated over cold_sets independent sets of inputs, outputs and scratch "
+                               "(cold_bytes in total, above the 256 MB last-level cache), the caches flushed before; "
+                               "frac_warm / kernel_ms_warm: %d launches on one set; frac_call / call_kernels_ms: every kernel of "
+                               "the call in order, rotated the same way; frac_call_warm: sum of the warm kernels" % KERNEL_BATCH},
         "cpu_baseline": {"value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
                          "sample": "%d calls of torch.jit.script(%s) on the same seeded CPU tensors" % (cpu_n, args.workload)},
         "per_config": per,

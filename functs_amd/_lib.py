@@ -130,6 +130,9 @@ _sig("fx_region_run_timed", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POIN
      ctypes.POINTER(ctypes.c_float), _i, _ip)
 _sig("fx_region_run_timed_batched", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp, _i,
      ctypes.POINTER(ctypes.c_float), _i, _ip)
+_sig("fx_region_run_timed_sets", _i, _vp, _vp, _i, ctypes.POINTER(ctypes.POINTER(FxArg)), _i,
+     ctypes.POINTER(ctypes.POINTER(_vp)), ctypes.POINTER(_vp), ctypes.POINTER(_vp), _vp, _i, _i,
+     ctypes.POINTER(ctypes.c_float))
 _sig("fx_compact_rows", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, ctypes.c_size_t, _vp, _vp)
 _sig("fx_compact_rows_scratch_bytes", ctypes.c_size_t, ctypes.c_int64)

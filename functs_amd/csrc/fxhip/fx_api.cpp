@@ -17,6 +17,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "fx_lower.h"
 
@@ -491,6 +492,69 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     for (auto& e : ev) (void)hipEventDestroy(e);
     if (n_kernels) *n_kernels = nk;
   }
+  return FX_OK;
+}
+
+// Launches over several argument sets of one plan in rotation, inside ONE event pair:
+// `which` < 0 launches every kernel of the call in order (a whole call per set), otherwise only
+// kernel `which` of the call (the others must have run on every set before: a kernel of a
+// compacting region reads what the count pass of its own set left in that set's scratch).
+// With sets that together exceed the last-level cache every launch works on cold lines.
+int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, const fx_arg* const* args, int n_args,
+                             void* const* const* out_ptrs, void* const* scratch, uint32_t* const* totals_host,
+                             void* stream_, int which, int rounds, float* ms_mean) {
+  if (!reg || !plan || !args || !out_ptrs || !ms_mean) return fail(FX_E_INVALID, "null argument");
+  if (n_sets < 1 || n_sets > 64 || rounds < 1 || rounds > 1000)
+    return fail(FX_E_INVALID, "fx_region_run_timed_sets: 1..64 sets, 1..1000 rounds");
+  fx::Plan* pl = const_cast<fx::Plan*>(P(plan));
+  if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
+  if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
+  if (which >= pl->launches) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
+  const bool compact = pl->mode == FX_MODE_COMPACT;
+  if (compact && (!scratch || !totals_host)) return fail(FX_E_INVALID, "compacting region needs scratch and totals per set");
+  hipStream_t stream = (hipStream_t)stream_;
+  // one untimed call per set: uploads the descriptor, leaves every set's scratch valid
+  for (int i = 0; i < n_sets; ++i) {
+    const int rc = run_impl(reg, plan, args[i], n_args, out_ptrs[i], compact ? scratch[i] : nullptr,
+                            compact ? totals_host[i] : nullptr, stream_, nullptr, 0, nullptr);
+    if (rc != FX_OK) return rc;
+  }
+  std::vector<FxDyn> dyn((size_t)n_sets);
+  for (int i = 0; i < n_sets; ++i) {
+    memset(&dyn[i], 0, sizeof(FxDyn));
+    const int rc = fill_dyn(pl, args[i], out_ptrs[i], compact ? scratch[i] : nullptr, compact ? totals_host[i] : nullptr,
+                            pl->dev_blob, &dyn[i]);
+    if (rc != FX_OK) return rc;
+  }
+  const uint32_t* sb = (const uint32_t*)pl->dev_blob;
+  FxLaunchInfo li;
+  li.blob_words = (uint32_t)pl->blob.size();
+  li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
+  li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
+  li.n_temps = pl->n_temps;
+  li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
+  const FxSpecKernels* spec = spec_of(pl);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  HIP_OK(hipEventCreate(&e0));
+  HIP_OK(hipEventCreate(&e1));
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipEventRecord(e0, stream));
+  for (int r = 0; r < rounds; ++r)
+    for (int i = 0; i < n_sets; ++i) {
+      if (!compact) {
+        HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+      } else {
+        if (which < 0 || which == 0) HIP_OK(fx_launch_compact_count(sb, li, &dyn[i], pl->grid_count, stream, spec));
+        if (which < 0 || which == 1) HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn[i], pl->grid, stream, spec));
+      }
+    }
+  HIP_OK(hipEventRecord(e1, stream));
+  HIP_OK(hipEventSynchronize(e1));
+  float ms = 0.f;
+  HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  *ms_mean = ms / (float)(rounds * n_sets);
   return FX_OK;
 }
 

@@ -365,6 +365,27 @@ class BoundCall:
         return [row[0] for row in outs]
 
 
+def timed_sets(bound, which=-1, rounds=1, stream=None):
+    """Mean duration in milliseconds of a call (which < 0) or of kernel `which` of a call,
+    launched over the BoundCalls in `bound` in rotation inside one HIP event pair
+    (fx_region_run_timed_sets).  All of them must come from the same region and plan."""
+    b0 = bound[0]
+    assert all(b.region is b0.region and b.plan.handle.value == b0.plan.handle.value for b in bound)
+    if stream is None:
+        stream = torch.cuda.current_stream(b0.device).cuda_stream
+    k = len(bound)
+    args = (ctypes.POINTER(FxArg) * k)(*[ctypes.cast(b.arr, ctypes.POINTER(FxArg)) for b in bound])
+    outs = (ctypes.POINTER(ctypes.c_void_p) * k)(*[ctypes.cast(b.ptrs, ctypes.POINTER(ctypes.c_void_p)) for b in bound])
+    scr = (ctypes.c_void_p * k)(*[b.scratch.data_ptr() if b.scratch is not None else None for b in bound])
+    tot = (ctypes.c_void_p * k)(*[b.totals.data_ptr() if b.totals is not None else None for b in bound])
+    ms = ctypes.c_float()
+    check(lib.fx_region_run_timed_sets(b0.region._h, b0.plan.handle, k, args, b0.n, outs, scr, tot,
+                                       ctypes.c_void_p(stream), int(which), int(rounds), ctypes.byref(ms)))
+    for b in bound:
+        b._stream = stream
+    return ms.value
+
+
 def compact_rows(mask, cols):
     """Stand-alone ``[c[mask] for c in cols]`` through fx_compact_rows."""
     n = mask.numel()

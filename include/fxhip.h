@@ -222,6 +222,18 @@ int fx_region_run_timed_batched(fx_region*, const fx_plan*, const fx_arg* args, 
                                 void* scratch, uint32_t* totals_host, void* stream, int repeat, float* kernel_ms,
                                 int cap, int* n_kernels);
 
+/* The kernels of a call launched over n_sets argument sets of one plan in rotation (set 0,
+ * 1, ..., n_sets-1, `rounds` times) inside ONE event pair on `stream`; *ms_mean is the mean
+ * per launched call (which < 0: every kernel of the call, in order) or per launch of kernel
+ * `which` of the call alone (0 .. fx_plan_launches-1).  Each set brings its own inputs, outputs,
+ * scratch and totals; with sets that together exceed the last-level cache (256 MB) every
+ * launch reads and writes cold lines, which the same buffers launched back to back do not.
+ * Every set is run once untimed first.  Measurement aid of the benchmark
+ * (the reference: functs/utils/evaluate.py:172-208 times whole calls on one input). */
+int fx_region_run_timed_sets(fx_region*, const fx_plan*, int n_sets, const fx_arg* const* args, int n_args,
+                             void* const* const* out_ptrs, void* const* scratch, uint32_t* const* totals_host,
+                             void* stream, int which, int rounds, float* ms_mean);
+
 /* The argument marshalling of fx_region_run without the launch (host only; the
  * analogue of GraphBuilder::prepareRunArgs, graph_builder.cpp:718-899).
  * dyn_out receives fx_dyn_bytes() bytes: the by-value block the kernels read. */

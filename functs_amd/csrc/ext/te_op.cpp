@@ -506,6 +506,9 @@ class RegionRunner {
       ws = var->take(fx_plan_scratch_bytes(plan), degree, device, (void*)stream.stream());
       ws.stream = (void*)stream.stream();
     }
+    // checked int64 loads of an earlier launch (integer arithmetic in regions is 32-bit)
+    TORCH_CHECK(!fx_async_error(1), "tssa::ParallelFunctor: an earlier fused region read an int64 element outside 32 bits "
+                "into integer arithmetic; its results are not valid (moves of int64 data are exact, arithmetic is 32-bit)");
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));

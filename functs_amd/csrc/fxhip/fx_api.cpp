@@ -347,6 +347,34 @@ int fx_device_count(void) {
   return n;
 }
 
+// Error word of checked int64 loads (fx_bytecode.h FX_I64): one word of pinned host memory
+// that every device can write; without a device (host-only marshalling for the emulator) a
+// plain word stands in.
+static std::mutex g_err_mu;
+static uint32_t* g_err_pinned = nullptr;
+static uint32_t g_err_plain = 0;
+static uint32_t* err_word(bool pinned) {
+  std::lock_guard<std::mutex> g(g_err_mu);
+  if (g_err_pinned) return g_err_pinned;
+  if (!pinned) return &g_err_plain;
+  void* p = nullptr;
+  if (hipHostMalloc(&p, 64, hipHostMallocPortable | hipHostMallocMapped) != hipSuccess) return nullptr;
+  g_err_pinned = (uint32_t*)p;
+  *g_err_pinned = 0;
+  return g_err_pinned;
+}
+
+int fx_async_error(int clear) {
+  std::lock_guard<std::mutex> g(g_err_mu);
+  uint32_t v = g_err_plain;
+  if (g_err_pinned) v |= *(volatile uint32_t*)g_err_pinned;
+  if (clear) {
+    g_err_plain = 0;
+    if (g_err_pinned) *(volatile uint32_t*)g_err_pinned = 0;
+  }
+  return v != 0;
+}
+
 // Fill the by-value dynamic block.  Exposed (without launching) so that host
 // tests can check the marshalling.
 // `safe`: a device address that can always be read.  Kernels clamp the address of
@@ -369,9 +397,11 @@ static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptr
       case fx::PtrSrc::FLAGS: return (uint64_t)(uintptr_t)((char*)scratch + pl->flags_off);
       case fx::PtrSrc::COUNTS: return (uint64_t)(uintptr_t)((char*)scratch + pl->counts_off);
       case fx::PtrSrc::TOTALS: return (uint64_t)(uintptr_t)totals_host;
+      case fx::PtrSrc::ERRWORD: return (uint64_t)(uintptr_t)err_word(safe != nullptr);
     }
     return 0;
   };
+  bool scalar_overflow = false;
   auto scal_of = [&](const fx::ScalSrc& s, int task) -> uint32_t {
     const fx::Value& v = R.vals[R.inputs[s.input]];
     const fx_arg& a = args[pl->arg_base[s.input] + (v.per_task ? task : 0)];
@@ -381,7 +411,9 @@ static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptr
       float f = (float)x;  // double -> float like graph_builder.cpp:850-854
       memcpy(&u, &f, 4);
     } else {
-      u = (uint32_t)(int32_t)(int64_t)x;
+      const int64_t i = v.kind == fx::VK_FLOAT ? (int64_t)a.fval : a.ival;
+      scalar_overflow = scalar_overflow || i != (int64_t)(int32_t)i;
+      u = (uint32_t)(int32_t)i;
     }
     return u;
   };
@@ -392,6 +424,8 @@ static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptr
   for (size_t i = 0; i < ns; ++i) dyn->s[i] = scal_of(pl->sscal[i], 0);
   for (int t = 0; t < T; ++t)
     for (size_t i = 0; i < nts; ++i) dyn->s[ns + t * nts + i] = scal_of(pl->tscal[i], t);
+  if (scalar_overflow) return fail(FX_E_LIMIT, "an integer scalar argument is outside 32 bits (integer arithmetic in regions is 32-bit)");
+  if (pl->uses_guard && safe && !err_word(true)) return fail(FX_E_HIP, "no pinned memory for the error word");
   return FX_OK;
 }
 

@@ -38,6 +38,14 @@ enum FxDtype : uint32_t {
   FX_U8 = 3,   // uint8 and bool
   FX_F16 = 4,
   FX_BF16 = 5,
+  // One 32-bit word of an int64 element, for programs that only move int64 data (select,
+  // slice, index, where, compaction ...): such an output is lowered twice, once per word, and
+  // is exact for every value.  FX_I64 itself stands for int64 data that takes part in 32-bit
+  // integer arithmetic: its loads check that the value fits (a value that does not sets the
+  // library's error word, fx_async_error) and its stores sign-extend; a load with FX_F_I2F
+  // converts the whole 64-bit value.
+  FX_I64LO = 6,
+  FX_I64HI = 7,
 };
 
 // value classes inside the VM (32-bit registers)
@@ -224,7 +232,8 @@ struct FxHeader {
   uint32_t slot_flags, slot_counts, slot_total;  // shared pointer slots used by compaction
   uint32_t total_words;
   uint32_t max_rows;     // stride of the per-task row-flag table
-  uint32_t pad[3];
+  uint32_t slot_err;     // 1 + shared pointer slot of the error word that FX_I64 loads report to (0: none)
+  uint32_t pad[2];
 };
 
 // dynamic (per call) arguments, passed by value in the kernarg segment

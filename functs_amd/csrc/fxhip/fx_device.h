@@ -34,6 +34,7 @@ struct FxCtx {
   uint32_t* temps;        // LDS, this lane's column: temps[(slot * FX_V + j) * FX_BLOCK]
   uint32_t wseg;          // lanes per segment of the wave reductions (rows per wave = 64 / wseg)
   int task;
+  uint64_t err;           // error word that guarded int64 loads report to (0: the region has none)
 };
 
 // Data buffers are plain device allocations: address them through the global
@@ -48,7 +49,7 @@ struct FxCtx {
 // element 0 of the buffer and end up with an unspecified value, like after any
 // arithmetic instruction; the host never passes a buffer without an element 0.
 __device__ __forceinline__ void fx_load_vec(uint64_t base_, const int32_t (&off)[FX_V], uint32_t M, uint32_t dt,
-                                            bool cvt, bool consecutive, uint32_t (&out)[FX_V]) {
+                                            bool cvt, bool consecutive, uint32_t (&out)[FX_V], uint64_t err = 0) {
   const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)base_;
   const uint32_t VM = (1u << FX_V) - 1u;
   // FX_V consecutive 32-bit elements in every lane that is live at all, and at least
@@ -71,9 +72,29 @@ __device__ __forceinline__ void fx_load_vec(uint64_t base_, const int32_t (&off)
   if (dt == FX_F32 || dt == FX_I32) {
 #pragma unroll
     for (int j = 0; j < FX_V; ++j) out[j] = *(const FX_AS1 uint32_t*)(base + (o[j] << 2));
-  } else if (dt == FX_I64) {  // values fit 32 bits: the low word is the value
+  } else if (dt == FX_I64) {
+    // int64 data in 32-bit arithmetic: the whole element is read.  Converted to float it is
+    // exact; as an integer the low word is the value, and an element that does not fit 32 bits
+    // is reported through the error word (the result of this launch is then not to be used).
+    uint64_t w[FX_V];
 #pragma unroll
-    for (int j = 0; j < FX_V; ++j) out[j] = *(const FX_AS1 uint32_t*)(base + (o[j] << 3));
+    for (int j = 0; j < FX_V; ++j) w[j] = *(const FX_AS1 uint64_t*)(base + (o[j] << 3));
+    if (cvt) {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) out[j] = f2u((float)(int64_t)w[j]);
+      return;
+    }
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) {
+      out[j] = (uint32_t)w[j];
+      bad = bad || (((M >> j) & 1u) && (int64_t)w[j] != (int64_t)(int32_t)(uint32_t)w[j]);
+    }
+    if (bad && err) __hip_atomic_store((uint32_t*)err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  } else if (dt == FX_I64LO || dt == FX_I64HI) {
+    const uint32_t hi = dt == FX_I64HI ? 4u : 0u;
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = *(const FX_AS1 uint32_t*)(base + (o[j] << 3) + hi);
   } else if (dt == FX_U8) {
 #pragma unroll
     for (int j = 0; j < FX_V; ++j) out[j] = base[o[j]];
@@ -105,6 +126,8 @@ __device__ __forceinline__ void fx_store(uint64_t base_, uint32_t o, uint32_t dt
     case FX_I64:
       *(FX_AS1 int64_t*)(base + (o << 3)) = (vt == FX_VT_I) ? (int64_t)(int32_t)v : (int64_t)u2f(v);
       break;
+    case FX_I64LO: *(FX_AS1 uint32_t*)(base + (o << 3)) = v; break;
+    case FX_I64HI: *(FX_AS1 uint32_t*)(base + (o << 3) + 4u) = v; break;
     case FX_U8: base[o] = (vt == FX_VT_I) ? (uint8_t)v : (uint8_t)(u2f(v) != 0.0f); break;
     case FX_F16: {
       __half hv = __float2half(vt == FX_VT_F ? u2f(v) : (float)(int32_t)v);
@@ -377,7 +400,7 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
       } else {
         int32_t off[FX_V];
         const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
-        fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B);
+        fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B, cx.err);
       }
     }
 
@@ -389,7 +412,7 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
         int32_t off[FX_V];
         const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
         if (op == FX_LDA) {
-          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, A);
+          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, A, cx.err);
         } else {
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
@@ -405,7 +428,7 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
         int32_t off[FX_V];
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) off[j] = (int32_t)A[j] + (int32_t)imm;
-        fx_load_vec(fx_ptr(cx, ia), off, M, dt, false, false, A);
+        fx_load_vec(fx_ptr(cx, ia), off, M, dt, false, false, A, cx.err);
       } break;
       case FX_IMMA:
 #pragma unroll
@@ -773,6 +796,7 @@ struct FxLead {
   int32_t cf[FX_MAXR];
   int32_t base;
   uint64_t p;
+  uint64_t err;
   uint32_t dt;
   bool cvt;
 };
@@ -796,6 +820,7 @@ __device__ __forceinline__ FxLead fx_lead_decode(const FxCtx& cx, int pc) {
   }
   ld.base = (int32_t)uni(a1.y) + (int32_t)uni(a1.x) * cx.task;
   ld.p = fx_ptr(cx, (int32_t)w.y);
+  ld.err = cx.err;
   return ld;
 }
 
@@ -803,7 +828,7 @@ template <int R>
 __device__ __forceinline__ void fx_lead_load(const FxLead& ld, const FxCoord<R>& q, uint32_t M, uint32_t (&P)[FX_V]) {
   int32_t off[FX_V];
   const bool consecutive = fx_offsets<R>(q, ld.cf, ld.base, off);
-  fx_load_vec(ld.p, off, M, ld.dt, ld.cvt, consecutive, P);
+  fx_load_vec(ld.p, off, M, ld.dt, ld.cvt, consecutive, P, ld.err);
 }
 
 // Leading loads of a batch of KP items, all in flight together.  When every item of the
@@ -974,6 +999,12 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
   cx.temps = L + la.temps_off + threadIdx.x;
   cx.wseg = 64;
   cx.task = w.task;
+  const uint32_t se = uni(L[FX_W(FxHeader, slot_err)]);
+  cx.err = 0;
+  if (se) {
+    const uint64_t p = cx.ptrs[se - 1u];
+    cx.err = ((uint64_t)uni((uint32_t)(p >> 32)) << 32) | (uint64_t)uni((uint32_t)p);
+  }
   return cx;
 }
 

@@ -231,7 +231,7 @@ struct SlotAlloc {
   }
 };
 
-struct Prog { uint32_t begin, end, vt; bool rowwave; };
+struct Prog { uint32_t begin, end, vt; bool rowwave; bool wide; };
 
 class Lowerer {
  public:
@@ -243,8 +243,13 @@ class Lowerer {
   int maxTemps = 0;
   bool allowRowWave = false;  // dense outputs only: a reduction over the last dim may use wave-wide ops
 
+  bool usesGuard = false;     // some program loads int64 data into 32-bit arithmetic (checked loads)
+
   Shape shapeOf(int vid);
-  Prog lower(int vid, const Shape& rootShape);
+  // half: which 32-bit word of an int64 output the program delivers (0 low, 1 high).  Prog::wide
+  // says that the low-word program moved int64 data as it is, so that the high words need a
+  // program of their own; otherwise the result fits 32 bits and its store sign-extends.
+  Prog lower(int vid, const Shape& rootShape, int half = 0);
 
  private:
   const Region& R_;
@@ -264,6 +269,22 @@ class Lowerer {
   bool loopVarBound_ = false;
   IdxExpr loopVar_;
   bool usedRowWave_ = false;
+  // int64 outputs: while only movement operators (views, *_rev merges, cat, index, where ...)
+  // lie between a value and the output, the value travels word by word and is exact
+  bool moveCtx_ = false;
+  int half_ = 0;
+  bool sawWide_ = false;
+  struct ArithCtx {   // operands of arithmetic: 32-bit values, int64 loads are checked
+    Lowerer& l; bool m; int h;
+    explicit ArithCtx(Lowerer& l_) : l(l_), m(l_.moveCtx_), h(l_.half_) { l.moveCtx_ = false; l.half_ = 0; }
+    ~ArithCtx() { l.moveCtx_ = m; l.half_ = h; }
+  };
+  void signExtendA() { emitI(FX_ILT, 0, 0, 0, FX_F_IMM); emitI(FX_INEG); }   // A = A < 0 ? -1 : 0
+  static uint32_t imm32(int64_t x, const char* what) {
+    FX_CHECK(x >= std::numeric_limits<int32_t>::min() && x <= std::numeric_limits<int32_t>::max(), FX_E_UNSUPPORTED,
+             what << ": integer constant " << x << " outside 32 bits in integer arithmetic (only moves of int64 data are 64-bit)");
+    return (uint32_t)(int32_t)x;
+  }
   // true when coordinate `d` of frame f is exactly the innermost root coordinate, nothing else
   // in the frame moves with it, and the whole extent fits one wave item
   bool rowWaveFrame(const Frame& f, int d, int64_t extent) const;
@@ -317,6 +338,7 @@ class Lowerer {
     int slot = 0; uint32_t dt = 0; IdxExpr addr;
     // imm
     uint32_t imm = 0;
+    int64_t imm64 = 0;       // integer constants: the whole value
     // affval
     IdxExpr val;
   };
@@ -325,6 +347,7 @@ class Lowerer {
   void emit(int vid, const Frame& f);                  // -> A, in the value's own class
   void emitAs(int vid, const Frame& f, uint32_t vt);   // -> A, converted to vt
   void emitOp(const Res& r);
+  void emitOpBody(const Res& r);
   void convertA(uint32_t from, uint32_t to) {
     if (from == to) return;
     emitI(from == FX_VT_I ? FX_I2F : FX_F2I);
@@ -992,7 +1015,11 @@ Lowerer::Res Lowerer::resolve(int vid, Frame f) {
           uint32_t vt = vt_of(v.dtype);
           if (post_i2f) { r.imm = fbits((float)(int64_t)x); r.vt = FX_VT_F; }
           else if (vt == FX_VT_F) { r.imm = fbits((float)x); r.vt = FX_VT_F; }
-          else { r.imm = (uint32_t)(int32_t)(v.dtype == FX_DT_BOOL ? (x != 0) : (int64_t)x); r.vt = FX_VT_I; }
+          else {
+            r.imm64 = v.dtype == FX_DT_BOOL ? (int64_t)(x != 0) : (sv.kind == VK_FLOAT ? (int64_t)x : sv.ival);
+            r.imm = (uint32_t)r.imm64;
+            r.vt = FX_VT_I;
+          }
           r.vid = vid;
           return r;
         }
@@ -1007,7 +1034,7 @@ Lowerer::Res Lowerer::resolve(int vid, Frame f) {
           uint32_t vt = vt_of(v.dtype);
           if (post_i2f) { r.imm = fbits((float)(int64_t)x); r.vt = FX_VT_F; }
           else if (vt == FX_VT_F) { r.imm = fbits((float)x); r.vt = FX_VT_F; }
-          else { r.imm = (uint32_t)(int32_t)(int64_t)x; r.vt = FX_VT_I; }
+          else { r.imm64 = sv.kind == VK_FLOAT ? (int64_t)x : sv.ival; r.imm = (uint32_t)r.imm64; r.vt = FX_VT_I; }
           r.vid = vid;
           return r;
         }
@@ -1046,20 +1073,44 @@ Lowerer::Res Lowerer::resolve(int vid, Frame f) {
 }
 
 void Lowerer::emitSimple(const Res& r, bool toB) {
+  // integer values on their way into an int64 output (move context): int64 data goes word by
+  // word, anything narrower is its own low word and its sign is the high word
+  const bool mv = moveCtx_ && !toB && r.vt == FX_VT_I && !r.post_i2f;
   switch (r.kind) {
-    case RK_LEAF:
+    case RK_LEAF: {
+      uint8_t dt = (uint8_t)r.dt;
+      bool sext = false;
+      if (r.dt == FX_I64 && !r.post_i2f) {
+        if (mv) { dt = half_ ? FX_I64HI : FX_I64LO; sawWide_ = true; }
+        else usesGuard = true;
+      } else if (mv && half_) {
+        sext = true;
+      }
       if (r.addr.affine()) {
-        emitI(toB ? FX_LDB : FX_LDA, r.slot, addAffine(r.addr), 0, r.post_i2f ? FX_F_I2F : 0, (uint8_t)r.dt);
+        emitI(toB ? FX_LDB : FX_LDA, r.slot, addAffine(r.addr), 0, r.post_i2f ? FX_F_I2F : 0, dt);
       } else {
         FX_CHECK(!toB, FX_E_INVALID, "indirect load into B");
-        emitIdx(r.addr);
-        emitI(FX_LDXA, r.slot, 0, 0, 0, (uint8_t)r.dt);
+        { ArithCtx a(*this); emitIdx(r.addr); }
+        if (r.post_i2f && r.dt == FX_I64) {
+          // the conversion needs the whole element: read both words and combine them as floats
+          // is not exact, so the checked 32-bit load stands here
+          usesGuard = true;
+        }
+        emitI(FX_LDXA, r.slot, 0, 0, 0, dt);
         if (r.post_i2f) emitI(FX_I2F);
       }
+      if (sext) signExtendA();
+    } break;
+    case RK_IMM:
+      if (mv && r.imm64 != (int64_t)(int32_t)r.imm) sawWide_ = true;
+      if (mv && half_) emitI(FX_IMMA, 0, 0, (uint32_t)((uint64_t)r.imm64 >> 32));
+      else {
+        if (r.vt == FX_VT_I && !mv) (void)imm32(r.imm64, "constant");
+        emitI(toB ? FX_IMMB : FX_IMMA, 0, 0, r.imm);
+      }
       break;
-    case RK_IMM: emitI(toB ? FX_IMMB : FX_IMMA, 0, 0, r.imm); break;
-    case RK_SCALAR: emitI(toB ? FX_SCLB : FX_SCLA, r.slot); break;
-    case RK_AFFVAL: emitIdx(r.val, toB, r.post_i2f); break;
+    case RK_SCALAR: emitI(toB ? FX_SCLB : FX_SCLA, r.slot); if (mv && half_) signExtendA(); break;
+    case RK_AFFVAL: emitIdx(r.val, toB, r.post_i2f); if (mv && half_) signExtendA(); break;
     default: FX_CHECK(false, FX_E_INVALID, "emitSimple on an operator");
   }
 }
@@ -1106,7 +1157,8 @@ bool Lowerer::operandSimple(const Operand& o, uint32_t vt, Res* res) {
     if (v.prod == P_CONST) {
       r.kind = RK_IMM;
       double x = v.kind == VK_FLOAT ? v.fval : (double)v.ival;
-      r.imm = vt == FX_VT_F ? fbits((float)x) : (uint32_t)(int32_t)(int64_t)x;
+      r.imm = vt == FX_VT_F ? fbits((float)x) : imm32(v.kind == VK_FLOAT ? (int64_t)x : v.ival, "scalar operand");
+      r.imm64 = (int64_t)(int32_t)r.imm;
       r.vt = vt;
     } else if (v.prod == P_INPUT) {
       r.kind = RK_SCALAR;
@@ -1144,6 +1196,7 @@ void Lowerer::emitOperandA(const Operand& o, uint32_t vt) {
     Res r;
     if (operandSimple(o, vt, &r)) { emitSimple(r, false); return; }
     emitIdx(intOf(o.vid), false, vt == FX_VT_F);
+    if (moveCtx_ && half_ && vt == FX_VT_I) signExtendA();
     return;
   }
   emitAs(o.vid, o.f, vt);
@@ -1222,7 +1275,31 @@ void Lowerer::emitReduce(uint16_t op, uint32_t identity, int64_t extent, const s
   --loopDepth_;
 }
 
+static bool isMovementOp(int op) {
+  switch (op) {
+    case FX_OP_TRIU: case FX_OP_TRIL: case FX_OP_SELECT_REV: case FX_OP_SLICE_REV: case FX_OP_FORALL_SELECT_REV:
+    case FX_OP_CAT: case FX_OP_STACK: case FX_OP_VIEW: case FX_OP_REPEAT: case FX_OP_INDEX: case FX_OP_WHERE:
+    case FX_OP_FULL: case FX_OP_SCALAR_TENSOR:
+      return true;
+    default: return false;
+  }
+}
+
 void Lowerer::emitOp(const Res& r) {
+  if (!moveCtx_ || (isMovementOp(V(r.vid).op) && !is_float_dt(V(r.vid).dtype) && !r.post_i2f)) {
+    emitOpBody(r);
+    return;
+  }
+  // arithmetic on the way into an int64 output: a 32-bit value whose sign is the high word
+  const int half = half_;
+  {
+    ArithCtx a(*this);
+    emitOpBody(r);
+  }
+  if (half) signExtendA();
+}
+
+void Lowerer::emitOpBody(const Res& r) {
   const int vid = r.vid;
   const Value& v = V(vid);
   const Frame& f = r.f;
@@ -1333,7 +1410,7 @@ void Lowerer::emitOp(const Res& r) {
     case FX_OP_WHERE: {
       Operand c = operandOf(arg(0), f, outShape), a = operandOf(arg(1), f, outShape), b = operandOf(arg(2), f, outShape);
       uint32_t cv = vt_of(V(arg(0)).dtype);
-      emitOperandA(c, cv);
+      { ArithCtx ac(*this); emitOperandA(c, cv); }
       if (cv == FX_VT_F) emitI(FX_FNZ);
       int tc = allocTemp();
       emitI(FX_STT, tc);
@@ -1518,7 +1595,7 @@ void Lowerer::emitOp(const Res& r) {
                "index: only integer index tensors are fused (bool masks go through fx_region_compact_rows)");
       size_t ir = shapeOf(idx).size();
       Frame fidx(f.begin(), f.begin() + ir);
-      emitAs(idx, fidx, FX_VT_I);
+      { ArithCtx ac(*this); emitAs(idx, fidx, FX_VT_I); }
       emitI(FX_IPMOD, 0, 0, (uint32_t)(int32_t)std::max<int64_t>(in[0], 1), FX_F_IMM);
       int t = allocTemp();
       emitI(FX_STT, t);
@@ -1630,7 +1707,7 @@ bool Lowerer::rowWaveFrame(const Frame& f, int d, int64_t extent) const {
   return true;
 }
 
-Prog Lowerer::lower(int vid, const Shape& rootShape) {
+Prog Lowerer::lower(int vid, const Shape& rootShape, int half) {
   FX_CHECK(rootShape.size() <= FX_MAXR, FX_E_UNSUPPORTED, "region outputs above rank " << FX_MAXR << " are not supported");
   rootRank_ = (int)rootShape.size();
   for (int i = 0; i < FX_MAXR; ++i) rootDim_[i] = i < rootRank_ ? rootShape[i] : 1;
@@ -1638,6 +1715,9 @@ Prog Lowerer::lower(int vid, const Shape& rootShape) {
   maskDepth_ = 0;
   loopDepth_ = 0;
   usedRowWave_ = false;
+  moveCtx_ = V(vid).kind == VK_TENSOR && V(vid).dtype == FX_DT_I64;
+  half_ = moveCtx_ ? half : 0;
+  sawWide_ = false;
   Frame f(rootRank_);
   for (int i = 0; i < rootRank_; ++i) f[i] = IdxExpr::root(i);
   Prog p;
@@ -1646,6 +1726,9 @@ Prog Lowerer::lower(int vid, const Shape& rootShape) {
   p.end = (uint32_t)code.size();
   p.vt = vt_of(V(vid).dtype);
   p.rowwave = usedRowWave_;
+  p.wide = sawWide_;
+  moveCtx_ = false;
+  half_ = 0;
   return p;
 }
 
@@ -1810,6 +1893,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
 
   int max_temps = 0, max_rank = 1;
   int64_t total_rows = 0, max_rows = 0;
+  bool uses_guard = false;
   for (auto& cb : classes) {
     std::vector<const fx_arg*> in(R.inputs.size());
     for (size_t i = 0; i < R.inputs.size(); ++i)
@@ -1833,15 +1917,18 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
       FX_CHECK(numel_of(s) * dtype_size(P->out_dtype[o]) < ((int64_t)1 << 32), FX_E_LIMIT,
                "output " << o << " is 4 GiB or larger; split the region");
       for (int t : cb.tasks) P->out_shape[o][t] = s;
+      // an int64 output that moves int64 data is two records, one per 32-bit word
+      Prog p0 = L.lower(R.outputs[o], s);
+      for (int half = 0; half < (p0.wide ? 2 : 1); ++half) {
+      Prog p = half == 0 ? p0 : L.lower(R.outputs[o], s, 1);
       FxOut od;
       memset(&od, 0, sizeof(od));
-      Prog p = L.lower(R.outputs[o], s);
       od.prog_begin = p.begin;
       od.prog_end = p.end;
       od.vt = p.vt;
       fillDims(od, s);
       od.numel = (uint32_t)numel_of(s);
-      od.dtype = storage_dt(P->out_dtype[o]);
+      od.dtype = p0.wide ? (half ? FX_I64HI : FX_I64LO) : storage_dt(P->out_dtype[o]);
       od.ptr_slot = (uint32_t)out_slot[o];
       od.task_stride = 0;
       if (p.rowwave) {
@@ -1877,7 +1964,9 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
       }
       max_rank = std::max<int>(max_rank, (int)s.size());
       cb.outs.push_back(od);
+      }
     }
+    uses_guard = uses_guard || L.usesGuard;
     // The second compaction pass walks the outputs in table order (half of the waves
     // backwards).  Narrow outputs read a few bytes of every kept row, i.e. the same 128-byte
     // lines as each other: next to each other in the walk, the second one finds them in L2.
@@ -1953,6 +2042,11 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   P->max_rank = max_rank;
   P->n_temps = (uint32_t)max_temps;
 
+  // checked int64 loads report to an error word of the library
+  int slot_err = 0;
+  if (uses_guard) slot_err = slots.ptrSlotSpecial(PtrSrc::ERRWORD) + 1;
+  P->uses_guard = uses_guard;
+
   // slot budget
   P->sptr = slots.sptr;
   P->tptr = slots.tptr;
@@ -2013,6 +2107,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   h.slot_flags = (uint32_t)slot_flags;
   h.slot_counts = (uint32_t)slot_counts;
   h.slot_total = (uint32_t)slot_total;
+  h.slot_err = (uint32_t)slot_err;
   appendStruct(blob, h);
   for (auto& cb : classes) {
     while (blob.size() % 4) blob.push_back(0);

@@ -67,7 +67,7 @@ struct Region {
 
 // where a dynamic pointer / scalar slot is filled from at run time
 struct PtrSrc {
-  enum Kind { INPUT, OUTPUT, FLAGS, COUNTS, TOTALS } kind;
+  enum Kind { INPUT, OUTPUT, FLAGS, COUNTS, TOTALS, ERRWORD } kind;
   int index;  // region input index / output index
 };
 struct ScalSrc {
@@ -83,6 +83,7 @@ struct Plan {
   uint32_t grid_count = 0;     // compaction pass 1
   uint32_t lds_bytes = 0;
   bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
+  bool uses_guard = false;       // some load checks int64 data against 32 bits and reports to the error word
   uint32_t n_temps = 0;
   int max_rank = 1;
   std::vector<PtrSrc> sptr, tptr;

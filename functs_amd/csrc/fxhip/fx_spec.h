@@ -177,7 +177,7 @@ __device__ __forceinline__ void fx_spec_prefetch(const FxCtx& cx, const FxCoord<
       constexpr FxInsn J = P::code[K];
       int32_t off[FX_V];
       const bool consecutive = fx_affine<R>(cx, q, J.b, rg.lc0, rg.lc1, off);
-      fx_load_vec(fx_ptr(cx, J.a), off, M, J.dt, (J.flags & FX_F_I2F) != 0, consecutive, ts.ld[K]);
+      fx_load_vec(fx_ptr(cx, J.a), off, M, J.dt, (J.flags & FX_F_I2F) != 0, consecutive, ts.ld[K], cx.err);
     }
     fx_spec_prefetch<P, R, K + 1, END, TS>(cx, q, ts, M, rg);
   }

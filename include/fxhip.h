@@ -241,6 +241,18 @@ int fx_region_marshal(fx_region*, const fx_plan*, const fx_arg* args, int n_args
                       void* scratch, uint32_t* totals_host, void* dyn_out, size_t dyn_cap);
 size_t fx_dyn_bytes(void);
 
+/* int64 in regions.  Programs that only MOVE int64 data (select / slice / index / where / cat /
+ * *_rev / row compaction ...) are exact for every value: they travel as two 32-bit words.
+ * Integer ARITHMETIC is 32-bit: an int64 tensor element that enters it (a + 3, a == b, a as an
+ * index) must fit 32 bits (a conversion to float uses the whole element and is exact).  The
+ * loads check that; an element that does not fit sets a sticky process-wide error word, and
+ * the outputs of that launch are not to be used.  fx_async_error returns 1 if it is set (after
+ * the stream has been synchronised it covers every launch before that) and clears it when
+ * `clear` is non-zero.  Integer constants and scalar arguments outside 32 bits are refused when
+ * the region is planned / run (FX_E_UNSUPPORTED / FX_E_LIMIT).  The reference computes in int64
+ * throughout (NNC kLong, functs/csrc/jit/ir/symbol_ext.cpp:17-117 for the eager bodies). */
+int fx_async_error(int clear);
+
 /* ---- stand-alone order-preserving row compaction (x[mask] for several x) ----
  * mask: n bytes (0/1); cols[i]: [n, rowlen[i]] fp32/int32 (4-byte) or int64 (8-byte) rows.
  * outs[i] must hold n * rowlen[i] elements.  Same contract as ATen

@@ -29,10 +29,19 @@ uint32_t half_to_f32(uint16_t h) {
   return (s << 31) | ((e + 112) << 23) | (m << 13);
 }
 
-uint32_t load_elem(const void* base, int64_t off, uint32_t dt) {
+// int64 data in 32-bit arithmetic: converted to float the whole value counts; as an integer
+// the low word is the value and an element that does not fit is reported through *err
+uint32_t load_elem(const void* base, int64_t off, uint32_t dt, bool cvt = false, uint32_t* err = nullptr) {
   switch (dt) {
     case FX_F32: case FX_I32: return ((const uint32_t*)base)[off];
-    case FX_I64: return (uint32_t)((const int64_t*)base)[off];
+    case FX_I64: {
+      const int64_t v = ((const int64_t*)base)[off];
+      if (cvt) return f2u((float)v);
+      if (v != (int64_t)(int32_t)v && err) *err = 1u;
+      return (uint32_t)v;
+    }
+    case FX_I64LO: return ((const uint32_t*)base)[2 * off];
+    case FX_I64HI: return ((const uint32_t*)base)[2 * off + 1];
     case FX_U8: return ((const uint8_t*)base)[off];
     case FX_F16: return half_to_f32(((const uint16_t*)base)[off]);
     case FX_BF16: return ((uint32_t)((const uint16_t*)base)[off]) << 16;
@@ -45,6 +54,8 @@ void store_elem(void* base, int64_t off, uint32_t dt, uint32_t vt, uint32_t v) {
     case FX_F32: ((uint32_t*)base)[off] = vt == FX_VT_F ? v : f2u((float)(int32_t)v); break;
     case FX_I32: ((int32_t*)base)[off] = vt == FX_VT_I ? (int32_t)v : (int32_t)u2f(v); break;
     case FX_I64: ((int64_t*)base)[off] = vt == FX_VT_I ? (int64_t)(int32_t)v : (int64_t)u2f(v); break;
+    case FX_I64LO: ((uint32_t*)base)[2 * off] = v; break;
+    case FX_I64HI: ((uint32_t*)base)[2 * off + 1] = v; break;
     case FX_U8: ((uint8_t*)base)[off] = vt == FX_VT_I ? (uint8_t)v : (uint8_t)(u2f(v) != 0.0f); break;
     case FX_BF16: {
       float f = vt == FX_VT_F ? u2f(v) : (float)(int32_t)v;
@@ -80,6 +91,7 @@ struct Ctx {
   const uint32_t* sscal;
   const uint32_t* tscal;
   int task;
+  uint32_t* err;
 };
 
 const void* ptr_of(const Ctx& cx, int32_t slot) {
@@ -156,8 +168,9 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
       const int32_t* c = l.c;
       if (ins.flags & FX_F_TMPB) B = temps[ins.a];
       else if ((ins.flags & FX_F_MEMB) && M) {
-        B = load_elem(ptr_of(cx, ins.a), affine_at(l, ins.b), ins.dt);
-        if (ins.flags & FX_F_I2F) B = f2u((float)(int32_t)B);
+        const bool wide = ins.dt == FX_I64 && (ins.flags & FX_F_I2F);
+        B = load_elem(ptr_of(cx, ins.a), affine_at(l, ins.b), ins.dt, wide, l.M ? cx.err : nullptr);
+        if ((ins.flags & FX_F_I2F) && !wide) B = f2u((float)(int32_t)B);
       }
       const float fa = u2f(A), fb = u2f(useimm ? ins.imm : B);
       const int32_t ia = (int32_t)A, ib = (int32_t)(useimm ? ins.imm : B);
@@ -168,11 +181,12 @@ void run(const Ctx& cx, int pc, int pc_end, std::vector<Lane>& L) {
           if (!M) break;
           const int32_t off = affine_at(l, ins.b);
           const bool is_load = ins.op == FX_LDA;
-          uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt) : (uint32_t)off;
-          if (ins.flags & FX_F_I2F) v = f2u((float)(int32_t)v);
+          const bool wide = is_load && ins.dt == FX_I64 && (ins.flags & FX_F_I2F);
+          uint32_t v = is_load ? load_elem(ptr_of(cx, ins.a), off, ins.dt, wide, l.M ? cx.err : nullptr) : (uint32_t)off;
+          if ((ins.flags & FX_F_I2F) && !wide) v = f2u((float)(int32_t)v);
           if (ins.op == FX_LDA || ins.op == FX_AFFA) A = v; else B = v;
         } break;
-        case FX_LDXA: if (M) A = load_elem(ptr_of(cx, ins.a), (int64_t)((int32_t)A + (int32_t)ins.imm), ins.dt); break;
+        case FX_LDXA: if (M) A = load_elem(ptr_of(cx, ins.a), (int64_t)((int32_t)A + (int32_t)ins.imm), ins.dt, false, cx.err); break;
         case FX_IMMA: if (M) A = ins.imm; break;
         case FX_IMMB: B = ins.imm; break;
         case FX_SCLA: if (M) { A = scalar_of(cx, ins.a); if (ins.flags & FX_F_I2F) A = f2u((float)(int32_t)A); } break;
@@ -295,6 +309,7 @@ extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_,
       cx.sscal = dyn->s;
       cx.tscal = dyn->s + h->n_sscal + (size_t)task * h->n_tscal;
       cx.task = task;
+      cx.err = h->slot_err ? (uint32_t*)(uintptr_t)dyn->p[h->slot_err - 1] : nullptr;
       if (h->mode == FX_MODE_DENSE) {
         for (uint32_t oi = 0; oi < cl.n_outs; ++oi) {
           const FxOut& od = outs[oi];

@@ -1,5 +1,8 @@
 // Python module functs_amd._C: same entry-point names as the reference's
 // functs._C (functs/csrc/jit/python/init.cpp:31-76, script_init.cpp:83-95).
+#include <torch/csrc/jit/passes/constant_propagation.h>
+#include <torch/csrc/jit/passes/freeze_module.h>
+#include <torch/csrc/jit/passes/shape_analysis.h>
 #include <torch/csrc/jit/python/pybind_utils.h>
 #include <torch/extension.h>
 
@@ -32,6 +35,35 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_fuse_masked_select", FuseMaskedSelect);
   m.def("_jit_pass_to_parallel_functor", ToParallelFunctor);
   m.def("_jit_pass_fait_pipeline", FaitPipeline);
+  // functs/csrc/jit/python/init.cpp:45: FaitGetRefineType (fait_pipeline.cpp:19-29) gives the graph
+  // inputs the types of the examples and propagates dtype / device / shape.  The propagation is
+  // libtorch's own; regions specialise on the shapes they are called with, so nothing downstream
+  // depends on it.  `refined_types` (per-value types of list elements in the reference) is accepted
+  // and left alone: a Python dict crosses this boundary by value in the reference as well.
+  m.def("_jit_pass_fait_shape_infer",
+        [](std::shared_ptr<Graph> g, std::vector<c10::TypePtr> type_hint, py::object /*refined_types*/) {
+          auto inputs = g->inputs();
+          TORCH_CHECK(type_hint.size() <= inputs.size(), "_jit_pass_fait_shape_infer: ", type_hint.size(),
+                      " type hints for ", inputs.size(), " graph inputs");
+          const size_t off = inputs.size() - type_hint.size();   // a leading `self` of a module graph
+          for (size_t i = 0; i < type_hint.size(); ++i) {
+            auto tt = type_hint[i]->cast<c10::TensorType>();
+            if (!tt) continue;
+            // the propagation wants complete types: contiguous strides for a hint that carries sizes only
+            auto sizes = tt->sizes().concrete_sizes();
+            if (sizes && tt->scalarType() && tt->device() && !tt->strides().concrete_sizes())
+              inputs[off + i]->setType(c10::TensorType::createContiguous(*tt->scalarType(), *tt->device(), *sizes));
+            else
+              inputs[off + i]->setType(tt);
+          }
+          torch::jit::ConstantPropagation(g);   // int[] arguments become constants the shape rules can read
+          torch::jit::PropagateInputShapes(g);
+        },
+        py::arg("graph"), py::arg("type_hint"), py::arg("refined_types") = py::dict());
+  // init.cpp:47-48: Freeze(Module*) folds attributes into the graph in place, Clone(Module*) copies
+  // (fait/passes/freeze_module.cpp:954-960).  Stock libtorch does both.
+  m.def("_jit_pass_freeze", [](torch::jit::Module& module) { module = torch::jit::freeze_module(module); });
+  m.def("_jit_pass_clone", [](torch::jit::Module& module) { return module.clone(); });
   m.def("_jit_pass_validate", Validate);
   m.def("_jit_pass_convert_profiling_instrumentation", ConvertProfilingInstrumentation);
   m.def("_prof_begin", profBegin);

@@ -127,7 +127,9 @@ std::string profilingResults(size_t count) {
   if (count == 0) count = 1;
   std::ostringstream out;
   const uint64_t launches = s.launches + (s.enabled ? regionLaunches() - s.launches_at_enable : 0);
-  if (launches > 0) out << "Kernel launch: " << launches / count << '\n';
+  // the reference counts every kernel of the process through CUPTI (fait/util/profile.cpp:29-46);
+  // this count covers the kernels the fused regions launch, not those of ATen or rocBLAS calls
+  if (launches > 0) out << "Kernel launch: " << launches / count << " (fused-region kernels only)\n";
   if (s.records.empty()) return out.str();
   auto cell = [&](const std::string& v) { out << std::setw(10) << v; };
   out << "\nRanges:\n" << std::left << std::setw(16) << "Label" << std::right;
@@ -200,6 +202,18 @@ extern "C" __attribute__((visibility("default"))) void disableProfiling() {
   if (s.enabled) s.launches += functs::regionLaunches() - s.launches_at_enable;
   s.enabled = false;
 }
+// The metric passes of the reference (fait/util/metrics.h:6-13) replay a range under CUPTI /
+// NVPerf to read occupancy counters inside the process.  On this platform counters are collected
+// from outside the process (rocprofv3 --pmc), so there is nothing to replay: metrics are reported
+// as not enabled, a profiler pass is empty, and one pass is all there is.  The symbols exist so
+// that a harness which resolves them from the library (functs/utils/prof.py:19-36) loads.
+extern "C" __attribute__((visibility("default"))) bool metricsEnabled() { return false; }
+extern "C" __attribute__((visibility("default"))) void initializeMetrics() {}
+extern "C" __attribute__((visibility("default"))) void finalizeMetrics() {}
+extern "C" __attribute__((visibility("default"))) void beginProfilerPass() {}
+extern "C" __attribute__((visibility("default"))) void endProfilerPass() {}
+extern "C" __attribute__((visibility("default"))) bool allPassesSubmitted() { return true; }
+
 extern "C" __attribute__((visibility("default"))) void printProfilingResults(size_t count) {
   std::cout << functs::profilingResults(count) << std::flush;
 }

@@ -20,6 +20,34 @@ from . import _C
 
 _lib = ctypes.CDLL(_C.__file__)
 _lib.printProfilingResults.argtypes = [ctypes.c_size_t]
+_lib.metricsEnabled.restype = ctypes.c_bool
+_lib.allPassesSubmitted.restype = ctypes.c_bool
+
+
+def metrics_enabled() -> bool:
+    """Counter passes inside the process (functs/utils/prof.py:16-36) have no counterpart here:
+    hardware counters are read with rocprofv3 from outside.  Always False."""
+    return bool(_lib.metricsEnabled())
+
+
+def initialize_metrics():
+    _lib.initializeMetrics()
+
+
+def finalize_metrics():
+    _lib.finalizeMetrics()
+
+
+def begin_profiler_pass():
+    _lib.beginProfilerPass()
+
+
+def end_profiler_pass():
+    _lib.endProfilerPass()
+
+
+def all_passes_submitted() -> bool:
+    return bool(_lib.allPassesSubmitted())
 
 
 def enable_profiling():

@@ -61,7 +61,28 @@ def test_generated_anchors_without_compiled_kernels_are_refused():
     preds, bases = _inputs(2, 3)
     r = configs.build_c5_generated_anchors(2, LEVELS)
     args = [preds.to(dev)] + [b.to(dev) for b in bases]
-    if r.specialized(*args):
-        pytest.skip("compiled kernels for this region are linked in")
-    with pytest.raises(FxError, match="compiled kernels"):
-        r(*args)
+    import functs_amd.aot as aot
+    aot.enable(False)   # as if the compiled kernels of this region were not linked in
+    try:
+        assert not r.specialized(*args)
+        with pytest.raises(FxError, match="compiled kernels"):
+            r(*args)
+    finally:
+        aot.enable(True)
+
+
+@pytest.mark.gpu
+def test_generated_anchors_equal_torch_on_the_gpu():
+    """Parity of the region with generated anchors on the GPU (its compiled kernels are linked
+    into the library: the interpreter's temporaries do not fit LDS for this region)."""
+    dev = torch.device("cuda:0")
+    preds, bases = _inputs(2, 3)
+    r = configs.build_c5_generated_anchors(2, LEVELS)
+    args = [preds.to(dev)] + [b.to(dev) for b in bases]
+    assert r.specialized(*args), "the compiled kernels of this region are not linked in"
+    out = run_region("hip", r, preds, *bases)
+    ref = _torch_reference(preds, bases)
+    for i in range(2):
+        assert_boxes_close(out[0][i], ref[i][0], "boxes[%d]" % i)
+        assert_close(out[1][i], ref[i][1], "cls[%d]" % i)
+        assert_close(out[2][i], ref[i][2], "obj[%d]" % i)

@@ -175,6 +175,31 @@ def test_c3_closed_forms():
         assert torch.equal(ss[c - 1], scores[m, c])
 
 
+def test_c3_decode_of_one_row_with_its_variances():
+    """Independent decode of single rows with loc != 0, written from the textbook SSD formulas
+    (centre variance 0.1, size variance 0.2): a swapped pair of variances, a dropped prior size or a
+    wrong sign fails here (with loc == 0 all of these vanish)."""
+    import math
+    loc, conf, priors = oc.c3_inputs(1, 40, 6)
+    bs, ss = oc.run("c3", loc, conf, priors)
+    scores = conf[0].softmax(-1)
+    checked = 0
+    for c in range(1, 6):
+        rows = torch.nonzero(scores[:, c] > 0.05).flatten().tolist()
+        for k, i in enumerate(rows[:3]):
+            pcx, pcy, pw, ph = [float(v) for v in priors[i]]
+            lx, ly, lw, lh = [float(v) for v in loc[0, i]]
+            cx, cy = pcx + lx * 0.1 * pw, pcy + ly * 0.1 * ph
+            w, h = pw * math.exp(lw * 0.2), ph * math.exp(lh * 0.2)
+            want = torch.tensor([cx - w / 2, cy - h / 2, cx + w / 2, cy + h / 2])
+            assert torch.allclose(bs[c - 1][k], want, rtol=1e-5, atol=1e-6), (c, i)
+            # the same row with the variances swapped is far outside that tolerance
+            cx2, w2 = pcx + lx * 0.2 * pw, pw * math.exp(lw * 0.1)
+            assert abs((cx2 - w2 / 2) - float(want[0])) > 1e-4 or abs(lx) + abs(lw) < 1e-2
+            checked += 1
+    assert checked >= 5
+
+
 def test_c4_matches_nn_lstm():
     """Cross-check of the cell formulas against torch.nn.LSTM with re-packed
     weights (the packing functs/benchmark/ai_model/lstm/lstm.py:168-175 uses)."""

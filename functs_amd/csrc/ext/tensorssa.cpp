@@ -54,6 +54,33 @@ bool isViewKind(Symbol k) {
   return kinds.count(k) != 0;
 }
 
+// View operators that have no immut:: twin but whose result is certainly a view of their first
+// argument: a later write to the buffer is seen through them, so the rewrite re-derives them from
+// the new version of their parent (by cloning the node), as the reference re-derives every value
+// AliasDb says aliases the buffer (convert_to_tensorssa.cpp:186-266).  There is no write-back
+// operator for them: a write THROUGH such a view leaves its whole tree untouched.
+bool isPlainViewKind(Symbol k) {
+  static const std::unordered_set<Symbol> kinds{
+      c10::aten::t,         c10::aten::transpose, c10::aten::expand,   c10::aten::expand_as, c10::aten::narrow,
+      c10::aten::view_as,   c10::aten::movedim,   c10::aten::swapaxes, c10::aten::swapdims,  c10::aten::diagonal,
+      c10::aten::numpy_T,   c10::aten::mT,        c10::aten::alias,    c10::aten::detach,    c10::aten::unfold,
+      c10::aten::as_strided, c10::aten::unflatten};
+  return kinds.count(k) != 0;
+}
+
+// does the result of `node` possibly share storage with its input `i` (a `Tensor(a)` argument
+// that some return repeats)?  True for the operators above and for those that view or copy
+// depending on their arguments (to, contiguous, flatten, reshape_as, chunk, split ...).
+bool mayReturnAliasOf(Node* node, size_t i) {
+  auto schema = node->maybeSchema();
+  if (!schema || i >= schema->arguments().size()) return false;
+  const auto* ai = schema->arguments()[i].alias_info();
+  if (!ai || ai->isWrite()) return false;
+  for (const auto& r : schema->returns())
+    if (r.alias_info()) return true;
+  return false;
+}
+
 // The view forest: every tracked tensor is either a root (owns fresh storage)
 // or a view of another tracked tensor (buffer_forest.h:50-65).
 class ViewForest {
@@ -61,6 +88,7 @@ class ViewForest {
   std::unordered_map<Value*, Value*> parent;
   std::unordered_map<Value*, std::vector<Value*>> children;
   std::unordered_set<Node*> mutations;
+  std::unordered_set<Value*> plain;   // views made by an operator of isPlainViewKind
 
   bool has(Value* v) const { return parent.count(v) != 0; }
   Value* parentOf(Value* v) const {
@@ -82,6 +110,7 @@ class ViewForest {
     Value* p = it->second;
     parent.erase(it);
     parent[to] = p;
+    if (plain.erase(from)) plain.insert(to);
     if (p)
       for (auto& c : children[p])
         if (c == from) c = to;
@@ -128,6 +157,9 @@ void buildForest(Block* b, ViewForest& f) {
     if (!isTensor(out)) continue;
     if (isViewKind(n->kind()) && f.has(n->input(0))) {
       f.addView(out, n->input(0));
+    } else if (isPlainViewKind(n->kind()) && n->outputs().size() == 1 && !n->inputs().empty() && f.has(n->input(0))) {
+      f.addView(out, n->input(0));
+      f.plain.insert(out);
     } else if ((n->kind() == c10::aten::copy_ || n->kind() == sym::Assign()) && f.has(n->input(0))) {
       f.addView(out, n->input(0));
       f.mutations.insert(n);
@@ -168,9 +200,22 @@ void pruneForest(std::shared_ptr<Graph> g, ViewForest& f) {
           // a write this pass does not understand
           if (user->kind() != c10::aten::copy_ && user->kind() != sym::Assign() && writesInput(user, u.offset))
             bad.insert(root);
+          // An operator that may hand back a view of the buffer which the forest does not track
+          // (to, contiguous, flatten, chunk ...): a write to the buffer that follows it would have
+          // to show through that view or not, depending on run-time facts.  With no such write the
+          // operator simply reads the latest version.
+          else if (!isViewKind(user->kind()) && !(isPlainViewKind(user->kind()) && u.offset == 0) &&
+                   mayReturnAliasOf(user, u.offset)) {
+            for (Node* m : f.mutations)
+              if (f.has(m->output(0)) && f.rootOf(m->output(0)) == root && !m->isBefore(user)) bad.insert(root);
+          }
       }
     }
   }
+  // a write through a plain view has no write-back operator
+  for (Node* m : f.mutations)
+    for (Value* v = m->output(0); v && f.has(v); v = f.parentOf(v))
+      if (f.plain.count(v)) bad.insert(f.rootOf(v));
   for (Value* r : bad) {
     std::vector<Node*> drop;
     for (Node* m : f.mutations)

@@ -1499,7 +1499,9 @@ void Lowerer::emitOpBody(const Res& r) {
       Shape s = shapeOf(arg(0));
       int d = normDim(constIntOf(arg(2), "forall_select_rev"), (int64_t)s.size(), "forall_select_rev");
       int64_t lo_b = constIntOf(arg(3), "loop lower bound"), hi_b = constIntOf(arg(4), "loop upper bound");
-      hi_b = std::min<int64_t>(hi_b, s[d]);
+      // eager mode raises IndexError when the loop indexes past the dimension
+      FX_CHECK(lo_b >= hi_b || (lo_b >= 0 && hi_b <= s[d]), FX_E_INVALID,
+               "collapsed loop over [" << lo_b << ", " << hi_b << ") indexes outside a dimension of size " << s[d]);
       Frame fs = f;
       fs.erase(fs.begin() + d);
       Shape slab = s; slab.erase(slab.begin() + d);

@@ -39,6 +39,19 @@ def test_c1_trip_counts(backend, n):
     assert_exact(got, oc.run("c1", a, b, n), "c1 n=%d" % n)
 
 
+def test_c1_trip_count_past_the_dimension_is_an_error():
+    """The oracle raises an index error for b[48] on 48 rows; the collapsed loop says so too instead
+    of stopping at the last row."""
+    from functs_amd._lib import C, FxError
+    from tests.support import emul
+    a, b, _ = oc.c1_inputs(1, 48, 0)
+    with pytest.raises((IndexError, RuntimeError)):   # TorchScript reports the IndexError as a RuntimeError
+        oc.run("c1", a, b, 49)
+    with pytest.raises(FxError) as e:
+        emul.run(configs.build_c1(), b, 49)
+    assert e.value.code == C["FX_E_INVALID"] and "outside a dimension" in str(e.value)
+
+
 def _check_yolo(got, ref, pred, what):
     boxes, cls, obj = got
     rboxes, rcls, robj = ref

@@ -111,6 +111,10 @@ _sig("fx_plan_output", _i, _vp, _i, _i, ctypes.POINTER(ctypes.c_int32), ctypes.P
      ctypes.POINTER(ctypes.c_int64))
 _sig("fx_plan_scratch_bytes", ctypes.c_size_t, _vp)
 _sig("fx_plan_launches", _i, _vp)
+_sig("fx_plan_streaming", _i, _vp)
+_sig("fx_plan_stream_info", _i, _vp, ctypes.POINTER(ctypes.c_int64), _i)
+_sig("fx_set_streaming", None, _i)
+_sig("fx_set_stream_spin_limit", None, ctypes.c_uint32)
 _sig("fx_plan_algorithmic_bytes", ctypes.c_int64, _vp)
 _sig("fx_plan_blob", _i, _vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)), ctypes.POINTER(ctypes.c_size_t))
 _sig("fx_plan_disasm", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)

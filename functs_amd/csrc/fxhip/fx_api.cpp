@@ -31,6 +31,10 @@ hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, c
 hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
                                      uint32_t grid, hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_copy(const void* src, void* dst, size_t bytes, uint32_t grid, hipStream_t stream);
+hipError_t fx_launch_compact_stream(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
+                                    hipStream_t stream, const FxSpecKernels* spec);
+uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled);
+bool fx_spec_has_stream(const FxSpecKernels* spec);
 hipError_t fx_launch_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                          const int32_t* rowlen, const int32_t* elsize, int n_cols,
                                          uint32_t* total_host, hipStream_t stream);
@@ -94,8 +98,11 @@ int fx_region_create(int parallel_degree, int is_parallel_map, fx_region** out) 
 
 void fx_region_destroy(fx_region* r) {
   if (!r) return;
-  for (auto& kv : r->r.plans)
+  for (auto& kv : r->r.plans) {
     if (kv.second->dev_blob) (void)hipFree(kv.second->dev_blob);
+    for (auto& st : kv.second->status)
+      if (st.ptr) (void)hipFree(st.ptr);
+  }
   delete r;
 }
 
@@ -227,6 +234,15 @@ static std::atomic<int> g_specialize{[] {
   const char* e = getenv("FXHIP_SPECIALIZE");
   return (e && e[0] == '0') ? 0 : 1;
 }()};
+// ---- streaming compaction: process-wide switches ----
+static std::atomic<int> g_stream_mode{[] {
+  const char* e = getenv("FXHIP_STREAM");
+  return (e && e[0] == '1') ? 1 : 0;
+}()};
+static std::atomic<uint32_t> g_stream_spin{[] {
+  const char* e = getenv("FXHIP_STREAM_SPIN");
+  return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
+}()};
 static std::mutex g_dump_mu;
 static std::string g_dump_dir;
 
@@ -322,7 +338,29 @@ int fx_plan_output(const fx_plan* p, int out_idx, int task, int32_t* dtype, int3
 }
 
 size_t fx_plan_scratch_bytes(const fx_plan* p) { return p ? P(p)->scratch_bytes : 0; }
-int fx_plan_launches(const fx_plan* p) { return p ? P(p)->launches : 0; }
+static bool stream_active(const fx::Plan* pl, const FxSpecKernels* spec);
+static const FxSpecKernels* spec_of(const fx::Plan* p);
+int fx_plan_launches(const fx_plan* p) {
+  if (!p) return 0;
+  if (P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) return P(p)->stream.grid > 0 ? 1 : 0;
+  return P(p)->launches;
+}
+int fx_plan_streaming(const fx_plan* p) { return (p && P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) ? 1 : 0; }
+int fx_plan_stream_info(const fx_plan* p, int64_t* out, int cap) {
+  if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_stream_info: out[>=8] required");
+  const fx::StreamInfo& si = P(p)->stream;
+  out[0] = si.ok ? 1 : 0;
+  out[1] = si.tile_rows;
+  out[2] = si.tiles_per_task;
+  out[3] = si.grid;
+  out[4] = si.win_stride;
+  out[5] = si.win_tcoef;
+  out[6] = si.win_lo;
+  out[7] = si.win_span;
+  return FX_OK;
+}
+void fx_set_streaming(int on) { g_stream_mode.store(on ? 1 : 0, std::memory_order_relaxed); }
+void fx_set_stream_spin_limit(uint32_t polls) { g_stream_spin.store(polls, std::memory_order_relaxed); }
 int64_t fx_plan_algorithmic_bytes(const fx_plan* p) { return p ? P(p)->alg_bytes : 0; }
 
 int fx_plan_blob(const fx_plan* p, const uint32_t** words, size_t* n_words) {
@@ -381,7 +419,7 @@ int fx_async_error(int clear) {
 // an element that is not live to element 0 of its buffer, so a tensor without
 // elements (whose pointer may be null) is given this address instead.
 static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
-                    uint32_t* totals_host, const void* safe, FxDyn* dyn) {
+                    uint32_t* totals_host, const void* safe, FxDyn* dyn, const void* status = nullptr) {
   const fx::Region& R = *pl->region;
   const int T = R.degree;
   auto ptr_of = [&](const fx::PtrSrc& s, int task) -> uint64_t {
@@ -398,6 +436,7 @@ static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptr
       case fx::PtrSrc::COUNTS: return (uint64_t)(uintptr_t)((char*)scratch + pl->counts_off);
       case fx::PtrSrc::TOTALS: return (uint64_t)(uintptr_t)totals_host;
       case fx::PtrSrc::ERRWORD: return (uint64_t)(uintptr_t)err_word(safe != nullptr);
+      case fx::PtrSrc::STATUS: return (uint64_t)(uintptr_t)status;
     }
     return 0;
   };
@@ -442,6 +481,98 @@ int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, i
 
 size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
 
+// ---- streaming compaction: per-stream status words ----
+#define FX_STREAM_LDS_LIMIT 64000u   // 64 KiB less the kernel's static tables
+#define FX_EPOCH_MAX ((1u << 23) - 1u)
+
+static FxLaunchInfo launch_info(const fx::Plan* pl) {
+  const fx::Region& R = *pl->region;
+  FxLaunchInfo li;
+  memset(&li, 0, sizeof(li));
+  li.blob_words = (uint32_t)pl->blob.size();
+  li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)R.degree);
+  li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)R.degree);
+  li.n_temps = pl->n_temps;
+  li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
+  if (pl->stream.ok) {
+    const fx::StreamInfo& si = pl->stream;
+    li.win_words = si.win_words;
+    li.s_tiles = si.tiles_per_task;
+    li.s_rows = si.rows;
+    li.s_tile_rows = si.tile_rows;
+    li.s_win_slot = si.win_slot;
+    li.s_win_stride = si.win_stride;
+    li.s_win_tcoef = si.win_tcoef;
+    li.s_win_lo = si.win_lo;
+    li.s_win_span = si.win_span;
+    li.n_sptr = (uint32_t)pl->sptr.size();
+    li.n_tptr = (uint32_t)pl->tptr.size();
+    li.spin_limit = g_stream_spin.load(std::memory_order_relaxed);
+    li.n_side = si.n_side;
+    for (int i = 0; i < 2; ++i) {
+      li.side_slot[i] = si.side_slot[i];
+      li.side_stride[i] = si.side_stride[i];
+      li.side_tcoef[i] = si.side_tcoef[i];
+      li.side_lo[i] = si.side_lo[i];
+      li.side_span[i] = si.side_span[i];
+      li.side_words[i] = si.side_words[i];
+    }
+  }
+  return li;
+}
+
+// does a call of this plan run as one streaming kernel (with the kernels it would use now)?
+static bool stream_active(const fx::Plan* pl, const FxSpecKernels* spec) {
+  if (!pl->stream.ok || !g_stream_mode.load(std::memory_order_relaxed)) return false;
+  const bool compiled = spec && fx_spec_has_stream(spec);
+  return fx_stream_lds_bytes(launch_info(pl), compiled) <= FX_STREAM_LDS_LIMIT;
+}
+
+// persistent workgroups: as many as stay resident together (two per CU: the kernel keeps the
+// next tile's rows in registers), striding over the tiles
+#define FX_STREAM_WG_PER_CU 2u
+static uint32_t stream_grid(const fx::Plan* pl) { return std::min<uint32_t>(pl->stream.grid, 256u * FX_STREAM_WG_PER_CU); }
+
+// Status words of `pl` for launches on `stream` (created on first use, at most four streams per
+// plan: calls on further streams take the two-pass form) and the epoch of the next call.
+static int stream_status(fx_region* reg, fx::Plan* pl, hipStream_t stream, int dev, void** ptr, uint32_t* epoch,
+                         int n_epochs) {
+  std::lock_guard<std::mutex> g(reg->mu);
+  fx::Plan::Status* st = nullptr;
+  for (auto& s : pl->status)
+    if (s.stream == (void*)stream && s.dev == dev) st = &s;
+  if (!st) {
+    if (pl->status.size() >= 4) { *ptr = nullptr; return FX_OK; }
+    void* d = nullptr;
+    const size_t bytes = (size_t)std::max<uint32_t>(pl->stream.grid, 1) * 4;
+    HIP_OK(hipMalloc(&d, bytes));
+    HIP_OK(hipMemset(d, 0, bytes));
+    pl->status.push_back({(void*)stream, d, 0u, dev});
+    st = &pl->status.back();
+  }
+  if (st->epoch + (uint32_t)n_epochs >= FX_EPOCH_MAX) {
+    // the tags wrap: clear the words behind everything already queued on the stream
+    HIP_OK(hipMemsetAsync(st->ptr, 0, (size_t)std::max<uint32_t>(pl->stream.grid, 1) * 4, stream));
+    st->epoch = 0;
+  }
+  *ptr = st->ptr;
+  *epoch = st->epoch + 1;
+  st->epoch += (uint32_t)n_epochs;
+  return FX_OK;
+}
+
+static int upload_blob(fx_region* reg, fx::Plan* pl, int dev) {
+  std::lock_guard<std::mutex> g(reg->mu);
+  if (!pl->dev_blob || pl->dev_id != dev) {
+    void* d = nullptr;
+    HIP_OK(hipMalloc(&d, pl->blob.size() * 4));
+    HIP_OK(hipMemcpy(d, pl->blob.data(), pl->blob.size() * 4, hipMemcpyHostToDevice));
+    pl->dev_blob = d;
+    pl->dev_id = dev;
+  }
+  return FX_OK;
+}
+
 static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
                     void* scratch, uint32_t* totals_host, void* stream_, float* kernel_ms, int cap, int* n_kernels,
                     int repeat = 1) {
@@ -455,26 +586,29 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
 
   int dev = 0;
   HIP_OK(hipGetDevice(&dev));
-  {
-    std::lock_guard<std::mutex> g(reg->mu);
-    if (!pl->dev_blob || pl->dev_id != dev) {
-      void* d = nullptr;
-      HIP_OK(hipMalloc(&d, pl->blob.size() * 4));
-      HIP_OK(hipMemcpy(d, pl->blob.data(), pl->blob.size() * 4, hipMemcpyHostToDevice));
-      pl->dev_blob = d;
-      pl->dev_id = dev;
-    }
+  int rc = upload_blob(reg, pl, dev);
+  if (rc != FX_OK) return rc;
+  const FxSpecKernels* spec = spec_of(pl);
+  if (!spec && pl->needs_compiled) {
+    char key[17];
+    snprintf(key, sizeof key, "%016llx", (unsigned long long)pl->spec_key);
+    return fail(FX_E_LIMIT, std::string("the interpreter's temporaries of this region need ") + std::to_string(pl->lds_bytes) +
+                                " bytes of LDS (limit 65536) and no compiled kernels for its programs (key " + key +
+                                ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
+  }
+  FxLaunchInfo li = launch_info(pl);
+  bool streaming = pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
+  void* status = nullptr;
+  uint32_t epoch = 0;
+  if (streaming) {
+    rc = stream_status(reg, pl, stream, dev, &status, &epoch, repeat);
+    if (rc != FX_OK) return rc;
+    if (!status) streaming = false;
   }
   FxDyn dyn;
-  int rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn);
+  rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn, status);
   if (rc != FX_OK) return rc;
   const uint32_t* sb = (const uint32_t*)pl->dev_blob;
-  FxLaunchInfo li;
-  li.blob_words = (uint32_t)pl->blob.size();
-  li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
-  li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
-  li.n_temps = pl->n_temps;
-  li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
   if (pl->mode == FX_MODE_COMPACT) {
     // Tasks without rows launch no tile: their total is published here.  The others hold a
     // mark until the last tile of the task stores the count (fx_region_wait_totals looks for
@@ -484,16 +618,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                            ? FX_TOTAL_PENDING
                            : 0u;
   }
-  const FxSpecKernels* spec = spec_of(pl);
-  if (!spec && pl->needs_compiled) {
-    char key[17];
-    snprintf(key, sizeof key, "%016llx", (unsigned long long)pl->spec_key);
-    return fail(FX_E_LIMIT, std::string("the interpreter's temporaries of this region need ") + std::to_string(pl->lds_bytes) +
-                                " bytes of LDS (limit 65536) and no compiled kernels for its programs (key " + key +
-                                ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
-  }
-  g_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
-  if (spec) g_spec_launches.fetch_add((uint64_t)pl->launches, std::memory_order_relaxed);
+  const int launches = streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
+  g_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
+  if (spec) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
   const bool timed = kernel_ms != nullptr;
@@ -508,6 +635,15 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
       HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
+  } else if (streaming) {
+    HIP_OK(mark(0));
+    for (int r = 0; r < repeat; ++r) {
+      li.epoch = epoch + (uint32_t)r;
+      li.total_units = pl->stream.grid;
+      HIP_OK(fx_launch_compact_stream(pl->max_rank, sb, li, &dyn, stream_grid(pl), stream, spec));
+    }
+    HIP_OK(mark(1));
+    nk = pl->stream.grid > 0 ? 1 : 0;
   } else {
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) HIP_OK(fx_launch_compact_count(sb, li, &dyn, pl->grid_count, stream, spec));
@@ -543,7 +679,6 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   fx::Plan* pl = const_cast<fx::Plan*>(P(plan));
   if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
   if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
-  if (which >= pl->launches) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
   const bool compact = pl->mode == FX_MODE_COMPACT;
   if (compact && (!scratch || !totals_host)) return fail(FX_E_INVALID, "compacting region needs scratch and totals per set");
   hipStream_t stream = (hipStream_t)stream_;
@@ -553,21 +688,27 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
                             compact ? totals_host[i] : nullptr, stream_, nullptr, 0, nullptr);
     if (rc != FX_OK) return rc;
   }
+  const FxSpecKernels* spec = spec_of(pl);
+  FxLaunchInfo li = launch_info(pl);
+  bool streaming = compact && stream_active(pl, spec);
+  void* status = nullptr;
+  uint32_t epoch = 0;
+  int dev = 0;
+  HIP_OK(hipGetDevice(&dev));
+  if (streaming) {
+    const int rc = stream_status(reg, pl, stream, dev, &status, &epoch, rounds * n_sets);
+    if (rc != FX_OK) return rc;
+    if (!status) streaming = false;
+  }
+  if (which >= (streaming ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
   std::vector<FxDyn> dyn((size_t)n_sets);
   for (int i = 0; i < n_sets; ++i) {
     memset(&dyn[i], 0, sizeof(FxDyn));
     const int rc = fill_dyn(pl, args[i], out_ptrs[i], compact ? scratch[i] : nullptr, compact ? totals_host[i] : nullptr,
-                            pl->dev_blob, &dyn[i]);
+                            pl->dev_blob, &dyn[i], status);
     if (rc != FX_OK) return rc;
   }
   const uint32_t* sb = (const uint32_t*)pl->dev_blob;
-  FxLaunchInfo li;
-  li.blob_words = (uint32_t)pl->blob.size();
-  li.n_p = (uint32_t)(pl->sptr.size() + pl->tptr.size() * (size_t)reg->r.degree);
-  li.n_s = (uint32_t)(pl->sscal.size() + pl->tscal.size() * (size_t)reg->r.degree);
-  li.n_temps = pl->n_temps;
-  li.total_units = pl->mode == FX_MODE_DENSE ? pl->grid : 0;
-  const FxSpecKernels* spec = spec_of(pl);
   hipEvent_t e0 = nullptr, e1 = nullptr;
   HIP_OK(hipEventCreate(&e0));
   HIP_OK(hipEventCreate(&e1));
@@ -577,6 +718,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     for (int i = 0; i < n_sets; ++i) {
       if (!compact) {
         HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+      } else if (streaming) {
+        li.epoch = epoch + (uint32_t)(r * n_sets + i);
+        li.total_units = pl->stream.grid;
+        HIP_OK(fx_launch_compact_stream(pl->max_rank, sb, li, &dyn[i], stream_grid(pl), stream, spec));
       } else {
         if (which < 0 || which == 0) HIP_OK(fx_launch_compact_count(sb, li, &dyn[i], pl->grid_count, stream, spec));
         if (which < 0 || which == 1) HIP_OK(fx_launch_compact_scatter(pl->max_rank, sb, li, &dyn[i], pl->grid, stream, spec));

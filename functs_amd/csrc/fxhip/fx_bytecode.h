@@ -157,6 +157,15 @@ struct FxLaunchInfo {
   uint32_t n_s;         // scalar slots in use
   uint32_t n_temps;     // LDS temp slots per lane
   uint32_t total_units; // dense kernel: number of FX_UNIT work units
+  // streaming compaction (zero otherwise): see FxLaunch in fx_device.h
+  uint32_t epoch, spin_limit, win_words;
+  uint32_t s_tiles, s_rows, s_tile_rows, s_win_slot, s_win_stride;
+  int32_t s_win_tcoef, s_win_lo;
+  uint32_t s_win_span, n_sptr, n_tptr;
+  uint32_t n_side;
+  uint32_t side_slot[2], side_stride[2];
+  int32_t side_tcoef[2], side_lo[2];
+  uint32_t side_span[2], side_words[2];
 };
 
 #define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table
@@ -233,7 +242,8 @@ struct FxHeader {
   uint32_t total_words;
   uint32_t max_rows;     // stride of the per-task row-flag table
   uint32_t slot_err;     // 1 + shared pointer slot of the error word that FX_I64 loads report to (0: none)
-  uint32_t pad[2];
+  uint32_t slot_status;  // streaming compaction: shared pointer slot of the tile status words
+  uint32_t pad[1];
 };
 
 // dynamic (per call) arguments, passed by value in the kernarg segment

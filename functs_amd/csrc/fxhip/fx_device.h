@@ -24,6 +24,7 @@ __device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballo
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
 
+#define FX_SIDE_WIN 2
 struct FxCtx {
   const fx_u32x4* insn;   // LDS: class instruction base
   const uint32_t* aff;    // LDS: class affine base (FX_AFF_WORDS words each)
@@ -35,6 +36,22 @@ struct FxCtx {
   uint32_t wseg;          // lanes per segment of the wave reductions (rows per wave = 64 / wseg)
   int task;
   uint64_t err;           // error word that guarded int64 loads report to (0: the region has none)
+  // Streaming row compaction: the rows of the tile of the region's widest row-major input sit in
+  // LDS; affine loads of that buffer read them there.  win[off - win_base] is element `off` of
+  // the buffer (nullptr: no window, every load goes to memory).
+  // all_win is a compile-time fact wherever a context is used (set from a constant next to
+  // where the context is made; everything is inlined): with it, EVERY affine load of the
+  // region's programs reads a window (the host only plans such regions for the streaming
+  // kernel), so the code holds no load from memory at all and a wave never waits for the
+  // memory pipeline (which would also mean waiting for every store it has issued).
+  bool all_win;
+  const uint32_t* win;
+  int32_t win_slot;
+  int32_t win_base;
+  // the same for up to FX_SIDE_WIN narrow inputs that are read row by row (anchor tables ...)
+  const uint32_t* side[FX_SIDE_WIN];
+  int32_t side_slot[FX_SIDE_WIN];
+  int32_t side_base[FX_SIDE_WIN];
 };
 
 // Data buffers are plain device allocations: address them through the global
@@ -149,6 +166,37 @@ __device__ __forceinline__ uint64_t fx_ptr(const FxCtx& cx, int32_t slot) {
   const uint32_t i = (slot & FX_SLOT_TASK) ? cx.tp_off + (uint32_t)(slot & 0xffff) : (uint32_t)(slot & 0xffff);
   const uint64_t p = cx.ptrs[i];
   return ((uint64_t)uni((uint32_t)(p >> 32)) << 32) | (uint64_t)uni((uint32_t)p);
+}
+
+// Affine load of an instruction: from the staged window when the buffer is the window's, from
+// memory otherwise.  The window holds 32-bit elements (float or int32).
+// the staged window that holds buffer `slot` (wave-uniform); selects, no branch
+__device__ __forceinline__ const uint32_t* fx_window_of(const FxCtx& cx, uint32_t slot, int32_t& base) {
+  const uint32_t* w = cx.win;
+  base = cx.win_base;
+#pragma unroll
+  for (int i = 0; i < FX_SIDE_WIN; ++i) {
+    const bool hit = slot == (uint32_t)cx.side_slot[i];
+    w = hit ? cx.side[i] : w;
+    base = hit ? cx.side_base[i] : base;
+  }
+  return w;
+}
+
+__device__ __forceinline__ void fx_load(const FxCtx& cx, int32_t slot, const int32_t (&off)[FX_V], uint32_t M,
+                                        uint32_t dt, bool cvt, bool consecutive, uint32_t (&out)[FX_V]) {
+  if (cx.all_win) {
+    int32_t wbase;
+    const uint32_t* wnd = fx_window_of(cx, uni((uint32_t)slot), wbase);
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) out[j] = wnd[((M >> j) & 1u) ? off[j] - wbase : 0];
+    if (cvt) {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) out[j] = f2u((float)(int32_t)out[j]);
+    }
+    return;
+  }
+  fx_load_vec(fx_ptr(cx, slot), off, M, dt, cvt, consecutive, out, cx.err);
 }
 
 __device__ __forceinline__ uint32_t fx_scalar(const FxCtx& cx, int32_t slot) {
@@ -400,7 +448,7 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
       } else {
         int32_t off[FX_V];
         const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
-        fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, B, cx.err);
+        fx_load(cx, ia, off, M, dt, cvt, consecutive, B);
       }
     }
 
@@ -412,7 +460,7 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
         int32_t off[FX_V];
         const bool consecutive = fx_affine<R>(cx, q, ib, lc0, lc1, off);
         if (op == FX_LDA) {
-          fx_load_vec(fx_ptr(cx, ia), off, M, dt, cvt, consecutive, A, cx.err);
+          fx_load(cx, ia, off, M, dt, cvt, consecutive, A);
         } else {
 #pragma unroll
           for (int j = 0; j < FX_V; ++j) {
@@ -799,6 +847,9 @@ struct FxLead {
   uint64_t err;
   uint32_t dt;
   bool cvt;
+  bool lds;              // the load reads a staged window (see FxCtx::all_win)
+  const uint32_t* win;
+  int32_t win_base;
 };
 
 template <int R>
@@ -821,6 +872,10 @@ __device__ __forceinline__ FxLead fx_lead_decode(const FxCtx& cx, int pc) {
   ld.base = (int32_t)uni(a1.y) + (int32_t)uni(a1.x) * cx.task;
   ld.p = fx_ptr(cx, (int32_t)w.y);
   ld.err = cx.err;
+  ld.lds = cx.all_win;
+  ld.win = nullptr;
+  ld.win_base = 0;
+  if (cx.all_win) ld.win = fx_window_of(cx, uni(w.y), ld.win_base);
   return ld;
 }
 
@@ -828,6 +883,15 @@ template <int R>
 __device__ __forceinline__ void fx_lead_load(const FxLead& ld, const FxCoord<R>& q, uint32_t M, uint32_t (&P)[FX_V]) {
   int32_t off[FX_V];
   const bool consecutive = fx_offsets<R>(q, ld.cf, ld.base, off);
+  if (ld.lds) {
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) P[j] = ld.win[((M >> j) & 1u) ? off[j] - ld.win_base : 0];
+    if (ld.cvt) {
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) P[j] = f2u((float)(int32_t)P[j]);
+    }
+    return;
+  }
   fx_load_vec(ld.p, off, M, ld.dt, ld.cvt, consecutive, P, ld.err);
 }
 
@@ -854,7 +918,17 @@ __device__ __forceinline__ void fx_lead_batch(const FxLead& ld, MI&& make_item, 
     o0[k] = M ? (uint32_t)off[0] : 0u;
     fast = fast && consecutive && !wave_any(M != 0u && M != VM) && wave_any(M == VM);
   }
-  if (fast) {
+  if (fast && ld.lds) {
+#pragma unroll
+    for (int k = 0; k < KP; ++k) {
+      const uint32_t* wp = ld.win + (Mk[k] ? (int32_t)o0[k] - ld.win_base : 0);
+      X[k * FX_V + 0] = wp[0]; X[k * FX_V + 1] = wp[1]; X[k * FX_V + 2] = wp[2]; X[k * FX_V + 3] = wp[3];
+    }
+    if (ld.cvt) {
+#pragma unroll
+      for (int j = 0; j < KP * FX_V; ++j) X[j] = f2u((float)(int32_t)X[j]);
+    }
+  } else if (fast) {
     const FX_AS1 uint8_t* base = (const FX_AS1 uint8_t*)ld.p;
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
@@ -908,11 +982,19 @@ __device__ __forceinline__ void fx_rows_batch(const FxCtx& cx, const FxLead& ld,
     o0[k] = live[k] ? off : 0u;
     e0[k] = gg * FX_V;
   }
-  const FX_AS1 uint8_t* src = (const FX_AS1 uint8_t*)ld.p;
+  if (ld.lds) {
 #pragma unroll
-  for (uint32_t k = 0; k < KP; ++k) {
-    const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)(src + (o0[k] << 2));
-    X[k * FX_V + 0] = v.x; X[k * FX_V + 1] = v.y; X[k * FX_V + 2] = v.z; X[k * FX_V + 3] = v.w;
+    for (uint32_t k = 0; k < KP; ++k) {
+      const uint32_t* wp = ld.win + (live[k] ? (int32_t)o0[k] - ld.win_base : 0);
+      X[k * FX_V + 0] = wp[0]; X[k * FX_V + 1] = wp[1]; X[k * FX_V + 2] = wp[2]; X[k * FX_V + 3] = wp[3];
+    }
+  } else {
+    const FX_AS1 uint8_t* src = (const FX_AS1 uint8_t*)ld.p;
+#pragma unroll
+    for (uint32_t k = 0; k < KP; ++k) {
+      const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)(src + (o0[k] << 2));
+      X[k * FX_V + 0] = v.x; X[k * FX_V + 1] = v.y; X[k * FX_V + 2] = v.z; X[k * FX_V + 3] = v.w;
+    }
   }
   if (ld.cvt) {
     asm volatile("" ::: "memory");
@@ -938,9 +1020,33 @@ struct FxLaunch {
   uint32_t n_p;         // pointers in use in FxDyn::p
   uint32_t n_s;         // scalars in use in FxDyn::s
   uint32_t temps_off;   // word offset of the temp area in LDS (multiple of 4)
-  uint32_t pad;         // keeps the struct at 24 bytes: the tables that follow it in the argument segment are 8-byte aligned
+  uint32_t epoch;       // streaming compaction: tag of this call's tile counts (1 .. 2^23 - 1)
   uint32_t total_units; // dense: work units of FX_UNIT elements; the grid strides over them
+  // streaming compaction (fx_compact_stream; one task class): everything a workgroup needs to
+  // find its rows of the window input comes from the argument segment, so that the loads of the
+  // tile are issued before anything else is read
+  uint32_t win_off;      // word offset of the window in LDS (multiple of 4)
+  uint32_t spin_limit;   // polls of a look-back wait before the workgroup counts the rows itself
+  uint32_t s_tiles;      // row tiles per task
+  uint32_t s_rows;       // rows per task
+  uint32_t s_tile_rows;  // rows per tile (<= FX_BLOCK)
+  uint32_t s_win_slot;   // pointer slot of the window input (FX_SLOT_TASK: per-task table)
+  uint32_t s_win_stride; // elements per row of the window input
+  int32_t s_win_tcoef;   // element offset per task
+  int32_t s_win_lo;      // smallest element offset a program reads inside a row
+  uint32_t s_win_span;   // elements from there to the largest one, inclusive
+  uint32_t n_sptr;       // layout of the pointer table: shared pointers, then n_tptr per task
+  uint32_t n_tptr;
+  uint32_t win_buf;      // words of the window (multiple of 4)
+  uint32_t n_side;       // side windows in use (at most 64 16-byte lines per lane group: 256 lines each)
+  uint32_t side_slot[FX_SIDE_WIN];
+  uint32_t side_stride[FX_SIDE_WIN];
+  int32_t side_tcoef[FX_SIDE_WIN];
+  int32_t side_lo[FX_SIDE_WIN];
+  uint32_t side_span[FX_SIDE_WIN];
+  uint32_t side_off[FX_SIDE_WIN];   // word offsets in LDS (multiples of 4)
 };
+static_assert(sizeof(FxLaunch) % 8 == 0, "the tables that follow FxLaunch in the argument segment are 8-byte aligned");
 #define FX_KERNARG_DYN_OFF (8 + sizeof(FxLaunch))
 
 template <uint32_t NT = FX_BLOCK>
@@ -999,6 +1105,12 @@ __device__ __forceinline__ FxCtx fx_make_ctx(uint32_t* L, const FxLaunch& la, co
   cx.temps = L + la.temps_off + threadIdx.x;
   cx.wseg = 64;
   cx.task = w.task;
+  cx.all_win = false;
+  cx.win = nullptr;
+  cx.win_slot = -1;
+  cx.win_base = 0;
+#pragma unroll
+  for (int i = 0; i < FX_SIDE_WIN; ++i) { cx.side[i] = nullptr; cx.side_slot[i] = -1; cx.side_base[i] = 0; }
   const uint32_t se = uni(L[FX_W(FxHeader, slot_err)]);
   cx.err = 0;
   if (se) {
@@ -1212,76 +1324,19 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_compact_count(const uint32_t* __r
 }
 
 // --------------------------------------------------------------------------
-// row compaction, pass 2.  One workgroup per (task, row tile):
-//   offset  = sum of the keep counts of the earlier tiles of this task
-//   row map = kept rows of this tile in source order (ballot + popcount prefix)
-//   for every output: evaluate its program on the kept rows only and write
-//   rows [offset, offset + kept) of the compacted output.
-// The last tile of a task also publishes the task's total.
+// Outputs of one row tile of a compaction: every output's program evaluated on the kept rows
+// (rowmap: their row numbers in source order), written to rows [prefix, prefix + n_kept) of the
+// compacted output.  Shared by the second pass of the two-pass form and the streaming kernel.
 // --------------------------------------------------------------------------
-template <int R, class S = FxInterp>
-__global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(const uint32_t* __restrict__ sb,
-                                                                              const FxLaunch la, const FxDyn) {
-  constexpr uint32_t NW = S::kWaves, NT = 64u * NW;   // the row tile is at most FX_BLOCK rows, NT >= FX_BLOCK
-  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
-  __shared__ uint32_t s_rowmap[FX_BLOCK];
-  __shared__ uint32_t s_wsum[NW];
-  __shared__ uint32_t s_woff[NW + 1];
-  __shared__ uint32_t s_prefix;
-  fx_stage<NT>(L, sb, la);
-  const FxWork w = fx_locate<false>(L, blockIdx.x);
-  FxCtx cx = fx_make_ctx(L, la, w);
-
-  const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
-  const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
-  const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
-  const uint32_t tile = w.local_block;
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const FX_AS1 uint8_t* flags =
-      (const FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * uni(L[FX_W(FxHeader, max_rows)]);
-  const FX_AS1 uint32_t* counts =
-      (const FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
-
-  // this thread's row flag and its share of the counts of the earlier tiles: both loads are
-  // issued before either value is used
-  const uint32_t row = tile * rt + threadIdx.x;
-  const bool in_tile = (threadIdx.x < rt) && (row < n_rows);
-  const uint32_t flag = in_tile ? (uint32_t)flags[row] : 0u;
-  // exclusive offset of this tile
-  uint32_t part = 0;
-  for (uint32_t t = threadIdx.x; t < tile; t += NT) part += counts[t];
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
-  if (lane == 0) s_wsum[wave] = part;
-
-  // row map of this tile
-  const bool keep = flag != 0u;
-  const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
-  const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
-  if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t p = 0;
-    for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
-    s_prefix = p;
-    uint32_t acc = 0;
-    s_woff[0] = 0;
-    for (uint32_t k = 1; k <= NW; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
-  }
-  __syncthreads();
-  if (keep) s_rowmap[s_woff[wave] + before] = row;
-  __syncthreads();
-  const uint32_t n_kept = uni(s_woff[NW]);
-  const uint32_t prefix = uni(s_prefix);
-  if (tile + 1 == uni(w.cls[FX_W(FxClass, n_rowtiles)]) && threadIdx.x == 0) {
-    // The host polls this word while the kernel still runs: a system-scope store goes through
-    // to host memory instead of waiting in L2 for the end of the kernel.  (Relaxed: the host
-    // reads the count only; everything else of the call is consumed in stream order.)
-    __hip_atomic_store((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])] + w.task, prefix + n_kept, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_SYSTEM);
-  }
-  if (n_kept == 0) return;
-
+struct FxNoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+// before_last(): called by every wave in front of the last output of its walk
+template <int R, class S, uint32_t NW, class HK = FxNoHook>
+__device__ __forceinline__ void fx_scatter_outputs(const FxCtx& cx, const FxWork& w, const uint32_t* L,
+                                                   const uint32_t* s_rowmap, const uint32_t n_kept,
+                                                   const uint32_t prefix, const uint32_t lane, const uint32_t wave,
+                                                   HK&& before_last = FxNoHook()) {
   const uint32_t n_outs = uni(w.cls[FX_W(FxClass, n_outs)]);
   const uint32_t* outs = L + uni(w.cls[FX_W(FxClass, off_outs)]);
   const uint32_t ow = sizeof(FxOut) / 4;
@@ -1295,6 +1350,7 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   // arithmetic-bound wide outputs of the other waves.
   const bool backwards = S::kWalk == 0 ? ((blockIdx.x + wave_u) & 1u) != 0 : S::kWalk == 2;
   for (uint32_t oo = 0; oo < n_outs; ++oo) {
+    if (oo + 1u == n_outs) before_last();
     const uint32_t oi = backwards ? n_outs - 1u - oo : oo;
     const uint32_t* od = outs + oi * ow;
     const uint32_t rowlen = uni(od[FX_W(FxOut, rowlen)]);
@@ -1450,3 +1506,319 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   }
 }
 
+// --------------------------------------------------------------------------
+// row compaction, pass 2.  One workgroup per (task, row tile):
+//   offset  = sum of the keep counts of the earlier tiles of this task
+//   row map = kept rows of this tile in source order (ballot + popcount prefix)
+//   for every output: evaluate its program on the kept rows only and write
+//   rows [offset, offset + kept) of the compacted output.
+// The last tile of a task also publishes the task's total.
+// --------------------------------------------------------------------------
+template <int R, class S = FxInterp>
+__global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(const uint32_t* __restrict__ sb,
+                                                                              const FxLaunch la, const FxDyn) {
+  constexpr uint32_t NW = S::kWaves, NT = 64u * NW;   // the row tile is at most FX_BLOCK rows, NT >= FX_BLOCK
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
+  __shared__ uint32_t s_rowmap[FX_BLOCK];
+  __shared__ uint32_t s_wsum[NW];
+  __shared__ uint32_t s_woff[NW + 1];
+  __shared__ uint32_t s_prefix;
+  fx_stage<NT>(L, sb, la);
+  const FxWork w = fx_locate<false>(L, blockIdx.x);
+  FxCtx cx = fx_make_ctx(L, la, w);
+
+  const uint32_t n_rows = uni(w.cls[FX_W(FxClass, n_rows)]);
+  const uint32_t rt = uni(L[FX_W(FxHeader, row_tile)]);
+  const uint32_t max_rowtiles = uni(L[FX_W(FxHeader, max_rowtiles)]);
+  const uint32_t tile = w.local_block;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const FX_AS1 uint8_t* flags =
+      (const FX_AS1 uint8_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_flags)])] + (size_t)w.task * uni(L[FX_W(FxHeader, max_rows)]);
+  const FX_AS1 uint32_t* counts =
+      (const FX_AS1 uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_counts)])] + (size_t)w.task * max_rowtiles;
+
+  // this thread's row flag and its share of the counts of the earlier tiles: both loads are
+  // issued before either value is used
+  const uint32_t row = tile * rt + threadIdx.x;
+  const bool in_tile = (threadIdx.x < rt) && (row < n_rows);
+  const uint32_t flag = in_tile ? (uint32_t)flags[row] : 0u;
+  // exclusive offset of this tile
+  uint32_t part = 0;
+  for (uint32_t t = threadIdx.x; t < tile; t += NT) part += counts[t];
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+  if (lane == 0) s_wsum[wave] = part;
+
+  // row map of this tile
+  const bool keep = flag != 0u;
+  const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+  const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+  if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t p = 0;
+    for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
+    s_prefix = p;
+    uint32_t acc = 0;
+    s_woff[0] = 0;
+    for (uint32_t k = 1; k <= NW; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
+  }
+  __syncthreads();
+  if (keep) s_rowmap[s_woff[wave] + before] = row;
+  __syncthreads();
+  const uint32_t n_kept = uni(s_woff[NW]);
+  const uint32_t prefix = uni(s_prefix);
+  if (tile + 1 == uni(w.cls[FX_W(FxClass, n_rowtiles)]) && threadIdx.x == 0) {
+    // The host polls this word while the kernel still runs: a system-scope store goes through
+    // to host memory instead of waiting in L2 for the end of the kernel.  (Relaxed: the host
+    // reads the count only; everything else of the call is consumed in stream order.)
+    __hip_atomic_store((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])] + w.task, prefix + n_kept, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  if (n_kept == 0) return;
+
+  fx_scatter_outputs<R, S, NW>(cx, w, L, s_rowmap, n_kept, prefix, lane, wave);
+}
+
+// --------------------------------------------------------------------------
+// Row compaction in ONE pass (opt-in, fx_set_streaming) for regions with one task class whose
+// inputs are all row-major matrices that the programs read row by row (the prediction tensor
+// of a detection head and its anchor tables).  Persistent workgroups stride over (task, row
+// tile) pairs:
+//   1. The tile's rows of every input are contiguous runs of memory.  They are fetched with
+//      coalesced 128-bit loads whose addresses come from the argument segment alone (issued
+//      before anything else for the first tile, and for the next tile while the current one is
+//      worked on: the lines travel in registers) and parked in LDS ("windows").  The programs
+//      then read nothing but LDS: the code holds no load from memory, so a wave never waits for
+//      the memory pipeline, where it would also wait for every store it has issued.
+//   2. mask program per row (from the window), ballot + popcount row map, tile count.
+//   3. The count is published in a status word tagged with the call's epoch; the tile's write
+//      offset is the sum of the counts of the earlier tiles of its task, read from their status
+//      words as they appear (earlier tiles never wait for later ones).  Every poll loop is
+//      bounded: when a word does not show up within spin_limit polls the workgroup counts the
+//      kept rows of the earlier tiles itself, from memory, so the kernel ends whatever the order
+//      in which workgroups are started.
+//   4. outputs as in the two-pass form (fx_scatter_outputs).
+// Status words belong to the library (one per tile, zero when allocated, never reset: a word
+// of an earlier call carries an older epoch).
+// --------------------------------------------------------------------------
+#ifndef FX_STREAM_OCC
+#define FX_STREAM_OCC 2   // waves per SIMD the register budget is set for: two workgroups per CU
+#endif
+#define FX_STATUS_BITS 9u   // a tile holds at most FX_BLOCK = 256 rows
+
+// Where the rows of tile `b` of the window input start, in 16-byte lines, and how many lines
+// they span.
+struct FxWinAddr {
+  const FX_AS1 fx_u32x4* g4;
+  uint32_t n_vec, shift, r0, rows, task_i, tile;
+  int32_t e0;
+};
+__device__ __forceinline__ FxWinAddr fx_win_addr_of(const FxLaunch& la, uint32_t b, uint32_t sl, uint32_t stride,
+                                                    int32_t tcoef, int32_t lo, uint32_t span) {
+  FxWinAddr a;
+  a.task_i = b / la.s_tiles;
+  a.tile = b - a.task_i * la.s_tiles;
+  a.r0 = a.tile * la.s_tile_rows;
+  a.rows = min(la.s_tile_rows, la.s_rows - a.r0);
+  const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
+  const uint64_t* gp = (const uint64_t*)(ka + FX_KERNARG_DYN_OFF);
+  const uint32_t pi = (sl & FX_SLOT_TASK) ? la.n_sptr + a.task_i * la.n_tptr + (sl & 0xffffu) : (sl & 0xffffu);
+  const uint64_t wp = gp[pi];
+  a.e0 = tcoef * (int32_t)a.task_i + (int32_t)(a.r0 * stride) + lo;   // >= 0 (host)
+  const uint32_t n_el = (a.rows - 1u) * stride + span;
+  const uint64_t a0 = wp + ((uint64_t)(uint32_t)a.e0 << 2);
+  a.shift = ((uint32_t)a0 & 15u) >> 2;            // elements between the 16-byte line and e0
+  a.g4 = (const FX_AS1 fx_u32x4*)(a0 & ~(uint64_t)15);
+  a.n_vec = (a.shift + n_el + 3u) >> 2;           // <= window words / 4 (host)
+  return a;
+}
+__device__ __forceinline__ FxWinAddr fx_win_addr(const FxLaunch& la, uint32_t b) {
+  return fx_win_addr_of(la, b, la.s_win_slot, la.s_win_stride, la.s_win_tcoef, la.s_win_lo, la.s_win_span);
+}
+__device__ __forceinline__ FxWinAddr fx_side_addr(const FxLaunch& la, uint32_t b, int i) {
+  return fx_win_addr_of(la, b, la.side_slot[i], la.side_stride[i], la.side_tcoef[i], la.side_lo[i], la.side_span[i]);
+}
+
+#define FX_WK 12   // 128-bit loads per lane that carry the next tile's rows while this tile is worked on
+template <int R, class S = FxInterp>
+__global__ __launch_bounds__(FX_BLOCK, FX_STREAM_OCC) void fx_compact_stream(const uint32_t* __restrict__ sb,
+                                                                            const FxLaunch la, const FxDyn) {
+  constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u;
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
+  __shared__ uint32_t s_rowmap[FX_BLOCK];
+  __shared__ uint32_t s_wsum[NW];
+  __shared__ uint32_t s_woff[NW + 1];
+  __shared__ uint32_t s_prefix, s_ok;
+  const uint32_t n_tiles = la.total_units;   // tiles of the whole call; the workgroups stride over them
+  const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
+  fx_u32x4* const w4 = (fx_u32x4*)(L + la.win_off);
+
+  // the rows of the first tile are on their way before anything else is read
+  fx_u32x4 wr[FX_WK];
+  {
+    const FxWinAddr a = fx_win_addr(la, blockIdx.x);
+#pragma unroll
+    for (uint32_t k = 0; k < FX_WK; ++k) {
+      const uint32_t v = threadIdx.x + k * NT;
+      if (v < a.n_vec) wr[k] = a.g4[v];
+    }
+  }
+  fx_u32x4 ws[FX_SIDE_WIN];   // side windows: one line per lane
+#pragma unroll
+  for (int i = 0; i < FX_SIDE_WIN; ++i) {
+    if ((uint32_t)i < la.n_side) {
+      const FxWinAddr a = fx_side_addr(la, blockIdx.x, i);
+      if (threadIdx.x < a.n_vec) ws[i] = a.g4[threadIdx.x];
+    }
+  }
+  fx_stage(L, sb, la);   // descriptor and tables; ends with a barrier
+  const uint32_t* cls0 = L + uni(L[FX_W(FxHeader, off_class)]);
+  const int mb = (int)uni(cls0[FX_W(FxClass, mask_begin)]), me = (int)uni(cls0[FX_W(FxClass, mask_end)]);
+  const uint32_t mask_vt = uni(cls0[FX_W(FxClass, mask_vt)]);
+
+  for (uint32_t b = blockIdx.x; b < n_tiles; b += gridDim.x) {
+    const FxWinAddr wa = fx_win_addr(la, b);
+    __syncthreads();   // the previous tile's window and row map are no longer read
+#pragma unroll
+    for (uint32_t k = 0; k < FX_WK; ++k) {
+      const uint32_t v = threadIdx.x + k * NT;
+      if (v < wa.n_vec) w4[v] = wr[k];
+    }
+    for (uint32_t v = threadIdx.x + FX_WK * NT; v < wa.n_vec; v += NT) w4[v] = wa.g4[v];
+    FxWinAddr sa[FX_SIDE_WIN];
+#pragma unroll
+    for (int i = 0; i < FX_SIDE_WIN; ++i) {
+      if ((uint32_t)i < la.n_side) {
+        sa[i] = fx_side_addr(la, b, i);
+        if (threadIdx.x < sa[i].n_vec) ((fx_u32x4*)(L + la.side_off[i]))[threadIdx.x] = ws[i];
+      }
+    }
+    __syncthreads();
+
+    // one task class: tile and task follow from the tile number
+    FxWork w;
+    w.cls = cls0;
+    w.local_block = wa.tile;
+    w.task = (int)uni(L[uni(L[FX_W(FxHeader, off_taskmap)]) + wa.task_i]);
+    FxCtx cx = fx_make_ctx(L, la, w);
+    cx.all_win = true;
+    cx.win = L + la.win_off + wa.shift;
+    cx.win_slot = (int32_t)la.s_win_slot;
+    cx.win_base = wa.e0;
+#pragma unroll
+    for (int i = 0; i < FX_SIDE_WIN; ++i) {
+      if ((uint32_t)i < la.n_side) {
+        cx.side[i] = L + la.side_off[i] + sa[i].shift;
+        cx.side_slot[i] = (int32_t)la.side_slot[i];
+        cx.side_base[i] = sa[i].e0;
+      }
+    }
+
+    // ---- mask, row map ----------------------------------------------------
+    auto mask_of = [&](const FxCtx& c, uint32_t row, bool live) -> bool {
+      FxCoord<1> q;
+      q.c0[0] = 0;
+      q.vd = 0;
+      q.step = 0;
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) q.cv[j] = 0;
+      q.cv[0] = live ? (int32_t)row : 0;
+      uint32_t A[FX_V];
+#pragma unroll
+      for (int j = 0; j < FX_V; ++j) A[j] = 0;
+      S::run_mask(c, mb, me, q, live ? 1u : 0u, A);
+      return live && (mask_vt == FX_VT_F ? (u2f(A[0]) != 0.0f) : (A[0] != 0u));
+    };
+    const uint32_t row = wa.r0 + threadIdx.x;
+    const bool keep = mask_of(cx, row, threadIdx.x < wa.rows);
+    const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+    const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) s_woff[wave + 1] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t acc = 0;
+      s_woff[0] = 0;
+      for (uint32_t k = 1; k <= NW; ++k) { acc += s_woff[k]; s_woff[k] = acc; }
+    }
+    __syncthreads();
+    if (keep) s_rowmap[s_woff[wave] + before] = row;
+    const uint32_t n_kept = uni(s_woff[NW]);
+
+    // ---- publish the count, sum the earlier tiles --------------------------
+    uint32_t* status = (uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_status)])];
+    if (threadIdx.x == 0)
+      __hip_atomic_store(status + b, (la.epoch << FX_STATUS_BITS) | n_kept, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0) {
+      const uint32_t first = b - wa.tile;
+      uint32_t part = 0;
+      bool ok = true;
+      for (uint32_t i = lane; i < wa.tile; i += 64u) {
+        uint32_t wv = 0, polls = 0;
+        for (;;) {
+          wv = __hip_atomic_load(status + first + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if ((wv >> FX_STATUS_BITS) == la.epoch) break;
+          if (polls >= la.spin_limit) { ok = false; break; }
+          ++polls;
+          __builtin_amdgcn_s_sleep(1);
+        }
+        part += ok ? (wv & ((1u << FX_STATUS_BITS) - 1u)) : 0u;
+      }
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+      const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
+      if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
+    }
+    __syncthreads();
+    if (uni(s_ok) == 0u) {
+      // an earlier tile has not reported in time: count its kept rows here, from memory
+      FxCtx cg = cx;
+      cg.all_win = false;
+      uint32_t cnt = 0;
+      for (uint32_t p = 0; p < wa.tile; ++p) {
+        const bool k2 = mask_of(cg, p * la.s_tile_rows + threadIdx.x, threadIdx.x < la.s_tile_rows);
+        cnt += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(k2));
+      }
+      __syncthreads();
+      if (lane == 0) s_wsum[wave] = cnt;
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t p = 0;
+        for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
+        s_prefix = p;
+      }
+      __syncthreads();
+    }
+    const uint32_t prefix = uni(s_prefix);
+    if (wa.tile + 1u == la.s_tiles && threadIdx.x == 0)
+      __hip_atomic_store((uint32_t*)cx.ptrs[uni(L[FX_W(FxHeader, slot_total)])] + w.task, prefix + n_kept, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
+
+    // ---- outputs.  The rows of this workgroup's next tile are requested in front of the last,
+    // widest output: behind the loads that the narrow outputs wait for, because loads return in
+    // order.  They travel in registers until the next turn of the loop parks them in LDS.
+    const uint32_t bn = b + gridDim.x;
+    auto prefetch = [&]() {
+      if (bn < n_tiles) {
+        const FxWinAddr na = fx_win_addr(la, bn);
+#pragma unroll
+        for (uint32_t k = 0; k < FX_WK; ++k) {
+          const uint32_t v = threadIdx.x + k * NT;
+          if (v < na.n_vec) wr[k] = na.g4[v];
+        }
+#pragma unroll
+        for (int i = 0; i < FX_SIDE_WIN; ++i) {
+          if ((uint32_t)i < la.n_side) {
+            const FxWinAddr a = fx_side_addr(la, bn, i);
+            if (threadIdx.x < a.n_vec) ws[i] = a.g4[threadIdx.x];
+          }
+        }
+      }
+    };
+    if (n_kept == 0) {
+      prefetch();
+      continue;
+    }
+    fx_scatter_outputs<R, S, NW>(cx, w, L, s_rowmap, n_kept, prefix, lane, wave, prefetch);
+  }
+}

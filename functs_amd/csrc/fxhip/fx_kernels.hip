@@ -188,6 +188,7 @@ const FxSpecKernels* fx_spec_find(uint64_t hash) {
   auto it = spec_table().find(hash);
   return it == spec_table().end() ? nullptr : &it->second;   // entries are never erased
 }
+bool fx_spec_has_stream(const FxSpecKernels* spec) { return spec && spec->stream != nullptr; }
 int fx_spec_count() {
   std::lock_guard<std::mutex> g(spec_mutex());
   return (int)spec_table().size();
@@ -207,7 +208,31 @@ static FxLaunch make_launch(const FxLaunchInfo& li) {
   la.n_s = li.n_s;
   la.temps_off = (li.blob_words + 2 * li.n_p + li.n_s + 3u) & ~3u;
   la.total_units = li.total_units;
-  la.pad = 0;
+  la.epoch = li.epoch;
+  la.win_off = la.temps_off;   // compiled kernels; the interpreter's launcher moves it behind the temporaries
+  la.spin_limit = li.spin_limit;
+  la.s_tiles = li.s_tiles;
+  la.s_rows = li.s_rows;
+  la.s_tile_rows = li.s_tile_rows;
+  la.s_win_slot = li.s_win_slot;
+  la.s_win_stride = li.s_win_stride;
+  la.s_win_tcoef = li.s_win_tcoef;
+  la.s_win_lo = li.s_win_lo;
+  la.s_win_span = li.s_win_span;
+  la.n_sptr = li.n_sptr;
+  la.n_tptr = li.n_tptr;
+  la.win_buf = li.win_words;
+  la.n_side = li.n_side;
+  uint32_t off = la.win_off + li.win_words;
+  for (int i = 0; i < FX_SIDE_WIN; ++i) {
+    la.side_slot[i] = li.side_slot[i];
+    la.side_stride[i] = li.side_stride[i];
+    la.side_tcoef[i] = li.side_tcoef[i];
+    la.side_lo[i] = li.side_lo[i];
+    la.side_span[i] = li.side_span[i];
+    la.side_off[i] = off;
+    off += li.side_words[i];
+  }
   return la;
 }
 
@@ -257,6 +282,36 @@ hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunc
     case 3: fx_compact_scatter<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
     case 4: fx_compact_scatter<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
     default: fx_compact_scatter<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+  }
+  return hipGetLastError();
+}
+
+// LDS a streaming launch needs: descriptor and tables, the interpreter's temporaries, the window
+uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled) {
+  const FxLaunch la = make_launch(li);
+  const uint32_t temps = compiled ? 0u : li.n_temps * FX_V * FX_BLOCK;
+  return (la.temps_off + temps + li.win_words + li.side_words[0] + li.side_words[1]) * 4u;
+}
+
+hipError_t fx_launch_compact_stream(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
+                                    hipStream_t stream, const FxSpecKernels* spec) {
+  if (grid == 0) return hipSuccess;
+  FxLaunch la = make_launch(li);
+  if (spec && spec->stream) return launch_spec(spec->stream, sb, la, dyn, grid, fx_stream_lds_bytes(li, true), stream);
+  {
+    // the interpreter's temporaries sit between the tables and the windows
+    const uint32_t shift = li.n_temps * FX_V * FX_BLOCK;
+    la.win_off += shift;
+    for (int i = 0; i < FX_SIDE_WIN; ++i) la.side_off[i] += shift;
+  }
+  const uint32_t lds = fx_stream_lds_bytes(li, false);
+  switch (rank) {
+    case 0:
+    case 1: fx_compact_stream<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 2: fx_compact_stream<2><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 3: fx_compact_stream<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 4: fx_compact_stream<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    default: fx_compact_stream<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
   }
   return hipGetLastError();
 }

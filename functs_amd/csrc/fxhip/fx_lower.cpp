@@ -1775,6 +1775,82 @@ static void fillDims(FxOut& o, const Shape& s) {
 }  // namespace
 
 // ---------------------------------------------------------------------------
+// Window input of a streaming compaction: a tensor input of 32-bit elements that every program
+// of the class reads through affine loads of the form  t * task + S * row + (offset inside the
+// row)  with one S and one t, so that the rows of a tile are one contiguous run of memory which
+// the programs use most of.  Returns false when there is none.
+// ---------------------------------------------------------------------------
+struct WinCand {
+  bool seen = false, bad = false;
+  int64_t stride = 0, tcoef = 0, lo = 0, hi = 0;
+};
+struct WinPick { int slot; int64_t stride, tcoef, lo, span; };
+static bool findWindow(const ClassBuild& cb, StreamInfo* si, std::vector<WinPick>* others) {
+  std::map<int, WinCand> cand;   // by pointer slot
+  bool indirect = false;
+  auto scan = [&](uint32_t pb, uint32_t pe, const int64_t* dim, int rank) {
+    for (uint32_t pc = pb; pc < pe; ++pc) {
+      const FxInsn& in = cb.code[pc];
+      const bool affine_load = in.op == FX_LDA || in.op == FX_LDB || (in.flags & FX_F_MEMB);
+      if (in.op == FX_LDXA) indirect = true;   // a load through a computed index: stays in memory
+      if (in.flags & FX_F_TMPB) continue;
+      if (!affine_load) continue;
+      WinCand& c = cand[in.a];
+      const FxAffine& a = cb.affs[in.b];
+      if ((in.dt != FX_F32 && in.dt != FX_I32) || a.rcoef[0] != 0 || a.rcoef[1] != 0) { c.bad = true; continue; }
+      const int64_t S = fx_aff_coef(&a, 0);
+      int64_t lo = a.base, hi = a.base;
+      for (int k = 1; k < FX_MAXR; ++k) {
+        const int64_t cf = fx_aff_coef(&a, k);
+        if (cf == 0) continue;
+        if (k >= rank) { c.bad = true; break; }
+        const int64_t ext = cf * (dim[k] - 1);
+        lo += std::min<int64_t>(ext, 0);
+        hi += std::max<int64_t>(ext, 0);
+      }
+      if (c.bad) continue;
+      if (S <= 0) { c.bad = true; continue; }
+      if (!c.seen) { c.seen = true; c.stride = S; c.tcoef = a.tcoef; c.lo = lo; c.hi = hi; }
+      else if (c.stride != S || c.tcoef != a.tcoef) c.bad = true;
+      else { c.lo = std::min(c.lo, lo); c.hi = std::max(c.hi, hi); }
+    }
+  };
+  const int64_t mdim[FX_MAXR] = {(int64_t)cb.cls.n_rows, 1, 1, 1, 1, 1};
+  scan(cb.cls.mask_begin, cb.cls.mask_end, mdim, 1);
+  for (const FxOut& od : cb.outs) {
+    int64_t dim[FX_MAXR];
+    for (int k = 0; k < FX_MAXR; ++k) dim[k] = od.dim[k];
+    scan(od.prog_begin, od.prog_end, dim, (int)std::max<uint32_t>(od.rank, 1));
+  }
+  int best = -1;
+  for (auto& kv : cand) {
+    const WinCand& c = kv.second;
+    if (!c.seen || c.bad || c.lo < 0 || c.tcoef < 0) continue;
+    const int64_t span = c.hi - c.lo + 1;
+    if (span > c.stride || 2 * span < c.stride) continue;   // rows must be mostly used, and not overlap
+    if (best < 0 || c.stride > cand[best].stride) best = kv.first;
+  }
+  if (best < 0 || indirect) return false;
+  // the streaming kernel reads every input from LDS: each of them must be a window
+  for (auto& kv : cand) {
+    const WinCand& c = kv.second;
+    if (kv.first == best) continue;
+    if (!c.seen || c.bad || c.lo < 0 || c.tcoef < 0) return false;
+    const int64_t span = c.hi - c.lo + 1;
+    if (span > c.stride) return false;
+    others->push_back({kv.first, c.stride, c.tcoef, c.lo, span});
+  }
+  if (others->size() > 2) return false;
+  const WinCand& c = cand[best];
+  si->win_slot = (uint32_t)best;
+  si->win_stride = (uint32_t)c.stride;
+  si->win_tcoef = (int32_t)c.tcoef;
+  si->win_lo = (int32_t)c.lo;
+  si->win_span = (uint32_t)(c.hi - c.lo + 1);
+  return true;
+}
+
+// ---------------------------------------------------------------------------
 // plan construction
 // ---------------------------------------------------------------------------
 static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args);
@@ -2044,6 +2120,42 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   P->max_rank = max_rank;
   P->n_temps = (uint32_t)max_temps;
 
+  // streaming form of a compaction: one task class with a window input
+  int slot_status = 0;
+  std::vector<WinPick> side_cand;
+  if (P->mode == FX_MODE_COMPACT && classes.size() == 1 && classes[0].cls.n_rows > 0 &&
+      findWindow(classes[0], &P->stream, &side_cand)) {
+    const ClassBuild& cb = classes[0];
+    StreamInfo& si = P->stream;
+    // a window must stay inside its buffer for every tile of every task
+    auto inside = [&](uint32_t slot, int64_t stride, int64_t tcoef, int64_t lo, int64_t span) {
+      const uint32_t idx = slot & 0xffffu;
+      const bool per_task = (slot & FX_SLOT_TASK) != 0;
+      const PtrSrc& src = per_task ? slots.tptr[idx] : slots.sptr[idx];
+      if (src.kind != PtrSrc::INPUT) return false;
+      const fx_arg& a = args[arg_base[src.index] + (R.vals[R.inputs[src.index]].per_task ? cb.tasks[0] : 0)];
+      int64_t extent = 1;
+      for (int d = 0; d < a.rank; ++d) extent += a.sizes[d] > 0 ? (a.sizes[d] - 1) * a.strides[d] : 0;
+      for (int d = 0; d < a.rank; ++d) if (a.sizes[d] == 0) extent = 0;
+      const int64_t last = tcoef * (T - 1) + (int64_t)(cb.cls.n_rows - 1) * stride + lo + span;
+      return last <= extent && last < ((int64_t)1 << 30);
+    };
+    if (inside(si.win_slot, si.win_stride, si.win_tcoef, si.win_lo, si.win_span)) {
+      si.ok = true;
+      si.rows = cb.cls.n_rows;
+      slot_status = slots.ptrSlotSpecial(PtrSrc::STATUS);
+      for (const WinPick& w : side_cand) {
+        if (!inside((uint32_t)w.slot, w.stride, w.tcoef, w.lo, w.span)) { si.ok = false; break; }
+        const uint32_t i = si.n_side++;
+        si.side_slot[i] = (uint32_t)w.slot;
+        si.side_stride[i] = (uint32_t)w.stride;
+        si.side_tcoef[i] = (int32_t)w.tcoef;
+        si.side_lo[i] = (int32_t)w.lo;
+        si.side_span[i] = (uint32_t)w.span;
+      }
+    }
+  }
+
   // checked int64 loads report to an error word of the library
   int slot_err = 0;
   if (uses_guard) slot_err = slots.ptrSlotSpecial(PtrSrc::ERRWORD) + 1;
@@ -2110,6 +2222,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   h.slot_counts = (uint32_t)slot_counts;
   h.slot_total = (uint32_t)slot_total;
   h.slot_err = (uint32_t)slot_err;
+  h.slot_status = (uint32_t)slot_status;
   appendStruct(blob, h);
   for (auto& cb : classes) {
     while (blob.size() % 4) blob.push_back(0);
@@ -2149,6 +2262,39 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   FX_CHECK(lds_descriptor <= 64 * 1024, FX_E_LIMIT,
            "region descriptor needs " << lds_descriptor << " bytes of LDS (limit 65536)");
   P->needs_compiled = P->lds_bytes > 64 * 1024;
+  if (P->stream.ok) {
+    // Rows per workgroup: the largest of 256 / 128 / 64 whose window fits LDS next to the
+    // descriptor (compiled kernels keep temporaries in registers; the interpreter checks its own
+    // budget when it launches); smaller while the launch would leave CUs without a workgroup.
+    StreamInfo& si = P->stream;
+    const int64_t budget = 64000 - (int64_t)lds_descriptor;
+    uint32_t rt = 0;
+    auto buf_words = [&](uint32_t rows) { return (3 + (int64_t)(rows - 1) * si.win_stride + si.win_span + 3) & ~(int64_t)3; };
+    auto side_words_of = [&](uint32_t rows, uint32_t i) {
+      return (3 + (int64_t)(rows - 1) * si.side_stride[i] + si.side_span[i] + 3) & ~(int64_t)3;
+    };
+    // a side window is one 16-byte line per lane: at most FX_BLOCK lines; wider ones stay in memory
+    auto side_total = [&](uint32_t rows) {
+      int64_t w = 0;
+      for (uint32_t i = 0; i < si.n_side; ++i)
+        w += side_words_of(rows, i) <= 4 * FX_BLOCK ? side_words_of(rows, i) : ((int64_t)1 << 40);   // must fit
+      return w;
+    };
+    for (uint32_t cand : {256u, 128u, 64u}) {
+      if ((buf_words(cand) + side_total(cand)) * 4 > budget) continue;
+      rt = cand;
+      const int64_t tiles = (int64_t)T * ((si.rows + cand - 1) / cand);
+      if (tiles >= 512 || cand == 64u) break;
+    }
+    if (rt == 0) si.ok = false;
+    else {
+      si.tile_rows = rt;
+      si.tiles_per_task = (si.rows + rt - 1) / rt;
+      si.grid = si.tiles_per_task * (uint32_t)T;
+      si.win_words = (uint32_t)buf_words(rt);
+      for (uint32_t i = 0; i < 2; ++i) si.side_words[i] = i < si.n_side ? (uint32_t)side_words_of(rt, i) : 0u;
+    }
+  }
   P->spec_key = spec_hash(*P);
   const Plan* res = P.get();
   R.plans[key] = std::move(P);

@@ -67,12 +67,32 @@ struct Region {
 
 // where a dynamic pointer / scalar slot is filled from at run time
 struct PtrSrc {
-  enum Kind { INPUT, OUTPUT, FLAGS, COUNTS, TOTALS, ERRWORD } kind;
+  enum Kind { INPUT, OUTPUT, FLAGS, COUNTS, TOTALS, ERRWORD, STATUS } kind;
   int index;  // region input index / output index
 };
 struct ScalSrc {
   int input;      // region input index
   bool as_float;  // store float(value) instead of int32(value)
+};
+
+// Streaming (one-pass) form of a row compaction, available when the region has one task class
+// and its widest row-major input is read row by row by every program (fx_compact_stream).
+struct StreamInfo {
+  bool ok = false;
+  uint32_t tile_rows = 0;       // rows per workgroup
+  uint32_t tiles_per_task = 0;
+  uint32_t rows = 0;            // rows per task
+  uint32_t grid = 0;
+  uint32_t win_slot = 0;        // pointer slot of the window input
+  uint32_t win_stride = 0;      // elements per row
+  int32_t win_tcoef = 0;        // element offset per task
+  int32_t win_lo = 0;           // smallest element offset the programs read inside a row
+  uint32_t win_span = 0;        // elements from there to the largest one, inclusive
+  uint32_t win_words = 0;       // LDS words of the window (multiple of 4)
+  // narrow inputs read row by row as well (at most 256 16-byte lines per tile): staged beside it
+  uint32_t n_side = 0;
+  uint32_t side_slot[2] = {0, 0}, side_stride[2] = {0, 0}, side_span[2] = {0, 0}, side_words[2] = {0, 0};
+  int32_t side_tcoef[2] = {0, 0}, side_lo[2] = {0, 0};
 };
 
 struct Plan {
@@ -83,6 +103,7 @@ struct Plan {
   uint32_t grid_count = 0;     // compaction pass 1
   uint32_t lds_bytes = 0;
   bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
+  StreamInfo stream;
   bool uses_guard = false;       // some load checks int64 data against 32 bits and reports to the error word
   uint32_t n_temps = 0;
   int max_rank = 1;
@@ -99,6 +120,10 @@ struct Plan {
   uint64_t spec_key = 0;       // spec_hash of this plan
   void* dev_blob = nullptr;
   int dev_id = -1;
+  // streaming compaction: tile status words, one buffer per launch stream (zero when allocated,
+  // never reset: every call tags its words with the next epoch)
+  struct Status { void* stream; void* ptr; uint32_t epoch; int dev; };
+  std::vector<Status> status;
 };
 
 // Builds (or fetches from the cache) the plan of `r` for these arguments.

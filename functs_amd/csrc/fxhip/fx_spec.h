@@ -34,6 +34,7 @@ struct FxSpecKernels {
   const void* count = nullptr;    // fx_compact_count<FxSpec<P>>
   const void* scatter = nullptr;  // fx_compact_scatter<R, FxSpec<P>>
   uint32_t scatter_threads = 0;   // workgroup size that kernel is compiled for
+  const void* stream = nullptr;   // fx_compact_stream<R, FxSpec<P>>
 };
 void fx_spec_register(uint64_t hash, const FxSpecKernels& k);
 const FxSpecKernels* fx_spec_find(uint64_t hash);
@@ -177,7 +178,7 @@ __device__ __forceinline__ void fx_spec_prefetch(const FxCtx& cx, const FxCoord<
       constexpr FxInsn J = P::code[K];
       int32_t off[FX_V];
       const bool consecutive = fx_affine<R>(cx, q, J.b, rg.lc0, rg.lc1, off);
-      fx_load_vec(fx_ptr(cx, J.a), off, M, J.dt, (J.flags & FX_F_I2F) != 0, consecutive, ts.ld[K], cx.err);
+      fx_load(cx, J.a, off, M, J.dt, (J.flags & FX_F_I2F) != 0, consecutive, ts.ld[K]);
     }
     fx_spec_prefetch<P, R, K + 1, END, TS>(cx, q, ts, M, rg);
   }
@@ -369,12 +370,14 @@ struct FxSpec {
 };
 
 struct FxSpecRegistrar {
-  FxSpecRegistrar(uint64_t hash, const void* dense, const void* count, const void* scatter, uint32_t scatter_threads) {
+  FxSpecRegistrar(uint64_t hash, const void* dense, const void* count, const void* scatter, uint32_t scatter_threads,
+                  const void* stream = nullptr) {
     FxSpecKernels k;
     k.dense = dense;
     k.count = count;
     k.scatter = scatter;
     k.scatter_threads = scatter_threads;
+    k.stream = stream;
     fx_spec_register(hash, k);
   }
 };
@@ -385,4 +388,5 @@ struct FxSpecRegistrar {
   static FxSpecRegistrar fx_registrar_##P(P::hash, (const void*)&fx_region_dense<R, FxSpec<P>>, nullptr, nullptr, 0);
 #define FX_SPEC_COMPACT(P, R)                                                                    \
   static FxSpecRegistrar fx_registrar_##P(P::hash, nullptr, (const void*)&fx_compact_count<FxSpec<P>>, \
-                                          (const void*)&fx_compact_scatter<R, FxSpec<P>>, 64u * FxSpec<P>::kWaves);
+                                          (const void*)&fx_compact_scatter<R, FxSpec<P>>, 64u * FxSpec<P>::kWaves, \
+                                          (const void*)&fx_compact_stream<R, FxSpec<P>>);

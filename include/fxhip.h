@@ -165,6 +165,24 @@ int fx_plan_output(const fx_plan*, int out_idx, int task, int32_t* dtype, int32_
 size_t fx_plan_scratch_bytes(const fx_plan*); /* device scratch the caller must provide to fx_region_run */
 int fx_plan_launches(const fx_plan*);         /* kernel launches one fx_region_run issues */
 int64_t fx_plan_algorithmic_bytes(const fx_plan*); /* compulsory input bytes + dense output bytes */
+/* Row compaction in one pass (opt-in).  A compacting region with one task class whose inputs are
+ * all read row by row (the prediction tensor of a detection head, its anchor tables) can run as
+ * ONE kernel: persistent workgroups park their rows of the inputs in LDS with coalesced loads,
+ * evaluate the mask from there, publish their kept-row count and take their write offset from
+ * the counts of the earlier tiles (every wait bounded; a workgroup that waits too long counts
+ * the earlier rows itself).  Results are identical to the two-pass form (count + scatter), which
+ * is the default because it is the faster one on the benchmark configurations but the smallest.
+ * fx_plan_streaming: 1 if fx_region_run would use the one-pass form for this plan now;
+ * fx_set_streaming: process-wide switch (default off; FXHIP_STREAM=1: on);
+ * fx_set_stream_spin_limit: polls before a workgroup stops waiting (default 4000; 0 makes every
+ * workgroup count for itself, for tests).  No reference counterpart: the reference leaves
+ * x[mask] to ATen (convert_to_tensorssa.cpp:422-443). */
+int fx_plan_streaming(const fx_plan*);
+/* out[0..8): one-pass form available, rows per tile, tiles per task, grid, and the window input's
+ * row stride, per-task offset, first and number of elements used per row (test hook) */
+int fx_plan_stream_info(const fx_plan*, int64_t* out, int cap);
+void fx_set_streaming(int on);
+void fx_set_stream_spin_limit(uint32_t polls);
 /* debugging / test hooks: the lowered bytecode blob (like CodeGen::getCodeText) */
 int fx_plan_blob(const fx_plan*, const uint32_t** words, size_t* n_words);
 int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);

@@ -143,6 +143,11 @@ _sig("fx_compact_rows_scratch_bytes", ctypes.c_size_t, ctypes.c_int64)
 _sig("fx_compact_rows_static", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, _vp)
 _sig("fx_async_error", _i, _i)
+_fp = ctypes.c_void_p
+_sig("fx_lstm_stack_workspace_bytes", ctypes.c_size_t, _i, _i, _i)
+_sig("fx_lstm_stack_workspace_clear_bytes", ctypes.c_size_t)
+_sig("fx_lstm_stack", _i, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp)
+_sig("fx_set_lstm_spin_limit", None, ctypes.c_uint32)
 _sig("fx_device_count", _i)
 _sig("fx_copy_bytes", _i, _vp, _vp, ctypes.c_size_t, _vp)
 

@@ -35,6 +35,8 @@ hipError_t fx_launch_compact_stream(int rank, const uint32_t* sb, const FxLaunch
                                     hipStream_t stream, const FxSpecKernels* spec);
 uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled);
 bool fx_spec_has_stream(const FxSpecKernels* spec);
+#include "fx_lstm_sched.h"
+int fx_launch_lstm_stack(const FxLstmArgs& a, int L, hipStream_t stream);
 hipError_t fx_launch_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                          const int32_t* rowlen, const int32_t* elsize, int n_cols,
                                          uint32_t* total_host, hipStream_t stream);
@@ -243,6 +245,7 @@ static std::atomic<uint32_t> g_stream_spin{[] {
   const char* e = getenv("FXHIP_STREAM_SPIN");
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
 }()};
+static std::atomic<uint32_t> g_lstm_spin{1000000u};   // polls of a barrier wait of fx_lstm_stack before it gives up
 static std::mutex g_dump_mu;
 static std::string g_dump_dir;
 
@@ -847,6 +850,43 @@ int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, voi
                                 (hipStream_t)stream_));
   return FX_OK;
 }
+
+// ---- stacked LSTM recurrence as one persistent kernel (fx_lstm.hip) ----
+size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers) {
+  if (batch < 1 || hidden < 1 || layers < 1) return 0;
+  return (size_t)FX_LSTM_BAR_WORDS * 4 + (size_t)2 * layers * batch * hidden * 4;
+}
+size_t fx_lstm_stack_workspace_clear_bytes(void) { return (size_t)FX_LSTM_BAR_WORDS * 4; }
+
+int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,
+                  const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
+                  int layers, void* workspace, size_t workspace_bytes, void* stream_) {
+  if (!x || !wih || !whh || !bih || !bhh || !h0 || !c0 || !out || !state_h || !state_c || !workspace)
+    return fail(FX_E_INVALID, "fx_lstm_stack: null argument");
+  if (seq_len < 1 || batch < 1 || hidden < 1 || layers < 1) return fail(FX_E_INVALID, "fx_lstm_stack: sizes must be positive");
+  if (workspace_bytes < fx_lstm_stack_workspace_bytes(batch, hidden, layers))
+    return fail(FX_E_INVALID, "fx_lstm_stack: workspace smaller than fx_lstm_stack_workspace_bytes");
+  if (((uintptr_t)workspace & 255u) != 0) return fail(FX_E_INVALID, "fx_lstm_stack: workspace must be 256-byte aligned");
+  FxLstmArgs a;
+  a.x = x; a.wih = wih; a.whh = whh; a.bih = bih; a.bhh = bhh; a.h0 = h0; a.c0 = c0;
+  a.out = out; a.state_h = state_h; a.state_c = state_c;
+  a.bar = (uint32_t*)workspace;
+  a.hbuf = (float*)((char*)workspace + (size_t)FX_LSTM_BAR_WORDS * 4);
+  a.err_host = err_word(true);
+  a.T = seq_len; a.B = batch; a.H = hidden;
+  a.spin_limit = g_lstm_spin.load(std::memory_order_relaxed);
+  const int rc = fx_launch_lstm_stack(a, layers, (hipStream_t)stream_);
+  if (rc == 1)
+    return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: hidden must be a multiple of 32 up to 1024, 1..4 layers, batch up to 16 (got hidden " +
+                                      std::to_string(hidden) + ", layers " + std::to_string(layers) + ", batch " + std::to_string(batch) + ")");
+  if (rc == 2)
+    return fail(FX_E_LIMIT, "fx_lstm_stack: " + std::to_string(hidden) + " workgroups would not be resident together on this device");
+  if (rc != 0) return fail(FX_E_HIP, std::string("fx_lstm_stack: ") + hipGetErrorString((hipError_t)(rc - 100)));
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  g_spec_launches.fetch_add(1, std::memory_order_relaxed);
+  return FX_OK;
+}
+void fx_set_lstm_spin_limit(uint32_t polls) { g_lstm_spin.store(polls, std::memory_order_relaxed); }
 
 int fx_copy_bytes(const void* src, void* dst, size_t bytes, void* stream) {
   if (bytes % 16) return fail(FX_E_INVALID, "fx_copy_bytes: size must be a multiple of 16");

@@ -291,6 +291,29 @@ int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* co
                            const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* total_host,
                            void* stream);
 
+/* ---- stacked LSTM recurrence as one launch ----
+ * The loop nest of functs/benchmark/ai_model/lstm/lstm.py:79-133
+ *   for t in [0, T): cur = x[t]
+ *     for j in [0, L): gates = cur @ wih[j] + bih[j] + h[j] @ whh[j] + bhh[j]   (gate order i, f, g, o)
+ *                      c[j] = sigmoid(f) * c[j] + sigmoid(i) * tanh(g); h[j] = sigmoid(o) * tanh(c[j]); cur = h[j]
+ *     out[t] = cur
+ * which the reference runs on the host, one fused kernel and two library GEMMs per (t, j)
+ * (the loops carry state: fait/passes/parallelize_loops.cpp:17, unroll_loops.cpp:59-65), as ONE
+ * persistent kernel: a workgroup per hidden unit keeps its columns of the weights in registers
+ * for the whole sequence, the diagonals t + j are separated by a device-wide barrier with bounded
+ * waits (a wait that is given up sets the error word of fx_async_error and ends the kernel).
+ * Contiguous fp32: x [T, B, H]; wih, whh [L, 4, H, H]; bih, bhh [L, 4, 1, H]; h0, c0, state_h,
+ * state_c [L, B, H]; out [T, B, H].  H a multiple of 32 up to 1024, L <= 4, B <= 16
+ * (FX_E_UNSUPPORTED otherwise), and H workgroups must be resident together (FX_E_LIMIT).
+ * workspace: fx_lstm_stack_workspace_bytes() of device memory, 256-byte aligned, whose first
+ * fx_lstm_stack_workspace_clear_bytes() bytes are zero when the kernel starts. */
+size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers);
+size_t fx_lstm_stack_workspace_clear_bytes(void);
+int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,
+                  const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
+                  int layers, void* workspace, size_t workspace_bytes, void* stream);
+void fx_set_lstm_spin_limit(uint32_t polls); /* barrier polls before a wait is given up (default 1000000; tests) */
+
 /* ---- device utilities ---- */
 int fx_device_count(void);
 /* plain 16-byte copy kernel of known size: counter calibration and bandwidth ceiling */

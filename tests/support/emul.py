@@ -14,9 +14,25 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libfx_emul.so")
 
 
+_LSTM_SO = os.path.join(_HERE, "liblstm_emul.so")
+
+
 def build():
     src = os.path.join(_HERE, "fx_emul.cpp")
     subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", src, "-o", _SO])
+    src = os.path.join(_HERE, "lstm_emul.cpp")
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", src, "-o", _LSTM_SO])
+
+
+def lstm_emul():
+    """ctypes handle of the CPU build of the persistent LSTM kernel's schedule and barrier."""
+    if not os.path.exists(_LSTM_SO):
+        build()
+    so = ctypes.CDLL(_LSTM_SO)
+    fp = ctypes.c_void_p
+    so.fx_lstm_emul.restype = ctypes.c_int
+    so.fx_lstm_emul.argtypes = [fp] * 10 + [ctypes.c_int] * 4 + [ctypes.c_uint32, ctypes.c_int]
+    return so
 
 
 def _load():

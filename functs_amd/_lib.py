@@ -144,6 +144,7 @@ _sig("fx_compact_rows_static", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), cty
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, _vp)
 _sig("fx_async_error", _i, _i)
 _fp = ctypes.c_void_p
+_sig("fx_lstm_stack_fits", ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int)
 _sig("fx_lstm_stack_workspace_bytes", ctypes.c_size_t, _i, _i, _i)
 _sig("fx_lstm_stack_workspace_clear_bytes", ctypes.c_size_t)
 _sig("fx_lstm_stack", _i, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp)

@@ -873,6 +873,7 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   ConstantPropagation(graph);
   EliminateCommonSubexpression(graph);
   EliminateDeadCode(graph);
+  if (CollapseRecurrentLoops(graph)) EliminateDeadCode(graph);   // buffers the collapsed node no longer reads
   CollapseAssignLoops(graph);
   ParallelizeLoops(graph);
   FuseOps(graph);

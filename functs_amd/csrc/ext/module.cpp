@@ -28,6 +28,7 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_convert_to_tensorssa", ConvertToTensorSSA);
   m.def("_jit_pass_fait_fuse_ops", FuseOps);
   m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
+  m.def("_jit_pass_collapse_recurrent_loops", CollapseRecurrentLoops);
   m.def("_jit_pass_parallelize_loops", ParallelizeLoops);
   m.def("_jit_pass_split_parallel_maps", SplitParallelMaps);
   m.def("_jit_pass_unroll_loops_with_deps", UnrollLoopsWithDeps);

@@ -21,6 +21,11 @@ void FuseOps(std::shared_ptr<torch::jit::Graph> graph);
 // parallelises loops with carried values (parallelize_loops.cpp:17).
 void CollapseAssignLoops(std::shared_ptr<torch::jit::Graph> graph);
 
+// The (time, layer) loop nest of a stacked LSTM (functs/benchmark/ai_model/lstm/lstm.py:79-133),
+// whose loops carry the states, becomes one fx::lstm_stack node when the static shapes fit the
+// persistent kernel; true if the graph changed.
+bool CollapseRecurrentLoops(std::shared_ptr<torch::jit::Graph> graph);
+
 // fait/passes/parallelize_loops.cpp:12-145: loops without carried values whose
 // list reads are list[i] and whose list writes are one append per list become
 // prim::ParallelMap(len, lists...){block(i, elems...) -> rets}.

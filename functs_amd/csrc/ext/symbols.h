@@ -47,6 +47,8 @@ FUNCTS_SYM(ParallelMap, "prim::ParallelMap")
 // a prim::Loop whose carried tensor is read and written only through slab i,
 // collapsed to one node (no reference counterpart, see fuse_ops.cpp)
 FUNCTS_SYM(ForallSelectRev, "fx::forall_select_rev")
+// the (time, layer) loop nest of a stacked LSTM collapsed to one node (recurrent.cpp)
+FUNCTS_SYM(LstmStack, "fx::lstm_stack")
 // attributes of tssa::ParallelFunctor
 FUNCTS_SYM(parallel_degree, "attr::parallel_degree")
 FUNCTS_SYM(is_parallel_args, "attr::is_parallel_args")

@@ -20,6 +20,7 @@
 #include <torch/csrc/jit/passes/common_subexpression_elimination.h>
 #include <torch/csrc/jit/runtime/custom_operator.h>
 
+#include <map>
 #include <mutex>
 #include <sstream>
 
@@ -146,6 +147,41 @@ Node* functorFromMap(Node* mapNode, Node* group) {
   return f;
 }
 
+// fx::lstm_stack (the collapsed loop nest of a stacked LSTM, recurrent.cpp) as a region of one
+// node: its tensor and int operands are the arguments, its None operands stay constants.
+Node* functorFromLstmStack(Node* n) {
+  Graph* g = n->owningGraph();
+  Node* f = g->createWithSubgraph(sym::ParallelFunctor());
+  auto sub = f->g(c10::attr::Subgraph);
+  sub->addInput()->setType(c10::NoneType::get());
+  std::vector<c10::TypePtr> types;
+  std::vector<Value*> operands;
+  for (Value* in : n->inputs()) {
+    if (in->node()->kind() == c10::prim::Constant) {
+      Node* c = sub->createClone(in->node(), [](Value* x) { return x; });
+      sub->appendNode(c);
+      operands.push_back(c->output());
+      continue;
+    }
+    f->addInput(in);
+    types.push_back(in->type());
+    operands.push_back(sub->addInput()->copyMetadata(in));
+  }
+  Node* k = sub->create(sym::LstmStack(), operands, n->outputs().size());
+  sub->appendNode(k);
+  for (size_t i = 0; i < n->outputs().size(); ++i) {
+    k->output(i)->copyMetadata(n->output(i));
+    sub->registerOutput(k->output(i));
+    f->addOutput()->copyMetadata(n->output(i));
+  }
+  f->tys_(sym::input_refine_types(), types);
+  f->i_(sym::parallel_degree(), 1);
+  f->i_(sym::is_parallel_map(), 0);
+  f->is_(sym::is_parallel_args(), std::vector<int64_t>(types.size(), 1));
+  f->i_(sym::compact_rows(), 0);
+  return f;
+}
+
 // A map whose body did not end up as exactly one fused group goes back to a
 // loop (ConvertInfusibleMapsToLoops, parallelize_loops.cpp:295-362).
 Node* mapBackToLoop(Node* mapNode) {
@@ -200,8 +236,8 @@ void toFunctorIn(Block* b) {
   for (auto it = b->nodes().begin(); it != b->nodes().end();) {
     Node* n = *it;
     ++it;
-    if (n->kind() == c10::prim::FusionGroup) {
-      Node* f = functorFromGroup(n);
+    if (n->kind() == c10::prim::FusionGroup || n->kind() == sym::LstmStack()) {
+      Node* f = n->kind() == sym::LstmStack() ? functorFromLstmStack(n) : functorFromGroup(n);
       f->insertBefore(n);
       for (size_t k = 0; k < n->outputs().size(); ++k) n->output(k)->replaceAllUsesWith(f->output(k));
       n->destroy();
@@ -826,13 +862,156 @@ void RegionRunner::build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue>
   FX_OK_OR_THROW(fx_region_finalize(var.region));
 }
 
+// --- fx::lstm_stack -----------------------------------------------------------
+// Barrier words and the h exchange buffer of the persistent kernel, one per (device, stream):
+// cleared when allocated, and every launch that ends without error leaves them clear
+// (include/fxhip.h fx_lstm_stack), so a call costs the one launch.
+struct LstmWorkspaces {
+  std::mutex mu;
+  std::map<std::pair<int, void*>, at::Tensor> by_stream;
+  at::Tensor get(c10::Device dev, void* stream, size_t bytes) {
+    std::lock_guard<std::mutex> lock(mu);
+    at::Tensor& t = by_stream[{(int)dev.index(), stream}];
+    if (!t.defined() || (size_t)t.numel() < bytes)
+      t = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kByte).device(dev));   // on the current stream
+    return t;
+  }
+  void reset() {
+    std::lock_guard<std::mutex> lock(mu);
+    by_stream.clear();
+  }
+};
+LstmWorkspaces& lstmWorkspaces() {
+  static LstmWorkspaces* w = new LstmWorkspaces();   // tensors must not outlive the HIP runtime's teardown order
+  return *w;
+}
+
+// fx::lstm_stack(x, wih, whh, bih, bhh, out?, state_h?, state_c?, T, L) -> (out, state_h, state_c)
+// is the loop nest
+//   for t in range(T): cur = x[t]
+//     for j in range(L): (the LSTM cell of layer j on cur, state_h[j], state_c[j]); cur = h
+//     out[t] = cur
+// in functional form: the results are new tensors, rows [0, T) of out and layers [0, L) of the
+// states rewritten, the rest copied from the operands.  None for out means a [T, B, H] buffer that
+// the loops fill completely, None for a state means zeros [L, B, H].
+void runLstmStack(Stack& stack) {
+  auto in = last(stack, 10);
+  auto tensorArg = [&](size_t i, const char* name) {
+    TORCH_CHECK(in[i].isTensor(), "fx::lstm_stack: ", name, " must be a tensor");
+    at::Tensor t = in[i].toTensor();
+    TORCH_CHECK(t.is_cuda(), "fx::lstm_stack runs on the GPU only; ", name, " is a ", t.device(), " tensor");
+    TORCH_CHECK(t.scalar_type() == at::kFloat, "fx::lstm_stack: ", name, " must be float32");
+    return t.contiguous();
+  };
+  auto optionalArg = [&](size_t i, const char* name) { return in[i].isNone() ? at::Tensor() : tensorArg(i, name); };
+  const at::Tensor x = tensorArg(0, "x"), wih = tensorArg(1, "wih"), whh = tensorArg(2, "whh"), bih = tensorArg(3, "bih"),
+                   bhh = tensorArg(4, "bhh");
+  const at::Tensor out0 = optionalArg(5, "out"), h0 = optionalArg(6, "state_h"), c0 = optionalArg(7, "state_c");
+  const int64_t T = std::max<int64_t>(in[8].toInt(), 0), L = std::max<int64_t>(in[9].toInt(), 0);   // a negative trip count runs no iteration
+  TORCH_CHECK(x.dim() == 3, "fx::lstm_stack: x must be [T, B, H]");
+  const int64_t B = x.size(1), H = x.size(2);
+  TORCH_CHECK(T <= x.size(0), "fx::lstm_stack: index ", x.size(0), " is out of bounds for dimension 0 of x with size ", x.size(0));
+  auto weightArg = [&](const at::Tensor& w, const char* name, int64_t rows) {
+    TORCH_CHECK(w.dim() == 4 && w.size(1) == 4 && w.size(2) == rows && w.size(3) == H && w.size(0) >= L,
+                "fx::lstm_stack: ", name, " must be [layers >= ", L, ", 4, ", rows, ", ", H, "], got ", w.sizes());
+  };
+  weightArg(wih, "wih", H);
+  weightArg(whh, "whh", H);
+  weightArg(bih, "bih", 1);
+  weightArg(bhh, "bhh", 1);
+  TORCH_CHECK(wih.size(0) == L || L == 0 || (wih.size(0) == whh.size(0) && bih.size(0) == bhh.size(0)),
+              "fx::lstm_stack: the weights disagree on the number of layers");
+  auto rowsArg = [&](const at::Tensor& t, const char* name, int64_t need) {
+    if (!t.defined()) return need;
+    TORCH_CHECK(t.dim() == 3 && t.size(1) == B && t.size(2) == H && t.size(0) >= need, "fx::lstm_stack: ", name,
+                " must be [>= ", need, ", ", B, ", ", H, "], got ", t.sizes());
+    return t.size(0);
+  };
+  const int64_t To = rowsArg(out0, "out", T), Lh = rowsArg(h0, "state_h", L), Lc = rowsArg(c0, "state_c", L);
+  if (!out0.defined() || !h0.defined() || !c0.defined())
+    TORCH_CHECK(c10::get_default_dtype_as_scalartype() == at::kFloat,
+                "fx::lstm_stack: the program creates its buffers with the default dtype, which must be float32");
+  c10::DeviceGuard guard(x.device());
+  const auto opts = x.options();
+  const bool runs = T > 0 && L > 0;
+  // a result whose every element the kernel writes starts uninitialised, any other one as a copy
+  auto result = [&](const at::Tensor& init, int64_t rows, bool all_written) {
+    if (all_written) return at::empty({rows, B, H}, opts);
+    return init.defined() ? init.clone() : at::zeros({rows, B, H}, opts);
+  };
+  at::Tensor out = result(out0, To, runs && To == T);
+  at::Tensor sh = result(h0, Lh, runs && Lh == L);
+  at::Tensor sc = result(c0, Lc, runs && Lc == L);
+  if (T > 0 && L == 0) out.narrow(0, 0, T).copy_(x.narrow(0, 0, T));   // no layer: out[t] = x[t]
+  if (runs) {
+    const int e = fx_async_error(1);
+    if (e != 0) lstmWorkspaces().reset();   // a given-up barrier wait leaves its words as they were
+    TORCH_CHECK(e == 0, "an earlier launch reported an error (", e, e == 2 ? ": a barrier wait of fx_lstm_stack was given up"
+                : ": int64 element outside 32 bits in integer arithmetic", "); its results are not valid");
+    TORCH_CHECK(T <= INT32_MAX && B <= INT32_MAX && H <= INT32_MAX, "fx::lstm_stack: sizes beyond 32 bits");
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index());
+    const size_t ws_bytes = fx_lstm_stack_workspace_bytes((int)B, (int)H, (int)L);
+    at::Tensor ws = lstmWorkspaces().get(x.device(), (void*)stream.stream(), ws_bytes);
+    TORCH_CHECK(((uintptr_t)ws.data_ptr() & 255u) == 0, "fx::lstm_stack: workspace is not 256-byte aligned");
+    FX_OK_OR_THROW(fx_lstm_stack(x.data_ptr<float>(), wih.data_ptr<float>(), whh.data_ptr<float>(), bih.data_ptr<float>(),
+                                 bhh.data_ptr<float>(), h0.defined() ? h0.data_ptr<float>() : nullptr,
+                                 c0.defined() ? c0.data_ptr<float>() : nullptr, out.data_ptr<float>(), sh.data_ptr<float>(),
+                                 sc.data_ptr<float>(), (int)T, (int)B, (int)H, (int)L, ws.data_ptr(), (size_t)ws.numel(),
+                                 (void*)stream.stream()));
+  }
+  drop(stack, 10);
+  push(stack, std::move(out));
+  push(stack, std::move(sh));
+  push(stack, std::move(sc));
+}
+
+// the region of a functor made by functorFromLstmStack: one fx::lstm_stack node over the arguments
+const Node* loneLstmStack(const Graph& sub) {
+  const Node* found = nullptr;
+  for (const Node* n : sub.nodes()) {
+    if (n->kind() == c10::prim::Constant) continue;
+    if (n->kind() != sym::LstmStack() || found) return nullptr;
+    found = n;
+  }
+  return found;
+}
+
 Operation createParallelFunctor(const Node* node) {
+  auto sub = node->g(c10::attr::Subgraph);
+  if (const Node* k = loneLstmStack(*sub)) {
+    // operand i of the node: argument number (position among the functor's inputs) or a constant
+    struct Operand { int arg; c10::IValue constant; };
+    std::vector<Operand> operands;
+    for (const Value* v : k->inputs()) {
+      if (v->node()->kind() == c10::prim::Constant) {
+        operands.push_back({-1, *toIValue(v)});
+        continue;
+      }
+      size_t pos = 0;
+      while (pos < sub->inputs().size() && sub->inputs()[pos] != v) ++pos;
+      TORCH_CHECK(pos >= 1 && pos < sub->inputs().size(), "ParallelFunctor: fx::lstm_stack operand is not an argument");
+      operands.push_back({(int)pos - 1, c10::IValue()});
+    }
+    const size_t n_args = sub->inputs().size() - 1;
+    return [operands, n_args](Stack& stack) {
+      std::vector<c10::IValue> args;
+      for (const c10::IValue& v : last(stack, n_args)) args.push_back(v);
+      drop(stack, n_args);
+      for (const Operand& o : operands) stack.push_back(o.arg < 0 ? o.constant : args[(size_t)o.arg]);
+      runLstmStack(stack);
+    };
+  }
   auto runner = std::make_shared<RegionRunner>(node);
   return [runner](Stack& stack) { runner->run(stack); };
 }
 
 RegisterOperators registerFunctor({
     Operator(sym::ParallelFunctor(), createParallelFunctor, c10::AliasAnalysisKind::PURE_FUNCTION),
+    // the collapsed node itself is an operator too: graphs that hold it outside a functor (between
+    // the passes, or when ToParallelFunctor is not run) analyse and execute
+    Operator("fx::lstm_stack(Tensor x, Tensor wih, Tensor whh, Tensor bih, Tensor bhh, Tensor? out, Tensor? state_h, "
+             "Tensor? state_c, int T, int L) -> (Tensor, Tensor, Tensor)",
+             [](Stack& stack) { runLstmStack(stack); }, c10::AliasAnalysisKind::PURE_FUNCTION),
 });
 
 }  // namespace

@@ -852,6 +852,14 @@ int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, voi
 }
 
 // ---- stacked LSTM recurrence as one persistent kernel (fx_lstm.hip) ----
+int fx_lstm_stack_fits(int batch, int hidden, int layers) {
+  if (hidden < 32 || hidden > 1024 || (hidden & (hidden - 1)) != 0) return 0;
+  if (layers < 1 || layers > 4 || batch < 1 || batch > 16) return 0;
+  // 1024 workgroups on 256 compute units: four per unit, 128 registers a lane, of which the
+  // weights may take 48 (at 512 and below two workgroups per unit suffice and every L fits)
+  if (hidden == 1024 && layers * (hidden / 32) > 48) return 0;
+  return 1;
+}
 size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers) {
   if (batch < 1 || hidden < 1 || layers < 1) return 0;
   return (size_t)FX_LSTM_BAR_WORDS * 4 + (size_t)2 * layers * batch * hidden * 4;
@@ -861,12 +869,15 @@ size_t fx_lstm_stack_workspace_clear_bytes(void) { return (size_t)FX_LSTM_BAR_WO
 int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,
                   const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
                   int layers, void* workspace, size_t workspace_bytes, void* stream_) {
-  if (!x || !wih || !whh || !bih || !bhh || !h0 || !c0 || !out || !state_h || !state_c || !workspace)
-    return fail(FX_E_INVALID, "fx_lstm_stack: null argument");
+  if (!x || !wih || !whh || !bih || !bhh || !out || !state_h || !state_c || !workspace)
+    return fail(FX_E_INVALID, "fx_lstm_stack: null argument");   // h0 / c0 may be null: zero initial state
   if (seq_len < 1 || batch < 1 || hidden < 1 || layers < 1) return fail(FX_E_INVALID, "fx_lstm_stack: sizes must be positive");
   if (workspace_bytes < fx_lstm_stack_workspace_bytes(batch, hidden, layers))
     return fail(FX_E_INVALID, "fx_lstm_stack: workspace smaller than fx_lstm_stack_workspace_bytes");
   if (((uintptr_t)workspace & 255u) != 0) return fail(FX_E_INVALID, "fx_lstm_stack: workspace must be 256-byte aligned");
+  if (!fx_lstm_stack_fits(batch, hidden, layers))
+    return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: hidden must be a power of two in 32..1024, 1..4 layers (1 at hidden 1024), batch up to 16 (got hidden " +
+                                      std::to_string(hidden) + ", layers " + std::to_string(layers) + ", batch " + std::to_string(batch) + ")");
   FxLstmArgs a;
   a.x = x; a.wih = wih; a.whh = whh; a.bih = bih; a.bhh = bhh; a.h0 = h0; a.c0 = c0;
   a.out = out; a.state_h = state_h; a.state_c = state_c;
@@ -876,9 +887,7 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
   a.T = seq_len; a.B = batch; a.H = hidden;
   a.spin_limit = g_lstm_spin.load(std::memory_order_relaxed);
   const int rc = fx_launch_lstm_stack(a, layers, (hipStream_t)stream_);
-  if (rc == 1)
-    return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: hidden must be a multiple of 32 up to 1024, 1..4 layers, batch up to 16 (got hidden " +
-                                      std::to_string(hidden) + ", layers " + std::to_string(layers) + ", batch " + std::to_string(batch) + ")");
+  if (rc == 1) return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: no kernel for these sizes");
   if (rc == 2)
     return fail(FX_E_LIMIT, "fx_lstm_stack: " + std::to_string(hidden) + " workgroups would not be resident together on this device");
   if (rc != 0) return fail(FX_E_HIP, std::string("fx_lstm_stack: ") + hipGetErrorString((hipError_t)(rc - 100)));

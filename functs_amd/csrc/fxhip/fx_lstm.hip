@@ -66,7 +66,7 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK) void fx_lstm_stack_kernel(const FxLs
   // thread (j, b) owns the cell state of its layer and batch row
   const int own_j = (int)threadIdx.x / B, own_b = (int)threadIdx.x % B;
   const bool owner = own_j < L;
-  float c_reg = owner ? a.c0[((size_t)own_j * B + own_b) * H + u] : 0.0f;
+  float c_reg = (owner && a.c0) ? a.c0[((size_t)own_j * B + own_b) * H + u] : 0.0f;
 
   const int n_steps = fx_lstm_steps(T, L);
   for (int d = 0; d < n_steps; ++d) {
@@ -76,19 +76,20 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK) void fx_lstm_stack_kernel(const FxLs
       const int t = fx_lstm_time(d, j, T);
       if (t < 0) continue;
       for (int b = 0; b < B; ++b) {
-        const float* src;
-        bool coherent;   // written by other workgroups during this launch
+        const float* src;   // null: zeros (no initial state given)
+        bool coherent;      // written by other workgroups during this launch
         if (half == 0) {
           if (j == 0) { src = a.x + ((size_t)t * B + b) * H; coherent = false; }
           else { src = a.hbuf + fx_lstm_hoff(rp, j - 1, b, 0, L, B, H); coherent = true; }
         } else {
-          if (t == 0) { src = a.h0 + ((size_t)j * B + b) * H; coherent = false; }
+          if (t == 0) { src = a.h0 ? a.h0 + ((size_t)j * B + b) * H : nullptr; coherent = false; }
           else { src = a.hbuf + fx_lstm_hoff(rp, j, b, 0, L, B, H); coherent = true; }
         }
         float v[HPT];
 #pragma unroll
         for (int m = 0; m < HPT; ++m)
-          v[m] = coherent ? __hip_atomic_load(src + sub + 32 * m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : src[sub + 32 * m];
+          v[m] = coherent ? __hip_atomic_load(src + sub + 32 * m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                          : (src ? src[sub + 32 * m] : 0.0f);
         float s = 0.0f;
 #pragma unroll
         for (int m = 0; m < HPT; ++m) s = __builtin_fmaf(w[j][m], v[m], s);
@@ -129,6 +130,7 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK) void fx_lstm_stack_kernel(const FxLs
       if (s_go == 0u) return;   // a wait was given up somewhere: every workgroup leaves
     }
   }
+  if (threadIdx.x == 0) fx_lstm_leave<DevAtomics>(a.bar, gridDim.x);
 }
 
 typedef void (*fx_lstm_kernel_t)(const FxLstmArgs);

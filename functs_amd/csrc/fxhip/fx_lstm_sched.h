@@ -20,14 +20,15 @@
 
 #define FX_LSTM_GROUPS 16u         // first-level barrier counters
 #define FX_LSTM_LINE 64u           // words between counters: one 256-byte line each
-#define FX_LSTM_BAR_WORDS ((FX_LSTM_GROUPS + 2u) * FX_LSTM_LINE)   // groups, top counter, error word
+#define FX_LSTM_BAR_WORDS ((FX_LSTM_GROUPS + 3u) * FX_LSTM_LINE)   // groups, top counter, error word, leave counter
 
 // arguments of the kernel (contiguous fp32 tensors; see fx_lstm_stack in include/fxhip.h)
 struct FxLstmArgs {
-  const float *x, *wih, *whh, *bih, *bhh, *h0, *c0;
+  const float *x, *wih, *whh, *bih, *bhh;
+  const float *h0, *c0;   // null: zero initial state
   float *out, *state_h, *state_c;
   float* hbuf;         // [2][L][B][H]: h of the cells of the last two steps
-  uint32_t* bar;       // FX_LSTM_BAR_WORDS words, zero when the kernel starts
+  uint32_t* bar;       // FX_LSTM_BAR_WORDS words, zero when the kernel starts (and again when it ends without error)
   uint32_t* err_host;  // pinned word that a given-up wait reports to as well (may be null)
   int T, B, H;
   uint32_t spin_limit;
@@ -44,7 +45,7 @@ FX_LSTM_HD inline uint32_t fx_lstm_hoff(int p, int j, int b, int u, int L, int B
 }
 
 // Arrival at the barrier that closes step `gen` (1-based) and the wait for everybody else.
-// Counters only grow; the caller hands in zeroed words once per launch.  Two levels: a workgroup
+// Counters only grow during a launch and start from zero (fx_lstm_leave puts them back).  Two levels: a workgroup
 // adds to its group's counter, the last arrival of a group adds to the top counter, everybody
 // polls the top counter.  Returns false when the wait was given up (poll limit reached, or another
 // workgroup had already given up): the error word is set and the caller must leave the kernel.
@@ -72,4 +73,17 @@ FX_LSTM_HD inline bool fx_lstm_barrier(uint32_t* bar, uint32_t gen, uint32_t wg,
   }
   A::acquire();
   return true;
+}
+
+// A workgroup that has passed its last barrier of the launch checks out; the last one to do so
+// puts every counter back to zero, so the same words serve the next launch on the stream without
+// a clear in between.  Nobody polls any more at that point: a workgroup checks out only after its
+// own last wait has ended.  A workgroup that gave up a wait does not check out: the error word
+// stays set and the counters stay as they are until the host clears the words.
+template <class A>
+FX_LSTM_HD inline void fx_lstm_leave(uint32_t* bar, uint32_t n_wg) {
+  uint32_t* leave = bar + (FX_LSTM_GROUPS + 2u) * FX_LSTM_LINE;
+  if (A::add_release(leave) + 1u != n_wg) return;
+  for (uint32_t g = 0; g <= FX_LSTM_GROUPS; ++g) A::store(bar + g * FX_LSTM_LINE, 0u);
+  A::store(leave, 0u);
 }

@@ -303,10 +303,19 @@ int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* co
  * for the whole sequence, the diagonals t + j are separated by a device-wide barrier with bounded
  * waits (a wait that is given up sets the error word of fx_async_error and ends the kernel).
  * Contiguous fp32: x [T, B, H]; wih, whh [L, 4, H, H]; bih, bhh [L, 4, 1, H]; h0, c0, state_h,
- * state_c [L, B, H]; out [T, B, H].  H a multiple of 32 up to 1024, L <= 4, B <= 16
- * (FX_E_UNSUPPORTED otherwise), and H workgroups must be resident together (FX_E_LIMIT).
+ * state_c [L, B, H]; out [T, B, H]; h0 / c0 may be null (zero initial state).  H is 32, 64, ...
+ * 1024 (a power of two), L <= 4, B <= 16 (FX_E_UNSUPPORTED otherwise), and H workgroups must be
+ * resident together (FX_E_LIMIT).
  * workspace: fx_lstm_stack_workspace_bytes() of device memory, 256-byte aligned, whose first
- * fx_lstm_stack_workspace_clear_bytes() bytes are zero when the kernel starts. */
+ * fx_lstm_stack_workspace_clear_bytes() bytes are zero when the kernel starts.  A launch that ends
+ * without error leaves them zero again, so one workspace, cleared once, serves launch after launch
+ * on one stream (launches that share a workspace must not overlap); after a launch that reported
+ * an error through fx_async_error the caller clears them again. */
+/* 1 when fx_lstm_stack is built for these sizes, 0 otherwise: the part of its conditions that
+ * needs no device, for a compiler pass that decides whether to emit the call (H a power of two in
+ * 32..1024, L <= 4, B <= 16, and the weight columns of all layers fit the registers of a
+ * workgroup at the occupancy that keeps H workgroups resident: L * H / 32 <= 48 for H = 1024). */
+int fx_lstm_stack_fits(int batch, int hidden, int layers);
 size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers);
 size_t fx_lstm_stack_workspace_clear_bytes(void);
 int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,

@@ -10,6 +10,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <thread>
 #include <vector>
@@ -31,7 +32,7 @@ void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
   const int H = a.H, B = a.B, T = a.T;
   std::vector<float> c((size_t)L * B);
   for (int j = 0; j < L; ++j)
-    for (int b = 0; b < B; ++b) c[j * B + b] = a.c0[((size_t)j * B + b) * H + u];
+    for (int b = 0; b < B; ++b) c[j * B + b] = a.c0 ? a.c0[((size_t)j * B + b) * H + u] : 0.0f;
   const int n_steps = fx_lstm_steps(T, L);
   for (int d = 0; d < n_steps; ++d) {
     const int rp = (d + 1) & 1;
@@ -40,7 +41,7 @@ void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
       if (t < 0) continue;
       for (int b = 0; b < B; ++b) {
         const float* cur = j == 0 ? a.x + ((size_t)t * B + b) * H : a.hbuf + fx_lstm_hoff(rp, j - 1, b, 0, L, B, H);
-        const float* hp = t == 0 ? a.h0 + ((size_t)j * B + b) * H : a.hbuf + fx_lstm_hoff(rp, j, b, 0, L, B, H);
+        const float* hp = t == 0 ? (a.h0 ? a.h0 + ((size_t)j * B + b) * H : nullptr) : a.hbuf + fx_lstm_hoff(rp, j, b, 0, L, B, H);
         float g[4];
         for (int k = 0; k < 4; ++k) {
           const float* wi = a.wih + ((size_t)(j * 4 + k) * H) * H + u;
@@ -48,7 +49,7 @@ void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
           float si = 0.f, sh = 0.f;
           for (int i = 0; i < H; ++i) {
             si += wi[(size_t)i * H] * cur[i];
-            sh += wh[(size_t)i * H] * hp[i];
+            sh += wh[(size_t)i * H] * (hp ? hp[i] : 0.0f);
           }
           g[k] = (si + a.bih[(size_t)(j * 4 + k) * H + u]) + (sh + a.bhh[(size_t)(j * 4 + k) * H + u]);
         }
@@ -68,13 +69,16 @@ void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
       if (!fx_lstm_barrier<HostAtomics>(a.bar, (uint32_t)(d + 1), (uint32_t)u, (uint32_t)n_wg, a.spin_limit)) return;
     }
   }
+  fx_lstm_leave<HostAtomics>(a.bar, (uint32_t)n_wg);
 }
 }  // namespace
 
-// returns the error word (0: every barrier was passed)
+// `launches` runs of the same sequence, one after the other, on barrier words that are cleared only
+// once (h0 / c0 may be null: zero initial state).  Returns the error word (0: every barrier was
+// passed), or -1 when a run without error did not leave every barrier word at zero.
 extern "C" int fx_lstm_emul(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh,
                             const float* h0, const float* c0, float* out, float* state_h, float* state_c, int T, int B,
-                            int H, int L, uint32_t spin_limit, int skip_wg) {
+                            int H, int L, uint32_t spin_limit, int skip_wg, int launches) {
   std::vector<uint32_t> bar(FX_LSTM_BAR_WORDS, 0u);
   std::vector<float> hbuf((size_t)2 * L * B * H, NAN);   // a value read before it is written poisons the result
   FxLstmArgs a;
@@ -82,8 +86,15 @@ extern "C" int fx_lstm_emul(const float* x, const float* wih, const float* whh, 
   a.out = out; a.state_h = state_h; a.state_c = state_c;
   a.hbuf = hbuf.data(); a.bar = bar.data(); a.err_host = nullptr;
   a.T = T; a.B = B; a.H = H; a.spin_limit = spin_limit;
-  std::vector<std::thread> th;
-  for (int u = 0; u < H; ++u) th.emplace_back(workgroup, std::cref(a), L, u, H, skip_wg);
-  for (auto& t : th) t.join();
-  return (int)bar[(FX_LSTM_GROUPS + 1u) * FX_LSTM_LINE];
+  for (int n = 0; n < launches; ++n) {
+    std::fill(hbuf.begin(), hbuf.end(), NAN);
+    std::vector<std::thread> th;
+    for (int u = 0; u < H; ++u) th.emplace_back(workgroup, std::cref(a), L, u, H, skip_wg);
+    for (auto& t : th) t.join();
+    const int err = (int)bar[(FX_LSTM_GROUPS + 1u) * FX_LSTM_LINE];
+    if (err) return err;
+    for (uint32_t w : bar)
+      if (w != 0u) return -1;
+  }
+  return 0;
 }

@@ -64,14 +64,15 @@ def test_reference_with_zero_states_is_the_oracle():
         assert torch.allclose(a, b, rtol=1e-6, atol=1e-7)
 
 
-def _emul(x, wih, whh, bih, bhh, h0, c0, spin=1 << 30, skip=-1):
+def _emul(x, wih, whh, bih, bhh, h0, c0, spin=1 << 30, skip=-1, launches=1):
     from tests.support import emul
     so = emul.lstm_emul()
     T, B, H = x.shape
     L = wih.size(0)
     out, sh, sc = torch.zeros(T, B, H), torch.zeros(L, B, H), torch.zeros(L, B, H)
-    ts = [t.contiguous() for t in (x, wih, whh, bih, bhh, h0, c0)]
-    err = so.fx_lstm_emul(*[t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(), sc.data_ptr(), T, B, H, L, spin, skip)
+    ts = [None if t is None else t.contiguous() for t in (x, wih, whh, bih, bhh, h0, c0)]
+    err = so.fx_lstm_emul(*[None if t is None else t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(),
+                          sc.data_ptr(), T, B, H, L, spin, skip, launches)
     return (out, sh, sc), err
 
 
@@ -83,6 +84,22 @@ def test_schedule_and_barrier_on_host_threads(T, H, L, B):
     _close(got, _reference(*args), "emul T=%d H=%d L=%d B=%d" % (T, H, L, B))
 
 
+def test_launches_in_a_row_share_barrier_words_cleared_once():
+    """The last workgroup to leave puts the counters back to zero (-1: it did not)."""
+    args = _inputs(11, 6, 64, 3, 2)
+    got, err = _emul(*args, launches=3)
+    assert err == 0
+    _close(got, _reference(*args), "third launch")
+
+
+def test_no_initial_state_means_zeros():
+    x, wih, whh, bih, bhh, _, _ = _inputs(5, 6, 32, 2, 2)
+    got, err = _emul(x, wih, whh, bih, bhh, None, None)
+    assert err == 0
+    z = torch.zeros(2, 2, 32)
+    _close(got, _reference(x, wih, whh, bih, bhh, z, z), "zero state")
+
+
 def test_a_wait_that_cannot_end_is_given_up():
     """One workgroup never arrives: every other one must give up after the poll limit, set the
     error word and return (on the GPU the kernel then ends instead of hanging)."""
@@ -91,31 +108,42 @@ def test_a_wait_that_cannot_end_is_given_up():
     assert err == 1
 
 
-def _gpu(x, wih, whh, bih, bhh, h0, c0):
+def _gpu(x, wih, whh, bih, bhh, h0, c0, launches=1):
+    """`launches` calls in a row on one workspace that is cleared once; the last call's results."""
     from functs_amd._lib import check, lib
     dev = torch.device("cuda:0")
     T, B, H = x.shape
     L = wih.size(0)
-    ts = [t.contiguous().to(dev) for t in (x, wih, whh, bih, bhh, h0, c0)]
-    out = torch.empty(T, B, H, device=dev)
-    sh, sc = torch.empty(L, B, H, device=dev), torch.empty(L, B, H, device=dev)
+    ts = [None if t is None else t.contiguous().to(dev) for t in (x, wih, whh, bih, bhh, h0, c0)]
     nbytes = lib.fx_lstm_stack_workspace_bytes(B, H, L)
     ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
     assert ws.data_ptr() % 256 == 0
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    check(lib.fx_lstm_stack(*[t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(), sc.data_ptr(), T, B, H, L,
-                            ws.data_ptr(), nbytes, stream))
-    torch.cuda.synchronize()
-    assert lib.fx_async_error(1) == 0
+    for _ in range(launches):
+        out = torch.full((T, B, H), float("nan"), device=dev)
+        sh, sc = torch.full((L, B, H), float("nan"), device=dev), torch.full((L, B, H), float("nan"), device=dev)
+        print("fx_lstm_stack T=%d B=%d H=%d L=%d" % (T, B, H, L), flush=True)
+        check(lib.fx_lstm_stack(*[None if t is None else t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(),
+                                sc.data_ptr(), T, B, H, L, ws.data_ptr(), nbytes, stream))
+        torch.cuda.synchronize()
+        assert lib.fx_async_error(1) == 0
+    assert int(ws[:lib.fx_lstm_stack_workspace_clear_bytes()].count_nonzero()) == 0   # left as it was found
     return out.cpu(), sh.cpu(), sc.cpu()
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("T,H,L,B", [(1, 32, 1, 1), (5, 64, 2, 1), (9, 128, 3, 2), (4, 32, 4, 3), (16, 256, 2, 1),
-                                     (64, 512, 2, 1), (8, 1024, 1, 2)])
+                                     (64, 512, 2, 1), (6, 512, 4, 16), (8, 1024, 1, 2)])
 def test_kernel_against_the_oracle(T, H, L, B):
     args = _inputs(T + H + L, T, H, L, B)
     _close(_gpu(*args), _reference(*args), "gpu T=%d H=%d L=%d B=%d" % (T, H, L, B))
+
+
+@pytest.mark.gpu
+def test_launches_in_a_row_on_one_workspace_and_no_initial_state():
+    x, wih, whh, bih, bhh, _, _ = _inputs(21, 10, 128, 2, 2)
+    z = torch.zeros(2, 2, 128)
+    _close(_gpu(x, wih, whh, bih, bhh, None, None, launches=3), _reference(x, wih, whh, bih, bhh, z, z), "third launch")
 
 
 @pytest.mark.gpu
@@ -146,3 +174,10 @@ def test_unsupported_shapes_are_refused():
     assert rc == C["FX_E_UNSUPPORTED"]
     rc = lib.fx_lstm_stack(p, p, p, p, p, p, p, p, p, p, 4, 1, 64, 5, ws.data_ptr(), 1 << 20, None)   # five layers
     assert rc == C["FX_E_UNSUPPORTED"]
+
+
+def test_sizes_the_kernel_is_built_for():
+    from functs_amd._lib import lib
+    assert lib.fx_lstm_stack_fits(1, 512, 2) == 1 and lib.fx_lstm_stack_fits(16, 512, 4) == 1
+    assert lib.fx_lstm_stack_fits(1, 1024, 1) == 1 and lib.fx_lstm_stack_fits(1, 1024, 2) == 0
+    assert lib.fx_lstm_stack_fits(1, 96, 2) == 0 and lib.fx_lstm_stack_fits(17, 64, 2) == 0 and lib.fx_lstm_stack_fits(1, 64, 5) == 0

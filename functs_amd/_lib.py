@@ -33,6 +33,35 @@ class FxArg(ctypes.Structure):
     ]
 
 
+class FxNmsDesc(ctypes.Structure):
+    """fx_nms_desc of include/fxhip.h."""
+    _fields_ = [
+        ("mode", ctypes.c_int32),
+        ("n_tasks", ctypes.c_int32),
+        ("rows", ctypes.c_uint32),
+        ("n_classes", ctypes.c_uint32),
+        ("boxes", ctypes.c_void_p),
+        ("boxes_task_stride", ctypes.c_int64),
+        ("scores", ctypes.c_void_p),
+        ("scores_task_stride", ctypes.c_int64),
+        ("factors", ctypes.c_void_p),
+        ("factors_task_stride", ctypes.c_int64),
+        ("labels", ctypes.c_void_p),
+        ("labels_task_stride", ctypes.c_int64),
+        ("counts", ctypes.c_void_p),
+        ("score_thr", ctypes.c_float),
+        ("iou_thr", ctypes.c_float),
+        ("max_num", ctypes.c_uint32),
+        ("key_capacity", ctypes.c_uint32),
+        ("dets", ctypes.c_void_p),
+        ("out_labels", ctypes.c_void_p),
+        ("out_index", ctypes.c_void_p),
+        ("n_out", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
 def _parse_header():
     """Opcode / dtype / error constants straight from the C header, so that the
     Python side can never drift from the ABI."""
@@ -144,6 +173,9 @@ _sig("fx_compact_rows_static", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), cty
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, _vp)
 _sig("fx_async_error", _i, _i)
 _fp = ctypes.c_void_p
+_sig("fx_sort_nms", ctypes.c_int, ctypes.POINTER(FxNmsDesc), ctypes.c_void_p)
+_sig("fx_sort_nms_workspace_bytes", ctypes.c_size_t, ctypes.c_int, ctypes.c_uint32)
+_sig("fx_sort_nms_workspace_clear_bytes", ctypes.c_size_t, ctypes.c_int)
 _sig("fx_lstm_stack_fits", ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int)
 _sig("fx_lstm_stack_workspace_bytes", ctypes.c_size_t, _i, _i, _i)
 _sig("fx_lstm_stack_workspace_clear_bytes", ctypes.c_size_t)

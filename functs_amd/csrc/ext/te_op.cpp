@@ -303,6 +303,14 @@ c10::ScalarType atDtype(int d) {
     TORCH_CHECK(rc__ >= 0, "fxhip: ", fx_last_error(), " (", #expr, ")"); \
   } while (0)
 
+// what earlier launches reported through the library's error word (include/fxhip.h fx_async_error)
+int checkAsyncError() {
+  const int e = fx_async_error(1);
+  TORCH_CHECK(e != FX_ASYNC_INT64, "tssa::ParallelFunctor: an earlier fused region read an int64 element outside 32 bits "
+              "into integer arithmetic; its results are not valid (moves of int64 data are exact, arithmetic is 32-bit)");
+  return e;
+}
+
 // device scratch and the pinned landing zone of the kept-row counts; a call
 // borrows one and hands it back, so concurrent calls never share
 struct Workspace {
@@ -542,9 +550,7 @@ class RegionRunner {
       ws = var->take(fx_plan_scratch_bytes(plan), degree, device, (void*)stream.stream());
       ws.stream = (void*)stream.stream();
     }
-    // checked int64 loads of an earlier launch (integer arithmetic in regions is 32-bit)
-    TORCH_CHECK(!fx_async_error(1), "tssa::ParallelFunctor: an earlier fused region read an int64 element outside 32 bits "
-                "into integer arithmetic; its results are not valid (moves of int64 data are exact, arithmetic is 32-bit)");
+    checkAsyncError();
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
@@ -944,10 +950,9 @@ void runLstmStack(Stack& stack) {
   at::Tensor sc = result(c0, Lc, runs && Lc == L);
   if (T > 0 && L == 0) out.narrow(0, 0, T).copy_(x.narrow(0, 0, T));   // no layer: out[t] = x[t]
   if (runs) {
-    const int e = fx_async_error(1);
-    if (e != 0) lstmWorkspaces().reset();   // a given-up barrier wait leaves its words as they were
-    TORCH_CHECK(e == 0, "an earlier launch reported an error (", e, e == 2 ? ": a barrier wait of fx_lstm_stack was given up"
-                : ": int64 element outside 32 bits in integer arithmetic", "); its results are not valid");
+    const int e = checkAsyncError();
+    if (e == FX_ASYNC_BARRIER) lstmWorkspaces().reset();   // a given-up barrier wait leaves its words as they were
+    TORCH_CHECK(e != FX_ASYNC_BARRIER, "fx::lstm_stack: a barrier wait of an earlier launch was given up; its results are not valid");
     TORCH_CHECK(T <= INT32_MAX && B <= INT32_MAX && H <= INT32_MAX, "fx::lstm_stack: sizes beyond 32 bits");
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index());
     const size_t ws_bytes = fx_lstm_stack_workspace_bytes((int)B, (int)H, (int)L);

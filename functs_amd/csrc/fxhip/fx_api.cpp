@@ -37,6 +37,9 @@ uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled);
 bool fx_spec_has_stream(const FxSpecKernels* spec);
 #include "fx_lstm_sched.h"
 int fx_launch_lstm_stack(const FxLstmArgs& a, int L, hipStream_t stream);
+int fx_launch_sort_nms(const fx_nms_desc& d, uint32_t key_cap, void* workspace, uint32_t* err_host, hipStream_t stream);
+size_t fx_nms_workspace_bytes(int n_tasks, uint32_t key_cap);
+size_t fx_nms_workspace_clear_bytes(int n_tasks);
 hipError_t fx_launch_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* cols, void* const* outs,
                                          const int32_t* rowlen, const int32_t* elsize, int n_cols,
                                          uint32_t* total_host, hipStream_t stream);
@@ -413,7 +416,7 @@ int fx_async_error(int clear) {
     g_err_plain = 0;
     if (g_err_pinned) *(volatile uint32_t*)g_err_pinned = 0;
   }
-  return v != 0;
+  return (int)v;
 }
 
 // Fill the by-value dynamic block.  Exposed (without launching) so that host
@@ -896,6 +899,46 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
   return FX_OK;
 }
 void fx_set_lstm_spin_limit(uint32_t polls) { g_lstm_spin.store(polls, std::memory_order_relaxed); }
+
+// ---- detection tail (fx_nms.hip) ----
+
+static uint32_t nms_key_cap(uint32_t want) {
+  uint32_t cap = 128;
+  while (cap < want) cap <<= 1;
+  return cap;
+}
+size_t fx_sort_nms_workspace_bytes(int n_tasks, uint32_t key_capacity) {
+  if (n_tasks < 1 || key_capacity < 1 || key_capacity > FX_NMS_MAX_CANDIDATES) return 0;
+  return fx_nms_workspace_bytes(n_tasks, nms_key_cap(key_capacity));
+}
+size_t fx_sort_nms_workspace_clear_bytes(int n_tasks) { return n_tasks < 1 ? 0 : fx_nms_workspace_clear_bytes(n_tasks); }
+
+int fx_sort_nms(const fx_nms_desc* desc, void* stream_) {
+  if (!desc) return fail(FX_E_INVALID, "fx_sort_nms: null descriptor");
+  fx_nms_desc d = *desc;
+  if (d.mode != 0 && d.mode != 1) return fail(FX_E_INVALID, "fx_sort_nms: mode must be 0 or 1");
+  if (d.n_tasks < 0) return fail(FX_E_INVALID, "fx_sort_nms: negative task count");
+  if (!d.boxes || !d.scores || !d.dets || !d.out_labels || !d.n_out) return fail(FX_E_INVALID, "fx_sort_nms: null argument");
+  if (((uintptr_t)d.boxes & 15u) != 0 || (d.boxes_task_stride & 3) != 0)
+    return fail(FX_E_INVALID, "fx_sort_nms: boxes must be 16-byte aligned and their task stride a multiple of 4");
+  if (d.max_num < 1 || d.max_num > FX_NMS_MAX_OUT)
+    return fail(FX_E_LIMIT, "fx_sort_nms: max_num must be 1.." + std::to_string(FX_NMS_MAX_OUT));
+  if (d.mode == 1 && d.n_classes < 1) return fail(FX_E_INVALID, "fx_sort_nms: n_classes must be positive in mode 1");
+  const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? d.n_classes : 1u);
+  if (items >= (1ull << 31)) return fail(FX_E_LIMIT, "fx_sort_nms: rows * classes beyond 31 bits");
+  if (d.key_capacity < 1 || d.key_capacity > FX_NMS_MAX_CANDIDATES)
+    return fail(FX_E_LIMIT, "fx_sort_nms: key_capacity must be 1.." + std::to_string(FX_NMS_MAX_CANDIDATES) +
+                                " (the reference's own single-pass branch ends at 10000 candidates)");
+  if (d.n_tasks == 0) return FX_OK;
+  const uint32_t cap = nms_key_cap(d.key_capacity);
+  if (!d.workspace || ((uintptr_t)d.workspace & 255u) != 0 || d.workspace_bytes < fx_nms_workspace_bytes(d.n_tasks, cap))
+    return fail(FX_E_INVALID, "fx_sort_nms: workspace must be 256-byte aligned and hold fx_sort_nms_workspace_bytes()");
+  const int rc = fx_launch_sort_nms(d, cap, d.workspace, err_word(true), (hipStream_t)stream_);
+  if (rc != 0) return fail(FX_E_HIP, std::string("fx_sort_nms: ") + hipGetErrorString((hipError_t)(rc - 100)));
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  g_spec_launches.fetch_add(1, std::memory_order_relaxed);
+  return FX_OK;
+}
 
 int fx_copy_bytes(const void* src, void* dst, size_t bytes, void* stream) {
   if (bytes % 16) return fail(FX_E_INVALID, "fx_copy_bytes: size must be a multiple of 16");

@@ -308,14 +308,30 @@ class BoundCall:
         self.device = dev
         T = region.degree
         self.outs = []
+        self._batched = []
         ptrs = (ctypes.c_void_p * max(plan.n_out * T, 1))()
         for o in range(plan.n_out):
             row = []
-            for t in range(T):
-                dt, shape = plan.out_meta[o][t]
-                ten = torch.empty(shape, dtype=dt, device=dev)
+            metas = [plan.out_meta[o][t] for t in range(T)]
+            if T > 1 and all(m == metas[0] for m in metas):
+                # one allocation per output, the tasks' tensors at equal, 256-byte aligned distances
+                # (what tssa::ParallelFunctor does as well): `batched` hands it on as [T, ...]
+                dt, shape = metas[0]
+                numel = 1
+                for d in shape:
+                    numel *= d
+                per = 256 // torch.empty(0, dtype=dt).element_size()
+                stride = max(-(-numel // per) * per, per)
+                buf = torch.empty(T * stride, dtype=dt, device=dev)
+                inner = torch.empty(shape, dtype=dt, device="meta").stride()
+                whole = buf.as_strided((T,) + tuple(shape), (stride,) + tuple(inner))
+                self._batched.append(whole)
+                row = [whole[t] for t in range(T)]
+            else:
+                self._batched.append(None)
+                row = [torch.empty(shape, dtype=dt, device=dev) for dt, shape in metas]
+            for t, ten in enumerate(row):
                 ptrs[o * T + t] = ten.data_ptr()
-                row.append(ten)
             self.outs.append(row)
         self.ptrs = ptrs
         self.scratch = torch.empty(max(plan.scratch_bytes, 1), dtype=torch.uint8, device=dev) if plan.compact else None
@@ -346,6 +362,15 @@ class BoundCall:
                                               self.totals.data_ptr() if self.totals is not None else None,
                                               ctypes.c_void_p(stream), int(repeat), ms, 4, ctypes.byref(nk)))
         return [ms[i] for i in range(nk.value)]
+
+    def batched(self, o):
+        """Output `o` of a map whose tasks all have the same shape as one tensor [T, ...] over the
+        tasks' buffers (dimension 0 strided), rows past a task's kept-row count unspecified; the
+        counts are `totals` (pinned host memory, written by the kernels).  A consumer on the same
+        stream that reads the counts from memory needs no synchronisation with the host."""
+        if self._batched[o] is None:
+            raise _lib.FxError(C["FX_E_INVALID"], "output %d is not one buffer (tasks of different shapes)" % o)
+        return self._batched[o]
 
     def results(self):
         """Outputs as the operator returns them: a tensor per output, or a list

@@ -264,11 +264,15 @@ size_t fx_dyn_bytes(void);
  * Integer ARITHMETIC is 32-bit: an int64 tensor element that enters it (a + 3, a == b, a as an
  * index) must fit 32 bits (a conversion to float uses the whole element and is exact).  The
  * loads check that; an element that does not fit sets a sticky process-wide error word, and
- * the outputs of that launch are not to be used.  fx_async_error returns 1 if it is set (after
- * the stream has been synchronised it covers every launch before that) and clears it when
- * `clear` is non-zero.  Integer constants and scalar arguments outside 32 bits are refused when
+ * the outputs of that launch are not to be used.  fx_async_error returns 0 or what the word
+ * holds (after the stream has been synchronised it covers every launch before that) and clears it
+ * when `clear` is non-zero: FX_ASYNC_INT64 from these loads, FX_ASYNC_BARRIER from a barrier wait
+ * that fx_lstm_stack gave up, FX_ASYNC_NMS_CAPACITY from fx_sort_nms (the latest report wins).  Integer constants and scalar arguments outside 32 bits are refused when
  * the region is planned / run (FX_E_UNSUPPORTED / FX_E_LIMIT).  The reference computes in int64
  * throughout (NNC kLong, functs/csrc/jit/ir/symbol_ext.cpp:17-117 for the eager bodies). */
+#define FX_ASYNC_INT64 1
+#define FX_ASYNC_BARRIER 2
+#define FX_ASYNC_NMS_CAPACITY 3
 int fx_async_error(int clear);
 
 /* ---- stand-alone order-preserving row compaction (x[mask] for several x) ----
@@ -322,6 +326,64 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
                   const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
                   int layers, void* workspace, size_t workspace_bytes, void* stream);
 void fx_set_lstm_spin_limit(uint32_t polls); /* barrier polls before a wait is given up (default 1000000; tests) */
+
+/* ---- detection tail: score threshold + sort + class-aware greedy NMS + top-k, one launch ----
+ * The step behind row compaction in the reference's detection programs, which it runs as ATen /
+ * torchvision kernels with host synchronisations in between:
+ *   mode 1  multiclass_nms (functs/benchmark/ai_model/yolov3/yolov3_bbox.py:104-138 with batched_nms
+ *           :141-171 and nms_wrapper :174-179): scores is cls [rows, n_classes], a candidate
+ *           (row, class) needs cls > score_thr, its score is cls * factors[row], its label the class;
+ *   mode 0  batched_nms alone (ssd_bbox.py:175-214): scores [rows], labels [rows] (null: one class),
+ *           a candidate needs score > score_thr (pass -INFINITY to take every row).
+ * Per task (image): candidates in order of descending score (equal scores by ascending index),
+ * a candidate is dropped when a kept one of the same class overlaps it with IoU > iou_thr
+ * (classes are told apart as the reference does: boxes moved by label * (largest candidate
+ * coordinate + 1)), the first max_num kept ones are returned.  IoU in float32 as torchvision's CPU
+ * kernel computes it: inter / ((area_i + area_j) - inter).
+ * Outputs have fixed shapes; rows from n_out[task] on are zero.  out_index is the candidate's
+ * position in the input (mode 0: row, mode 1: row * n_classes + class).
+ * `counts` (valid rows per task) and `n_out` may be device memory or pinned host memory: a count
+ * that a compaction wrote is read by the kernel, not by the host.
+ * Limits: at most FX_NMS_MAX_CANDIDATES candidates per task - `key_capacity` says how many the
+ * launch is sized for (rounded up to a power of two >= 128); a task with more returns zeros, sets
+ * its n_out to FX_NMS_OVERFLOW and reports FX_ASYNC_NMS_CAPACITY through fx_async_error - and
+ * max_num <= FX_NMS_MAX_OUT.  boxes must be 16-byte
+ * aligned, boxes_task_stride a multiple of 4.  Task strides are in elements. */
+#define FX_NMS_MAX_CANDIDATES 16384
+#define FX_NMS_MAX_OUT 1024
+#define FX_NMS_OVERFLOW 0xffffffffu
+typedef struct fx_nms_desc {
+  int32_t mode;
+  int32_t n_tasks;
+  uint32_t rows;        /* rows per task (at most; see counts) */
+  uint32_t n_classes;   /* mode 1 */
+  const float* boxes;   /* [rows, 4] per task, x1 y1 x2 y2 */
+  int64_t boxes_task_stride;
+  const float* scores;
+  int64_t scores_task_stride;
+  const float* factors; /* mode 1, [rows] per task; null: 1 */
+  int64_t factors_task_stride;
+  const int64_t* labels; /* mode 0, [rows] per task; null: one class */
+  int64_t labels_task_stride;
+  const uint32_t* counts; /* [n_tasks] valid rows per task; null: rows */
+  float score_thr;
+  float iou_thr;
+  uint32_t max_num;
+  uint32_t key_capacity;
+  float* dets;           /* [n_tasks, max_num, 5]: x1 y1 x2 y2 score */
+  int64_t* out_labels;   /* [n_tasks, max_num] */
+  int64_t* out_index;    /* [n_tasks, max_num] or null */
+  uint32_t* n_out;       /* [n_tasks] */
+  void* workspace;       /* fx_sort_nms_workspace_bytes() of device memory, 256-byte aligned */
+  size_t workspace_bytes;
+} fx_nms_desc;
+/* workspace: the first fx_sort_nms_workspace_clear_bytes() bytes are zero when a launch starts; every
+ * launch leaves them zero, so one workspace, cleared once, serves launch after launch on one stream
+ * as long as n_tasks and key_capacity stay the same (they fix where the counters lie; launches
+ * that share a workspace must not overlap). */
+size_t fx_sort_nms_workspace_bytes(int n_tasks, uint32_t key_capacity);
+size_t fx_sort_nms_workspace_clear_bytes(int n_tasks);
+int fx_sort_nms(const fx_nms_desc* desc, void* stream);
 
 /* ---- device utilities ---- */
 int fx_device_count(void);

@@ -1,0 +1,214 @@
+// CanonicalizeOps and HoistLoopInvariants: the two clean-up passes in front of region formation.
+//
+// CanonicalizeOps (fait/passes/canonicalize.cpp:148-157) brings spellings that mean the same to the
+// one spelling the later passes know:
+//   arange(end)                    -> arange(0, end)
+//   max.other / min.other          -> maximum / minimum
+//   new_zeros / new_ones(self, ..) -> zeros / ones with self's dtype and device
+//   pow(x, n), n a constant int >= 1 -> products (square and multiply)
+//   slice / immut::slice without start and end, step 1 -> the tensor itself
+//   t() of a matrix                -> transpose(0, 1)
+//   to.dtype / to.other            -> to(device, dtype)
+//   view                           -> reshape
+// Two rewrites of the reference are narrowed on purpose: its slice rule drops the operator
+// whatever the step is (canonicalize.cpp:72-80: x[::2] would become x), and its pow rule yields
+// x * x for every odd exponent above one (canonicalize.cpp:51-70: the first set bit is skipped
+// while `base` is still unset); here the step must be 1 and pow(x, n) is x multiplied n times.
+//
+// HoistLoopInvariants (fait/passes/licm.cpp:55-66, called first thing by ParallelizeLoops,
+// parallelize_loops.cpp:128-131): scalar-valued pure nodes of a loop or map body whose operands
+// are all defined outside move in front of the loop, innermost loops first, so that trip counts
+// and sizes stop looking like per-iteration values.
+#include <torch/csrc/jit/ir/constants.h>
+
+#include <unordered_set>
+
+#include "passes.h"
+#include "symbols.h"
+
+namespace functs {
+using namespace torch::jit;
+
+namespace {
+
+bool isTensorValue(const Value* v) { return v->type()->kind() == c10::TypeKind::TensorType; }
+bool isNone(Value* v) { return v->mustBeNone(); }
+std::optional<int64_t> constInt(Value* v) {
+  auto c = toIValue(v);
+  if (c && c->isInt()) return c->toInt();
+  return std::nullopt;
+}
+
+// a node of kind `k` at the insertion point (operands in schema order, keyword-only ones included)
+Value* make(Graph* g, Symbol k, at::ArrayRef<Value*> inputs, c10::TypePtr type = c10::TensorType::get()) {
+  Node* n = g->create(k, inputs, 1);
+  g->insertNode(n);
+  n->output()->setType(std::move(type));
+  return n->output();
+}
+
+// dtype / device of `self` as values: constants when the type says so, prim::dtype / prim::device otherwise
+Value* dtypeOf(Graph* g, Value* self) {
+  auto tt = self->type()->cast<c10::TensorType>();
+  if (tt && tt->scalarType()) return g->insertConstant((int64_t)*tt->scalarType());
+  return make(g, c10::prim::dtype, {self}, c10::IntType::get());
+}
+Value* deviceOf(Graph* g, Value* self) { return make(g, c10::prim::device, {self}, c10::DeviceObjType::get()); }
+
+// returns true when `n` was replaced (and destroyed)
+bool rewrite(Node* n) {
+  Graph* g = n->owningGraph();
+  const Symbol k = n->kind();
+  const size_t ni = n->inputs().size();
+  WithInsertPoint at(n);
+  auto replaceWith = [&](Value* v) {
+    v->node()->setSourceRange(n->sourceRange());
+    v->setType(n->output(0)->type());   // what was known about the result stays known
+    n->output(0)->replaceAllUsesWith(v);
+    n->destroy();
+    return true;
+  };
+  if (k == c10::aten::arange && ni == 5 && !isTensorValue(n->input(0))) {   // arange(end, dtype, layout, device, pin_memory)
+    Value* zero = g->insertConstant((int64_t)0);
+    return replaceWith(make(g, c10::aten::arange, {zero, n->input(0), n->input(1), n->input(2), n->input(3), n->input(4)}));
+  }
+  if ((k == c10::aten::max || k == c10::aten::min) && ni == 2 && n->outputs().size() == 1 && isTensorValue(n->input(0)) &&
+      isTensorValue(n->input(1))) {
+    return replaceWith(make(g, k == c10::aten::max ? c10::aten::maximum : c10::aten::minimum, {n->input(0), n->input(1)}));
+  }
+  if ((k == c10::aten::new_zeros || k == c10::aten::new_ones) && ni == 6) {   // (self, size, dtype, layout, device, pin_memory)
+    Value* self = n->input(0);
+    Value* dtype = isNone(n->input(2)) ? dtypeOf(g, self) : n->input(2);
+    Value* device = isNone(n->input(4)) ? deviceOf(g, self) : n->input(4);
+    Value* none = g->insertConstant(c10::IValue());
+    return replaceWith(make(g, k == c10::aten::new_zeros ? c10::aten::zeros : c10::aten::ones,
+                                 {n->input(1), dtype, none, device, none}));
+  }
+  if (k == c10::aten::pow && ni == 2 && isTensorValue(n->input(0))) {
+    auto e = constInt(n->input(1));
+    if (!e || *e < 1 || *e > 64) return false;
+    // square and multiply: result = product of the squares that the set bits of e select
+    Value* sq = n->input(0);
+    Value* acc = nullptr;
+    for (int64_t left = *e; left > 0; left >>= 1) {
+      if (left & 1) acc = acc ? make(g, c10::aten::mul, {acc, sq}) : sq;
+      if (left > 1) sq = make(g, c10::aten::mul, {sq, sq});
+    }
+    if (acc == n->input(0)) return false;   // e == 1: pow(x, 1) keeps its own node (a copy, not an alias)
+    return replaceWith(acc);
+  }
+  if ((k == c10::aten::slice || k == sym::Slice()) && ni == 5 && isNone(n->input(2)) && isNone(n->input(3)) &&
+      constInt(n->input(4)) == std::optional<int64_t>(1)) {
+    // the graph is functionalized: nothing writes through the view that aten::slice returns
+    n->output(0)->replaceAllUsesWith(n->input(0));
+    n->destroy();
+    return true;
+  }
+  if (k == c10::aten::t && ni == 1) {
+    auto tt = n->input(0)->type()->cast<c10::TensorType>();
+    if (!tt || !tt->dim() || *tt->dim() != 2) return false;   // t() of a vector is the vector
+    Value* zero = g->insertConstant((int64_t)0);
+    Value* one = g->insertConstant((int64_t)1);
+    Value* tr = make(g, c10::aten::transpose, {n->input(0), zero, one});
+    tr->node()->setSourceRange(n->sourceRange());
+    tr->setType(tt->dimensionedOnly());   // still a matrix of that element type: a t() of it is rewritten as well
+    n->output(0)->replaceAllUsesWith(tr);
+    n->destroy();
+    return true;
+  }
+  if (k == c10::aten::to && isTensorValue(n->input(0))) {
+    Value* self = n->input(0);
+    Value* f = g->insertConstant(false);
+    Value* none = g->insertConstant(c10::IValue());
+    // to.dtype(self, dtype, non_blocking, copy, memory_format)
+    if (ni == 5 && n->input(1)->type()->kind() == c10::TypeKind::IntType)
+      return replaceWith(make(g, c10::aten::to, {self, deviceOf(g, self), n->input(1), f, f, none}));
+    // to.other(self, other, non_blocking, copy, memory_format)
+    if (ni == 5 && isTensorValue(n->input(1)))
+      return replaceWith(make(g, c10::aten::to, {self, deviceOf(g, n->input(1)), dtypeOf(g, n->input(1)), f, f, none}));
+    return false;
+  }
+  if (k == c10::aten::view && ni == 2 && n->input(1)->type()->cast<c10::ListType>()) {
+    return replaceWith(make(g, c10::aten::reshape, {n->input(0), n->input(1)}));
+  }
+  return false;
+}
+
+void canonicalizeIn(Block* b) {
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) canonicalizeIn(inner);
+    rewrite(n);
+  }
+}
+
+// ---------------------------------------------------------------------------
+bool scalarLike(const c10::TypePtr& t) {
+  switch (t->kind()) {
+    case c10::TypeKind::IntType:
+    case c10::TypeKind::FloatType:
+    case c10::TypeKind::BoolType:
+    case c10::TypeKind::DeviceObjType:
+    case c10::TypeKind::NoneType:
+      return true;
+    case c10::TypeKind::TupleType:
+      for (const auto& e : t->containedTypes())
+        if (!scalarLike(e)) return false;
+      return true;
+    default:
+      return false;   // tensors stay (licm.cpp:25-27); lists can be appended to
+  }
+}
+
+bool definedOutside(Value* v, Block* body) {
+  for (Block* b = v->node()->owningBlock(); b; b = b->owningNode() ? b->owningNode()->owningBlock() : nullptr)
+    if (b == body) return false;
+  return true;
+}
+
+// operators without side effects that cannot fail for operands that are valid outside the loop
+const std::unordered_set<Symbol>& hoistable() {
+  using namespace c10;
+  static const std::unordered_set<Symbol> s{
+      aten::size, aten::dim, aten::add, aten::sub, aten::mul, aten::neg, aten::eq, aten::ne, aten::lt, aten::le,
+      aten::gt, aten::ge, aten::__range_length, aten::__derive_index, aten::__not__, aten::__and__, aten::__or__, aten::Int,
+      aten::Float, aten::Bool, aten::min, aten::max, prim::device, prim::dtype, prim::TupleConstruct, prim::TupleIndex,
+      prim::TupleUnpack, prim::min, prim::max};
+  return s;
+}
+
+bool invariant(Node* n, Block* body) {
+  if (n->outputs().empty() || !n->blocks().empty() || n->hasSideEffects()) return false;
+  if (!hoistable().count(n->kind())) return false;
+  for (Value* o : n->outputs())
+    if (!scalarLike(o->type())) return false;
+  for (Value* in : n->inputs())
+    if (!definedOutside(in, body)) return false;
+  return true;
+}
+
+bool hoistIn(Block* b) {
+  bool changed = false;
+  for (Node* n : b->nodes()) {
+    for (Block* inner : n->blocks()) changed = hoistIn(inner) || changed;   // innermost loops first
+    if (n->kind() != c10::prim::Loop && n->kind() != sym::ParallelMap()) continue;
+    Block* body = n->blocks()[0];
+    for (auto it = body->nodes().begin(); it != body->nodes().end();) {
+      Node* m = *it;
+      ++it;
+      if (m->kind() == c10::prim::Constant || !invariant(m, body)) continue;
+      m->moveBefore(n);   // what it produced inside an inner loop has already arrived here, so one walk suffices
+      changed = true;
+    }
+  }
+  return changed;
+}
+
+}  // namespace
+
+void CanonicalizeOps(std::shared_ptr<Graph> graph) { canonicalizeIn(graph->block()); }
+
+bool HoistLoopInvariants(std::shared_ptr<Graph> graph) { return hoistIn(graph->block()); }
+
+}  // namespace functs

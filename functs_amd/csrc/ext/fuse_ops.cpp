@@ -86,6 +86,11 @@ bool isFusableNode(Node* node) {
   }
   if (!fusableSymbols().count(node->kind())) return false;
   if (node->kind() != sym::ForallSelectRev() && !node->blocks().empty()) return false;
+  // a region is compiled for one element type: a dtype operand that is computed at run time
+  // (prim::dtype of a tensor whose type is not known) keeps its operator outside
+  if (node->maybeSchema())
+    for (size_t i = 0; i < node->inputs().size() && i < node->schema().arguments().size(); ++i)
+      if (node->schema().arguments()[i].name() == "dtype" && node->input(i)->node()->kind() != c10::prim::Constant) return false;
   // scalar arithmetic that shares a symbol with a tensor operator stays outside
   if (node->kind() == c10::aten::add || node->kind() == c10::aten::sub || node->kind() == c10::aten::mul ||
       node->kind() == c10::aten::neg || node->kind() == c10::aten::eq || node->kind() == c10::aten::ne ||
@@ -873,6 +878,9 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   ConstantPropagation(graph);
   EliminateCommonSubexpression(graph);
   EliminateDeadCode(graph);
+  CanonicalizeOps(graph);       // fait_pipeline.cpp:39
+  HoistLoopInvariants(graph);   // parallelize_loops.cpp:130
+  EliminateCommonSubexpression(graph);
   if (CollapseRecurrentLoops(graph)) EliminateDeadCode(graph);   // buffers the collapsed node no longer reads
   CollapseAssignLoops(graph);
   ParallelizeLoops(graph);

@@ -29,6 +29,8 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_fait_fuse_ops", FuseOps);
   m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
   m.def("_jit_pass_collapse_recurrent_loops", CollapseRecurrentLoops);
+  m.def("_jit_pass_canonicalize_ops", CanonicalizeOps);
+  m.def("_jit_pass_hoist_loop_invariants", HoistLoopInvariants);
   m.def("_jit_pass_parallelize_loops", ParallelizeLoops);
   m.def("_jit_pass_split_parallel_maps", SplitParallelMaps);
   m.def("_jit_pass_unroll_loops_with_deps", UnrollLoopsWithDeps);

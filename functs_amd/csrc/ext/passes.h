@@ -26,6 +26,14 @@ void CollapseAssignLoops(std::shared_ptr<torch::jit::Graph> graph);
 // persistent kernel; true if the graph changed.
 bool CollapseRecurrentLoops(std::shared_ptr<torch::jit::Graph> graph);
 
+// fait/passes/canonicalize.cpp:148-157 (on a functionalized graph): one spelling per meaning
+// (arange(end), max.other, new_zeros, pow with a constant exponent, empty slices, t(), to.dtype /
+// to.other, view).
+void CanonicalizeOps(std::shared_ptr<torch::jit::Graph> graph);
+// fait/passes/licm.cpp:55-66: scalar-valued pure nodes of loop and map bodies whose operands are
+// defined outside move in front of the loop; true if the graph changed.
+bool HoistLoopInvariants(std::shared_ptr<torch::jit::Graph> graph);
+
 // fait/passes/parallelize_loops.cpp:12-145: loops without carried values whose
 // list reads are list[i] and whose list writes are one append per list become
 // prim::ParallelMap(len, lists...){block(i, elems...) -> rets}.

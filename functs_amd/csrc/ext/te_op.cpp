@@ -647,7 +647,8 @@ struct Translator {
   // dtype argument (ScalarType constant or None) -> fx dtype or -1
   int dtypeArg(const Value* v) {
     auto iv = toIValue(v);
-    if (!iv || iv->isNone()) return -1;
+    TORCH_CHECK(iv, "ParallelFunctor: a dtype operand inside a fused region must be a constant");
+    if (iv->isNone()) return -1;
     return fxDtype(static_cast<c10::ScalarType>(iv->toInt()));
   }
 

@@ -483,6 +483,54 @@ def main():
                 "bound": "one workgroup per image: the candidate scan reads the image's class scores once; "
                          "sort and the greedy walk run in LDS"}
 
+    def run_rows():
+        """The stand-alone row compaction of the C ABI (fx_compact_rows: count, scan, scatter) on
+        700 000 rows of 16 float32 with half of them kept, next to the library's plain copy kernel
+        on the same number of bytes."""
+        import ctypes
+        from functs_amd import _lib
+        n, w = 700000, 16
+        g = torch.Generator().manual_seed(0)
+        mask = (torch.rand(n, generator=g) < 0.5).to(dev)
+        col = torch.rand(n, w, generator=g).to(dev)
+        out = torch.empty_like(col)
+        m8 = mask.view(torch.uint8)
+        src, dst = (ctypes.c_void_p * 1)(col.data_ptr()), (ctypes.c_void_p * 1)(out.data_ptr())
+        rowlen, elsize = (ctypes.c_int32 * 1)(w), (ctypes.c_int32 * 1)(4)
+        sb = _lib.lib.fx_compact_rows_scratch_bytes(n)
+        scratch = torch.empty(sb, dtype=torch.uint8, device=dev)
+        total = torch.zeros(1, dtype=torch.int32).pin_memory()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+        def call():
+            _lib.check(_lib.lib.fx_compact_rows(m8.data_ptr(), n, src, dst, rowlen, elsize, 1, scratch.data_ptr(), sb,
+                                                total.data_ptr(), stream))
+
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        kept = int(total[0])
+        reps = max(args.steps // 5, 5)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        moved = 2 * n + n * w * 4 + kept * w * 4    # mask twice (count, scatter), rows in, kept rows out
+        a, b = torch.empty(moved // 2 // 16 * 16, dtype=torch.uint8, device=dev), torch.empty(moved // 2 // 16 * 16, dtype=torch.uint8, device=dev)
+        _lib.copy_bytes(a, b)
+        e0.record()
+        for _ in range(reps):
+            _lib.copy_bytes(a, b)
+        e1.record()
+        torch.cuda.synchronize()
+        copy_us = e0.elapsed_time(e1) * 1e3 / reps
+        return {"workload": "fx_compact_rows, 700000 rows x 16 float32, half kept (warm)", "launches_per_call": 3,
+                "call_us": round(us, 1), "bytes_moved": moved, "gbps": round(moved / (us * 1e-6) / 1e9, 1),
+                "copy_kernel_same_bytes_us": round(copy_us, 1), "copy_kernel_gbps": round(2 * a.numel() / (copy_us * 1e-6) / 1e9, 1)}
+
     def run_stream():
         """Not one of the five configurations: one big fused elementwise region (sigmoid(2x + 1) on
         [8192, 4096] fp32), the shape on which the dense kernel itself meets the HBM roofline."""
@@ -528,6 +576,10 @@ def main():
             per["c4"] = run_c4()
         except Exception as e:
             per["c4"] = {"error": str(e)[:200]}
+        try:
+            per["standalone_compact_rows"] = run_rows()
+        except Exception as e:
+            per["standalone_compact_rows"] = {"error": str(e)[:200]}
         try:
             per["c5_nms_tail"] = run_tail()
         except Exception as e:

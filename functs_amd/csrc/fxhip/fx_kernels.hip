@@ -44,6 +44,8 @@ struct FxCols {
   void* dst[8];
   int32_t words[8];   // 4-byte words per row (elsize 4/8) or bytes per row (elsize 1)
   int32_t bytes[8];   // 1 = byte column, 0 = word column
+  int32_t vec[8];     // word column whose rows are whole 16-byte groups at 16-byte aligned addresses
+  uint32_t magic[8], shift[8];   // division by the units of a row (groups when vec, else words / bytes)
   int32_t n;
 };
 
@@ -137,18 +139,44 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rows_scatter(const uint8_t* __res
     if (c >= cols.n) break;
     const uint32_t w = (uint32_t)cols.words[c];
     const uint32_t n_el = n_kept * w;
+    const uint32_t magic = cols.magic[c], shift = cols.shift[c];
     if (cols.bytes[c]) {
       const FX_AS1 uint8_t* src = (const FX_AS1 uint8_t*)cols.src[c];
       FX_AS1 uint8_t* dst = (FX_AS1 uint8_t*)cols.dst[c] + (size_t)prefix * w;
       for (uint32_t e = threadIdx.x; e < n_el; e += FX_BLOCK) {
-        const uint32_t r = e / w, k = e - r * w;
+        const uint32_t r = fx_fastdiv(e, magic, shift), k = e - r * w;
         dst[e] = src[(size_t)s_rowmap[r] * w + k];
       }
+    } else if (cols.vec[c]) {
+      // a lane moves one 16-byte group; four groups per lane are in flight
+      const uint32_t g = w >> 2, n_g = n_kept * g;
+      const FX_AS1 fx_u32x4* src = (const FX_AS1 fx_u32x4*)cols.src[c];
+      FX_AS1 fx_u32x4* dst = (FX_AS1 fx_u32x4*)cols.dst[c] + (size_t)prefix * g;
+      for (uint32_t e0 = threadIdx.x; e0 < n_g; e0 += 4u * FX_BLOCK) {
+        fx_u32x4 v[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4u; ++u) {
+          const uint32_t e = e0 + u * FX_BLOCK;
+          if (e < n_g) {
+            const uint32_t r = fx_fastdiv(e, magic, shift), k = e - r * g;
+            v[u] = src[(size_t)s_rowmap[r] * g + k];
+          }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4u; ++u) {
+          const uint32_t e = e0 + u * FX_BLOCK;
+          if (e < n_g) dst[e] = v[u];
+        }
+      }
+    } else if (w == 1u) {
+      const FX_AS1 uint32_t* src = (const FX_AS1 uint32_t*)cols.src[c];
+      FX_AS1 uint32_t* dst = (FX_AS1 uint32_t*)cols.dst[c] + (size_t)prefix;
+      for (uint32_t e = threadIdx.x; e < n_kept; e += FX_BLOCK) dst[e] = src[s_rowmap[e]];
     } else {
       const FX_AS1 uint32_t* src = (const FX_AS1 uint32_t*)cols.src[c];
       FX_AS1 uint32_t* dst = (FX_AS1 uint32_t*)cols.dst[c] + (size_t)prefix * w;
       for (uint32_t e = threadIdx.x; e < n_el; e += FX_BLOCK) {
-        const uint32_t r = e / w, k = e - r * w;
+        const uint32_t r = fx_fastdiv(e, magic, shift), k = e - r * w;
         dst[e] = src[(size_t)s_rowmap[r] * w + k];
       }
     }
@@ -320,13 +348,17 @@ hipError_t fx_launch_compact_rows(const uint8_t* mask, int64_t n, const void* co
                                   const int32_t* rowlen, const int32_t* elsize, int n_cols, uint32_t* counts,
                                   uint32_t* total_host, hipStream_t stream) {
   FxCols c;
-  for (int i = 0; i < 8; ++i) { c.src[i] = nullptr; c.dst[i] = nullptr; c.words[i] = 0; c.bytes[i] = 0; }
+  for (int i = 0; i < 8; ++i) {
+    c.src[i] = nullptr; c.dst[i] = nullptr; c.words[i] = 0; c.bytes[i] = 0; c.vec[i] = 0; c.magic[i] = 0; c.shift[i] = 0;
+  }
   c.n = n_cols;
   for (int i = 0; i < n_cols; ++i) {
     c.src[i] = cols[i];
     c.dst[i] = outs[i];
     c.bytes[i] = elsize[i] == 1 ? 1 : 0;
     c.words[i] = elsize[i] == 1 ? rowlen[i] : rowlen[i] * (elsize[i] / 4);
+    c.vec[i] = !c.bytes[i] && c.words[i] >= 4 && (c.words[i] & 3) == 0 && (((uintptr_t)cols[i] | (uintptr_t)outs[i]) & 15u) == 0;
+    fx_fastdiv_make((uint32_t)std::max(c.vec[i] ? c.words[i] / 4 : c.words[i], 1), &c.magic[i], &c.shift[i]);
   }
   const uint32_t tiles = (uint32_t)((n + FX_BLOCK - 1) / FX_BLOCK);
   fx_rows_count<<<tiles, FX_BLOCK, 0, stream>>>(mask, (uint32_t)n, counts);

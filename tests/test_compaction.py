@@ -86,3 +86,22 @@ def test_standalone_compact_rows_edge_masks():
     for mask in (torch.zeros(1000, dtype=torch.bool), torch.ones(1000, dtype=torch.bool)):
         (got,) = compact_rows(mask.to(dev), [a.to(dev)])
         assert_exact(got.cpu(), a[mask])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [300, 70000])
+def test_standalone_compact_rows_row_shapes(n):
+    """Rows that are whole 16-byte groups (moved as such), rows that are not, single words,
+    64-bit elements, and a source that is not 16-byte aligned (moved word by word)."""
+    from functs_amd import compact_rows
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(n + 1)
+    mask = torch.rand(n, generator=g) < 0.6
+    cols = [torch.rand(n, 8, generator=g), torch.rand(n, 85, generator=g), torch.rand(n, generator=g),
+            torch.randint(0, 1 << 50, (n, 2), generator=g), torch.rand(n, 20, 4, generator=g),
+            torch.rand(n * 12 + 1, generator=g)[1:].view(n, 12)]
+    dev_cols = [c.to(dev) for c in cols[:-1]] + [torch.rand(n * 12 + 1, generator=g).to(dev)[1:].view(n, 12)]
+    cols[-1] = dev_cols[-1].cpu()
+    assert dev_cols[-1].data_ptr() % 16 == 4
+    got = compact_rows(mask.to(dev), dev_cols)
+    assert_exact([t.cpu() for t in got], [c[mask] for c in cols], "row shapes n=%d" % n)

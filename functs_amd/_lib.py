@@ -178,7 +178,6 @@ _sig("fx_sort_nms_workspace_bytes", ctypes.c_size_t, ctypes.c_int, ctypes.c_uint
 _sig("fx_sort_nms_workspace_clear_bytes", ctypes.c_size_t, ctypes.c_int)
 _sig("fx_lstm_stack_fits", ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int)
 _sig("fx_lstm_stack_workspace_bytes", ctypes.c_size_t, _i, _i, _i)
-_sig("fx_lstm_stack_workspace_clear_bytes", ctypes.c_size_t)
 _sig("fx_lstm_stack", _i, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp)
 _sig("fx_set_lstm_spin_limit", None, ctypes.c_uint32)
 _sig("fx_device_count", _i)

@@ -23,6 +23,7 @@
 #include <map>
 #include <mutex>
 #include <sstream>
+#include <tuple>
 
 #include "../../../include/fxhip.h"
 #include "passes.h"
@@ -870,17 +871,19 @@ void RegionRunner::build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue>
 }
 
 // --- fx::lstm_stack -----------------------------------------------------------
-// Barrier words and the h exchange buffer of the persistent kernel, one per (device, stream):
-// cleared when allocated, and every launch that ends without error leaves them clear
-// (include/fxhip.h fx_lstm_stack), so a call costs the one launch.
+// Control words and the h exchange buffer of the persistent kernel, one per (device, stream) and
+// shape (batch, hidden, layers): cleared when allocated, and every launch that ends without error
+// leaves them ready for the next one (include/fxhip.h fx_lstm_stack), so a call costs the one launch.
 struct LstmWorkspaces {
   std::mutex mu;
-  std::map<std::pair<int, void*>, at::Tensor> by_stream;
-  at::Tensor get(c10::Device dev, void* stream, size_t bytes) {
+  std::map<std::tuple<int, void*, int64_t, int64_t, int64_t>, at::Tensor> by_stream;
+  at::Tensor get(c10::Device dev, void* stream, int64_t B, int64_t H, int64_t L) {
     std::lock_guard<std::mutex> lock(mu);
-    at::Tensor& t = by_stream[{(int)dev.index(), stream}];
-    if (!t.defined() || (size_t)t.numel() < bytes)
+    at::Tensor& t = by_stream[{(int)dev.index(), stream, B, H, L}];
+    if (!t.defined()) {
+      const size_t bytes = fx_lstm_stack_workspace_bytes((int)B, (int)H, (int)L);
       t = at::zeros({(int64_t)bytes}, at::TensorOptions().dtype(at::kByte).device(dev));   // on the current stream
+    }
     return t;
   }
   void reset() {
@@ -952,12 +955,11 @@ void runLstmStack(Stack& stack) {
   if (T > 0 && L == 0) out.narrow(0, 0, T).copy_(x.narrow(0, 0, T));   // no layer: out[t] = x[t]
   if (runs) {
     const int e = checkAsyncError();
-    if (e == FX_ASYNC_BARRIER) lstmWorkspaces().reset();   // a given-up barrier wait leaves its words as they were
-    TORCH_CHECK(e != FX_ASYNC_BARRIER, "fx::lstm_stack: a barrier wait of an earlier launch was given up; its results are not valid");
+    if (e == FX_ASYNC_BARRIER) lstmWorkspaces().reset();   // a given-up wait leaves the workspace as it was
+    TORCH_CHECK(e != FX_ASYNC_BARRIER, "fx::lstm_stack: a wait of an earlier launch was given up; its results are not valid");
     TORCH_CHECK(T <= INT32_MAX && B <= INT32_MAX && H <= INT32_MAX, "fx::lstm_stack: sizes beyond 32 bits");
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index());
-    const size_t ws_bytes = fx_lstm_stack_workspace_bytes((int)B, (int)H, (int)L);
-    at::Tensor ws = lstmWorkspaces().get(x.device(), (void*)stream.stream(), ws_bytes);
+    at::Tensor ws = lstmWorkspaces().get(x.device(), (void*)stream.stream(), B, H, L);
     TORCH_CHECK(((uintptr_t)ws.data_ptr() & 255u) == 0, "fx::lstm_stack: workspace is not 256-byte aligned");
     FX_OK_OR_THROW(fx_lstm_stack(x.data_ptr<float>(), wih.data_ptr<float>(), whh.data_ptr<float>(), bih.data_ptr<float>(),
                                  bhh.data_ptr<float>(), h0.defined() ? h0.data_ptr<float>() : nullptr,

@@ -248,7 +248,7 @@ static std::atomic<uint32_t> g_stream_spin{[] {
   const char* e = getenv("FXHIP_STREAM_SPIN");
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
 }()};
-static std::atomic<uint32_t> g_lstm_spin{1000000u};   // polls of a barrier wait of fx_lstm_stack before it gives up
+static std::atomic<uint32_t> g_lstm_spin{1000000u};   // polls of a wait of fx_lstm_stack before it is given up
 static std::mutex g_dump_mu;
 static std::string g_dump_dir;
 
@@ -858,16 +858,15 @@ int fx_compact_rows(const uint8_t* mask, int64_t n, const void* const* cols, voi
 int fx_lstm_stack_fits(int batch, int hidden, int layers) {
   if (hidden < 32 || hidden > 1024 || (hidden & (hidden - 1)) != 0) return 0;
   if (layers < 1 || layers > 4 || batch < 1 || batch > 16) return 0;
-  // 1024 workgroups on 256 compute units: four per unit, 128 registers a lane, of which the
-  // weights may take 48 (at 512 and below two workgroups per unit suffice and every L fits)
-  if (hidden == 1024 && layers * (hidden / 32) > 48) return 0;
+  // 1024 hidden units are resident together only at four waves per SIMD, 128 registers a lane, of
+  // which the weight columns may take 64 (at 512 and below every L fits)
+  if (hidden == 1024 && layers * (hidden / 32) > 64) return 0;
   return 1;
 }
 size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers) {
   if (batch < 1 || hidden < 1 || layers < 1) return 0;
-  return (size_t)FX_LSTM_BAR_WORDS * 4 + (size_t)2 * layers * batch * hidden * 4;
+  return (size_t)FX_LSTM_CTL_WORDS * 4 + (size_t)2 * layers * batch * hidden * 8;
 }
-size_t fx_lstm_stack_workspace_clear_bytes(void) { return (size_t)FX_LSTM_BAR_WORDS * 4; }
 
 int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,
                   const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
@@ -879,13 +878,13 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
     return fail(FX_E_INVALID, "fx_lstm_stack: workspace smaller than fx_lstm_stack_workspace_bytes");
   if (((uintptr_t)workspace & 255u) != 0) return fail(FX_E_INVALID, "fx_lstm_stack: workspace must be 256-byte aligned");
   if (!fx_lstm_stack_fits(batch, hidden, layers))
-    return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: hidden must be a power of two in 32..1024, 1..4 layers (1 at hidden 1024), batch up to 16 (got hidden " +
+    return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: hidden must be a power of two in 32..1024, 1..4 layers (2 at hidden 1024), batch up to 16 (got hidden " +
                                       std::to_string(hidden) + ", layers " + std::to_string(layers) + ", batch " + std::to_string(batch) + ")");
   FxLstmArgs a;
   a.x = x; a.wih = wih; a.whh = whh; a.bih = bih; a.bhh = bhh; a.h0 = h0; a.c0 = c0;
   a.out = out; a.state_h = state_h; a.state_c = state_c;
-  a.bar = (uint32_t*)workspace;
-  a.hbuf = (float*)((char*)workspace + (size_t)FX_LSTM_BAR_WORDS * 4);
+  a.ctl = (uint32_t*)workspace;
+  a.hbuf = (uint64_t*)((char*)workspace + (size_t)FX_LSTM_CTL_WORDS * 4);
   a.err_host = err_word(true);
   a.T = seq_len; a.B = batch; a.H = hidden;
   a.spin_limit = g_lstm_spin.load(std::memory_order_relaxed);

@@ -1,16 +1,25 @@
-// Schedule and device-wide barrier of the persistent stacked-LSTM kernel (fx_lstm.hip), written
-// so that the same text also builds for the CPU, where tests run it with one host thread per
+// Schedule and hand-over protocol of the persistent stacked-LSTM kernel (fx_lstm.hip), written so
+// that the same text also builds for the CPU, where tests run it with one host thread per
 // workgroup (tests/support/lstm_emul.cpp) to check the schedule, the buffer parities and the
-// barrier protocol without a GPU.
+// protocol without a GPU.
 //
 // The recurrence (functs/benchmark/ai_model/lstm/lstm.py:79-133): for t in [0, T), for layer j in
 // [0, L): gates(t, j) need the output of layer j - 1 at time t and the state of layer j at time
 // t - 1.  Cells (t, j) with the same d = t + j are independent, so the kernel walks the
-// T + L - 1 diagonals d and computes every active layer of a diagonal between two barriers.
+// T + L - 1 diagonals d and computes every active layer of a diagonal in one step.
 //   h of (t, j), computed in step d, is written to hbuf[d & 1][j]; step d reads its inputs from
 //   hbuf[(d - 1) & 1] (layer j - 1 at time t and layer j at time t - 1 were both computed in
-//   step d - 1), from x (layer 0) and from h0 (t == 0).  Writing parity d & 1 in step d while
-//   parity (d - 1) & 1 is read needs one barrier per step and no other ordering.
+//   step d - 1), from x (layer 0) and from h0 (t == 0).
+// Hand-over without a barrier: every element of hbuf is 64 bits, the value and the TAG of the
+// step that wrote it (one atomic store), and a reader polls the elements it needs until they
+// carry the tag of the step it expects.  A workgroup writes step d only after it has read all
+// it needs of step d - 1, and nobody can be in step d + 1, whose writes land on the parity that
+// step d reads, before every workgroup has written step d: the two parities suffice.
+// Tags are base + d + 1, where base is a word of the workspace that the last workgroup to leave
+// advances past the tags of the launch, so the elements a launch finds from earlier launches
+// never carry a tag it waits for (a zeroed workspace carries tag 0, which no step has).
+// Every poll loop is bounded: a reader that gives up sets the error word and its workgroup
+// leaves; the others give up in turn.
 #pragma once
 #include <stdint.h>
 
@@ -18,17 +27,20 @@
 #define FX_LSTM_HD
 #endif
 
-#define FX_LSTM_GROUPS 16u         // first-level barrier counters
-#define FX_LSTM_LINE 64u           // words between counters: one 256-byte line each
-#define FX_LSTM_BAR_WORDS ((FX_LSTM_GROUPS + 3u) * FX_LSTM_LINE)   // groups, top counter, error word, leave counter
+#define FX_LSTM_LINE 64u                          // words between the control words: one 256-byte line each
+#define FX_LSTM_W_BASE 0u                         // tag base of the next launch
+#define FX_LSTM_W_LEAVE (1u * FX_LSTM_LINE)       // workgroups that have left
+#define FX_LSTM_W_ERR (2u * FX_LSTM_LINE)         // a wait was given up
+#define FX_LSTM_CTL_WORDS (3u * FX_LSTM_LINE)
+#define FX_LSTM_TAG_WRAP 0x80000000u              // the base starts over (and the tags are cleared) beyond this
 
 // arguments of the kernel (contiguous fp32 tensors; see fx_lstm_stack in include/fxhip.h)
 struct FxLstmArgs {
   const float *x, *wih, *whh, *bih, *bhh;
   const float *h0, *c0;   // null: zero initial state
   float *out, *state_h, *state_c;
-  float* hbuf;         // [2][L][B][H]: h of the cells of the last two steps
-  uint32_t* bar;       // FX_LSTM_BAR_WORDS words, zero when the kernel starts (and again when it ends without error)
+  uint64_t* hbuf;      // [2][L][B][H] (value, tag): h of the cells of the last two steps
+  uint32_t* ctl;       // FX_LSTM_CTL_WORDS control words
   uint32_t* err_host;  // pinned word that a given-up wait reports to as well (may be null)
   int T, B, H;
   uint32_t spin_limit;
@@ -43,47 +55,28 @@ FX_LSTM_HD inline int fx_lstm_time(int d, int j, int T) {
 FX_LSTM_HD inline uint32_t fx_lstm_hoff(int p, int j, int b, int u, int L, int B, int H) {
   return (uint32_t)((((p * L + j) * B + b) * H) + u);
 }
+FX_LSTM_HD inline uint64_t fx_lstm_pack(uint32_t value_bits, uint32_t tag) { return ((uint64_t)tag << 32) | value_bits; }
+FX_LSTM_HD inline uint32_t fx_lstm_tag_of(uint64_t e) { return (uint32_t)(e >> 32); }
+// tag of what step d writes / of what step d reads (written by step d - 1)
+FX_LSTM_HD inline uint32_t fx_lstm_tag_written(uint32_t base, int d) { return base + (uint32_t)d + 1u; }
+FX_LSTM_HD inline uint32_t fx_lstm_tag_read(uint32_t base, int d) { return base + (uint32_t)d; }
 
-// Arrival at the barrier that closes step `gen` (1-based) and the wait for everybody else.
-// Counters only grow during a launch and start from zero (fx_lstm_leave puts them back).  Two levels: a workgroup
-// adds to its group's counter, the last arrival of a group adds to the top counter, everybody
-// polls the top counter.  Returns false when the wait was given up (poll limit reached, or another
-// workgroup had already given up): the error word is set and the caller must leave the kernel.
-//   A: atomics policy { add_release(uint32_t*) -> old value, load(uint32_t*), store(uint32_t*, v),
-//                       acquire(), pause() }
+// A workgroup that has finished its last step checks out; the last one to do so (nobody reads
+// or writes hbuf any more) moves the tag base past this launch's tags and puts the counter back
+// to zero, so the same workspace serves the next launch on the stream without a clear in
+// between.  Past FX_LSTM_TAG_WRAP the base starts over at zero and the tags in hbuf are cleared
+// first.  A workgroup that gave up a wait does not check out: the error word stays set and the
+// host clears the whole workspace before it is used again.
+//   A: atomics policy { add(uint32_t*) -> old value, load(uint32_t*), store(uint32_t*, v), store64(uint64_t*, v) }
 template <class A>
-FX_LSTM_HD inline bool fx_lstm_barrier(uint32_t* bar, uint32_t gen, uint32_t wg, uint32_t n_wg, uint32_t spin_limit) {
-  const uint32_t n_groups = n_wg < FX_LSTM_GROUPS ? n_wg : FX_LSTM_GROUPS;
-  const uint32_t grp = wg % n_groups;
-  const uint32_t members = n_wg / n_groups + (grp < n_wg % n_groups ? 1u : 0u);
-  uint32_t* top = bar + FX_LSTM_GROUPS * FX_LSTM_LINE;
-  uint32_t* err = bar + (FX_LSTM_GROUPS + 1u) * FX_LSTM_LINE;
-  const uint32_t old = A::add_release(bar + grp * FX_LSTM_LINE);
-  if (old + 1u == gen * members) (void)A::add_release(top);
-  const uint32_t want = gen * n_groups;
-  uint32_t polls = 0;
-  for (;;) {
-    if (A::load(top) >= want) break;
-    if (A::load(err) != 0u || polls >= spin_limit) {
-      A::store(err, 1u);
-      return false;
-    }
-    ++polls;
-    A::pause();
+FX_LSTM_HD inline void fx_lstm_leave(uint32_t* ctl, uint32_t n_wg, uint32_t base, uint32_t n_steps, uint64_t* hbuf,
+                                     uint32_t n_elems) {
+  if (A::add(ctl + FX_LSTM_W_LEAVE) + 1u != n_wg) return;
+  uint32_t next = base + n_steps;
+  if (next >= FX_LSTM_TAG_WRAP) {
+    for (uint32_t i = 0; i < n_elems; ++i) A::store64(hbuf + i, 0ull);
+    next = 0u;
   }
-  A::acquire();
-  return true;
-}
-
-// A workgroup that has passed its last barrier of the launch checks out; the last one to do so
-// puts every counter back to zero, so the same words serve the next launch on the stream without
-// a clear in between.  Nobody polls any more at that point: a workgroup checks out only after its
-// own last wait has ended.  A workgroup that gave up a wait does not check out: the error word
-// stays set and the counters stay as they are until the host clears the words.
-template <class A>
-FX_LSTM_HD inline void fx_lstm_leave(uint32_t* bar, uint32_t n_wg) {
-  uint32_t* leave = bar + (FX_LSTM_GROUPS + 2u) * FX_LSTM_LINE;
-  if (A::add_release(leave) + 1u != n_wg) return;
-  for (uint32_t g = 0; g <= FX_LSTM_GROUPS; ++g) A::store(bar + g * FX_LSTM_LINE, 0u);
-  A::store(leave, 0u);
+  A::store(ctl + FX_LSTM_W_BASE, next);
+  A::store(ctl + FX_LSTM_W_LEAVE, 0u);
 }

@@ -304,24 +304,25 @@ int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* co
  * which the reference runs on the host, one fused kernel and two library GEMMs per (t, j)
  * (the loops carry state: fait/passes/parallelize_loops.cpp:17, unroll_loops.cpp:59-65), as ONE
  * persistent kernel: a workgroup per hidden unit keeps its columns of the weights in registers
- * for the whole sequence, the diagonals t + j are separated by a device-wide barrier with bounded
- * waits (a wait that is given up sets the error word of fx_async_error and ends the kernel).
+ * for the whole sequence; the diagonals t + j follow each other without a barrier, every h value
+ * travels with the tag of the step that wrote it and readers poll for the tag they expect, with
+ * bounded waits (a wait that is given up reports FX_ASYNC_BARRIER through fx_async_error and ends
+ * the kernel).
  * Contiguous fp32: x [T, B, H]; wih, whh [L, 4, H, H]; bih, bhh [L, 4, 1, H]; h0, c0, state_h,
  * state_c [L, B, H]; out [T, B, H]; h0 / c0 may be null (zero initial state).  H is 32, 64, ...
  * 1024 (a power of two), L <= 4, B <= 16 (FX_E_UNSUPPORTED otherwise), and H workgroups must be
  * resident together (FX_E_LIMIT).
- * workspace: fx_lstm_stack_workspace_bytes() of device memory, 256-byte aligned, whose first
- * fx_lstm_stack_workspace_clear_bytes() bytes are zero when the kernel starts.  A launch that ends
- * without error leaves them zero again, so one workspace, cleared once, serves launch after launch
- * on one stream (launches that share a workspace must not overlap); after a launch that reported
- * an error through fx_async_error the caller clears them again. */
+ * workspace: fx_lstm_stack_workspace_bytes() of device memory, 256-byte aligned, all zero when it
+ * is used for the first time.  A launch that ends without error leaves it ready for the next one,
+ * so one workspace, cleared once, serves launch after launch on one stream as long as batch,
+ * hidden and layers stay the same (launches that share a workspace must not overlap); after a
+ * launch that reported an error the caller clears it again. */
 /* 1 when fx_lstm_stack is built for these sizes, 0 otherwise: the part of its conditions that
  * needs no device, for a compiler pass that decides whether to emit the call (H a power of two in
  * 32..1024, L <= 4, B <= 16, and the weight columns of all layers fit the registers of a
- * workgroup at the occupancy that keeps H workgroups resident: L * H / 32 <= 48 for H = 1024). */
+ * workgroup at the occupancy that keeps all workgroups resident: L <= 2 for H = 1024). */
 int fx_lstm_stack_fits(int batch, int hidden, int layers);
 size_t fx_lstm_stack_workspace_bytes(int batch, int hidden, int layers);
-size_t fx_lstm_stack_workspace_clear_bytes(void);
 int fx_lstm_stack(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh, const float* h0,
                   const float* c0, float* out, float* state_h, float* state_c, int seq_len, int batch, int hidden,
                   int layers, void* workspace, size_t workspace_bytes, void* stream);

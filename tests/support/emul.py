@@ -31,7 +31,7 @@ def lstm_emul():
     so = ctypes.CDLL(_LSTM_SO)
     fp = ctypes.c_void_p
     so.fx_lstm_emul.restype = ctypes.c_int
-    so.fx_lstm_emul.argtypes = [fp] * 10 + [ctypes.c_int] * 4 + [ctypes.c_uint32, ctypes.c_int, ctypes.c_int]
+    so.fx_lstm_emul.argtypes = [fp] * 10 + [ctypes.c_int] * 4 + [ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_uint32]
     return so
 
 

@@ -6,7 +6,8 @@ are taken in another order than the oracle's BLAS takes them, plus 5e-6 absolute
 of up to 2 x 1024 products of magnitude 0.1, whose rounding error (a few 1e-6) does not shrink
 with the result when that happens to be near zero.
 On the CPU, the kernel's schedule (diagonals t + j, two parities of the h buffer) and its
-device-wide barrier run with one host thread per workgroup (tests/support/lstm_emul.cpp)."""
+hand-over protocol (values tagged with their step, bounded polls, the tag base carried from launch
+to launch) run with one host thread per workgroup (tests/support/lstm_emul.cpp)."""
 import ctypes
 
 import pytest
@@ -64,7 +65,7 @@ def test_reference_with_zero_states_is_the_oracle():
         assert torch.allclose(a, b, rtol=1e-6, atol=1e-7)
 
 
-def _emul(x, wih, whh, bih, bhh, h0, c0, spin=1 << 30, skip=-1, launches=1):
+def _emul(x, wih, whh, bih, bhh, h0, c0, spin=1 << 30, skip=-1, launches=1, base0=0):
     from tests.support import emul
     so = emul.lstm_emul()
     T, B, H = x.shape
@@ -72,7 +73,7 @@ def _emul(x, wih, whh, bih, bhh, h0, c0, spin=1 << 30, skip=-1, launches=1):
     out, sh, sc = torch.zeros(T, B, H), torch.zeros(L, B, H), torch.zeros(L, B, H)
     ts = [None if t is None else t.contiguous() for t in (x, wih, whh, bih, bhh, h0, c0)]
     err = so.fx_lstm_emul(*[None if t is None else t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(),
-                          sc.data_ptr(), T, B, H, L, spin, skip, launches)
+                          sc.data_ptr(), T, B, H, L, spin, skip, launches, base0)
     return (out, sh, sc), err
 
 
@@ -84,12 +85,25 @@ def test_schedule_and_barrier_on_host_threads(T, H, L, B):
     _close(got, _reference(*args), "emul T=%d H=%d L=%d B=%d" % (T, H, L, B))
 
 
-def test_launches_in_a_row_share_barrier_words_cleared_once():
-    """The last workgroup to leave puts the counters back to zero (-1: it did not)."""
+def test_launches_in_a_row_share_a_workspace_cleared_once():
+    """The last workgroup to leave moves the tag base past the launch's tags (-1: it did not), so
+    the values the next launch finds never carry a tag it waits for - also for the shortest
+    sequences, whose tags would repeat from launch to launch otherwise."""
     args = _inputs(11, 6, 64, 3, 2)
     got, err = _emul(*args, launches=3)
     assert err == 0
     _close(got, _reference(*args), "third launch")
+    args = _inputs(12, 1, 32, 2, 1)
+    got, err = _emul(*args, launches=4)
+    assert err == 0
+    _close(got, _reference(*args), "fourth launch of a one-step sequence")
+
+
+def test_the_tag_base_starts_over_before_it_wraps():
+    args = _inputs(13, 5, 32, 2, 1)
+    got, err = _emul(*args, launches=3, base0=0x80000000 - 8)
+    assert err == 0
+    _close(got, _reference(*args), "launch after the tags were cleared")
 
 
 def test_no_initial_state_means_zeros():
@@ -101,7 +115,7 @@ def test_no_initial_state_means_zeros():
 
 
 def test_a_wait_that_cannot_end_is_given_up():
-    """One workgroup never arrives: every other one must give up after the poll limit, set the
+    """One workgroup stops writing: every other one must give up after the poll limit, set the
     error word and return (on the GPU the kernel then ends instead of hanging)."""
     args = _inputs(3, 6, 32, 2, 1)
     _, err = _emul(*args, spin=2000, skip=5)
@@ -127,13 +141,12 @@ def _gpu(x, wih, whh, bih, bhh, h0, c0, launches=1):
                                 sc.data_ptr(), T, B, H, L, ws.data_ptr(), nbytes, stream))
         torch.cuda.synchronize()
         assert lib.fx_async_error(1) == 0
-    assert int(ws[:lib.fx_lstm_stack_workspace_clear_bytes()].count_nonzero()) == 0   # left as it was found
     return out.cpu(), sh.cpu(), sc.cpu()
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("T,H,L,B", [(1, 32, 1, 1), (5, 64, 2, 1), (9, 128, 3, 2), (4, 32, 4, 3), (16, 256, 2, 1),
-                                     (64, 512, 2, 1), (6, 512, 4, 16), (8, 1024, 1, 2)])
+                                     (64, 512, 2, 1), (6, 512, 4, 16), (8, 1024, 1, 2), (7, 1024, 2, 1)])
 def test_kernel_against_the_oracle(T, H, L, B):
     args = _inputs(T + H + L, T, H, L, B)
     _close(_gpu(*args), _reference(*args), "gpu T=%d H=%d L=%d B=%d" % (T, H, L, B))
@@ -179,5 +192,5 @@ def test_unsupported_shapes_are_refused():
 def test_sizes_the_kernel_is_built_for():
     from functs_amd._lib import lib
     assert lib.fx_lstm_stack_fits(1, 512, 2) == 1 and lib.fx_lstm_stack_fits(16, 512, 4) == 1
-    assert lib.fx_lstm_stack_fits(1, 1024, 1) == 1 and lib.fx_lstm_stack_fits(1, 1024, 2) == 0
+    assert lib.fx_lstm_stack_fits(1, 1024, 2) == 1 and lib.fx_lstm_stack_fits(1, 1024, 3) == 0
     assert lib.fx_lstm_stack_fits(1, 96, 2) == 0 and lib.fx_lstm_stack_fits(17, 64, 2) == 0 and lib.fx_lstm_stack_fits(1, 64, 5) == 0

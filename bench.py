@@ -307,6 +307,10 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch the library's plain copy kernel on BYTES (3 times): the known-size reference "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
+    ap.add_argument("--cold-profile", type=int, default=0, metavar="ROUNDS",
+                    help="profiling aid: nothing but ROUNDS rounds of the workload's kernels, every call on the next of the "
+                         "rotated buffer sets (cold lines), the caches flushed first; what a kernel trace or a counter run of "
+                         "this command sees of the region's kernels is all cold")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this path runs on ONE GPU. Its map tasks and row ranges are independent and "
@@ -318,6 +322,28 @@ def main():
     import functs_amd.aot as aot
     if args.interpreter:
         aot.enable(False)
+
+    if args.copy_calibration:
+        from functs_amd import _lib
+        n = args.copy_calibration // 4
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.copy_bytes(src, dst)
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+
+    if args.cold_profile:
+        from functs_amd.region import timed_sets
+        w = Workload(args.workload, dev)
+        n_sets = w.grow_cold()
+        flush(dev)
+        call_ms = [timed_sets([s[i] for s in w.sets], which=-1, rounds=args.cold_profile) for i in range(len(w.bound))]
+        print(json.dumps({"mode": "cold-profile", "workload": w.desc, "cold_sets": n_sets,
+                          "cold_bytes": n_sets * w.touched_bytes(), "rounds": args.cold_profile,
+                          "launches_per_call": w.launches, "call_kernels_ms": [round(m, 5) for m in call_ms],
+                          "calls_of_every_kernel": n_sets * (args.cold_profile + 2)}))
+        return
 
     def run_one(name, with_cpu):
         w = Workload(name, dev)
@@ -371,22 +397,12 @@ def main():
             rec["cpu"] = (us, n, cores)
         return rec
 
-    if args.copy_calibration:
-        from functs_amd import _lib
-        n = args.copy_calibration // 4
-        src = torch.ones(n, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            _lib.copy_bytes(src, dst)
-        torch.cuda.synchronize()
-        assert torch.equal(src, dst)
-
     def run_c4():
         """The stacked LSTM: its (time, layer) loops carry state, the reference runs them on the
         host.  Here the loop nest is collapsed into one node whose functor runs one persistent
-        kernel per call (weights read once, 65 dependent steps behind a device-wide barrier), so
-        the figure of merit is the latency of the call; the HBM fraction is reported for
-        completeness, the kernel is bound by the latency of its dependent steps."""
+        kernel per call (weights read once, 65 dependent steps that hand the h vectors from all
+        workgroups to all workgroups), so the figure of merit is the latency of the call; the HBM
+        fraction is reported for completeness, the kernel is bound by the latency of its steps."""
         from functs_amd.benchmark.inputs import INPUTS
         import functs_amd.aot as aot
         import functs_amd.jit as fj
@@ -434,7 +450,8 @@ def main():
                 "us_per_dependent_step": round(dev_us / (seq_len + layers - 1), 2),
                 "algorithmic_bytes": alg, "gbps_call": round(alg / (cold_us * 1e-6) / 1e9, 1),
                 "frac_hbm_peak": round(alg / (cold_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 5),
-                "bound": "latency of %d dependent steps (device-wide barrier each), not HBM" % (seq_len + layers - 1)}
+                "bound": "latency of %d dependent steps (each one hand-over of the h vectors between all workgroups through the "
+                         "memory side of the caches), not HBM" % (seq_len + layers - 1)}
 
     def run_tail():
         """The step behind the hot path: c5's compaction followed by the detection tail

@@ -53,8 +53,8 @@ __device__ __forceinline__ bool overlaps(const Box& a, float area_a, const Box& 
   return iou > thr;
 }
 
-// workspace: per task FX_NMS_WS_WORDS counters (candidates, finished slices, largest coordinate;
-// zero between launches) in front of all tasks' key buffers
+// workspace: per task FX_NMS_WS_WORDS counters (candidates, finished slices, largest coordinate,
+// row count + 1; zero between launches) in front of all tasks' key buffers
 #define FX_NMS_WS_WORDS 64u
 __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nms_desc d, const uint32_t key_cap,
                                                                     const uint32_t slices, uint32_t* const ws,
@@ -84,11 +84,27 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   int64_t* out_labels = d.out_labels + (size_t)task * d.max_num;
   int64_t* out_index = d.out_index ? d.out_index + (size_t)task * d.max_num : nullptr;
 
-  // one read of the task's row count per workgroup: the count may lie in host memory
+  // The task's row count may lie in host memory, where a read costs a trip over the bus and the
+  // reads of many workgroups queue up: slice 0 reads it and passes it on through the workspace
+  // (count + 1 in ctr[3]); a slice that does not see it within its polls reads it itself.
   if (tid == 0) {
     s_count = 0u;
     s_maxc = 0u;
-    s_base = d.counts ? min(d.rows, __hip_atomic_load(d.counts + task, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)) : d.rows;
+    uint32_t rows = d.rows;
+    if (d.counts) {
+      uint32_t seen = 0u;
+      if (slice != 0u)
+        for (uint32_t polls = 0; polls < 4096u && seen == 0u; ++polls) {
+          seen = __hip_atomic_load(&ctr[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (seen == 0u) __builtin_amdgcn_s_sleep(2);
+        }
+      if (seen == 0u) {
+        seen = min(d.rows, __hip_atomic_load(d.counts + task, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)) + 1u;
+        if (slice == 0u) __hip_atomic_store(&ctr[3], seen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      rows = seen - 1u;
+    }
+    s_base = rows;
   }
   __syncthreads();
   const uint32_t rows = s_base;
@@ -183,6 +199,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     __hip_atomic_store(&ctr[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(&ctr[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(&ctr[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&ctr[3], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (count > key_cap) {   // more candidates than the launch was sized for: reported, nothing returned
     if (tid == 0) {

@@ -147,6 +147,8 @@ _sig("fx_set_stream_spin_limit", None, ctypes.c_uint32)
 _sig("fx_plan_algorithmic_bytes", ctypes.c_int64, _vp)
 _sig("fx_plan_blob", _i, _vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)), ctypes.POINTER(ctypes.c_size_t))
 _sig("fx_plan_disasm", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_plan_head_info", _i, _vp, ctypes.POINTER(ctypes.c_int64), _i)
+_sig("fx_set_head_kernel", None, _i)
 _sig("fx_plan_spec_key", ctypes.c_uint64, _vp)
 _sig("fx_plan_specialized", _i, _vp)
 _sig("fx_plan_spec_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)

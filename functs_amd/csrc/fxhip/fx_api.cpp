@@ -35,6 +35,10 @@ hipError_t fx_launch_compact_stream(int rank, const uint32_t* sb, const FxLaunch
                                     hipStream_t stream, const FxSpecKernels* spec);
 uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled);
 bool fx_spec_has_stream(const FxSpecKernels* spec);
+// fx_head.hip
+hipError_t fx_launch_head_stream(const FxHeadLaunch& hl, const FxDyn* dyn, hipStream_t stream);
+hipError_t fx_head_resident(uint32_t lds_bytes, uint32_t* workgroups, uint32_t* per_cu);
+uint32_t fx_head_lds_bytes(const FxHeadLaunch& hl);
 #include "fx_lstm_sched.h"
 int fx_launch_lstm_stack(const FxLstmArgs& a, int L, hipStream_t stream);
 int fx_launch_sort_nms(const fx_nms_desc& d, uint32_t key_cap, void* workspace, uint32_t* err_host, hipStream_t stream);
@@ -244,6 +248,11 @@ static std::atomic<int> g_stream_mode{[] {
   const char* e = getenv("FXHIP_STREAM");
   return (e && e[0] == '1') ? 1 : 0;
 }()};
+// ---- detection-head kernel (fx_head.h): on unless FXHIP_HEAD=0 ----
+static std::atomic<int> g_head_mode{[] {
+  const char* e = getenv("FXHIP_HEAD");
+  return (e && e[0] == '0') ? 0 : 1;
+}()};
 static std::atomic<uint32_t> g_stream_spin{[] {
   const char* e = getenv("FXHIP_STREAM_SPIN");
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
@@ -346,12 +355,34 @@ int fx_plan_output(const fx_plan* p, int out_idx, int task, int32_t* dtype, int3
 size_t fx_plan_scratch_bytes(const fx_plan* p) { return p ? P(p)->scratch_bytes : 0; }
 static bool stream_active(const fx::Plan* pl, const FxSpecKernels* spec);
 static const FxSpecKernels* spec_of(const fx::Plan* p);
+static bool head_active(const fx::Plan* pl) {
+  // (with compiled kernels switched off, fx_set_specialization(0), everything runs in the interpreter)
+  return pl->mode == FX_MODE_COMPACT && pl->head.ok && g_head_mode.load(std::memory_order_relaxed) != 0 &&
+         g_specialize.load(std::memory_order_relaxed) != 0;
+}
+void fx_set_head_kernel(int on) { g_head_mode.store(on ? 1 : 0, std::memory_order_relaxed); }
+int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
+  if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_head_info: out[>=8] required");
+  const FxHeadInfo& hi = P(p)->head;
+  out[0] = hi.ok ? 1 : 0;
+  out[1] = head_active(P(p)) ? 1 : 0;
+  out[2] = (int64_t)(hi.norm_hash & 0xffffffffull);
+  out[3] = (int64_t)(hi.norm_hash >> 32);
+  out[4] = hi.C;
+  out[5] = hi.S;
+  out[6] = hi.n_rows;
+  out[7] = hi.n_tasks;
+  return FX_OK;
+}
 int fx_plan_launches(const fx_plan* p) {
   if (!p) return 0;
+  if (head_active(P(p))) return 1;
   if (P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) return P(p)->stream.grid > 0 ? 1 : 0;
   return P(p)->launches;
 }
-int fx_plan_streaming(const fx_plan* p) { return (p && P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) ? 1 : 0; }
+int fx_plan_streaming(const fx_plan* p) {
+  return (p && P(p)->mode == FX_MODE_COMPACT && !head_active(P(p)) && stream_active(P(p), spec_of(P(p)))) ? 1 : 0;
+}
 int fx_plan_stream_info(const fx_plan* p, int64_t* out, int cap) {
   if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_stream_info: out[>=8] required");
   const fx::StreamInfo& si = P(p)->stream;
@@ -541,29 +572,92 @@ static uint32_t stream_grid(const fx::Plan* pl) { return std::min<uint32_t>(pl->
 
 // Status words of `pl` for launches on `stream` (created on first use, at most four streams per
 // plan: calls on further streams take the two-pass form) and the epoch of the next call.
-static int stream_status(fx_region* reg, fx::Plan* pl, hipStream_t stream, int dev, void** ptr, uint32_t* epoch,
-                         int n_epochs) {
+static int status_words(fx_region* reg, std::vector<fx::Plan::Status>& list, size_t words, hipStream_t stream, int dev,
+                        void** ptr, uint32_t* epoch, int n_epochs) {
   std::lock_guard<std::mutex> g(reg->mu);
   fx::Plan::Status* st = nullptr;
-  for (auto& s : pl->status)
+  for (auto& s : list)
     if (s.stream == (void*)stream && s.dev == dev) st = &s;
+  const size_t bytes = std::max<size_t>(words, 1) * 4;
   if (!st) {
-    if (pl->status.size() >= 4) { *ptr = nullptr; return FX_OK; }
+    if (list.size() >= 4) { *ptr = nullptr; return FX_OK; }
     void* d = nullptr;
-    const size_t bytes = (size_t)std::max<uint32_t>(pl->stream.grid, 1) * 4;
     HIP_OK(hipMalloc(&d, bytes));
     HIP_OK(hipMemset(d, 0, bytes));
-    pl->status.push_back({(void*)stream, d, 0u, dev});
-    st = &pl->status.back();
+    list.push_back({(void*)stream, d, 0u, dev});
+    st = &list.back();
   }
   if (st->epoch + (uint32_t)n_epochs >= FX_EPOCH_MAX) {
     // the tags wrap: clear the words behind everything already queued on the stream
-    HIP_OK(hipMemsetAsync(st->ptr, 0, (size_t)std::max<uint32_t>(pl->stream.grid, 1) * 4, stream));
+    HIP_OK(hipMemsetAsync(st->ptr, 0, bytes, stream));
     st->epoch = 0;
   }
   *ptr = st->ptr;
   *epoch = st->epoch + 1;
   st->epoch += (uint32_t)n_epochs;
+  return FX_OK;
+}
+static int stream_status(fx_region* reg, fx::Plan* pl, hipStream_t stream, int dev, void** ptr, uint32_t* epoch,
+                         int n_epochs) {
+  return status_words(reg, pl->status, pl->stream.grid, stream, dev, ptr, epoch, n_epochs);
+}
+
+// ---- detection-head kernel: geometry of a launch ----
+// Rows of a sub-tile: what FX_HEAD_KV 128-bit loads per lane carry, at most FX_HEAD_SUB.
+static uint32_t head_sub_rows(const FxHeadInfo& hi) {
+  const uint32_t cap = (FX_HEAD_KV * FX_BLOCK * 4u - 6u) / hi.S;
+  return std::min<uint32_t>(FX_HEAD_SUB, cap);
+}
+static size_t head_status_words(const FxHeadInfo& hi) {
+  const uint32_t min_chunk = std::min<uint32_t>(FX_HEAD_MIN_CHUNK, std::max<uint32_t>(hi.n_rows, 1u));
+  return (size_t)hi.n_tasks * ((hi.n_rows + min_chunk - 1) / min_chunk);
+}
+static bool head_fits(const fx::Plan* pl) {
+  // a sub-tile of at least 8 rows, and counts of up to FX_BLOCK rows in a status word
+  return head_active(pl) && head_sub_rows(pl->head) >= 8u;
+}
+// Every image's rows are dealt to its workgroups in equal runs, as few workgroups as give every
+// resident slot of the device one (more only when a chunk would exceed FX_BLOCK rows, fewer when
+// it would fall below FX_HEAD_MIN_CHUNK).
+static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
+  const FxHeadInfo& hi = pl->head;
+  memset(hl, 0, sizeof(*hl));
+  hl->n_rows = hi.n_rows;
+  hl->n_tasks = hi.n_tasks;
+  hl->sub_rows = head_sub_rows(hi);
+  hl->S = hi.S;
+  hl->C = hi.C;
+  fx_fastdiv_make(hi.C / 4u, &hl->g_magic, &hl->g_shift);
+  hl->thr_bits = hi.thr_bits;
+  hl->spin_limit = g_stream_spin.load(std::memory_order_relaxed);
+  hl->n_sptr = (uint32_t)pl->sptr.size();
+  hl->n_tptr = (uint32_t)pl->tptr.size();
+  hl->pred_slot = hi.pred_slot;
+  hl->anc_slot = hi.anc_slot;
+  hl->strd_slot = hi.strd_slot;
+  hl->pred_tcoef = hi.pred_tcoef;
+  hl->anc_tcoef = hi.anc_tcoef;
+  hl->strd_tcoef = hi.strd_tcoef;
+  for (int k = 0; k < 3; ++k) {
+    hl->out_slot[k] = hi.out_slot[k];
+    hl->out_tstride[k] = hi.out_tstride[k];
+  }
+  if (pl->head_resident == 0) {
+    // One slot per CU is left free: a launch that needs every slot the occupancy rule allows does
+    // not get all of its workgroups placed at once, and the stragglers cost a second round.
+    uint32_t wg = 0, per_cu = 1;
+    HIP_OK(fx_head_resident(fx_head_lds_bytes(*hl), &wg, &per_cu));
+    if (per_cu >= 3) wg -= wg / per_cu;
+    if (const char* e = getenv("FXHIP_HEAD_RESIDENT")) wg = (uint32_t)atoi(e);
+    pl->head_resident = std::max<uint32_t>(wg, 1u);
+  }
+  const uint32_t per_task = std::max<uint32_t>(1u, pl->head_resident / std::max<uint32_t>(hi.n_tasks, 1u));
+  uint32_t cr = (hi.n_rows + per_task - 1) / per_task;
+  const uint32_t min_chunk = std::min<uint32_t>(FX_HEAD_MIN_CHUNK, std::max<uint32_t>(hi.n_rows, 1u));
+  cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
+  if (const char* e = getenv("FXHIP_HEAD_CHUNK")) cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(1u, (uint32_t)atoi(e)));
+  hl->chunk_rows = cr;
+  hl->chunks = (hi.n_rows + cr - 1) / cr;
   return FX_OK;
 }
 
@@ -603,9 +697,21 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                                 ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
   }
   FxLaunchInfo li = launch_info(pl);
-  bool streaming = pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
+  bool head = head_fits(pl);
+  FxHeadLaunch hl;
   void* status = nullptr;
   uint32_t epoch = 0;
+  if (head) {
+    rc = head_launch_info(pl, &hl);
+    if (rc != FX_OK) return rc;
+    void* hstatus = nullptr;
+    rc = status_words(reg, pl->head_status, head_status_words(pl->head), stream, dev, &hstatus, &epoch, repeat);
+    if (rc != FX_OK) return rc;
+    if (!hstatus) head = false;
+    hl.status = (uint32_t*)hstatus;
+    hl.totals = totals_host;
+  }
+  bool streaming = !head && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
   if (streaming) {
     rc = stream_status(reg, pl, stream, dev, &status, &epoch, repeat);
     if (rc != FX_OK) return rc;
@@ -624,9 +730,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                            ? FX_TOTAL_PENDING
                            : 0u;
   }
-  const int launches = streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
+  const int launches = head ? (hl.chunks * hl.n_tasks > 0 ? 1 : 0) : streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
   g_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
-  if (spec) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
+  if (spec || head) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
   const bool timed = kernel_ms != nullptr;
@@ -641,6 +747,14 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
       HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
+  } else if (head) {
+    HIP_OK(mark(0));
+    for (int r = 0; r < repeat; ++r) {
+      hl.epoch = epoch + (uint32_t)r;
+      HIP_OK(fx_launch_head_stream(hl, &dyn, stream));
+    }
+    HIP_OK(mark(1));
+    nk = hl.chunks * hl.n_tasks > 0 ? 1 : 0;
   } else if (streaming) {
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
@@ -696,17 +810,28 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   }
   const FxSpecKernels* spec = spec_of(pl);
   FxLaunchInfo li = launch_info(pl);
-  bool streaming = compact && stream_active(pl, spec);
   void* status = nullptr;
   uint32_t epoch = 0;
   int dev = 0;
   HIP_OK(hipGetDevice(&dev));
+  bool head = compact && head_fits(pl);
+  FxHeadLaunch hl;
+  if (head) {
+    int rc = head_launch_info(pl, &hl);
+    if (rc != FX_OK) return rc;
+    void* hstatus = nullptr;
+    rc = status_words(reg, pl->head_status, head_status_words(pl->head), stream, dev, &hstatus, &epoch, rounds * n_sets);
+    if (rc != FX_OK) return rc;
+    if (!hstatus) head = false;
+    hl.status = (uint32_t*)hstatus;
+  }
+  bool streaming = !head && compact && stream_active(pl, spec);
   if (streaming) {
     const int rc = stream_status(reg, pl, stream, dev, &status, &epoch, rounds * n_sets);
     if (rc != FX_OK) return rc;
     if (!status) streaming = false;
   }
-  if (which >= (streaming ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
+  if (which >= ((streaming || head) ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
   std::vector<FxDyn> dyn((size_t)n_sets);
   for (int i = 0; i < n_sets; ++i) {
     memset(&dyn[i], 0, sizeof(FxDyn));
@@ -724,6 +849,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     for (int i = 0; i < n_sets; ++i) {
       if (!compact) {
         HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+      } else if (head) {
+        hl.epoch = epoch + (uint32_t)(r * n_sets + i);
+        hl.totals = totals_host[i];
+        HIP_OK(fx_launch_head_stream(hl, &dyn[i], stream));
       } else if (streaming) {
         li.epoch = epoch + (uint32_t)(r * n_sets + i);
         li.total_units = pl->stream.grid;

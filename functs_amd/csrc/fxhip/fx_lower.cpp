@@ -2296,6 +2296,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
     }
   }
   P->spec_key = spec_hash(*P);
+  match_head(P.get());
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;

@@ -18,6 +18,7 @@
 
 #include "../../../include/fxhip.h"
 #include "fx_bytecode.h"
+#include "fx_head.h"
 
 namespace fx {
 
@@ -104,6 +105,7 @@ struct Plan {
   uint32_t lds_bytes = 0;
   bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
   StreamInfo stream;
+  FxHeadInfo head;               // the plan is the decode + score filter of a detection head (fx_head.h)
   bool uses_guard = false;       // some load checks int64 data against 32 bits and reports to the error word
   uint32_t n_temps = 0;
   int max_rank = 1;
@@ -124,7 +126,13 @@ struct Plan {
   // never reset: every call tags its words with the next epoch)
   struct Status { void* stream; void* ptr; uint32_t epoch; int dev; };
   std::vector<Status> status;
+  // the same for the chunks of the detection-head kernel, and the workgroups of it the device holds at once
+  std::vector<Status> head_status;
+  uint32_t head_resident = 0;
 };
+
+// Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?
+void match_head(Plan* p);
 
 // Builds (or fetches from the cache) the plan of `r` for these arguments.
 const Plan* plan_region(Region& r, const fx_arg* args, int n_args);

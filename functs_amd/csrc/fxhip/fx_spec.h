@@ -75,13 +75,16 @@ constexpr int fx_spec_n_insn() { return (int)(sizeof(P::code) / sizeof(P::code[0
 // round trip per stretch instead of one per load.  Dense regions only: in a row compaction
 // the loads of a narrow output are gathers over the kept rows, which gain nothing from being
 // in flight together (measured), and the registers they hold cost a wave per SIMD.
+#ifndef FX_SPEC_HOIST_COMPACT
+#define FX_SPEC_HOIST_COMPACT 0
+#endif
 #ifndef FX_SPEC_HOIST
 #define FX_SPEC_HOIST 8
 #endif
 template <class P>
 constexpr int fx_spec_hoist_cap() {
   for (int e = 0; e < P::n_entries; ++e)
-    if (P::entries[e].kind == 1) return 0;   // a mask program: this is a row compaction
+    if (P::entries[e].kind == 1) return FX_SPEC_HOIST_COMPACT;   // a mask program: this is a row compaction
   return FX_SPEC_HOIST;
 }
 

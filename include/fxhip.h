@@ -171,7 +171,8 @@ int64_t fx_plan_algorithmic_bytes(const fx_plan*); /* compulsory input bytes + d
  * evaluate the mask from there, publish their kept-row count and take their write offset from
  * the counts of the earlier tiles (every wait bounded; a workgroup that waits too long counts
  * the earlier rows itself).  Results are identical to the two-pass form (count + scatter), which
- * is the default because it is the faster one on the benchmark configurations but the smallest.
+ * is the default because it is the faster one on the benchmark configurations but the smallest
+ * (the detection-head regions among them have a kernel of their own, below).
  * fx_plan_streaming: 1 if fx_region_run would use the one-pass form for this plan now;
  * fx_set_streaming: process-wide switch (default off; FXHIP_STREAM=1: on);
  * fx_set_stream_spin_limit: polls before a workgroup stops waiting (default 4000; 0 makes every
@@ -183,6 +184,25 @@ int fx_plan_streaming(const fx_plan*);
 int fx_plan_stream_info(const fx_plan*, int64_t* out, int cap);
 void fx_set_streaming(int on);
 void fx_set_stream_spin_limit(uint32_t polls);
+/* The decode + score filter of a YOLO-style detection head in one launch.  A compacting region
+ * whose lowered programs ARE that computation (sigmoid of the centre offsets, exp of the sizes,
+ * anchors [N, 4] and strides [N], objectness threshold, kept rows of boxes [K, 4], class scores
+ * [K, C] and objectness [K] out of predictions [images, N, 5 + C]; the reference's flagship
+ * post-processing, functs/benchmark/ai_model/yolov3/yolov3_bbox.py:12-23 and 104-130) runs through
+ * a hand-written kernel instead of the generic two passes: every workgroup streams a run of
+ * consecutive prediction rows through LDS, publishes its kept-row count at once and takes its
+ * write offset from the counts of the earlier workgroups of its image (every wait bounded, as
+ * in the one-pass form above, with the same poll limit).  The programs are compared instruction
+ * by instruction (any number of rows, images and classes C with C % 4 == 0, any threshold); a
+ * region that differs anywhere keeps the generic kernels.  Results are bit-identical to those.
+ * fx_set_head_kernel: process-wide switch, default on (FXHIP_HEAD=0: off; also off while
+ * fx_set_specialization(0) holds).  fx_plan_head_info: out[0..8) = region recognised, kernel
+ * in use now, low and high word of the hash of the normalised programs, C, 5 + C, rows, images
+ * (test hook).  This is where the reference compiles the subgraph of the loop body with NVRTC
+ * (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1414) and leaves x[mask] to ATen
+ * (convert_to_tensorssa.cpp:422-443). */
+void fx_set_head_kernel(int on);
+int fx_plan_head_info(const fx_plan*, int64_t* out, int cap);
 /* debugging / test hooks: the lowered bytecode blob (like CodeGen::getCodeText) */
 int fx_plan_blob(const fx_plan*, const uint32_t** words, size_t* n_words);
 int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);

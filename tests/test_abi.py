@@ -77,14 +77,20 @@ def test_plan_metadata_and_disasm():
     preds, anchors, strides = oc.c5_inputs(0, [2, 3], 3)
     arr, n, _ = r._flatten([preds, anchors, strides])
     p = r.plan(arr, n)
-    # two kernels in the two-pass form (the default), one in the streaming form
+    # this region is the detection head that has a kernel of its own (one launch); without it
+    # two kernels in the two-pass form, one in the streaming form
     assert p.n_out == 3 and p.compact
-    assert p.launches == 2 and _lib.lib.fx_plan_streaming(p.handle) == 0
-    _lib.lib.fx_set_streaming(1)
+    assert _lib.lib.fx_plan_launches(p.handle) == 1 and _lib.lib.fx_plan_streaming(p.handle) == 0
+    _lib.lib.fx_set_head_kernel(0)
     try:
-        assert _lib.lib.fx_plan_launches(p.handle) == 1 and _lib.lib.fx_plan_streaming(p.handle) == 1
+        assert _lib.lib.fx_plan_launches(p.handle) == 2 and _lib.lib.fx_plan_streaming(p.handle) == 0
+        _lib.lib.fx_set_streaming(1)
+        try:
+            assert _lib.lib.fx_plan_launches(p.handle) == 1 and _lib.lib.fx_plan_streaming(p.handle) == 1
+        finally:
+            _lib.lib.fx_set_streaming(0)
     finally:
-        _lib.lib.fx_set_streaming(0)
+        _lib.lib.fx_set_head_kernel(1)
     assert p.out_meta[1][2] == (torch.float32, (preds.size(1), 80))
     assert p.alg_bytes == (preds.numel() + anchors.numel() + strides.numel()) * 4
     assert p.scratch_bytes > 0

@@ -12,6 +12,15 @@ from oracle import configs as oc
 from tests.util import assert_boxes_close, assert_close, assert_exact, run_region
 
 
+@pytest.fixture(autouse=True)
+def generic_kernels_only():
+    """The detection-head regions used here have a kernel of their own (tests/test_head_stream.py);
+    these tests are about the generic one-pass form."""
+    lib.fx_set_head_kernel(0)
+    yield
+    lib.fx_set_head_kernel(1)
+
+
 def _stream_info(r, *args):
     arr, n, _ = r._flatten(args)
     p = r.plan(arr, n)

@@ -195,6 +195,40 @@ def recorded_traffic(kernel, workload):
     return None, None
 
 
+def head_kernel_in_use(plan):
+    """Does a call of this plan run the hand-written detection-head kernel (fx_head_stream)?"""
+    import ctypes
+    from functs_amd import _lib
+    out = (ctypes.c_int64 * 8)()
+    _lib.check(_lib.lib.fx_plan_head_info(plan.handle, out, 8))
+    return bool(out[1])
+
+
+def copy_reference_ms(dev, nbytes, rounds=4):
+    """The library's plain copy kernel moving the same number of bytes (half read, half written)
+    on cold lines: pairs of buffers that together exceed the last-level cache, in rotation, the
+    caches flushed first.  What the memory system gives a kernel that does nothing else."""
+    import torch
+    from functs_amd import _lib
+    half = max(nbytes // 2 // 16 * 16, 16)
+    n_pairs = max(4, -(-COLD_BYTES // (2 * half)))
+    pairs = [(torch.empty(half, dtype=torch.uint8, device=dev), torch.empty(half, dtype=torch.uint8, device=dev))
+             for _ in range(n_pairs)]
+    for a, b in pairs:
+        a.zero_()
+        _lib.copy_bytes(a, b)
+    flush(dev)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(rounds):
+        for a, b in pairs:
+            _lib.copy_bytes(a, b)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (rounds * n_pairs)
+
+
 def measure(w, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -304,6 +338,9 @@ def main():
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--interpreter", action="store_true",
                     help="run every region with the bytecode interpreter (no ahead-of-time compiled kernels)")
+    ap.add_argument("--no-head-kernel", action="store_true",
+                    help="run the detection-head regions (c2, c5) with the generic row-compaction kernels (count + scatter) "
+                         "instead of the hand-written fx_head_stream")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch the library's plain copy kernel on BYTES (3 times): the known-size reference "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -322,6 +359,9 @@ def main():
     import functs_amd.aot as aot
     if args.interpreter:
         aot.enable(False)
+    if args.no_head_kernel:
+        from functs_amd import _lib
+        _lib.lib.fx_set_head_kernel(0)
 
     if args.copy_calibration:
         from functs_amd import _lib
@@ -368,6 +408,7 @@ def main():
             "cold_bytes": n_sets * w.touched_bytes(),
             "launches_per_call": w.launches,
             "row_compaction": any(bc.plan.compact for bc in w.bound),
+            "head_kernel": any(head_kernel_in_use(bc.plan) for bc in w.bound),
             "algorithmic_bytes": alg,
             "dominant_kernel_index": dom_i,
             "gbps_dominant_kernel": round(alg / (dom * 1e-3) / 1e9, 1),
@@ -603,7 +644,8 @@ def main():
             per["c5_nms_tail"] = {"error": str(e)[:200]}
     cpu_us, cpu_n, cores = head.pop("cpu")
     dom_ms = head["kernel_us"][head["dominant_kernel_index"]] / 1e3
-    dom_kernel = "fx_compact_scatter" if head["row_compaction"] else "fx_region_dense"
+    dom_kernel = "fx_head_stream" if head.get("head_kernel") else ("fx_compact_scatter" if head["row_compaction"] else "fx_region_dense")
+    copy_ms = copy_reference_ms(dev, head["algorithmic_bytes"])
     traffic, traffic_src = recorded_traffic(dom_kernel, args.workload)
     out = {
         "metric": "per-call latency",
@@ -640,11 +682,15 @@ def main():
                      "call_kernels_ms": round(head["call_kernels_us"] / 1e3, 5),
                      "kernel_ms_single_launch": round(head["kernel_us_single_launch"][head["dominant_kernel_index"]] / 1e3, 5),
                      "cold_sets": head["cold_sets"], "cold_bytes": head["cold_bytes"],
+                     "copy_same_bytes_ms": round(copy_ms, 5),
+                     "copy_same_bytes_frac": round(head["algorithmic_bytes"] / (copy_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "timing": "HIP events on the launch stream around back-to-back launches, mean per launch. frac / kernel_ms: "
                                "the dominant kernel rotated over cold_sets independent sets of inputs, outputs and scratch "
                                "(cold_bytes in total, above the 256 MB last-level cache), the caches flushed before; "
                                "frac_warm / kernel_ms_warm: %d launches on one set; frac_call / call_kernels_ms: every kernel of "
-                               "the call in order, rotated the same way; frac_call_warm: sum of the warm kernels" % KERNEL_BATCH},
+                               "the call in order, rotated the same way; frac_call_warm: sum of the warm kernels; "
+                               "copy_same_bytes_ms / _frac: the library's plain copy kernel moving algorithmic_bytes (half read, "
+                               "half written) on cold lines, the same way" % KERNEL_BATCH},
         "cpu_baseline": {"value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
                          "sample": "%d calls of torch.jit.script(%s) on the same seeded CPU tensors" % (cpu_n, args.workload)},
         "per_config": per,

@@ -648,14 +648,12 @@ static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
     uint32_t wg = 0, per_cu = 1;
     HIP_OK(fx_head_resident(fx_head_lds_bytes(*hl), &wg, &per_cu));
     if (per_cu >= 3) wg -= wg / per_cu;
-    if (const char* e = getenv("FXHIP_HEAD_RESIDENT")) wg = (uint32_t)atoi(e);
     pl->head_resident = std::max<uint32_t>(wg, 1u);
   }
   const uint32_t per_task = std::max<uint32_t>(1u, pl->head_resident / std::max<uint32_t>(hi.n_tasks, 1u));
   uint32_t cr = (hi.n_rows + per_task - 1) / per_task;
   const uint32_t min_chunk = std::min<uint32_t>(FX_HEAD_MIN_CHUNK, std::max<uint32_t>(hi.n_rows, 1u));
   cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
-  if (const char* e = getenv("FXHIP_HEAD_CHUNK")) cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(1u, (uint32_t)atoi(e)));
   hl->chunk_rows = cr;
   hl->chunks = (hi.n_rows + cr - 1) / cr;
   return FX_OK;

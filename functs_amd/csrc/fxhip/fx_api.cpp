@@ -656,6 +656,11 @@ static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
   cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
   hl->chunk_rows = cr;
   hl->chunks = (hi.n_rows + cr - 1) / cr;
+  // A launch whose first sub-tiles alone are megabytes of requests floods the memory system: there
+  // the counts get a head start (fx_head.hip; neutral on some boxes, 5 us of 26 on others).  A
+  // small launch would only lose the time.
+  const uint64_t first_bytes = (uint64_t)hl->chunks * hi.n_tasks * std::min<uint32_t>(cr, hl->sub_rows) * hi.S * 4u;
+  hl->bulk_delay = first_bytes >= FX_HEAD_FLOOD_BYTES ? FX_HEAD_BULK_DELAY : 0u;
   return FX_OK;
 }
 

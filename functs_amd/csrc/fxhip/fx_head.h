@@ -16,6 +16,8 @@
 #define FX_HEAD_NSUB 4u        // most sub-tiles of a chunk: a chunk holds at most FX_BLOCK rows
 #define FX_HEAD_KV 6u          // 128-bit loads per lane that carry a sub-tile
 #define FX_HEAD_STATUS_BITS 9u // a chunk's count is at most FX_BLOCK
+#define FX_HEAD_FLOOD_BYTES (8u << 20)   // first sub-tiles of a launch from which on the counts are sent ahead of the rows
+#define FX_HEAD_BULK_DELAY 128u           // by this many units of 64 clocks
 #define FX_HEAD_MIN_CHUNK 64u  // fewest rows of a chunk unless the image has fewer
 // hash of the normalised programs of the detection-head region (fx_head_match.cpp)
 #define FX_HEAD_NORM_HASH 0xed6ab9314c50ff65ull
@@ -47,7 +49,7 @@ struct FxHeadLaunch {
   uint32_t pred_slot, anc_slot, strd_slot;
   int32_t pred_tcoef, anc_tcoef, strd_tcoef;
   uint32_t out_slot[3], out_tstride[3];
-  uint32_t pad;
+  uint32_t bulk_delay;           // big launches: waves without a gather wait this long (units of 64 clocks) before they ask for rows
   uint32_t* status;              // one word per chunk, tagged with the epoch
   uint32_t* totals;              // pinned host memory: kept rows per task
 };

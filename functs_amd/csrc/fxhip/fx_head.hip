@@ -45,7 +45,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
   __shared__ uint32_t s_rowmap[FX_HEAD_SUB];
   __shared__ uint8_t s_keep[FX_BLOCK];
   __shared__ uint32_t s_wsum[NW];
-  __shared__ uint32_t s_prefix, s_ok, s_nk, s_total;
+  __shared__ uint32_t s_prefix, s_ok, s_nk, s_total, s_told;
   const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
   const uint32_t b = blockIdx.x;
   const uint32_t task = b / hl.chunks, chunk = b - task * hl.chunks;
@@ -60,22 +60,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
   // element 0 of this task's rows
   const FX_AS1 float* pred = (const FX_AS1 float*)fxh_ptr(hl, hl.pred_slot, task) + (int64_t)hl.pred_tcoef * task;
 
-  // ---- requests: objectness of the chunk (wave 0), first look at the earlier chunks (wave 1),
-  // rows of the first sub-tile (everybody)
-  float o[NSUB];
-  uint32_t pw[2] = {0, 0};
-  if (wave == 0) {
-#pragma unroll
-    for (uint32_t j = 0; j < NSUB; ++j) {
-      const uint32_t r = j * 64u + lane;
-      o[j] = r < c_rows ? pred[(size_t)(c_r0 + r) * S + 4u] : 0.0f;
-    }
-  } else if (wave == 1) {
-#pragma unroll
-    for (uint32_t j = 0; j < 2; ++j)
-      if (j * 64u + lane < chunk)
-        pw[j] = __hip_atomic_load(hl.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
   fx_u32x4 wr[KV];
   uint32_t shift = 0, n_vec = 0;
   auto request = [&](uint32_t s) {
@@ -90,6 +74,73 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
       if (v < n_vec) wr[k] = g4[v];
     }
   };
+  uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
+  // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the image.
+  auto look_back = [&]() {
+    const uint32_t first = b - chunk;
+    uint32_t part = 0;
+    bool ok = true;
+    for (uint32_t i = lane; i < chunk; i += 64u) {
+      uint32_t wv = i < 64u ? pw[0] : (i < 128u ? pw[1] : 0u), polls = 0;
+      while ((wv >> FX_HEAD_STATUS_BITS) != hl.epoch) {
+        if (polls >= hl.spin_limit) { ok = false; break; }
+        ++polls;
+        __builtin_amdgcn_s_sleep(1);
+        wv = __hip_atomic_load(hl.status + first + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      part += ok ? (wv & ((1u << FX_HEAD_STATUS_BITS) - 1u)) : 0u;
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
+    const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
+    if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
+    // The image's last chunk tells the host the image's total as soon as it is known, before
+    // any of its rows has arrived: its own count comes from its status word (wave 0 publishes
+    // it right after the gather).  The host polls the word while the kernel still runs: a
+    // system-scope store goes through to host memory instead of waiting in L2 for the end of
+    // the kernel.
+    if (chunk + 1u == hl.chunks && all_ok) {
+      uint32_t wv = 0, polls = 0;
+      bool own = true;
+      for (;;) {
+        wv = __hip_atomic_load(hl.status + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((wv >> FX_HEAD_STATUS_BITS) == hl.epoch) break;
+        if (polls >= hl.spin_limit) { own = false; break; }
+        ++polls;
+        __builtin_amdgcn_s_sleep(1);
+      }
+      if (own && lane == 0) {
+        __hip_atomic_store(hl.totals + task, part + (wv & ((1u << FX_HEAD_STATUS_BITS) - 1u)), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+        s_told = 1u;
+      }
+    }
+  };
+  // ---- requests: objectness of the chunk (wave 0), first look at the earlier chunks (wave 1),
+  // rows of the first sub-tile (everybody).  In a launch that floods the memory system
+  // (hl.bulk_delay) the waves that carry no gather hold their requests back for a moment: the
+  // counts, a few bytes per row that every later workgroup of the image waits for, then reach the
+  // memory system ahead of the bulk instead of somewhere in a queue of tens of megabytes.
+  float o[NSUB];
+  if (wave == 0) {
+#pragma unroll
+    for (uint32_t j = 0; j < NSUB; ++j) {
+      const uint32_t r = j * 64u + lane;
+      o[j] = r < c_rows ? pred[(size_t)(c_r0 + r) * S + 4u] : 0.0f;
+    }
+  } else {
+    if (wave == 1) {
+      if (lane == 0) s_told = 0u;
+#pragma unroll
+      for (uint32_t j = 0; j < 2; ++j)
+        if (j * 64u + lane < chunk)
+          pw[j] = __hip_atomic_load(hl.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    for (uint32_t d = 0; d < hl.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
+    // (big launches: by now the earlier chunks have published; the image's total leaves for the
+    // host before this wave waits for any row)
+    if (wave == 1 && hl.bulk_delay != 0u) look_back();
+  }
   request(0);
 
   // ---- kept flags and count of the chunk; published at once
@@ -124,25 +175,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
       const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
       if (keep) s_rowmap[__popcll(bal & ((1ull << lane) - 1ull))] = lane;
       if (lane == 0) s_nk = (uint32_t)__popcll(bal);
-    } else if (wave == 1 && s == 0) {
-      // one look-back per workgroup
-      const uint32_t first = b - chunk;
-      uint32_t part = 0;
-      bool ok = true;
-      for (uint32_t i = lane; i < chunk; i += 64u) {
-        uint32_t wv = i < 64u ? pw[0] : (i < 128u ? pw[1] : 0u), polls = 0;
-        while ((wv >> FX_HEAD_STATUS_BITS) != hl.epoch) {
-          if (polls >= hl.spin_limit) { ok = false; break; }
-          ++polls;
-          __builtin_amdgcn_s_sleep(1);
-          wv = __hip_atomic_load(hl.status + first + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        part += ok ? (wv & ((1u << FX_HEAD_STATUS_BITS) - 1u)) : 0u;
-      }
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
-      const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
-      if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
+    } else if (wave == 1 && s == 0 && hl.bulk_delay == 0u) {
+      look_back();
     }
     __syncthreads();
     if (s == 0) {
@@ -164,10 +198,9 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
         __syncthreads();
       }
       prefix = uni(s_prefix);
-      // The host polls this word while the kernel still runs: a system-scope store goes through
-      // to host memory instead of waiting in L2 for the end of the kernel.
-      if (chunk + 1u == hl.chunks && threadIdx.x == 0)
-        __hip_atomic_store(hl.totals + task, prefix + uni(s_total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      // (the total of the image, unless wave 1 has told the host already)
+      if (chunk + 1u == hl.chunks && threadIdx.x == 0 && s_told == 0u)
+        __hip_atomic_store(hl.totals + task, prefix + s_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     const uint32_t n_kept = uni(s_nk);
     const uint32_t* W = L + sh;

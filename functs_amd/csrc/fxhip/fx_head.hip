@@ -94,9 +94,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
     for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
     const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
     if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
-    // The image's last chunk tells the host the image's total as soon as it is known, before
-    // any of its rows has arrived: its own count comes from its status word (wave 0 publishes
-    // it right after the gather).  The host polls the word while the kernel still runs: a
+    // The image's last chunk tells the host the image's total as soon as it is known: its own
+    // count comes from its status word (wave 0 publishes it right after the gather).  The host polls the word while the kernel still runs: a
     // system-scope store goes through to host memory instead of waiting in L2 for the end of
     // the kernel.
     if (chunk + 1u == hl.chunks && all_ok) {
@@ -137,9 +136,6 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
           pw[j] = __hip_atomic_load(hl.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     for (uint32_t d = 0; d < hl.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
-    // (big launches: by now the earlier chunks have published; the image's total leaves for the
-    // host before this wave waits for any row)
-    if (wave == 1 && hl.bulk_delay != 0u) look_back();
   }
   request(0);
 
@@ -175,7 +171,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
       const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
       if (keep) s_rowmap[__popcll(bal & ((1ull << lane) - 1ull))] = lane;
       if (lane == 0) s_nk = (uint32_t)__popcll(bal);
-    } else if (wave == 1 && s == 0 && hl.bulk_delay == 0u) {
+    } else if (wave == 1 && s == 0) {
       look_back();
     }
     __syncthreads();

@@ -700,7 +700,16 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                                 ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
   }
   FxLaunchInfo li = launch_info(pl);
-  bool head = head_fits(pl);
+  // The one-launch forms tag their status words with the call's epoch, which travels in the
+  // kernel arguments: a captured launch would be replayed with the epoch of the capture and read
+  // the counts of an earlier replay.  Under stream capture the two-pass form is recorded instead.
+  hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap_status) != hipSuccess) {
+    (void)hipGetLastError();
+    cap_status = hipStreamCaptureStatusNone;
+  }
+  const bool capturing = cap_status != hipStreamCaptureStatusNone;
+  bool head = !capturing && head_fits(pl);
   FxHeadLaunch hl;
   void* status = nullptr;
   uint32_t epoch = 0;
@@ -714,7 +723,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     hl.status = (uint32_t*)hstatus;
     hl.totals = totals_host;
   }
-  bool streaming = !head && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
+  bool streaming = !head && !capturing && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
   if (streaming) {
     rc = stream_status(reg, pl, stream, dev, &status, &epoch, repeat);
     if (rc != FX_OK) return rc;

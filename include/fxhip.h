@@ -195,8 +195,10 @@ void fx_set_stream_spin_limit(uint32_t polls);
  * in the one-pass form above, with the same poll limit).  The programs are compared instruction
  * by instruction (any number of rows, images and classes C with C % 4 == 0, any threshold); a
  * region that differs anywhere keeps the generic kernels.  Results are bit-identical to those.
- * fx_set_head_kernel: process-wide switch, default on (FXHIP_HEAD=0: off; also off while
- * fx_set_specialization(0) holds).  fx_plan_head_info: out[0..8) = region recognised, kernel
+ * A call recorded under stream capture takes the generic two passes (the one-launch forms tag
+ * their status words with an epoch that travels in the kernel arguments and would be frozen in
+ * the graph).  fx_set_head_kernel: process-wide switch, default on (FXHIP_HEAD=0: off; also off
+ * while fx_set_specialization(0) holds).  fx_plan_head_info: out[0..8) = region recognised, kernel
  * in use now, low and high word of the hash of the normalised programs, C, 5 + C, rows, images
  * (test hook).  This is where the reference compiles the subgraph of the loop body with NVRTC
  * (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1414) and leaves x[mask] to ATen

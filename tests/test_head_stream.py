@@ -188,3 +188,40 @@ def test_predictions_that_start_at_an_odd_address():
     ref = r(pred.to(dev), anchors.to(dev), strides.to(dev))
     torch.cuda.synchronize()
     assert_exact([t.cpu() for t in got], [t.cpu() for t in ref], "odd start")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,classes,batch", [(100000, 4, None), (300000, 4, None), (60000, 8, 16)])
+def test_long_images_and_launches_beyond_what_the_device_holds_at_once(n, classes, batch):
+    """More than 128 chunks per image (the look-back polls the later words one round at a time) and
+    more workgroups than are resident together (later workgroups wait only for earlier ones)."""
+    args = _inputs(n, classes, batch or 1, seed=3)
+    one, two = _both(_head(batch=batch), *args)
+    assert_exact(one, two, "n=%d classes=%d batch=%s" % (n, classes, batch))
+
+
+@pytest.mark.gpu
+def test_replays_of_a_captured_call():
+    """A call recorded into a HIP graph takes the two-pass form (the one-launch form's epoch would
+    be frozen in the recorded arguments); every replay must follow its inputs."""
+    dev = torch.device("cuda:0")
+    n, classes, batch = 700, 80, 2
+    r = _head(batch=batch)
+    pred, anchors, strides = [t.to(dev) for t in _inputs(n, classes, batch, seed=0)]
+    bc = r.bind(pred, anchors, strides)
+    bc.launch()                       # descriptor upload and allocations happen here, not under capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        bc.launch()
+    for seed in (1, 2, 3):
+        new = _inputs(n, classes, batch, seed=seed)[0]
+        if seed == 2:
+            new[0, :, 4] = -20.0      # nothing kept in image 0
+        pred.copy_(new.to(dev))
+        ref = r(pred.clone(), anchors, strides)      # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = bc.results()
+        assert_exact([[t.cpu() for t in row] for row in got], [[t.cpu() for t in row] for row in ref], "replay %d" % seed)

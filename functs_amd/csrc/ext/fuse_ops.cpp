@@ -841,6 +841,62 @@ void splitIn(Block* b) {
 void SplitParallelMaps(std::shared_ptr<Graph> graph) { splitIn(graph->block()); }
 
 // ---------------------------------------------------------------------------
+// CanonicalizeFusableMaps (fait/passes/parallelize_loops.cpp:458-502): a map whose body is one
+// fusion group takes the group's arguments in one order, whatever the order in which the body
+// used them: the map index first (added when the body does not use it), then the map's own
+// parameters in their order, then what the group takes from outside; the map returns the group's
+// results in the group's order.
+// ---------------------------------------------------------------------------
+namespace {
+void canonicalizeMapsIn(Block* b) {
+  for (Node* n : b->nodes()) {
+    for (Block* inner : n->blocks()) canonicalizeMapsIn(inner);
+    if (n->kind() != sym::ParallelMap()) continue;
+    Block* mb = n->blocks()[0];
+    if (mb->nodes().begin() == mb->nodes().end()) continue;
+    Node* group = *mb->nodes().begin();
+    if (group->kind() != prim::FusionGroup || group->blocks().empty()) continue;
+    Block* gb = group->blocks()[0];
+    // every parameter of the map is one argument of the group, and nothing else uses it
+    bool plain = true;
+    for (Value* p : mb->inputs()) {
+      if (p == mb->inputs()[0] && !p->hasUses()) continue;
+      plain = plain && p->uses().size() == 1 && p->uses()[0].user == group;
+    }
+    if (!plain) continue;
+    std::vector<size_t> perm;
+    Value* index = mb->inputs()[0];
+    if (index->hasUses()) {
+      perm.push_back(index->uses()[0].offset);
+    } else {
+      group->insertInput(0, index);
+      gb->insertInput(0)->setType(c10::IntType::get());
+      perm.push_back(0);
+    }
+    for (size_t k = 1; k < mb->inputs().size(); ++k) perm.push_back(mb->inputs()[k]->uses()[0].offset);
+    for (size_t k = 0; k < group->inputs().size(); ++k)
+      if (!std::count(perm.begin(), perm.end(), k)) perm.push_back(k);
+    group->permuteInputs(perm);
+    gb->permuteInputs(perm);
+    // results: only when every result of the group is returned once by the map (a group that
+    // compacts rows keeps its row mask to itself)
+    std::vector<size_t> ret;
+    bool all_returned = group->outputs().size() == mb->outputs().size();
+    for (Value* out : group->outputs()) {
+      all_returned = all_returned && out->uses().size() == 1 && out->uses()[0].user == mb->return_node();
+      if (all_returned) ret.push_back(out->uses()[0].offset);
+    }
+    if (all_returned) {
+      mb->permuteOutputs(ret);
+      n->permuteOutputs(ret);
+    }
+  }
+}
+}  // namespace
+
+void CanonicalizeFusableMaps(std::shared_ptr<Graph> graph) { canonicalizeMapsIn(graph->block()); }
+
+// ---------------------------------------------------------------------------
 // Validate
 // ---------------------------------------------------------------------------
 namespace {
@@ -897,6 +953,7 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   }
   FuseMaskedSelect(graph);
   SplitParallelMaps(graph);
+  CanonicalizeFusableMaps(graph);   // fait_pipeline.cpp:61
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
   Validate(graph);

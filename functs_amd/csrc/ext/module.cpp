@@ -27,6 +27,7 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_tensorssa_remove_update", TensorSSARemoveUpdate);
   m.def("_jit_pass_convert_to_tensorssa", ConvertToTensorSSA);
   m.def("_jit_pass_fait_fuse_ops", FuseOps);
+  m.def("_jit_pass_fait_canonicalize_fusable_maps", CanonicalizeFusableMaps);
   m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
   m.def("_jit_pass_collapse_recurrent_loops", CollapseRecurrentLoops);
   m.def("_jit_pass_canonicalize_ops", CanonicalizeOps);

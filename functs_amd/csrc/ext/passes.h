@@ -40,6 +40,9 @@ bool HoistLoopInvariants(std::shared_ptr<torch::jit::Graph> graph);
 void ParallelizeLoops(std::shared_ptr<torch::jit::Graph> graph);
 // fait/passes/parallelize_loops.cpp:152-293: every fusion group of a map body gets a map of its own
 void SplitParallelMaps(std::shared_ptr<torch::jit::Graph> graph);
+// fait/passes/parallelize_loops.cpp:458-502: the group of a fusable map takes the map index, the
+// map's parameters in their order, then the values from outside; results in the group's order
+void CanonicalizeFusableMaps(std::shared_ptr<torch::jit::Graph> graph);
 // fait/passes/unroll_loops.cpp:11-77, parallelize_loops.cpp:372-456; true if the graph changed
 bool UnrollLoopsWithDeps(std::shared_ptr<torch::jit::Graph> graph);
 bool UnrollSimpleMaps(std::shared_ptr<torch::jit::Graph> graph);

@@ -111,6 +111,29 @@ def build_c3_classes(n_fg=80):
     return r.finalize()
 
 
+def build_c3_fused(n_fg=80, thr=0.05, var_xy=0.1, var_wh=0.2, first=1):
+    """build_c3_decode and build_c3_classes as ONE ParallelMap over the classes whose body holds
+    the decode and the softmax as well (what the TorchScript route makes of c3 when it sinks the
+    dense producer into the class map).  The library runs it as one launch of its SSD head kernel;
+    lowered generically every task redoes the softmax."""
+    r = Region(parallel_degree=n_fg, is_parallel_map=True)
+    loc = r.tensor_input(torch.float32, 3)
+    conf = r.tensor_input(torch.float32, 3)
+    priors = r.tensor_input(torch.float32, 2)
+    l0 = loc.select(0, 0)
+    cxcy = priors.slice(1, 0, 2) + l0.slice(1, 0, 2) * var_xy * priors.slice(1, 2, None)
+    wh = priors.slice(1, 2, None) * (l0.slice(1, 2, None) * var_wh).exp()
+    boxes = r.op("FULL", r.int_list([r.op("SIZE", priors, 0), 4]), 0.0, dtype=torch.float32)
+    boxes = boxes.slice_rev(cxcy - wh / 2, 1, 0, 2)
+    boxes = boxes.slice_rev(cxcy + wh / 2, 1, 2, None)
+    scores = conf.select(0, 0).softmax(-1)
+    sc = scores.select(1, r.op("INT_ADD", r.task_index(), first))
+    r.output(boxes)
+    r.output(sc)
+    r.compact_rows(sc > thr)
+    return r.finalize()
+
+
 # shape for which `python -m functs_amd.aot` compiles the region below (its reduction extents are
 # part of the programs, so the compiled kernels serve this shape only)
 COLUMN_STANDARDIZE_SHAPE = (777, 12)

@@ -80,5 +80,11 @@ PYBIND11_MODULE(_C, m) {
     auto* fn = cu->create_function(c10::QualifiedName(name), std::move(graph));
     return torch::jit::StrongFunctionPtr(std::move(cu), fn);
   });
+  m.def("_functor_host_timing", functorHostTiming);
+  m.def("_functor_host_times", []() {
+    py::dict d;
+    for (const auto& kv : functorHostTimes()) d[py::str(kv.first)] = kv.second;
+    return d;
+  });
   m.def("_fxhip_library", []() { return functs::fxhipLibraryPath(); });
 }

@@ -58,6 +58,12 @@ void FuseMaskedSelect(std::shared_ptr<torch::jit::Graph> graph);
 // is_parallel_args, input_refine_types).
 void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
 
+// Host time of tssa::ParallelFunctor by section (flatten, plan, alloc, launch, views, wait_counts,
+// resize, push): switching on clears the sums; the read gives "calls" and the mean microseconds per
+// operator call of every section.
+void functorHostTiming(bool on);
+std::vector<std::pair<std::string, double>> functorHostTimes();
+
 // fait/passes/validate_graph.cpp:6-38: every use is dominated by its definition.
 void Validate(std::shared_ptr<torch::jit::Graph> graph);
 

@@ -20,6 +20,8 @@
 #include <torch/csrc/jit/passes/common_subexpression_elimination.h>
 #include <torch/csrc/jit/runtime/custom_operator.h>
 
+#include <atomic>
+#include <chrono>
 #include <map>
 #include <mutex>
 #include <sstream>
@@ -312,6 +314,26 @@ int checkAsyncError() {
   return e;
 }
 
+// Host time of the operator by section, summed over calls while switched on: where a call's
+// time goes between popping the arguments and pushing the results.
+enum HostSection { HS_FLATTEN, HS_PLAN, HS_ALLOC, HS_LAUNCH, HS_VIEWS, HS_WAIT, HS_RESIZE, HS_PUSH, HS_COUNT };
+const char* const kHostSectionNames[HS_COUNT] = {"flatten", "plan", "alloc", "launch", "views", "wait_counts", "resize", "push"};
+std::atomic<bool> g_host_timing{false};
+std::atomic<uint64_t> g_host_ns[HS_COUNT];
+std::atomic<uint64_t> g_host_calls{0};
+struct HostClock {
+  const bool on = g_host_timing.load(std::memory_order_relaxed);
+  std::chrono::steady_clock::time_point last;
+  HostClock() { if (on) last = std::chrono::steady_clock::now(); }
+  void tick(HostSection s) {
+    if (!on) return;
+    const auto now = std::chrono::steady_clock::now();
+    g_host_ns[s].fetch_add((uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(now - last).count(),
+                           std::memory_order_relaxed);
+    last = now;
+  }
+};
+
 // device scratch and the pinned landing zone of the kept-row counts; a call
 // borrows one and hands it back, so concurrent calls never share
 struct Workspace {
@@ -397,6 +419,7 @@ class RegionRunner {
       for (size_t o = 0; o < n_outs_; ++o) push(stack, c10::List<at::Tensor>());
       return;
     }
+    HostClock clock;
     // flatten arguments
     std::vector<fx_arg> args;
     std::vector<at::Tensor> keep;
@@ -478,6 +501,7 @@ class RegionRunner {
     }
     TORCH_CHECK(have_device, "ParallelFunctor: a region needs at least one tensor argument");
     c10::DeviceGuard guard(device);
+    clock.tick(HS_FLATTEN);
 
     Variant* var;
     {
@@ -526,6 +550,7 @@ class RegionRunner {
       std::lock_guard<std::mutex> lock(var->mu);
       layout = var->layouts.emplace(plan, std::move(lay)).first->second;
     }
+    clock.tick(HS_PLAN);
     typedef OutSlot Slot;
     std::vector<Slot> slots;   // a copy only where the kept-row counts change the sizes
     if (compact_) slots = layout->slots;
@@ -552,9 +577,11 @@ class RegionRunner {
       ws.stream = (void*)stream.stream();
     }
     checkAsyncError();
+    clock.tick(HS_ALLOC);
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
+    clock.tick(HS_LAUNCH);
     std::vector<std::vector<at::Tensor>> outs(n_out);
     for (int o = 0; o < n_out; ++o) {
       if (degree == 1) {
@@ -571,11 +598,13 @@ class RegionRunner {
         outs[o].emplace_back(std::move(impl));
       }
     }
+    clock.tick(HS_VIEWS);
     if (compact_) {
       // The kept-row counts decide the output shapes.  ATen's nonzero / masked index
       // synchronise the stream for that; here the counts arrive through pinned memory early
       // in the second pass, and the outputs are valid in stream order.
       FX_OK_OR_THROW(fx_region_wait_totals(plan, (const uint32_t*)ws.totals.data_ptr(), (void*)stream.stream()));
+      clock.tick(HS_WAIT);
       const int32_t* tot = ws.totals.data_ptr<int32_t>();
       for (int o = 0; o < n_out; ++o)
         for (int64_t t = 0; t < degree; ++t) {
@@ -585,11 +614,14 @@ class RegionRunner {
         }
       var->give(std::move(ws));
     }
+    clock.tick(HS_RESIZE);
     drop(stack, n_stack_);
     for (int o = 0; o < n_out; ++o) {
       if (is_map_) push(stack, c10::List<at::Tensor>(std::move(outs[o])));
       else push(stack, std::move(outs[o][0]));
     }
+    clock.tick(HS_PUSH);
+    if (clock.on) g_host_calls.fetch_add(1, std::memory_order_relaxed);
   }
 
  private:
@@ -1025,6 +1057,23 @@ RegisterOperators registerFunctor({
 }  // namespace
 
 void ToParallelFunctor(std::shared_ptr<Graph> graph) { toFunctorIn(graph->block()); }
+
+void functorHostTiming(bool on) {
+  if (on) {
+    for (auto& v : g_host_ns) v.store(0);
+    g_host_calls.store(0);
+  }
+  g_host_timing.store(on);
+}
+
+std::vector<std::pair<std::string, double>> functorHostTimes() {
+  std::vector<std::pair<std::string, double>> out;
+  const uint64_t calls = g_host_calls.load();
+  out.emplace_back("calls", (double)calls);
+  for (int s = 0; s < HS_COUNT; ++s)
+    out.emplace_back(kHostSectionNames[s], calls ? (double)g_host_ns[s].load() / 1e3 / (double)calls : 0.0);
+  return out;
+}
 
 std::string fxhipLibraryPath() { return "functs_amd/lib/libfxhip.so"; }
 

@@ -39,6 +39,11 @@ bool fx_spec_has_stream(const FxSpecKernels* spec);
 hipError_t fx_launch_head_stream(const FxHeadLaunch& hl, const FxDyn* dyn, hipStream_t stream);
 hipError_t fx_head_resident(uint32_t lds_bytes, uint32_t* workgroups, uint32_t* per_cu);
 uint32_t fx_head_lds_bytes(const FxHeadLaunch& hl);
+// fx_cmap.hip
+hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, hipStream_t stream);
+hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* workgroups);
+uint32_t fx_cmap_lds_bytes(const FxCmapLaunch& hl);
+uint32_t fx_cmap_chunk_rows();
 #include "fx_lstm_sched.h"
 int fx_launch_lstm_stack(const FxLstmArgs& a, int L, hipStream_t stream);
 int fx_launch_sort_nms(const fx_nms_desc& d, uint32_t key_cap, void* workspace, uint32_t* err_host, hipStream_t stream);
@@ -360,10 +365,26 @@ static bool head_active(const fx::Plan* pl) {
   return pl->mode == FX_MODE_COMPACT && pl->head.ok && g_head_mode.load(std::memory_order_relaxed) != 0 &&
          g_specialize.load(std::memory_order_relaxed) != 0;
 }
+static bool cmap_active(const fx::Plan* pl) {
+  return pl->mode == FX_MODE_COMPACT && pl->cmap.ok && g_head_mode.load(std::memory_order_relaxed) != 0 &&
+         g_specialize.load(std::memory_order_relaxed) != 0;
+}
 void fx_set_head_kernel(int on) { g_head_mode.store(on ? 1 : 0, std::memory_order_relaxed); }
 int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
   if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_head_info: out[>=8] required");
   const FxHeadInfo& hi = P(p)->head;
+  const FxCmapInfo& ci = P(p)->cmap;
+  if (ci.ok || (!hi.ok && ci.norm_hash && !hi.norm_hash)) {
+    out[0] = ci.ok ? 2 : 0;
+    out[1] = cmap_active(P(p)) ? 1 : 0;
+    out[2] = (int64_t)(ci.norm_hash & 0xffffffffull);
+    out[3] = (int64_t)(ci.norm_hash >> 32);
+    out[4] = ci.n_tasks;
+    out[5] = ci.C;
+    out[6] = ci.n_rows;
+    out[7] = ci.first;
+    return FX_OK;
+  }
   out[0] = hi.ok ? 1 : 0;
   out[1] = head_active(P(p)) ? 1 : 0;
   out[2] = (int64_t)(hi.norm_hash & 0xffffffffull);
@@ -376,12 +397,12 @@ int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
 }
 int fx_plan_launches(const fx_plan* p) {
   if (!p) return 0;
-  if (head_active(P(p))) return 1;
+  if (head_active(P(p)) || cmap_active(P(p))) return 1;
   if (P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) return P(p)->stream.grid > 0 ? 1 : 0;
   return P(p)->launches;
 }
 int fx_plan_streaming(const fx_plan* p) {
-  return (p && P(p)->mode == FX_MODE_COMPACT && !head_active(P(p)) && stream_active(P(p), spec_of(P(p)))) ? 1 : 0;
+  return (p && P(p)->mode == FX_MODE_COMPACT && !head_active(P(p)) && !cmap_active(P(p)) && stream_active(P(p), spec_of(P(p)))) ? 1 : 0;
 }
 int fx_plan_stream_info(const fx_plan* p, int64_t* out, int cap) {
   if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_stream_info: out[>=8] required");
@@ -573,7 +594,7 @@ static uint32_t stream_grid(const fx::Plan* pl) { return std::min<uint32_t>(pl->
 // Status words of `pl` for launches on `stream` (created on first use, at most four streams per
 // plan: calls on further streams take the two-pass form) and the epoch of the next call.
 static int status_words(fx_region* reg, std::vector<fx::Plan::Status>& list, size_t words, hipStream_t stream, int dev,
-                        void** ptr, uint32_t* epoch, int n_epochs) {
+                        void** ptr, uint32_t* epoch, int n_epochs, uint32_t epoch_max = FX_EPOCH_MAX) {
   std::lock_guard<std::mutex> g(reg->mu);
   fx::Plan::Status* st = nullptr;
   for (auto& s : list)
@@ -587,7 +608,7 @@ static int status_words(fx_region* reg, std::vector<fx::Plan::Status>& list, siz
     list.push_back({(void*)stream, d, 0u, dev});
     st = &list.back();
   }
-  if (st->epoch + (uint32_t)n_epochs >= FX_EPOCH_MAX) {
+  if (st->epoch + (uint32_t)n_epochs >= epoch_max) {
     // the tags wrap: clear the words behind everything already queued on the stream
     HIP_OK(hipMemsetAsync(st->ptr, 0, bytes, stream));
     st->epoch = 0;
@@ -664,6 +685,45 @@ static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
   return FX_OK;
 }
 
+// ---- class-map head kernel (fx_cmap.h): geometry of a launch ----
+#define FX_CMAP_EPOCH_MAX 0xffffu   // the epoch tag of its 64-bit status words has 16 bits
+static size_t cmap_status_words(const FxCmapInfo& ci) {
+  const uint32_t chunks = (ci.n_rows + fx_cmap_chunk_rows() - 1) / fx_cmap_chunk_rows();
+  return (size_t)chunks * ((ci.n_tasks + 7u) / 8u) * 2u;
+}
+// One workgroup per chunk of rows; the kernel is chosen only when the device holds all of them
+// at once (a workgroup waits for the counts of the chunks before its own).
+static int cmap_launch_info(fx::Plan* pl, FxCmapLaunch* hl, bool* fits) {
+  const FxCmapInfo& ci = pl->cmap;
+  memset(hl, 0, sizeof(*hl));
+  hl->n_rows = ci.n_rows;
+  hl->n_tasks = ci.n_tasks;
+  hl->chunk_rows = fx_cmap_chunk_rows();
+  hl->chunks = (ci.n_rows + hl->chunk_rows - 1) / hl->chunk_rows;
+  hl->C = ci.C;
+  hl->first = ci.first;
+  hl->thr_bits = ci.thr_bits;
+  hl->var_xy_bits = ci.var_xy_bits;
+  hl->var_wh_bits = ci.var_wh_bits;
+  hl->spin_limit = g_stream_spin.load(std::memory_order_relaxed);
+  hl->n_sptr = (uint32_t)pl->sptr.size();
+  hl->n_tptr = (uint32_t)pl->tptr.size();
+  hl->conf_slot = ci.conf_slot;
+  hl->loc_slot = ci.loc_slot;
+  hl->pri_slot = ci.pri_slot;
+  for (int k = 0; k < 2; ++k) {
+    hl->out_slot[k] = ci.out_slot[k];
+    hl->out_tstride[k] = ci.out_tstride[k];
+  }
+  if (pl->head_resident == 0) {
+    uint32_t wg = 0;
+    HIP_OK(fx_cmap_resident(fx_cmap_lds_bytes(*hl), &wg));
+    pl->head_resident = std::max<uint32_t>(wg, 1u);
+  }
+  *fits = hl->chunks <= pl->head_resident;
+  return FX_OK;
+}
+
 static int upload_blob(fx_region* reg, fx::Plan* pl, int dev) {
   std::lock_guard<std::mutex> g(reg->mu);
   if (!pl->dev_blob || pl->dev_id != dev) {
@@ -723,7 +783,21 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     hl.status = (uint32_t*)hstatus;
     hl.totals = totals_host;
   }
-  bool streaming = !head && !capturing && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
+  bool cmap = !head && !capturing && cmap_active(pl);
+  FxCmapLaunch cl;
+  if (cmap) {
+    rc = cmap_launch_info(pl, &cl, &cmap);
+    if (rc != FX_OK) return rc;
+  }
+  if (cmap) {
+    void* cstatus = nullptr;
+    rc = status_words(reg, pl->head_status, cmap_status_words(pl->cmap), stream, dev, &cstatus, &epoch, repeat, FX_CMAP_EPOCH_MAX);
+    if (rc != FX_OK) return rc;
+    if (!cstatus) cmap = false;
+    cl.status = (uint32_t*)cstatus;
+    cl.totals = totals_host;
+  }
+  bool streaming = !head && !cmap && !capturing && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
   if (streaming) {
     rc = stream_status(reg, pl, stream, dev, &status, &epoch, repeat);
     if (rc != FX_OK) return rc;
@@ -742,9 +816,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                            ? FX_TOTAL_PENDING
                            : 0u;
   }
-  const int launches = head ? (hl.chunks * hl.n_tasks > 0 ? 1 : 0) : streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
+  const int launches = head ? (hl.chunks * hl.n_tasks > 0 ? 1 : 0) : cmap ? (cl.chunks > 0 ? 1 : 0) : streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
   g_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
-  if (spec || head) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
+  if (spec || head || cmap) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
   const bool timed = kernel_ms != nullptr;
@@ -767,6 +841,14 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     }
     HIP_OK(mark(1));
     nk = hl.chunks * hl.n_tasks > 0 ? 1 : 0;
+  } else if (cmap) {
+    HIP_OK(mark(0));
+    for (int r = 0; r < repeat; ++r) {
+      cl.epoch = epoch + (uint32_t)r;
+      HIP_OK(fx_launch_classmap_head(cl, &dyn, stream));
+    }
+    HIP_OK(mark(1));
+    nk = cl.chunks > 0 ? 1 : 0;
   } else if (streaming) {
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
@@ -837,13 +919,29 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     if (!hstatus) head = false;
     hl.status = (uint32_t*)hstatus;
   }
-  bool streaming = !head && compact && stream_active(pl, spec);
+  bool cmap = !head && compact && cmap_active(pl);
+  FxCmapLaunch cl;
+  if (cmap) {
+    int rc = cmap_launch_info(pl, &cl, &cmap);
+    if (rc != FX_OK) return rc;
+  }
+  if (cmap) {
+    if ((uint32_t)(rounds * n_sets) >= FX_CMAP_EPOCH_MAX)
+      return fail(FX_E_INVALID, "fx_region_run_timed_sets: at most 65534 launches of this kernel in one call");
+    void* cstatus = nullptr;
+    const int rc = status_words(reg, pl->head_status, cmap_status_words(pl->cmap), stream, dev, &cstatus, &epoch, rounds * n_sets,
+                                FX_CMAP_EPOCH_MAX);
+    if (rc != FX_OK) return rc;
+    if (!cstatus) cmap = false;
+    cl.status = (uint32_t*)cstatus;
+  }
+  bool streaming = !head && !cmap && compact && stream_active(pl, spec);
   if (streaming) {
     const int rc = stream_status(reg, pl, stream, dev, &status, &epoch, rounds * n_sets);
     if (rc != FX_OK) return rc;
     if (!status) streaming = false;
   }
-  if (which >= ((streaming || head) ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
+  if (which >= ((streaming || head || cmap) ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
   std::vector<FxDyn> dyn((size_t)n_sets);
   for (int i = 0; i < n_sets; ++i) {
     memset(&dyn[i], 0, sizeof(FxDyn));
@@ -865,6 +963,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
         hl.epoch = epoch + (uint32_t)(r * n_sets + i);
         hl.totals = totals_host[i];
         HIP_OK(fx_launch_head_stream(hl, &dyn[i], stream));
+      } else if (cmap) {
+        cl.epoch = epoch + (uint32_t)(r * n_sets + i);
+        cl.totals = totals_host[i];
+        HIP_OK(fx_launch_classmap_head(cl, &dyn[i], stream));
       } else if (streaming) {
         li.epoch = epoch + (uint32_t)(r * n_sets + i);
         li.total_units = pl->stream.grid;

@@ -1,0 +1,243 @@
+// fx_classmap_head: decode + per-class score filter of an SSD-style detection head in one launch
+// (see fx_cmap.h for what it stands in for and when it is chosen).
+//
+// A workgroup owns a CHUNK of 32 consecutive priors; the host launches it only when all
+// workgroups are resident together.
+//   1. Every half-wave takes four rows of class scores (a lane holds four consecutive floats,
+//      one 128-bit load per row) and computes their softmax with butterfly reductions inside the
+//      half-wave; the first 32 threads also decode the chunk's boxes.  Results stay in LDS.
+//   2. Per class, the rows above the threshold are one ballot (two classes per ballot: 32 rows
+//      each).  The chunk publishes its counts in status words of 64 bits: eight 6-bit counts and
+//      the call's epoch, so that one load brings eight classes of an earlier chunk.
+//   3. The write offset of the chunk for every class is the sum of the counts of the earlier
+//      chunks: all threads read those words (eight loads in flight per lane), polling the ones
+//      that are not there yet.  Every poll loop is bounded: when a word does not show up within
+//      spin_limit polls the workgroup computes the earlier chunks itself, so the kernel ends
+//      whatever the order in which workgroups are started.  The last chunk tells the host the
+//      totals as soon as it knows them (system-scope stores to pinned memory).
+//   4. Kept rows go to their compacted places: the score, and the box as one 128-bit store.
+// The arithmetic repeats the lowered programs operation for operation (fx_exp, fx_fmax, no
+// contraction; the reductions in the order of the row-per-wave-segment softmax of the dense
+// kernel), so the results are bit-identical to the generic kernels on the region split in two.
+// Status words belong to the library (zero when allocated, never reset between calls: a word
+// of an earlier call carries an older epoch).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+#include "fx_cmap.h"
+#include "fx_device.h"
+
+namespace {
+
+#define FX_CMAP_DYN_OFF sizeof(FxCmapLaunch)
+#define FX_CMAP_R 32u         // rows of a chunk
+#define FX_CMAP_RPH 4u        // rows per half-wave: FX_CMAP_R / 8
+#define FX_CMAP_BATCH 8u      // status words a lane asks for at once
+
+__device__ __forceinline__ uint64_t fxc_ptr(const FxCmapLaunch& hl, uint32_t slot, uint32_t task) {
+  const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
+  const uint64_t* gp = (const uint64_t*)(ka + FX_CMAP_DYN_OFF);
+  const uint32_t pi = (slot & FX_SLOT_TASK) ? hl.n_sptr + task * hl.n_tptr + (slot & 0xffffu) : (slot & 0xffffu);
+  return gp[pi];
+}
+
+__global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch hl, const FxDyn) {
+  constexpr uint32_t NT = FX_BLOCK, R = FX_CMAP_R, RPH = FX_CMAP_RPH, U = FX_CMAP_BATCH;
+  extern __shared__ __attribute__((aligned(16))) float s_y[];   // R rows of CP floats: the softmax of the chunk
+  __shared__ fx_u32x4 s_box[R];
+  __shared__ uint32_t s_cnt[FX_CMAP_MAX_TASKS], s_prefix[FX_CMAP_MAX_TASKS];
+  __shared__ uint32_t s_ok;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = uni(tid >> 6);
+  const uint32_t b = blockIdx.x;
+  const uint32_t C = hl.C, CP = C | 1u, T = hl.n_tasks, NG = (T + 7u) >> 3;
+  const float thr = u2f(hl.thr_bits), var_xy = u2f(hl.var_xy_bits), var_wh = u2f(hl.var_wh_bits);
+  const FX_AS1 float* conf = (const FX_AS1 float*)fxc_ptr(hl, hl.conf_slot, 0);
+  const FX_AS1 float* loc = (const FX_AS1 float*)fxc_ptr(hl, hl.loc_slot, 0);
+  const FX_AS1 float* pri = (const FX_AS1 float*)fxc_ptr(hl, hl.pri_slot, 0);
+  uint64_t* status = (uint64_t*)hl.status;
+
+  // ---- softmax (and boxes) of chunk cb into LDS; the counts per class into s_cnt.  With
+  // `publish` the counts also go to the chunk's status words.
+  auto compute_chunk = [&](uint32_t cb, bool boxes, bool publish) {
+    const uint32_t r0 = cb * R, rows = min(R, hl.n_rows - r0);
+    const uint32_t hw = tid >> 5, l = tid & 31u, c0 = l * 4u;
+    float x[RPH][4];
+#pragma unroll
+    for (uint32_t k = 0; k < RPH; ++k) {
+      const uint32_t row = hw + k * 8u;
+      const FX_AS1 float* src = conf + (size_t)(r0 + row) * C + c0;
+      if (row < rows && c0 + 3u < C) {
+        const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)src;
+        x[k][0] = u2f(v.x); x[k][1] = u2f(v.y); x[k][2] = u2f(v.z); x[k][3] = u2f(v.w);
+      } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) x[k][j] = (row < rows && c0 + j < C) ? src[j] : 0.0f;
+      }
+    }
+    fx_u32x4_a4 lv = {0u, 0u, 0u, 0u}, pv = {0u, 0u, 0u, 0u};
+    if (boxes && tid < rows) {
+      lv = *(const FX_AS1 fx_u32x4_a4*)(loc + (size_t)(r0 + tid) * 4u);
+      pv = *(const FX_AS1 fx_u32x4_a4*)(pri + (size_t)(r0 + tid) * 4u);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < RPH; ++k) {
+      const uint32_t row = hw + k * 8u;
+      float m = -__builtin_inff();
+#pragma unroll
+      for (uint32_t j = 0; j < 4; ++j)
+        if (c0 + j < C) m = fx_fmax(m, x[k][j]);
+#pragma unroll
+      for (int o = 16; o >= 1; o >>= 1) m = fx_fmax(m, __shfl_xor(m, o, 64));
+      float e[4], v = 0.0f;
+#pragma unroll
+      for (uint32_t j = 0; j < 4; ++j) {
+        e[j] = fx_exp(x[k][j] - m);
+        if (c0 + j < C) v = v + e[j];
+      }
+#pragma unroll
+      for (int o = 16; o >= 1; o >>= 1) v = v + __shfl_xor(v, o, 64);
+      if (row < rows) {
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+          if (c0 + j < C) s_y[row * CP + c0 + j] = e[j] / v;
+      }
+    }
+    if (boxes && tid < rows) {
+      const float l0 = u2f(lv.x), l1 = u2f(lv.y), l2 = u2f(lv.z), l3 = u2f(lv.w);
+      const float p0 = u2f(pv.x), p1 = u2f(pv.y), p2 = u2f(pv.z), p3 = u2f(pv.w);
+      // half sizes (p * exp(l * var_wh)) / 2, centres p + (l * var_xy) * p_size
+      const float hx = (p2 * fx_exp(l2 * var_wh)) / 2.0f, hy = (p3 * fx_exp(l3 * var_wh)) / 2.0f;
+      const float cx = p0 + (l0 * var_xy) * p2, cy = p1 + (l1 * var_xy) * p3;
+      fx_u32x4 ob;
+      ob.x = f2u(cx - hx); ob.y = f2u(cy - hy); ob.z = f2u(cx + hx); ob.w = f2u(cy + hy);
+      s_box[tid] = ob;
+    }
+    __syncthreads();
+    // counts: a wave takes groups of eight classes, two classes per ballot
+    const uint32_t row = lane & 31u, sub = lane >> 5;
+    for (uint32_t g = wave; g < NG; g += NT / 64u) {
+      uint64_t word = 0;
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t t = g * 8u + k * 2u + sub;
+        const bool keep = t < T && row < rows && s_y[row * CP + hl.first + t] > thr;
+        const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+        const uint32_t n0 = (uint32_t)__popc((uint32_t)bal), n1 = (uint32_t)__popc((uint32_t)(bal >> 32));
+        word |= ((uint64_t)n0 << (12u * k)) | ((uint64_t)n1 << (12u * k + 6u));
+        if (row == 0 && t < T) s_cnt[t] = sub ? n1 : n0;
+      }
+      if (publish && lane == 0)
+        __hip_atomic_store(status + (size_t)cb * NG + g, ((uint64_t)hl.epoch << 48) | word, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+
+  if (tid < FX_CMAP_MAX_TASKS) s_prefix[tid] = 0u;
+  if (tid == 0) s_ok = 1u;
+  compute_chunk(b, true, true);   // (its barrier also orders the two stores above)
+
+  // ---- look-back: thread (i0, g) sums the counts of classes 8g .. 8g+7 over chunks i0, i0 + rp, ...
+  {
+    const uint32_t g = tid % NG, i0 = tid / NG, rp = NT / NG;   // rp rows of status words side by side
+    uint32_t acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    bool ok = true;
+    if (i0 < rp) {
+      for (uint32_t ib = i0; ib < b; ib += rp * U) {
+        uint64_t w[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+          const uint32_t i = ib + u * rp;
+          w[u] = i < b ? __hip_atomic_load(status + (size_t)i * NG + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                       : ((uint64_t)hl.epoch << 48);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+          const uint32_t i = ib + u * rp;
+          uint32_t polls = 0;
+          while ((uint32_t)(w[u] >> 48) != hl.epoch) {
+            if (polls >= hl.spin_limit) { ok = false; break; }
+            ++polls;
+            __builtin_amdgcn_s_sleep(1);
+            w[u] = __hip_atomic_load(status + (size_t)i * NG + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          if (!ok) break;
+#pragma unroll
+          for (uint32_t k = 0; k < 8; ++k) acc[k] += (uint32_t)(w[u] >> (6u * k)) & 63u;
+        }
+        if (!ok) break;
+      }
+    }
+    if (!ok) s_ok = 0u;
+    if (i0 < rp && b > 0) {
+#pragma unroll
+      for (uint32_t k = 0; k < 8; ++k)
+        if (acc[k] != 0u) atomicAdd(&s_prefix[g * 8u + k], acc[k]);   // (entries behind the last class stay unused)
+    }
+  }
+  __syncthreads();
+  if (uni(s_ok) == 0u) {
+    // an earlier chunk has not reported in time: compute the earlier chunks here
+    __syncthreads();
+    if (tid < FX_CMAP_MAX_TASKS) s_prefix[tid] = 0u;
+    for (uint32_t cb = 0; cb < b; ++cb) {
+      __syncthreads();   // s_y and s_cnt of the round before are no longer read
+      compute_chunk(cb, false, false);
+      __syncthreads();
+      if (tid < T) s_prefix[tid] += s_cnt[tid];
+    }
+    __syncthreads();
+    compute_chunk(b, true, false);
+    __syncthreads();
+  }
+  // the totals, as soon as they are known
+  if (b + 1u == hl.chunks && tid < T)
+    __hip_atomic_store(hl.totals + tid, s_prefix[tid] + s_cnt[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+
+  // ---- kept rows to their compacted places
+  {
+    const uint32_t rows = min(R, hl.n_rows - b * R);
+    const uint32_t row = lane & 31u, sub = lane >> 5;
+    for (uint32_t g = wave; g < NG; g += NT / 64u) {
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t t = g * 8u + k * 2u + sub;
+        const float y = (t < T && row < rows) ? s_y[row * CP + hl.first + t] : 0.0f;
+        const bool keep = t < T && row < rows && y > thr;
+        const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+        if (keep) {
+          const uint32_t half = sub ? (uint32_t)(bal >> 32) : (uint32_t)bal;
+          const uint32_t dst = s_prefix[t] + (uint32_t)__popc(half & ((1u << row) - 1u));
+          FX_AS1 float* sc = (FX_AS1 float*)fxc_ptr(hl, hl.out_slot[0], t) + (size_t)hl.out_tstride[0] * t;
+          FX_AS1 float* bx = (FX_AS1 float*)fxc_ptr(hl, hl.out_slot[1], t) + (size_t)hl.out_tstride[1] * t;
+          sc[dst] = y;
+          *(FX_AS1 fx_u32x4_a4*)(bx + (size_t)dst * 4u) = s_box[row];
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+uint32_t fx_cmap_lds_bytes(const FxCmapLaunch& hl) { return FX_CMAP_R * (hl.C | 1u) * 4u; }
+uint32_t fx_cmap_chunk_rows() { return FX_CMAP_R; }
+
+// Workgroups of the kernel that the current device holds at once.
+hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* workgroups) {
+  int dev = 0, cus = 0, per_cu = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return e;
+  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)&fx_classmap_head, (int)FX_BLOCK, (size_t)lds_bytes);
+  if (e != hipSuccess) return e;
+  *workgroups = (uint32_t)std::max(per_cu, 1) * (uint32_t)std::max(cus, 1);
+  return hipSuccess;
+}
+
+hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, hipStream_t stream) {
+  if (hl.chunks == 0) return hipSuccess;
+  void* args[2] = {(void*)&hl, (void*)dyn};
+  return hipLaunchKernel((const void*)&fx_classmap_head, dim3(hl.chunks), dim3(FX_BLOCK), args, fx_cmap_lds_bytes(hl), stream);
+}

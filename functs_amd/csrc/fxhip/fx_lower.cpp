@@ -2297,6 +2297,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   }
   P->spec_key = spec_hash(*P);
   match_head(P.get());
+  match_classmap(P.get());
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;

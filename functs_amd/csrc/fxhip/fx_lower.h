@@ -18,6 +18,7 @@
 
 #include "../../../include/fxhip.h"
 #include "fx_bytecode.h"
+#include "fx_cmap.h"
 #include "fx_head.h"
 
 namespace fx {
@@ -106,6 +107,7 @@ struct Plan {
   bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
   StreamInfo stream;
   FxHeadInfo head;               // the plan is the decode + score filter of a detection head (fx_head.h)
+  FxCmapInfo cmap;               // the plan is the decode + per-class score filter of an SSD-style head (fx_cmap.h)
   bool uses_guard = false;       // some load checks int64 data against 32 bits and reports to the error word
   uint32_t n_temps = 0;
   int max_rank = 1;
@@ -133,6 +135,8 @@ struct Plan {
 
 // Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?
 void match_head(Plan* p);
+// Fills p->cmap: does the plan compute the decode + per-class score filter of an SSD-style head (fx_cmap_match.cpp)?
+void match_classmap(Plan* p);
 
 // Builds (or fetches from the cache) the plan of `r` for these arguments.
 const Plan* plan_region(Region& r, const fx_arg* args, int n_args);

@@ -37,7 +37,10 @@ HBM_PEAK_GBPS = 8000.0
 KERNEL_BATCH = 10   # launches of a kernel inside one event pair (see measure)
 
 
-def build_workload(name, dev):
+def build_workload(name, dev, fused=True):
+    """`fused`: c3 as ONE region (decode + softmax inside the class map, run by the library's SSD
+    head kernel), as the TorchScript route builds it; otherwise as the two regions of the
+    reference's pipeline (dense decode + softmax, then the class map) on the generic kernels."""
     import torch
     from functs_amd import configs
     from functs_amd.benchmark.inputs import INPUTS
@@ -59,7 +62,10 @@ def build_workload(name, dev):
         calls = [(configs.build_c5(16), G(*cpu_args))]
         desc = "c5 ParallelMap x16 YOLOv3-style post-proc [16,10647,85]"
     elif name == "c3":
-        calls = [(configs.build_c3_decode(), G(*cpu_args)), (configs.build_c3_classes(80), None)]
+        if fused:
+            calls = [(configs.build_c3_fused(80), G(*cpu_args))]
+        else:
+            calls = [(configs.build_c3_decode(), G(*cpu_args)), (configs.build_c3_classes(80), None)]
         desc = "c3 SSD300-style post-proc [1,8732,4]+[1,8732,81]"
     return desc, calls, cpu_args
 
@@ -73,10 +79,10 @@ class Workload:
     inputs, outputs and scratch (set 0 is the one the latency loops use; the others exist so
     that timed kernels can be rotated over more memory than the caches hold)."""
 
-    def __init__(self, name, dev, sets=1):
+    def __init__(self, name, dev, sets=1, fused=True):
         import torch
         self.name = name
-        self.desc, calls, self.cpu_args = build_workload(name, dev)
+        self.desc, calls, self.cpu_args = build_workload(name, dev, fused)
         self.calls = calls
         self.dev = dev
         self.sets = []
@@ -157,6 +163,8 @@ class Workload:
         (intermediates between two regions of one config count zero)."""
         import torch
         total = self.bound[0].plan.alg_bytes
+        if self.name == "c3":   # loc, conf and priors read once, whichever way the regions are cut
+            total = sum(a.numel() * a.element_size() for a in self.cpu_args)
         last = self.bound[-1]
         last.launch()
         outs = last.results()
@@ -196,12 +204,15 @@ def recorded_traffic(kernel, workload):
 
 
 def head_kernel_in_use(plan):
-    """Does a call of this plan run the hand-written detection-head kernel (fx_head_stream)?"""
+    """Does a call of this plan run one of the hand-written head kernels?  Its name
+    (fx_head_stream: YOLO-style heads; fx_classmap_head: SSD-style heads) or None."""
     import ctypes
     from functs_amd import _lib
     out = (ctypes.c_int64 * 8)()
     _lib.check(_lib.lib.fx_plan_head_info(plan.handle, out, 8))
-    return bool(out[1])
+    if not out[1]:
+        return None
+    return {1: "fx_head_stream", 2: "fx_classmap_head"}[int(out[0])]
 
 
 def copy_reference_ms(dev, nbytes, rounds=4):
@@ -375,7 +386,7 @@ def main():
 
     if args.cold_profile:
         from functs_amd.region import timed_sets
-        w = Workload(args.workload, dev)
+        w = Workload(args.workload, dev, fused=not args.no_head_kernel)
         n_sets = w.grow_cold()
         flush(dev)
         call_ms = [timed_sets([s[i] for s in w.sets], which=-1, rounds=args.cold_profile) for i in range(len(w.bound))]
@@ -386,7 +397,7 @@ def main():
         return
 
     def run_one(name, with_cpu):
-        w = Workload(name, dev)
+        w = Workload(name, dev, fused=not args.no_head_kernel)
         ms, kern, single = measure(w, args.steps, args.warmup)
         alg = w.algorithmic_bytes()
         # the same kernels with consecutive launches rotated over buffer sets that together
@@ -408,7 +419,7 @@ def main():
             "cold_bytes": n_sets * w.touched_bytes(),
             "launches_per_call": w.launches,
             "row_compaction": any(bc.plan.compact for bc in w.bound),
-            "head_kernel": any(head_kernel_in_use(bc.plan) for bc in w.bound),
+            "head_kernel": next((k for k in (head_kernel_in_use(bc.plan) for bc in w.bound) if k), None),
             "algorithmic_bytes": alg,
             "dominant_kernel_index": dom_i,
             "gbps_dominant_kernel": round(alg / (dom * 1e-3) / 1e9, 1),
@@ -418,9 +429,19 @@ def main():
             "frac_hbm_peak_call": frac(sum(cold_regions)),
             "frac_hbm_peak_call_warm": frac(sum(kern)),
         }
-        rec["compiled_kernels"] = all(bc.region.specialized(*bc.args) for bc in w.bound)
-        if rec["compiled_kernels"]:
-            # the same launches through the bytecode interpreter
+        if name == "c3" and rec["head_kernel"]:
+            # the two regions of the reference's pipeline on the generic kernels, for comparison
+            del w
+            w = Workload(name, dev, fused=False)
+            measure(w, 5, 3)
+            w.grow_cold()
+            split_cold, split_regions = w.cold_times_ms(rounds)
+            rec["split_regions_kernel_us"] = [round(k * 1e3, 2) for k in split_cold]
+            rec["split_regions_call_kernels_us"] = round(sum(split_regions) * 1e3, 2)
+            rec["split_regions_launches_per_call"] = w.launches
+        rec["compiled_kernels"] = rec["head_kernel"] is not None or all(bc.region.specialized(*bc.args) for bc in w.bound)
+        if all(bc.region.specialized(*bc.args) for bc in w.bound):
+            # the same launches through the bytecode interpreter (c3: of the two regions)
             aot.enable(False)
             _, ikern, _ = measure(w, max(args.steps // 4, 5), 3)
             aot.enable(True)
@@ -644,7 +665,7 @@ def main():
             per["c5_nms_tail"] = {"error": str(e)[:200]}
     cpu_us, cpu_n, cores = head.pop("cpu")
     dom_ms = head["kernel_us"][head["dominant_kernel_index"]] / 1e3
-    dom_kernel = "fx_head_stream" if head.get("head_kernel") else ("fx_compact_scatter" if head["row_compaction"] else "fx_region_dense")
+    dom_kernel = head.get("head_kernel") or ("fx_compact_scatter" if head["row_compaction"] else "fx_region_dense")
     copy_ms = copy_reference_ms(dev, head["algorithmic_bytes"])
     traffic, traffic_src = recorded_traffic(dom_kernel, args.workload)
     out = {

@@ -956,6 +956,10 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   CanonicalizeFusableMaps(graph);   // fait_pipeline.cpp:61
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
+  if (SinkProducersIntoMaps(graph)) {
+    ConstantPropagation(graph);
+    EliminateDeadCode(graph);
+  }
   Validate(graph);
 }
 

@@ -80,6 +80,8 @@ PYBIND11_MODULE(_C, m) {
     auto* fn = cu->create_function(c10::QualifiedName(name), std::move(graph));
     return torch::jit::StrongFunctionPtr(std::move(cu), fn);
   });
+  m.def("_jit_pass_sink_producers_into_maps", SinkProducersIntoMaps);
+  m.def("_set_sink_producers", setSinkProducers);
   m.def("_functor_host_timing", functorHostTiming);
   m.def("_functor_host_times", []() {
     py::dict d;

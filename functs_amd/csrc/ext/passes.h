@@ -58,6 +58,15 @@ void FuseMaskedSelect(std::shared_ptr<torch::jit::Graph> graph);
 // is_parallel_args, input_refine_types).
 void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
 
+// A plain functor whose results only feed a compacting map functor (as shared arguments) and size
+// queries sinks into the map, when the library then runs the merged region as one hand-written
+// kernel (SSD-style heads: decode + softmax, then one score filter per class); size queries on the
+// producer's results become constants of the static shapes.  The reference keeps the two functors
+// (fait/passes/te_op.cpp:135-236).  True if the graph changed; setSinkProducers(false) switches
+// the pass off for the process.
+bool SinkProducersIntoMaps(std::shared_ptr<torch::jit::Graph> graph);
+void setSinkProducers(bool on);
+
 // Host time of tssa::ParallelFunctor by section (flatten, plan, alloc, launch, views, wait_counts,
 // resize, push): switching on clears the sums; the read gives "calls" and the mean microseconds per
 // operator call of every section.

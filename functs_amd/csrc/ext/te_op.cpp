@@ -18,6 +18,8 @@
 #include <c10/core/DeviceGuard.h>
 #include <torch/csrc/jit/ir/constants.h>
 #include <torch/csrc/jit/passes/common_subexpression_elimination.h>
+#include <torch/csrc/jit/passes/constant_propagation.h>
+#include <torch/csrc/jit/passes/dead_code_elimination.h>
 #include <torch/csrc/jit/runtime/custom_operator.h>
 
 #include <atomic>
@@ -422,83 +424,10 @@ class RegionRunner {
     HostClock clock;
     // flatten arguments
     std::vector<fx_arg> args;
-    std::vector<at::Tensor> keep;
     std::ostringstream sig;
-    sig << degree;
     c10::Device device(c10::kCPU);
     bool have_device = false;
-    auto addTensor = [&](const at::Tensor& t) {
-      TORCH_CHECK(t.is_cuda(), "tssa::ParallelFunctor runs on the GPU only; got a ", t.device(), " tensor");
-      TORCH_CHECK(t.dim() <= FX_ARG_MAX_RANK, "tensor rank above ", FX_ARG_MAX_RANK);
-      if (!have_device) { device = t.device(); have_device = true; }
-      fx_arg a;
-      memset(&a, 0, sizeof(a));
-      a.kind = 0;
-      a.dtype = fxDtype(t.scalar_type());
-      a.ptr = t.data_ptr();
-      a.rank = (int32_t)t.dim();
-      for (int64_t d = 0; d < t.dim(); ++d) { a.sizes[d] = t.size(d); a.strides[d] = t.stride(d); }
-      args.push_back(a);
-      sig << "|t" << a.dtype << "r" << a.rank;
-    };
-    auto addScalar = [&](const c10::IValue& v) {
-      fx_arg a;
-      memset(&a, 0, sizeof(a));
-      if (v.isDouble()) { a.kind = 2; a.fval = v.toDouble(); sig << "|f"; }
-      else if (v.isBool()) { a.kind = 3; a.ival = v.toBool(); sig << "|b"; }
-      else if (v.isInt()) { a.kind = 1; a.ival = v.toInt(); sig << "|i"; }
-      else if (v.isDevice() || v.isNone()) { a.kind = 1; a.ival = 0; sig << "|d"; }  // placement only: outputs follow the tensors
-      else TORCH_CHECK(false, "ParallelFunctor: unsupported scalar argument ", v.tagKind());
-      args.push_back(a);
-    };
-    // A value that is itself a list or tuple of scalars (int[], float[], bool[], Tuple[int, ...];
-    // per task: List[List[int]], List[Tuple[int, int]] ..., graph_builder.cpp:736-857) travels as
-    // its elements; their number is part of the signature.  All tasks must agree on it.
-    auto addValue = [&](const c10::IValue& v, size_t k, int64_t* n_elems) {
-      if (v.isTensor()) { addTensor(v.toTensor()); return; }
-      if (v.isList() || v.isTuple()) {
-        const auto elems = v.isList() ? v.toListRef() : at::ArrayRef<c10::IValue>(v.toTupleRef().elements());
-        TORCH_CHECK(*n_elems < 0 || *n_elems == (int64_t)elems.size(), "ParallelFunctor: argument ", k,
-                    ": the tasks' lists differ in length");
-        if (*n_elems < 0) sig << "|L" << elems.size();
-        *n_elems = (int64_t)elems.size();
-        for (const c10::IValue& e : elems) {
-          TORCH_CHECK(!e.isTensor() && !e.isList() && !e.isTuple(), "ParallelFunctor: argument ", k,
-                      ": nested lists of this kind are not supported");
-          addScalar(e);
-        }
-        return;
-      }
-      addScalar(v);
-    };
-    for (size_t k = 0; k < n_args_; ++k) {
-      const c10::IValue& v = inputs[first + k];
-      const bool per_task = is_map_ && is_par_[k] != 0;
-      int64_t n_elems = -1;
-      if (per_task) {
-        TORCH_CHECK(v.isList(), "ParallelFunctor: argument ", k, " must be a list with one entry per task");
-        auto lst = v.toListRef();
-        TORCH_CHECK((int64_t)lst.size() >= degree, "ParallelFunctor: list argument ", k, " is shorter than the trip count");
-        // element-major: all tasks' first elements, then all second elements ... (one region input each)
-        if (degree > 0 && (lst[0].isList() || lst[0].isTuple())) {
-          const auto first_elems = lst[0].isList() ? lst[0].toListRef() : at::ArrayRef<c10::IValue>(lst[0].toTupleRef().elements());
-          const size_t n = first_elems.size();
-          sig << "|L" << n;
-          for (size_t e = 0; e < n; ++e)
-            for (int64_t t = 0; t < degree; ++t) {
-              const auto elems = lst[t].isList() ? lst[t].toListRef() : at::ArrayRef<c10::IValue>(lst[t].toTupleRef().elements());
-              TORCH_CHECK(elems.size() == n, "ParallelFunctor: argument ", k, ": the tasks' lists differ in length");
-              TORCH_CHECK(!elems[e].isTensor() && !elems[e].isList() && !elems[e].isTuple(), "ParallelFunctor: argument ",
-                          k, ": nested lists of this kind are not supported");
-              addScalar(elems[e]);
-            }
-        } else {
-          for (int64_t t = 0; t < degree; ++t) addValue(lst[t], k, &n_elems);
-        }
-      } else {
-        addValue(v, k, &n_elems);
-      }
-    }
+    flatten(inputs, first, degree, /*dry=*/false, args, sig, device, have_device);
     TORCH_CHECK(have_device, "ParallelFunctor: a region needs at least one tensor argument");
     c10::DeviceGuard guard(device);
     clock.tick(HS_FLATTEN);
@@ -624,6 +553,40 @@ class RegionRunner {
     if (clock.on) g_host_calls.fetch_add(1, std::memory_order_relaxed);
   }
 
+  // What the library makes of the region for arguments of these types (meta tensors stand for
+  // them; nothing runs): `kind` is the first word of fx_plan_head_info when that kernel is in
+  // use (0: the generic kernels), `shapes` the shapes of task 0's results.
+  void dryRun(const std::vector<c10::IValue>& samples, int64_t* kind, std::vector<std::vector<int64_t>>* shapes) {
+    TORCH_CHECK(samples.size() == n_stack_, "dryRun: argument count");
+    int64_t degree = degree_;
+    size_t first = 0;
+    if (degree_ < 0) {
+      degree = samples[0].toInt();
+      first = 1;
+    }
+    if (!is_map_) degree = 1;
+    TORCH_CHECK(degree >= 1, "dryRun: empty map");
+    std::vector<fx_arg> args;
+    std::ostringstream sig;
+    c10::Device device(c10::kCPU);
+    bool have_device = false;
+    flatten(samples, first, degree, /*dry=*/true, args, sig, device, have_device);
+    Variant var;
+    build(var, degree, samples, first);
+    const fx_plan* plan = nullptr;
+    FX_OK_OR_THROW(fx_region_plan(var.region, args.data(), (int)args.size(), &plan));
+    int64_t info[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    FX_OK_OR_THROW(fx_plan_head_info(plan, info, 8));
+    *kind = info[1] ? info[0] : 0;
+    shapes->clear();
+    for (int o = 0; o < fx_plan_num_outputs(plan); ++o) {
+      int32_t dt = 0, rank = 0;
+      int64_t sizes[FX_ARG_MAX_RANK];
+      FX_OK_OR_THROW(fx_plan_output(plan, o, 0, &dt, &rank, sizes));
+      shapes->emplace_back(sizes, sizes + rank);
+    }
+  }
+
  private:
   std::shared_ptr<Graph> graph_;
   std::vector<int64_t> is_par_;
@@ -632,6 +595,86 @@ class RegionRunner {
   size_t n_args_ = 0, n_stack_ = 0, n_outs_ = 0;
   std::mutex mu_;
   std::map<std::string, std::unique_ptr<Variant>> variants_;
+
+  // The arguments as the C ABI takes them (tensors by pointer, sizes and strides; lists and tuples
+  // of scalars as their elements) and the signature that selects the region variant.  `dry`:
+  // tensors stand for their types only (no device, no pointer).
+  void flatten(at::ArrayRef<c10::IValue> inputs, size_t first, int64_t degree, bool dry, std::vector<fx_arg>& args,
+               std::ostringstream& sig, c10::Device& device, bool& have_device) {
+    sig << degree;
+    auto addTensor = [&](const at::Tensor& t) {
+      TORCH_CHECK(dry || t.is_cuda(), "tssa::ParallelFunctor runs on the GPU only; got a ", t.device(), " tensor");
+      TORCH_CHECK(t.dim() <= FX_ARG_MAX_RANK, "tensor rank above ", FX_ARG_MAX_RANK);
+      if (!have_device) { device = t.device(); have_device = true; }
+      fx_arg a;
+      memset(&a, 0, sizeof(a));
+      a.kind = 0;
+      a.dtype = fxDtype(t.scalar_type());
+      a.ptr = dry ? nullptr : t.data_ptr();
+      a.rank = (int32_t)t.dim();
+      for (int64_t d = 0; d < t.dim(); ++d) { a.sizes[d] = t.size(d); a.strides[d] = t.stride(d); }
+      args.push_back(a);
+      sig << "|t" << a.dtype << "r" << a.rank;
+    };
+    auto addScalar = [&](const c10::IValue& v) {
+      fx_arg a;
+      memset(&a, 0, sizeof(a));
+      if (v.isDouble()) { a.kind = 2; a.fval = v.toDouble(); sig << "|f"; }
+      else if (v.isBool()) { a.kind = 3; a.ival = v.toBool(); sig << "|b"; }
+      else if (v.isInt()) { a.kind = 1; a.ival = v.toInt(); sig << "|i"; }
+      else if (v.isDevice() || v.isNone()) { a.kind = 1; a.ival = 0; sig << "|d"; }  // placement only: outputs follow the tensors
+      else TORCH_CHECK(false, "ParallelFunctor: unsupported scalar argument ", v.tagKind());
+      args.push_back(a);
+    };
+    // A value that is itself a list or tuple of scalars (int[], float[], bool[], Tuple[int, ...];
+    // per task: List[List[int]], List[Tuple[int, int]] ..., graph_builder.cpp:736-857) travels as
+    // its elements; their number is part of the signature.  All tasks must agree on it.
+    auto addValue = [&](const c10::IValue& v, size_t k, int64_t* n_elems) {
+      if (v.isTensor()) { addTensor(v.toTensor()); return; }
+      if (v.isList() || v.isTuple()) {
+        const auto elems = v.isList() ? v.toListRef() : at::ArrayRef<c10::IValue>(v.toTupleRef().elements());
+        TORCH_CHECK(*n_elems < 0 || *n_elems == (int64_t)elems.size(), "ParallelFunctor: argument ", k,
+                    ": the tasks' lists differ in length");
+        if (*n_elems < 0) sig << "|L" << elems.size();
+        *n_elems = (int64_t)elems.size();
+        for (const c10::IValue& e : elems) {
+          TORCH_CHECK(!e.isTensor() && !e.isList() && !e.isTuple(), "ParallelFunctor: argument ", k,
+                      ": nested lists of this kind are not supported");
+          addScalar(e);
+        }
+        return;
+      }
+      addScalar(v);
+    };
+    for (size_t k = 0; k < n_args_; ++k) {
+      const c10::IValue& v = inputs[first + k];
+      const bool per_task = is_map_ && is_par_[k] != 0;
+      int64_t n_elems = -1;
+      if (per_task) {
+        TORCH_CHECK(v.isList(), "ParallelFunctor: argument ", k, " must be a list with one entry per task");
+        auto lst = v.toListRef();
+        TORCH_CHECK((int64_t)lst.size() >= degree, "ParallelFunctor: list argument ", k, " is shorter than the trip count");
+        // element-major: all tasks' first elements, then all second elements ... (one region input each)
+        if (degree > 0 && (lst[0].isList() || lst[0].isTuple())) {
+          const auto first_elems = lst[0].isList() ? lst[0].toListRef() : at::ArrayRef<c10::IValue>(lst[0].toTupleRef().elements());
+          const size_t n = first_elems.size();
+          sig << "|L" << n;
+          for (size_t e = 0; e < n; ++e)
+            for (int64_t t = 0; t < degree; ++t) {
+              const auto elems = lst[t].isList() ? lst[t].toListRef() : at::ArrayRef<c10::IValue>(lst[t].toTupleRef().elements());
+              TORCH_CHECK(elems.size() == n, "ParallelFunctor: argument ", k, ": the tasks' lists differ in length");
+              TORCH_CHECK(!elems[e].isTensor() && !elems[e].isList() && !elems[e].isTuple(), "ParallelFunctor: argument ",
+                          k, ": nested lists of this kind are not supported");
+              addScalar(elems[e]);
+            }
+        } else {
+          for (int64_t t = 0; t < degree; ++t) addValue(lst[t], k, &n_elems);
+        }
+      } else {
+        addValue(v, k, &n_elems);
+      }
+    }
+  }
 
   void build(Variant& var, int64_t degree, at::ArrayRef<c10::IValue> inputs, size_t first);
 };
@@ -1054,9 +1097,196 @@ RegisterOperators registerFunctor({
              [](Stack& stack) { runLstmStack(stack); }, c10::AliasAnalysisKind::PURE_FUNCTION),
 });
 
+
+// ---------------------------------------------------------------------------
+// pass: a dense producer sinks into the class map that consumes it
+// ---------------------------------------------------------------------------
+std::atomic<bool> g_sink_producers{true};
+
+bool isPlainFunctor(const Node* n) {
+  return n->kind() == sym::ParallelFunctor() && n->i(sym::is_parallel_map()) == 0 &&
+         (!n->hasAttribute(sym::compact_rows()) || n->i(sym::compact_rows()) == 0);
+}
+
+// a meta tensor of a complete static type
+bool sampleOf(const c10::TypePtr& type, c10::IValue* out) {
+  auto tt = type->cast<c10::TensorType>();
+  if (!tt || !tt->scalarType()) return false;
+  auto sizes = tt->sizes().concrete_sizes();
+  if (!sizes) return false;
+  // a type without strides stands for the contiguous layout (another layout at run time gets its
+  // own plan, as always)
+  auto strides = tt->strides().concrete_sizes();
+  const auto options = at::TensorOptions().dtype(*tt->scalarType()).device(c10::kMeta);
+  *out = strides ? at::empty_strided(*sizes, *strides, options) : at::empty(*sizes, options);
+  return true;
+}
+
+// F1 = plain functor, F2 = compacting map functor that reads F1's results as shared arguments.
+// Returns true if the graph changed.
+bool trySink(Node* f2) {
+  Graph* g = f2->owningGraph();
+  const auto par2 = f2->is(sym::is_parallel_args());
+  const size_t first2 = f2->i(sym::parallel_degree()) < 0 ? 1 : 0;
+  Node* f1 = nullptr;
+  for (size_t k = first2; k < f2->inputs().size(); ++k) {
+    Node* p = f2->input(k)->node();
+    if (par2[k - first2] != 0 || !isPlainFunctor(p) || p->owningBlock() != f2->owningBlock()) continue;
+    if (f1 && p != f1) return false;
+    f1 = p;
+  }
+  if (!f1) return false;
+  for (Node* n : f1->g(c10::attr::Subgraph)->nodes())
+    if (n->kind() == sym::LstmStack() || n->kind() == sym::ForallSelectRev()) return false;
+  // F1's results may only feed F2 and size queries with a constant dimension
+  for (Value* o : f1->outputs())
+    for (const Use& u : o->uses()) {
+      if (u.user == f2) continue;
+      if (u.user->kind() == c10::aten::size && u.user->inputs().size() == 2 && constant_as<int64_t>(u.user->input(1))) continue;
+      return false;
+    }
+  // static types of F1's arguments, and what F1 returns for them
+  std::vector<c10::IValue> samples1;
+  for (const c10::TypePtr& t : f1->tys(sym::input_refine_types())) {
+    c10::IValue v;
+    if (!sampleOf(t, &v)) return false;
+    samples1.push_back(v);
+  }
+  if (samples1.size() != f1->inputs().size()) return false;
+  std::vector<std::vector<int64_t>> shapes1;
+  try {
+    int64_t kind1 = 0;
+    RegionRunner r1(f1);
+    r1.dryRun(samples1, &kind1, &shapes1);
+  } catch (const c10::Error&) {
+    return false;
+  }
+  if (shapes1.size() != f1->outputs().size()) return false;
+  // size queries on F1's results become constants (the pipeline works on static shapes)
+  bool changed = false;
+  for (size_t o = 0; o < f1->outputs().size(); ++o) {
+    const auto uses = f1->output(o)->uses();
+    for (const Use& u : uses) {
+      if (u.user == f2) continue;
+      int64_t d = *constant_as<int64_t>(u.user->input(1));
+      const int64_t rank = (int64_t)shapes1[o].size();
+      if (d < 0) d += rank;
+      if (d < 0 || d >= rank) return changed;
+      WithInsertPoint guard(u.user);
+      u.user->output()->replaceAllUsesWith(g->insertConstant(shapes1[o][d]));
+      u.user->destroy();
+      changed = true;
+    }
+  }
+  // the trip count: a constant, or a node of constants
+  int64_t degree = f2->i(sym::parallel_degree());
+  if (degree < 0) {
+    Value* len = f2->input(0);
+    auto c = constant_as<int64_t>(len);
+    if (!c && len->node()->kind() != c10::prim::Param) {
+      auto st = runNodeIfInputsAreConstant(len->node());
+      if (st && st->size() == 1 && (*st)[0].isInt()) c = (*st)[0].toInt();
+    }
+    if (!c) return changed;
+    degree = *c;
+  }
+  if (degree < 1) return changed;
+  // the merged functor: F1's arguments (shared), then F2's other arguments
+  Node* f = g->createWithSubgraph(sym::ParallelFunctor());
+  auto sub = f->g(c10::attr::Subgraph);
+  auto sub1 = f1->g(c10::attr::Subgraph);
+  auto sub2 = f2->g(c10::attr::Subgraph);
+  std::vector<int64_t> par;
+  std::vector<c10::TypePtr> types;
+  std::vector<c10::IValue> samples;
+  std::unordered_map<Value*, Value*> map1, map2;
+  Value* idx = sub->addInput()->setType(c10::IntType::get());
+  map2[sub2->inputs()[0]] = idx;
+  const auto types1 = f1->tys(sym::input_refine_types());
+  for (size_t k = 0; k < f1->inputs().size(); ++k) {
+    f->addInput(f1->input(k));
+    types.push_back(types1[k]);
+    par.push_back(0);
+    samples.push_back(samples1[k]);
+    map1[sub1->inputs()[k + 1]] = sub->addInput()->copyMetadata(sub1->inputs()[k + 1]);
+  }
+  {
+    // F1's placeholder for the task index
+    WithInsertPoint guard(sub->block());
+    map1[sub1->inputs()[0]] = sub->insertConstant(c10::IValue());
+  }
+  auto destroyMerged = [&]() { f->destroy(); };
+  const auto types2 = f2->tys(sym::input_refine_types());
+  for (size_t k = first2; k < f2->inputs().size(); ++k) {
+    Value* in = f2->input(k);
+    Value* p = sub2->inputs()[k - first2 + 1];
+    if (in->node() == f1) continue;   // bound below, once F1's nodes are in
+    c10::IValue v;
+    if (par2[k - first2] != 0 || !sampleOf(types2[k - first2], &v)) { destroyMerged(); return changed; }
+    f->addInput(in);
+    types.push_back(types2[k - first2]);
+    par.push_back(0);
+    samples.push_back(v);
+    map2[p] = sub->addInput()->copyMetadata(p);
+  }
+  std::vector<Value*> no_returns;
+  cloneBlockInto(sub1->block(), sub.get(), map1, &no_returns);
+  for (size_t k = first2; k < f2->inputs().size(); ++k) {
+    Value* in = f2->input(k);
+    if (in->node() == f1) map2[sub2->inputs()[k - first2 + 1]] = map1.at(sub1->outputs()[in->offset()]);
+  }
+  cloneBlockInto(sub2->block(), sub.get(), map2);
+  cseRegion(sub);
+  EliminateDeadCode(sub);
+  f->i_(sym::parallel_degree(), degree);
+  f->i_(sym::is_parallel_map(), 1);
+  f->i_(sym::compact_rows(), 1);
+  f->is_(sym::is_parallel_args(), par);
+  f->tys_(sym::input_refine_types(), types);
+  for (Value* out : f2->outputs()) f->addOutput()->copyMetadata(out);
+  // only when the library runs the merged region as one of its hand-written kernels: lowered
+  // generically every task would redo the producer
+  int64_t kind = 0;
+  try {
+    std::vector<std::vector<int64_t>> shapes;
+    RegionRunner rm(f);
+    rm.dryRun(samples, &kind, &shapes);
+  } catch (const c10::Error&) {
+    kind = 0;
+  }
+  if (kind == 0) { destroyMerged(); return changed; }
+  f->insertBefore(f2);
+  for (size_t k = 0; k < f2->outputs().size(); ++k) f2->output(k)->replaceAllUsesWith(f->output(k));
+  f2->destroy();
+  f1->destroy();
+  return true;
+}
+
+bool sinkIn(Block* b) {
+  bool changed = false;
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) changed |= sinkIn(inner);
+    if (n->kind() != sym::ParallelFunctor() || n->i(sym::is_parallel_map()) == 0 || !n->hasAttribute(sym::compact_rows()) ||
+        n->i(sym::compact_rows()) == 0)
+      continue;
+    changed |= trySink(n);
+  }
+  return changed;
+}
+
 }  // namespace
 
 void ToParallelFunctor(std::shared_ptr<Graph> graph) { toFunctorIn(graph->block()); }
+
+bool SinkProducersIntoMaps(std::shared_ptr<Graph> graph) {
+  if (!g_sink_producers.load()) return false;
+  const bool changed = sinkIn(graph->block());
+  if (changed) EliminateDeadCode(graph);
+  return changed;
+}
+void setSinkProducers(bool on) { g_sink_producers.store(on); }
 
 void functorHostTiming(bool on) {
   if (on) {

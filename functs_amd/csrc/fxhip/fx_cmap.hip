@@ -10,8 +10,8 @@
 //      each).  The chunk publishes its counts in status words of 64 bits: eight 6-bit counts and
 //      the call's epoch, so that one load brings eight classes of an earlier chunk.
 //   3. The write offset of the chunk for every class is the sum of the counts of the earlier
-//      chunks: all threads read those words (eight loads in flight per lane), polling the ones
-//      that are not there yet.  Every poll loop is bounded: when a word does not show up within
+//      chunks: all threads read those words (twelve loads in flight per lane) and ask again,
+//      together, for the ones that are not there yet.  Every poll loop is bounded: when a word does not show up within
 //      spin_limit polls the workgroup computes the earlier chunks itself, so the kernel ends
 //      whatever the order in which workgroups are started.  The last chunk tells the host the
 //      totals as soon as it knows them (system-scope stores to pinned memory).
@@ -33,7 +33,7 @@ namespace {
 #define FX_CMAP_DYN_OFF sizeof(FxCmapLaunch)
 #define FX_CMAP_R 32u         // rows of a chunk
 #define FX_CMAP_RPH 4u        // rows per half-wave: FX_CMAP_R / 8
-#define FX_CMAP_BATCH 8u      // status words a lane asks for at once
+#define FX_CMAP_BATCH 12u     // status words a lane asks for at once
 
 __device__ __forceinline__ uint64_t fxc_ptr(const FxCmapLaunch& hl, uint32_t slot, uint32_t task) {
   const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
@@ -48,6 +48,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
   __shared__ fx_u32x4 s_box[R];
   __shared__ uint32_t s_cnt[FX_CMAP_MAX_TASKS], s_prefix[FX_CMAP_MAX_TASKS];
   __shared__ uint32_t s_ok;
+  __shared__ uint64_t s_sc[FX_CMAP_MAX_TASKS], s_bx[FX_CMAP_MAX_TASKS];   // where every task's scores and boxes go
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = uni(tid >> 6);
   const uint32_t b = blockIdx.x;
   const uint32_t C = hl.C, CP = C | 1u, T = hl.n_tasks, NG = (T + 7u) >> 3;
@@ -79,6 +80,14 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     if (boxes && tid < rows) {
       lv = *(const FX_AS1 fx_u32x4_a4*)(loc + (size_t)(r0 + tid) * 4u);
       pv = *(const FX_AS1 fx_u32x4_a4*)(pri + (size_t)(r0 + tid) * 4u);
+    }
+    // The argument segment lies in host memory: a load from it with an address that differs from
+    // lane to lane costs a trip over the bus.  Every task's destinations are fetched once, behind
+    // the loads of the scores (loads return in order), and parked in LDS after the softmax.
+    uint64_t q_sc = 0, q_bx = 0;
+    if (publish && tid < T) {
+      q_sc = fxc_ptr(hl, hl.out_slot[0], tid);
+      q_bx = fxc_ptr(hl, hl.out_slot[1], tid);
     }
 #pragma unroll
     for (uint32_t k = 0; k < RPH; ++k) {
@@ -113,6 +122,10 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
       ob.x = f2u(cx - hx); ob.y = f2u(cy - hy); ob.z = f2u(cx + hx); ob.w = f2u(cy + hy);
       s_box[tid] = ob;
     }
+    if (publish && tid < T) {
+      s_sc[tid] = q_sc + (uint64_t)hl.out_tstride[0] * tid * 4u;
+      s_bx[tid] = q_bx + (uint64_t)hl.out_tstride[1] * tid * 4u;
+    }
     __syncthreads();
     // counts: a wave takes groups of eight classes, two classes per ballot
     const uint32_t row = lane & 31u, sub = lane >> 5;
@@ -135,7 +148,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
 
   if (tid < FX_CMAP_MAX_TASKS) s_prefix[tid] = 0u;
   if (tid == 0) s_ok = 1u;
-  compute_chunk(b, true, true);   // (its barrier also orders the two stores above)
+  compute_chunk(b, true, true);   // (its barrier also orders the stores above)
 
   // ---- look-back: thread (i0, g) sums the counts of classes 8g .. 8g+7 over chunks i0, i0 + rp, ...
   {
@@ -143,29 +156,33 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     uint32_t acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
     bool ok = true;
     if (i0 < rp) {
-      for (uint32_t ib = i0; ib < b; ib += rp * U) {
+      for (uint32_t ib = i0; ib < b && ok; ib += rp * U) {
+        // The words of a batch are asked for together, and asked for again together as long as
+        // some of them still carry an older epoch: workgroups run in step, so the first look
+        // usually comes a moment before the neighbours' counts land.
         uint64_t w[U];
+        uint32_t pending = 0, polls = 0;
 #pragma unroll
-        for (uint32_t u = 0; u < U; ++u) {
-          const uint32_t i = ib + u * rp;
-          w[u] = i < b ? __hip_atomic_load(status + (size_t)i * NG + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                       : ((uint64_t)hl.epoch << 48);
-        }
+        for (uint32_t u = 0; u < U; ++u)
+          if (ib + u * rp < b) pending |= 1u << u;
+        while (pending) {
 #pragma unroll
-        for (uint32_t u = 0; u < U; ++u) {
-          const uint32_t i = ib + u * rp;
-          uint32_t polls = 0;
-          while ((uint32_t)(w[u] >> 48) != hl.epoch) {
+          for (uint32_t u = 0; u < U; ++u)
+            if ((pending >> u) & 1u)
+              w[u] = __hip_atomic_load(status + (size_t)(ib + u * rp) * NG + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (uint32_t u = 0; u < U; ++u)
+            if (((pending >> u) & 1u) && (uint32_t)(w[u] >> 48) == hl.epoch) {
+              pending &= ~(1u << u);
+#pragma unroll
+              for (uint32_t k = 0; k < 8; ++k) acc[k] += (uint32_t)(w[u] >> (6u * k)) & 63u;
+            }
+          if (pending) {
             if (polls >= hl.spin_limit) { ok = false; break; }
             ++polls;
-            __builtin_amdgcn_s_sleep(1);
-            w[u] = __hip_atomic_load(status + (size_t)i * NG + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_sleep(2);
           }
-          if (!ok) break;
-#pragma unroll
-          for (uint32_t k = 0; k < 8; ++k) acc[k] += (uint32_t)(w[u] >> (6u * k)) & 63u;
         }
-        if (!ok) break;
       }
     }
     if (!ok) s_ok = 0u;
@@ -208,8 +225,8 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
         if (keep) {
           const uint32_t half = sub ? (uint32_t)(bal >> 32) : (uint32_t)bal;
           const uint32_t dst = s_prefix[t] + (uint32_t)__popc(half & ((1u << row) - 1u));
-          FX_AS1 float* sc = (FX_AS1 float*)fxc_ptr(hl, hl.out_slot[0], t) + (size_t)hl.out_tstride[0] * t;
-          FX_AS1 float* bx = (FX_AS1 float*)fxc_ptr(hl, hl.out_slot[1], t) + (size_t)hl.out_tstride[1] * t;
+          FX_AS1 float* sc = (FX_AS1 float*)s_sc[t];
+          FX_AS1 float* bx = (FX_AS1 float*)s_bx[t];
           sc[dst] = y;
           *(FX_AS1 fx_u32x4_a4*)(bx + (size_t)dst * 4u) = s_box[row];
         }

@@ -143,7 +143,13 @@ def test_compiled_equals_interpreter_torchscript_route(name):
         aot.enable(True)
     assert len(fast) == len(slow)
     for x, y in zip(fast, slow):
-        assert x.shape == y.shape and torch.equal(x, y)
+        assert x.shape == y.shape
+        if name == "c3":
+            # one region (decode + softmax inside the class map): the hand-written kernel sums a
+            # row of scores across the lanes of a half-wave, the interpreter one by one per class
+            torch.testing.assert_close(x, y, rtol=1e-6, atol=1e-9)
+        else:
+            assert torch.equal(x, y)
 
 
 

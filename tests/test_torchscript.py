@@ -1,6 +1,8 @@
 """The TorchScript route: functs_amd.jit.script -> build (region formation ->
 tssa::ParallelFunctor).  CPU tests check the graphs; the gpu tests run the built
 functions on cuda:0 against stock TorchScript on the CPU (the oracle)."""
+from typing import List
+
 import pytest
 import torch
 
@@ -80,12 +82,66 @@ def test_c5_is_one_parallel_map_functor():
 
 
 def test_c3_is_decode_plus_class_map():
+    """As in the reference the pipeline makes a dense functor (decode + softmax) and a class map;
+    the last pass sinks the first into the second, because the library runs the merged region as
+    one kernel (its size query on the scores becomes the constant of the static shape)."""
     args = oc.c3_inputs(0, 60, 7)
-    f = _built("c3", args)
+    _C._set_sink_producers(False)
+    try:
+        f = _built("c3", args)
+    finally:
+        _C._set_sink_producers(True)
     fs = _functors(f.graph)
     assert [n.i("is_parallel_map") for n in fs] == [0, 1]
     assert [n.i("compact_rows") for n in fs] == [0, 1]
     assert "aten::softmax" in _kinds(fs[0].g("Subgraph"))
+    f = _built("c3", args)
+    fs = _functors(f.graph)
+    assert len(fs) == 1 and "aten::size" not in _kinds(f.graph)
+    n = fs[0]
+    assert n.i("is_parallel_map") == 1 and n.i("compact_rows") == 1 and n.i("parallel_degree") == 6
+    assert list(getattr(n, "is")("is_parallel_args")) == [0, 0, 0]
+    kinds = _kinds(n.g("Subgraph"))
+    assert "aten::softmax" in kinds and "immut::select" in kinds and kinds[-1] == "aten::gt"
+
+
+def test_a_producer_with_other_readers_is_not_sunk():
+    def g(loc: torch.Tensor, conf: torch.Tensor, priors: torch.Tensor):
+        l0 = loc[0]
+        cxcy = priors[:, :2] + l0[:, :2] * 0.1 * priors[:, 2:]
+        wh = priors[:, 2:] * torch.exp(l0[:, 2:] * 0.2)
+        boxes = torch.cat([cxcy - wh / 2, cxcy + wh / 2], 1)
+        scores = conf[0].softmax(-1)
+        out_b: List[torch.Tensor] = []
+        out_s: List[torch.Tensor] = []
+        for c in range(1, scores.size(1)):
+            sc = scores[:, c]
+            m = sc > 0.05
+            out_b.append(boxes[m])
+            out_s.append(sc[m])
+        return out_b, out_s, boxes      # the decoded boxes are a result of their own
+
+    def other_decode(loc: torch.Tensor, conf: torch.Tensor, priors: torch.Tensor):
+        # the producer only feeds the map, but the merged region is not one the library has a
+        # kernel for (boxes by cat, sigmoid scores): lowered generically every class would redo it
+        l0 = loc[0]
+        cxcy = priors[:, :2] + l0[:, :2] * 0.1 * priors[:, 2:]
+        wh = priors[:, 2:] * torch.exp(l0[:, 2:] * 0.2)
+        boxes = torch.cat([cxcy - wh / 2, cxcy + wh / 2], 1)
+        scores = conf[0].sigmoid()
+        out_b: List[torch.Tensor] = []
+        out_s: List[torch.Tensor] = []
+        for c in range(1, scores.size(1)):
+            sc = scores[:, c]
+            m = sc > 0.05
+            out_b.append(boxes[m])
+            out_s.append(sc[m])
+        return out_b, out_s
+
+    args = oc.c3_inputs(0, 60, 7)
+    for fn in (g, other_decode):
+        built = fj.build(fj.script(fn), list(args))
+        assert [n.i("is_parallel_map") for n in _functors(built.graph)] == [0, 1], fn.__name__
 
 
 def _mixed_body(x: torch.Tensor):
@@ -289,6 +345,16 @@ def test_c3_torchscript_gpu(n_priors, n_cls):
     gb, gs = _cpu(_built("c3", args)(*_cuda(args)))
     assert_close(gb, list(rb), "c3 boxes", rtol=1e-5, atol=1e-6)
     assert_close(gs, list(rs), "c3 scores")
+    # the two functors of the reference's pipeline give the same bits
+    _C._set_sink_producers(False)
+    try:
+        two = _built("c3", args)
+    finally:
+        _C._set_sink_producers(True)
+    assert len(_functors(two.graph)) == 2
+    tb, ts = _cpu(two(*_cuda(args)))
+    assert_exact(gb, tb, "c3 boxes, one functor vs two")
+    assert_exact(gs, ts, "c3 scores, one functor vs two")
 
 
 def test_c4_lstm_is_functionalized_and_keeps_its_loops():

@@ -40,8 +40,8 @@ hipError_t fx_launch_head_stream(const FxHeadLaunch& hl, const FxDyn* dyn, hipSt
 hipError_t fx_head_resident(uint32_t lds_bytes, uint32_t* workgroups, uint32_t* per_cu);
 uint32_t fx_head_lds_bytes(const FxHeadLaunch& hl);
 // fx_cmap.hip
-hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, hipStream_t stream);
-hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* workgroups);
+hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, bool wide, hipStream_t stream);
+hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* wide, uint32_t* narrow);
 uint32_t fx_cmap_lds_bytes(const FxCmapLaunch& hl);
 uint32_t fx_cmap_chunk_rows();
 #include "fx_lstm_sched.h"
@@ -693,7 +693,7 @@ static size_t cmap_status_words(const FxCmapInfo& ci) {
 }
 // One workgroup per chunk of rows; the kernel is chosen only when the device holds all of them
 // at once (a workgroup waits for the counts of the chunks before its own).
-static int cmap_launch_info(fx::Plan* pl, FxCmapLaunch* hl, bool* fits) {
+static int cmap_launch_info(fx::Plan* pl, FxCmapLaunch* hl, bool* fits, bool* wide) {
   const FxCmapInfo& ci = pl->cmap;
   memset(hl, 0, sizeof(*hl));
   hl->n_rows = ci.n_rows;
@@ -716,11 +716,13 @@ static int cmap_launch_info(fx::Plan* pl, FxCmapLaunch* hl, bool* fits) {
     hl->out_tstride[k] = ci.out_tstride[k];
   }
   if (pl->head_resident == 0) {
-    uint32_t wg = 0;
-    HIP_OK(fx_cmap_resident(fx_cmap_lds_bytes(*hl), &wg));
-    pl->head_resident = std::max<uint32_t>(wg, 1u);
+    uint32_t w = 0, n = 0;
+    HIP_OK(fx_cmap_resident(fx_cmap_lds_bytes(*hl), &w, &n));
+    pl->cmap_resident_wide = w;
+    pl->head_resident = std::max<uint32_t>(n, 1u);
   }
-  *fits = hl->chunks <= pl->head_resident;
+  *wide = hl->chunks <= pl->cmap_resident_wide;
+  *fits = *wide || hl->chunks <= pl->head_resident;
   return FX_OK;
 }
 
@@ -783,10 +785,10 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     hl.status = (uint32_t*)hstatus;
     hl.totals = totals_host;
   }
-  bool cmap = !head && !capturing && cmap_active(pl);
+  bool cmap = !head && !capturing && cmap_active(pl), cmap_wide = false;
   FxCmapLaunch cl;
   if (cmap) {
-    rc = cmap_launch_info(pl, &cl, &cmap);
+    rc = cmap_launch_info(pl, &cl, &cmap, &cmap_wide);
     if (rc != FX_OK) return rc;
   }
   if (cmap) {
@@ -845,7 +847,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
       cl.epoch = epoch + (uint32_t)r;
-      HIP_OK(fx_launch_classmap_head(cl, &dyn, stream));
+      HIP_OK(fx_launch_classmap_head(cl, &dyn, cmap_wide, stream));
     }
     HIP_OK(mark(1));
     nk = cl.chunks > 0 ? 1 : 0;
@@ -919,10 +921,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     if (!hstatus) head = false;
     hl.status = (uint32_t*)hstatus;
   }
-  bool cmap = !head && compact && cmap_active(pl);
+  bool cmap = !head && compact && cmap_active(pl), cmap_wide = false;
   FxCmapLaunch cl;
   if (cmap) {
-    int rc = cmap_launch_info(pl, &cl, &cmap);
+    int rc = cmap_launch_info(pl, &cl, &cmap, &cmap_wide);
     if (rc != FX_OK) return rc;
   }
   if (cmap) {
@@ -966,7 +968,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
       } else if (cmap) {
         cl.epoch = epoch + (uint32_t)(r * n_sets + i);
         cl.totals = totals_host[i];
-        HIP_OK(fx_launch_classmap_head(cl, &dyn[i], stream));
+        HIP_OK(fx_launch_classmap_head(cl, &dyn[i], cmap_wide, stream));
       } else if (streaming) {
         li.epoch = epoch + (uint32_t)(r * n_sets + i);
         li.total_units = pl->stream.grid;

@@ -2,15 +2,19 @@
 // (see fx_cmap.h for what it stands in for and when it is chosen).
 //
 // A workgroup owns a CHUNK of 32 consecutive priors; the host launches it only when all
-// workgroups are resident together.
-//   1. Every half-wave takes four rows of class scores (a lane holds four consecutive floats,
+// workgroups are resident together.  The work of a chunk is a chain of short dependent steps, so
+// the workgroup is wide (512 threads, two rows per half-wave: two waves on every SIMD hide each
+// other's latencies; with 1024 threads a CU took one workgroup only and the launch of 273 ran in
+// two rounds) or, when only that launch fits the device at once, 256 threads and four rows per
+// half-wave.
+//   1. Every half-wave takes its rows of class scores (a lane holds four consecutive floats,
 //      one 128-bit load per row) and computes their softmax with butterfly reductions inside the
 //      half-wave; the first 32 threads also decode the chunk's boxes.  Results stay in LDS.
 //   2. Per class, the rows above the threshold are one ballot (two classes per ballot: 32 rows
 //      each).  The chunk publishes its counts in status words of 64 bits: eight 6-bit counts and
 //      the call's epoch, so that one load brings eight classes of an earlier chunk.
 //   3. The write offset of the chunk for every class is the sum of the counts of the earlier
-//      chunks: all threads read those words (twelve loads in flight per lane) and ask again,
+//      chunks: all threads read those words (several loads in flight per lane) and ask again,
 //      together, for the ones that are not there yet.  Every poll loop is bounded: when a word does not show up within
 //      spin_limit polls the workgroup computes the earlier chunks itself, so the kernel ends
 //      whatever the order in which workgroups are started.  The last chunk tells the host the
@@ -28,12 +32,17 @@
 #include "fx_cmap.h"
 #include "fx_device.h"
 
+// a hook for timing the phases of a workgroup from a test program; nothing in the library
+#ifndef FX_CMAP_STAMP
+#define FX_CMAP_STAMP(k)
+#endif
+
 namespace {
 
 #define FX_CMAP_DYN_OFF sizeof(FxCmapLaunch)
 #define FX_CMAP_R 32u         // rows of a chunk
-#define FX_CMAP_RPH 4u        // rows per half-wave: FX_CMAP_R / 8
-#define FX_CMAP_BATCH 12u     // status words a lane asks for at once
+#define FX_CMAP_WIDE 512u     // threads of a workgroup: two rows per half-wave ...
+#define FX_CMAP_NARROW 256u   // ... or four rows per half-wave, when the device cannot hold the wide launch at once
 
 __device__ __forceinline__ uint64_t fxc_ptr(const FxCmapLaunch& hl, uint32_t slot, uint32_t task) {
   const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
@@ -42,8 +51,10 @@ __device__ __forceinline__ uint64_t fxc_ptr(const FxCmapLaunch& hl, uint32_t slo
   return gp[pi];
 }
 
-__global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch hl, const FxDyn) {
-  constexpr uint32_t NT = FX_BLOCK, R = FX_CMAP_R, RPH = FX_CMAP_RPH, U = FX_CMAP_BATCH;
+template <uint32_t NT>
+__global__ __launch_bounds__(NT) void fx_classmap_head(const FxCmapLaunch hl, const FxDyn) {
+  // RPH rows per half-wave; U status words a lane asks for at once
+  constexpr uint32_t R = FX_CMAP_R, RPH = R * 32u / NT, U = NT >= 512u ? 6u : 12u;
   extern __shared__ __attribute__((aligned(16))) float s_y[];   // R rows of CP floats: the softmax of the chunk
   __shared__ fx_u32x4 s_box[R];
   __shared__ uint32_t s_cnt[FX_CMAP_MAX_TASKS], s_prefix[FX_CMAP_MAX_TASKS];
@@ -66,7 +77,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     float x[RPH][4];
 #pragma unroll
     for (uint32_t k = 0; k < RPH; ++k) {
-      const uint32_t row = hw + k * 8u;
+      const uint32_t row = hw + k * (NT / 32u);
       const FX_AS1 float* src = conf + (size_t)(r0 + row) * C + c0;
       if (row < rows && c0 + 3u < C) {
         const fx_u32x4_a4 v = *(const FX_AS1 fx_u32x4_a4*)src;
@@ -89,27 +100,49 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
       q_sc = fxc_ptr(hl, hl.out_slot[0], tid);
       q_bx = fxc_ptr(hl, hl.out_slot[1], tid);
     }
+    if (publish) FX_CMAP_STAMP(6);
+    // The four rows of a half-wave go through every step together: their reductions are
+    // independent, so four lane exchanges are in flight at a time instead of one.
+    float m[RPH], v[RPH], e[RPH][4];
 #pragma unroll
     for (uint32_t k = 0; k < RPH; ++k) {
-      const uint32_t row = hw + k * 8u;
-      float m = -__builtin_inff();
+      m[k] = -__builtin_inff();
 #pragma unroll
       for (uint32_t j = 0; j < 4; ++j)
-        if (c0 + j < C) m = fx_fmax(m, x[k][j]);
+        if (c0 + j < C) m[k] = fx_fmax(m[k], x[k][j]);
+    }
 #pragma unroll
-      for (int o = 16; o >= 1; o >>= 1) m = fx_fmax(m, __shfl_xor(m, o, 64));
-      float e[4], v = 0.0f;
+    for (int o = 16; o >= 1; o >>= 1) {
+      float t[RPH];
+#pragma unroll
+      for (uint32_t k = 0; k < RPH; ++k) t[k] = __shfl_xor(m[k], o, 64);
+#pragma unroll
+      for (uint32_t k = 0; k < RPH; ++k) m[k] = fx_fmax(m[k], t[k]);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < RPH; ++k) {
+      v[k] = 0.0f;
 #pragma unroll
       for (uint32_t j = 0; j < 4; ++j) {
-        e[j] = fx_exp(x[k][j] - m);
-        if (c0 + j < C) v = v + e[j];
+        e[k][j] = fx_exp(x[k][j] - m[k]);
+        if (c0 + j < C) v[k] = v[k] + e[k][j];
       }
+    }
 #pragma unroll
-      for (int o = 16; o >= 1; o >>= 1) v = v + __shfl_xor(v, o, 64);
+    for (int o = 16; o >= 1; o >>= 1) {
+      float t[RPH];
+#pragma unroll
+      for (uint32_t k = 0; k < RPH; ++k) t[k] = __shfl_xor(v[k], o, 64);
+#pragma unroll
+      for (uint32_t k = 0; k < RPH; ++k) v[k] = v[k] + t[k];
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < RPH; ++k) {
+      const uint32_t row = hw + k * (NT / 32u);
       if (row < rows) {
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
-          if (c0 + j < C) s_y[row * CP + c0 + j] = e[j] / v;
+          if (c0 + j < C) s_y[row * CP + c0 + j] = e[k][j] / v[k];
       }
     }
     if (boxes && tid < rows) {
@@ -122,6 +155,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
       ob.x = f2u(cx - hx); ob.y = f2u(cy - hy); ob.z = f2u(cx + hx); ob.w = f2u(cy + hy);
       s_box[tid] = ob;
     }
+    if (publish) FX_CMAP_STAMP(1);
     if (publish && tid < T) {
       s_sc[tid] = q_sc + (uint64_t)hl.out_tstride[0] * tid * 4u;
       s_bx[tid] = q_bx + (uint64_t)hl.out_tstride[1] * tid * 4u;
@@ -131,10 +165,16 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     const uint32_t row = lane & 31u, sub = lane >> 5;
     for (uint32_t g = wave; g < NG; g += NT / 64u) {
       uint64_t word = 0;
+      float yk[4];
 #pragma unroll
       for (uint32_t k = 0; k < 4; ++k) {
         const uint32_t t = g * 8u + k * 2u + sub;
-        const bool keep = t < T && row < rows && s_y[row * CP + hl.first + t] > thr;
+        yk[k] = (t < T && row < rows) ? s_y[row * CP + hl.first + t] : -__builtin_inff();
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t t = g * 8u + k * 2u + sub;
+        const bool keep = t < T && row < rows && yk[k] > thr;
         const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
         const uint32_t n0 = (uint32_t)__popc((uint32_t)bal), n1 = (uint32_t)__popc((uint32_t)(bal >> 32));
         word |= ((uint64_t)n0 << (12u * k)) | ((uint64_t)n1 << (12u * k + 6u));
@@ -146,9 +186,11 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     }
   };
 
+  FX_CMAP_STAMP(0);
   if (tid < FX_CMAP_MAX_TASKS) s_prefix[tid] = 0u;
   if (tid == 0) s_ok = 1u;
-  compute_chunk(b, true, true);   // (its barrier also orders the stores above)
+  compute_chunk(b, true, true);
+  FX_CMAP_STAMP(2);   // (its barrier also orders the stores above)
 
   // ---- look-back: thread (i0, g) sums the counts of classes 8g .. 8g+7 over chunks i0, i0 + rp, ...
   {
@@ -193,6 +235,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
     }
   }
   __syncthreads();
+  FX_CMAP_STAMP(3);
   if (uni(s_ok) == 0u) {
     // an earlier chunk has not reported in time: compute the earlier chunks here
     __syncthreads();
@@ -211,28 +254,40 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
   if (b + 1u == hl.chunks && tid < T)
     __hip_atomic_store(hl.totals + tid, s_prefix[tid] + s_cnt[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 
+  FX_CMAP_STAMP(4);
   // ---- kept rows to their compacted places
   {
     const uint32_t rows = min(R, hl.n_rows - b * R);
     const uint32_t row = lane & 31u, sub = lane >> 5;
+    const fx_u32x4 box = s_box[row];
     for (uint32_t g = wave; g < NG; g += NT / 64u) {
+      // everything a class needs is read before the first store of the group is issued
+      float yk[4];
+      uint32_t pk[4];
+      uint64_t sk[4], bk[4];
+#pragma unroll
+      for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t t = min(g * 8u + k * 2u + sub, T - 1u);
+        yk[k] = s_y[min(row, rows - 1u) * CP + hl.first + t];
+        pk[k] = s_prefix[t];
+        sk[k] = s_sc[t];
+        bk[k] = s_bx[t];
+      }
 #pragma unroll
       for (uint32_t k = 0; k < 4; ++k) {
         const uint32_t t = g * 8u + k * 2u + sub;
-        const float y = (t < T && row < rows) ? s_y[row * CP + hl.first + t] : 0.0f;
-        const bool keep = t < T && row < rows && y > thr;
+        const bool keep = t < T && row < rows && yk[k] > thr;
         const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
         if (keep) {
           const uint32_t half = sub ? (uint32_t)(bal >> 32) : (uint32_t)bal;
-          const uint32_t dst = s_prefix[t] + (uint32_t)__popc(half & ((1u << row) - 1u));
-          FX_AS1 float* sc = (FX_AS1 float*)s_sc[t];
-          FX_AS1 float* bx = (FX_AS1 float*)s_bx[t];
-          sc[dst] = y;
-          *(FX_AS1 fx_u32x4_a4*)(bx + (size_t)dst * 4u) = s_box[row];
+          const uint32_t dst = pk[k] + (uint32_t)__popc(half & ((1u << row) - 1u));
+          ((FX_AS1 float*)sk[k])[dst] = yk[k];
+          *(FX_AS1 fx_u32x4_a4*)((FX_AS1 float*)bk[k] + (size_t)dst * 4u) = box;
         }
       }
     }
   }
+  FX_CMAP_STAMP(5);
 }
 
 }  // namespace
@@ -240,21 +295,30 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_classmap_head(const FxCmapLaunch 
 uint32_t fx_cmap_lds_bytes(const FxCmapLaunch& hl) { return FX_CMAP_R * (hl.C | 1u) * 4u; }
 uint32_t fx_cmap_chunk_rows() { return FX_CMAP_R; }
 
-// Workgroups of the kernel that the current device holds at once.
-hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* workgroups) {
+// Workgroups of the kernel that the current device holds at once: of the wide form, of the narrow form.
+hipError_t fx_cmap_resident(uint32_t lds_bytes, uint32_t* wide, uint32_t* narrow) {
   int dev = 0, cus = 0, per_cu = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (e != hipSuccess) return e;
-  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)&fx_classmap_head, (int)FX_BLOCK, (size_t)lds_bytes);
+  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)&fx_classmap_head<FX_CMAP_WIDE>, (int)FX_CMAP_WIDE,
+                                                   (size_t)lds_bytes);
   if (e != hipSuccess) return e;
-  *workgroups = (uint32_t)std::max(per_cu, 1) * (uint32_t)std::max(cus, 1);
+  *wide = (uint32_t)std::max(per_cu, 0) * (uint32_t)std::max(cus, 1);
+  e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)&fx_classmap_head<FX_CMAP_NARROW>, (int)FX_CMAP_NARROW,
+                                                   (size_t)lds_bytes);
+  if (e != hipSuccess) return e;
+  *narrow = (uint32_t)std::max(per_cu, 0) * (uint32_t)std::max(cus, 1);
   return hipSuccess;
 }
 
-hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, hipStream_t stream) {
+hipError_t fx_launch_classmap_head(const FxCmapLaunch& hl, const FxDyn* dyn, bool wide, hipStream_t stream) {
   if (hl.chunks == 0) return hipSuccess;
   void* args[2] = {(void*)&hl, (void*)dyn};
-  return hipLaunchKernel((const void*)&fx_classmap_head, dim3(hl.chunks), dim3(FX_BLOCK), args, fx_cmap_lds_bytes(hl), stream);
+  if (wide)
+    return hipLaunchKernel((const void*)&fx_classmap_head<FX_CMAP_WIDE>, dim3(hl.chunks), dim3(FX_CMAP_WIDE), args,
+                           fx_cmap_lds_bytes(hl), stream);
+  return hipLaunchKernel((const void*)&fx_classmap_head<FX_CMAP_NARROW>, dim3(hl.chunks), dim3(FX_CMAP_NARROW), args,
+                         fx_cmap_lds_bytes(hl), stream);
 }

@@ -131,6 +131,7 @@ struct Plan {
   // the same for the chunks of the detection-head kernel, and the workgroups of it the device holds at once
   std::vector<Status> head_status;
   uint32_t head_resident = 0;
+  uint32_t cmap_resident_wide = 0;   // class-map head kernel: workgroups of its wide form
 };
 
 // Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?

@@ -924,11 +924,54 @@ void Validate(std::shared_ptr<Graph> graph) {
 // ---------------------------------------------------------------------------
 // pipeline
 // ---------------------------------------------------------------------------
+ValueTypeMap& refinedTypes() {
+  thread_local ValueTypeMap map;
+  return map;
+}
+
+namespace {
+// Is the list only read (indexed, measured, iterated by maps and loops)?
+bool listIsOnlyRead(const Value* list) {
+  for (const Use& u : list->uses()) {
+    const auto* schema = u.user->maybeSchema();
+    if (!schema) continue;   // prim::Loop, prim::ParallelMap, prim::If ...: lists travel through unchanged
+    const auto& args = schema->arguments();
+    if (u.offset < args.size() && args[u.offset].alias_info() && args[u.offset].alias_info()->isWrite()) return false;
+  }
+  return true;
+}
+struct RefinedTypesScope {
+  RefinedTypesScope() { refinedTypes().clear(); }
+  ~RefinedTypesScope() { refinedTypes().clear(); }
+};
+}  // namespace
+
 void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_types) {
-  // RefineInputTypes (refine_types.cpp:179-195): tensor arguments take the example's type
-  for (size_t i = 0; i < input_types.size() && i < graph->inputs().size(); ++i)
-    if (input_types[i] && input_types[i]->kind() == c10::TypeKind::TensorType && isTensorValue(graph->inputs()[i]))
-      graph->inputs()[i]->setType(input_types[i]);
+  RefinedTypesScope scope;
+  // RefineInputTypes (refine_types.cpp:179-195): tensor arguments take the example's type; a list
+  // argument whose example is a tuple of tensors keeps the tuple type in the side table
+  for (size_t i = 0; i < input_types.size() && i < graph->inputs().size(); ++i) {
+    Value* in = graph->inputs()[i];
+    if (!input_types[i]) continue;
+    if (input_types[i]->kind() == c10::TypeKind::TensorType && isTensorValue(in)) {
+      in->setType(input_types[i]);
+    } else if (input_types[i]->kind() == c10::TypeKind::TupleType && in->type()->kind() == c10::TypeKind::ListType &&
+               in->type()->expectRef<c10::ListType>().getElementType()->kind() == c10::TypeKind::TensorType) {
+      const auto& elems = input_types[i]->expectRef<c10::TupleType>().elements();
+      bool tensors = !elems.empty();
+      for (const auto& e : elems) tensors = tensors && e->kind() == c10::TypeKind::TensorType;
+      if (!tensors || !listIsOnlyRead(in)) continue;
+      refinedTypes()[in] = input_types[i];
+      // the length of the example is the length (the pipeline is specialised to the example's shapes)
+      const auto uses = in->uses();
+      for (const Use& u : uses) {
+        if (u.user->kind() != c10::aten::len) continue;
+        WithInsertPoint guard(u.user);
+        u.user->output()->replaceAllUsesWith(graph->insertConstant((int64_t)elems.size()));
+        u.user->destroy();
+      }
+    }
+  }
   ConvertProfilingInstrumentation(graph);   // fait.cpp:137: range markers first, they cut regions
   LowerSimpleTuples(graph);
   ConstantPropagation(graph);

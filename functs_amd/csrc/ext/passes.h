@@ -6,6 +6,7 @@
 
 #include <memory>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 namespace functs {
@@ -79,6 +80,13 @@ void Validate(std::shared_ptr<torch::jit::Graph> graph);
 // functs/csrc/jit/passes/fait/fait_pipeline.cpp:31-68 (the passes of it that the
 // fused-region path needs), on an already functionalized graph.
 void FaitPipeline(std::shared_ptr<torch::jit::Graph> graph, std::vector<c10::TypePtr> input_types);
+
+// Refined list types (fait/passes/refine_types.cpp:57-81, 175-195): a list argument whose example
+// is a tuple of tensors keeps that tuple type beside its List[Tensor] type while the pipeline runs.
+// A map functor then records the unified element type for the argument
+// (fait/passes/te_op.cpp:43-59), and len() of such a list is the constant of the example.
+using ValueTypeMap = std::unordered_map<const torch::jit::Value*, c10::TypePtr>;
+ValueTypeMap& refinedTypes();   // of the pipeline run in progress on this thread
 
 std::string fxhipLibraryPath();
 

@@ -131,7 +131,17 @@ Node* functorFromMap(Node* mapNode, Node* group) {
     if (pos != mb->inputs().end()) {
       size_t li = pos - mb->inputs().begin();  // list argument of the map
       f->addInput(mapNode->input(li));
-      types.push_back(mapNode->input(li)->type());
+      // a refined list records the unified type of its elements (te_op.cpp:43-59)
+      c10::TypePtr recorded = mapNode->input(li)->type();
+      auto refined = refinedTypes().find(mapNode->input(li));
+      if (refined != refinedTypes().end()) {
+        const auto& elems = refined->second->expectRef<c10::TupleType>().elements();
+        std::stringstream why_not;
+        auto unified = c10::unifyTypeList(elems, why_not);
+        if (unified) recorded = *unified;
+        TORCH_CHECK(!len || *len <= (int64_t)elems.size(), "ParallelMap: ", *len, " tasks over a list of ", elems.size());
+      }
+      types.push_back(recorded);
       par.push_back(1);
     } else {
       TORCH_CHECK(in->node()->owningBlock() != mb, "ParallelMap: group input defined inside the map body");

@@ -197,12 +197,24 @@ void fx_set_stream_spin_limit(uint32_t polls);
  * region that differs anywhere keeps the generic kernels.  Results are bit-identical to those.
  * A call recorded under stream capture takes the generic two passes (the one-launch forms tag
  * their status words with an epoch that travels in the kernel arguments and would be frozen in
- * the graph).  fx_set_head_kernel: process-wide switch, default on (FXHIP_HEAD=0: off; also off
- * while fx_set_specialization(0) holds).  fx_plan_head_info: out[0..8) = region recognised, kernel
- * in use now, low and high word of the hash of the normalised programs, C, 5 + C, rows, images
- * (test hook).  This is where the reference compiles the subgraph of the loop body with NVRTC
- * (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1414) and leaves x[mask] to ATen
- * (convert_to_tensorssa.cpp:422-443). */
+ * the graph).
+ * The same for an SSD-style head (functs/benchmark/ai_model/ssd/ssd_bbox.py:163-214): a map over
+ * the foreground classes whose body decodes the boxes from offsets [1, N, 4] and priors [N, 4]
+ * with two variances, takes the softmax of the scores [1, N, C] and keeps, for its class, the rows
+ * above a threshold as boxes [K, 4] and scores [K].  Lowered generically every task would redo
+ * the decode and the softmax; a plan whose programs ARE that computation (any N, C <= 128, first
+ * class, threshold, variances) runs as one launch of a kernel that computes every row once, when
+ * the device holds a workgroup per 32 rows at once (up to 16 384 or 65 536 rows; more rows keep the
+ * generic kernels).  Bit-identical to the generic kernels on the same computation split in a
+ * dense region (decode + softmax) and a class map over its results; the generic kernels on the
+ * fused region itself sum the softmax in another order (1e-6 relative).
+ * fx_set_head_kernel: process-wide switch for both kernels, default on (FXHIP_HEAD=0: off; also
+ * off while fx_set_specialization(0) holds).  fx_plan_head_info (test hook): out[0] = 1 (YOLO-style
+ * head recognised), 2 (SSD-style head) or 0; out[1] = that kernel is in use now; out[2], out[3] = low
+ * and high word of the hash of the normalised programs; then C, 5 + C, rows, images (kind 1) or
+ * classes filtered, C, rows, first class (kind 2).  This is where the reference compiles the
+ * subgraph of the loop body with NVRTC (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1414) and leaves
+ * x[mask] to ATen (convert_to_tensorssa.cpp:422-443). */
 void fx_set_head_kernel(int on);
 int fx_plan_head_info(const fx_plan*, int64_t* out, int cap);
 /* debugging / test hooks: the lowered bytecode blob (like CodeGen::getCodeText) */

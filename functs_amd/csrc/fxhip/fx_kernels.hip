@@ -38,7 +38,9 @@
 //   pass 2 (only above FX_SCAN_DIRECT tiles): exclusive scan of the counts
 //   pass 3: ballot/prefix row map in LDS, coalesced row copies
 // --------------------------------------------------------------------------
-#define FX_SCAN_DIRECT 2048
+// (up to here a tile sums the counts in front of it itself: 32 loads per lane at most, against a
+// third launch whose one workgroup walks the counts 256 at a time)
+#define FX_SCAN_DIRECT 8192
 struct FxCols {
   const void* src[8];
   void* dst[8];

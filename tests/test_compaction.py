@@ -65,7 +65,7 @@ def test_parallel_map_compaction_ragged_tasks(backend):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n", [1, 100, 256, 300000, 700000])
+@pytest.mark.parametrize("n", [1, 100, 256, 300000, 700000, 2200000])   # the last one: more tiles than sum their predecessors directly
 def test_standalone_compact_rows(n):
     from functs_amd import compact_rows
     dev = torch.device("cuda:0")

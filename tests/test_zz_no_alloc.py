@@ -34,9 +34,9 @@ def _call(static, mask, cols, outs, total):
 def test_static_matches_caller_scratch_two_calls_in_a_row():
     dev = torch.device("cuda:0")
     total = torch.zeros(1, dtype=torch.int32).pin_memory()
-    # the first call takes the scan path (more than 2048 tiles of 256 rows), the second, smaller
+    # the first call takes the scan path (more than 8192 tiles of 256 rows), the second, smaller
     # one the direct path, over tile counts that the first call left in the shared array
-    for n in (700001, 4097):
+    for n in (2200001, 4097):
         g = torch.Generator().manual_seed(n)
         mask = torch.rand(n, generator=g) < 0.5
         a = torch.rand(n, 4, generator=g)

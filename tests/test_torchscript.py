@@ -338,11 +338,13 @@ def test_c5_torchscript_gpu_new_batch_size_same_function():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n_priors,n_cls", [(60, 7), (8732, 81)])
+@pytest.mark.parametrize("n_priors,n_cls", [(60, 7), (8732, 81), (33, 2), (1917, 91), (8732, 21), (24564, 21)])
 def test_c3_torchscript_gpu(n_priors, n_cls):
     args = oc.c3_inputs(0, n_priors, n_cls)
     rb, rs = oc.run("c3", *args)
-    gb, gs = _cpu(_built("c3", args)(*_cuda(args)))
+    one = _built("c3", args)
+    assert len(_functors(one.graph)) == 1
+    gb, gs = _cpu(one(*_cuda(args)))
     assert_close(gb, list(rb), "c3 boxes", rtol=1e-5, atol=1e-6)
     assert_close(gs, list(rs), "c3 scores")
     # the two functors of the reference's pipeline give the same bits
@@ -355,6 +357,20 @@ def test_c3_torchscript_gpu(n_priors, n_cls):
     tb, ts = _cpu(two(*_cuda(args)))
     assert_exact(gb, tb, "c3 boxes, one functor vs two")
     assert_exact(gs, ts, "c3 scores, one functor vs two")
+
+
+@pytest.mark.gpu
+def test_c3_torchscript_gpu_other_numbers_of_priors_same_function():
+    """The merged functor is built for the example's shapes; another number of priors gets a
+    plan of its own at run time (the class count is part of the function: its trip count)."""
+    f = _built("c3", oc.c3_inputs(0, 500, 21))
+    assert len(_functors(f.graph)) == 1
+    for n in (500, 77, 3000):
+        args = oc.c3_inputs(n, n, 21)
+        rb, rs = oc.run("c3", *args)
+        gb, gs = _cpu(f(*_cuda(args)))
+        assert_close(gb, list(rb), "c3 boxes n=%d" % n, rtol=1e-5, atol=1e-6)
+        assert_close(gs, list(rs), "c3 scores n=%d" % n)
 
 
 def test_c4_lstm_is_functionalized_and_keeps_its_loops():

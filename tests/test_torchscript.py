@@ -105,6 +105,17 @@ def test_c3_is_decode_plus_class_map():
     assert "aten::softmax" in kinds and "immut::select" in kinds and kinds[-1] == "aten::gt"
 
 
+def test_nothing_is_sunk_while_the_head_kernels_are_switched_off():
+    from functs_amd._lib import lib
+    args = oc.c3_inputs(0, 60, 7)
+    lib.fx_set_head_kernel(0)
+    try:
+        f = _built("c3", args)
+    finally:
+        lib.fx_set_head_kernel(1)
+    assert [n.i("is_parallel_map") for n in _functors(f.graph)] == [0, 1]
+
+
 def test_a_producer_with_other_readers_is_not_sunk():
     def g(loc: torch.Tensor, conf: torch.Tensor, priors: torch.Tensor):
         l0 = loc[0]

@@ -19,8 +19,10 @@
 // parallelize_loops.cpp:128-131): scalar-valued pure nodes of a loop or map body whose operands
 // are all defined outside move in front of the loop, innermost loops first, so that trip counts
 // and sizes stop looking like per-iteration values.
+#include <ATen/ATen.h>
 #include <torch/csrc/jit/ir/constants.h>
 
+#include <sstream>
 #include <unordered_set>
 
 #include "passes.h"
@@ -206,6 +208,127 @@ bool hoistIn(Block* b) {
 }
 
 }  // namespace
+
+namespace {
+
+// ---- static type queries ---------------------------------------------------------------------
+// What the static types say about `v`: its own tensor type, or, for an element read from a list
+// argument with a refined type, the element's type (the unified one when the index is not a
+// constant).
+c10::TensorTypePtr staticTensorType(Value* v) {
+  if (auto tt = v->type()->cast<c10::TensorType>())
+    if (tt->scalarType() || tt->sizes().size() || tt->device()) return tt;
+  Node* n = v->node();
+  if (n->kind() != c10::aten::__getitem__) return nullptr;
+  auto it = refinedTypes().find(n->input(0));
+  if (it == refinedTypes().end()) return nullptr;
+  const auto& elems = it->second->expectRef<c10::TupleType>().elements();
+  if (auto idx = constInt(n->input(1))) {
+    int64_t i = *idx < 0 ? *idx + (int64_t)elems.size() : *idx;
+    if (i < 0 || i >= (int64_t)elems.size()) return nullptr;
+    return elems[i]->cast<c10::TensorType>();
+  }
+  std::stringstream why_not;
+  auto unified = c10::unifyTypeList(elems, why_not);
+  return unified ? (*unified)->cast<c10::TensorType>() : nullptr;
+}
+
+bool foldQueriesIn(Block* b) {
+  static const Symbol kNumel = Symbol::fromQualString("aten::numel");
+  bool changed = false;
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) changed |= foldQueriesIn(inner);
+    const auto k = n->kind();
+    if (k != c10::aten::size && k != c10::prim::dtype && k != c10::prim::device && k != c10::aten::dim && k != kNumel)
+      continue;
+    if (n->inputs().empty() || n->outputs().size() != 1) continue;
+    auto tt = staticTensorType(n->input(0));
+    if (!tt) continue;
+    Graph* g = n->owningGraph();
+    WithInsertPoint guard(n);
+    Value* c = nullptr;
+    if (k == c10::aten::size && n->inputs().size() == 2) {
+      auto d = constInt(n->input(1));
+      auto rank = tt->sizes().size();
+      if (d && rank) {
+        int64_t dim = *d < 0 ? *d + (int64_t)*rank : *d;
+        if (dim >= 0 && dim < (int64_t)*rank && tt->sizes()[dim]) c = g->insertConstant(*tt->sizes()[dim]);
+      }
+    } else if (k == c10::aten::size && n->inputs().size() == 1) {
+      if (auto sizes = tt->sizes().concrete_sizes()) c = g->insertConstant(c10::IValue(c10::List<int64_t>(*sizes)));
+    } else if (k == kNumel) {
+      if (auto sizes = tt->sizes().concrete_sizes()) {
+        int64_t numel = 1;
+        for (int64_t v : *sizes) numel *= v;
+        c = g->insertConstant(numel);
+      }
+    } else if (k == c10::aten::dim) {
+      if (auto rank = tt->sizes().size()) c = g->insertConstant((int64_t)*rank);
+    } else if (k == c10::prim::dtype) {
+      if (tt->scalarType()) c = g->insertConstant((int64_t)*tt->scalarType());
+    } else if (k == c10::prim::device) {
+      // only a GPU: a function built from CPU examples still runs on whatever device its
+      // arguments live on, and what it creates there must follow them
+      if (tt->device() && tt->device()->is_cuda()) c = g->insertConstant(c10::IValue(*tt->device()));
+    }
+    if (!c) continue;
+    n->output()->replaceAllUsesWith(c);
+    n->destroy();
+    changed = true;
+  }
+  return changed;
+}
+
+}  // namespace
+
+bool FoldStaticTypeQueries(std::shared_ptr<Graph> graph) { return foldQueriesIn(graph->block()); }
+
+namespace {
+// A tensor constant whose elements are all one value (what constant propagation makes of
+// zeros_like(c), new_zeros, full over a folded shape) goes back to being a fill: inside a region a
+// fill costs nothing, a constant is an argument that is read from memory.
+bool fillsIn(Block* b) {
+  bool changed = false;
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    for (Block* inner : n->blocks()) changed |= fillsIn(inner);
+    if (n->kind() != c10::prim::Constant || !isTensorValue(n->output())) continue;
+    auto iv = toIValue(n->output());
+    if (!iv || !iv->isTensor()) continue;
+    const at::Tensor t = iv->toTensor();
+    if (!t.defined() || t.numel() < 16 || t.is_sparse() || !t.is_contiguous()) continue;
+    const auto st = t.scalar_type();
+    if (st != c10::kFloat && st != c10::kLong && st != c10::kInt && st != c10::kBool) continue;
+    const at::Tensor flat = t.reshape({-1});
+    if (!at::eq(flat, flat[0]).all().item<bool>()) continue;
+    Graph* g = n->owningGraph();
+    WithInsertPoint guard(n);
+    Value* sizes = g->insertConstant(c10::IValue(c10::List<int64_t>(t.sizes().vec())));
+    Value* none = g->insertConstant(c10::IValue());
+    Value* dtype = g->insertConstant((int64_t)st);
+    Value* device = g->insertConstant(c10::IValue(t.device()));
+    const c10::Scalar v = flat[0].item();
+    Value* fill = nullptr;
+    auto type = c10::TensorType::create(t);
+    if (v.to<double>() == 0.0) {
+      fill = make(g, c10::aten::zeros, {sizes, dtype, none, device, none}, type);
+    } else {
+      Value* value = st == c10::kFloat ? g->insertConstant(v.to<double>())
+                                       : (st == c10::kBool ? g->insertConstant(v.to<bool>()) : g->insertConstant(v.to<int64_t>()));
+      fill = make(g, c10::aten::full, {sizes, value, dtype, none, device, none}, type);
+    }
+    n->output()->replaceAllUsesWith(fill);
+    n->destroy();
+    changed = true;
+  }
+  return changed;
+}
+}  // namespace
+
+bool UniformConstantsToFills(std::shared_ptr<Graph> graph) { return fillsIn(graph->block()); }
 
 void CanonicalizeOps(std::shared_ptr<Graph> graph) { canonicalizeIn(graph->block()); }
 

@@ -188,7 +188,16 @@ bool worthFusing(const std::vector<Node*>& nodes) {
     if (n->kind() == sym::ForallSelectRev()) working += 2;
     else working += workingSymbols().count(n->kind());
   }
-  return working >= 2;
+  if (working < 2) return false;
+  // a region takes its device from its tensor arguments: fills over constant shapes alone stay eager
+  std::vector<Value*> inputs, outputs;
+  groupInOut(nodes, inputs, outputs);
+  for (Value* in : inputs) {
+    if (isTensorValue(in)) return true;
+    if (auto lt = in->type()->cast<c10::ListType>())
+      if (lt->getElementType()->kind() == c10::TypeKind::TensorType) return true;
+  }
+  return false;
 }
 
 // Reverse greedy sweeps (fuse_ops.cpp:364-425): starting at the end of the block,
@@ -946,8 +955,9 @@ struct RefinedTypesScope {
 };
 }  // namespace
 
-void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_types) {
+bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_types) {
   RefinedTypesScope scope;
+  bool specialized = false;
   // RefineInputTypes (refine_types.cpp:179-195): tensor arguments take the example's type; a list
   // argument whose example is a tuple of tensors keeps the tuple type in the side table
   for (size_t i = 0; i < input_types.size() && i < graph->inputs().size(); ++i) {
@@ -969,12 +979,15 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
         WithInsertPoint guard(u.user);
         u.user->output()->replaceAllUsesWith(graph->insertConstant((int64_t)elems.size()));
         u.user->destroy();
+        specialized = true;
       }
     }
   }
   ConvertProfilingInstrumentation(graph);   // fait.cpp:137: range markers first, they cut regions
   LowerSimpleTuples(graph);
+  specialized = FoldStaticTypeQueries(graph) || specialized;
   ConstantPropagation(graph);
+  UniformConstantsToFills(graph);
   EliminateCommonSubexpression(graph);
   EliminateDeadCode(graph);
   CanonicalizeOps(graph);       // fait_pipeline.cpp:39
@@ -990,6 +1003,7 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   const bool unrolled_maps = UnrollSimpleMaps(graph);
   if (unrolled_loops || unrolled_maps) {
     ConstantPropagation(graph);
+    UniformConstantsToFills(graph);
     EliminateCommonSubexpression(graph);
     EliminateDeadCode(graph);
     FuseOps(graph);
@@ -999,11 +1013,14 @@ void FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   CanonicalizeFusableMaps(graph);   // fait_pipeline.cpp:61
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
-  if (SinkProducersIntoMaps(graph)) {
+  if (SinkProducersIntoMaps(graph)) {   // (folds size queries on the producer's results)
     ConstantPropagation(graph);
+    UniformConstantsToFills(graph);
     EliminateDeadCode(graph);
+    specialized = true;
   }
   Validate(graph);
+  return specialized;
 }
 
 }  // namespace functs

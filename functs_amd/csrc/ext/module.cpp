@@ -6,6 +6,8 @@
 #include <torch/csrc/jit/python/pybind_utils.h>
 #include <torch/extension.h>
 
+#include <torch/csrc/autograd/python_variable.h>
+
 #include "passes.h"
 #include "tensorssa.h"
 
@@ -31,6 +33,8 @@ PYBIND11_MODULE(_C, m) {
   m.def("_jit_pass_collapse_assign_loops", CollapseAssignLoops);
   m.def("_jit_pass_collapse_recurrent_loops", CollapseRecurrentLoops);
   m.def("_jit_pass_canonicalize_ops", CanonicalizeOps);
+  m.def("_jit_pass_fold_static_type_queries", FoldStaticTypeQueries);
+  m.def("_jit_pass_uniform_constants_to_fills", UniformConstantsToFills);
   m.def("_jit_pass_hoist_loop_invariants", HoistLoopInvariants);
   m.def("_jit_pass_parallelize_loops", ParallelizeLoops);
   m.def("_jit_pass_split_parallel_maps", SplitParallelMaps);
@@ -87,6 +91,38 @@ PYBIND11_MODULE(_C, m) {
     py::dict d;
     for (const auto& kv : functorHostTimes()) d[py::str(kv.first)] = kv.second;
     return d;
+  });
+  // Hash of the shapes and dtypes of the tensor arguments (lists and tuples of tensors element by
+  // element): the key under which functs_amd.jit keeps the graphs it has built for a function.
+  m.def("_shape_key", [](const py::args& args) -> uint64_t {
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&h](uint64_t v) {
+      h ^= v;
+      h *= 1099511628211ull;
+    };
+    auto tensor = [&mix](PyObject* o) {
+      const at::Tensor& t = THPVariable_Unpack(o);
+      mix(0x7e50ull + (uint64_t)t.dim());
+      for (int64_t d : t.sizes()) mix((uint64_t)d);
+      mix((uint64_t)t.scalar_type());
+    };
+    for (const py::handle& a : args) {
+      PyObject* o = a.ptr();
+      if (THPVariable_Check(o)) {
+        tensor(o);
+      } else if (PyList_Check(o) || PyTuple_Check(o)) {
+        const Py_ssize_t n = PySequence_Fast_GET_SIZE(o);
+        mix(0x115700ull + (uint64_t)n);
+        for (Py_ssize_t i = 0; i < n; ++i) {
+          PyObject* e = PySequence_Fast_GET_ITEM(o, i);
+          if (THPVariable_Check(e)) tensor(e);
+          else mix(0x5ca1a7ull);
+        }
+      } else {
+        mix(0x5ca1a7ull);
+      }
+    }
+    return h;
   });
   m.def("_fxhip_library", []() { return functs::fxhipLibraryPath(); });
 }

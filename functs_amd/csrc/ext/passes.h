@@ -31,6 +31,16 @@ bool CollapseRecurrentLoops(std::shared_ptr<torch::jit::Graph> graph);
 // (arange(end), max.other, new_zeros, pow with a constant exponent, empty slices, t(), to.dtype /
 // to.other, view).
 void CanonicalizeOps(std::shared_ptr<torch::jit::Graph> graph);
+// Queries that the static types answer become constants: size(x, d), size(x), numel, dim, dtype of
+// a value whose type (an argument's example, or an element of a list argument with a refined
+// type) says so; device only when the type names a GPU.  With them the index arithmetic that a
+// model runs on its shapes (anchor and prior generators: arange, repeat, stack over feature-map
+// sizes) is folded by constant propagation when the function is built.  The reference gets there
+// through InferShape + constant folding (fait_pipeline.cpp:47-49).  True if the graph changed.
+bool FoldStaticTypeQueries(std::shared_ptr<torch::jit::Graph> graph);
+// Tensor constants of 16 or more elements that all hold one value become zeros / full nodes again
+// (run behind every constant propagation of the pipeline, which folds fills over static shapes).
+bool UniformConstantsToFills(std::shared_ptr<torch::jit::Graph> graph);
 // fait/passes/licm.cpp:55-66: scalar-valued pure nodes of loop and map bodies whose operands are
 // defined outside move in front of the loop; true if the graph changed.
 bool HoistLoopInvariants(std::shared_ptr<torch::jit::Graph> graph);
@@ -79,7 +89,10 @@ void Validate(std::shared_ptr<torch::jit::Graph> graph);
 
 // functs/csrc/jit/passes/fait/fait_pipeline.cpp:31-68 (the passes of it that the
 // fused-region path needs), on an already functionalized graph.
-void FaitPipeline(std::shared_ptr<torch::jit::Graph> graph, std::vector<c10::TypePtr> input_types);
+// Returns true when the graph now holds constants taken from the example's shapes (size, len,
+// dtype or device queries folded): the built function then serves arguments of those shapes only,
+// and the caller keys its built functions by shape (functs_amd/jit.py).
+bool FaitPipeline(std::shared_ptr<torch::jit::Graph> graph, std::vector<c10::TypePtr> input_types);
 
 // Refined list types (fait/passes/refine_types.cpp:57-81, 175-195): a list argument whose example
 // is a tuple of tensors keeps that tuple type beside its List[Tensor] type while the pipeline runs.

@@ -285,14 +285,24 @@ bool isZerosLike(Value* v, Value* first, Value* x) {
   Node* z = v->node();
   if (z->kind() != c10::aten::zeros || z->inputs().size() != 5) return false;
   Node* lc = z->input(0)->node();
-  if (lc->kind() != c10::prim::ListConstruct || lc->inputs().size() != 3 || lc->input(0) != first) return false;
   auto xt = x->type()->cast<c10::TensorType>();
   auto xs = xt ? xt->sizes().concrete_sizes() : std::nullopt;
-  for (int64_t d = 1; d <= 2; ++d) {
-    Value* e = lc->input((size_t)d);
-    Node* en = e->node();
-    const bool same_dim = en->kind() == c10::aten::size && en->inputs().size() == 2 && en->input(0) == x && isConst(en->input(1), d);
-    if (!same_dim && !(xs && isConst(e, (*xs)[(size_t)d]))) return false;
+  if (auto whole = toIValue(z->input(0))) {
+    // the sizes as one constant list (static shapes folded): [first, x.size(1), x.size(2)] by value
+    auto f = constant_as<int64_t>(first);
+    if (!whole->isIntList() || !f || !xs || xs->size() != 3) return false;
+    const auto v = whole->toIntVector();
+    if (v.size() != 3 || v[0] != *f || v[1] != (*xs)[1] || v[2] != (*xs)[2]) return false;
+  } else {
+    if (lc->kind() != c10::prim::ListConstruct || lc->inputs().size() != 3) return false;
+    auto f = constant_as<int64_t>(first);
+    if (lc->input(0) != first && !(f && isConst(lc->input(0), *f))) return false;
+    for (int64_t d = 1; d <= 2; ++d) {
+      Value* e = lc->input((size_t)d);
+      Node* en = e->node();
+      const bool same_dim = en->kind() == c10::aten::size && en->inputs().size() == 2 && en->input(0) == x && isConst(en->input(1), d);
+      if (!same_dim && !(xs && isConst(e, (*xs)[(size_t)d]))) return false;
+    }
   }
   auto none = [](Value* a) { return a->mustBeNone(); };
   if (!none(z->input(1)) && !isConst(z->input(1), (int64_t)c10::kFloat)) return false;   // None: the default dtype, checked at run time

@@ -659,6 +659,9 @@ static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
   hl->pred_tcoef = hi.pred_tcoef;
   hl->anc_tcoef = hi.anc_tcoef;
   hl->strd_tcoef = hi.strd_tcoef;
+  hl->folded = hi.folded ? 1u : 0u;
+  hl->half_slot = hi.half_slot;
+  hl->half_tcoef = hi.half_tcoef;
   for (int k = 0; k < 3; ++k) {
     hl->out_slot[k] = hi.out_slot[k];
     hl->out_tstride[k] = hi.out_tstride[k];

@@ -21,6 +21,9 @@
 #define FX_HEAD_MIN_CHUNK 64u  // fewest rows of a chunk unless the image has fewer
 // hash of the normalised programs of the detection-head region (fx_head_match.cpp)
 #define FX_HEAD_NORM_HASH 0xed6ab9314c50ff65ull
+// the same region with the anchors folded into box centres [N, 2] and half sizes [N, 2] and the
+// strides as [N, 1] (what constant propagation leaves of anchors generated from static shapes)
+#define FX_HEAD_NORM_HASH_FOLDED 0x680166c2c9e835ddull
 
 // What the matcher found (host).
 struct FxHeadInfo {
@@ -28,6 +31,9 @@ struct FxHeadInfo {
   uint64_t norm_hash = 0;        // hash of the normalised programs (reported also when they do not match)
   uint32_t pred_slot = 0, anc_slot = 0, strd_slot = 0;   // pointer slots (FX_SLOT_TASK: per-task table)
   int32_t pred_tcoef = 0, anc_tcoef = 0, strd_tcoef = 0; // element offset per task
+  bool folded = false;           // centres and half sizes instead of anchors: anc_* is the centres', half_* the half sizes'
+  uint32_t half_slot = 0;
+  int32_t half_tcoef = 0;
   uint32_t S = 0, C = 0;         // floats per prediction row (5 + C), classes
   uint32_t thr_bits = 0;         // objectness threshold (float bits)
   uint32_t n_rows = 0, n_tasks = 0;
@@ -50,6 +56,9 @@ struct FxHeadLaunch {
   int32_t pred_tcoef, anc_tcoef, strd_tcoef;
   uint32_t out_slot[3], out_tstride[3];
   uint32_t bulk_delay;           // big launches: waves without a gather wait this long (units of 64 clocks) before they ask for rows
+  uint32_t folded;               // 1: anc_slot holds box centres [N, 2], half_slot half sizes [N, 2]
+  uint32_t half_slot;
+  int32_t half_tcoef;
   uint32_t* status;              // one word per chunk, tagged with the epoch
   uint32_t* totals;              // pinned host memory: kept rows per task
 };

@@ -34,6 +34,7 @@
 namespace {
 
 #define FX_HEAD_DYN_OFF sizeof(FxHeadLaunch)
+typedef uint32_t fx_u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));   // 64 bits, 4-byte aligned
 
 __device__ __forceinline__ uint64_t fxh_ptr(const FxHeadLaunch& hl, uint32_t slot, uint32_t task) {
   const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
@@ -210,15 +211,25 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
       const uint32_t r = threadIdx.x, src = s_rowmap[r], row = rs0 + src;
       const FX_AS1 float* anc = (const FX_AS1 float*)fxh_ptr(hl, hl.anc_slot, task) + (int64_t)hl.anc_tcoef * task;
       const FX_AS1 float* strd = (const FX_AS1 float*)fxh_ptr(hl, hl.strd_slot, task) + (int64_t)hl.strd_tcoef * task;
-      const fx_u32x4_a4 an = *(const FX_AS1 fx_u32x4_a4*)(anc + (size_t)row * 4u);
       const float st = strd[row];
-      const float a0 = u2f(an.x), a1 = u2f(an.y), a2 = u2f(an.z), a3 = u2f(an.w);
+      // base of the centre and of the half size: from the anchor corners, or folded ahead of time
+      float bcx, bcy, bhw, bhh;
+      if (hl.folded) {
+        const FX_AS1 float* hf = (const FX_AS1 float*)fxh_ptr(hl, hl.half_slot, task) + (int64_t)hl.half_tcoef * task;
+        const fx_u32x2_a4 c2 = *(const FX_AS1 fx_u32x2_a4*)(anc + (size_t)row * 2u);
+        const fx_u32x2_a4 h2 = *(const FX_AS1 fx_u32x2_a4*)(hf + (size_t)row * 2u);
+        bcx = u2f(c2.x); bcy = u2f(c2.y); bhw = u2f(h2.x); bhh = u2f(h2.y);
+      } else {
+        const fx_u32x4_a4 an = *(const FX_AS1 fx_u32x4_a4*)(anc + (size_t)row * 4u);
+        const float a0 = u2f(an.x), a1 = u2f(an.y), a2 = u2f(an.z), a3 = u2f(an.w);
+        bcx = (a0 + a2) * 0.5f; bcy = (a1 + a3) * 0.5f; bhw = (a2 - a0) * 0.5f; bhh = (a3 - a1) * 0.5f;
+      }
       const uint32_t* p = W + src * S;
       const float p0 = u2f(p[0]), p1 = u2f(p[1]), p2 = u2f(p[2]), p3 = u2f(p[3]), p4 = u2f(p[4]);
       // half sizes ((hi - lo) * 0.5) * exp(p), centres ((lo + hi) * 0.5) + ((sigmoid(p) - 0.5) * stride)
-      const float hw = ((a2 - a0) * 0.5f) * fx_exp(p2), hh = ((a3 - a1) * 0.5f) * fx_exp(p3);
-      const float cx = ((a0 + a2) * 0.5f) + ((fx_sigmoid(p0) - 0.5f) * st);
-      const float cy = ((a1 + a3) * 0.5f) + ((fx_sigmoid(p1) - 0.5f) * st);
+      const float hw = bhw * fx_exp(p2), hh = bhh * fx_exp(p3);
+      const float cx = bcx + ((fx_sigmoid(p0) - 0.5f) * st);
+      const float cy = bcy + ((fx_sigmoid(p1) - 0.5f) * st);
       fx_u32x4 ob;
       ob.x = f2u(cx - hw); ob.y = f2u(cy - hh); ob.z = f2u(cx + hw); ob.w = f2u(cy + hh);
       FX_AS1 float* box = (FX_AS1 float*)fxh_ptr(hl, hl.out_slot[1], task) + (size_t)hl.out_tstride[1] * task;

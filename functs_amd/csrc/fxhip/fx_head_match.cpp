@@ -57,8 +57,10 @@ void match_head(Plan* P) {
   const uint32_t C = o_cls.rowlen, S = C + 5;
 
   Hasher hs;
-  std::map<int32_t, int> buf_class;   // pointer slot -> 0 (predictions), 1 (anchors), 2 (strides), in order of first use
-  int32_t slot_of[3] = {0, 0, 0}, tcoef_of[3] = {0, 0, 0};
+  // pointer slot -> buffer in order of first use: predictions, anchors, strides; with folded anchors
+  // predictions, half sizes, strides, centres
+  std::map<int32_t, int> buf_class;
+  int32_t slot_of[4] = {0, 0, 0, 0}, tcoef_of[4] = {0, 0, 0, 0}, coef0_of[4] = {0, 0, 0, 0};
   bool bad = false;
   uint32_t thr_bits = 0;
   auto walk = [&](uint32_t pb, uint32_t pe, bool is_mask) {
@@ -75,18 +77,18 @@ void match_head(Plan* P) {
         int bc;
         if (it == buf_class.end()) {
           bc = (int)buf_class.size();
-          if (bc >= 3) { bad = true; return; }
+          if (bc >= 4) { bad = true; return; }
           buf_class[x.a] = bc;
           slot_of[bc] = x.a;
           tcoef_of[bc] = aff[x.b].tcoef;
+          coef0_of[bc] = fx_aff_coef(&aff[x.b], 0);
         } else {
           bc = it->second;
         }
         const FxAffine& a = aff[x.b];
         if (a.tcoef != tcoef_of[bc] || a.rcoef[0] != 0 || a.rcoef[1] != 0) { bad = true; return; }
-        // the row stride of each buffer is fixed by its role
-        const int32_t want0 = bc == 0 ? (int32_t)S : (bc == 1 ? 4 : 1);
-        if (fx_aff_coef(&a, 0) != want0) { bad = true; return; }
+        // the row stride of each buffer is fixed by its role (checked below, once the form is known)
+        if (fx_aff_coef(&a, 0) != coef0_of[bc]) { bad = true; return; }
         hs.mix((uint64_t)bc);
         for (int k = 1; k < FX_MAXR; ++k) hs.mix((uint64_t)(uint32_t)fx_aff_coef(&a, k));
         hs.mix((uint64_t)(uint32_t)a.base);
@@ -120,15 +122,28 @@ void match_head(Plan* P) {
     walk(outs[k].prog_begin, outs[k].prog_end, false);
   }
   hi.norm_hash = hs.h;
-  if (bad || buf_class.size() != 3 || hs.h != kHeadHash) return;
+  if (bad) return;
+  const bool plain = buf_class.size() == 3 && hs.h == kHeadHash && coef0_of[0] == (int32_t)S && coef0_of[1] == 4 &&
+                     coef0_of[2] == 1;
+  const bool folded = buf_class.size() == 4 && hs.h == FX_HEAD_NORM_HASH_FOLDED && coef0_of[0] == (int32_t)S &&
+                      coef0_of[1] == 2 && coef0_of[2] == 1 && coef0_of[3] == 2;
+  if (!plain && !folded) return;
   // 32-bit addressing of the kernel: checked for the prediction tensor by the plan already
   // (every buffer of a region lies below 4 GiB)
   hi.pred_slot = (uint32_t)slot_of[0];
-  hi.anc_slot = (uint32_t)slot_of[1];
   hi.strd_slot = (uint32_t)slot_of[2];
   hi.pred_tcoef = tcoef_of[0];
-  hi.anc_tcoef = tcoef_of[1];
   hi.strd_tcoef = tcoef_of[2];
+  hi.folded = folded;
+  if (folded) {
+    hi.half_slot = (uint32_t)slot_of[1];
+    hi.half_tcoef = tcoef_of[1];
+    hi.anc_slot = (uint32_t)slot_of[3];
+    hi.anc_tcoef = tcoef_of[3];
+  } else {
+    hi.anc_slot = (uint32_t)slot_of[1];
+    hi.anc_tcoef = tcoef_of[1];
+  }
   hi.S = S;
   hi.C = C;
   hi.thr_bits = thr_bits;

@@ -13,18 +13,36 @@ import torch
 from . import _C  # noqa: F401  (registers immut:: operators and tssa::ParallelFunctor)
 
 
-class AotScriptFunction(object):
-    """Callable around the compiled graph (functs/jit/_script.py:12-26)."""
+def _shape_key(args):
+    """Hash of the shapes and dtypes of the tensor arguments (lists of tensors element by element)."""
+    return _C._shape_key(*args)
 
-    def __init__(self, aot_script_fn, **kwargs):
+
+class AotScriptFunction(object):
+    """Callable around the compiled graph (functs/jit/_script.py:12-26).
+
+    The pipeline folds what the example's shapes answer (``x.size(0)``, ``len(xs)``, dtypes) into
+    constants, as the reference's does: a graph built that way serves arguments of those shapes
+    only.  Such a function keeps the functionalized script it was built from and builds a graph
+    per set of argument shapes, the first one from the example; ``graph`` is that first one."""
+
+    def __init__(self, aot_script_fn, source=None, key=None, **kwargs):
         self._aot_script_fn = aot_script_fn
+        self._source = source
+        self._variants = {key: aot_script_fn} if source is not None else None
 
     @property
     def graph(self):
         return self._aot_script_fn.graph
 
     def __call__(self, *args, **kwargs):
-        return self._aot_script_fn(*args, **kwargs)
+        if self._variants is None:
+            return self._aot_script_fn(*args, **kwargs)
+        key = _shape_key(args)
+        fn = self._variants.get(key)
+        if fn is None:
+            fn = self._variants[key] = _compile(self._source, args)[0]
+        return fn(*args, **kwargs)
 
 
 def extract_type_hint_from_tensor(input_):
@@ -80,8 +98,8 @@ class GraphedFunction(AotScriptFunction):
     region cannot be captured: its output shapes need a synchronisation per call.
     """
 
-    def __init__(self, aot_script_fn):
-        super().__init__(aot_script_fn)
+    def __init__(self, aot_script_fn, source=None, key=None):
+        super().__init__(aot_script_fn, source=source, key=key)
         if "compact_rows=1" in str(aot_script_fn.graph):
             raise ValueError("a function with a row-compacting region cannot run as a HIP graph")
         self._captures = {}
@@ -113,13 +131,14 @@ class GraphedFunction(AotScriptFunction):
             static = [self._map(a, lambda t: t.clone()) for a in args]
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
+            run = super().__call__   # (builds the graph for these shapes first, if they are new)
             with torch.cuda.stream(side):
                 for _ in range(2):
-                    self._aot_script_fn(*static)
+                    run(*static)
             torch.cuda.current_stream().wait_stream(side)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                out = self._aot_script_fn(*static)
+                out = run(*static)
             cap = self._captures[key] = (graph, static, out)
         graph, static, out = cap
 
@@ -141,13 +160,19 @@ def build(fn, example_input: List[object], hip_graph: bool = False) -> AotScript
     (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
         raise AttributeError("only a functionalized jit script can be built")
+    aot, specialized = _compile(fn, example_input)
+    source, key = (fn, _shape_key(example_input)) if specialized else (None, None)
+    return GraphedFunction(aot, source, key) if hip_graph else AotScriptFunction(aot, source, key)
+
+
+def _compile(fn, example_input):
+    """(compiled function, whether its graph holds constants of the example's shapes)"""
     g = fn.graph.copy()
     if isinstance(fn, torch.jit.ScriptModule):
         _strip_self(g)
     hints = [extract_type_hint_from_tensor(i) for i in example_input]
-    _C._jit_pass_fait_pipeline(g, hints)
-    aot = _C._create_function_from_graph("forward", g)
-    return GraphedFunction(aot) if hip_graph else AotScriptFunction(aot)
+    specialized = bool(_C._jit_pass_fait_pipeline(g, hints))
+    return _C._create_function_from_graph("forward", g), specialized
 
 
 def script(fn, backend="jit", remove_update=True, enable_dce_cse=True, add_clone=False):

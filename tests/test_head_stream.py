@@ -43,6 +43,43 @@ def _head(thr=0.3, obj_col=4, half=0.5, batch=None):
     return r.finalize()
 
 
+def _head_folded(thr=0.3, batch=None):
+    """The same head after constant propagation has folded anchors that were generated from static
+    shapes: box centres [N, 2] and half sizes [N, 2] instead of anchors, strides as [N, 1]."""
+    r = Region(parallel_degree=batch, is_parallel_map=True) if batch else Region()
+    preds = r.tensor_input(torch.float32, 3)
+    strd = r.tensor_input(torch.float32, 2)
+    ctr = r.tensor_input(torch.float32, 2)
+    half = r.tensor_input(torch.float32, 2)
+    if batch:
+        i = r.task_index()
+        pred = preds.slice(0, i, r.op("INT_ADD", i, 1))
+    else:
+        pred = preds
+    pred1 = pred.slice_rev(pred.slice(2, 0, 2).sigmoid(), 2, 0, 2)
+    obj = pred1.select(2, 4).sigmoid()
+    cls = pred1.slice(2, 5, None).sigmoid()
+    p = pred1.select(0, 0)
+    xy = ctr + (p.slice(1, 0, 2) - 0.5) * strd
+    wh = half * p.slice(1, 2, 4).exp()
+    boxes = r.op("FULL", r.int_list([r.op("SIZE", ctr, 0), 4]), 0.0, dtype=torch.float32)
+    boxes = boxes.select_rev(xy.select(1, 0) - wh.select(1, 0), 1, 0)
+    boxes = boxes.select_rev(xy.select(1, 1) - wh.select(1, 1), 1, 1)
+    boxes = boxes.select_rev(xy.select(1, 0) + wh.select(1, 0), 1, 2)
+    boxes = boxes.select_rev(xy.select(1, 1) + wh.select(1, 1), 1, 3)
+    obj0 = obj.select(0, 0)
+    r.output(boxes)
+    r.output(cls.select(0, 0))
+    r.output(obj0)
+    r.compact_rows(obj0 >= thr)
+    return r.finalize()
+
+
+def _folded(pred, anchors, strides):
+    """Arguments of _head_folded from those of _head (the folding is exact: sums and halvings)."""
+    return pred, strides.unsqueeze(-1), (anchors[:, :2] + anchors[:, 2:]) * 0.5, (anchors[:, 2:] - anchors[:, :2]) * 0.5
+
+
 def _inputs(n, classes, batch, seed=0):
     g = torch.Generator().manual_seed(seed)
     pred = torch.randn(batch, n, 5 + classes, generator=g)
@@ -77,6 +114,13 @@ def test_classes_rows_images_and_threshold_are_parameters():
     for classes, n, batch, thr in ((8, 100, None, 0.3), (4, 1, 3, 0.5), (80, 10647, 2, 0.05), (12, 777, 5, 0.9)):
         info, _ = _info(_head(thr=thr, batch=batch), *_inputs(n, classes, batch or 1))
         assert info[0] == 1 and info[4] == classes and info[6] == n and info[7] == (batch or 1), (classes, n, batch, info)
+
+
+def test_the_head_with_folded_anchors_is_recognised():
+    for classes, n, batch in ((8, 100, None), (80, 10647, 16)):
+        info, p = _info(_head_folded(batch=batch), *_folded(*_inputs(n, classes, batch or 1)))
+        assert info[0] == 1 and info[1] == 1 and info[4] == classes and info[6] == n and info[7] == (batch or 1)
+        assert lib.fx_plan_launches(p.handle) == 1
 
 
 def test_other_regions_keep_the_generic_kernels():
@@ -132,6 +176,16 @@ def test_any_number_of_rows_images_and_classes(n, classes, batch):
     for t, k in enumerate(kept):
         near = int(((torch.sigmoid(pred[t, :, 4]) - 0.3).abs() < 1e-6).sum())
         assert abs(objs[t].shape[0] - int(k.sum())) <= near
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,classes,batch", [(1, 4, None), (65, 80, 2), (1000, 12, 16), (10647, 80, None), (10647, 80, 16)])
+def test_folded_anchors_bit_exact_against_both_other_forms(n, classes, batch):
+    args = _inputs(n, classes, batch or 1, seed=n + classes)
+    one, two = _both(_head_folded(batch=batch), *_folded(*args))
+    assert_exact(one, two, "folded anchors: head kernel vs two passes")
+    plain = run_region("hip", _head(batch=batch), *args)
+    assert_exact(one, plain, "folded anchors vs anchors")
 
 
 @pytest.mark.gpu

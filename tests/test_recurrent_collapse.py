@@ -158,7 +158,9 @@ def test_the_benchmark_program_becomes_one_functor_around_one_node():
     assert [i.type().kind() for i in ins[5:8]] == ["NoneType"] * 3
     assert "aten::zeros" not in _kinds(built.graph) and "aten::zeros" not in _kinds(sub)
     assert f.i("parallel_degree") == 1 and f.i("is_parallel_map") == 0
-    assert len(list(f.inputs())) == 7 and len(list(f.outputs())) == 3   # 5 tensors, the two trip counts
+    # 5 tensors; the two trip counts are constants of the static shapes (x.size(0), wih.size(0))
+    assert len(list(f.inputs())) == 5 and len(list(f.outputs())) == 3
+    assert [i.node().kind() for i in ins[8:10]] == ["prim::Constant"] * 2
 
 
 def test_a_functionalized_graph_holds_the_node_after_the_pass_alone():
@@ -186,10 +188,18 @@ def test_operand_and_update_order_do_not_matter():
 def test_trip_counts_computed_inside_the_time_loop_are_moved_out():
     x, wih, whh, bih, bhh = oc.c4_inputs(4, 9, 64, 3, 1)
     h0, c0 = _states(4, 3, 1, 64)
-    built = fj.build(fj.script(lstm_first_layer_only), [x, wih, whh, bih, bhh, h0, c0])
+    args = [x, wih, whh, bih, bhh, h0, c0]
+    # the pass alone, on a graph whose size queries are still nodes (the whole pipeline folds them
+    # to constants of the static shapes first)
+    g = fj.script(lstm_first_layer_only).graph.copy()
+    _C._jit_pass_fait_shape_infer(g, [fj.extract_type_hint_from_tensor(a) for a in args], None)
+    assert _C._jit_pass_collapse_recurrent_loops(g)
+    kinds = _kinds(g)
+    assert "prim::Loop" not in kinds and kinds.count("aten::sub") == 2   # T - 2 and L - 1, in front of the node
+    assert kinds.index("fx::lstm_stack") > max(i for i, k in enumerate(kinds) if k == "aten::sub")
+    built = fj.build(fj.script(lstm_first_layer_only), args)
     kinds = _kinds(built.graph)
-    assert "prim::Loop" not in kinds and kinds.count("aten::sub") == 2   # T - 2 and L - 1, in front of the functor
-    assert len(_functors(built.graph)) == 1
+    assert "prim::Loop" not in kinds and "aten::sub" not in kinds and len(_functors(built.graph)) == 1
 
 
 @pytest.mark.parametrize("fn", [lstm_with_relu_gate, lstm_wrong_gate_order, lstm_reads_the_wrong_state])

@@ -195,6 +195,9 @@ void fx_set_stream_spin_limit(uint32_t polls);
  * in the one-pass form above, with the same poll limit).  The programs are compared instruction
  * by instruction (any number of rows, images and classes C with C % 4 == 0, any threshold); a
  * region that differs anywhere keeps the generic kernels.  Results are bit-identical to those.
+ * A second form of the same head is recognised too: anchors folded ahead of time into box centres
+ * [N, 2] and half sizes [N, 2], strides as [N, 1] (what constant propagation leaves of anchors
+ * that a model generates from static feature-map sizes).
  * A call recorded under stream capture takes the generic two passes (the one-launch forms tag
  * their status words with an epoch that travels in the kernel arguments and would be frozen in
  * the graph).

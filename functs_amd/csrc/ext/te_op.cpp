@@ -360,6 +360,8 @@ struct OutLayout {
   std::vector<int64_t> total;      // elements to allocate per output
   std::vector<int32_t> dtype;      // FX dtype per output
   std::vector<int64_t> item;       // element size per output
+  std::vector<int64_t> base;       // a map's outputs share ONE allocation: byte offset of each output in it
+  int64_t block_bytes = 0;
 };
 
 struct Variant {
@@ -486,6 +488,11 @@ class RegionRunner {
         lay->dtype[o] = dt;
         lay->item[o] = item;
       }
+      lay->base.resize(n_out);
+      for (int o = 0; o < n_out; ++o) {
+        lay->base[o] = lay->block_bytes;
+        lay->block_bytes += (lay->total[o] * lay->item[o] + 255) / 256 * 256;
+      }
       std::lock_guard<std::mutex> lock(var->mu);
       layout = var->layouts.emplace(plan, std::move(lay)).first->second;
     }
@@ -494,18 +501,24 @@ class RegionRunner {
     std::vector<Slot> slots;   // a copy only where the kept-row counts change the sizes
     if (compact_) slots = layout->slots;
     const Slot* slot_of = compact_ ? slots.data() : layout->slots.data();
+    // A map: ONE allocation for all outputs of all tasks (an allocation costs about a
+    // microsecond of host time); a single task: one tensor per output.
     std::vector<at::Tensor> buffers(n_out);
+    at::Tensor block;
     std::vector<void*> ptrs((size_t)n_out * degree);
+    if (degree > 1)
+      block = at::empty({std::max<int64_t>(layout->block_bytes, 1)}, at::TensorOptions().dtype(at::kByte).device(device));
     for (int o = 0; o < n_out; ++o) {
       const int32_t dt = layout->dtype[o];
       const int64_t item = layout->item[o];
+      char* base;
       if (degree == 1) {
         const Slot& sl = slot_of[(size_t)o * degree];
         buffers[o] = at::empty(at::IntArrayRef(sl.sizes, sl.rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
+        base = (char*)buffers[o].data_ptr();
       } else {
-        buffers[o] = at::empty({layout->total[o]}, at::TensorOptions().dtype(atDtype(dt)).device(device));
+        base = (char*)block.data_ptr() + layout->base[o];
       }
-      char* base = (char*)buffers[o].data_ptr();
       for (int64_t t = 0; t < degree; ++t)
         ptrs[(size_t)o * degree + t] = base + slot_of[(size_t)o * degree + t].offset_elems * item;
     }
@@ -530,9 +543,9 @@ class RegionRunner {
       outs[o].reserve(degree);
       for (int64_t t = 0; t < degree; ++t) {
         const Slot& sl = slot_of[(size_t)o * degree + t];
-        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(buffers[o].storage()),
-                                                         buffers[o].key_set(), buffers[o].dtype());
-        impl->set_storage_offset(sl.offset_elems);
+        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(block.storage()), block.key_set(),
+                                                         c10::scalarTypeToTypeMeta(atDtype(layout->dtype[o])));
+        impl->set_storage_offset(layout->base[o] / layout->item[o] + sl.offset_elems);
         impl->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
         outs[o].emplace_back(std::move(impl));
       }

@@ -302,6 +302,10 @@ bool fillsIn(Block* b) {
     if (!t.defined() || t.numel() < 16 || t.is_sparse() || !t.is_contiguous()) continue;
     const auto st = t.scalar_type();
     if (st != c10::kFloat && st != c10::kLong && st != c10::kInt && st != c10::kBool) continue;
+    // only where a region can absorb the fill: a reader outside regions would run it on every call
+    bool absorbed = !n->output()->uses().empty();
+    for (const Use& u : n->output()->uses()) absorbed = absorbed && isFusableNode(u.user);
+    if (!absorbed) continue;
     const at::Tensor flat = t.reshape({-1});
     if (!at::eq(flat, flat[0]).all().item<bool>()) continue;
     Graph* g = n->owningGraph();

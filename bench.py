@@ -559,7 +559,7 @@ def main():
                 "kept_rows_per_image": [min(rows), max(rows)], "candidates_per_image": [min(cand), max(cand)],
                 "detections_per_image": [min(kept), max(kept)],
                 "nms_bytes_read": read, "nms_gbps": round(read / (e0.elapsed_time(e1) * 1e-3 / n) / 1e9, 1),
-                "bound": "one workgroup per image: the candidate scan reads the image's class scores once; "
+                "bound": "the candidate scan reads the image's class scores once (a workgroup per CU, shared out over the images); "
                          "sort and the greedy walk run in LDS"}
 
     def run_rows():

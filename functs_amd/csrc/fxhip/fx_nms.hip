@@ -25,9 +25,15 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "../../../include/fxhip.h"
+
+// a hook for timing the phases of a task's last workgroup from a test program; nothing in the library
+#ifndef FX_NMS_STAMP
+#define FX_NMS_STAMP(k)
+#endif
 
 #define FX_NMS_THREADS 1024u
 #define FX_NMS_CHUNK 64u
@@ -110,6 +116,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   const uint32_t rows = s_base;
   __syncthreads();   // s_base is used again below
 
+  FX_NMS_STAMP(0);
   // 1. candidates: four 128-bit loads per thread in flight, one LDS atomic per wave and round
   const uint32_t all_items = rows * C;   // < 2^32 (host)
   // this workgroup's share: a multiple of four items, so that its 128-bit loads stay aligned
@@ -170,6 +177,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   for (int o = 32; o >= 1; o >>= 1) my_max = max(my_max, (uint32_t)__shfl_xor((int)my_max, o, 64));
   if (lane == 0u) atomicMax(&s_maxc, my_max);
   __syncthreads();
+  FX_NMS_STAMP(1);
   {
     // hand this workgroup's keys over and take a ticket
     const uint32_t mine = min(s_count, key_cap);
@@ -191,6 +199,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     __syncthreads();
     if (s_ticket != slices - 1u) return;   // somebody else finishes the task
   }
+  FX_NMS_STAMP(2);
   // the last workgroup of the task: everything the others wrote is visible
   const uint32_t count = __hip_atomic_load(&ctr[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const uint32_t maxc = __hip_atomic_load(&ctr[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -221,6 +230,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   // Stages whose partners lie at most 64 apart stay inside aligned blocks of 128 keys: a wave
   // runs all of them on its blocks without a workgroup barrier (LDS accesses of one wave are
   // performed in order), so a phase costs one barrier per wider stage plus one.
+  FX_NMS_STAMP(3);
   uint32_t n2 = 128u;
   while (n2 < count) n2 <<= 1;
   for (uint32_t i = count + tid; i < n2; i += FX_NMS_THREADS) s_keys[i] = ~0ull;
@@ -251,6 +261,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     __syncthreads();
   }
 
+  FX_NMS_STAMP(4);
   // 3. greedy walk
   if (tid == 0) s_nk = 0u;
   __syncthreads();
@@ -339,6 +350,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     __syncthreads();
     nk = s_nk;
   }
+  FX_NMS_STAMP(5);
   // rows past the kept ones are zero: the outputs have a fixed shape
   for (uint32_t k = nk * 5u + tid; k < d.max_num * 5u; k += FX_NMS_THREADS) dets[k] = 0.0f;
   for (uint32_t k = nk + tid; k < d.max_num; k += FX_NMS_THREADS) {
@@ -350,12 +362,20 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
 
 }  // namespace
 
-// slices of a task: enough workgroups to fill the device, none with less than one round of loads
+// slices of a task: a workgroup per CU over all tasks (a CU takes one workgroup of 1024 threads at
+// a time: with two per CU the second half of the launch starts when the first ends, 16 us into
+// the kernel for 16 images), none with less than one round of loads
 uint32_t fx_nms_slices(const fx_nms_desc& d) {
   const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? d.n_classes : 1u);
   const uint64_t per_round = (uint64_t)FX_NMS_THREADS * 16u;
   uint64_t s = (items + per_round - 1) / per_round;
-  const uint64_t want = d.n_tasks > 0 ? (512u + (uint32_t)d.n_tasks - 1u) / (uint32_t)d.n_tasks : 1u;
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    else cus = 256;
+  }
+  const uint64_t want = d.n_tasks > 0 ? std::max<uint32_t>((uint32_t)cus / (uint32_t)d.n_tasks, 1u) : 1u;
   if (s > want) s = want;
   if (s > 64) s = 64;
   return s < 1 ? 1u : (uint32_t)s;

@@ -191,3 +191,29 @@ def test_scores_that_start_at_an_odd_address():
     ref = r(loc.to(dev), conf.to(dev), priors.to(dev))
     torch.cuda.synchronize()
     assert_exact([[t.cpu() for t in o] for o in got], [[t.cpu() for t in o] for o in ref], "odd start")
+
+
+@pytest.mark.gpu
+def test_the_epoch_of_the_status_words_wraps():
+    """The tag of a status word has 16 bits: after 65 534 calls on a stream the library clears the
+    words (in stream order) and starts the epochs over.  Calls on either side of the wrap must see
+    only their own counts."""
+    dev = torch.device("cuda:0")
+    loc, conf, priors = [t.to(dev) for t in _inputs(200, 9, seed=2)]
+    r = configs.build_c3_fused(8)
+    bc = r.bind(loc, conf, priors)
+    bc.launch()
+    torch.cuda.synchronize()
+    ref = [[t.clone() for t in o] for o in bc.results()]
+    for i in range(66000):
+        bc.launch()
+        if i % 256 == 0:
+            torch.cuda.synchronize()      # (the pinned count words of a call must not be reused while it is in flight)
+        if i % 8192 == 0 or i > 65500 and i % 64 == 0:
+            torch.cuda.synchronize()
+            got = bc.results()
+            assert_exact([[t.cpu() for t in o] for o in got], [[t.cpu() for t in o] for o in ref], "call %d" % i)
+    # other inputs right after the wrap
+    loc2, conf2, priors2 = _inputs(200, 9, seed=3)
+    got = run_region("hip", r, loc2, conf2, priors2)
+    assert_exact(got, _split(loc2, conf2, priors2), "new inputs after the wrap")

@@ -123,7 +123,6 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   const uint32_t share = (((all_items + slices - 1u) / slices) + 3u) & ~3u;
   const uint32_t first = min(slice * share, all_items);
   const uint32_t n_items = min(first + share, all_items);   // end of the share
-  uint32_t my_max = 0u;                // below orderable() of every value
   const bool vec = (((uintptr_t)scores) & 15u) == 0u;
   constexpr uint32_t U = 4u, PER_ROUND = FX_NMS_THREADS * U * 4u;
   for (uint32_t base = first; base < n_items; base += PER_ROUND) {
@@ -163,28 +162,18 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
       for (uint32_t e = 0; e < 4u; ++e) {
         if ((mine >> (u * 4u + e)) & 1u) {
           const uint32_t i = base + (u * FX_NMS_THREADS + tid) * 4u + e;
-          const uint32_t r = i / C;
-          float s = v[u][e];
-          if (d.mode == 1 && factors) s = s * factors[r];
-          if (slot < key_cap) s_keys[slot] = ((uint64_t)(~orderable(s)) << 32) | (uint64_t)i;
+          // (the raw score for now: the row's factor is applied by the finishing workgroup)
+          if (slot < key_cap) s_keys[slot] = ((uint64_t)(~orderable(v[u][e])) << 32) | (uint64_t)i;
           ++slot;
-          const float4 b = *(const float4*)(boxes + (size_t)r * 4u);
-          my_max = max(my_max, max(max(orderable(b.x), orderable(b.y)), max(orderable(b.z), orderable(b.w))));
         }
       }
   }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) my_max = max(my_max, (uint32_t)__shfl_xor((int)my_max, o, 64));
-  if (lane == 0u) atomicMax(&s_maxc, my_max);
   __syncthreads();
   FX_NMS_STAMP(1);
   {
     // hand this workgroup's keys over and take a ticket
     const uint32_t mine = min(s_count, key_cap);
-    if (tid == 0) {
-      s_base = atomicAdd(&ctr[0], s_count);
-      atomicMax(&ctr[2], s_maxc);
-    }
+    if (tid == 0) s_base = atomicAdd(&ctr[0], s_count);
     __syncthreads();
     const uint32_t gbase = s_base;
     // Keys and counters are written with device-scope atomic accesses, which go through to the
@@ -202,7 +191,6 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   FX_NMS_STAMP(2);
   // the last workgroup of the task: everything the others wrote is visible
   const uint32_t count = __hip_atomic_load(&ctr[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const uint32_t maxc = __hip_atomic_load(&ctr[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   if (tid == 0) {   // the counters are zero again for the next launch
     __hip_atomic_store(&ctr[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -222,9 +210,26 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     }
     return;
   }
-  for (uint32_t k = tid; k < count; k += FX_NMS_THREADS)
-    s_keys[k] = __hip_atomic_load(&g_keys[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const float class_step = from_orderable(maxc) + 1.0f;
+  // The largest coordinate of the candidates' boxes (classes are told apart by moving boxes by a
+  // multiple of it): taken here, one box per thread, not in the scan, where a gather per
+  // candidate would sit between the rounds of loads.
+  uint32_t my_max = 0u;                // below orderable() of every value
+  for (uint32_t k = tid; k < count; k += FX_NMS_THREADS) {
+    uint64_t key = __hip_atomic_load(&g_keys[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t r = (uint32_t)key / C;
+    if (d.mode == 1 && factors) {
+      const float sc = from_orderable(~(uint32_t)(key >> 32)) * factors[r];
+      key = ((uint64_t)(~orderable(sc)) << 32) | (uint64_t)(uint32_t)key;
+    }
+    s_keys[k] = key;
+    const float4 b = *(const float4*)(boxes + (size_t)r * 4u);
+    my_max = max(my_max, max(max(orderable(b.x), orderable(b.y)), max(orderable(b.z), orderable(b.w))));
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) my_max = max(my_max, (uint32_t)__shfl_xor((int)my_max, o, 64));
+  if (lane == 0u) atomicMax(&s_maxc, my_max);
+  __syncthreads();
+  const float class_step = from_orderable(s_maxc) + 1.0f;
 
   // 2. bitonic sort (ascending keys = descending score, ascending index); the tail is padding.
   // Stages whose partners lie at most 64 apart stay inside aligned blocks of 128 keys: a wave

@@ -107,6 +107,15 @@ bool isFusableNode(Node* node) {
           node->kind() == c10::aten::neg))
       return false;
   }
+  // max: the reduction along a dimension whose indices nobody reads; max(x) over everything and
+  // max with used indices stay ATen's
+  if (node->kind() == c10::aten::max) {
+    bool any_tensor = false;
+    for (Value* in : node->inputs()) any_tensor = any_tensor || isTensorValue(in);
+    if (any_tensor && !(node->inputs().size() >= 2 && node->outputs().size() == 2 && !node->output(1)->hasUses() &&
+                        !isTensorValue(node->input(1))))
+      return false;
+  }
   // bool-mask indexing is data dependent: never inside a group (it is folded in
   // afterwards by FuseMaskedSelect when possible)
   if (isIndexLike(node)) {

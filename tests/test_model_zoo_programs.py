@@ -1,0 +1,135 @@
+"""Programs in the style of the reference's recurrent benchmark models (its NASRNN cell loop,
+functs/benchmark/ai_model/nasrnn/nasrnn.py:39-101, and its seq2seq greedy decoder, a `while` loop
+that ends on a value computed on the device and writes one row of an int64 result per step,
+functs/benchmark/ai_model/seq2seq/seq2seq.py:95-142), written here as functions with the weights
+as arguments.  Their loops carry state, so they stay host loops around one fused region per step
+(the matrix products are ATen's); the tests check the graphs and, on the GPU, the results against
+eager mode (1e-4 relative after the recurrence, the decoder's tokens exactly)."""
+import pytest
+import torch
+from torch import Tensor
+
+import functs_amd.aot as aot
+import functs_amd.jit as fj
+
+
+def nas_cell_loop(inputs: Tensor, w_ih: Tensor, w_hh: Tensor):
+    """inputs [T, B, I]; w_ih [8, I, H]; w_hh [8, H, H]."""
+    state_c = torch.zeros(inputs.size(1), w_hh.size(2), device=inputs.device)
+    state_m = torch.zeros(inputs.size(1), w_hh.size(2), device=inputs.device)
+    for i in range(inputs.size(0)):
+        ih = torch.matmul(inputs[i], w_ih)
+        hh = torch.matmul(state_m, w_hh)
+        l1_0 = torch.sigmoid(ih[0] + hh[0])
+        l1_1 = torch.relu(ih[1] + hh[1])
+        l1_2 = torch.sigmoid(ih[2] + hh[2])
+        l1_3 = torch.relu(ih[3] + hh[3])
+        l1_4 = torch.tanh(ih[4] + hh[4])
+        l1_5 = torch.sigmoid(ih[5] + hh[5])
+        l1_6 = torch.tanh(ih[6] + hh[6])
+        l1_7 = torch.sigmoid(ih[7] + hh[7])
+        l2_0 = torch.tanh(torch.tanh(l1_0 * l1_1) + state_c)
+        l2_1 = torch.tanh(l1_2 + l1_3)
+        l2_2 = torch.tanh(l1_4 * l1_5)
+        l2_3 = torch.sigmoid(l1_6 + l1_7)
+        state_c = l2_0 * l2_1
+        state_m = torch.tanh(state_c * torch.tanh(l2_2 + l2_3))
+    return state_c + state_m
+
+
+def greedy_decoder(emb: Tensor, w_ih: Tensor, w_hh: Tensor, b_ih: Tensor, b_hh: Tensor, w_out: Tensor, b_out: Tensor,
+                   std: Tensor, h: Tensor, c: Tensor, max_length: int):
+    """emb [V, H]; w_ih / w_hh [4, H, H]; b_ih / b_hh [4, H]; w_out [H, V]; b_out [V]; std [L, B, V]
+    (a bias per step that steers the tokens); h, c [B, H].  Ends when every row emits token 0."""
+    batch = h.size(0)
+    tokens = torch.zeros(max_length, batch, dtype=torch.int64, device=h.device)
+    output = torch.full([batch], 1, dtype=torch.int64, device=h.device)
+    cond = True
+    step = 0
+    while cond:
+        x = emb[output]
+        ih = torch.matmul(x, w_ih)
+        hh = torch.matmul(h, w_hh)
+        ingate = torch.sigmoid(ih[0] + b_ih[0] + hh[0] + b_hh[0])
+        forgetgate = torch.sigmoid(ih[1] + b_ih[1] + hh[1] + b_hh[1])
+        cellgate = torch.tanh(ih[2] + b_ih[2] + hh[2] + b_hh[2])
+        outgate = torch.sigmoid(ih[3] + b_ih[3] + hh[3] + b_hh[3])
+        c = forgetgate * c + ingate * cellgate
+        h = outgate * torch.tanh(c)
+        output = (torch.matmul(h, w_out) + b_out + std[step]).argmax(1)
+        tokens[step] = output
+        step = step + 1
+        cond = bool((torch.max(output) > 0).item()) and step < max_length
+    return tokens, h
+
+
+def _nas_inputs(seed=0, T=12, B=2, I=64, H=64):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.rand(T, B, I, generator=g), (torch.rand(8, I, H, generator=g) - 0.5) * 0.3,
+            (torch.rand(8, H, H, generator=g) - 0.5) * 0.3]
+
+
+def _decoder_inputs(seed=0, V=50, H=32, B=3, L=9, stop_at=6):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: (torch.rand(*s, generator=g) - 0.5) * 0.4
+    std = torch.zeros(L, B, V)
+    for t in range(L):                      # steer: token 1 + t % 7 until stop_at, then token 0 for every row
+        std[t, :, 0 if t >= stop_at else 1 + t % 7] = 1000.0
+    return [r(V, H), r(4, H, H), r(4, H, H), r(4, H), r(4, H), r(H, V), r(V), std, r(B, H), r(B, H), L]
+
+
+def _kinds(block, out=None):
+    out = [] if out is None else out
+    for n in block.nodes():
+        out.append(n.kind())
+        for b in n.blocks():
+            _kinds(b, out)
+    return out
+
+
+def _cuda(args):
+    return [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
+
+
+def test_the_cell_of_a_step_is_one_region():
+    built = fj.build(fj.script(nas_cell_loop), _nas_inputs())
+    kinds = _kinds(built.graph)
+    assert kinds.count("prim::Loop") == 1 and kinds.count("aten::matmul") == 2
+    assert kinds.count("tssa::ParallelFunctor") == 1          # inside the loop: the whole cell
+    for k in ("aten::sigmoid", "aten::tanh", "aten::relu"):
+        assert k not in kinds                                  # nothing of the cell is left outside
+
+
+def test_the_decoder_is_functionalized_and_keeps_its_while_loop():
+    f = fj.script(greedy_decoder)
+    kinds = _kinds(f.graph)
+    assert "aten::copy_" not in kinds and "aten::index_put_" not in kinds
+    assert "immut::select_rev" in kinds                        # tokens[step] = output
+    built = fj.build(f, _decoder_inputs())
+    kinds = _kinds(built.graph)
+    assert kinds.count("prim::Loop") == 1 and "aten::item" in kinds
+
+
+@pytest.mark.gpu
+def test_nas_cell_loop_equals_eager():
+    args = _nas_inputs()
+    built = fj.build(fj.script(nas_cell_loop), args)
+    total0, _ = aot.launch_stats()
+    got = built(*_cuda(args))
+    torch.cuda.synchronize()
+    total1, _ = aot.launch_stats()
+    assert total1 - total0 == args[0].size(0)                  # one launch per step
+    torch.testing.assert_close(got.cpu(), nas_cell_loop(*args), rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("stop_at", [1, 6, 100])
+def test_greedy_decoder_equals_eager(stop_at):
+    args = _decoder_inputs(stop_at=stop_at)
+    built = fj.build(fj.script(greedy_decoder), args)
+    tokens, h = built(*_cuda(args))
+    ref_tokens, ref_h = greedy_decoder(*args)
+    assert torch.equal(tokens.cpu(), ref_tokens)
+    steps = min(stop_at + 1, args[-1])
+    assert int((ref_tokens.sum(1) > 0).sum()) == min(stop_at, args[-1]) and steps >= 1
+    torch.testing.assert_close(h.cpu(), ref_h, rtol=1e-4, atol=1e-6)

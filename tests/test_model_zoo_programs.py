@@ -5,6 +5,8 @@ functs/benchmark/ai_model/seq2seq/seq2seq.py:95-142), written here as functions 
 as arguments.  Their loops carry state, so they stay host loops around one fused region per step
 (the matrix products are ATen's); the tests check the graphs and, on the GPU, the results against
 eager mode (1e-4 relative after the recurrence, the decoder's tokens exactly)."""
+from typing import List
+
 import pytest
 import torch
 from torch import Tensor
@@ -63,6 +65,43 @@ def greedy_decoder(emb: Tensor, w_ih: Tensor, w_hh: Tensor, b_ih: Tensor, b_hh: 
     return tokens, h
 
 
+def fcos_levels(cls_scores: List[Tensor], bbox_preds: List[Tensor], centerness: List[Tensor], points: List[Tensor],
+                strides: List[float]):
+    """An anchor-free head in the style of the reference's FCOS post-processing
+    (functs/benchmark/ai_model/fcos/fcos_bbox.py): per level, NCHW maps are flattened, scores are
+    weighted by the centre-ness, boxes are decoded from distances to the four sides, and the rows
+    whose best class passes a threshold are kept.  Levels differ in size: a map with ragged tasks."""
+    out_boxes: List[Tensor] = []
+    out_scores: List[Tensor] = []
+    for i in range(len(cls_scores)):
+        cls = cls_scores[i]
+        scores = cls[0].permute(1, 2, 0).reshape(-1, cls.size(1)).sigmoid()
+        ctr = centerness[i][0].permute(1, 2, 0).reshape(-1).sigmoid()
+        dist = bbox_preds[i][0].permute(1, 2, 0).reshape(-1, 4) * strides[i]
+        scores = scores * ctr.unsqueeze(-1)
+        pts = points[i]
+        boxes = torch.stack([pts[:, 0] - dist[:, 0], pts[:, 1] - dist[:, 1], pts[:, 0] + dist[:, 2], pts[:, 1] + dist[:, 3]], -1)
+        best, _ = scores.max(1)
+        keep = best > 0.3
+        out_boxes.append(boxes[keep])
+        out_scores.append(scores[keep])
+    return out_boxes, out_scores
+
+
+def _fcos_inputs(seed=0, classes=20, sizes=((20, 24), (10, 12), (5, 6))):
+    g = torch.Generator().manual_seed(seed)
+    cls, box, ctr, pts, strides = [], [], [], [], []
+    for k, (h, w) in enumerate(sizes):
+        cls.append(torch.randn(1, classes, h, w, generator=g))
+        box.append(torch.rand(1, 4, h, w, generator=g) * 4)
+        ctr.append(torch.randn(1, 1, h, w, generator=g) + 1.0)
+        stride = 8.0 * 2 ** k
+        ys, xs = torch.meshgrid(torch.arange(h), torch.arange(w), indexing="ij")
+        pts.append(torch.stack([xs.reshape(-1), ys.reshape(-1)], -1).float() * stride + stride / 2)
+        strides.append(stride)
+    return [cls, box, ctr, pts, strides]
+
+
 def _nas_inputs(seed=0, T=12, B=2, I=64, H=64):
     g = torch.Generator().manual_seed(seed)
     return [torch.rand(T, B, I, generator=g), (torch.rand(8, I, H, generator=g) - 0.5) * 0.3,
@@ -88,7 +127,13 @@ def _kinds(block, out=None):
 
 
 def _cuda(args):
-    return [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
+    def go(a):
+        if isinstance(a, torch.Tensor):
+            return a.cuda()
+        if isinstance(a, list):
+            return [go(e) for e in a]
+        return a
+    return [go(a) for a in args]
 
 
 def test_the_cell_of_a_step_is_one_region():
@@ -133,3 +178,29 @@ def test_greedy_decoder_equals_eager(stop_at):
     steps = min(stop_at + 1, args[-1])
     assert int((ref_tokens.sum(1) > 0).sum()) == min(stop_at, args[-1]) and steps >= 1
     torch.testing.assert_close(h.cpu(), ref_h, rtol=1e-4, atol=1e-6)
+
+
+def test_the_anchor_free_head_is_one_map_over_ragged_levels():
+    built = fj.build(fj.script(fcos_levels), _fcos_inputs())
+    kinds = _kinds(built.graph)
+    fs = [n for n in built.graph.nodes() if n.kind() == "tssa::ParallelFunctor"]
+    assert "prim::Loop" not in kinds and len(fs) == 1
+    f = fs[0]
+    assert f.i("is_parallel_map") == 1 and f.i("compact_rows") == 1 and f.i("parallel_degree") == 3
+
+
+@pytest.mark.gpu
+def test_anchor_free_head_equals_eager():
+    args = _fcos_inputs()
+    built = fj.build(fj.script(fcos_levels), args)
+    total0, _ = aot.launch_stats()
+    boxes, scores = built(*_cuda(args))
+    torch.cuda.synchronize()
+    total1, _ = aot.launch_stats()
+    assert total1 - total0 == 2                                # count + scatter over the three levels together
+    ref_boxes, ref_scores = fcos_levels(*args)
+    assert [t.shape for t in boxes] == [t.shape for t in ref_boxes] and sum(t.shape[0] for t in ref_boxes) > 50
+    for a, b in zip(boxes, ref_boxes):
+        torch.testing.assert_close(a.cpu(), b, rtol=1e-5, atol=1e-5)
+    for a, b in zip(scores, ref_scores):
+        torch.testing.assert_close(a.cpu(), b, rtol=1e-5, atol=1e-7)

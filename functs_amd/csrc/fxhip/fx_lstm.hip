@@ -26,6 +26,15 @@
 #define FX_LSTM_BLOCK 256
 #define FX_LSTM_MAXB 16
 #define FX_LSTM_UPW 2   // hidden units per workgroup
+#ifndef FX_LSTM_FIRST_LOOK
+#define FX_LSTM_FIRST_LOOK 8
+#endif
+// hooks for timing the phases of a step in a test build; nothing in the library
+#ifndef FX_LSTM_STAMP
+#define FX_LSTM_STAMP(k)
+#define FX_LSTM_STAMP_END()
+#define FX_LSTM_STAMP_DECL
+#endif
 
 namespace {
 // Everything that crosses workgroups (the tagged h values, the control words) is written and read
@@ -47,6 +56,20 @@ struct DevAtomics {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 };
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// every lane gets the sum over its row of 16 lanes: neighbours, pairs, then the mirrored half rows and rows
+__device__ __forceinline__ float row_sum(float v) {
+  v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141>(v);   // row_half_mirror
+  v = dpp_add<0x140>(v);   // row_mirror
+  return v;
+}
+__device__ __forceinline__ float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
 }  // namespace
 
 // 1024 workgroups (HPT = 32) are resident together only at four waves per SIMD, i.e. within 128
@@ -55,15 +78,21 @@ template <int L, int HPT, int UPW>
 __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lstm_stack_kernel(const FxLstmArgs a) {
   // the input vectors of one batch row of a step: x[t] and, per layer, the h it reads
   extern __shared__ __attribute__((aligned(16))) float s_vec[];   // [L + 1][H]
-  __shared__ float s_gate[UPW][L][FX_LSTM_MAXB][4];
+  __shared__ float s_gate[2][UPW][L][FX_LSTM_MAXB][4];   // activated gates, by parity of the step
   __shared__ uint32_t s_abort;
+  FX_LSTM_STAMP_DECL
   constexpr int NT = FX_LSTM_BLOCK * UPW;                             // threads: four waves per hidden unit
   constexpr int HH = HPT * 32;                                        // H
   constexpr int EPT = (HH + NT - 1) / NT;                             // elements of a vector per thread
   const int H = a.H, B = a.B, T = a.T;
   const int tid = (int)threadIdx.x;
   const int ul = tid / FX_LSTM_BLOCK;                                 // which of the workgroup's units
-  const int u = (int)blockIdx.x * UPW + ul;
+  // Workgroups go to the chip's eight dies in turn, and every die has a cache of its own: the
+  // workgroups of a die take neighbouring hidden units, so that a die fetches its eighth of every
+  // weight row once (lines of a row are shared by 32 units) instead of every die fetching all of it.
+  const int n_wg = (int)gridDim.x;
+  const int wg = (n_wg % 8 == 0) ? ((int)blockIdx.x % 8) * (n_wg / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
+  const int u = wg * UPW + ul;
   const int lane = (int)(threadIdx.x & 63u), gate = (int)((threadIdx.x >> 6) & 3u);
   const int half = lane >> 5, sub = lane & 31;
   if (threadIdx.x == 0) s_abort = 0u;
@@ -91,6 +120,7 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
   for (int d = 0; d < n_steps; ++d) {
     const int rp = (d + 1) & 1;   // parity written by step d - 1
     const uint32_t want = fx_lstm_tag_read(base, d);
+    FX_LSTM_STAMP(0);
     for (int b = 0; b < B; ++b) {
       // --- the workgroup fetches the vectors of a batch row once, for all its waves ---
       // slot 0: x[t] (layer 0 active); slot j + 1: what layer j reads as its own previous h, which
@@ -105,38 +135,46 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
             if (tid + k * NT < HH) s_vec[tid + k * NT] = xr[tid + k * NT];
         }
       }
-      const uint64_t* src[L];   // tagged sources of this step (null: the slot is not tagged or not needed)
+      FX_LSTM_STAMP(1);
+      // tagged sources of this step.  A slot that is not tagged or not needed is loaded all the same
+      // (and ignored): the loads of a round are then issued together, without a branch and a wait
+      // between them, and a round takes one trip to the memory side instead of one per layer.
+      bool need[L];
+      const uint64_t* src[L];
 #pragma unroll
       for (int j = 0; j < L; ++j) {
         const int tj = fx_lstm_time(d, j, T);
         const bool next_active = j + 1 < L && fx_lstm_time(d, j + 1, T) >= 0;
-        src[j] = nullptr;
+        need[j] = false;
+        src[j] = a.hbuf + fx_lstm_hoff(rp, j, b, 0, L, B, H);
         if (tj == 0) {
           const float* hr = a.h0 ? a.h0 + ((size_t)j * B + b) * H : nullptr;
 #pragma unroll
           for (int k = 0; k < EPT; ++k)
             if (tid + k * NT < HH) s_vec[(j + 1) * HH + tid + k * NT] = hr ? hr[tid + k * NT] : 0.0f;
         } else if (tj > 0 || next_active) {
-          src[j] = a.hbuf + fx_lstm_hoff(rp, j, b, 0, L, B, H);
+          need[j] = true;
         }
       }
       {
         float val[L][EPT];
         uint32_t polls = 0;
+        __builtin_amdgcn_s_sleep(FX_LSTM_FIRST_LOOK);
         for (;;) {
           bool ready = true;
+          uint64_t e[L][EPT];
 #pragma unroll
-          for (int j = 0; j < L; ++j) {
-            if (!src[j]) continue;
+          for (int j = 0; j < L; ++j)
+#pragma unroll
+            for (int k = 0; k < EPT; ++k)
+              e[j][k] = __hip_atomic_load(src[j] + min(tid + k * NT, HH - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int j = 0; j < L; ++j)
 #pragma unroll
             for (int k = 0; k < EPT; ++k) {
-              if (tid + k * NT < HH) {
-                const uint64_t e = __hip_atomic_load(src[j] + tid + k * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ready = ready && fx_lstm_tag_of(e) == want;
-                val[j][k] = __uint_as_float((uint32_t)e);
-              }
+              ready = ready && (!need[j] || tid + k * NT >= HH || fx_lstm_tag_of(e[j][k]) == want);
+              val[j][k] = __uint_as_float((uint32_t)e[j][k]);
             }
-          }
           if (ready) break;
           if (++polls > a.spin_limit || ((polls & 255u) == 0u && DevAtomics::load(a.ctl + FX_LSTM_W_ERR) != 0u)) {
             // given up (or somebody else has): the workgroup leaves at the end of this step's reads
@@ -147,15 +185,17 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
           }
           __builtin_amdgcn_s_sleep(1);
         }
+        FX_LSTM_STAMP(2);
 #pragma unroll
         for (int j = 0; j < L; ++j) {
-          if (!src[j]) continue;
+          if (!need[j]) continue;
 #pragma unroll
           for (int k = 0; k < EPT; ++k)
             if (tid + k * NT < HH) s_vec[(j + 1) * HH + tid + k * NT] = val[j][k];
         }
       }
       __syncthreads();
+      FX_LSTM_STAMP(3);
       // --- dot products: lanes 0-31 the layer's input, lanes 32-63 its own previous h ---
 #pragma unroll
       for (int j = 0; j < L; ++j) {
@@ -164,21 +204,25 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
         float s = 0.0f;
 #pragma unroll
         for (int m = 0; m < HPT; ++m) s = __builtin_fmaf(w[j][m], vsrc[sub + 32 * m], s);
-#pragma unroll
-        for (int o = 16; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
-        const float other = __shfl(s, 32, 64);   // the hh half's sum, for lane 0
-        if (lane == 0) s_gate[ul][j][b][gate] = (s + b_ih[j]) + (other + b_hh[j]);
+        // sums over the rows of 16 lanes inside the vector unit, then the four row sums through
+        // scalar registers: lanes 0-31 are the input's half, lanes 32-63 the half of the own h
+        s = row_sum(s);
+        const float ih = lane_value(s, 0) + lane_value(s, 16);
+        const float hh = lane_value(s, 32) + lane_value(s, 48);
+        const float g = (ih + b_ih[j]) + (hh + b_hh[j]);
+        // every gate's wave applies its own activation; the owner is left with the cell update
+        if (lane == 0) s_gate[d & 1][ul][j][b][gate] = gate == 2 ? fx_tanh(g) : fx_sigmoid(g);
       }
+      FX_LSTM_STAMP(4);
       __syncthreads();   // the vectors are overwritten by the next batch row; the gates are complete
+      FX_LSTM_STAMP(5);
     }
     if (s_abort != 0u) return;   // a wait was given up: every wave of the workgroup leaves, nothing is checked out
     if (owner) {
       const int t = fx_lstm_time(d, own_j, T);
       if (t >= 0) {
-        const float ig = fx_sigmoid(s_gate[ul][own_j][own_b][0]);
-        const float fg = fx_sigmoid(s_gate[ul][own_j][own_b][1]);
-        const float gg = fx_tanh(s_gate[ul][own_j][own_b][2]);
-        const float og = fx_sigmoid(s_gate[ul][own_j][own_b][3]);
+        const float* gt = s_gate[d & 1][ul][own_j][own_b];
+        const float ig = gt[0], fg = gt[1], gg = gt[2], og = gt[3];
         c_reg = (fg * c_reg) + (ig * gg);
         const float h = og * fx_tanh(c_reg);
         DevAtomics::store64(a.hbuf + fx_lstm_hoff(d & 1, own_j, own_b, u, L, B, H),
@@ -190,8 +234,11 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
         }
       }
     }
-    __syncthreads();   // the gates have been read before the next step overwrites them
+    // no barrier here: the next step writes the gates of the other parity, and the one after it
+    // comes behind two barriers that the owners pass only after they have read these
+    FX_LSTM_STAMP(6);
   }
+  FX_LSTM_STAMP_END();
   if (threadIdx.x == 0)
     fx_lstm_leave<DevAtomics>(a.ctl, gridDim.x, base, (uint32_t)n_steps, a.hbuf, (uint32_t)(2 * L * B * H));
 }

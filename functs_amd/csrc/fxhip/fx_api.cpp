@@ -1139,7 +1139,7 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
   const int rc = fx_launch_lstm_stack(a, layers, (hipStream_t)stream_);
   if (rc == 1) return fail(FX_E_UNSUPPORTED, "fx_lstm_stack: no kernel for these sizes");
   if (rc == 2)
-    return fail(FX_E_LIMIT, "fx_lstm_stack: " + std::to_string(hidden) + " workgroups would not be resident together on this device");
+    return fail(FX_E_LIMIT, "fx_lstm_stack: " + std::to_string(hidden / 2) + " workgroups of 512 threads would not be resident together on this device");
   if (rc != 0) return fail(FX_E_HIP, std::string("fx_lstm_stack: ") + hipGetErrorString((hipError_t)(rc - 100)));
   g_launches.fetch_add(1, std::memory_order_relaxed);
   g_spec_launches.fetch_add(1, std::memory_order_relaxed);

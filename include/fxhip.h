@@ -340,15 +340,16 @@ int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* co
  *     out[t] = cur
  * which the reference runs on the host, one fused kernel and two library GEMMs per (t, j)
  * (the loops carry state: fait/passes/parallelize_loops.cpp:17, unroll_loops.cpp:59-65), as ONE
- * persistent kernel: a workgroup per hidden unit keeps its columns of the weights in registers
- * for the whole sequence; the diagonals t + j follow each other without a barrier, every h value
+ * persistent kernel: a workgroup per two hidden units keeps their columns of the weights in
+ * registers for the whole sequence (thread k row k of them, and element k of the step's vectors);
+ * the diagonals t + j follow each other without a barrier between workgroups, every h value
  * travels with the tag of the step that wrote it and readers poll for the tag they expect, with
  * bounded waits (a wait that is given up reports FX_ASYNC_BARRIER through fx_async_error and ends
  * the kernel).
  * Contiguous fp32: x [T, B, H]; wih, whh [L, 4, H, H]; bih, bhh [L, 4, 1, H]; h0, c0, state_h,
  * state_c [L, B, H]; out [T, B, H]; h0 / c0 may be null (zero initial state).  H is 32, 64, ...
- * 1024 (a power of two), L <= 4, B <= 16 (FX_E_UNSUPPORTED otherwise), and H workgroups must be
- * resident together (FX_E_LIMIT).
+ * 1024 (a power of two), L <= 4, B <= 16 (FX_E_UNSUPPORTED otherwise), and H / 2 workgroups of
+ * 512 threads must be resident together (FX_E_LIMIT).
  * workspace: fx_lstm_stack_workspace_bytes() of device memory, 256-byte aligned, all zero when it
  * is used for the first time.  A launch that ends without error leaves it ready for the next one,
  * so one workspace, cleared once, serves launch after launch on one stream as long as batch,

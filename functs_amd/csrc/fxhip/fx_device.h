@@ -229,7 +229,12 @@ __device__ __forceinline__ float fx_sigmoid(float x) {
   const float tl = __builtin_fmaf(nx, l2e_hi, -th) + nx * l2e_lo;
   float e = __builtin_amdgcn_exp2f(th);
   e = __builtin_fmaf(e, tl * ln2, e);
-  return __builtin_amdgcn_rcpf(1.0f + e);
+  float r = __builtin_amdgcn_rcpf(1.0f + e);
+  // below about -88.7 (and at -inf) exp2 overflows and the correction term makes inf - inf; at +inf
+  // the low word is inf - inf.  NaN inputs fail both comparisons and stay NaN.
+  r = (th > 128.0f) ? 0.0f : r;
+  r = (th < -150.0f) ? 1.0f : r;
+  return r;
 }
 
 // exp through the hardware exp2 with a two-word log2(e): about 1.2e-7 relative error

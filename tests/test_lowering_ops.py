@@ -432,3 +432,20 @@ def test_tril_and_triu_over_every_diagonal(backend):
     for d in diags:
         refs += [torch.tril(t, d), torch.triu(t, d)]
     assert_exact(got, refs, "tril/triu")
+
+
+def test_transcendentals_at_the_ends_of_the_range(backend):
+    """sigmoid / tanh / exp where exp overflows or underflows, at the infinities and at NaN: the
+    eager kernels the reference runs there (ATen) return 0, 1, +-1, inf, NaN, never a NaN made on
+    the way."""
+    r = Region()
+    x = r.tensor_input(torch.float32, 1)
+    r.output(x.sigmoid())
+    r.output(x.tanh())
+    r.output(x.exp())
+    r.finalize()
+    t = torch.tensor([float("-inf"), -1e30, -200.0, -104.0, -100.0, -90.0, -88.8, -88.0, -20.0, -0.0, 0.0, 20.0, 88.0,
+                      88.8, 100.0, 200.0, 1e30, float("inf"), float("nan")] * 7)
+    sig, tanh, exp = run_region(backend, r, t)
+    for got, ref in ((sig, t.sigmoid()), (tanh, t.tanh()), (exp, t.exp())):
+        torch.testing.assert_close(got, ref, rtol=1e-5, atol=1e-37, equal_nan=True)

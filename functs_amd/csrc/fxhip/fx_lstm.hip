@@ -28,7 +28,7 @@
 #define FX_LSTM_MAXB 16
 #define FX_LSTM_UPW 2   // hidden units per workgroup
 #ifndef FX_LSTM_FIRST_LOOK
-#define FX_LSTM_FIRST_LOOK 9   // units of 64 clocks; 8 to 10 are equally good on the benchmark shape, 0 and 16 cost 40 and 8 %
+#define FX_LSTM_FIRST_LOOK 8   // units of 64 clocks; 7 to 10 are within 4 % of each other on the benchmark shape, 0 and 16 cost 40 and 8 %
 #endif
 // hooks for timing the phases of a step in a test build; nothing in the library
 #ifndef FX_LSTM_STAMP
@@ -273,28 +273,40 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
         if ((lane & 3) == 0) s_part[it & 1][g][wave][lane >> 2] = total;
       }
       FX_LSTM_STAMP(4);
+      // the cell states of this batch row, read ahead of the barrier (a lane reads what it wrote itself)
+      float c_prev[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) c_prev[g] = wave == 0 ? s_c[b][(lane & 15) + 16 * g] : 0.0f;
       __syncthreads();
       FX_LSTM_STAMP(5);
-      if (s_abort != 0u) return;   // a wait was given up: every wave of the workgroup leaves, nothing is checked out
-      // --- sixteen lanes a pair of layers: biases, gates, cells ---
-      if (wave == 0) {
+      // A wait that was given up: every wave of the workgroup leaves, nothing is checked out.  The
+      // first wave looks at the word together with the waves' sums and leaves before it would store.
+      if (wave != 0) {
+        if (s_abort != 0u) return;
+      } else {
+        // --- sixteen lanes a pair of layers: biases, gates, cells ---
+        float part[NG][NW];
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+          for (int w = 0; w < NW; ++w) part[g][w] = s_part[it & 1][g][w][lane & 15];
+        const uint32_t aborted = s_abort;
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
-          float sum = 0.0f;
 #pragma unroll
-          for (int w = 0; w < NW; ++w) sum += s_part[it & 1][g][w][lane & 15];
-          // lanes 0-15 of the wave: value lane >> 2 ... of THIS pair; the value index of a lane here is
-          // lane & 15 = (jl * 2 + ul) * 4 + gate
+          for (int span = 1; span < NW; span *= 2)
+#pragma unroll
+            for (int w = 0; w + span < NW; w += 2 * span) part[g][w] += part[g][w + span];
+          // the value of a lane here is lane & 15 = (layer in the pair * 2 + unit) * 4 + gate, as for the biases
           const int v = lane & 15, gt = v & 3, ul = (v >> 2) & 1, j = 2 * g + (v >> 3);
-          // the biases were loaded for lane = 4 * value + gate; here lane & 15 = 4 * (jl * 2 + ul) + gate: the same
-          const float pre = (sum + f_bias_ih[g]) + f_bias_hh[g];
+          const float pre = (part[g][0] + f_bias_ih[g]) + f_bias_hh[g];
           const float act = gt == 2 ? fx_tanh(pre) : fx_sigmoid(pre);
           const float fg = quad_lane<1>(act), gg = quad_lane<2>(act), og = quad_lane<3>(act);
           const int t = (j < L) ? fx_lstm_time(d, j, T) : -1;
+          if (g == 0 && aborted != 0u) return;
           if (lane < 16 && gt == 0 && t >= 0) {
-            const int cl = lane + 16 * g;
-            const float c = (fg * s_c[b][cl]) + (act * gg);
-            s_c[b][cl] = c;
+            const float c = (fg * c_prev[g]) + (act * gg);
+            s_c[b][lane + 16 * g] = c;
             const float h = og * fx_tanh(c);
             const int u = u0 + ul;
             DevAtomics::store64(a.hbuf + fx_lstm_hoff(d & 1, j, b, u, L, B, H),

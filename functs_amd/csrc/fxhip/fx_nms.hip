@@ -13,8 +13,9 @@
 //   2. bitonic sort of the keys: descending score, equal scores by ascending index (a stable
 //      descending sort);
 //   3. candidates are taken 64 at a time in that order.  Each is tested against the kept list
-//      (16 threads per candidate), the 64 x 64 overlaps inside the chunk become one 64-bit row
-//      per candidate, and one wave resolves the chunk in order with register shuffles.  The
+//      (16 threads per candidate), the 64 x 64 overlaps inside the chunk become one 64-bit word
+//      per candidate (its overlapping predecessors), and one wave resolves the chunk: all
+//      candidates decide together in rounds, as many as the longest chain of overlaps.  The
 //      walk ends when max_num boxes are kept: later candidates cannot change earlier decisions.
 // The workspace counters are zero when a launch starts and zero again when it ends.
 // The number of valid rows per task is read from memory (device or pinned host), so the count a
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   __shared__ float s_carea[FX_NMS_CHUNK];
   __shared__ uint32_t s_cidx[FX_NMS_CHUNK], s_clabel[FX_NMS_CHUNK];
   __shared__ float s_cscore[FX_NMS_CHUNK];
-  __shared__ uint32_t s_sup[FX_NMS_CHUNK][2];   // later candidates of the chunk that candidate i overlaps
+  __shared__ uint32_t s_in[FX_NMS_CHUNK][2];    // earlier candidates of the chunk that overlap candidate j
   __shared__ uint32_t s_dead[2];                // candidates of the chunk that the kept list overlaps
   __shared__ uint32_t s_count, s_maxc, s_nk, s_base, s_ticket;
 
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   for (uint32_t pos = 0; pos < count && nk < d.max_num; pos += FX_NMS_CHUNK) {
     const uint32_t m = min(FX_NMS_CHUNK, count - pos);
     if (tid < FX_NMS_CHUNK) {
-      s_sup[tid][0] = 0u; s_sup[tid][1] = 0u;
+      s_in[tid][0] = 0u; s_in[tid][1] = 0u;
       if (tid < 2u) s_dead[tid] = 0u;
       if (tid < m) {
         const uint64_t key = s_keys[pos + tid];
@@ -311,36 +312,45 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
       if (i < m) {
         const Box ib{s_obox[i][0], s_obox[i][1], s_obox[i][2], s_obox[i][3]};
         const float ia = s_carea[i];
-        uint32_t bits = 0u;
 #pragma unroll
         for (uint32_t jj = 0; jj < 4u; ++jj) {
           const uint32_t j = j0 + jj;
           if (j > i && j < m) {
             const Box jb{s_obox[j][0], s_obox[j][1], s_obox[j][2], s_obox[j][3]};
-            if (overlaps(ib, ia, jb, s_carea[j], d.iou_thr)) bits |= 1u << (j & 31u);
+            if (overlaps(ib, ia, jb, s_carea[j], d.iou_thr)) atomicOr(&s_in[j][i >> 5], 1u << (i & 31u));
           }
         }
-        if (bits) atomicOr(&s_sup[i][j0 >> 5], bits);   // the four candidates lie in one word
       }
     }
     __syncthreads();
     if (wave == 0u) {
-      // in order: candidate i is kept unless something kept before it overlaps it
-      const uint32_t sup_lo = s_sup[lane][0], sup_hi = s_sup[lane][1];
-      uint64_t dead = ((uint64_t)s_dead[1] << 32) | (uint64_t)s_dead[0];
-      uint64_t keep = 0ull;
-      uint32_t kept_now = 0u;
-      const uint32_t room = d.max_num - nk;
-      for (uint32_t i = 0; i < m && kept_now < room; ++i) {
-        const uint32_t lo = (uint32_t)__shfl((int)sup_lo, (int)i, 64), hi = (uint32_t)__shfl((int)sup_hi, (int)i, 64);
-        if (((dead >> i) & 1ull) == 0ull) {
-          keep |= 1ull << i;
-          dead |= ((uint64_t)hi << 32) | (uint64_t)lo;
-          ++kept_now;
-        }
+      // In order, candidate i is kept unless a kept one before it overlaps it.  All candidates
+      // decide together, round after round: one with a kept overlapping predecessor is dead, one
+      // whose overlapping predecessors are all dead is kept, the others wait; the first undecided
+      // candidate always decides, and with few overlaps two or three rounds settle the chunk
+      // (a walk from candidate to candidate costs 64 dependent steps).
+      const uint64_t in = ((uint64_t)s_in[lane][1] << 32) | (uint64_t)s_in[lane][0];
+      const uint64_t valid = m >= 64u ? ~0ull : (1ull << m) - 1ull;
+      uint64_t deadm = (((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)s_dead[1]) << 32) |
+                        (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)s_dead[0])) | ~valid;
+      uint64_t keptm = 0ull;
+      bool decided = ((deadm >> lane) & 1ull) != 0ull;
+      for (;;) {
+        const bool now_dead = !decided && (in & keptm) != 0ull;
+        const bool now_kept = !decided && !now_dead && (in & ~deadm) == 0ull;
+        const uint64_t nd = __ballot(now_dead), nkp = __ballot(now_kept);
+        if ((nd | nkp) == 0ull) break;
+        deadm |= nd;
+        keptm |= nkp;
+        decided = decided || now_dead || now_kept;
       }
+      // the walk ends when max_num are kept: the first `room` of them in order
+      const uint32_t room = d.max_num - nk;
+      const uint32_t rank = (uint32_t)__popcll(keptm & ((1ull << lane) - 1ull));
+      const uint64_t keep = __ballot(((keptm >> lane) & 1ull) != 0ull && rank < room);
+      const uint32_t kept_now = (uint32_t)__popcll(keep);
       if ((keep >> lane) & 1ull) {
-        const uint32_t slot = nk + (uint32_t)__popcll(keep & ((1ull << lane) - 1ull));
+        const uint32_t slot = nk + rank;
         s_kbox[slot][0] = s_obox[lane][0]; s_kbox[slot][1] = s_obox[lane][1];
         s_kbox[slot][2] = s_obox[lane][2]; s_kbox[slot][3] = s_obox[lane][3];
         s_karea[slot] = s_carea[lane];

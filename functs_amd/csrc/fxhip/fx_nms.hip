@@ -118,7 +118,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   __syncthreads();   // s_base is used again below
 
   FX_NMS_STAMP(0);
-  // 1. candidates: four 128-bit loads per thread in flight, one LDS atomic per wave and round
+  // 1. candidates: four 128-bit loads per thread in flight
   const uint32_t all_items = rows * C;   // < 2^32 (host)
   // this workgroup's share: a multiple of four items, so that its 128-bit loads stay aligned
   const uint32_t share = (((all_items + slices - 1u) / slices) + 3u) & ~3u;
@@ -145,18 +145,10 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
 #pragma unroll
       for (uint32_t e = 0; e < 4u; ++e)
         if (v[u][e] > d.score_thr) mine |= 1u << (u * 4u + e);
-    const uint32_t cnt = (uint32_t)__popc(mine);
-    uint32_t incl = cnt;   // inclusive scan over the wave
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const uint32_t t = (uint32_t)__shfl_up((int)incl, o, 64);
-      if ((int)lane >= o) incl += t;
-    }
-    const uint32_t wave_total = (uint32_t)__shfl((int)incl, 63, 64);
-    if (wave_total == 0u) continue;
-    uint32_t wbase = 0u;
-    if (lane == 0u) wbase = atomicAdd(&s_count, wave_total);
-    uint32_t slot = (uint32_t)__shfl((int)wbase, 0, 64) + incl - cnt;
+    // few elements pass a detector's threshold: a lane that has some takes its places with one LDS
+    // atomic (the order of arrival does not matter), the others go straight on to the next loads
+    if (mine == 0u) continue;
+    uint32_t slot = atomicAdd(&s_count, (uint32_t)__popc(mine));
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u)
 #pragma unroll

@@ -219,6 +219,30 @@ def test_batched_nms_equals_the_oracle(n, classes):
 
 
 @pytest.mark.gpu
+def test_a_chain_of_overlaps_is_resolved_in_order():
+    """Every box overlaps only its neighbours in score order (IoU 7/13 with the next, 1/4 with the one
+    after): whether a box is kept depends on all boxes before it, the longest chain a chunk can hold."""
+    from functs_amd import detection
+    n = 300
+    x = torch.arange(n, dtype=torch.float32) * 3.0
+    b = torch.stack([x, torch.zeros(n), x + 10.0, torch.full((n,), 5.0)], 1)
+    s = torch.linspace(0.99, 0.01, n)
+    lab = torch.zeros(n, dtype=torch.int64)
+    dets, keep = onms.batched_nms(b, s, lab)
+    assert keep.tolist() == list(range(0, n, 2))                  # every other box
+    dev = torch.device("cuda:0")
+    gd, gk = detection.batched_nms(b.to(dev), s.to(dev), lab.to(dev))
+    assert gk.cpu().tolist() == keep.tolist() and torch.equal(gd.cpu(), dets)
+    # the same chain broken in places: a gap starts a new chain
+    b2 = b.clone()
+    b2[97:, 0] += 100.0
+    b2[97:, 2] += 100.0
+    dets, keep = onms.batched_nms(b2, s, lab)
+    gd, gk = detection.batched_nms(b2.to(dev), s.to(dev), lab.to(dev))
+    assert gk.cpu().tolist() == keep.tolist() and torch.equal(gd.cpu(), dets)
+
+
+@pytest.mark.gpu
 def test_more_candidates_than_the_launch_is_sized_for_is_reported():
     from functs_amd import detection
     from functs_amd._lib import FxError

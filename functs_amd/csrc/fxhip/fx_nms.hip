@@ -49,6 +49,35 @@ __device__ __forceinline__ float from_orderable(uint32_t o) {
   return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
 }
 
+// the value of lane (own lane ^ J), inside the vector unit
+template <uint32_t J>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v, uint32_t lane) {
+  typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+  if constexpr (J == 1u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false);        // quad_perm [1, 0, 3, 2]
+  else if constexpr (J == 2u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
+  else if constexpr (J == 4u) {
+    // a rotation of the row of 16 by 4 one way and the other; which of the two is lane ^ 4 depends on bit 2
+    const uint32_t from_below = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xf, 0xf, false);   // row_ror:4: from lane - 4
+    const uint32_t from_above = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x12C, 0xf, 0xf, false);   // row_ror:12: from lane + 4
+    return (lane & 4u) ? from_below : from_above;
+  } else if constexpr (J == 8u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);   // row_ror:8
+  else if constexpr (J == 16u) {
+    const u32x2v t = __builtin_amdgcn_permlane16_swap(v, v, false, false);   // x: rows 0, 0, 2, 2; y: rows 1, 1, 3, 3
+    return (lane & 16u) ? t.x : t.y;
+  } else {
+    const u32x2v t = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // x: lower half twice; y: upper half twice
+    return (lane & 32u) ? t.x : t.y;
+  }
+}
+// one stage of the bitonic network on a key a lane, partners J lanes apart: the lower lane keeps
+// the smaller key where the run ascends
+template <uint32_t J>
+__device__ __forceinline__ uint64_t bitonic_step(uint64_t key, bool up, uint32_t lane) {
+  const uint64_t other = ((uint64_t)lane_xor<J>((uint32_t)(key >> 32), lane) << 32) | (uint64_t)lane_xor<J>((uint32_t)key, lane);
+  const bool keep_min = ((lane & J) == 0u) == up;
+  return ((key < other) == keep_min) ? key : other;
+}
+
 struct Box { float x1, y1, x2, y2; };
 
 __device__ __forceinline__ bool overlaps(const Box& a, float area_a, const Box& b, float area_b, float thr) {
@@ -241,11 +270,25 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   };
   auto narrow_stages = [&](uint32_t k_first, uint32_t k_last) {   // every stage j <= 64 of phases k_first .. k_last
     for (uint32_t blk = wave; blk < (n2 >> 7); blk += FX_NMS_THREADS / 64u) {
-      for (uint32_t k = k_first; k <= k_last; k <<= 1)
-        for (uint32_t j = min(k >> 1, 64u); j > 0u; j >>= 1) {
-          exchange((blk << 7) + (((lane & ~(j - 1u)) << 1) | (lane & (j - 1u))), j, k);
-          __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      // the block's 128 keys in registers, two a lane (positions lane and lane + 64): the stages
+      // exchange them between lanes, LDS is read and written once per call
+      const uint32_t p0 = (blk << 7) + lane;
+      uint64_t ka = s_keys[p0], kb = s_keys[p0 + 64u];
+      for (uint32_t k = k_first; k <= k_last; k <<= 1) {
+        const bool up_a = (p0 & k) == 0u, up_b = ((p0 + 64u) & k) == 0u;
+        if (k >= 128u) {   // partners 64 apart: the lane's own two keys (up_a == up_b here)
+          const bool sw = (ka > kb) == up_a;
+          const uint64_t lo = sw ? kb : ka, hi = sw ? ka : kb;
+          ka = lo; kb = hi;
         }
+        if (k >= 64u) { ka = bitonic_step<32>(ka, up_a, lane); kb = bitonic_step<32>(kb, up_b, lane); }
+        if (k >= 32u) { ka = bitonic_step<16>(ka, up_a, lane); kb = bitonic_step<16>(kb, up_b, lane); }
+        if (k >= 16u) { ka = bitonic_step<8>(ka, up_a, lane); kb = bitonic_step<8>(kb, up_b, lane); }
+        if (k >= 8u) { ka = bitonic_step<4>(ka, up_a, lane); kb = bitonic_step<4>(kb, up_b, lane); }
+        if (k >= 4u) { ka = bitonic_step<2>(ka, up_a, lane); kb = bitonic_step<2>(kb, up_b, lane); }
+        ka = bitonic_step<1>(ka, up_a, lane); kb = bitonic_step<1>(kb, up_b, lane);
+      }
+      s_keys[p0] = ka; s_keys[p0 + 64u] = kb;
     }
   };
   narrow_stages(2u, 128u);

@@ -114,14 +114,14 @@ __global__ __launch_bounds__(NT) void fx_classmap_head(const FxCmapLaunch hl, co
       for (uint32_t j = 0; j < 4; ++j)
         if (c0 + j < C) m[k] = fx_fmax(m[k], x[k][j]);
     }
-#pragma unroll
-    for (int o = 16; o >= 1; o >>= 1) {
-      float t[RPH];
-#pragma unroll
-      for (uint32_t k = 0; k < RPH; ++k) t[k] = __shfl_xor(m[k], o, 64);
-#pragma unroll
-      for (uint32_t k = 0; k < RPH; ++k) m[k] = fx_fmax(m[k], t[k]);
-    }
+#define FX_CMAP_STEP(O)                                                              \
+  {                                                                                  \
+    float t[RPH];                                                                    \
+    _Pragma("unroll") for (uint32_t k = 0; k < RPH; ++k) t[k] = fx_lane_xor_f<(O)>(m[k], lane); \
+    _Pragma("unroll") for (uint32_t k = 0; k < RPH; ++k) m[k] = fx_fmax(m[k], t[k]); \
+  }
+    FX_CMAP_STEP(16u) FX_CMAP_STEP(8u) FX_CMAP_STEP(4u) FX_CMAP_STEP(2u) FX_CMAP_STEP(1u)
+#undef FX_CMAP_STEP
 #pragma unroll
     for (uint32_t k = 0; k < RPH; ++k) {
       v[k] = 0.0f;
@@ -131,14 +131,14 @@ __global__ __launch_bounds__(NT) void fx_classmap_head(const FxCmapLaunch hl, co
         if (c0 + j < C) v[k] = v[k] + e[k][j];
       }
     }
-#pragma unroll
-    for (int o = 16; o >= 1; o >>= 1) {
-      float t[RPH];
-#pragma unroll
-      for (uint32_t k = 0; k < RPH; ++k) t[k] = __shfl_xor(v[k], o, 64);
-#pragma unroll
-      for (uint32_t k = 0; k < RPH; ++k) v[k] = v[k] + t[k];
-    }
+#define FX_CMAP_STEP(O)                                                              \
+  {                                                                                  \
+    float t[RPH];                                                                    \
+    _Pragma("unroll") for (uint32_t k = 0; k < RPH; ++k) t[k] = fx_lane_xor_f<(O)>(v[k], lane); \
+    _Pragma("unroll") for (uint32_t k = 0; k < RPH; ++k) v[k] = v[k] + t[k];         \
+  }
+    FX_CMAP_STEP(16u) FX_CMAP_STEP(8u) FX_CMAP_STEP(4u) FX_CMAP_STEP(2u) FX_CMAP_STEP(1u)
+#undef FX_CMAP_STEP
 #pragma unroll
     for (uint32_t k = 0; k < RPH; ++k) {
       const uint32_t row = hw + k * (NT / 32u);

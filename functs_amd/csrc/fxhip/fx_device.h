@@ -267,6 +267,31 @@ __device__ __forceinline__ float fx_tanh(float x) {
   return ax < 0.625f ? small : big;
 }
 
+// the value of lane (own lane ^ J), inside the vector unit
+template <uint32_t J>
+__device__ __forceinline__ uint32_t fx_lane_xor(uint32_t v, uint32_t lane) {
+  typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+  if constexpr (J == 1u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false);        // quad_perm [1, 0, 3, 2]
+  else if constexpr (J == 2u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
+  else if constexpr (J == 4u) {
+    // a rotation of the row of 16 by 4 one way and the other; which of the two is lane ^ 4 depends on bit 2
+    const uint32_t from_below = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xf, 0xf, false);   // row_ror:4: from lane - 4
+    const uint32_t from_above = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x12C, 0xf, 0xf, false);   // row_ror:12: from lane + 4
+    return (lane & 4u) ? from_below : from_above;
+  } else if constexpr (J == 8u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);   // row_ror:8
+  else if constexpr (J == 16u) {
+    const u32x2v t = __builtin_amdgcn_permlane16_swap(v, v, false, false);   // x: rows 0, 0, 2, 2; y: rows 1, 1, 3, 3
+    return (lane & 16u) ? t.x : t.y;
+  } else {
+    const u32x2v t = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // x: lower half twice; y: upper half twice
+    return (lane & 32u) ? t.x : t.y;
+  }
+}
+template <uint32_t J>
+__device__ __forceinline__ float fx_lane_xor_f(float v, uint32_t lane) {
+  return __uint_as_float(fx_lane_xor<J>(__float_as_uint(v), lane));
+}
+
 // NaN-propagating min / max (ATen semantics for maximum/minimum/clamp)
 __device__ __forceinline__ float fx_fmax(float a, float b) { return (a > b || a != a) ? a : b; }
 __device__ __forceinline__ float fx_fmin(float a, float b) { return (a < b || a != a) ? a : b; }
@@ -668,13 +693,15 @@ __device__ __forceinline__ void fx_step(const FxCtx& cx, const FxCoord<R>& q, TS
         for (int j = 0; j < FX_V; ++j) {
           if ((M >> j) & 1u) v = is_max ? fx_fmax(v, u2f(A[j])) : v + u2f(A[j]);
         }
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) {
-          if ((uint32_t)o < cx.wseg) {  // wave-uniform: the butterfly stays inside a segment
-            const float t = __shfl_xor(v, o, 64);
-            v = is_max ? fx_fmax(v, t) : v + t;
-          }
-        }
+        // the butterfly stays inside a segment (wave-uniform); the exchanges stay inside the vector unit
+        const uint32_t ln = threadIdx.x & 63u;
+#define FX_WSTEP(O)                                   \
+  if ((uint32_t)(O) < cx.wseg) {                      \
+    const float t = fx_lane_xor_f<(O)>(v, ln);        \
+    v = is_max ? fx_fmax(v, t) : v + t;               \
+  }
+        FX_WSTEP(32u) FX_WSTEP(16u) FX_WSTEP(8u) FX_WSTEP(4u) FX_WSTEP(2u) FX_WSTEP(1u)
+#undef FX_WSTEP
 #pragma unroll
         for (int j = 0; j < FX_V; ++j) A[j] = f2u(v);
       } break;

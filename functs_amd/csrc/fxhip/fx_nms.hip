@@ -30,6 +30,7 @@
 #include <mutex>
 
 #include "../../../include/fxhip.h"
+#include "fx_device.h"
 
 // a hook for timing the phases of a task's last workgroup from a test program; nothing in the library
 #ifndef FX_NMS_STAMP
@@ -49,31 +50,11 @@ __device__ __forceinline__ float from_orderable(uint32_t o) {
   return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
 }
 
-// the value of lane (own lane ^ J), inside the vector unit
-template <uint32_t J>
-__device__ __forceinline__ uint32_t lane_xor(uint32_t v, uint32_t lane) {
-  typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
-  if constexpr (J == 1u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false);        // quad_perm [1, 0, 3, 2]
-  else if constexpr (J == 2u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
-  else if constexpr (J == 4u) {
-    // a rotation of the row of 16 by 4 one way and the other; which of the two is lane ^ 4 depends on bit 2
-    const uint32_t from_below = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xf, 0xf, false);   // row_ror:4: from lane - 4
-    const uint32_t from_above = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x12C, 0xf, 0xf, false);   // row_ror:12: from lane + 4
-    return (lane & 4u) ? from_below : from_above;
-  } else if constexpr (J == 8u) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false);   // row_ror:8
-  else if constexpr (J == 16u) {
-    const u32x2v t = __builtin_amdgcn_permlane16_swap(v, v, false, false);   // x: rows 0, 0, 2, 2; y: rows 1, 1, 3, 3
-    return (lane & 16u) ? t.x : t.y;
-  } else {
-    const u32x2v t = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // x: lower half twice; y: upper half twice
-    return (lane & 32u) ? t.x : t.y;
-  }
-}
 // one stage of the bitonic network on a key a lane, partners J lanes apart: the lower lane keeps
 // the smaller key where the run ascends
 template <uint32_t J>
 __device__ __forceinline__ uint64_t bitonic_step(uint64_t key, bool up, uint32_t lane) {
-  const uint64_t other = ((uint64_t)lane_xor<J>((uint32_t)(key >> 32), lane) << 32) | (uint64_t)lane_xor<J>((uint32_t)key, lane);
+  const uint64_t other = ((uint64_t)fx_lane_xor<J>((uint32_t)(key >> 32), lane) << 32) | (uint64_t)fx_lane_xor<J>((uint32_t)key, lane);
   const bool keep_min = ((lane & J) == 0u) == up;
   return ((key < other) == keep_min) ? key : other;
 }

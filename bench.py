@@ -560,7 +560,7 @@ def main():
                 "detections_per_image": [min(kept), max(kept)],
                 "nms_bytes_read": read, "nms_gbps": round(read / (e0.elapsed_time(e1) * 1e-3 / n) / 1e9, 1),
                 "bound": "the candidate scan reads the image's class scores once (a workgroup per CU, shared out over the images); "
-                         "sort and the greedy walk run in LDS"}
+                         "sort and the greedy walk are done by the last workgroup of an image (registers and LDS)"}
 
     def run_rows():
         """The stand-alone row compaction of the C ABI (fx_compact_rows: count and scatter; a scan

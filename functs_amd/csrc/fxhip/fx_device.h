@@ -292,6 +292,17 @@ __device__ __forceinline__ float fx_lane_xor_f(float v, uint32_t lane) {
   return __uint_as_float(fx_lane_xor<J>(__float_as_uint(v), lane));
 }
 
+// the sum over the wave, in every lane (integer: the order of the additions does not matter)
+__device__ __forceinline__ uint32_t fx_wave_sum(uint32_t v, uint32_t lane) {
+  v += fx_lane_xor<32u>(v, lane);
+  v += fx_lane_xor<16u>(v, lane);
+  v += fx_lane_xor<8u>(v, lane);
+  v += fx_lane_xor<4u>(v, lane);
+  v += fx_lane_xor<2u>(v, lane);
+  v += fx_lane_xor<1u>(v, lane);
+  return v;
+}
+
 // NaN-propagating min / max (ATen semantics for maximum/minimum/clamp)
 __device__ __forceinline__ float fx_fmax(float a, float b) { return (a > b || a != a) ? a : b; }
 __device__ __forceinline__ float fx_fmin(float a, float b) { return (a < b || a != a) ? a : b; }
@@ -1577,8 +1588,7 @@ __global__ __launch_bounds__(64 * S::kWaves, S::kOcc) void fx_compact_scatter(co
   // exclusive offset of this tile
   uint32_t part = 0;
   for (uint32_t t = threadIdx.x; t < tile; t += NT) part += counts[t];
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+  part = fx_wave_sum(part, threadIdx.x & 63u);
   if (lane == 0) s_wsum[wave] = part;
 
   // row map of this tile
@@ -1796,8 +1806,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_STREAM_OCC) void fx_compact_stream(con
         }
         part += ok ? (wv & ((1u << FX_STATUS_BITS) - 1u)) : 0u;
       }
-#pragma unroll
-      for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+      part = fx_wave_sum(part, threadIdx.x & 63u);
       const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
       if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
     }

@@ -94,8 +94,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_head_stream(const FxHeadLaunch hl
       }
       part += ok ? (wv & ((1u << FX_HEAD_STATUS_BITS) - 1u)) : 0u;
     }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, 64);
+    part = fx_wave_sum(part, lane);
     const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
     if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
     // The image's last chunk tells the host the image's total as soon as it is known: its own

@@ -108,8 +108,7 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rows_scatter(const uint8_t* __res
   uint32_t part = 0;
   if (!SCANNED) {
     for (uint32_t t = threadIdx.x; t < tile; t += FX_BLOCK) part += counts[t];
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) part += __shfl_xor(part, o, 64);
+    part = fx_wave_sum(part, lane);
     if (lane == 0) s_wsum[wave] = part;
   }
   const uint32_t row = tile * FX_BLOCK + threadIdx.x;

@@ -33,6 +33,7 @@
 // hooks for timing the phases of a step in a test build; nothing in the library
 #ifndef FX_LSTM_STAMP
 #define FX_LSTM_STAMP(k)
+#define FX_LSTM_PSTAMP(k)
 #define FX_LSTM_STAMP_END()
 #define FX_LSTM_STAMP_DECL
 #endif
@@ -117,6 +118,7 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
   const int H = a.H, B = a.B, T = a.T;
   const int tid = (int)threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
+  FX_LSTM_PSTAMP(0);
   // Workgroups go to the chip's eight dies in turn, and every die has a cache of its own: the
   // workgroups of a die take neighbouring hidden units, so that a die fetches its eighth of every
   // weight row once (lines of a row are shared by 32 units) instead of every die fetching all of it.
@@ -170,6 +172,7 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
     }
   }
   __syncthreads();
+  FX_LSTM_PSTAMP(1);
 
   const int n_steps = fx_lstm_steps(T, L);
   // x of the next (step, batch row) is asked for at the top of a step, ahead of the polls, and is

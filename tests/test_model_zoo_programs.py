@@ -88,6 +88,29 @@ def fcos_levels(cls_scores: List[Tensor], bbox_preds: List[Tensor], centerness: 
     return out_boxes, out_scores
 
 
+def crop_masks(proto: Tensor, coeffs: Tensor, boxes: Tensor):
+    """Mask assembly in the style of the reference's YOLACT post-processing
+    (functs/benchmark/ai_model/yolact/yolact_mask.py): prototype masks are combined linearly per
+    detection (a library GEMM, outside any region), squashed, and cut to the detection's box with
+    comparisons against pixel coordinates; the elementwise part is one region."""
+    h, w, n = proto.size(0), proto.size(1), coeffs.size(0)
+    masks = (proto @ coeffs.t()).sigmoid()                        # [h, w, n]
+    rows = torch.arange(h, device=proto.device, dtype=proto.dtype).view(-1, 1, 1).expand(h, w, n)
+    cols = torch.arange(w, device=proto.device, dtype=proto.dtype).view(1, -1, 1).expand(h, w, n)
+    x1, y1, x2, y2 = boxes[:, 0], boxes[:, 1], boxes[:, 2], boxes[:, 3]
+    inside = (cols >= x1.view(1, 1, -1)) & (cols < x2.view(1, 1, -1)) & (rows >= y1.view(1, 1, -1)) & (rows < y2.view(1, 1, -1))
+    return masks * inside.to(masks.dtype)
+
+
+def _crop_inputs(seed=0, h=34, w=38, k=8, n=5):
+    g = torch.Generator().manual_seed(seed)
+    proto = torch.randn(h, w, k, generator=g)
+    coeffs = torch.randn(n, k, generator=g)
+    xy = torch.rand(n, 2, generator=g) * 20
+    boxes = torch.cat([xy, xy + torch.rand(n, 2, generator=g) * 15 + 2], 1)
+    return [proto, coeffs, boxes]
+
+
 def _fcos_inputs(seed=0, classes=20, sizes=((20, 24), (10, 12), (5, 6))):
     g = torch.Generator().manual_seed(seed)
     cls, box, ctr, pts, strides = [], [], [], [], []
@@ -204,3 +227,14 @@ def test_anchor_free_head_equals_eager():
         torch.testing.assert_close(a.cpu(), b, rtol=1e-5, atol=1e-5)
     for a, b in zip(scores, ref_scores):
         torch.testing.assert_close(a.cpu(), b, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_mask_assembly_equals_eager():
+    args = _crop_inputs()
+    built = fj.build(fj.script(crop_masks), args)
+    got = built(*_cuda(args))
+    ref = crop_masks(*args)
+    assert got.shape == ref.shape and (ref != 0).sum().item() > 100 and (ref == 0).sum().item() > 100
+    torch.testing.assert_close(got.cpu(), ref, rtol=1e-5, atol=1e-6)
+    assert "tssa::ParallelFunctor" in _kinds(built.graph)          # the elementwise part runs as a region

@@ -4,7 +4,9 @@ that ends on a value computed on the device and writes one row of an int64 resul
 functs/benchmark/ai_model/seq2seq/seq2seq.py:95-142), written here as functions with the weights
 as arguments.  Their loops carry state, so they stay host loops around one fused region per step
 (the matrix products are ATen's); the tests check the graphs and, on the GPU, the results against
-eager mode (1e-4 relative after the recurrence, the decoder's tokens exactly)."""
+eager mode (1e-4 relative after the recurrence, the decoder's tokens exactly).  Two detection
+post-processing programs follow: an anchor-free head over pyramid levels of different sizes (one
+compacting map over ragged tasks) and mask assembly behind a library GEMM (one dense region)."""
 from typing import List
 
 import pytest

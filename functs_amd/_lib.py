@@ -149,6 +149,12 @@ _sig("fx_plan_blob", _i, _vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32)), c
 _sig("fx_plan_disasm", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)
 _sig("fx_plan_head_info", _i, _vp, ctypes.POINTER(ctypes.c_int64), _i)
 _sig("fx_set_head_kernel", None, _i)
+_sig("fx_plan_rowstream_info", _i, _vp, ctypes.POINTER(ctypes.c_int64), _i)
+_sig("fx_plan_rowstream_why", _i, _vp, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_plan_rowstream_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)
+_sig("fx_set_rowstream", None, _i)
+_sig("fx_plan_rowstream_launch", _i, _vp, ctypes.c_uint32, ctypes.c_uint32, _vp, ctypes.c_size_t)
+_sig("fx_rowstream_count", _i)
 _sig("fx_plan_spec_key", ctypes.c_uint64, _vp)
 _sig("fx_plan_specialized", _i, _vp)
 _sig("fx_plan_spec_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)

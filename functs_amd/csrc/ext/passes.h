@@ -78,6 +78,14 @@ void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
 bool SinkProducersIntoMaps(std::shared_ptr<torch::jit::Graph> graph);
 void setSinkProducers(bool on);
 
+// Plans the region of every tssa::ParallelFunctor of a built graph for the static types in its
+// input_refine_types (meta tensors stand for them; nothing runs, no device is needed), as the
+// reference compiles every functor when its operator is created (fait/fuser/graph_builder.cpp:
+// 259-712).  With a dump directory set in the library (fx_spec_dump_dir) the regions without
+// compiled kernels leave their sources there.  Returns one line per functor: what was planned and
+// which kernels serve it.
+std::vector<std::string> PlanFunctors(std::shared_ptr<torch::jit::Graph> graph);
+
 // Host time of tssa::ParallelFunctor by section (flatten, plan, alloc, launch, views, wait_counts,
 // resize, push): switching on clears the sums; the read gives "calls" and the mean microseconds per
 // operator call of every section.

@@ -579,7 +579,8 @@ class RegionRunner {
   // What the library makes of the region for arguments of these types (meta tensors stand for
   // them; nothing runs): `kind` is the first word of fx_plan_head_info when that kernel is in
   // use (0: the generic kernels), `shapes` the shapes of task 0's results.
-  void dryRun(const std::vector<c10::IValue>& samples, int64_t* kind, std::vector<std::vector<int64_t>>* shapes) {
+  void dryRun(const std::vector<c10::IValue>& samples, int64_t* kind, std::vector<std::vector<int64_t>>* shapes,
+              int64_t* rowstream = nullptr, std::string* rowstream_why = nullptr) {
     TORCH_CHECK(samples.size() == n_stack_, "dryRun: argument count");
     int64_t degree = degree_;
     size_t first = 0;
@@ -601,6 +602,15 @@ class RegionRunner {
     int64_t info[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     FX_OK_OR_THROW(fx_plan_head_info(plan, info, 8));
     *kind = info[1] ? info[0] : 0;
+    if (rowstream) {
+      FX_OK_OR_THROW(fx_plan_rowstream_info(plan, rowstream, 8));
+      if (rowstream_why) {
+        char buf[256];
+        buf[0] = 0;
+        fx_plan_rowstream_why(plan, buf, sizeof buf);
+        *rowstream_why = buf;
+      }
+    }
     shapes->clear();
     for (int o = 0; o < fx_plan_num_outputs(plan); ++o) {
       int32_t dt = 0, rank = 0;
@@ -1310,6 +1320,77 @@ bool SinkProducersIntoMaps(std::shared_ptr<Graph> graph) {
   return changed;
 }
 void setSinkProducers(bool on) { g_sink_producers.store(on); }
+
+// ---------------------------------------------------------------------------
+// every functor of a built graph planned for its static argument types
+// ---------------------------------------------------------------------------
+namespace {
+void planIn(Block* b, std::vector<std::string>* report) {
+  for (Node* n : b->nodes()) {
+    for (Block* inner : n->blocks()) planIn(inner, report);
+    if (n->kind() != sym::ParallelFunctor()) continue;
+    std::ostringstream line;
+    const auto sub = n->g(c10::attr::Subgraph);
+    bool special = false;
+    for (Node* k : sub->nodes())
+      if (k->kind() == sym::LstmStack()) special = true;
+    if (special) { report->push_back("lstm_stack functor: a kernel of its own, nothing to plan"); continue; }
+    const auto types = n->tys(sym::input_refine_types());
+    const auto par = n->is(sym::is_parallel_args());
+    const int64_t degree = n->i(sym::parallel_degree());
+    const bool is_map = n->i(sym::is_parallel_map()) != 0;
+    if (degree < 0) { report->push_back("functor with a run-time trip count: planned when it runs"); continue; }
+    std::vector<c10::IValue> samples;
+    bool ok = types.size() == n->inputs().size() && par.size() == types.size();
+    for (size_t k = 0; ok && k < types.size(); ++k) {
+      c10::IValue v;
+      if (is_map && par[k] != 0) {
+        // the unified element type of a per-task list
+        auto et = types[k];
+        if (auto lt = et->cast<c10::ListType>()) et = lt->getElementType();
+        if (!sampleOf(et, &v)) { ok = false; break; }
+        c10::List<at::Tensor> lst;
+        for (int64_t t = 0; t < degree; ++t) lst.push_back(v.toTensor());
+        samples.emplace_back(lst);
+      } else if (sampleOf(types[k], &v)) {
+        samples.push_back(v);
+      } else if (auto c = toIValue(n->input(k))) {
+        samples.push_back(*c);
+      } else {
+        ok = false;
+      }
+    }
+    if (!ok) { report->push_back("functor with arguments without a static type: planned when it runs"); continue; }
+    try {
+      int64_t kind = 0, rs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      std::vector<std::vector<int64_t>> shapes;
+      std::string why;
+      RegionRunner r(n);
+      r.dryRun(samples, &kind, &shapes, rs, &why);
+      line << "functor planned: " << shapes.size() << " output(s)";
+      if (n->hasAttribute(sym::compact_rows()) && n->i(sym::compact_rows()) != 0) {
+        if (rs[0]) {
+          char hx[32];
+          snprintf(hx, sizeof hx, "%08llx%08llx", (unsigned long long)rs[3], (unsigned long long)rs[2]);
+          line << ", row-stream key " << hx << (rs[1] ? " (kernel linked)" : " (no kernel linked)");
+        } else {
+          line << ", no row-stream form: " << why;
+        }
+        if (kind) line << ", hand-written kernel " << kind;
+      }
+    } catch (const c10::Error& e) {
+      line << "functor not planned: " << e.what_without_backtrace();
+    }
+    report->push_back(line.str());
+  }
+}
+}  // namespace
+
+std::vector<std::string> PlanFunctors(std::shared_ptr<Graph> graph) {
+  std::vector<std::string> report;
+  planIn(graph->block(), &report);
+  return report;
+}
 
 void functorHostTiming(bool on) {
   if (on) {

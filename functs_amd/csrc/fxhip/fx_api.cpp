@@ -17,6 +17,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "fx_lower.h"
@@ -258,6 +259,11 @@ static std::atomic<int> g_head_mode{[] {
   const char* e = getenv("FXHIP_HEAD");
   return (e && e[0] == '0') ? 0 : 1;
 }()};
+// ---- generated row-stream kernels (fx_rs.h): on unless FXHIP_ROWSTREAM=0 ----
+static std::atomic<int> g_rs_mode{[] {
+  const char* e = getenv("FXHIP_ROWSTREAM");
+  return (e && e[0] == '0') ? 0 : 1;
+}()};
 static std::atomic<uint32_t> g_stream_spin{[] {
   const char* e = getenv("FXHIP_STREAM_SPIN");
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
@@ -280,6 +286,27 @@ static void dump_spec_source(const fx::Plan* p) {
   {
     std::lock_guard<std::mutex> g(g_dump_mu);
     dir = g_dump_dir;
+  }
+  if (!dir.empty() && p->rs.ok && !fx_rs_find(p->rs.key)) {
+    char rname[64];
+    snprintf(rname, sizeof(rname), "/fx_rs_%016llx.hip", (unsigned long long)p->rs.key);
+    const std::string rpath = dir + rname;
+    if (FILE* f = fopen(rpath.c_str(), "r")) {
+      fclose(f);
+    } else {
+      std::string label = "row compaction, outputs of task 0:";
+      for (size_t o = 0; o < p->out_shape.size(); ++o) {
+        label += " [";
+        const auto& sh = p->out_shape[o][0];
+        for (size_t d = 0; d < sh.size(); ++d) label += (d ? "," : "") + std::to_string(sh[d]);
+        label += "]";
+      }
+      const std::string src = fx::rs_source(*p, label);
+      if (FILE* f = fopen(rpath.c_str(), "w")) {
+        fwrite(src.data(), 1, src.size(), f);
+        fclose(f);
+      }
+    }
   }
   if (dir.empty() || p->spec_key == 0 || fx_spec_find(p->spec_key)) return;
   char name[64];
@@ -360,6 +387,8 @@ int fx_plan_output(const fx_plan* p, int out_idx, int task, int32_t* dtype, int3
 size_t fx_plan_scratch_bytes(const fx_plan* p) { return p ? P(p)->scratch_bytes : 0; }
 static bool stream_active(const fx::Plan* pl, const FxSpecKernels* spec);
 static const FxSpecKernels* spec_of(const fx::Plan* p);
+static const FxRsKernel* rs_of(const fx::Plan* pl);
+static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl);
 static bool head_active(const fx::Plan* pl) {
   // (with compiled kernels switched off, fx_set_specialization(0), everything runs in the interpreter)
   return pl->mode == FX_MODE_COMPACT && pl->head.ok && g_head_mode.load(std::memory_order_relaxed) != 0 &&
@@ -386,7 +415,7 @@ int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
     return FX_OK;
   }
   out[0] = hi.ok ? 1 : 0;
-  out[1] = head_active(P(p)) ? 1 : 0;
+  out[1] = (head_active(P(p)) && !rs_of(P(p))) ? 1 : 0;
   out[2] = (int64_t)(hi.norm_hash & 0xffffffffull);
   out[3] = (int64_t)(hi.norm_hash >> 32);
   out[4] = hi.C;
@@ -395,14 +424,60 @@ int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
   out[7] = hi.n_tasks;
   return FX_OK;
 }
+void fx_set_rowstream(int on) { g_rs_mode.store(on ? 1 : 0, std::memory_order_relaxed); }
+int fx_rowstream_count(void) { return fx_rs_count(); }
+int fx_plan_rowstream_info(const fx_plan* p, int64_t* out, int cap) {
+  if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_rowstream_info: out[>=8] required");
+  const FxRsInfo& ri = P(p)->rs;
+  out[0] = ri.ok ? 1 : 0;
+  out[1] = rs_of(P(p)) ? 1 : 0;
+  out[2] = (int64_t)(ri.key & 0xffffffffull);
+  out[3] = (int64_t)(ri.key >> 32);
+  out[4] = ri.S;
+  out[5] = ri.n_rows;
+  out[6] = ri.n_tasks;
+  out[7] = ri.n_in;
+  return FX_OK;
+}
+int fx_plan_rowstream_why(const fx_plan* p, char* buf, size_t cap) {
+  if (!p || !buf || cap == 0) return fail(FX_E_INVALID, "null argument");
+  const std::string& s = P(p)->rs.why;
+  const size_t n = std::min(cap - 1, s.size());
+  memcpy(buf, s.data(), n);
+  buf[n] = 0;
+  return (int)s.size();
+}
+int fx_plan_rowstream_launch(const fx_plan* p, uint32_t chunk_rows, uint32_t sub_rows, void* out, size_t cap) {
+  if (!p || !out || cap < sizeof(FxRsLaunch)) return fail(FX_E_INVALID, "fx_plan_rowstream_launch: out too small");
+  if (!P(p)->rs.ok) return fail(FX_E_UNSUPPORTED, "this plan has no row-stream form: " + P(p)->rs.why);
+  FxRsLaunch rl;
+  rs_fill_params(P(p), &rl);
+  if (chunk_rows == 0 || chunk_rows > FX_BLOCK || sub_rows == 0 || sub_rows > rl.sub_rows)
+    return fail(FX_E_INVALID, "fx_plan_rowstream_launch: chunk rows 1.." + std::to_string(FX_BLOCK) + ", sub-tile rows 1.." + std::to_string(rl.sub_rows));
+  rl.chunk_rows = chunk_rows;
+  rl.chunks = (rl.n_rows + chunk_rows - 1) / chunk_rows;
+  rl.sub_rows = sub_rows;
+  memcpy(out, &rl, sizeof(rl));
+  return (int)sizeof(rl);
+}
+int fx_plan_rowstream_source(const fx_plan* p, const char* label, char* buf, size_t cap) {
+  if (!p || !buf || cap == 0) return fail(FX_E_INVALID, "null argument");
+  FX_TRY
+  std::string s = fx::rs_source(*P(p), label ? label : "");
+  size_t n = std::min(cap - 1, s.size());
+  memcpy(buf, s.data(), n);
+  buf[n] = 0;
+  return (int)s.size();
+  FX_CATCH
+}
 int fx_plan_launches(const fx_plan* p) {
   if (!p) return 0;
-  if (head_active(P(p)) || cmap_active(P(p))) return 1;
+  if (rs_of(P(p)) || head_active(P(p)) || cmap_active(P(p))) return 1;
   if (P(p)->mode == FX_MODE_COMPACT && stream_active(P(p), spec_of(P(p)))) return P(p)->stream.grid > 0 ? 1 : 0;
   return P(p)->launches;
 }
 int fx_plan_streaming(const fx_plan* p) {
-  return (p && P(p)->mode == FX_MODE_COMPACT && !head_active(P(p)) && !cmap_active(P(p)) && stream_active(P(p), spec_of(P(p)))) ? 1 : 0;
+  return (p && P(p)->mode == FX_MODE_COMPACT && !rs_of(P(p)) && !head_active(P(p)) && !cmap_active(P(p)) && stream_active(P(p), spec_of(P(p)))) ? 1 : 0;
 }
 int fx_plan_stream_info(const fx_plan* p, int64_t* out, int cap) {
   if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_stream_info: out[>=8] required");
@@ -688,6 +763,83 @@ static int head_launch_info(fx::Plan* pl, FxHeadLaunch* hl) {
   return FX_OK;
 }
 
+// ---- generated row-stream kernels (fx_rs.h): when, and the geometry of a launch ----
+static const FxRsKernel* rs_of(const fx::Plan* pl) {
+  if (pl->mode != FX_MODE_COMPACT || !pl->rs.ok || !g_rs_mode.load(std::memory_order_relaxed) ||
+      !g_specialize.load(std::memory_order_relaxed))
+    return nullptr;
+  const FxRsKernel* k = fx_rs_find(pl->rs.key);
+  return (k && k->S == pl->rs.S) ? k : nullptr;
+}
+// Rows of a sub-tile: what FX_RS_KV 128-bit loads per lane carry, at most FX_RS_SUB.
+static uint32_t rs_sub_rows(const FxRsInfo& ri) {
+  const uint32_t cap = (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S;
+  return std::min<uint32_t>(FX_RS_SUB, cap);
+}
+static uint32_t rs_lds_bytes(const FxRsInfo& ri) { return (((rs_sub_rows(ri) * ri.S + 3u + 3u) >> 2) + 1u) * 16u; }
+static size_t rs_status_words(const FxRsInfo& ri) {
+  const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
+  return (size_t)ri.n_tasks * ((ri.n_rows + min_chunk - 1) / min_chunk);
+}
+// Every task's rows are dealt to its workgroups in equal runs, as few workgroups as give every
+// resident slot of the device one (more only when a chunk would exceed FX_BLOCK rows, fewer when
+// it would fall below FX_RS_MIN_CHUNK).
+static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl) {
+  const FxRsInfo& ri = pl->rs;
+  memset(rl, 0, sizeof(*rl));
+  rl->n_rows = ri.n_rows;
+  rl->n_tasks = ri.n_tasks;
+  rl->sub_rows = rs_sub_rows(ri);
+  rl->spin_limit = g_stream_spin.load(std::memory_order_relaxed);
+  rl->n_sptr = (uint32_t)pl->sptr.size();
+  rl->n_tptr = (uint32_t)pl->tptr.size();
+  rl->n_sscal = (uint32_t)pl->sscal.size();
+  rl->n_tscal = (uint32_t)pl->tscal.size();
+  for (uint32_t k = 0; k < FX_RS_MAX_IN; ++k) {
+    rl->in_slot[k] = ri.in_slot[k];
+    rl->in_tcoef[k] = ri.in_tcoef[k];
+  }
+  for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) {
+    rl->out_slot[k] = ri.out_slot[k];
+    rl->out_tstride[k] = ri.out_tstride[k];
+  }
+  for (uint32_t k = 0; k < FX_RS_MAX_FIMM; ++k) rl->fimm[k] = ri.fimm[k];
+  rl->slot_err = ri.slot_err;
+}
+static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) {
+  const FxRsInfo& ri = pl->rs;
+  rs_fill_params(pl, rl);
+  if (pl->rs_resident == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    HIP_OK(hipGetDevice(&dev));
+    HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri)));
+    uint32_t wg = (uint32_t)std::max(per_cu, 1) * (uint32_t)std::max(cus, 1);
+    // One slot per CU is left free: a launch that needs every slot the occupancy rule allows does
+    // not get all of its workgroups placed at once, and the stragglers cost a second round.
+    if (per_cu >= 3) wg -= wg / (uint32_t)per_cu;
+    pl->rs_resident = std::max<uint32_t>(wg, 1u);
+    pl->rs_per_cu = (uint32_t)std::max(per_cu, 1);
+  }
+  const uint32_t per_task = std::max<uint32_t>(1u, pl->rs_resident / std::max<uint32_t>(ri.n_tasks, 1u));
+  uint32_t cr = (ri.n_rows + per_task - 1) / per_task;
+  const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
+  cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
+  rl->chunk_rows = cr;
+  rl->chunks = (ri.n_rows + cr - 1) / cr;
+  // A launch whose first sub-tiles alone are megabytes of requests floods the memory system: there
+  // the counts get a head start.  A small launch would only lose the time.
+  const uint64_t first_bytes = (uint64_t)rl->chunks * ri.n_tasks * std::min<uint32_t>(cr, rl->sub_rows) * ri.S * 4u;
+  rl->bulk_delay = first_bytes >= FX_RS_FLOOD_BYTES ? FX_RS_BULK_DELAY : 0u;
+  return FX_OK;
+}
+static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const FxRsLaunch& rl, const FxDyn* dyn, hipStream_t stream) {
+  const uint32_t grid = rl.chunks * rl.n_tasks;
+  if (grid == 0) return hipSuccess;
+  void* args[2] = {(void*)&rl, (void*)dyn};
+  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri), stream);
+}
+
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----
 #define FX_CMAP_EPOCH_MAX 0xffffu   // the epoch tag of its 64-bit status words has 16 bits
 static size_t cmap_status_words(const FxCmapInfo& ci) {
@@ -774,10 +926,22 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     cap_status = hipStreamCaptureStatusNone;
   }
   const bool capturing = cap_status != hipStreamCaptureStatusNone;
-  bool head = !capturing && head_fits(pl);
-  FxHeadLaunch hl;
   void* status = nullptr;
   uint32_t epoch = 0;
+  const FxRsKernel* rsk = capturing ? nullptr : rs_of(pl);
+  FxRsLaunch rl;
+  if (rsk) {
+    rc = rs_launch_info(pl, rsk, &rl);
+    if (rc != FX_OK) return rc;
+    void* rstatus = nullptr;
+    rc = status_words(reg, pl->head_status, rs_status_words(pl->rs), stream, dev, &rstatus, &epoch, repeat);
+    if (rc != FX_OK) return rc;
+    if (!rstatus) rsk = nullptr;
+    rl.status = (uint32_t*)rstatus;
+    rl.totals = totals_host;
+  }
+  bool head = !rsk && !capturing && head_fits(pl);
+  FxHeadLaunch hl;
   if (head) {
     rc = head_launch_info(pl, &hl);
     if (rc != FX_OK) return rc;
@@ -788,7 +952,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     hl.status = (uint32_t*)hstatus;
     hl.totals = totals_host;
   }
-  bool cmap = !head && !capturing && cmap_active(pl), cmap_wide = false;
+  bool cmap = !rsk && !head && !capturing && cmap_active(pl), cmap_wide = false;
   FxCmapLaunch cl;
   if (cmap) {
     rc = cmap_launch_info(pl, &cl, &cmap, &cmap_wide);
@@ -802,7 +966,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     cl.status = (uint32_t*)cstatus;
     cl.totals = totals_host;
   }
-  bool streaming = !head && !cmap && !capturing && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
+  bool streaming = !rsk && !head && !cmap && !capturing && pl->mode == FX_MODE_COMPACT && stream_active(pl, spec);
   if (streaming) {
     rc = stream_status(reg, pl, stream, dev, &status, &epoch, repeat);
     if (rc != FX_OK) return rc;
@@ -821,9 +985,9 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
                            ? FX_TOTAL_PENDING
                            : 0u;
   }
-  const int launches = head ? (hl.chunks * hl.n_tasks > 0 ? 1 : 0) : cmap ? (cl.chunks > 0 ? 1 : 0) : streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
+  const int launches = rsk ? (rl.chunks * rl.n_tasks > 0 ? 1 : 0) : head ? (hl.chunks * hl.n_tasks > 0 ? 1 : 0) : cmap ? (cl.chunks > 0 ? 1 : 0) : streaming ? (pl->stream.grid > 0 ? 1 : 0) : pl->launches;
   g_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
-  if (spec || head || cmap) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
+  if (spec || rsk || head || cmap) g_spec_launches.fetch_add((uint64_t)launches, std::memory_order_relaxed);
   // optional per-kernel timing with events on the launch stream
   hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
   const bool timed = kernel_ms != nullptr;
@@ -838,6 +1002,14 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
       HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
+  } else if (rsk) {
+    HIP_OK(mark(0));
+    for (int r = 0; r < repeat; ++r) {
+      rl.epoch = epoch + (uint32_t)r;
+      HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn, stream));
+    }
+    HIP_OK(mark(1));
+    nk = rl.chunks * rl.n_tasks > 0 ? 1 : 0;
   } else if (head) {
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
@@ -913,7 +1085,18 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   uint32_t epoch = 0;
   int dev = 0;
   HIP_OK(hipGetDevice(&dev));
-  bool head = compact && head_fits(pl);
+  const FxRsKernel* rsk = compact ? rs_of(pl) : nullptr;
+  FxRsLaunch rl;
+  if (rsk) {
+    int rc = rs_launch_info(pl, rsk, &rl);
+    if (rc != FX_OK) return rc;
+    void* rstatus = nullptr;
+    rc = status_words(reg, pl->head_status, rs_status_words(pl->rs), stream, dev, &rstatus, &epoch, rounds * n_sets);
+    if (rc != FX_OK) return rc;
+    if (!rstatus) rsk = nullptr;
+    rl.status = (uint32_t*)rstatus;
+  }
+  bool head = !rsk && compact && head_fits(pl);
   FxHeadLaunch hl;
   if (head) {
     int rc = head_launch_info(pl, &hl);
@@ -924,7 +1107,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     if (!hstatus) head = false;
     hl.status = (uint32_t*)hstatus;
   }
-  bool cmap = !head && compact && cmap_active(pl), cmap_wide = false;
+  bool cmap = !rsk && !head && compact && cmap_active(pl), cmap_wide = false;
   FxCmapLaunch cl;
   if (cmap) {
     int rc = cmap_launch_info(pl, &cl, &cmap, &cmap_wide);
@@ -940,13 +1123,13 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     if (!cstatus) cmap = false;
     cl.status = (uint32_t*)cstatus;
   }
-  bool streaming = !head && !cmap && compact && stream_active(pl, spec);
+  bool streaming = !rsk && !head && !cmap && compact && stream_active(pl, spec);
   if (streaming) {
     const int rc = stream_status(reg, pl, stream, dev, &status, &epoch, rounds * n_sets);
     if (rc != FX_OK) return rc;
     if (!status) streaming = false;
   }
-  if (which >= ((streaming || head || cmap) ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
+  if (which >= ((streaming || rsk || head || cmap) ? 1 : pl->launches)) return fail(FX_E_INVALID, "fx_region_run_timed_sets: the call has no such kernel");
   std::vector<FxDyn> dyn((size_t)n_sets);
   for (int i = 0; i < n_sets; ++i) {
     memset(&dyn[i], 0, sizeof(FxDyn));
@@ -964,6 +1147,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
     for (int i = 0; i < n_sets; ++i) {
       if (!compact) {
         HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+      } else if (rsk) {
+        rl.epoch = epoch + (uint32_t)(r * n_sets + i);
+        rl.totals = totals_host[i];
+        HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn[i], stream));
       } else if (head) {
         hl.epoch = epoch + (uint32_t)(r * n_sets + i);
         hl.totals = totals_host[i];

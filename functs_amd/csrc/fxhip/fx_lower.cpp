@@ -2298,6 +2298,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   P->spec_key = spec_hash(*P);
   match_head(P.get());
   match_classmap(P.get());
+  rs_analyze(P.get());
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;
@@ -2306,7 +2307,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
 // ---------------------------------------------------------------------------
 // disassembler (debugging aid, the analogue of CodeGen::getCodeText)
 // ---------------------------------------------------------------------------
-static const char* opname(uint32_t op) {
+const char* opname(uint32_t op) {
   static const char* names[] = {
       "NOP", "LDA", "LDB", "LDXA", "AFFA", "AFFB", "IMMA", "IMMB", "SCLA", "SCLB", "STT", "LDTA", "LDTB", "MOVBA",
       "SWAP", "MIF", "MELSE", "MMERGE", "MEND", "MIFR", "FNEG", "FABS", "EXP", "LOG", "SQRT", "RSQRT", "RCP", "SIGMOID",

@@ -20,6 +20,7 @@
 #include "fx_bytecode.h"
 #include "fx_cmap.h"
 #include "fx_head.h"
+#include "fx_rs.h"
 
 namespace fx {
 
@@ -108,6 +109,7 @@ struct Plan {
   StreamInfo stream;
   FxHeadInfo head;               // the plan is the decode + score filter of a detection head (fx_head.h)
   FxCmapInfo cmap;               // the plan is the decode + per-class score filter of an SSD-style head (fx_cmap.h)
+  FxRsInfo rs;                   // the plan has a row-stream form (fx_rs.h): key of the generated kernel that serves it
   bool uses_guard = false;       // some load checks int64 data against 32 bits and reports to the error word
   uint32_t n_temps = 0;
   int max_rank = 1;
@@ -132,6 +134,7 @@ struct Plan {
   std::vector<Status> head_status;
   uint32_t head_resident = 0;
   uint32_t cmap_resident_wide = 0;   // class-map head kernel: workgroups of its wide form
+  uint32_t rs_resident = 0, rs_per_cu = 0;   // row-stream kernel: workgroups the device holds at once
 };
 
 // Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?
@@ -148,6 +151,11 @@ int kernel_rank(int rank);
 // cannot be specialised.  spec_source writes the translation unit that specialises it.
 uint64_t spec_hash(const Plan& p);
 std::string spec_source(const Plan& p, const std::string& label);
+// Row-stream form of a compacting plan (fx_rs.h, fx_rs_gen.cpp): rs_analyze fills p->rs,
+// rs_source writes the translation unit of the kernel that serves every plan with that key.
+void rs_analyze(Plan* p);
+std::string rs_source(const Plan& p, const std::string& label);
+const char* opname(uint32_t op);
 
 int dtype_size(int dt);
 

@@ -1,0 +1,85 @@
+// Row-stream kernels: a row compaction whose widest input is a row-major matrix read row by
+// row, run as ONE launch of a kernel that is GENERATED from the region's own lowered programs.
+//
+// The generator (fx_rs_gen.cpp) executes the bytecode of the mask and of every output
+// symbolically, once per output column with the column index a constant, into ONE expression
+// graph per row: predicates of select_rev / slice_rev / cat / stack chains that depend on the
+// column fold away, loads and sub-expressions that several columns share exist once (the
+// decoded centre and half size of a box serve its four corners), loads of neighbouring elements
+// become one wide load.  Long runs of columns that execute the same instructions (the class
+// scores of a detection head) become a vector form, four columns per lane.  The result is a
+// HIP translation unit (spec/fx_rs_<key>.hip) holding a policy class for the skeleton of
+// fx_rowstream.h; built into the library, it serves every plan whose programs produce the same
+// key: any number of rows and tasks, any pointers, any per-task offsets, and any VALUES of the
+// floating-point constants (thresholds, scale factors) as long as equal constants stay equal.
+//
+// This is the counterpart of the reference's per-subgraph code generator
+// (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121); the compiler runs when the library is
+// built instead of when the operator is created (CompileToNVRTC, :1319-1414).
+#pragma once
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "fx_bytecode.h"
+
+#define FX_RS_VERSION 1u
+#define FX_RS_MAX_IN 8u         // input buffers of a region
+#define FX_RS_MAX_OUT 8u        // outputs
+#define FX_RS_MAX_FIMM 24u      // distinct floating-point constants
+#define FX_RS_SUB 64u           // most rows of a sub-tile (one ballot)
+#define FX_RS_NSUB 4u           // most sub-tiles of a chunk: a chunk holds at most FX_BLOCK rows
+#define FX_RS_KV 6u             // 128-bit loads per lane that carry a sub-tile
+#define FX_RS_STATUS_BITS 9u    // a chunk's count is at most FX_BLOCK
+#define FX_RS_MIN_CHUNK 64u     // fewest rows of a chunk unless a task has fewer
+#define FX_RS_FLOOD_BYTES (8u << 20)   // first sub-tiles of a launch from which on the counts are sent ahead of the rows
+#define FX_RS_BULK_DELAY 128u          // by this many units of 64 clocks
+#define FX_RS_VEC_MIN 8u        // shortest run of alike columns that takes the vector form
+#define FX_RS_MAX_UNROLL 64u    // most columns evaluated one by one per row
+
+// What the analysis of a plan found (host).
+struct FxRsInfo {
+  bool ok = false;
+  std::string why;              // when not ok: what rules the region out
+  uint64_t key = 0;             // of the generated kernel that serves this plan
+  uint32_t S = 0;               // elements per row of the window input
+  uint32_t n_rows = 0, n_tasks = 0;
+  uint32_t n_in = 0;
+  uint32_t in_slot[FX_RS_MAX_IN] = {};     // pointer slot of each input (FX_SLOT_TASK: per-task table); 0 is the window
+  int32_t in_tcoef[FX_RS_MAX_IN] = {};     // element offset per task
+  uint32_t n_out = 0;
+  uint32_t out_slot[FX_RS_MAX_OUT] = {};
+  uint32_t out_tstride[FX_RS_MAX_OUT] = {};
+  uint32_t n_fimm = 0;
+  uint32_t fimm[FX_RS_MAX_FIMM] = {};      // values (float bits) of this plan's floating-point constants
+  uint32_t slot_err = 0;        // 1 + shared pointer slot of the error word of guarded int64 loads (0: none)
+};
+
+// Kernel arguments (by value, followed by the FxDyn block in the argument segment).
+struct FxRsLaunch {
+  uint32_t n_rows, n_tasks;
+  uint32_t chunks, chunk_rows;  // workgroups per task and rows of each (<= FX_BLOCK)
+  uint32_t sub_rows;            // rows of a sub-tile (<= FX_RS_SUB; the window holds them)
+  uint32_t epoch, spin_limit;
+  uint32_t n_sptr, n_tptr, n_sscal, n_tscal;
+  uint32_t bulk_delay;          // big launches: waves without a gather wait this long (units of 64 clocks) before they ask for rows
+  uint32_t in_slot[FX_RS_MAX_IN];
+  int32_t in_tcoef[FX_RS_MAX_IN];
+  uint32_t out_slot[FX_RS_MAX_OUT], out_tstride[FX_RS_MAX_OUT];
+  uint32_t fimm[FX_RS_MAX_FIMM];
+  uint32_t slot_err, pad0;
+  uint32_t* status;             // one word per chunk, tagged with the epoch
+  uint32_t* totals;             // pinned host memory: kept rows per task
+};
+static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte boundary");
+
+// ---- host side: generated kernels linked into the library ----
+struct FxRsKernel {
+  const void* fn = nullptr;     // fx_rs_kernel<P>
+  uint32_t S = 0;               // row length the kernel is generated for
+  uint32_t static_lds = 0;      // bytes of its static LDS tables
+};
+void fx_rs_register(uint64_t key, const FxRsKernel& k);
+const FxRsKernel* fx_rs_find(uint64_t key);
+int fx_rs_count();

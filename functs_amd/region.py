@@ -274,6 +274,27 @@ class Region:
         check(lib.fx_plan_spec_source(p.handle, label.encode(), buf, len(buf)))
         return buf.value.decode()
 
+    def rowstream_info(self, *args):
+        """Row-stream form of a compacting region for these arguments (fx_plan_rowstream_info):
+        a dict with `ok` (the form exists), `active` (a generated kernel for it is linked and
+        enabled), `key`, `row_elements`, `rows`, `tasks`, `inputs` and, when not ok, `why`."""
+        arr, n, _ = self._flatten(args)
+        p = self.plan(arr, n)
+        out = (ctypes.c_int64 * 8)()
+        check(lib.fx_plan_rowstream_info(p.handle, out, 8))
+        why = ctypes.create_string_buffer(512)
+        check(lib.fx_plan_rowstream_why(p.handle, why, len(why)))
+        return {"ok": bool(out[0]), "active": bool(out[1]), "key": (int(out[3]) << 32) | int(out[2]), "row_elements": int(out[4]),
+                "rows": int(out[5]), "tasks": int(out[6]), "inputs": int(out[7]), "why": why.value.decode()}
+
+    def rowstream_source(self, *args, label=""):
+        """HIP translation unit of the generated row-stream kernel for these arguments."""
+        arr, n, _ = self._flatten(args)
+        p = self.plan(arr, n)
+        buf = ctypes.create_string_buffer(1 << 22)
+        check(lib.fx_plan_rowstream_source(p.handle, label.encode(), buf, len(buf)))
+        return buf.value.decode()
+
     def spec_key(self, *args):
         arr, n, _ = self._flatten(args)
         return int(lib.fx_plan_spec_key(self.plan(arr, n).handle))

@@ -220,6 +220,41 @@ void fx_set_stream_spin_limit(uint32_t polls);
  * x[mask] to ATen (convert_to_tensorssa.cpp:422-443). */
 void fx_set_head_kernel(int on);
 int fx_plan_head_info(const fx_plan*, int64_t* out, int cap);
+
+/* ---- generated row-stream kernels ----
+ * A compacting region whose widest input is a row-major matrix of 32-bit elements that every
+ * program reads row by row (the predictions of a detection head; any mask, any outputs built
+ * from elementwise operators and the access / assign family, no reductions) has a ROW-STREAM
+ * form: one launch in which every workgroup streams a run of consecutive rows through LDS,
+ * publishes its kept-row count at once and takes its write offset from the counts of the
+ * earlier workgroups of its task (every wait bounded).  The kernel is GENERATED from the
+ * region's own lowered programs: fx_plan_rowstream_source writes a HIP translation unit in which
+ * each program has been executed symbolically per output column, so that predicates of the
+ * select_rev / slice_rev / cat / stack chains that depend on the column are decided, and loads
+ * and sub-expressions shared between columns exist once per row.  Built into the library
+ * (csrc/fxhip/spec/fx_rs_<key>.hip; `python -m functs_amd.aot` writes them), it serves every
+ * plan with the same key: any number of rows and tasks, any per-task offsets, any values of the
+ * floating-point constants (thresholds, scale factors) as long as equal constants stay equal.
+ * Results are bit-identical to the generic kernels.  A plan without a linked kernel, and a call
+ * recorded under stream capture, takes the generic two passes.
+ * Stands where the reference generates and compiles CUDA for every subgraph
+ * (fait/tensorexpr/cuda_codegen_tssa.cpp:881-1121, :1319-1414) and leaves x[mask] to ATen
+ * (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
+ * fx_plan_rowstream_info: out[0] = the plan has a row-stream form, out[1] = a generated kernel
+ * for it is linked and enabled (fx_region_run uses it), out[2], out[3] = low and high word of its
+ * key, out[4] = elements per row of the streamed input, out[5] = rows, out[6] = tasks,
+ * out[7] = input buffers.  fx_plan_rowstream_why: what rules the form out (empty when out[0]).
+ * fx_set_rowstream: process-wide switch, default on (FXHIP_ROWSTREAM=0: off; also off while
+ * fx_set_specialization(0) holds). */
+int fx_plan_rowstream_info(const fx_plan*, int64_t* out, int cap);
+int fx_plan_rowstream_why(const fx_plan*, char* buf, size_t cap);               /* returns the full length */
+int fx_plan_rowstream_source(const fx_plan*, const char* label, char* buf, size_t cap); /* returns the full length */
+void fx_set_rowstream(int on);
+/* test hook: the argument block of a generated kernel for this plan (what travels in front of the
+ * marshalled block of fx_region_marshal) with the given rows per workgroup and per sub-tile, so
+ * that a generated unit compiled for the CPU can be driven without a device */
+int fx_plan_rowstream_launch(const fx_plan*, uint32_t chunk_rows, uint32_t sub_rows, void* out, size_t cap);
+int fx_rowstream_count(void);                   /* generated row-stream kernels linked into the library */
 /* debugging / test hooks: the lowered bytecode blob (like CodeGen::getCodeText) */
 int fx_plan_blob(const fx_plan*, const uint32_t** words, size_t* n_words);
 int fx_plan_disasm(const fx_plan*, char* buf, size_t cap);

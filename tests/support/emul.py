@@ -79,3 +79,68 @@ def run(region, *args):
     if region.is_map:
         return [list(r) for r in outs]
     return [r[0] for r in outs]
+
+
+# ---- generated row-stream kernels on the CPU ----------------------------------------------
+_RS_SRC = os.path.join(_HERE, "fx_rs_host.cpp")
+_RS_DIR = os.path.join(_HERE, "_rs_build")
+_FXHIP = os.path.join(os.path.dirname(os.path.dirname(_HERE)), "functs_amd", "csrc", "fxhip")
+_rs_cache = {}
+
+
+def rowstream_host(region, *args, label="test"):
+    """The row-stream unit the generator writes for `region` with these arguments, compiled for
+    the CPU (tests/support/fx_rs_host.cpp); returns (ctypes handle, source text)."""
+    src = region.rowstream_source(*args, label=label)
+    key = region.rowstream_info(*args)["key"]
+    if key in _rs_cache:
+        return _rs_cache[key], src
+    os.makedirs(_RS_DIR, exist_ok=True)
+    gen = os.path.join(_RS_DIR, "fx_rs_%016x.hip" % key)
+    so_path = os.path.join(_RS_DIR, "fx_rs_%016x.so" % key)
+    with open(gen, "w") as f:
+        f.write(src)
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-fPIC", "-shared", "-x", "c++", "-ffp-contract=off",
+                           "-DFX_RS_GENERATED=\"%s\"" % gen, "-I", os.path.join(_FXHIP, "spec"), _RS_SRC, "-o", so_path])
+    so = ctypes.CDLL(so_path)
+    so.fx_rs_host_key.restype = ctypes.c_uint64
+    so.fx_rs_host_launch_bytes.restype = ctypes.c_size_t
+    so.fx_rs_host_run.restype = ctypes.c_int
+    so.fx_rs_host_run.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32]
+    assert so.fx_rs_host_key() == key
+    _rs_cache[key] = so
+    return so, src
+
+
+def run_rowstream(region, *args, chunk_rows=100, sub_rows=None, threads=7):
+    """Evaluate a compacting `region` on CPU tensors through its GENERATED row-stream code
+    (compiled for the CPU); returns what Region.__call__ returns."""
+    so, _ = rowstream_host(region, *args)
+    arr, n, keep = region._flatten(args)
+    p = region.plan(arr, n)
+    T = region.degree
+    outs, ptrs = [], (ctypes.c_void_p * max(p.n_out * T, 1))()
+    for o in range(p.n_out):
+        row = []
+        for t in range(T):
+            dt, shape = p.out_meta[o][t]
+            ten = torch.zeros(shape, dtype=dt)
+            ptrs[o * T + t] = ten.data_ptr()
+            row.append(ten)
+        outs.append(row)
+    scratch = torch.zeros(max(p.scratch_bytes, 1), dtype=torch.uint8)
+    totals = torch.zeros(T, dtype=torch.int32)
+    dyn = ctypes.create_string_buffer(lib.fx_dyn_bytes())
+    check(lib.fx_region_marshal(region._h, p.handle, arr, n, ptrs, scratch.data_ptr(), totals.data_ptr(), dyn, len(dyn)))
+    la = ctypes.create_string_buffer(so.fx_rs_host_launch_bytes())
+    info = region.rowstream_info(*args)
+    max_sub = min(64, (6 * 256 * 4 - 6) // info["row_elements"])
+    sub = max_sub if sub_rows is None else min(sub_rows, max_sub)
+    check(lib.fx_plan_rowstream_launch(p.handle, min(chunk_rows, 256), sub, la, len(la)))
+    rc = so.fx_rs_host_run(la, dyn, totals.data_ptr(), threads)
+    assert rc == 0, rc
+    tl = totals.tolist()
+    outs = [[ten.narrow(0, 0, tl[t]) for t, ten in enumerate(row)] for row in outs]
+    if region.is_map:
+        return [list(r) for r in outs]
+    return [r[0] for r in outs]

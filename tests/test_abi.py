@@ -82,6 +82,7 @@ def test_plan_metadata_and_disasm():
     assert p.n_out == 3 and p.compact
     assert _lib.lib.fx_plan_launches(p.handle) == 1 and _lib.lib.fx_plan_streaming(p.handle) == 0
     _lib.lib.fx_set_head_kernel(0)
+    _lib.lib.fx_set_rowstream(0)
     try:
         assert _lib.lib.fx_plan_launches(p.handle) == 2 and _lib.lib.fx_plan_streaming(p.handle) == 0
         _lib.lib.fx_set_streaming(1)
@@ -91,6 +92,7 @@ def test_plan_metadata_and_disasm():
             _lib.lib.fx_set_streaming(0)
     finally:
         _lib.lib.fx_set_head_kernel(1)
+        _lib.lib.fx_set_rowstream(1)
     assert p.out_meta[1][2] == (torch.float32, (preds.size(1), 80))
     assert p.alg_bytes == (preds.numel() + anchors.numel() + strides.numel()) * 4
     assert p.scratch_bytes > 0

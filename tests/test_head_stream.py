@@ -13,6 +13,15 @@ from oracle import configs as oc
 from tests.util import assert_boxes_close, assert_close, assert_exact, run_region
 
 
+@pytest.fixture(autouse=True)
+def hand_written_kernel_only():
+    """These tests are about the hand-written kernel: the generated row-stream kernels, which
+    come first where one is linked (tests/test_rowstream.py), are switched off."""
+    lib.fx_set_rowstream(0)
+    yield
+    lib.fx_set_rowstream(1)
+
+
 def _head(thr=0.3, obj_col=4, half=0.5, batch=None):
     """The region of configs.build_c2 / build_c5 with its constants as parameters."""
     r = Region(parallel_degree=batch, is_parallel_map=True) if batch else Region()

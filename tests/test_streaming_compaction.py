@@ -17,8 +17,10 @@ def generic_kernels_only():
     """The detection-head regions used here have a kernel of their own (tests/test_head_stream.py);
     these tests are about the generic one-pass form."""
     lib.fx_set_head_kernel(0)
+    lib.fx_set_rowstream(0)
     yield
     lib.fx_set_head_kernel(1)
+    lib.fx_set_rowstream(1)
 
 
 def _stream_info(r, *args):

@@ -218,3 +218,69 @@ def build_c5_generated_anchors(batch, levels):
     r.output(obj)
     r.compact_rows(keep)
     return r.finalize()
+
+
+# ---- other spellings of the detection head ------------------------------------------------
+# Decode + score filter of a YOLO-style head as programs in the field write it: the reference's own
+# model joins the four corners with torch.stack and pads the class scores with a zero column
+# (yolov3_bbox.py:12-23, 227-228), others concatenate the two corner pairs, keep the objectness in
+# another column, filter on a class score, or return one matrix per image.  None of them is the
+# text of build_c2 / build_c5; all of them are row compactions over a row-major prediction matrix,
+# which is what the generated row-stream kernels are for.  `python -m functs_amd.aot` generates
+# the kernels of HEAD_VARIANTS (80 classes, the benchmark's row length).
+HEAD_VARIANTS = {
+    "stack": dict(decode="stack"),
+    "cat": dict(decode="cat"),
+    "stack_padded": dict(decode="stack", pad=True),
+    "objectness_first": dict(obj_col=0),
+    "quarter_size": dict(half=0.25),
+    "class_score_mask": dict(mask_class=17),
+    "one_matrix": dict(decode="cat", joined=True),
+}
+
+
+def build_head_variant(batch=None, thr=0.3, decode="assign", pad=False, obj_col=4, half=0.5, mask_class=None, joined=False):
+    """A detection-head region.  pred [B, N, 5 + C] (columns: four box values, objectness at
+    obj_col among the first five, C class scores from column 5), anchors [N, 4], strides [N].
+    decode: how the corners are joined ("assign": four select assigns, "stack", "cat"); pad: the
+    class scores get a zero column behind them; mask_class: rows are kept on sigmoid(class score)
+    instead of the objectness; joined: one output [K, 4 + 1 + C] instead of three."""
+    r = Region(parallel_degree=batch, is_parallel_map=True) if batch else Region()
+    preds = r.tensor_input(torch.float32, 3)
+    anchors = r.tensor_input(torch.float32, 2)
+    strides = r.tensor_input(torch.float32, 1)
+    if batch:
+        i = r.task_index()
+        pred = preds.slice(0, i, r.op("INT_ADD", i, 1))
+    else:
+        pred = preds
+    box_cols = [c for c in range(5) if c != obj_col]
+    p = pred.select(0, 0)
+    pxy = r.stack([p.select(1, box_cols[0]), p.select(1, box_cols[1])], 1).sigmoid() if obj_col < 2 else p.slice(1, 0, 2).sigmoid()
+    pwh = r.stack([p.select(1, box_cols[2]), p.select(1, box_cols[3])], 1) if obj_col < 4 else p.slice(1, 2, 4)
+    obj = p.select(1, obj_col).sigmoid()
+    cls = p.slice(1, 5, None).sigmoid()
+    xy = (anchors.slice(1, 0, 2) + anchors.slice(1, 2, None)) * 0.5 + (pxy - 0.5) * strides.unsqueeze(-1)
+    wh = (anchors.slice(1, 2, None) - anchors.slice(1, 0, 2)) * half * pwh.exp()
+    if decode == "stack":
+        boxes = r.stack([xy.select(1, 0) - wh.select(1, 0), xy.select(1, 1) - wh.select(1, 1),
+                         xy.select(1, 0) + wh.select(1, 0), xy.select(1, 1) + wh.select(1, 1)], -1)
+    elif decode == "cat":
+        boxes = r.cat([xy - wh, xy + wh], 1)
+    else:
+        boxes = r.op("FULL", r.int_list([r.op("SIZE", anchors, 0), 4]), 0.0, dtype=torch.float32)
+        boxes = boxes.select_rev(xy.select(1, 0) - wh.select(1, 0), 1, 0)
+        boxes = boxes.select_rev(xy.select(1, 1) - wh.select(1, 1), 1, 1)
+        boxes = boxes.select_rev(xy.select(1, 0) + wh.select(1, 0), 1, 2)
+        boxes = boxes.select_rev(xy.select(1, 1) + wh.select(1, 1), 1, 3)
+    if pad:
+        cls = r.cat([cls, r.op("FULL", r.int_list([r.op("SIZE", anchors, 0), 1]), 0.0, dtype=torch.float32)], 1)
+    keep = (cls.select(1, mask_class) if mask_class is not None else obj) >= thr
+    if joined:
+        r.output(r.cat([boxes, obj.unsqueeze(-1), cls], 1))
+    else:
+        r.output(boxes)
+        r.output(cls)
+        r.output(obj)
+    r.compact_rows(keep)
+    return r.finalize()

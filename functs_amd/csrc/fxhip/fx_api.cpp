@@ -271,6 +271,7 @@ static std::atomic<uint32_t> g_stream_spin{[] {
 static std::atomic<uint32_t> g_lstm_spin{1000000u};   // polls of a wait of fx_lstm_stack before it is given up
 static std::mutex g_dump_mu;
 static std::string g_dump_dir;
+static int g_dump_what = 3;   // bit 0: program tables (fx_spec_*), bit 1: row-stream units (fx_rs_*)
 
 static std::atomic<uint64_t> g_launches{0}, g_spec_launches{0};
 
@@ -283,11 +284,13 @@ static const FxSpecKernels* spec_of(const fx::Plan* p) {
 // the translation unit that would specialise it there (one file per key).
 static void dump_spec_source(const fx::Plan* p) {
   std::string dir;
+  int what = 3;
   {
     std::lock_guard<std::mutex> g(g_dump_mu);
     dir = g_dump_dir;
+    what = g_dump_what;
   }
-  if (!dir.empty() && p->rs.ok && !fx_rs_find(p->rs.key)) {
+  if (!dir.empty() && (what & 2) && p->rs.ok && !fx_rs_find(p->rs.key)) {
     char rname[64];
     snprintf(rname, sizeof(rname), "/fx_rs_%016llx.hip", (unsigned long long)p->rs.key);
     const std::string rpath = dir + rname;
@@ -308,7 +311,7 @@ static void dump_spec_source(const fx::Plan* p) {
       }
     }
   }
-  if (dir.empty() || p->spec_key == 0 || fx_spec_find(p->spec_key)) return;
+  if (dir.empty() || !(what & 1) || p->spec_key == 0 || fx_spec_find(p->spec_key)) return;
   char name[64];
   snprintf(name, sizeof(name), "/fx_spec_%016llx.hip", (unsigned long long)p->spec_key);
   const std::string path = dir + name;
@@ -368,6 +371,10 @@ int fx_spec_dump_dir(const char* dir) {
   g_dump_dir = dir ? dir : "";
   return FX_OK;
 }
+void fx_spec_dump_what(int what) {
+  std::lock_guard<std::mutex> g(g_dump_mu);
+  g_dump_what = what & 3;
+}
 
 int fx_plan_num_outputs(const fx_plan* p) { return p ? (int)P(p)->out_dtype.size() : 0; }
 
@@ -388,7 +395,7 @@ size_t fx_plan_scratch_bytes(const fx_plan* p) { return p ? P(p)->scratch_bytes 
 static bool stream_active(const fx::Plan* pl, const FxSpecKernels* spec);
 static const FxSpecKernels* spec_of(const fx::Plan* p);
 static const FxRsKernel* rs_of(const fx::Plan* pl);
-static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl);
+static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl, const FxRsKernel* kern);
 static bool head_active(const fx::Plan* pl) {
   // (with compiled kernels switched off, fx_set_specialization(0), everything runs in the interpreter)
   return pl->mode == FX_MODE_COMPACT && pl->head.ok && g_head_mode.load(std::memory_order_relaxed) != 0 &&
@@ -451,7 +458,7 @@ int fx_plan_rowstream_launch(const fx_plan* p, uint32_t chunk_rows, uint32_t sub
   if (!p || !out || cap < sizeof(FxRsLaunch)) return fail(FX_E_INVALID, "fx_plan_rowstream_launch: out too small");
   if (!P(p)->rs.ok) return fail(FX_E_UNSUPPORTED, "this plan has no row-stream form: " + P(p)->rs.why);
   FxRsLaunch rl;
-  rs_fill_params(P(p), &rl);
+  rs_fill_params(P(p), &rl, nullptr);
   if (chunk_rows == 0 || chunk_rows > FX_BLOCK || sub_rows == 0 || sub_rows > rl.sub_rows)
     return fail(FX_E_INVALID, "fx_plan_rowstream_launch: chunk rows 1.." + std::to_string(FX_BLOCK) + ", sub-tile rows 1.." + std::to_string(rl.sub_rows));
   rl.chunk_rows = chunk_rows;
@@ -771,12 +778,20 @@ static const FxRsKernel* rs_of(const fx::Plan* pl) {
   const FxRsKernel* k = fx_rs_find(pl->rs.key);
   return (k && k->S == pl->rs.S) ? k : nullptr;
 }
-// Rows of a sub-tile: what FX_RS_KV 128-bit loads per lane carry, at most FX_RS_SUB.
-static uint32_t rs_sub_rows(const FxRsInfo& ri) {
-  const uint32_t cap = (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S;
-  return std::min<uint32_t>(FX_RS_SUB, cap);
+// Rows of a sub-tile: what FX_RS_KV 128-bit loads per lane carry, at most FX_RS_SUB, and no more
+// than keep the window and the staged outputs of a workgroup within FX_RS_LDS_BUDGET (six
+// workgroups per CU).
+#define FX_RS_LDS_BUDGET 26000u
+static uint32_t rs_sub_rows(const FxRsInfo& ri, const FxRsKernel* k = nullptr) {
+  uint32_t rows = std::min<uint32_t>(FX_RS_SUB, (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S);
+  if (k && k->n_staged) rows = std::min<uint32_t>(rows, std::max<uint32_t>(8u, (FX_RS_LDS_BUDGET / 4u - 8u * (k->n_staged + 1u)) / (ri.S + k->stage_row_words)));
+  return rows;
 }
-static uint32_t rs_lds_bytes(const FxRsInfo& ri) { return (((rs_sub_rows(ri) * ri.S + 3u + 3u) >> 2) + 1u) * 16u; }
+// the window, then the staged outputs (fx_rowstream.h lays them out the same way)
+static uint32_t rs_lds_bytes(const FxRsInfo& ri, const FxRsKernel* k) {
+  const uint32_t sub = rs_sub_rows(ri, k);
+  return (((sub * ri.S + 3u + 3u) >> 2) + 1u) * 16u + (sub * k->stage_row_words + 8u * k->n_staged) * 4u;
+}
 static size_t rs_status_words(const FxRsInfo& ri) {
   const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
   return (size_t)ri.n_tasks * ((ri.n_rows + min_chunk - 1) / min_chunk);
@@ -784,12 +799,12 @@ static size_t rs_status_words(const FxRsInfo& ri) {
 // Every task's rows are dealt to its workgroups in equal runs, as few workgroups as give every
 // resident slot of the device one (more only when a chunk would exceed FX_BLOCK rows, fewer when
 // it would fall below FX_RS_MIN_CHUNK).
-static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl) {
+static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl, const FxRsKernel* kern = nullptr) {
   const FxRsInfo& ri = pl->rs;
   memset(rl, 0, sizeof(*rl));
   rl->n_rows = ri.n_rows;
   rl->n_tasks = ri.n_tasks;
-  rl->sub_rows = rs_sub_rows(ri);
+  rl->sub_rows = rs_sub_rows(ri, kern);
   rl->spin_limit = g_stream_spin.load(std::memory_order_relaxed);
   rl->n_sptr = (uint32_t)pl->sptr.size();
   rl->n_tptr = (uint32_t)pl->tptr.size();
@@ -808,12 +823,12 @@ static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl) {
 }
 static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) {
   const FxRsInfo& ri = pl->rs;
-  rs_fill_params(pl, rl);
+  rs_fill_params(pl, rl, kern);
   if (pl->rs_resident == 0) {
     int dev = 0, cus = 0, per_cu = 0;
     HIP_OK(hipGetDevice(&dev));
     HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri)));
+    HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri, kern)));
     uint32_t wg = (uint32_t)std::max(per_cu, 1) * (uint32_t)std::max(cus, 1);
     // One slot per CU is left free: a launch that needs every slot the occupancy rule allows does
     // not get all of its workgroups placed at once, and the stragglers cost a second round.
@@ -837,7 +852,7 @@ static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const Fx
   const uint32_t grid = rl.chunks * rl.n_tasks;
   if (grid == 0) return hipSuccess;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri), stream);
+  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----

@@ -47,6 +47,9 @@ FX_RS_FN float rs_tanh(float x) { return fx_tanh(x); }
 struct FxRsRt {
   const FxRsLaunch& la;
   uint32_t task;
+  uint32_t* stg[FX_RS_MAX_OUT];   // LDS: where a staged output's kept rows of the sub-tile are put together
+  uint32_t ph[FX_RS_MAX_OUT];     // and the phase of the run in memory (first element's index mod 4)
+  FX_RS_FN const uint32_t* staged(int k) const { return stg[k]; }
   FX_RS_FN uint64_t ptr(uint32_t slot) const {
     const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
     const uint64_t* gp = (const uint64_t*)(ka + sizeof(FxRsLaunch));
@@ -135,13 +138,24 @@ FX_RS_FN void rs_st4(const FxRsRt& rt, int k, uint32_t off, uint32_t a, uint32_t
   v.x = a; v.y = b; v.z = c; v.w = d;
   __builtin_nontemporal_store(v, (FX_AS1 fx_u32x4_a4*)((FX_AS1 uint8_t*)rt.out(k) + ((off + rt.ooff(k)) << 2)));
 }
+// staged outputs (plain 32-bit elements): into LDS, and from there to element `e` of the output
+// buffer (the task's offset included; e a multiple of four for the group)
+FX_RS_FN void rs_stl(const FxRsRt& rt, int k, uint32_t off, uint32_t v) { rt.stg[k][rt.ph[k] + off] = v; }
+FX_RS_FN void rs_st_at(const FxRsRt& rt, int k, uint32_t e, uint32_t v) {
+  __builtin_nontemporal_store(v, (FX_AS1 uint32_t*)((FX_AS1 uint8_t*)rt.out(k) + (e << 2)));
+}
+FX_RS_FN void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  fx_u32x4 v;
+  v.x = a; v.y = b; v.z = c; v.w = d;
+  __builtin_nontemporal_store(v, (FX_AS1 fx_u32x4*)((FX_AS1 uint8_t*)rt.out(k) + (e << 2)));
+}
 
 }  // namespace
 #include "fx_rs_ops.h"
 namespace {
 
 template <class P>
-__global__ __launch_bounds__(FX_BLOCK) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
+__global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
   constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, KV = FX_RS_KV, NSUB = FX_RS_NSUB, S = P::S;
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];   // the window: sub_rows rows of S elements
   __shared__ uint32_t s_rowmap[FX_RS_SUB];
@@ -157,7 +171,17 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rs_kernel(const FxRsLaunch la, co
   const uint32_t n_sub0 = (c_rows + la.sub_rows - 1u) / la.sub_rows;
   const uint32_t sub_rows = (c_rows + n_sub0 - 1u) / n_sub0;
   const uint32_t n_sub = (c_rows + sub_rows - 1u) / sub_rows;
-  const FxRsRt rt{la, task};
+  FxRsRt rt{la, task, {}, {}};
+  {
+    // staged outputs behind the window, each sub_rows rows and a group of slack
+    uint32_t* sp = L + ((((la.sub_rows * S + 3u + 3u) >> 2) + 1u) << 2);
+#pragma unroll
+    for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) {
+      rt.stg[k] = sp;
+      rt.ph[k] = 0u;
+      if (k < P::n_out && P::stage_rowlen[k] != 0u) sp += la.sub_rows * P::stage_rowlen[k] + 8u;
+    }
+  }
   // element 0 of this task's rows of the window input
   const FX_AS1 uint32_t* win = (const FX_AS1 uint32_t*)rt.in(0) + (int64_t)la.in_tcoef[0] * task;
 
@@ -169,11 +193,10 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rs_kernel(const FxRsLaunch la, co
     shift = ((uint32_t)a0 & 15u) >> 2;   // elements between the 16-byte line and the first row
     const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(a0 & ~(uint64_t)15);
     n_vec = (shift + rows * S + 3u) >> 2;   // <= KV * NT (host)
+    // every line is used once; lanes past the end ask for the last line again rather than branch,
+    // so that the requests leave back to back
 #pragma unroll
-    for (uint32_t k = 0; k < KV; ++k) {
-      const uint32_t v = threadIdx.x + k * NT;
-      if (v < n_vec) wr[k] = __builtin_nontemporal_load(&g4[v]);   // every line is used once
-    }
+    for (uint32_t k = 0; k < KV; ++k) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
   };
   uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
   // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
@@ -260,15 +283,21 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rs_kernel(const FxRsLaunch la, co
       const uint32_t v = threadIdx.x + k * NT;
       if (v < n_vec) ((fx_u32x4*)L)[v] = wr[k];
     }
-    if (s + 1u < n_sub) request(s + 1u);
+    // all of the sub-tile is parked before the next one is asked for: interleaved, every new
+    // request would be waited for where the next old line is parked
+    asm volatile("" ::: "memory");
+    // (wave 1 looks back first where it does: its polls wait for everything it has asked for)
+    const bool looks_back = wave == 1u && s == 0u;
+    if (s + 1u < n_sub && !looks_back) request(s + 1u);
     const uint32_t t_r0 = s * sub_rows, t_rows = min(sub_rows, c_rows - t_r0);
     if (wave == 0) {
       const bool keep = lane < t_rows && s_keep[t_r0 + lane] != 0u;
       const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
       if (keep) s_rowmap[__popcll(bal & ((1ull << lane) - 1ull))] = lane;
       if (lane == 0) s_nk = (uint32_t)__popcll(bal);
-    } else if (wave == 1 && s == 0) {
+    } else if (looks_back) {
       look_back();
+      if (s + 1u < n_sub) request(s + 1u);
     }
     __syncthreads();
     if (s == 0) {
@@ -298,26 +327,35 @@ __global__ __launch_bounds__(FX_BLOCK) void fx_rs_kernel(const FxRsLaunch la, co
     const uint32_t* Wb = L + sh;
     const uint32_t orow = prefix + before;          // first compacted row of this sub-tile
     const uint32_t rs0 = c_r0 + t_r0;               // first source row of this sub-tile
+    fx_rs_phases<P, 0u>(rt, orow);
     // ---- the columns with code of their own: one kept row per lane
     if (P::n_row_cols != 0u && threadIdx.x < n_kept) {
       const uint32_t src = s_rowmap[threadIdx.x];
-      P::template row<FxRsRt>(rt, Wb + src * S, rs0 + src, orow + threadIdx.x);
+      P::template row<FxRsRt>(rt, Wb + src * S, rs0 + src, orow + threadIdx.x, threadIdx.x);
     }
     // ---- vector segments: four columns per lane
     fx_rs_segments<P>(typename P::Vecs{}, rt, Wb, s_rowmap, n_kept, rs0, orow, threadIdx.x, NT);
+    // ---- outputs put together in LDS leave as aligned runs
+    if (P::n_staged != 0u) {
+      __syncthreads();
+      fx_rs_copy_out<P, 0u>(rt, n_kept, orow, threadIdx.x, NT);
+    }
     before += n_kept;
   }
 }
 
 struct FxRsRegistrar {
-  FxRsRegistrar(uint64_t key, const void* fn, uint32_t S) {
+  FxRsRegistrar(uint64_t key, const void* fn, uint32_t S, uint32_t stage_row_words, uint32_t n_staged) {
     FxRsKernel k;
     k.fn = fn;
     k.S = S;
+    k.stage_row_words = stage_row_words;
+    k.n_staged = n_staged;
     fx_rs_register(key, k);
   }
 };
 
 }  // namespace
 
-#define FX_RS_REGISTER(P) static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P>, P::S);
+#define FX_RS_REGISTER(P) \
+  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P>, P::S, P::stage_row_words, P::n_staged);

@@ -24,7 +24,7 @@
 
 #include "fx_bytecode.h"
 
-#define FX_RS_VERSION 1u
+#define FX_RS_VERSION 2u
 #define FX_RS_MAX_IN 8u         // input buffers of a region
 #define FX_RS_MAX_OUT 8u        // outputs
 #define FX_RS_MAX_FIMM 24u      // distinct floating-point constants
@@ -35,6 +35,7 @@
 #define FX_RS_MIN_CHUNK 64u     // fewest rows of a chunk unless a task has fewer
 #define FX_RS_FLOOD_BYTES (8u << 20)   // first sub-tiles of a launch from which on the counts are sent ahead of the rows
 #define FX_RS_BULK_DELAY 128u          // by this many units of 64 clocks
+#define FX_RS_OCC 6              // waves per SIMD the register budget of a generated kernel is set for (80 registers)
 #define FX_RS_VEC_MIN 8u        // shortest run of alike columns that takes the vector form
 #define FX_RS_MAX_UNROLL 64u    // most columns evaluated one by one per row
 
@@ -78,7 +79,8 @@ static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte
 struct FxRsKernel {
   const void* fn = nullptr;     // fx_rs_kernel<P>
   uint32_t S = 0;               // row length the kernel is generated for
-  uint32_t static_lds = 0;      // bytes of its static LDS tables
+  uint32_t stage_row_words = 0; // elements per kept row that the kernel puts together in LDS before they leave
+  uint32_t n_staged = 0;        // outputs that take that route
 };
 void fx_rs_register(uint64_t key, const FxRsKernel& k);
 const FxRsKernel* fx_rs_find(uint64_t key);

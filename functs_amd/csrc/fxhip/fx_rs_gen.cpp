@@ -121,6 +121,10 @@ struct Model {
   FxRsInfo info;
   std::map<int32_t, int> input_of;            // pointer slot -> input index
   std::set<int> tcoef_seen;
+  // what the loads that are really executed (for some column) read of each pointer slot
+  struct LoadStat { bool bad = false; int64_t S = 0; std::set<int64_t> used; };
+  std::map<int32_t, LoadStat> stats;
+  bool collecting = false;
   std::map<uint32_t, int> fimm_of;            // float bits -> class
   std::vector<OutDesc> outs;
   uint32_t mask_begin = 0, mask_end = 0, mask_vt = 0;
@@ -203,6 +207,19 @@ struct Exec {
   }
   int loadNode(const FxInsn& in) {
     const Aff a = affOf(in.b);
+    if (m.collecting) {
+      // can the rows of this input be staged?  32-bit elements as they are, one row length, every
+      // element inside its row
+      Model::LoadStat& st = m.stats[in.a];
+      const int64_t last = a.cst + (int64_t)a.cl * ((int64_t)len - 1);
+      const int64_t lo = std::min(a.cst, last), hi = std::max(a.cst, last);
+      if ((in.dt != FX_F32 && in.dt != FX_I32) || (in.flags & FX_F_I2F) || a.c0 <= 0 || lo < 0 || hi >= a.c0) st.bad = true;
+      else if (st.S == 0) st.S = a.c0;
+      else if (st.S != a.c0) st.bad = true;
+      if (!st.bad && a.tcoef != 0 && a.tcoef < a.c0) st.bad = true;   // tasks that walk along the row: each reads a column
+      if (!st.bad)
+        for (int64_t x = lo; x <= hi; ++x) st.used.insert(x);
+    }
     const int k = m.inputOf(in.a);
     // per-task offset: one per input
     if (!m.tcoef_seen.count(k)) {
@@ -412,6 +429,7 @@ struct Exec {
         } break;
         case FX_LDXA: {
           if (M == M_FALSE) break;
+          if (m.collecting) m.stats[in.a].bad = true;   // a load through a computed index stays in memory
           Node n;
           n.kind = K_LOADX;
           // a dead element reads element 0
@@ -456,6 +474,14 @@ struct Exec {
             bool inr = a >= in.a && a < in.b;
             if (st > 1) inr = inr && ((a - in.a) % st == 0);
             A = g.cst(inr ? 1u : 0u);
+          } else if (g.nodes[A].kind == K_AFF && g.nodes[A].i[1] == 0) {
+            // a value that walks with the column only: decided for the whole segment, or the
+            // segment is not one
+            const int64_t x0 = g.nodes[A].i[0], x1 = x0 + g.nodes[A].i[2] * ((int64_t)len - 1);
+            const int64_t lo = std::min(x0, x1), up = std::max(x0, x1);
+            if (up < in.a || lo >= in.b) A = g.cst(0);
+            else if (lo >= in.a && up < in.b && (int32_t)in.imm <= 1) A = g.cst(1);
+            else throw Unsupported{"a predicate changes inside a vector segment"};
           } else {
             Node n;
             n.kind = K_IRANGE;
@@ -554,40 +580,39 @@ bool buildModel(const Plan& P, Model& m) {
       info.out_tstride[k] = o.task_stride;
     }
 
-    // ---- the window input: the 32-bit row-major input with the longest rows, every load of
-    // it inside its row
+    // ---- the window input: the 32-bit row-major input with the longest rows whose loads all stay
+    // inside their row.  What counts are the loads that are executed for some column (a load
+    // behind a column predicate is not executed for the other columns): a first run of every
+    // program, column by column, collects them.
     {
-      struct Cand { bool bad = false; int64_t S = 0; };
-      std::map<int32_t, Cand> cand;
-      auto scan = [&](uint32_t pb, uint32_t pe, const uint32_t* dim) {
-        for (uint32_t pc = pb; pc < pe; ++pc) {
-          const FxInsn& in = m.ins[pc];
-          if (in.op == FX_LDXA) { cand[in.a].bad = true; continue; }
-          if (!isAffineLoad(in)) continue;
-          Cand& c = cand[in.a];
-          if ((uint32_t)in.b >= m.n_aff) { c.bad = true; continue; }
-          const FxAffine& a = m.aff[in.b];
-          if ((in.dt != FX_F32 && in.dt != FX_I32) || (in.flags & FX_F_I2F) || a.rcoef[0] || a.rcoef[1]) { c.bad = true; continue; }
-          const int64_t S = fx_aff_coef(&a, 0);
-          int64_t lo = a.base, hi = a.base;
-          for (int k = 1; k < FX_MAXR; ++k) {
-            const int64_t ext = (int64_t)fx_aff_coef(&a, k) * ((int64_t)(dim ? dim[k] : 1u) - 1);
-            lo += std::min<int64_t>(ext, 0);
-            hi += std::max<int64_t>(ext, 0);
-          }
-          if (S <= 0 || lo < 0 || hi >= S) { c.bad = true; continue; }
-          if (c.S == 0) c.S = S;
-          else if (c.S != S) c.bad = true;
+      m.collecting = true;
+      Graph scratch;
+      {
+        Exec ex(m, scratch);
+        ex.run(m.mask_begin, m.mask_end);
+      }
+      for (const OutDesc& od : m.outs)
+        for (uint32_t col = 0; col < od.rowlen; ++col) {
+          Exec ex(m, scratch);
+          coordsOf(od, col, ex.c);
+          ex.run(od.prog_begin, od.prog_end);
         }
-      };
-      scan(m.mask_begin, m.mask_end, nullptr);
-      for (const OutDesc& od : m.outs) scan(od.prog_begin, od.prog_end, od.dim);
-      for (auto& kv : cand)
-        if (!kv.second.bad && kv.second.S > 0 && (m.win_slot < 0 || kv.second.S > cand[m.win_slot].S)) m.win_slot = kv.first;
+      m.collecting = false;
+      for (auto& kv : m.stats)
+        if (!kv.second.bad && kv.second.S > 0 && (m.win_slot < 0 || kv.second.S > m.stats[m.win_slot].S)) m.win_slot = kv.first;
       if (m.win_slot < 0) throw Unsupported{"no row-major 32-bit input that is read row by row"};
-      info.S = (uint32_t)cand[m.win_slot].S;
+      info.S = (uint32_t)m.stats[m.win_slot].S;
+      // streaming whole rows pays when most of a row is used
+      if (2 * (int64_t)m.stats[m.win_slot].used.size() < (int64_t)info.S) throw Unsupported{"less than half of every row of the widest input is read"};
       // a sub-tile of at least 8 rows in what FX_RS_KV 128-bit loads per lane carry
       if ((FX_RS_KV * FX_BLOCK * 4u - 6u) / info.S < 8u) throw Unsupported{"rows of the window input too long for a sub-tile"};
+      // the numbering of inputs and constants starts over: the key pass below fixes it
+      m.input_of.clear();
+      m.tcoef_seen.clear();
+      m.fimm_of.clear();
+      info.n_in = 0;
+      info.n_fimm = 0;
+      for (uint32_t k = 0; k < FX_RS_MAX_IN; ++k) { info.in_slot[k] = 0; info.in_tcoef[k] = 0; }
     }
 
     m.key.mix(FX_RS_VERSION);
@@ -858,6 +883,11 @@ std::string keyHex(uint64_t k) {
 }
 
 bool raw32(const OutDesc& od) { return (od.dtype == FX_F32 && od.vt == FX_VT_F) || (od.dtype == FX_I32 && od.vt == FX_VT_I); }
+// An output whose rows are not whole 16-byte groups is put together in LDS and leaves as one
+// aligned run per sub-tile (its kept rows are consecutive in memory): stores that start at any
+// 4-byte address, and single columns written with a stride of one row, cost a launch a quarter
+// of its time.
+bool staged(const OutDesc& od) { return raw32(od) && od.rowlen > 4 && od.rowlen % 4 != 0; }
 
 std::string emitSource(const Model& m, const std::string& label) {
   const std::string hx = keyHex(m.info.key);
@@ -875,6 +905,7 @@ std::string emitSource(const Model& m, const std::string& label) {
     o << "struct RS_" << hx << "_V" << k << " {\n"
       << "  static constexpr uint32_t out = " << sg.out << ", col0 = " << sg.col0 << ", len = " << sg.len
       << ", rowlen = " << od.rowlen << ", dtype = " << dtName(od.dtype) << ", vt = " << od.vt << ";\n"
+      << "  static constexpr bool staged = " << (staged(od) ? "true" : "false") << ";\n"
       << "  template <class RT>\n"
       << "  static FX_RS_FN uint32_t elem(const RT& rt, const uint32_t* W, uint32_t row, uint32_t t) {\n";
     Emitter em(m, m.g_vec[k], true, o, "    ");
@@ -885,7 +916,16 @@ std::string emitSource(const Model& m, const std::string& label) {
     << "  static constexpr uint64_t key = 0x" << hx << "ull;\n"
     << "  static constexpr uint32_t S = " << m.info.S << ", n_in = " << m.info.n_in << ", n_out = " << m.info.n_out
     << ", n_fimm = " << m.info.n_fimm << ";\n"
-    << "  // is the row kept?  Every load goes to memory: the mask runs ahead of the rows.\n"
+    << "  // elements per row of the outputs that are put together in LDS (0: written as they are computed)\n"
+    << "  static constexpr uint32_t stage_rowlen[" << FX_RS_MAX_OUT << "] = {";
+  for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) o << (k ? ", " : "") << ((k < m.outs.size() && staged(m.outs[k])) ? m.outs[k].rowlen : 0u);
+  {
+    uint32_t words = 0, n = 0;
+    for (const OutDesc& od : m.outs)
+      if (staged(od)) { words += od.rowlen; ++n; }
+    o << "};\n  static constexpr uint32_t stage_row_words = " << words << ", n_staged = " << n << ";\n";
+  }
+  o << "  // is the row kept?  Every load goes to memory: the mask runs ahead of the rows.\n"
     << "  template <class RT>\n"
     << "  static FX_RS_FN bool mask(const RT& rt, uint32_t row) {\n"
     << "    const uint32_t* W = nullptr; (void)W; const uint32_t t = 0; (void)t;\n";
@@ -897,11 +937,12 @@ std::string emitSource(const Model& m, const std::string& label) {
   }
   o << "  }\n"
     << "  // the columns that need code of their own, for one kept row: W is the row in the window,\n"
-    << "  // row its index in the task, orow its index among the kept rows\n"
+    << "  // row its index in the task, orow its index among the kept rows of the task, lrow among those\n"
+    << "  // of the sub-tile\n"
     << "  static constexpr uint32_t n_row_cols = " << m.row_cols.size() << ";\n"
     << "  template <class RT>\n"
-    << "  static FX_RS_FN void row(const RT& rt, const uint32_t* W, uint32_t row, uint32_t orow) {\n"
-    << "    const uint32_t t = 0; (void)t; (void)W; (void)row; (void)orow;\n";
+    << "  static FX_RS_FN void row(const RT& rt, const uint32_t* W, uint32_t row, uint32_t orow, uint32_t lrow) {\n"
+    << "    const uint32_t t = 0; (void)t; (void)W; (void)row; (void)orow; (void)lrow;\n";
   {
     Emitter em(m, m.g_row, true, o, "    ");
     std::vector<int> roots;
@@ -913,7 +954,10 @@ std::string emitSource(const Model& m, const std::string& label) {
       const OutDesc& od = m.outs[s.out];
       size_t e = k + 1;
       while (e < m.row_cols.size() && e - k < 4 && m.row_cols[e].out == s.out && m.row_cols[e].col0 == m.row_cols[e - 1].col0 + 1) ++e;
-      if (e - k == 4 && raw32(od)) {
+      if (staged(od)) {
+        o << "    rs_stl(rt, " << s.out << ", lrow * " << od.rowlen << "u + " << s.col0 << "u, " << em.ref(s.result) << ");\n";
+        ++k;
+      } else if (e - k == 4 && raw32(od)) {
         o << "    rs_st4(rt, " << s.out << ", orow * " << od.rowlen << "u + " << s.col0 << "u";
         for (size_t j = k; j < e; ++j) o << ", " << em.ref(m.row_cols[j].result);
         o << ");\n";

@@ -139,6 +139,13 @@ FX_RS_FN void fx_rs_segment(const RT& rt, const uint32_t* Wb, const uint32_t* ro
       const uint32_t t = (V::len % 4u == 0u || t0 + j < V::len) ? t0 + j : V::len - 1u;
       v[j] = V::template elem<RT>(rt, W, row, t);
     }
+    if constexpr (V::staged) {
+      // the output is put together in LDS (fx_rs_copy_out writes it): row r of the sub-tile's kept rows
+#pragma unroll
+      for (uint32_t j = 0; j < 4u; ++j)
+        if (V::len % 4u == 0u || t0 + j < V::len) rs_stl(rt, V::out, r * V::rowlen + V::col0 + t0 + j, v[j]);
+      continue;
+    }
     const uint32_t o0 = (orow + r) * V::rowlen + V::col0 + t0;
     if (raw && (V::len % 4u == 0u || t0 + 4u <= V::len)) {
       rs_st4(rt, V::out, o0, v[0], v[1], v[2], v[3]);
@@ -149,6 +156,39 @@ FX_RS_FN void fx_rs_segment(const RT& rt, const uint32_t* Wb, const uint32_t* ro
     }
   }
 }
+// phase in memory of the run of staged output K that starts at kept row orow
+template <class P, uint32_t K, class RT>
+FX_RS_FN void fx_rs_phases(RT& rt, uint32_t orow) {
+  if constexpr (K < P::n_out) {
+    if constexpr (P::stage_rowlen[K] != 0u) rt.ph[K] = (rt.ooff(K) + orow * P::stage_rowlen[K]) & 3u;
+    fx_rs_phases<P, K + 1u, RT>(rt, orow);
+  }
+}
+// The kept rows of a sub-tile of staged output K leave LDS as one run of n_kept * rowlen
+// consecutive elements from element e0 of the output: whole 16-byte groups where memory has them,
+// single elements at the two ends.  rt.staged(K) holds the run at the same phase as memory
+// (element i of the run at index (e0 & 3) + i), so the groups are aligned on both sides.
+template <class P, uint32_t K, class RT>
+FX_RS_FN void fx_rs_copy_out(const RT& rt, uint32_t n_kept, uint32_t orow, uint32_t tid, uint32_t nt) {
+  if constexpr (K < P::n_out) {
+    constexpr uint32_t RL = P::stage_rowlen[K];
+    if constexpr (RL != 0u) {
+      const uint32_t n = n_kept * RL;
+      const uint32_t e0 = rt.ooff(K) + orow * RL, ph = rt.ph[K];   // = e0 & 3 (fx_rs_phases)
+      const uint32_t* src = rt.staged(K);   // element i of the run at src[ph + i]
+      const uint32_t head = n < ((4u - ph) & 3u) ? n : ((4u - ph) & 3u);
+      const uint32_t groups = (n - head) >> 2, tail = (n - head) & 3u;
+      for (uint32_t g = tid; g < groups; g += nt) {
+        const uint32_t i = ph + head + 4u * g;   // a multiple of four
+        rs_st4_at(rt, K, e0 - ph + i, src[i], src[i + 1u], src[i + 2u], src[i + 3u]);
+      }
+      for (uint32_t i = tid; i < head; i += nt) rs_st_at(rt, K, e0 + i, src[ph + i]);
+      for (uint32_t i = tid; i < tail; i += nt) rs_st_at(rt, K, e0 + head + 4u * groups + i, src[ph + head + 4u * groups + i]);
+    }
+    fx_rs_copy_out<P, K + 1u, RT>(rt, n_kept, orow, tid, nt);
+  }
+}
+
 template <class P, class RT>
 FX_RS_FN void fx_rs_segments(FxRsList<>, const RT&, const uint32_t*, const uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t,
                              uint32_t) {}

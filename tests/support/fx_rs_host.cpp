@@ -10,6 +10,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <algorithm>
 #include <vector>
 
 #define FX_RS_HOST 1
@@ -55,6 +56,9 @@ struct FxRsRt {
   uint32_t task;
   const FxDyn* dyn;
   uint32_t* errw;
+  uint32_t* stg[FX_RS_MAX_OUT];
+  uint32_t ph[FX_RS_MAX_OUT];
+  const uint32_t* staged(int k) const { return stg[k]; }
   uint64_t ptr(uint32_t slot) const {
     const uint32_t pi = (slot & FX_SLOT_TASK) ? la.n_sptr + task * la.n_tptr + (slot & 0xffffu) : (slot & 0xffffu);
     return dyn->p[pi];
@@ -140,6 +144,18 @@ void rs_st4(const FxRsRt& rt, int k, uint32_t off, uint32_t a, uint32_t b, uint3
   rs_st<FX_F32, FX_VT_F>(rt, k, off + 3, d);
 }
 
+void rs_stl(const FxRsRt& rt, int k, uint32_t off, uint32_t v) { rt.stg[k][rt.ph[k] + off] = v; }
+void rs_st_at(const FxRsRt& rt, int k, uint32_t e, uint32_t v) {
+  memcpy((uint8_t*)(uintptr_t)rt.out(k) + ((size_t)e << 2), &v, 4);
+}
+void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  if (e & 3u) __builtin_trap();   // a group that is not aligned in memory
+  rs_st_at(rt, k, e, a);
+  rs_st_at(rt, k, e + 1, b);
+  rs_st_at(rt, k, e + 2, c);
+  rs_st_at(rt, k, e + 3, d);
+}
+
 }  // namespace
 #include "../../functs_amd/csrc/fxhip/fx_rs_ops.h"
 namespace {
@@ -154,7 +170,14 @@ void run_policy(const FxRsLaunch& la, const FxDyn* dyn, uint32_t* totals, uint32
   const uint32_t S = P::S;
   uint32_t errw = 0;
   for (uint32_t task = 0; task < la.n_tasks; ++task) {
-    FxRsRt rt{la, task, dyn, &errw};
+    FxRsRt rt{la, task, dyn, &errw, {}, {}};
+    // staged outputs: sub_rows rows each and a group of slack, poisoned before every sub-tile
+    std::vector<std::vector<uint32_t>> stage(FX_RS_MAX_OUT);
+    for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) {
+      stage[k].assign(k < P::n_out && P::stage_rowlen[k] ? (size_t)la.sub_rows * P::stage_rowlen[k] + 8u : 8u, 0u);
+      rt.stg[k] = stage[k].data();
+      rt.ph[k] = 0;
+    }
     const uint32_t* win = (const uint32_t*)(uintptr_t)rt.in(0) + (int64_t)la.in_tcoef[0] * task;
     uint32_t prefix = 0;
     for (uint32_t chunk = 0; chunk < la.chunks; ++chunk) {
@@ -179,10 +202,14 @@ void run_policy(const FxRsLaunch& la, const FxDyn* dyn, uint32_t* totals, uint32
           if (keep[t_r0 + r]) rowmap.push_back(r);
         const uint32_t n_kept = (uint32_t)rowmap.size();
         const uint32_t orow = prefix + before;
+        for (auto& st : stage) std::fill(st.begin(), st.end(), 0xdeadbeefu);
+        fx_rs_phases<P, 0u, FxRsRt>(rt, orow);
         if (P::n_row_cols != 0u)
-          for (uint32_t r = 0; r < n_kept; ++r) P::template row<FxRsRt>(rt, Wb + rowmap[r] * S, rs0 + rowmap[r], orow + r);
+          for (uint32_t r = 0; r < n_kept; ++r) P::template row<FxRsRt>(rt, Wb + rowmap[r] * S, rs0 + rowmap[r], orow + r, r);
         for (uint32_t tid = 0; tid < nt; ++tid)
           fx_rs_segments<P, FxRsRt>(typename P::Vecs{}, rt, Wb, rowmap.data(), n_kept, rs0, orow, tid, nt);
+        if (P::n_staged != 0u)
+          for (uint32_t tid = 0; tid < nt; ++tid) fx_rs_copy_out<P, 0u, FxRsRt>(rt, n_kept, orow, tid, nt);
         before += n_kept;
       }
       prefix += before;

@@ -778,18 +778,25 @@ static const FxRsKernel* rs_of(const fx::Plan* pl) {
   const FxRsKernel* k = fx_rs_find(pl->rs.key);
   return (k && k->S == pl->rs.S) ? k : nullptr;
 }
-// Rows of a sub-tile: what FX_RS_KV 128-bit loads per lane carry, at most FX_RS_SUB, and no more
-// than keep the window and the staged outputs of a workgroup within FX_RS_LDS_BUDGET (six
-// workgroups per CU).
-#define FX_RS_LDS_BUDGET 26000u
-static uint32_t rs_sub_rows(const FxRsInfo& ri, const FxRsKernel* k = nullptr) {
-  uint32_t rows = std::min<uint32_t>(FX_RS_SUB, (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S);
-  if (k && k->n_staged) rows = std::min<uint32_t>(rows, std::max<uint32_t>(8u, (FX_RS_LDS_BUDGET / 4u - 8u * (k->n_staged + 1u)) / (ri.S + k->stage_row_words)));
-  return rows;
+// Geometry of a launch.  Rows of a sub-tile: at most FX_RS_SUB and what FX_RS_KV 128-bit loads per
+// lane carry.  A workgroup pays about one trip to memory per sub-tile (the next one is asked for
+// when the current one has arrived), so the number of sub-tiles per chunk counts first, then how
+// full they are: measured on 16 x 10647 rows of 85 elements, chunks of 111 rows in two sub-tiles
+// take 23.4 us, in three 25.8 us; with a staged output 167 rows in three sub-tiles of 56 take
+// 24.3 us, 134 rows in three of 45 25.2 us, 223 rows in four 26.3 us.  Every candidate sub-tile
+// size fixes the LDS of a workgroup, with it the workgroups that are resident together, and with
+// them the chunk (every task's rows dealt to as many workgroups as are resident, at least
+// FX_RS_MIN_CHUNK rows, at most FX_BLOCK): the candidate with the fewest sub-tiles per chunk
+// wins, the larger sub-tile among equals.
+static uint32_t rs_env(const char* name) {   // tuning aids: 0 when not set
+  const char* e = getenv(name);
+  return e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
+}
+static uint32_t rs_max_sub_rows(const FxRsInfo& ri) {
+  return std::min<uint32_t>(FX_RS_SUB, (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S);
 }
 // the window, then the staged outputs (fx_rowstream.h lays them out the same way)
-static uint32_t rs_lds_bytes(const FxRsInfo& ri, const FxRsKernel* k) {
-  const uint32_t sub = rs_sub_rows(ri, k);
+static uint32_t rs_lds_bytes(const FxRsInfo& ri, const FxRsKernel* k, uint32_t sub) {
   return (((sub * ri.S + 3u + 3u) >> 2) + 1u) * 16u + (sub * k->stage_row_words + 8u * k->n_staged) * 4u;
 }
 static size_t rs_status_words(const FxRsInfo& ri) {
@@ -804,7 +811,8 @@ static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl, const FxRsKernel*
   memset(rl, 0, sizeof(*rl));
   rl->n_rows = ri.n_rows;
   rl->n_tasks = ri.n_tasks;
-  rl->sub_rows = rs_sub_rows(ri, kern);
+  rl->sub_rows = rs_max_sub_rows(ri);
+  (void)kern;
   rl->spin_limit = g_stream_spin.load(std::memory_order_relaxed);
   rl->n_sptr = (uint32_t)pl->sptr.size();
   rl->n_tptr = (uint32_t)pl->tptr.size();
@@ -824,24 +832,44 @@ static void rs_fill_params(const fx::Plan* pl, FxRsLaunch* rl, const FxRsKernel*
 static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) {
   const FxRsInfo& ri = pl->rs;
   rs_fill_params(pl, rl, kern);
-  if (pl->rs_resident == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
+  if (pl->rs_sub_rows == 0) {
+    int dev = 0, cus = 0;
     HIP_OK(hipGetDevice(&dev));
     HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri, kern)));
-    uint32_t wg = (uint32_t)std::max(per_cu, 1) * (uint32_t)std::max(cus, 1);
-    // One slot per CU is left free: a launch that needs every slot the occupancy rule allows does
-    // not get all of its workgroups placed at once, and the stragglers cost a second round.
-    if (per_cu >= 3) wg -= wg / (uint32_t)per_cu;
-    pl->rs_resident = std::max<uint32_t>(wg, 1u);
-    pl->rs_per_cu = (uint32_t)std::max(per_cu, 1);
+    const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
+    const uint32_t forced_sub = rs_env("FXHIP_RS_SUB_ROWS"), forced_chunk = rs_env("FXHIP_RS_CHUNK_ROWS");
+    uint32_t best_sub = 0, best_cr = 0, best_n = 0;
+    for (uint32_t sub = rs_max_sub_rows(ri); sub >= 8u; sub = sub > 8u ? std::max<uint32_t>(8u, sub - 8u) : 0u) {
+      if (forced_sub && sub > forced_sub) continue;
+      int per_cu = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri, kern, sub)) != hipSuccess || per_cu < 1) {
+        (void)hipGetLastError();
+        continue;
+      }
+      // at most the occupancy the kernels are compiled for: a launch that needs a seventh slot per CU
+      // (kernels that happen to stay below 73 registers) is not placed at once and takes 27.4 us
+      // where six per CU take 23.4 us
+      per_cu = std::min(per_cu, (int)FX_RS_OCC);
+      const uint32_t resident = (uint32_t)per_cu * (uint32_t)std::max(cus, 1);
+      const uint32_t per_task = std::max<uint32_t>(1u, resident / std::max<uint32_t>(ri.n_tasks, 1u));
+      uint32_t cr = (ri.n_rows + per_task - 1) / per_task;
+      cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
+      if (forced_chunk) cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(forced_chunk, min_chunk));
+      const uint32_t n = (cr + sub - 1) / sub;
+      if (rs_env("FXHIP_RS_VERBOSE"))
+        fprintf(stderr, "[fxhip] row-stream geometry: sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
+                sub, rs_lds_bytes(ri, kern, sub), per_cu, cr, n);
+      if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; }
+      if (forced_sub || sub == 8u) break;
+    }
+    if (best_sub == 0) return fail(FX_E_LIMIT, "row-stream kernel: no sub-tile size fits the device");
+    pl->rs_sub_rows = best_sub;
+    pl->rs_chunk_rows = best_cr;
   }
-  const uint32_t per_task = std::max<uint32_t>(1u, pl->rs_resident / std::max<uint32_t>(ri.n_tasks, 1u));
-  uint32_t cr = (ri.n_rows + per_task - 1) / per_task;
-  const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
-  cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
-  rl->chunk_rows = cr;
-  rl->chunks = (ri.n_rows + cr - 1) / cr;
+  rl->sub_rows = pl->rs_sub_rows;
+  rl->chunk_rows = pl->rs_chunk_rows;
+  rl->chunks = (ri.n_rows + rl->chunk_rows - 1) / rl->chunk_rows;
+  const uint32_t cr = rl->chunk_rows;
   // A launch whose first sub-tiles alone are megabytes of requests floods the memory system: there
   // the counts get a head start.  A small launch would only lose the time.
   const uint64_t first_bytes = (uint64_t)rl->chunks * ri.n_tasks * std::min<uint32_t>(cr, rl->sub_rows) * ri.S * 4u;
@@ -852,7 +880,7 @@ static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const Fx
   const uint32_t grid = rl.chunks * rl.n_tasks;
   if (grid == 0) return hipSuccess;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern), stream);
+  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----

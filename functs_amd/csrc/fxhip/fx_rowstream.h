@@ -274,9 +274,13 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     request(0);
   }
 
-  uint32_t prefix = 0, before = 0;
+  uint32_t prefix = 0, before = 0, staged_kept = 0, staged_orow = 0;
   for (uint32_t s = 0; s < n_sub; ++s) {
     if (s) __syncthreads();   // the window and the row map of the sub-tile before are no longer read
+    // Outputs that the sub-tile before put together in LDS leave now, as aligned runs, while the
+    // next window is parked: behind the barrier above everything is in place, and the barrier
+    // below keeps this sub-tile's values out of the buffers until everything has left.
+    if (P::n_staged != 0u && s) fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
     const uint32_t sh = shift;
 #pragma unroll
     for (uint32_t k = 0; k < KV; ++k) {
@@ -335,12 +339,13 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     }
     // ---- vector segments: four columns per lane
     fx_rs_segments<P>(typename P::Vecs{}, rt, Wb, s_rowmap, n_kept, rs0, orow, threadIdx.x, NT);
-    // ---- outputs put together in LDS leave as aligned runs
-    if (P::n_staged != 0u) {
-      __syncthreads();
-      fx_rs_copy_out<P, 0u>(rt, n_kept, orow, threadIdx.x, NT);
-    }
+    staged_kept = n_kept;
+    staged_orow = orow;
     before += n_kept;
+  }
+  if (P::n_staged != 0u) {
+    __syncthreads();
+    fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
   }
 }
 

@@ -161,7 +161,7 @@ _sig("fx_plan_spec_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_
 _sig("fx_set_specialization", None, _i)
 _sig("fx_specialization_count", _i)
 _sig("fx_spec_dump_dir", _i, ctypes.c_char_p)
-_sig("fx_spec_dump_what", None, _i)
+_sig("fx_spec_dump_what", _i, _i)
 _sig("fx_region_wait_totals", _i, _vp, _vp, _vp)
 _sig("fx_launch_stats", None, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64))
 _sig("fx_region_marshal", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,

@@ -74,10 +74,45 @@ def lstm(seed: int = 0, seq_len: int = 64, hidden: int = 512, layers: int = 2, b
     return x, wih, whh, bih, bhh
 
 
+def yolov3_head(seed: int = 0, batch: int = 16, grids=YOLO_GRIDS, classes: int = 80):
+    """Per level the NCHW map of the head [B, 3 * (5 + C), G, G] and its base anchors [3, 4]."""
+    g = _gen(seed)
+    maps = [torch.randn(batch, 3 * (5 + classes), cells, cells, generator=g) for cells in grids]
+    bases = []
+    for level in range(len(grids)):
+        half = torch.tensor(YOLO_BASE_SIZES[level], dtype=torch.float32) * 0.5
+        centre = torch.full((1, 2), YOLO_STRIDES[level] / 2.0)
+        bases.append(torch.cat([centre - half, centre + half], dim=1))
+    return maps, bases
+
+
+def attention_steps(seed: int = 0, batch: int = 1, heads: int = 12, length: int = 50, depth: int = 64, start: int = 32):
+    g = _gen(seed)
+    x = torch.randn(batch, heads, 1, depth, generator=g)
+    k = torch.zeros(batch, heads, length, depth)
+    v = torch.zeros(batch, heads, length, depth)
+    k[:, :, :start] = torch.randn(batch, heads, start, depth, generator=g)
+    v[:, :, :start] = torch.randn(batch, heads, start, depth, generator=g)
+    bound = (6.0 / (2 * depth)) ** 0.5
+    ws = [(torch.rand(heads, depth, depth, generator=g) * 2 - 1) * bound for _ in range(4)]
+    return (x, k, v) + tuple(ws) + (start,)
+
+
+def delta2bbox(seed: int = 0, n: int = 8732, classes: int = 4):
+    g = _gen(seed)
+    rois = torch.rand(n, 4, generator=g) * 150
+    rois[:, 2:] += rois[:, :2]
+    deltas = torch.randn(n, 4 * classes, generator=g)
+    return rois, deltas
+
+
 INPUTS = {
     "c1": get_started,
     "c2": yolov3_postproc,
     "c3": ssd_postproc,
     "c4": lstm,
     "c5": yolov3_batched,
+    "yolo_head": yolov3_head,
+    "attention": attention_steps,
+    "delta2bbox": delta2bbox,
 }

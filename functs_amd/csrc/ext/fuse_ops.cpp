@@ -15,6 +15,8 @@
 #include <unordered_map>
 #include <unordered_set>
 
+#include <torch/csrc/jit/passes/remove_mutation.h>
+
 #include "passes.h"
 #include "symbols.h"
 
@@ -741,6 +743,65 @@ bool unrollIn(Block* b, bool maps) {
 
 }  // namespace
 
+// A short loop over the elements of list arguments whose example elements differ in shape (the
+// levels of a feature pyramid): inside a loop or a map the elements have no static shape, written
+// out every level has its own (fait/passes/refine_types.cpp:57-81 keeps the per-element types for
+// exactly this; the reference's detection heads walk their levels with such loops,
+// yolov3_bbox.py:209-216).  Appends to lists are kept in order; RemoveListMutation turns them into
+// list constructions afterwards.
+bool readsRaggedList(Block* body) {
+  for (Node* n : body->nodes()) {
+    if (n->kind() != c10::aten::__getitem__) continue;
+    auto it = refinedTypes().find(n->input(0));
+    if (it == refinedTypes().end()) continue;
+    const auto& elems = it->second->expectRef<c10::TupleType>().elements();
+    for (const auto& e : elems)
+      if (*e != *elems[0]) return true;
+  }
+  return false;
+}
+
+bool tryUnrollRagged(Node* loop) {
+  auto trip = constant_as<int64_t>(loop->input(0));
+  auto cond = constant_as<bool>(loop->input(1));
+  Block* body = loop->blocks()[0];
+  auto next = constant_as<bool>(body->outputs()[0]);
+  if (!trip || *trip < 0 || *trip > 8 || !cond || !*cond || !next || !*next) return false;
+  for (Node* n : body->nodes()) {
+    if (!n->blocks().empty()) return false;
+    if (n->hasSideEffects() && n->kind() != c10::aten::append) return false;
+  }
+  if (!readsRaggedList(body)) return false;
+  Graph* g = loop->owningGraph();
+  WithInsertPoint guard(loop);
+  std::vector<Value*> carried(loop->inputs().begin() + 2, loop->inputs().end());
+  for (int64_t i = 0; i < *trip; ++i) {
+    std::unordered_map<Value*, Value*> vm;
+    vm[body->inputs()[0]] = g->insertConstant(i);
+    for (size_t k = 0; k < carried.size(); ++k) vm[body->inputs()[k + 1]] = carried[k];
+    cloneBodyBefore(body, loop, vm);
+    for (size_t k = 0; k < carried.size(); ++k) {
+      Value* r = body->outputs()[k + 1];
+      auto it = vm.find(r);
+      carried[k] = it != vm.end() ? it->second : r;
+    }
+  }
+  for (size_t k = 0; k < carried.size(); ++k) loop->output(k)->replaceAllUsesWith(carried[k]);
+  loop->destroy();
+  return true;
+}
+
+bool UnrollRaggedListLoops(std::shared_ptr<Graph> graph) {
+  bool changed = false;
+  Block* b = graph->block();
+  for (auto it = b->nodes().begin(); it != b->nodes().end();) {
+    Node* n = *it;
+    ++it;
+    if (n->kind() == c10::prim::Loop) changed = tryUnrollRagged(n) || changed;
+  }
+  return changed;
+}
+
 bool UnrollLoopsWithDeps(std::shared_ptr<Graph> graph) { return unrollIn(graph->block(), false); }
 bool UnrollSimpleMaps(std::shared_ptr<Graph> graph) { return unrollIn(graph->block(), true); }
 
@@ -994,7 +1055,21 @@ bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   }
   ConvertProfilingInstrumentation(graph);   // fait.cpp:137: range markers first, they cut regions
   LowerSimpleTuples(graph);
-  specialized = FoldStaticTypeQueries(graph) || specialized;
+  if (UnrollRaggedListLoops(graph)) {
+    ConstantPropagation(graph);      // list[constant] of a constant list, arithmetic on the level index
+    RemoveListMutation(graph);       // the appends of what were iterations become list constructions
+    specialized = true;
+  }
+  // InferShape + constant folding (fait_pipeline.cpp:47-49): sizes of intermediate values that
+  // the program asks for (new_zeros(n, x.size(1), 1)) fold like those of the arguments; twice,
+  // because a folded size is what lets the next creation operator be typed
+  for (int round = 0; round < 3; ++round) {
+    const bool typed = InferStaticShapes(graph);
+    const bool folded = FoldStaticTypeQueries(graph);
+    specialized = specialized || folded;
+    ConstantPropagation(graph);
+    if (!typed && !folded) break;
+  }
   ConstantPropagation(graph);
   UniformConstantsToFills(graph);
   EliminateCommonSubexpression(graph);
@@ -1022,6 +1097,7 @@ bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   CanonicalizeFusableMaps(graph);   // fait_pipeline.cpp:61
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
+  InferStaticShapes(graph);   // results of the functors, and the argument types of the functors behind them
   if (SinkProducersIntoMaps(graph)) {   // (folds size queries on the producer's results)
     ConstantPropagation(graph);
     UniformConstantsToFills(graph);

@@ -78,6 +78,14 @@ void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
 bool SinkProducersIntoMaps(std::shared_ptr<torch::jit::Graph> graph);
 void setSinkProducers(bool on);
 
+// Static types of intermediate values (the reference's InferShape, fait/passes/refine_types.cpp:
+// 420-685, run at fait_pipeline.cpp:47): every operator node whose tensor arguments have complete
+// static types and whose other arguments are constants is run on meta tensors of those types, and
+// its results take the types of what comes back; a tssa::ParallelFunctor is lowered for its
+// argument types instead (nothing runs) and its input_refine_types are brought up to date.  Shapes
+// that depend on data stay unknown.  True if a type was set.
+bool InferStaticShapes(std::shared_ptr<torch::jit::Graph> graph);
+
 // Plans the region of every tssa::ParallelFunctor of a built graph for the static types in its
 // input_refine_types (meta tensors stand for them; nothing runs, no device is needed), as the
 // reference compiles every functor when its operator is created (fait/fuser/graph_builder.cpp:

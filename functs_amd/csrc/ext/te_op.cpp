@@ -22,6 +22,7 @@
 #include <torch/csrc/jit/passes/dead_code_elimination.h>
 #include <torch/csrc/jit/runtime/custom_operator.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <map>
@@ -580,7 +581,7 @@ class RegionRunner {
   // them; nothing runs): `kind` is the first word of fx_plan_head_info when that kernel is in
   // use (0: the generic kernels), `shapes` the shapes of task 0's results.
   void dryRun(const std::vector<c10::IValue>& samples, int64_t* kind, std::vector<std::vector<int64_t>>* shapes,
-              int64_t* rowstream = nullptr, std::string* rowstream_why = nullptr) {
+              int64_t* rowstream = nullptr, std::string* rowstream_why = nullptr, std::vector<c10::ScalarType>* dtypes = nullptr) {
     TORCH_CHECK(samples.size() == n_stack_, "dryRun: argument count");
     int64_t degree = degree_;
     size_t first = 0;
@@ -617,6 +618,7 @@ class RegionRunner {
       int64_t sizes[FX_ARG_MAX_RANK];
       FX_OK_OR_THROW(fx_plan_output(plan, o, 0, &dt, &rank, sizes));
       shapes->emplace_back(sizes, sizes + rank);
+      if (dtypes) dtypes->push_back(atDtype(dt));
     }
   }
 
@@ -898,6 +900,20 @@ void Translator::node(const Node* n) {
   }
   if (k == aten::tensor) {
     int dt = dtypeArg(n->input(1));
+    // a short constant list (torch.tensor([0.1, 0.1, 0.2, 0.2])): its elements stacked
+    auto iv = toIValue(n->input(0));
+    if (iv && (iv->isDoubleList() || iv->isIntList() || iv->isBoolList())) {
+      std::vector<int> elems;
+      if (iv->isDoubleList())
+        for (double x : iv->toDoubleVector()) elems.push_back(op(FX_OP_SCALAR_TENSOR, {cfloat(x)}, dt < 0 ? FX_DT_F32 : dt));
+      else if (iv->isIntList())
+        for (int64_t x : iv->toIntVector()) elems.push_back(op(FX_OP_SCALAR_TENSOR, {cint(x)}, dt < 0 ? FX_DT_I64 : dt));
+      else
+        for (bool x : iv->toBoolList()) elems.push_back(op(FX_OP_SCALAR_TENSOR, {cbool(x)}, dt < 0 ? FX_DT_BOOL : dt));
+      TORCH_CHECK(!elems.empty() && elems.size() <= 64, "aten::tensor of ", elems.size(), " constants inside a fused region");
+      out(op(FX_OP_STACK, {tlist(elems), cint(0)}));
+      return;
+    }
     out(op(FX_OP_SCALAR_TENSOR, {in(0)}, dt));
     return;
   }
@@ -1141,6 +1157,14 @@ bool isPlainFunctor(const Node* n) {
          (!n->hasAttribute(sym::compact_rows()) || n->i(sym::compact_rows()) == 0);
 }
 
+// The dry runs of the passes plan regions that the built graph may not keep (a producer before it
+// sinks, a merged functor that is not taken): those leave no sources in a capture directory.
+struct NoSourceDump {
+  int before;
+  NoSourceDump() : before(fx_spec_dump_what(0)) {}
+  ~NoSourceDump() { fx_spec_dump_what(before); }
+};
+
 // a meta tensor of a complete static type
 bool sampleOf(const c10::TypePtr& type, c10::IValue* out) {
   auto tt = type->cast<c10::TensorType>();
@@ -1155,20 +1179,46 @@ bool sampleOf(const c10::TypePtr& type, c10::IValue* out) {
   return true;
 }
 
+// what stands for a functor argument when the region is only lowered: a meta tensor of its static
+// type, the value of a constant, any device for a device (placement does not enter the lowering)
+bool sampleOfArg(const c10::TypePtr& type, Value* v, c10::IValue* out) {
+  if (sampleOf(type, out)) return true;
+  if (auto c = toIValue(v)) {
+    *out = *c;
+    return true;
+  }
+  if (v->type()->kind() == c10::TypeKind::DeviceObjType) {
+    *out = c10::IValue(c10::Device(c10::kCPU));
+    return true;
+  }
+  return false;
+}
+
 // F1 = plain functor, F2 = compacting map functor that reads F1's results as shared arguments.
 // Returns true if the graph changed.
+bool trySinkProducer(Node* f2, Node* f1);
+
 bool trySink(Node* f2) {
-  Graph* g = f2->owningGraph();
   const auto par2 = f2->is(sym::is_parallel_args());
   const size_t first2 = f2->i(sym::parallel_degree()) < 0 ? 1 : 0;
-  Node* f1 = nullptr;
+  // the plain functors among the producers of F2's shared arguments, the last one first: of a
+  // chain of producers the one next to the map sinks first, then the one that fed it
+  std::vector<Node*> producers;
   for (size_t k = first2; k < f2->inputs().size(); ++k) {
     Node* p = f2->input(k)->node();
     if (par2[k - first2] != 0 || !isPlainFunctor(p) || p->owningBlock() != f2->owningBlock()) continue;
-    if (f1 && p != f1) return false;
-    f1 = p;
+    if (std::find(producers.begin(), producers.end(), p) == producers.end()) producers.push_back(p);
   }
-  if (!f1) return false;
+  std::sort(producers.begin(), producers.end(), [](Node* a, Node* b) { return b->isBefore(a); });
+  for (Node* f1 : producers)
+    if (trySinkProducer(f2, f1)) return true;
+  return false;
+}
+
+bool trySinkProducer(Node* f2, Node* f1) {
+  Graph* g = f2->owningGraph();
+  const auto par2 = f2->is(sym::is_parallel_args());
+  const size_t first2 = f2->i(sym::parallel_degree()) < 0 ? 1 : 0;
   for (Node* n : f1->g(c10::attr::Subgraph)->nodes())
     if (n->kind() == sym::LstmStack() || n->kind() == sym::ForallSelectRev()) return false;
   // F1's results may only feed F2 and size queries with a constant dimension
@@ -1176,18 +1226,37 @@ bool trySink(Node* f2) {
     for (const Use& u : o->uses()) {
       if (u.user == f2) continue;
       if (u.user->kind() == c10::aten::size && u.user->inputs().size() == 2 && constant_as<int64_t>(u.user->input(1))) continue;
+      if (u.user->kind() == c10::prim::device) continue;   // answered by F1's own arguments, below
       return false;
     }
+  // where F1's results live is where its tensor arguments live
+  {
+    Value* some_tensor = nullptr;
+    for (Value* in : f1->inputs())
+      if (!some_tensor && isTensorValue(in)) some_tensor = in;
+    for (Value* o : f1->outputs()) {
+      const auto uses = o->uses();
+      for (const Use& u : uses) {
+        if (u.user->kind() != c10::prim::device) continue;
+        if (!some_tensor) return false;
+        u.user->replaceInput(0, some_tensor);
+      }
+    }
+  }
   // static types of F1's arguments, and what F1 returns for them
   std::vector<c10::IValue> samples1;
-  for (const c10::TypePtr& t : f1->tys(sym::input_refine_types())) {
-    c10::IValue v;
-    if (!sampleOf(t, &v)) return false;
-    samples1.push_back(v);
+  {
+    const auto types1 = f1->tys(sym::input_refine_types());
+    if (types1.size() != f1->inputs().size()) return false;
+    for (size_t k = 0; k < types1.size(); ++k) {
+      c10::IValue v;
+      if (!sampleOfArg(types1[k], f1->input(k), &v)) return false;
+      samples1.push_back(v);
+    }
   }
-  if (samples1.size() != f1->inputs().size()) return false;
   std::vector<std::vector<int64_t>> shapes1;
   try {
+    NoSourceDump quiet;
     int64_t kind1 = 0;
     RegionRunner r1(f1);
     r1.dryRun(samples1, &kind1, &shapes1);
@@ -1201,6 +1270,7 @@ bool trySink(Node* f2) {
     const auto uses = f1->output(o)->uses();
     for (const Use& u : uses) {
       if (u.user == f2) continue;
+      if (u.user->kind() != c10::aten::size) continue;
       int64_t d = *constant_as<int64_t>(u.user->input(1));
       const int64_t rank = (int64_t)shapes1[o].size();
       if (d < 0) d += rank;
@@ -1255,7 +1325,7 @@ bool trySink(Node* f2) {
     Value* p = sub2->inputs()[k - first2 + 1];
     if (in->node() == f1) continue;   // bound below, once F1's nodes are in
     c10::IValue v;
-    if (par2[k - first2] != 0 || !sampleOf(types2[k - first2], &v)) { destroyMerged(); return changed; }
+    if (par2[k - first2] != 0 || !sampleOfArg(types2[k - first2], in, &v)) { destroyMerged(); return changed; }
     f->addInput(in);
     types.push_back(types2[k - first2]);
     par.push_back(0);
@@ -1279,15 +1349,20 @@ bool trySink(Node* f2) {
   for (Value* out : f2->outputs()) f->addOutput()->copyMetadata(out);
   // only when the library runs the merged region as one of its hand-written kernels: lowered
   // generically every task would redo the producer
-  int64_t kind = 0;
+  int64_t kind = 0, rs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   try {
+    NoSourceDump quiet;
     std::vector<std::vector<int64_t>> shapes;
     RegionRunner rm(f);
-    rm.dryRun(samples, &kind, &shapes);
+    rm.dryRun(samples, &kind, &shapes, rs);
   } catch (const c10::Error&) {
     kind = 0;
+    rs[0] = 0;
   }
-  if (kind == 0) { destroyMerged(); return changed; }
+  // ... or as a row-stream kernel: then the merged region is a row compaction whose programs stay
+  // inside the rows of one task (no reduction, most of every row of the widest input used), so a
+  // task evaluates the producer for its own kept rows only and nothing is done twice
+  if (kind == 0 && rs[0] == 0) { destroyMerged(); return changed; }
   f->insertBefore(f2);
   for (size_t k = 0; k < f2->outputs().size(); ++k) f2->output(k)->replaceAllUsesWith(f->output(k));
   f2->destroy();
@@ -1304,7 +1379,7 @@ bool sinkIn(Block* b) {
     if (n->kind() != sym::ParallelFunctor() || n->i(sym::is_parallel_map()) == 0 || !n->hasAttribute(sym::compact_rows()) ||
         n->i(sym::compact_rows()) == 0)
       continue;
-    changed |= trySink(n);
+    if (trySink(n)) return true;   // the block changed under the walk: the caller starts over
   }
   return changed;
 }
@@ -1315,11 +1390,168 @@ void ToParallelFunctor(std::shared_ptr<Graph> graph) { toFunctorIn(graph->block(
 
 bool SinkProducersIntoMaps(std::shared_ptr<Graph> graph) {
   if (!g_sink_producers.load()) return false;
-  const bool changed = sinkIn(graph->block());
-  if (changed) EliminateDeadCode(graph);
+  bool changed = false;
+  for (int round = 0; round < 64 && sinkIn(graph->block()); ++round) {   // a chain of producers sinks one by one
+    changed = true;
+    EliminateDeadCode(graph);
+  }
   return changed;
 }
 void setSinkProducers(bool on) { g_sink_producers.store(on); }
+
+// ---------------------------------------------------------------------------
+// static shapes of intermediate values
+// ---------------------------------------------------------------------------
+namespace {
+
+bool completeTensorType(const c10::TypePtr& t) {
+  auto tt = t->cast<c10::TensorType>();
+  return tt && tt->scalarType() && tt->sizes().concrete_sizes();
+}
+
+c10::TypePtr typeOfSample(const at::Tensor& t, const c10::optional<c10::Device>& device) {
+  return c10::TensorType::create(t.scalar_type(), device, c10::VaryingShape<int64_t>(t.sizes().vec()),
+                                 c10::VaryingShape<int64_t>(t.strides().vec()), false);
+}
+
+// The node run on meta tensors of its arguments' static types: what it returns carries the
+// shapes of its results.  Only nodes whose other arguments are constants, and only operators
+// (nodes with blocks are walked, not run).
+bool inferNode(Node* n) {
+  // an element of a list argument with a refined type, at a constant index: the element's type
+  if (n->kind() == c10::aten::__getitem__ && isTensorValue(n->output()) && !completeTensorType(n->output()->type())) {
+    auto it = refinedTypes().find(n->input(0));
+    auto idx = constant_as<int64_t>(n->input(1));
+    if (it == refinedTypes().end() || !idx) return false;
+    const auto& elems = it->second->expectRef<c10::TupleType>().elements();
+    const int64_t i = *idx < 0 ? *idx + (int64_t)elems.size() : *idx;
+    if (i < 0 || i >= (int64_t)elems.size() || !completeTensorType(elems[i])) return false;
+    n->output()->setType(elems[i]);
+    return true;
+  }
+  if (n->blocks().size() != 0 || n->kind() == c10::prim::Constant || n->kind() == c10::prim::ListConstruct ||
+      n->kind() == c10::prim::TupleConstruct || n->kind().is_prim() && n->kind() != c10::prim::NumToTensor)
+    return false;
+  bool wanted = false;
+  for (Value* o : n->outputs()) wanted = wanted || (isTensorValue(o) && !completeTensorType(o->type()));
+  if (!wanted || !n->maybeOperator()) return false;
+  const std::string ns = n->kind().ns().toUnqualString();
+  if (ns != "aten" && ns != "immut") return false;
+  Stack stack;
+  c10::optional<c10::Device> device;
+  for (Value* in : n->inputs()) {
+    c10::IValue v;
+    if (isTensorValue(in)) {
+      if (auto c = toIValue(in)) {
+        if (!c->isTensor() || !c->toTensor().defined()) return false;
+        const at::Tensor t = c->toTensor();
+        if (!device) device = t.device();
+        stack.emplace_back(at::empty_strided(t.sizes(), t.strides(), t.options().device(c10::kMeta)));
+        continue;
+      }
+      if (!sampleOf(in->type(), &v)) return false;
+      if (!device) device = in->type()->expectRef<c10::TensorType>().device();
+      stack.push_back(v);
+    } else if (in->type()->kind() == c10::TypeKind::ListType && in->node()->kind() == c10::prim::ListConstruct &&
+               in->type()->expectRef<c10::ListType>().getElementType()->kind() == c10::TypeKind::TensorType) {
+      c10::List<at::Tensor> lst;
+      for (Value* e : in->node()->inputs()) {
+        if (!sampleOf(e->type(), &v)) return false;
+        if (!device) device = e->type()->expectRef<c10::TensorType>().device();
+        lst.push_back(v.toTensor());
+      }
+      stack.emplace_back(lst);
+    } else if (auto c = toIValue(in)) {
+      stack.push_back(*c);
+    } else if (in->type()->kind() == c10::TypeKind::DeviceObjType) {
+      stack.emplace_back(c10::Device(c10::kMeta));   // where a tensor is created does not change its shape
+    } else {
+      return false;
+    }
+  }
+  try {
+    n->getOperation()(stack);
+  } catch (const std::exception&) {
+    return false;   // shapes that depend on data, arguments the operator refuses on this device
+  }
+  if (stack.size() != n->outputs().size()) return false;
+  bool changed = false;
+  for (size_t k = 0; k < n->outputs().size(); ++k) {
+    Value* o = n->output(k);
+    if (!isTensorValue(o) || !stack[k].isTensor() || !stack[k].toTensor().defined() || completeTensorType(o->type())) continue;
+    o->setType(typeOfSample(stack[k].toTensor(), device));
+    changed = true;
+  }
+  return changed;
+}
+
+// A functor lowered for the static types of its arguments (nothing runs): types of its results,
+// and its input_refine_types brought up to date.
+bool inferFunctor(Node* n) {
+  if (n->i(sym::parallel_degree()) < 0) return false;
+  for (Node* k : n->g(c10::attr::Subgraph)->nodes())
+    if (k->kind() == sym::LstmStack()) return false;
+  const bool is_map = n->i(sym::is_parallel_map()) != 0;
+  const auto par = n->is(sym::is_parallel_args());
+  auto types = n->tys(sym::input_refine_types());
+  if (types.size() != n->inputs().size() || par.size() != types.size()) return false;
+  std::vector<c10::IValue> samples;
+  c10::optional<c10::Device> device;
+  bool refreshed = false;
+  for (size_t k = 0; k < types.size(); ++k) {
+    c10::IValue v;
+    if (is_map && par[k] != 0) {
+      auto et = types[k];
+      if (auto lt = et->cast<c10::ListType>()) et = lt->getElementType();
+      if (!sampleOf(et, &v)) return false;
+      c10::List<at::Tensor> lst;
+      for (int64_t t = 0; t < n->i(sym::parallel_degree()); ++t) lst.push_back(v.toTensor());
+      samples.emplace_back(lst);
+      continue;
+    }
+    // the value's own type, when the walk has given it one, is newer than the attribute
+    if (isTensorValue(n->input(k)) && completeTensorType(n->input(k)->type()) && !completeTensorType(types[k])) {
+      types[k] = n->input(k)->type();
+      refreshed = true;
+    }
+    if (!sampleOfArg(types[k], n->input(k), &v)) return false;
+    if (v.isTensor() && !device) device = types[k]->expectRef<c10::TensorType>().device();
+    samples.push_back(v);
+  }
+  if (refreshed) n->tys_(sym::input_refine_types(), types);
+  if (is_map) return refreshed;   // results are lists
+  bool wanted = false;
+  for (Value* o : n->outputs()) wanted = wanted || !completeTensorType(o->type());
+  if (!wanted) return refreshed;
+  std::vector<std::vector<int64_t>> shapes;
+  std::vector<c10::ScalarType> dtypes;
+  try {
+    NoSourceDump quiet;
+    int64_t kind = 0;
+    RegionRunner r(n);
+    r.dryRun(samples, &kind, &shapes, nullptr, nullptr, &dtypes);
+  } catch (const c10::Error&) {
+    return refreshed;
+  }
+  if (shapes.size() != n->outputs().size()) return refreshed;
+  for (size_t k = 0; k < shapes.size(); ++k)
+    n->output(k)->setType(c10::TensorType::createContiguous(dtypes[k], device ? *device : c10::Device(c10::kCPU), shapes[k]));
+  return true;
+}
+
+bool inferIn(Block* b) {
+  bool changed = false;
+  for (Node* n : b->nodes()) {
+    if (n->kind() == sym::ParallelFunctor()) changed |= inferFunctor(n);
+    else changed |= inferNode(n);
+    for (Block* inner : n->blocks()) changed |= inferIn(inner);
+  }
+  return changed;
+}
+
+}  // namespace
+
+bool InferStaticShapes(std::shared_ptr<Graph> graph) { return inferIn(graph->block()); }
 
 // ---------------------------------------------------------------------------
 // every functor of a built graph planned for its static argument types
@@ -1352,10 +1584,8 @@ void planIn(Block* b, std::vector<std::string>* report) {
         c10::List<at::Tensor> lst;
         for (int64_t t = 0; t < degree; ++t) lst.push_back(v.toTensor());
         samples.emplace_back(lst);
-      } else if (sampleOf(types[k], &v)) {
+      } else if (sampleOfArg(types[k], n->input(k), &v)) {
         samples.push_back(v);
-      } else if (auto c = toIValue(n->input(k))) {
-        samples.push_back(*c);
       } else {
         ok = false;
       }

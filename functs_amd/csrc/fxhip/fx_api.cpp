@@ -371,9 +371,11 @@ int fx_spec_dump_dir(const char* dir) {
   g_dump_dir = dir ? dir : "";
   return FX_OK;
 }
-void fx_spec_dump_what(int what) {
+int fx_spec_dump_what(int what) {
   std::lock_guard<std::mutex> g(g_dump_mu);
+  const int before = g_dump_what;
   g_dump_what = what & 3;
+  return before;
 }
 
 int fx_plan_num_outputs(const fx_plan* p) { return p ? (int)P(p)->out_dtype.size() : 0; }
@@ -956,7 +958,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     char key[17];
     snprintf(key, sizeof key, "%016llx", (unsigned long long)pl->spec_key);
     return fail(FX_E_LIMIT, std::string("the interpreter's temporaries of this region need ") + std::to_string(pl->lds_bytes) +
-                                " bytes of LDS (limit 65536) and no compiled kernels for its programs (key " + key +
+                                " bytes of LDS (limit 162816) and no compiled kernels for its programs (key " + key +
                                 ") are linked in or enabled: generate them with fx_plan_spec_source / python -m functs_amd.aot");
   }
   FxLaunchInfo li = launch_info(pl);

@@ -272,6 +272,32 @@ uint32_t fx_lds_bytes(const FxLaunchInfo& li) {
 // compiled kernels keep their temporaries in registers
 static uint32_t lds_bytes_compiled(const FxLaunchInfo& li) { return make_launch(li).temps_off * 4u; }
 
+// A workgroup may take all 160 KB of a CU's LDS on this device; more than the default 64 KB has
+// to be granted per kernel (and device) before the launch.  The interpreter's temporaries (4 KB
+// each per workgroup) are what needs it.
+template <class K>
+static hipError_t allow_lds(K kernel, uint32_t bytes) {
+  if (bytes <= 64u * 1024u) return hipSuccess;
+  static std::mutex mu;
+  static std::unordered_map<uint64_t, uint32_t> granted;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t key = ((uint64_t)(uintptr_t)(const void*)kernel << 6) ^ (uint64_t)dev;
+  std::lock_guard<std::mutex> g(mu);
+  uint32_t& have = granted[key];
+  if (have >= bytes) return hipSuccess;
+  e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) have = bytes;
+  return e;
+}
+#define FX_LAUNCH_LDS(kernel, grid, lds, stream, ...)          \
+  do {                                                         \
+    const hipError_t e__ = allow_lds(&kernel, lds);            \
+    if (e__ != hipSuccess) return e__;                         \
+    kernel<<<grid, FX_BLOCK, lds, stream>>>(__VA_ARGS__);      \
+  } while (0)
+
 hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                            hipStream_t stream, const FxSpecKernels* spec) {
   if (grid == 0) return hipSuccess;
@@ -280,11 +306,11 @@ hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li,
   if (spec && spec->dense) return launch_spec(spec->dense, sb, la, dyn, grid, lds_bytes_compiled(li), stream);
   switch (rank) {
     case 0:
-    case 1: fx_region_dense<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 2: fx_region_dense<2><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 3: fx_region_dense<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 4: fx_region_dense<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    default: fx_region_dense<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 1: FX_LAUNCH_LDS(fx_region_dense<1>, grid, lds, stream, sb, la, *dyn); break;
+    case 2: FX_LAUNCH_LDS(fx_region_dense<2>, grid, lds, stream, sb, la, *dyn); break;
+    case 3: FX_LAUNCH_LDS(fx_region_dense<3>, grid, lds, stream, sb, la, *dyn); break;
+    case 4: FX_LAUNCH_LDS(fx_region_dense<4>, grid, lds, stream, sb, la, *dyn); break;
+    default: FX_LAUNCH_LDS(fx_region_dense<FX_MAXR>, grid, lds, stream, sb, la, *dyn); break;
   }
   return hipGetLastError();
 }
@@ -293,7 +319,7 @@ hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, c
                                    hipStream_t stream, const FxSpecKernels* spec) {
   if (grid == 0) return hipSuccess;
   if (spec && spec->count) return launch_spec(spec->count, sb, make_launch(li), dyn, grid, lds_bytes_compiled(li), stream);
-  fx_compact_count<FxInterp><<<grid, FX_BLOCK, fx_lds_bytes(li), stream>>>(sb, make_launch(li), *dyn);
+  FX_LAUNCH_LDS(fx_compact_count<FxInterp>, grid, fx_lds_bytes(li), stream, sb, make_launch(li), *dyn);
   return hipGetLastError();
 }
 
@@ -306,11 +332,11 @@ hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunc
     return launch_spec(spec->scatter, sb, la, dyn, grid, lds_bytes_compiled(li), stream, spec->scatter_threads);
   switch (rank) {
     case 0:
-    case 1: fx_compact_scatter<1><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 2: fx_compact_scatter<2><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 3: fx_compact_scatter<3><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    case 4: fx_compact_scatter<4><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
-    default: fx_compact_scatter<FX_MAXR><<<grid, FX_BLOCK, lds, stream>>>(sb, la, *dyn); break;
+    case 1: FX_LAUNCH_LDS(fx_compact_scatter<1>, grid, lds, stream, sb, la, *dyn); break;
+    case 2: FX_LAUNCH_LDS(fx_compact_scatter<2>, grid, lds, stream, sb, la, *dyn); break;
+    case 3: FX_LAUNCH_LDS(fx_compact_scatter<3>, grid, lds, stream, sb, la, *dyn); break;
+    case 4: FX_LAUNCH_LDS(fx_compact_scatter<4>, grid, lds, stream, sb, la, *dyn); break;
+    default: FX_LAUNCH_LDS(fx_compact_scatter<FX_MAXR>, grid, lds, stream, sb, la, *dyn); break;
   }
   return hipGetLastError();
 }

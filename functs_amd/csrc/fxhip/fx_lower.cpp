@@ -2261,7 +2261,9 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   const uint32_t lds_descriptor = P->lds_bytes - (uint32_t)((size_t)max_temps * FX_V * FX_BLOCK * 4);
   FX_CHECK(lds_descriptor <= 64 * 1024, FX_E_LIMIT,
            "region descriptor needs " << lds_descriptor << " bytes of LDS (limit 65536)");
-  P->needs_compiled = P->lds_bytes > 64 * 1024;
+  // (a workgroup of the interpreter may take the 160 KB of a CU: 36 temporaries; the launchers
+  // ask for what goes beyond the default 64 KB)
+  P->needs_compiled = P->lds_bytes > 160 * 1024 - 1024;
   if (P->stream.ok) {
     // Rows per workgroup: the largest of 256 / 128 / 64 whose window fits LDS next to the
     // descriptor (compiled kernels keep temporaries in registers; the interpreter checks its own

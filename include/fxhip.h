@@ -273,7 +273,7 @@ void fx_set_specialization(int on);             /* process-wide switch, default 
 int fx_specialization_count(void);              /* specialised regions linked into the library */
 void fx_launch_stats(uint64_t* total, uint64_t* specialised); /* region kernel launches of this process so far */
 int fx_spec_dump_dir(const char* dir);          /* plans without specialised kernels leave their source in dir (NULL: stop) */
-void fx_spec_dump_what(int what);               /* which sources: 1 program tables (fx_spec_*), 2 row-stream units (fx_rs_*), 3 both (default) */
+int fx_spec_dump_what(int what);                /* which sources: 1 program tables (fx_spec_*), 2 row-stream units (fx_rs_*), 3 both (default), 0 none; returns the setting before */
 
 /* ---- execution (replaces CudaCodeGenTssa::call_raw, cuda_codegen_tssa.cpp:1167-1290) ----
  * out_ptrs[out_idx * parallel_degree + task] = device buffer of that output.

@@ -772,6 +772,19 @@ bool tryUnrollRagged(Node* loop) {
     if (n->hasSideEffects() && n->kind() != c10::aten::append) return false;
   }
   if (!readsRaggedList(body)) return false;
+  // Only where the levels are joined afterwards (every list the body appends to is read by cat /
+  // stack alone): what follows then needs the shapes of all levels.  Levels whose results stay
+  // apart are independent tasks of different shapes: a map runs them in one launch.
+  bool appends = false;
+  for (Node* n : body->nodes()) {
+    if (n->kind() != c10::aten::append) continue;
+    appends = true;
+    for (const Use& u : n->input(0)->uses()) {
+      if (u.user == n) continue;
+      if (u.user->kind() != c10::aten::cat && u.user->kind() != c10::aten::stack) return false;
+    }
+  }
+  if (!appends) return false;
   Graph* g = loop->owningGraph();
   WithInsertPoint guard(loop);
   std::vector<Value*> carried(loop->inputs().begin() + 2, loop->inputs().end());

@@ -204,11 +204,16 @@ def recorded_traffic(kernel, workload):
 
 
 def head_kernel_in_use(plan):
-    """Does a call of this plan run one of the hand-written head kernels?  Its name
-    (fx_head_stream: YOLO-style heads; fx_classmap_head: SSD-style heads) or None."""
+    """Does a call of this plan run as ONE launch of a compaction kernel built for its shape of
+    work?  The kernel's name or None: fx_rs_kernel is the row-stream kernel GENERATED from the
+    region's own programs; fx_head_stream (YOLO-style heads) and fx_classmap_head (SSD-style
+    heads) are the hand-written ones."""
     import ctypes
     from functs_amd import _lib
     out = (ctypes.c_int64 * 8)()
+    _lib.check(_lib.lib.fx_plan_rowstream_info(plan.handle, out, 8))
+    if out[1]:
+        return "fx_rs_kernel"
     _lib.check(_lib.lib.fx_plan_head_info(plan.handle, out, 8))
     if not out[1]:
         return None
@@ -322,11 +327,30 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0):
     return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us, cold_us, cold_sync_us
 
 
-def cpu_baseline(name, budget_s):
+def set_kernels(rowstream, head):
+    """Which kernels a compacting region may run: the generated row-stream kernels, the
+    hand-written head kernels; with both off, the generic count + scatter pair."""
+    from functs_amd import _lib
+    _lib.lib.fx_set_rowstream(1 if rowstream else 0)
+    _lib.lib.fx_set_head_kernel(1 if head else 0)
+
+
+def cpu_baseline(name, budget_s, threads=None):
     import torch
     from oracle import configs as oc
     fn = oc.scripted(name)
     cpu_args = getattr(oc, name + "_inputs")(0)
+    before = torch.get_num_threads()
+    if threads:
+        torch.set_num_threads(threads)
+    try:
+        return _cpu_loop(fn, cpu_args, budget_s)
+    finally:
+        torch.set_num_threads(before)
+
+
+def _cpu_loop(fn, cpu_args, budget_s):
+    import torch
     for _ in range(2):
         fn(*cpu_args)
     n, t0 = 0, time.perf_counter()
@@ -349,9 +373,14 @@ def main():
     ap.add_argument("--no-per-config", action="store_true")
     ap.add_argument("--interpreter", action="store_true",
                     help="run every region with the bytecode interpreter (no ahead-of-time compiled kernels)")
+    ap.add_argument("--no-rowstream", action="store_true",
+                    help="run compacting regions without the generated row-stream kernels (fx_rs_kernel): the detection heads "
+                         "(c2, c5) then run the hand-written fx_head_stream")
     ap.add_argument("--no-head-kernel", action="store_true",
-                    help="run the detection-head regions (c2, c5) with the generic row-compaction kernels (count + scatter) "
-                         "instead of the hand-written fx_head_stream")
+                    help="run compacting regions with the generic row-compaction kernels (count + scatter): neither the "
+                         "generated row-stream kernels nor the hand-written head kernels")
+    ap.add_argument("--cpu-seconds-per-config", type=float, default=2.0,
+                    help="CPU time spent on the baseline of each configuration other than the headline one")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch the library's plain copy kernel on BYTES (3 times): the known-size reference "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
@@ -370,9 +399,8 @@ def main():
     import functs_amd.aot as aot
     if args.interpreter:
         aot.enable(False)
-    if args.no_head_kernel:
-        from functs_amd import _lib
-        _lib.lib.fx_set_head_kernel(0)
+    use_rs, use_head = not (args.no_rowstream or args.no_head_kernel), not args.no_head_kernel
+    set_kernels(use_rs, use_head)
 
     if args.copy_calibration:
         from functs_amd import _lib
@@ -386,7 +414,7 @@ def main():
 
     if args.cold_profile:
         from functs_amd.region import timed_sets
-        w = Workload(args.workload, dev, fused=not args.no_head_kernel)
+        w = Workload(args.workload, dev, fused=use_head)
         n_sets = w.grow_cold()
         flush(dev)
         call_ms = [timed_sets([s[i] for s in w.sets], which=-1, rounds=args.cold_profile) for i in range(len(w.bound))]
@@ -397,7 +425,7 @@ def main():
         return
 
     def run_one(name, with_cpu):
-        w = Workload(name, dev, fused=not args.no_head_kernel)
+        w = Workload(name, dev, fused=use_head)
         ms, kern, single = measure(w, args.steps, args.warmup)
         alg = w.algorithmic_bytes()
         # the same kernels with consecutive launches rotated over buffer sets that together
@@ -439,6 +467,34 @@ def main():
             rec["split_regions_kernel_us"] = [round(k * 1e3, 2) for k in split_cold]
             rec["split_regions_call_kernels_us"] = round(sum(split_regions) * 1e3, 2)
             rec["split_regions_launches_per_call"] = w.launches
+        if rec["row_compaction"] and rec["head_kernel"]:
+            # the same call on the library's other kernels for it: with the generated row-stream
+            # kernels off (the hand-written head kernel where one matches the region) and on the
+            # generic pair (count + scatter), every launch on cold lines as above
+            def other(rowstream, head, fused):
+                set_kernels(rowstream, head)
+                try:
+                    w2 = Workload(name, dev, fused=fused)
+                    measure(w2, 5, 3)
+                    w2.grow_cold()
+                    k, regions = w2.cold_times_ms(rounds)
+                    which = next((x for x in (head_kernel_in_use(bc.plan) for bc in w2.bound) if x), None)
+                    return which, [round(x * 1e3, 2) for x in k], sum(regions)
+                finally:
+                    set_kernels(use_rs, use_head)
+            if rec["head_kernel"] == "fx_rs_kernel":
+                which, k, tot = other(False, True, True)
+                if which:
+                    rec["handwritten_kernel"] = which
+                    rec["handwritten_kernel_us"] = k
+                    rec["handwritten_frac_call"] = frac(tot)
+            which, k, tot = other(False, False, name != "c3")
+            rec["generic_kernel_us"] = k
+            rec["generic_call_kernels_us"] = round(tot * 1e3, 2)
+            rec["generic_frac_call"] = frac(tot)
+        copy_ms = copy_reference_ms(dev, alg)
+        rec["copy_same_bytes_us"] = round(copy_ms * 1e3, 2)
+        rec["copy_same_bytes_frac"] = frac(copy_ms)
         rec["compiled_kernels"] = rec["head_kernel"] is not None or all(bc.region.specialized(*bc.args) for bc in w.bound)
         if all(bc.region.specialized(*bc.args) for bc in w.bound):
             # the same launches through the bytecode interpreter (c3: of the two regions)
@@ -454,9 +510,13 @@ def main():
         rec["torchscript_route_drained_latency_us_warm"] = round(sync_us, 2)
         rec["torchscript_route_functors"] = n_functors
         rec["torchscript_route_compiled_share"] = round(spec_share, 3)
+        us, n, cores = cpu_baseline(name, args.cpu_seconds if with_cpu else args.cpu_seconds_per_config)
+        rec["cpu_baseline"] = {"value": round(us, 1), "unit": "us", "cores": cores, "kind": "port",
+                               "sample": "%d calls of torch.jit.script(%s) on the same seeded CPU tensors" % (n, name)}
         if with_cpu:
-            us, n, cores = cpu_baseline(name, args.cpu_seconds)
-            rec["cpu"] = (us, n, cores)
+            us1, n1, _ = cpu_baseline(name, min(args.cpu_seconds / 3, 4.0), threads=1)
+            rec["cpu_baseline_one_thread"] = {"value": round(us1, 1), "unit": "us", "cores": 1, "kind": "port",
+                                              "sample": "%d calls, torch.set_num_threads(1)" % n1}
         return rec
 
     def run_c4():
@@ -499,7 +559,12 @@ def main():
         graph_us = (time.perf_counter() - t0) * 1e6 / n_rep
         seq_len, layers = cpu_args[0].size(0), cpu_args[1].size(0)
         alg = 17072128  # weights + biases + x + out, each once
-        return {"workload": "c4 stacked LSTM 2x512, T=64, B=1", "torchscript_route_latency_us": round(us, 1),
+        c_us, c_n, c_cores = cpu_baseline("c4", args.cpu_seconds_per_config)
+        copy_ms = copy_reference_ms(dev, alg)
+        return {"workload": "c4 stacked LSTM 2x512, T=64, B=1",
+                "cpu_baseline": {"value": round(c_us, 1), "unit": "us", "cores": c_cores, "kind": "port",
+                                 "sample": "%d calls of torch.jit.script(c4) on the same seeded CPU tensors" % c_n},
+                "copy_same_bytes_us": round(copy_ms * 1e3, 2), "torchscript_route_latency_us": round(us, 1),
                 "torchscript_route_latency_us_synced": round(sync_us, 1),
                 "torchscript_route_latency_us_cold": round(cold_us, 1),
                 "torchscript_route_latency_us_cold_synced": round(cold_sync_us, 1),
@@ -610,6 +675,32 @@ def main():
                 "call_us": round(us, 1), "bytes_moved": moved, "gbps": round(moved / (us * 1e-6) / 1e9, 1),
                 "copy_kernel_same_bytes_us": round(copy_us, 1), "copy_kernel_gbps": round(2 * a.numel() / (copy_us * 1e-6) / 1e9, 1)}
 
+    def run_variants():
+        """Detection heads that are NOT the text of the benchmark's region (corners joined by stack
+        or cat, a padded class matrix, objectness in another column, another size constant, rows
+        kept on a class score, one joined output matrix) on c5's inputs: each runs as one launch of
+        the row-stream kernel generated from its own programs; cold lines, as for the configs."""
+        from functs_amd import configs
+        from functs_amd.benchmark.inputs import INPUTS
+        from functs_amd.region import timed_sets
+        cpu_args = INPUTS["c5"](0)
+        out = {}
+        for vname, kw in configs.HEAD_VARIANTS.items():
+            region = configs.build_head_variant(batch=16, **kw)
+            bound = [region.bind(*[a.clone().to(dev) for a in cpu_args]) for _ in range(6)]
+            for bc in bound:
+                bc.launch()
+            res = bound[0].results()
+            torch.cuda.synchronize()
+            alg = bound[0].plan.alg_bytes + sum(t.numel() * t.element_size() for o in res for t in (o if isinstance(o, list) else [o]))
+            flush(dev)
+            ms = timed_sets(bound, which=-1, rounds=8)
+            out[vname] = {"kernel": head_kernel_in_use(bound[0].plan), "launches_per_call": bound[0].plan.launches,
+                          "call_kernels_us": round(ms * 1e3, 2), "algorithmic_bytes": alg,
+                          "frac_hbm_peak_call": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            del bound
+        return out
+
     def run_stream():
         """Not one of the five configurations: one big fused elementwise region (sigmoid(2x + 1) on
         [8192, 4096] fp32), the shape on which the dense kernel itself meets the HBM roofline."""
@@ -640,7 +731,7 @@ def main():
     if not args.no_per_config:
         for name in ("c1", "c2", "c3", "c5"):
             if name == args.workload:
-                per[name] = {k: v for k, v in head.items() if k != "cpu"}
+                per[name] = dict(head)
                 continue
             try:
                 r = run_one(name, False)
@@ -651,6 +742,10 @@ def main():
             per["elementwise_stream"] = run_stream()
         except Exception as e:
             per["elementwise_stream"] = {"error": str(e)[:200]}
+        try:
+            per["head_variants"] = run_variants()
+        except Exception as e:
+            per["head_variants"] = {"error": str(e)[:200]}
         try:
             per["c4"] = run_c4()
         except Exception as e:
@@ -663,10 +758,9 @@ def main():
             per["c5_nms_tail"] = run_tail()
         except Exception as e:
             per["c5_nms_tail"] = {"error": str(e)[:200]}
-    cpu_us, cpu_n, cores = head.pop("cpu")
     dom_ms = head["kernel_us"][head["dominant_kernel_index"]] / 1e3
     dom_kernel = head.get("head_kernel") or ("fx_compact_scatter" if head["row_compaction"] else "fx_region_dense")
-    copy_ms = copy_reference_ms(dev, head["algorithmic_bytes"])
+    copy_ms = head["copy_same_bytes_us"] / 1e3
     traffic, traffic_src = recorded_traffic(dom_kernel, args.workload)
     out = {
         "metric": "per-call latency",
@@ -712,8 +806,8 @@ def main():
                                "the call in order, rotated the same way; frac_call_warm: sum of the warm kernels; "
                                "copy_same_bytes_ms / _frac: the library's plain copy kernel moving algorithmic_bytes (half read, "
                                "half written) on cold lines, the same way" % KERNEL_BATCH},
-        "cpu_baseline": {"value": round(cpu_us, 1), "unit": "us", "cores": cores, "kind": "port",
-                         "sample": "%d calls of torch.jit.script(%s) on the same seeded CPU tensors" % (cpu_n, args.workload)},
+        "cpu_baseline": head["cpu_baseline"],
+        "cpu_baseline_one_thread": head["cpu_baseline_one_thread"],
         "per_config": per,
     }
     print(json.dumps(out))

@@ -181,6 +181,8 @@ _sig("fx_compact_rows_scratch_bytes", ctypes.c_size_t, ctypes.c_int64)
 _sig("fx_compact_rows_static", _i, _vp, ctypes.c_int64, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
      ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i, _vp, _vp)
 _sig("fx_async_error", _i, _i)
+_sig("fx_async_error_take", _i, _i)
+_sig("fx_async_error_report", None, _i)
 _fp = ctypes.c_void_p
 _sig("fx_sort_nms", ctypes.c_int, ctypes.POINTER(FxNmsDesc), ctypes.c_void_p)
 _sig("fx_sort_nms_workspace_bytes", ctypes.c_size_t, ctypes.c_int, ctypes.c_uint32)

@@ -19,6 +19,7 @@
 // parallelize_loops.cpp:128-131): scalar-valued pure nodes of a loop or map body whose operands
 // are all defined outside move in front of the loop, innermost loops first, so that trip counts
 // and sizes stop looking like per-iteration values.
+#include <cmath>
 #include <ATen/ATen.h>
 #include <torch/csrc/jit/ir/constants.h>
 
@@ -307,7 +308,9 @@ bool fillsIn(Block* b) {
     for (const Use& u : n->output()->uses()) absorbed = absorbed && isFusableNode(u.user);
     if (!absorbed) continue;
     const at::Tensor flat = t.reshape({-1});
-    if (!at::eq(flat, flat[0]).all().item<bool>()) continue;
+    // uniform bit for bit: +0.0 and -0.0 compare equal and are different constants
+    const at::Tensor bits = st == c10::kFloat ? flat.view(c10::kInt) : flat;
+    if (!at::eq(bits, bits[0]).all().item<bool>()) continue;
     Graph* g = n->owningGraph();
     WithInsertPoint guard(n);
     Value* sizes = g->insertConstant(c10::IValue(c10::List<int64_t>(t.sizes().vec())));
@@ -317,7 +320,7 @@ bool fillsIn(Block* b) {
     const c10::Scalar v = flat[0].item();
     Value* fill = nullptr;
     auto type = c10::TensorType::create(t);
-    if (v.to<double>() == 0.0) {
+    if (v.to<double>() == 0.0 && !std::signbit(v.to<double>())) {   // aten::zeros makes +0.0
       fill = make(g, c10::aten::zeros, {sizes, dtype, none, device, none}, type);
     } else {
       Value* value = st == c10::kFloat ? g->insertConstant(v.to<double>())

@@ -94,8 +94,10 @@ PYBIND11_MODULE(_C, m) {
     for (const auto& kv : functorHostTimes()) d[py::str(kv.first)] = kv.second;
     return d;
   });
-  // Hash of the shapes and dtypes of the tensor arguments (lists and tuples of tensors element by
-  // element): the key under which functs_amd.jit keeps the graphs it has built for a function.
+  // Hash of the shapes, dtypes and devices of the tensor arguments (lists and tuples of tensors
+  // element by element) and of the kind of every other argument: the key under which
+  // functs_amd.jit keeps the graphs it has built for a function.  The device is part of it because
+  // a built graph holds folded prim::device constants and constant tensors on its example's device.
   m.def("_shape_key", [](const py::args& args) -> uint64_t {
     uint64_t h = 1469598103934665603ull;
     auto mix = [&h](uint64_t v) {
@@ -107,6 +109,11 @@ PYBIND11_MODULE(_C, m) {
       mix(0x7e50ull + (uint64_t)t.dim());
       for (int64_t d : t.sizes()) mix((uint64_t)d);
       mix((uint64_t)t.scalar_type());
+      mix(0xde71ceull + ((uint64_t)(uint8_t)t.device().type() << 8) + (uint64_t)(uint8_t)t.device().index());
+    };
+    auto other = [&mix](PyObject* o) {   // bool before int: a Python bool is an int
+      mix(o == Py_None ? 0x5ca1a0ull : PyBool_Check(o) ? 0x5ca1a1ull : PyLong_Check(o) ? 0x5ca1a2ull : PyFloat_Check(o) ? 0x5ca1a3ull
+          : PyUnicode_Check(o) ? 0x5ca1a4ull : 0x5ca1a7ull);
     };
     for (const py::handle& a : args) {
       PyObject* o = a.ptr();
@@ -118,10 +125,10 @@ PYBIND11_MODULE(_C, m) {
         for (Py_ssize_t i = 0; i < n; ++i) {
           PyObject* e = PySequence_Fast_GET_ITEM(o, i);
           if (THPVariable_Check(e)) tensor(e);
-          else mix(0x5ca1a7ull);
+          else other(e);
         }
       } else {
-        mix(0x5ca1a7ull);
+        other(o);
       }
     }
     return h;

@@ -319,12 +319,22 @@ c10::ScalarType atDtype(int d) {
     TORCH_CHECK(rc__ >= 0, "fxhip: ", fx_last_error(), " (", #expr, ")"); \
   } while (0)
 
-// what earlier launches reported through the library's error word (include/fxhip.h fx_async_error)
-int checkAsyncError() {
+// What earlier launches reported through the library's error word (include/fxhip.h
+// fx_async_error): every report is an error of this call, whichever operator made it - the word
+// is cleared by reading it, so a report that is not raised here would be lost.
+void resetLstmWorkspaces();
+void checkAsyncError() {
   const int e = fx_async_error(1);
-  TORCH_CHECK(e != FX_ASYNC_INT64, "tssa::ParallelFunctor: an earlier fused region read an int64 element outside 32 bits "
-              "into integer arithmetic; its results are not valid (moves of int64 data are exact, arithmetic is 32-bit)");
-  return e;
+  if (e == 0) return;
+  if (e & FX_ASYNC_BARRIER) resetLstmWorkspaces();   // a given-up wait leaves its workspace marked: the next call takes a cleared one
+  std::string what;
+  if (e & FX_ASYNC_INT64)
+    what += " a fused region read an int64 element outside 32 bits into integer arithmetic (moves of int64 data are exact, "
+            "arithmetic is 32-bit);";
+  if (e & FX_ASYNC_BARRIER) what += " fx::lstm_stack gave up a wait between its workgroups (its results were filled with NaN);";
+  if (e & FX_ASYNC_NMS_CAPACITY) what += " fx_sort_nms found more candidates in an image than the launch was sized for;";
+  if (e & ~(FX_ASYNC_INT64 | FX_ASYNC_BARRIER | FX_ASYNC_NMS_CAPACITY)) what += " unknown report " + std::to_string(e) + ";";
+  TORCH_CHECK(false, "functs_amd: an earlier launch reported an error, its results are not valid:", what);
 }
 
 // Host time of the operator by section, summed over calls while switched on: where a call's
@@ -1019,6 +1029,7 @@ LstmWorkspaces& lstmWorkspaces() {
   static LstmWorkspaces* w = new LstmWorkspaces();   // tensors must not outlive the HIP runtime's teardown order
   return *w;
 }
+void resetLstmWorkspaces() { lstmWorkspaces().reset(); }
 
 // fx::lstm_stack(x, wih, whh, bih, bhh, out?, state_h?, state_c?, T, L) -> (out, state_h, state_c)
 // is the loop nest
@@ -1078,9 +1089,7 @@ void runLstmStack(Stack& stack) {
   at::Tensor sc = result(c0, Lc, runs && Lc == L);
   if (T > 0 && L == 0) out.narrow(0, 0, T).copy_(x.narrow(0, 0, T));   // no layer: out[t] = x[t]
   if (runs) {
-    const int e = checkAsyncError();
-    if (e == FX_ASYNC_BARRIER) lstmWorkspaces().reset();   // a given-up wait leaves the workspace as it was
-    TORCH_CHECK(e != FX_ASYNC_BARRIER, "fx::lstm_stack: a wait of an earlier launch was given up; its results are not valid");
+    checkAsyncError();
     TORCH_CHECK(T <= INT32_MAX && B <= INT32_MAX && H <= INT32_MAX, "fx::lstm_stack: sizes beyond 32 bits");
     auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index());
     at::Tensor ws = lstmWorkspaces().get(x.device(), (void*)stream.stream(), B, H, L);

@@ -555,6 +555,19 @@ int fx_async_error(int clear) {
   return (int)v;
 }
 
+void fx_async_error_report(int bits) {
+  std::lock_guard<std::mutex> g(g_err_mu);
+  g_err_plain |= (uint32_t)bits;
+}
+int fx_async_error_take(int mask) {
+  std::lock_guard<std::mutex> g(g_err_mu);
+  uint32_t v = g_err_plain;
+  if (g_err_pinned) v |= *(volatile uint32_t*)g_err_pinned;
+  g_err_plain &= ~(uint32_t)mask;
+  if (g_err_pinned) *(volatile uint32_t*)g_err_pinned = *(volatile uint32_t*)g_err_pinned & ~(uint32_t)mask;
+  return (int)(v & (uint32_t)mask);
+}
+
 // Fill the by-value dynamic block.  Exposed (without launching) so that host
 // tests can check the marshalling.
 // `safe`: a device address that can always be read.  Kernels clamp the address of

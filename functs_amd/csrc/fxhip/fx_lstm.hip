@@ -125,7 +125,8 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
   const int n_wg = (int)gridDim.x;
   const int wg = (n_wg % 8 == 0) ? ((int)blockIdx.x % 8) * (n_wg / 8) + (int)blockIdx.x / 8 : (int)blockIdx.x;
   const int u0 = wg * UPW;
-  if (tid == 0) s_abort = 0u;
+  // a workspace that still carries a given-up wait is refused (below, behind the first barrier)
+  if (tid == 0) s_abort = fx_lstm_refused<DevAtomics>(a.ctl) ? 1u : 0u;
   // tags of this launch start behind those of every launch before it
   const uint32_t base = DevAtomics::load(a.ctl + FX_LSTM_W_BASE);
 
@@ -172,6 +173,11 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
     }
   }
   __syncthreads();
+  if (s_abort != 0u) {   // uniform: written once, ahead of the barrier
+    if (tid == 0 && a.err_host) __hip_atomic_store(a.err_host, (uint32_t)FX_ASYNC_BARRIER, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    fx_lstm_poison(a, L, (uint32_t)tid, (uint32_t)NT);
+    return;
+  }
   FX_LSTM_PSTAMP(1);
 
   const int n_steps = fx_lstm_steps(T, L);
@@ -285,7 +291,10 @@ __global__ __launch_bounds__(FX_LSTM_BLOCK * UPW, HPT >= 32 ? 4 : 2) void fx_lst
       // A wait that was given up: every wave of the workgroup leaves, nothing is checked out.  The
       // first wave looks at the word together with the waves' sums and leaves before it would store.
       if (wave != 0) {
-        if (s_abort != 0u) return;
+        if (s_abort != 0u) {   // the results are not to be used: the waves without cells say so in the data
+          fx_lstm_poison(a, L, (uint32_t)(tid - 64), (uint32_t)(NT - 64));
+          return;
+        }
       } else {
         // --- sixteen lanes a pair of layers: biases, gates, cells ---
         float part[NG][NW];

@@ -61,6 +61,27 @@ FX_LSTM_HD inline uint32_t fx_lstm_tag_of(uint64_t e) { return (uint32_t)(e >> 3
 FX_LSTM_HD inline uint32_t fx_lstm_tag_written(uint32_t base, int d) { return base + (uint32_t)d + 1u; }
 FX_LSTM_HD inline uint32_t fx_lstm_tag_read(uint32_t base, int d) { return base + (uint32_t)d; }
 
+// A wait that was given up: the launch's results are not to be used, and its workspace stays
+// marked (the error word) until the host clears it.  Two rules make that visible in the data
+// itself, whatever the caller does with the error report:
+//   a workgroup that gives up fills out, state_h and state_c with NaN before it leaves (a
+//   workgroup that has already finished may write a few values after that; the report still says
+//   that the launch failed);
+//   a launch that finds the error word set does no step at all: every workgroup reports the
+//   error again, fills the results with NaN and leaves.
+template <class A>
+FX_LSTM_HD inline bool fx_lstm_refused(uint32_t* ctl) { return A::load(ctl + FX_LSTM_W_ERR) != 0u; }
+// element first, first + stride, ... of the three results
+FX_LSTM_HD inline void fx_lstm_poison(const FxLstmArgs& a, int L, uint32_t first, uint32_t stride) {
+  const float nan = __builtin_nanf("");
+  const uint32_t n_out = (uint32_t)a.T * (uint32_t)a.B * (uint32_t)a.H, n_state = (uint32_t)L * (uint32_t)a.B * (uint32_t)a.H;
+  for (uint32_t i = first; i < n_out; i += stride) a.out[i] = nan;
+  for (uint32_t i = first; i < n_state; i += stride) {
+    a.state_h[i] = nan;
+    a.state_c[i] = nan;
+  }
+}
+
 // A workgroup that has finished its last step checks out; the last one to do so (nobody reads
 // or writes hbuf any more) moves the tag base past this launch's tags and puts the counter back
 // to zero, so the same workspace serves the next launch on the stream without a clear in

@@ -182,10 +182,14 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     // Keys and counters are written with device-scope atomic accesses, which go through to the
     // memory side of the caches, and the ticket is taken only after they have been acknowledged:
     // no release / acquire fence, which on this device would write back and invalidate whole
-    // caches once per workgroup.
+    // caches once per workgroup.  This rests on the device: a relaxed device-scope store is
+    // performed at the memory side of the caches by the time it is acknowledged (vmcnt).  The
+    // compiler is told the order explicitly: nothing moves across the signal fences.
     for (uint32_t k = tid; k < mine; k += FX_NMS_THREADS)
       if (gbase + k < key_cap) __hip_atomic_store(&g_keys[gbase + k], s_keys[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __syncthreads();
     if (tid == 0) s_ticket = atomicAdd(&ctr[1], 1u);
     __syncthreads();

@@ -47,8 +47,7 @@ class NmsResult:
         """Per image (dets [K, 5], labels [K], index [K]), the way the reference returns them."""
         n = self.n.cpu()   # waits for the launch
         if bool((n < 0).any()):   # FX_NMS_OVERFLOW
-            if lib.fx_async_error(0) == C["FX_ASYNC_NMS_CAPACITY"]:
-                lib.fx_async_error(1)
+            lib.fx_async_error_take(C["FX_ASYNC_NMS_CAPACITY"])   # this report is handled here; others stay
             raise _lib.FxError(C["FX_E_LIMIT"], "fx_sort_nms: an image has more candidates than the launch was sized for "
                                "(key_capacity; at most %d)" % MAX_CANDIDATES)
         out = []

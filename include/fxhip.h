@@ -337,16 +337,25 @@ size_t fx_dyn_bytes(void);
  * Integer ARITHMETIC is 32-bit: an int64 tensor element that enters it (a + 3, a == b, a as an
  * index) must fit 32 bits (a conversion to float uses the whole element and is exact).  The
  * loads check that; an element that does not fit sets a sticky process-wide error word, and
- * the outputs of that launch are not to be used.  fx_async_error returns 0 or what the word
- * holds (after the stream has been synchronised it covers every launch before that) and clears it
- * when `clear` is non-zero: FX_ASYNC_INT64 from these loads, FX_ASYNC_BARRIER from a barrier wait
- * that fx_lstm_stack gave up, FX_ASYNC_NMS_CAPACITY from fx_sort_nms (the latest report wins).  Integer constants and scalar arguments outside 32 bits are refused when
- * the region is planned / run (FX_E_UNSUPPORTED / FX_E_LIMIT).  The reference computes in int64
- * throughout (NNC kLong, functs/csrc/jit/ir/symbol_ext.cpp:17-117 for the eager bodies). */
+ * the outputs of that launch are not to be used.  Integer constants and scalar arguments outside
+ * 32 bits are refused when the region is planned / run (FX_E_UNSUPPORTED / FX_E_LIMIT).  The
+ * reference computes in int64 throughout (NNC kLong, functs/csrc/jit/ir/symbol_ext.cpp:17-117 for
+ * the eager bodies).
+ *
+ * The error word is a set of bits: FX_ASYNC_INT64 from these loads, FX_ASYNC_BARRIER from a wait
+ * that fx_lstm_stack gave up, FX_ASYNC_NMS_CAPACITY from fx_sort_nms (of the reports that kernels
+ * make the latest one is kept).  After the stream has been synchronised the word covers every
+ * launch before that.  fx_async_error returns the word and, when `clear` is non-zero, clears all
+ * of it; fx_async_error_take(mask) returns and clears only the bits of `mask`, for a caller that
+ * handles one kind of report and must leave the others to whoever handles those. */
 #define FX_ASYNC_INT64 1
 #define FX_ASYNC_BARRIER 2
-#define FX_ASYNC_NMS_CAPACITY 3
+#define FX_ASYNC_NMS_CAPACITY 4
 int fx_async_error(int clear);
+int fx_async_error_take(int mask);
+/* Adds bits to the word from the host: for code built on the library that finds such an error
+ * itself and reports it where its callers already look. */
+void fx_async_error_report(int bits);
 
 /* ---- stand-alone order-preserving row compaction (x[mask] for several x) ----
  * mask: n bytes (0/1); cols[i]: [n, rowlen[i]] fp32/int32 (4-byte) or int64 (8-byte) rows.
@@ -380,8 +389,11 @@ int fx_compact_rows_static(const uint8_t* mask, int64_t n, const void* const* co
  * registers for the whole sequence (thread k row k of them, and element k of the step's vectors);
  * the diagonals t + j follow each other without a barrier between workgroups, every h value
  * travels with the tag of the step that wrote it and readers poll for the tag they expect, with
- * bounded waits (a wait that is given up reports FX_ASYNC_BARRIER through fx_async_error and ends
- * the kernel).
+ * bounded waits.  A wait that is given up reports FX_ASYNC_BARRIER through fx_async_error, fills
+ * out / state_h / state_c with NaN and ends the kernel; its workspace stays marked, and every
+ * later launch on it does no step, reports the error again and returns NaN, until the caller has
+ * cleared the workspace.  A caller must therefore look at fx_async_error after synchronising and
+ * before it uses the results (or test them for NaN), and clear the workspace after an error.
  * Contiguous fp32: x [T, B, H]; wih, whh [L, 4, H, H]; bih, bhh [L, 4, 1, H]; h0, c0, state_h,
  * state_c [L, B, H]; out [T, B, H]; h0 / c0 may be null (zero initial state).  H is 32, 64, ...
  * 1024 (a power of two), L <= 4, B <= 16 (FX_E_UNSUPPORTED otherwise), and H / 2 workgroups of

@@ -26,12 +26,15 @@ def build():
 
 def lstm_emul():
     """ctypes handle of the CPU build of the persistent LSTM kernel's schedule and barrier."""
-    if not os.path.exists(_LSTM_SO):
+    sources = [os.path.join(_HERE, "lstm_emul.cpp"), os.path.join(_HERE, "..", "..", "functs_amd", "csrc", "fxhip", "fx_lstm_sched.h")]
+    if not os.path.exists(_LSTM_SO) or any(os.path.exists(s) and os.path.getmtime(s) > os.path.getmtime(_LSTM_SO) for s in sources):
         build()
     so = ctypes.CDLL(_LSTM_SO)
     fp = ctypes.c_void_p
     so.fx_lstm_emul.restype = ctypes.c_int
     so.fx_lstm_emul.argtypes = [fp] * 10 + [ctypes.c_int] * 4 + [ctypes.c_uint32, ctypes.c_int, ctypes.c_int, ctypes.c_uint32]
+    so.fx_lstm_emul_give_up.restype = ctypes.c_int
+    so.fx_lstm_emul_give_up.argtypes = [fp] * 10 + [ctypes.c_int] * 4 + [ctypes.c_uint32, ctypes.c_int]
     return so
 
 

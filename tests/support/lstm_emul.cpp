@@ -31,13 +31,15 @@ float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
 float bits_to_float(uint32_t b) { float f; memcpy(&f, &b, 4); return f; }
 uint32_t float_to_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
 
-// element i of a tagged vector, polled until it carries `want`; false: given up
-bool read_tagged(const FxLstmArgs& a, const uint64_t* p, uint32_t want, float* out) {
+// element i of a tagged vector, polled until it carries `want`; false: given up (the results
+// are filled with NaN, as the kernel's workgroup does on its way out)
+bool read_tagged(const FxLstmArgs& a, int L, const uint64_t* p, uint32_t want, float* out) {
   for (uint32_t polls = 0;; ++polls) {
     const uint64_t e = HostAtomics::load64(p);
     if (fx_lstm_tag_of(e) == want) { *out = bits_to_float((uint32_t)e); return true; }
     if (polls > a.spin_limit || ((polls & 255u) == 255u && HostAtomics::load(a.ctl + FX_LSTM_W_ERR) != 0u)) {
       HostAtomics::store(a.ctl + FX_LSTM_W_ERR, 1u);
+      fx_lstm_poison(a, L, 0u, 1u);
       return false;
     }
     std::this_thread::yield();
@@ -47,6 +49,10 @@ bool read_tagged(const FxLstmArgs& a, const uint64_t* p, uint32_t want, float* o
 // what one workgroup (hidden unit u) does; skip_wg: that workgroup stops writing after step 0
 void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
   const int H = a.H, B = a.B, T = a.T;
+  if (fx_lstm_refused<HostAtomics>(a.ctl)) {   // the workspace carries a given-up wait
+    fx_lstm_poison(a, L, (uint32_t)u, (uint32_t)n_wg);
+    return;
+  }
   const uint32_t base = HostAtomics::load(a.ctl + FX_LSTM_W_BASE);
   std::vector<float> c((size_t)L * B), cur(H), hp(H), hnew((size_t)L * B);
   for (int j = 0; j < L; ++j)
@@ -63,9 +69,9 @@ void workgroup(const FxLstmArgs& a, int L, int u, int n_wg, int skip_wg) {
       for (int b = 0; b < B; ++b) {
         for (int i = 0; i < H; ++i) {
           if (j == 0) cur[i] = a.x[((size_t)t * B + b) * H + i];
-          else if (!read_tagged(a, a.hbuf + fx_lstm_hoff(rp, j - 1, b, i, L, B, H), want, &cur[i])) return;
+          else if (!read_tagged(a, L, a.hbuf + fx_lstm_hoff(rp, j - 1, b, i, L, B, H), want, &cur[i])) return;
           if (t == 0) hp[i] = a.h0 ? a.h0[((size_t)j * B + b) * H + i] : 0.0f;
-          else if (!read_tagged(a, a.hbuf + fx_lstm_hoff(rp, j, b, i, L, B, H), want, &hp[i])) return;
+          else if (!read_tagged(a, L, a.hbuf + fx_lstm_hoff(rp, j, b, i, L, B, H), want, &hp[i])) return;
         }
         float g[4];
         for (int k = 0; k < 4; ++k) {
@@ -138,4 +144,54 @@ extern "C" int fx_lstm_emul(const float* x, const float* wih, const float* whh, 
     if (ctl[FX_LSTM_W_BASE] != expect_base || ctl[FX_LSTM_W_LEAVE] != 0u) return -1;
   }
   return 0;
+}
+
+// A wait that is given up, and what comes after it on the same workspace.  Three launches:
+//   1: workgroup `skip_wg` stops writing, the others give up;
+//   2: the same workspace, not cleared, every workgroup at work: must be refused;
+//   3: the workspace cleared: must run.
+// Before each launch the results are filled with 0.5.  Returns bits: 1 launch 1 set the error
+// word, 2 its results hold no value other than NaN or what the stopped workgroup wrote,
+// 4 launch 2 left the error word set, 8 its results are all NaN, 16 launch 3 ended without error
+// (its results are in out / state_h / state_c).
+extern "C" int fx_lstm_emul_give_up(const float* x, const float* wih, const float* whh, const float* bih, const float* bhh,
+                                    const float* h0, const float* c0, float* out, float* state_h, float* state_c, int T,
+                                    int B, int H, int L, uint32_t spin_limit, int skip_wg) {
+  std::vector<uint32_t> ctl(FX_LSTM_CTL_WORDS, 0u);
+  std::vector<uint64_t> hbuf((size_t)2 * L * B * H, 0ull);
+  FxLstmArgs a;
+  a.x = x; a.wih = wih; a.whh = whh; a.bih = bih; a.bhh = bhh; a.h0 = h0; a.c0 = c0;
+  a.out = out; a.state_h = state_h; a.state_c = state_c;
+  a.hbuf = hbuf.data(); a.ctl = ctl.data(); a.err_host = nullptr;
+  a.T = T; a.B = B; a.H = H; a.spin_limit = spin_limit;
+  const size_t n_out = (size_t)T * B * H, n_state = (size_t)L * B * H;
+  auto launch = [&](int skip) {
+    std::fill(out, out + n_out, 0.5f);
+    std::fill(state_h, state_h + n_state, 0.5f);
+    std::fill(state_c, state_c + n_state, 0.5f);
+    std::vector<std::thread> th;
+    for (int u = 0; u < H; ++u) th.emplace_back(workgroup, std::cref(a), L, u, H, skip);
+    for (auto& t : th) t.join();
+  };
+  // every element NaN, except (when given) those of hidden unit `but`
+  auto poisoned = [&](int but) {
+    auto all_nan = [&](const float* p, size_t n) {
+      for (size_t i = 0; i < n; ++i)
+        if (!std::isnan(p[i]) && (int)(i % (size_t)H) != but) return false;
+      return true;
+    };
+    return all_nan(out, n_out) && all_nan(state_h, n_state) && all_nan(state_c, n_state);
+  };
+  int bits = 0;
+  launch(skip_wg);
+  if (ctl[FX_LSTM_W_ERR] != 0u) bits |= 1;
+  if (poisoned(skip_wg)) bits |= 2;
+  launch(-1);
+  if (ctl[FX_LSTM_W_ERR] != 0u) bits |= 4;
+  if (poisoned(-1)) bits |= 8;
+  std::fill(ctl.begin(), ctl.end(), 0u);
+  std::fill(hbuf.begin(), hbuf.end(), 0ull);
+  launch(-1);
+  if (ctl[FX_LSTM_W_ERR] == 0u) bits |= 16;
+  return bits;
 }

@@ -128,3 +128,45 @@ def test_integer_constants_and_scalars_outside_32_bits_are_refused():
     with pytest.raises(FxError) as e:
         emul.run(r, torch.arange(4, dtype=torch.int32), BIG)
     assert e.value.code == C["FX_E_LIMIT"]
+
+
+def test_the_error_word_is_a_set_of_bits_and_a_caller_takes_only_its_own():
+    """fx_async_error_take clears the bits its caller handles and leaves the others to whoever
+    handles those; fx_async_error(1) clears everything."""
+    from functs_amd._lib import C
+    lib.fx_async_error(1)
+    lib.fx_async_error_report(C["FX_ASYNC_BARRIER"] | C["FX_ASYNC_NMS_CAPACITY"])
+    assert lib.fx_async_error_take(C["FX_ASYNC_NMS_CAPACITY"]) == C["FX_ASYNC_NMS_CAPACITY"]
+    assert lib.fx_async_error_take(C["FX_ASYNC_NMS_CAPACITY"]) == 0
+    assert lib.fx_async_error(0) == C["FX_ASYNC_BARRIER"]
+    assert lib.fx_async_error(1) == C["FX_ASYNC_BARRIER"] and lib.fx_async_error(0) == 0
+    assert len({C["FX_ASYNC_INT64"], C["FX_ASYNC_BARRIER"], C["FX_ASYNC_NMS_CAPACITY"]}) == 3
+    assert C["FX_ASYNC_INT64"] & C["FX_ASYNC_BARRIER"] == 0 and (C["FX_ASYNC_INT64"] | C["FX_ASYNC_BARRIER"]) & C["FX_ASYNC_NMS_CAPACITY"] == 0
+
+
+@pytest.mark.gpu
+def test_the_operator_raises_on_every_kind_of_report_and_works_again_after_it():
+    """Whatever an earlier launch reported (a given-up wait of fx::lstm_stack, an NMS overflow, an
+    int64 element outside 32 bits), the next fused-region call raises it; the word is cleared by
+    that, so the call after it runs."""
+    import functs_amd.jit as fj
+    from functs_amd._lib import C
+    from torch import Tensor
+
+    def f(a: Tensor):
+        b = a.clone()
+        b[0] = b[1] * 2.0
+        return b.sigmoid()
+
+    x = torch.rand(64, 8)
+    fn = fj.build(fj.script(f), [x])
+    xg = x.cuda()
+    ref = fn(xg).cpu()
+    for bits, word in ((C["FX_ASYNC_BARRIER"], "lstm_stack"), (C["FX_ASYNC_NMS_CAPACITY"], "candidates"), (C["FX_ASYNC_INT64"], "int64"),
+                       (C["FX_ASYNC_BARRIER"] | C["FX_ASYNC_INT64"], "lstm_stack")):
+        lib.fx_async_error(1)
+        lib.fx_async_error_report(bits)
+        with pytest.raises(RuntimeError, match=word):
+            fn(xg)
+        assert lib.fx_async_error(0) == 0
+        assert torch.equal(fn(xg).cpu(), ref)

@@ -122,6 +122,27 @@ def test_a_wait_that_cannot_end_is_given_up():
     assert err == 1
 
 
+def test_after_a_given_up_wait_the_workspace_refuses_work_until_it_is_cleared():
+    """The launch that gives up fills its results with NaN; the next launch on the same workspace
+    (whatever the host did with the error report in between) does no step, reports the error
+    again and returns NaN; on a cleared workspace the sequence runs."""
+    from tests.support import emul
+    so = emul.lstm_emul()
+    args = _inputs(4, 6, 32, 2, 1)
+    x = args[0]
+    T, B, H = x.shape
+    L = args[1].size(0)
+    out, sh, sc = torch.zeros(T, B, H), torch.zeros(L, B, H), torch.zeros(L, B, H)
+    ts = [t.contiguous() for t in args]
+    bits = so.fx_lstm_emul_give_up(*[t.data_ptr() for t in ts], out.data_ptr(), sh.data_ptr(), sc.data_ptr(),
+                                   T, B, H, L, 2000, 5)
+    assert bits & 1, "the first launch did not give up"
+    assert bits & 2, "the launch that gave up left values that look like results"
+    assert bits & 4 and bits & 8, "the launch on the workspace of a given-up wait ran"
+    assert bits & 16, "the launch on the cleared workspace failed"
+    _close((out, sh, sc), _reference(*args), "launch on the cleared workspace")
+
+
 def _gpu(x, wih, whh, bih, bhh, h0, c0, launches=1):
     """`launches` calls in a row on one workspace that is cleared once; the last call's results."""
     from functs_amd._lib import check, lib

@@ -150,3 +150,25 @@ def test_other_shapes_get_a_graph_of_their_own():
         assert [tuple(t.shape) for t in got] == [tuple(t.shape) for t in ref], g
         torch.testing.assert_close(got[2].cpu(), ref[2], rtol=1e-5, atol=1e-7)
     assert len(built._variants) == 3
+
+
+def test_a_constant_of_negative_zeros_keeps_its_sign():
+    """A uniform constant tensor becomes a fill inside its region; -0.0 == 0.0, but a fill with
+    zeros would lose the sign (1 / x, copysign and bitwise comparisons tell them apart)."""
+    def f(x: Tensor):
+        # (the literal -0.0 reaches the graph as +0.0: the sign is made by arithmetic)
+        return x + torch.full([32], 0.0).neg(), x + torch.tensor([1.0, -1.0] * 16) * 0.0
+
+    g = torch.jit.script(f).graph.copy()
+    torch._C._jit_pass_constant_propagation(g)
+    assert "aten::full" not in _kinds(g) and "aten::neg" not in _kinds(g)    # both are tensor constants now
+    assert _C._jit_pass_uniform_constants_to_fills(g)
+    kinds = _kinds(g)
+    assert "aten::zeros" not in kinds and kinds.count("aten::full") == 1   # the mixed one stays a constant
+    value = list([n for n in g.nodes() if n.kind() == "aten::full"][0].inputs())[1].toIValue()
+    import math
+    assert value == 0.0 and math.copysign(1.0, value) == -1.0
+    fn = torch._C._create_function_from_graph("f", g)
+    x = torch.full([32], -0.0)
+    a, _ = fn(x)
+    assert bool(torch.signbit(a).all())

@@ -324,7 +324,15 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0):
             ring.append(fn(*sets[i % n_sets]))
             torch.cuda.synchronize()
         cold_sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
-    return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us, cold_us, cold_sync_us
+    # host time of the operator by section (mean microseconds per operator call), warm calls
+    from functs_amd import _C
+    _C._functor_host_timing(True)
+    for _ in range(steps):
+        fn(*args)
+    torch.cuda.synchronize()
+    host = {k: round(v, 2) for k, v in _C._functor_host_times().items()}
+    _C._functor_host_timing(False)
+    return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us, cold_us, cold_sync_us, host
 
 
 def set_kernels(rowstream, head):
@@ -502,8 +510,9 @@ def main():
             _, ikern, _ = measure(w, max(args.steps // 4, 5), 3)
             aot.enable(True)
             rec["interpreter_kernel_us"] = [round(k * 1e3, 2) for k in ikern]
-        ts_us, n_functors, spec_share, sync_us, cold_us, cold_sync_us = torchscript_route(
+        ts_us, n_functors, spec_share, sync_us, cold_us, cold_sync_us, host = torchscript_route(
             name, w.cpu_args, dev, args.steps, args.warmup, COLD_BYTES)
+        rec["torchscript_route_host_us"] = host
         rec["torchscript_route_latency_us"] = round(cold_us, 2)
         rec["torchscript_route_drained_latency_us"] = round(cold_sync_us, 2)
         rec["torchscript_route_latency_us_warm"] = round(ts_us, 2)
@@ -531,7 +540,7 @@ def main():
         from functs_amd.benchmark import PROGRAMS
         cpu_args = INPUTS["c4"](0)
         n_rep = max(args.steps // 10, 5)
-        us, n_functors, spec_share, sync_us, cold_us, cold_sync_us = torchscript_route("c4", cpu_args, dev, n_rep, 2, COLD_BYTES)
+        us, n_functors, spec_share, sync_us, cold_us, cold_sync_us, _ = torchscript_route("c4", cpu_args, dev, n_rep, 2, COLD_BYTES)
         fn = fj.build(fj.script(PROGRAMS["c4"]), list(cpu_args))
         gargs = [a.to(dev) for a in cpu_args]
         fn(*gargs)
@@ -614,12 +623,21 @@ def main():
             res = detection.multiclass_nms_batched(bc.batched(0), bc.batched(1), bc.batched(2), counts=bc.totals)
         e1.record()
         torch.cuda.synchronize()
+        # the same through the TorchScript route: the scripted loop with functs::multiclass_nms in it
+        # (functs_amd/benchmark/programs.py yolov3_batched_nms), which the pipeline turns into the
+        # functor with padded outputs, ONE batched tail launch and one wait at the end
+        ts_args = INPUTS["c5_nms"](0)
+        ts_us, ts_functors, _, ts_sync_us, ts_cold_us, ts_cold_sync_us, ts_host = torchscript_route(
+            "c5_nms", ts_args, dev, n, max(args.warmup // 4, 3), COLD_BYTES)
         kept = [int(k) for k in res.n.cpu()]
         rows = bc.totals.tolist()
         cand = [int((bc.batched(1)[t, :rows[t]] > 0.05).sum()) for t in range(16)]
         read = sum(r * (80 + 4 + 1) * 4 for r in rows)
         return {"workload": "c5 compaction + multiclass NMS tail, 16 images (class logits shifted by -6)",
                 "latency_us": round(us, 1), "launches_per_call": bc.plan.launches + 1,
+                "torchscript_route_latency_us": round(ts_cold_us, 1), "torchscript_route_drained_latency_us": round(ts_cold_sync_us, 1),
+                "torchscript_route_latency_us_warm": round(ts_us, 1), "torchscript_route_drained_latency_us_warm": round(ts_sync_us, 1),
+                "torchscript_route_functors": ts_functors, "torchscript_route_host_us": ts_host,
                 "nms_kernel_us": round(e0.elapsed_time(e1) * 1e3 / n, 1),
                 "kept_rows_per_image": [min(rows), max(rows)], "candidates_per_image": [min(cand), max(cand)],
                 "detections_per_image": [min(kept), max(kept)],

@@ -44,6 +44,8 @@ class FxNmsDesc(ctypes.Structure):
         ("boxes_task_stride", ctypes.c_int64),
         ("scores", ctypes.c_void_p),
         ("scores_task_stride", ctypes.c_int64),
+        ("scores_row_stride", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
         ("factors", ctypes.c_void_p),
         ("factors_task_stride", ctypes.c_int64),
         ("labels", ctypes.c_void_p),

@@ -52,6 +52,15 @@ def yolov3_batched(seed: int = 0, grids=YOLO_GRIDS, batch: int = 16):
     return yolov3_postproc(seed, grids, batch)
 
 
+def yolov3_batched_nms(seed: int = 0, grids=YOLO_GRIDS, batch: int = 16, shift: float = 6.0):
+    """The inputs of yolov3_batched with the class logits lowered by `shift`, so that about 1e-3 of
+    the class scores pass the tail's 0.05, as behind a trained head (with N(0, 1) logits nearly all
+    (row, class) pairs of an image would be candidates of the NMS)."""
+    preds, anchors, strides = yolov3_postproc(seed, grids, batch)
+    preds[..., 5:] -= shift
+    return preds, anchors, strides
+
+
 def ssd_postproc(seed: int = 0, n_priors: int = 8732, n_cls: int = 81):
     g = _gen(seed)
     loc = 0.5 * torch.randn(1, n_priors, 4, generator=g)
@@ -86,6 +95,15 @@ def yolov3_head(seed: int = 0, batch: int = 16, grids=YOLO_GRIDS, classes: int =
     return maps, bases
 
 
+def yolov3_head_nms(seed: int = 0, batch: int = 16, grids=YOLO_GRIDS, classes: int = 80, shift: float = 6.0):
+    """The inputs of yolov3_head with the class logits of every anchor lowered by `shift` (see
+    yolov3_batched_nms)."""
+    maps, bases = yolov3_head(seed, batch, grids, classes)
+    for m in maps:
+        m.view(batch, 3, 5 + classes, m.size(2), m.size(3))[:, :, 5:] -= shift
+    return maps, bases
+
+
 def attention_steps(seed: int = 0, batch: int = 1, heads: int = 12, length: int = 50, depth: int = 64, start: int = 32):
     g = _gen(seed)
     x = torch.randn(batch, heads, 1, depth, generator=g)
@@ -112,7 +130,9 @@ INPUTS = {
     "c3": ssd_postproc,
     "c4": lstm,
     "c5": yolov3_batched,
+    "c5_nms": yolov3_batched_nms,
     "yolo_head": yolov3_head,
+    "yolo_head_nms": yolov3_head_nms,
     "attention": attention_steps,
     "delta2bbox": delta2bbox,
 }

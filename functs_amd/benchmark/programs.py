@@ -4,14 +4,16 @@ benchmark models.  They are inputs to functs_amd.jit.script / build.
   get_started      examples/get_started.py:10-15
   yolov3_postproc  functs/benchmark/ai_model/yolov3/yolov3_bbox.py:12-23, 206-243
   yolov3_batched   the per-image loop of yolov3_bbox.py:233-241
+  yolov3_batched_nms  the same loop with its tail, multiclass_nms (yolov3_bbox.py:104-138, 233-243)
   ssd_postproc     functs/benchmark/ai_model/ssd/ssd_bbox.py:121-154, 163-172, 268
   lstm             functs/benchmark/ai_model/lstm/lstm.py:79-133
   yolov3_head      the whole detection head up to the NMS as the reference's model structures it,
                    functs/benchmark/ai_model/yolov3/yolov3_bbox.py:12-23, 78-101, 194-243
+  yolov3_head_nms  the same with the NMS tail of yolov3_bbox.py:104-179 behind the per-image filter
   attention_steps  functs/benchmark/simpleops/attention/attention.py:38-58
   delta2bbox       functs/benchmark/ai_model/ssd/ssd_bbox.py:121-154
 """
-from typing import List
+from typing import List, Tuple
 
 import torch
 from torch import Tensor
@@ -54,6 +56,17 @@ def yolov3_batched(preds: Tensor, anchors: Tensor, strides: Tensor):
         out_c.append(c)
         out_o.append(o)
     return out_b, out_c, out_o
+
+
+def yolov3_batched_nms(preds: Tensor, anchors: Tensor, strides: Tensor):
+    """The per-image loop of the reference's forward with its tail (yolov3_bbox.py:233-243): decode,
+    confidence filter, then multiclass_nms (:104-138) on the kept rows.  functs::multiclass_nms is
+    the operator that stands where the reference calls its Python function of that name."""
+    det_results: List[Tuple[Tensor, Tensor]] = []
+    for i in range(preds.size(0)):
+        b, c, o = yolov3_postproc(preds[i:i + 1], anchors, strides)
+        det_results.append(torch.ops.functs.multiclass_nms(b, c, o, 0.05, 0.45, 100, False))
+    return det_results
 
 
 def ssd_postproc(loc: Tensor, conf: Tensor, priors: Tensor):
@@ -123,13 +136,11 @@ def _decode_stack(anchors: Tensor, pred: Tensor, stride: Tensor):
     return boxes.clone()
 
 
-def yolov3_head(pred_maps: List[Tensor], base_anchors: List[Tensor]):
-    """The detection head as the reference's model structures it (yolov3_bbox.py:194-243), up to the
-    NMS: per level the NCHW map is permuted, flattened and its centre offsets squashed in place,
-    the levels are concatenated, anchors and strides are generated from the feature-map sizes, the
-    boxes are decoded for the whole batch, the class scores get a zero column, and a loop over the
-    images keeps the rows whose objectness passes the confidence threshold.
-    pred_maps: per level [B, A * (5 + C), H, W]; base_anchors: per level [A, 4]."""
+def _yolov3_head_scores(pred_maps: List[Tensor], base_anchors: List[Tensor]):
+    """yolov3_bbox.py:194-238: per level the NCHW map is permuted, flattened and its centre offsets
+    squashed in place, the levels are concatenated, anchors and strides are generated from the
+    feature-map sizes, the boxes are decoded for the whole batch and the class scores get a zero
+    column.  Returns boxes [B, N, 4], class scores [B, N, C + 1], objectness [B, N]."""
     featmap_strides = [32, 16, 8]
     num_imgs = pred_maps[0].size(0)
     num_attrib = pred_maps[0].size(1) // base_anchors[0].size(0)
@@ -153,16 +164,38 @@ def yolov3_head(pred_maps: List[Tensor], base_anchors: List[Tensor]):
     bboxes = _decode_stack(anchors, bbox_preds, strides.unsqueeze(-1))
     padding = bboxes.new_zeros(num_imgs, bboxes.size(1), 1)
     cls_scores = torch.cat([cls_scores, padding], dim=-1)
+    return bboxes, cls_scores, objectness
+
+
+def yolov3_head(pred_maps: List[Tensor], base_anchors: List[Tensor]):
+    """The detection head as the reference's model structures it (yolov3_bbox.py:194-243), up to the
+    NMS: the scores of _yolov3_head_scores, then a loop over the images that keeps the rows whose
+    objectness passes the confidence threshold.
+    pred_maps: per level [B, A * (5 + C), H, W]; base_anchors: per level [A, 4]."""
+    bboxes, cls_scores, objectness = _yolov3_head_scores(pred_maps, base_anchors)
     out_b: List[Tensor] = []
     out_s: List[Tensor] = []
     out_o: List[Tensor] = []
-    for i in range(num_imgs):
+    for i in range(bboxes.size(0)):
         o = objectness[i]
         keep = o >= 0.005
         out_b.append(bboxes[i][keep, :])
         out_s.append(cls_scores[i][keep, :])
         out_o.append(o[keep])
     return out_b, out_s, out_o
+
+
+def yolov3_head_nms(pred_maps: List[Tensor], base_anchors: List[Tensor]):
+    """The whole of the reference's forward (yolov3_bbox.py:194-243): the head, and per image the
+    confidence filter followed by multiclass_nms (:104-138) on the kept rows, whose class scores
+    carry the padding column that multiclass_nms cuts off again (:113)."""
+    bboxes, cls_scores, objectness = _yolov3_head_scores(pred_maps, base_anchors)
+    det_results: List[Tuple[Tensor, Tensor]] = []
+    for i in range(bboxes.size(0)):
+        o = objectness[i]
+        keep = o >= 0.005
+        det_results.append(torch.ops.functs.multiclass_nms(bboxes[i][keep, :], cls_scores[i][keep, :], o[keep], 0.05, 0.45, 100, True))
+    return det_results
 
 
 def attention_steps(x: Tensor, k: Tensor, v: Tensor, wq: Tensor, wk: Tensor, wv: Tensor, wo: Tensor, start_len: int):
@@ -217,7 +250,9 @@ PROGRAMS = {
     "c3": ssd_postproc,
     "c4": lstm,
     "c5": yolov3_batched,
+    "c5_nms": yolov3_batched_nms,
     "yolo_head": yolov3_head,
+    "yolo_head_nms": yolov3_head_nms,
     "attention": attention_steps,
     "delta2bbox": delta2bbox,
 }

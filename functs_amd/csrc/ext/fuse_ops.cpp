@@ -5,6 +5,7 @@
 // per block, a group needs two "working" operators, non-tensor constants stay
 // outside, index-like operators only as group outputs) and
 // fait/passes/parallelize_loops.cpp:12-126.
+#include <iostream>
 #include <torch/csrc/jit/ir/constants.h>
 #include <torch/csrc/jit/passes/common_subexpression_elimination.h>
 #include <torch/csrc/jit/passes/constant_propagation.h>
@@ -195,9 +196,18 @@ Node* commitGroup(const std::vector<Node*>& nodes, Node* insertBefore) {
 
 bool worthFusing(const std::vector<Node*>& nodes) {
   size_t working = 0;
+  static const std::unordered_set<Symbol> comparisons{c10::aten::gt, c10::aten::ge, c10::aten::lt, c10::aten::le, c10::aten::eq, c10::aten::ne};
   for (Node* n : nodes) {
     if (n->kind() == sym::ForallSelectRev()) working += 2;
     else working += workingSymbols().count(n->kind());
+    // A comparison whose result is the mask of x[mask] selections behind the group: the group
+    // becomes a row compaction (FuseMaskedSelect), which outside a region is a nonzero with its
+    // host synchronisation plus a gather per selection.
+    if (comparisons.count(n->kind()) && isTensorValue(n->output()))
+      for (const Use& u : n->output()->uses())
+        if (u.user->kind() == c10::prim::ListConstruct && u.user->inputs().size() == 1)
+          for (const Use& lu : u.user->output()->uses())
+            if (isIndexLike(lu.user) && lu.offset == 1) working += 1;
   }
   if (working < 2) return false;
   // a region takes its device from its tensor arguments: fills over constant shapes alone stay eager
@@ -1041,6 +1051,11 @@ struct RefinedTypesScope {
 bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_types) {
   RefinedTypesScope scope;
   bool specialized = false;
+  // FUNCTS_PIPELINE_TRACE=1: the graph after the region-forming stages, on stderr
+  static const bool tracing = getenv("FUNCTS_PIPELINE_TRACE") && atoi(getenv("FUNCTS_PIPELINE_TRACE")) != 0;
+  auto trace = [&](const char* stage) {
+    if (tracing) std::cerr << "---- after " << stage << " ----\n" << graph->toString(false) << std::endl;
+  };
   // RefineInputTypes (refine_types.cpp:179-195): tensor arguments take the example's type; a list
   // argument whose example is a tuple of tensors keeps the tuple type in the side table
   for (size_t i = 0; i < input_types.size() && i < graph->inputs().size(); ++i) {
@@ -1092,8 +1107,11 @@ bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
   EliminateCommonSubexpression(graph);
   if (CollapseRecurrentLoops(graph)) EliminateDeadCode(graph);   // buffers the collapsed node no longer reads
   CollapseAssignLoops(graph);
+  trace("canonicalisation");
   ParallelizeLoops(graph);
+  trace("ParallelizeLoops");
   FuseOps(graph);
+  trace("FuseOps");
   // what did not fuse inside short dependent loops and parameter-only maps is written out and
   // gets a second chance across iterations (fait_pipeline.cpp:52-55)
   const bool unrolled_loops = UnrollLoopsWithDeps(graph);
@@ -1106,10 +1124,13 @@ bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
     FuseOps(graph);
   }
   FuseMaskedSelect(graph);
+  trace("FuseMaskedSelect");
   SplitParallelMaps(graph);
   CanonicalizeFusableMaps(graph);   // fait_pipeline.cpp:61
+  trace("SplitParallelMaps");
   ToParallelFunctor(graph);
   EliminateDeadCode(graph);
+  trace("ToParallelFunctor");
   InferStaticShapes(graph);   // results of the functors, and the argument types of the functors behind them
   if (SinkProducersIntoMaps(graph)) {   // (folds size queries on the producer's results)
     ConstantPropagation(graph);
@@ -1117,6 +1138,7 @@ bool FaitPipeline(std::shared_ptr<Graph> graph, std::vector<c10::TypePtr> input_
     EliminateDeadCode(graph);
     specialized = true;
   }
+  FuseDetectionTail(graph);
   Validate(graph);
   return specialized;
 }

@@ -88,6 +88,7 @@ PYBIND11_MODULE(_C, m) {
   m.def("_set_sink_producers", setSinkProducers);
   m.def("_plan_functors", PlanFunctors);
   m.def("_jit_pass_infer_static_shapes", InferStaticShapes);
+  m.def("_jit_pass_fuse_detection_tail", FuseDetectionTail);
   m.def("_functor_host_timing", functorHostTiming);
   m.def("_functor_host_times", []() {
     py::dict d;

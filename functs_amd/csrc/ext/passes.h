@@ -78,6 +78,16 @@ void ToParallelFunctor(std::shared_ptr<torch::jit::Graph> graph);
 bool SinkProducersIntoMaps(std::shared_ptr<torch::jit::Graph> graph);
 void setSinkProducers(bool on);
 
+// A per-image loop of functs::multiclass_nms(list_b[i], list_s[i], list_f[i], constants...) over
+// three result lists of one compacting map functor becomes
+//   functor[padded_outputs=1] -> functs::multiclass_nms_batched -> functs::unbatch_detections
+// (detection_ops.cpp): the functor returns its outputs at full size and the kept-row counts as a
+// tensor without waiting for them, the tail of all images is one launch behind it on the stream,
+// and the only wait is the one that cuts the final results to size.  The reference runs the tail
+// per image, as ATen and torchvision kernels with host synchronisations in between
+// (yolov3_bbox.py:104-179, 233-243).  True if the graph changed.
+bool FuseDetectionTail(std::shared_ptr<torch::jit::Graph> graph);
+
 // Static types of intermediate values (the reference's InferShape, fait/passes/refine_types.cpp:
 // 420-685, run at fait_pipeline.cpp:47): every operator node whose tensor arguments have complete
 // static types and whose other arguments are constants is run on meta tensors of those types, and

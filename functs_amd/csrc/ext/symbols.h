@@ -55,6 +55,9 @@ FUNCTS_SYM(is_parallel_args, "attr::is_parallel_args")
 FUNCTS_SYM(input_refine_types, "attr::input_refine_types")
 FUNCTS_SYM(is_parallel_map, "attr::is_parallel_map")
 FUNCTS_SYM(compact_rows, "attr::compact_rows")
+// a compacting functor that returns every output at its full size (one tensor [tasks, rows, ...])
+// and the kept-row counts as one more tensor, without waiting for them (detection_ops.cpp)
+FUNCTS_SYM(padded_outputs, "attr::padded_outputs")
 #undef FUNCTS_SYM
 }  // namespace sym
 

@@ -14,6 +14,7 @@
 // pops the arguments, pushes one IValue per output; outputs are freshly
 // allocated, inputs are never written.
 #include <ATen/ATen.h>
+#include <ATen/core/CachingHostAllocator.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/DeviceGuard.h>
 #include <torch/csrc/jit/ir/constants.h>
@@ -422,7 +423,9 @@ class RegionRunner {
         is_par_(node->is(sym::is_parallel_args())),
         degree_(node->i(sym::parallel_degree())),
         is_map_(node->i(sym::is_parallel_map()) != 0),
-        compact_(node->hasAttribute(sym::compact_rows()) && node->i(sym::compact_rows()) != 0) {
+        compact_(node->hasAttribute(sym::compact_rows()) && node->i(sym::compact_rows()) != 0),
+        padded_(node->hasAttribute(sym::padded_outputs()) && node->i(sym::padded_outputs()) != 0) {
+    TORCH_CHECK(!padded_ || compact_, "ParallelFunctor: padded_outputs is an attribute of compacting functors");
     n_args_ = graph_->inputs().size() - 1;
     TORCH_CHECK(is_par_.size() == n_args_, "ParallelFunctor: is_parallel_args does not match the subgraph");
     n_stack_ = n_args_ + (degree_ < 0 ? 1 : 0);
@@ -440,6 +443,7 @@ class RegionRunner {
     if (!is_map_) degree = 1;
     TORCH_CHECK(degree >= 0, "ParallelFunctor: negative trip count");
     if (degree == 0) {  // an empty map
+      TORCH_CHECK(!padded_, "ParallelFunctor: a map with padded outputs needs at least one task");
       drop(stack, n_stack_);
       for (size_t o = 0; o < n_outs_; ++o) push(stack, c10::List<at::Tensor>());
       return;
@@ -541,6 +545,49 @@ class RegionRunner {
     }
     checkAsyncError();
     clock.tick(HS_ALLOC);
+    if (padded_) {
+      // Every output at its full size, the kept-row counts as a tensor of their own (pinned host
+      // memory that the kernels write and the next kernel on the stream reads): nobody waits.
+      at::Tensor counts = at::empty({degree}, at::TensorOptions().dtype(at::kInt).pinned_memory(true));
+      FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(), ws.scratch.data_ptr(),
+                                   (uint32_t*)counts.data_ptr(), (void*)stream.stream()));
+      // the block is not handed out again before the launch has written it
+      at::getHostAllocator(at::kCUDA)->record_event(counts.data_ptr(), counts.storage().data_ptr().get_context(), stream.unwrap());
+      clock.tick(HS_LAUNCH);
+      var->give(std::move(ws));
+      drop(stack, n_stack_);
+      for (int o = 0; o < n_out; ++o) {
+        if (degree == 1) {
+          push(stack, is_map_ ? buffers[o].unsqueeze(0) : std::move(buffers[o]));
+          continue;
+        }
+        const Slot& first_slot = slot_of[(size_t)o * degree];
+        const int64_t task_stride = slot_of[(size_t)o * degree + 1].offset_elems - first_slot.offset_elems;
+        std::vector<int64_t> sizes{degree}, strides{task_stride};
+        int64_t inner = 1;
+        for (int d = 0; d < first_slot.rank; ++d) inner *= first_slot.sizes[d];
+        for (int d = 0; d < first_slot.rank; ++d) {
+          sizes.push_back(first_slot.sizes[d]);
+          inner /= std::max<int64_t>(first_slot.sizes[d], 1);
+          strides.push_back(first_slot.sizes[d] == 0 ? 1 : inner);
+        }
+        for (int64_t t = 1; t < degree; ++t) {
+          const Slot& sl = slot_of[(size_t)o * degree + t];
+          TORCH_CHECK(sl.rank == first_slot.rank && std::equal(sl.sizes, sl.sizes + sl.rank, first_slot.sizes) &&
+                          sl.offset_elems == first_slot.offset_elems + t * task_stride,
+                      "ParallelFunctor: padded outputs need tasks of one size");
+        }
+        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(block.storage()), block.key_set(),
+                                                         c10::scalarTypeToTypeMeta(atDtype(layout->dtype[o])));
+        impl->set_storage_offset(layout->base[o] / layout->item[o] + first_slot.offset_elems);
+        impl->set_sizes_and_strides(sizes, strides);
+        push(stack, at::Tensor(std::move(impl)));
+      }
+      push(stack, std::move(counts));
+      clock.tick(HS_PUSH);
+      if (clock.on) g_host_calls.fetch_add(1, std::memory_order_relaxed);
+      return;
+    }
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
@@ -636,7 +683,7 @@ class RegionRunner {
   std::shared_ptr<Graph> graph_;
   std::vector<int64_t> is_par_;
   int64_t degree_;
-  bool is_map_, compact_;
+  bool is_map_, compact_, padded_;
   size_t n_args_ = 0, n_stack_ = 0, n_outs_ = 0;
   std::mutex mu_;
   std::map<std::string, std::unique_ptr<Variant>> variants_;

@@ -1416,7 +1416,10 @@ int fx_sort_nms(const fx_nms_desc* desc, void* stream_) {
   if (d.max_num < 1 || d.max_num > FX_NMS_MAX_OUT)
     return fail(FX_E_LIMIT, "fx_sort_nms: max_num must be 1.." + std::to_string(FX_NMS_MAX_OUT));
   if (d.mode == 1 && d.n_classes < 1) return fail(FX_E_INVALID, "fx_sort_nms: n_classes must be positive in mode 1");
-  const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? d.n_classes : 1u);
+  if (d.mode == 0) d.scores_row_stride = 0;
+  if (d.scores_row_stride != 0 && d.scores_row_stride < d.n_classes)
+    return fail(FX_E_INVALID, "fx_sort_nms: scores_row_stride must be 0 or at least n_classes");
+  const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? std::max(d.n_classes, d.scores_row_stride) : 1u);
   if (items >= (1ull << 31)) return fail(FX_E_LIMIT, "fx_sort_nms: rows * classes beyond 31 bits");
   if (d.key_capacity < 1 || d.key_capacity > FX_NMS_MAX_CANDIDATES)
     return fail(FX_E_LIMIT, "fx_sort_nms: key_capacity must be 1.." + std::to_string(FX_NMS_MAX_CANDIDATES) +

@@ -92,7 +92,9 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   const uint32_t task = blockIdx.x / slices, slice = blockIdx.x - task * slices;
   uint32_t* const ctr = ws + (size_t)task * FX_NMS_WS_WORDS;   // [0] candidates, [1] finished slices, [2] largest coordinate
   uint64_t* const g_keys = (uint64_t*)(ws + (size_t)d.n_tasks * FX_NMS_WS_WORDS) + (size_t)task * key_cap;
-  const uint32_t C = d.mode == 1 ? d.n_classes : 1u;
+  // NC classes, in rows of C elements (C > NC: columns behind the class scores that are not candidates)
+  const uint32_t NC = d.mode == 1 ? d.n_classes : 1u;
+  const uint32_t C = (d.mode == 1 && d.scores_row_stride != 0u) ? d.scores_row_stride : NC;
   const float* boxes = d.boxes + (int64_t)task * d.boxes_task_stride;
   const float* scores = d.scores + (int64_t)task * d.scores_task_stride;
   const float* factors = d.factors ? d.factors + (int64_t)task * d.factors_task_stride : nullptr;
@@ -158,6 +160,14 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     // few elements pass a detector's threshold: a lane that has some takes its places with one LDS
     // atomic (the order of arrival does not matter), the others go straight on to the next loads
     if (mine == 0u) continue;
+    if (C != NC) {   // columns behind the class scores are no candidates
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u)
+#pragma unroll
+        for (uint32_t e = 0; e < 4u; ++e)
+          if (((mine >> (u * 4u + e)) & 1u) && (base + (u * FX_NMS_THREADS + tid) * 4u + e) % C >= NC) mine &= ~(1u << (u * 4u + e));
+      if (mine == 0u) continue;
+    }
     uint32_t slot = atomicAdd(&s_count, (uint32_t)__popc(mine));
 #pragma unroll
     for (uint32_t u = 0; u < U; ++u)
@@ -207,7 +217,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
   }
   if (count > key_cap) {   // more candidates than the launch was sized for: reported, nothing returned
     if (tid == 0) {
-      d.n_out[task] = FX_NMS_OVERFLOW;
+      __hip_atomic_store(d.n_out + task, FX_NMS_OVERFLOW, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       if (err_host) __hip_atomic_store(err_host, (uint32_t)FX_ASYNC_NMS_CAPACITY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     for (uint32_t k = tid; k < d.max_num * 5u; k += FX_NMS_THREADS) dets[k] = 0.0f;
@@ -308,7 +318,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
         s_cbox[tid][0] = b.x; s_cbox[tid][1] = b.y; s_cbox[tid][2] = b.z; s_cbox[tid][3] = b.w;
         s_obox[tid][0] = x1; s_obox[tid][1] = y1; s_obox[tid][2] = x2; s_obox[tid][3] = y2;
         s_carea[tid] = (x2 - x1) * (y2 - y1);
-        s_cidx[tid] = idx;
+        s_cidx[tid] = d.mode == 1 ? r * NC + label : idx;   // position among the candidates proper
         s_clabel[tid] = label;
         s_cscore[tid] = from_orderable(~(uint32_t)(key >> 32));
       }
@@ -392,7 +402,8 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
     out_labels[k] = 0;
     if (out_index) out_index[k] = 0;
   }
-  if (tid == 0) d.n_out[task] = nk;
+  // (system scope: a count in pinned host memory goes through to the host, which may be polling it)
+  if (tid == 0) __hip_atomic_store(d.n_out + task, nk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 }  // namespace
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(FX_NMS_THREADS) void fx_sort_nms_kernel(const fx_nm
 // a time: with two per CU the second half of the launch starts when the first ends, 16 us into
 // the kernel for 16 images), none with less than one round of loads
 uint32_t fx_nms_slices(const fx_nms_desc& d) {
-  const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? d.n_classes : 1u);
+  const uint64_t items = (uint64_t)d.rows * (d.mode == 1 ? std::max(d.n_classes, d.scores_row_stride) : 1u);
   const uint64_t per_round = (uint64_t)FX_NMS_THREADS * 16u;
   uint64_t s = (items + per_round - 1) / per_round;
   static int cus = 0;

@@ -418,7 +418,7 @@ void fx_set_lstm_spin_limit(uint32_t polls); /* barrier polls before a wait is g
  * The step behind row compaction in the reference's detection programs, which it runs as ATen /
  * torchvision kernels with host synchronisations in between:
  *   mode 1  multiclass_nms (functs/benchmark/ai_model/yolov3/yolov3_bbox.py:104-138 with batched_nms
- *           :141-171 and nms_wrapper :174-179): scores is cls [rows, n_classes], a candidate
+ *           :141-171 and nms_wrapper :174-179): scores is cls [rows, n_classes] (rows scores_row_stride apart), a candidate
  *           (row, class) needs cls > score_thr, its score is cls * factors[row], its label the class;
  *   mode 0  batched_nms alone (ssd_bbox.py:175-214): scores [rows], labels [rows] (null: one class),
  *           a candidate needs score > score_thr (pass -INFINITY to take every row).
@@ -448,6 +448,10 @@ typedef struct fx_nms_desc {
   int64_t boxes_task_stride;
   const float* scores;
   int64_t scores_task_stride;
+  uint32_t scores_row_stride; /* mode 1: elements from one row of scores to the next; 0: n_classes.  Larger: the row
+                                 carries columns behind its class scores (the reference's padding column,
+                                 yolov3_bbox.py:237-238, which multiclass_nms cuts off again, :113) that are not candidates */
+  uint32_t reserved0;
   const float* factors; /* mode 1, [rows] per task; null: 1 */
   int64_t factors_task_stride;
   const int64_t* labels; /* mode 0, [rows] per task; null: one class */

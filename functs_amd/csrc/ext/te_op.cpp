@@ -380,6 +380,39 @@ struct Variant {
   fx_region* region = nullptr;
   std::mutex mu;
   std::vector<Workspace> pool;
+  // the output block of the next call of a map, allocated while the last call's kernels ran
+  at::Tensor next_block;
+  void* next_stream = nullptr;
+  // likewise the output tensors of the next call of a single task (one per output, at full size)
+  std::vector<at::Tensor> next_buffers;
+  const fx_plan* next_buffers_plan = nullptr;
+  void* next_buffers_stream = nullptr;
+  std::vector<at::Tensor> takeBuffers(const fx_plan* plan, void* stream) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (next_buffers_plan != plan || next_buffers_stream != stream) return {};
+    next_buffers_plan = nullptr;
+    return std::move(next_buffers);
+  }
+  void prepareBuffers(const fx_plan* plan, void* stream, std::vector<at::Tensor> buffers) {
+    std::lock_guard<std::mutex> lock(mu);
+    next_buffers = std::move(buffers);
+    next_buffers_plan = plan;
+    next_buffers_stream = stream;
+  }
+  at::Tensor takeBlock(int64_t bytes, c10::Device device, void* stream) {
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      if (next_block.defined() && next_block.numel() == bytes && next_block.device() == device && next_stream == stream)
+        return std::move(next_block);
+    }
+    return at::empty({bytes}, at::TensorOptions().dtype(at::kByte).device(device));
+  }
+  void prepareBlock(int64_t bytes, c10::Device device, void* stream) {
+    at::Tensor b = at::empty({bytes}, at::TensorOptions().dtype(at::kByte).device(device));   // on the current stream
+    std::lock_guard<std::mutex> lock(mu);
+    next_block = std::move(b);
+    next_stream = stream;
+  }
   std::unordered_map<const fx_plan*, std::shared_ptr<const OutLayout>> layouts;   // plans live as long as the region
   ~Variant() {
     if (region) fx_region_destroy(region);
@@ -521,15 +554,21 @@ class RegionRunner {
     std::vector<at::Tensor> buffers(n_out);
     at::Tensor block;
     std::vector<void*> ptrs((size_t)n_out * degree);
-    if (degree > 1)
-      block = at::empty({std::max<int64_t>(layout->block_bytes, 1)}, at::TensorOptions().dtype(at::kByte).device(device));
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
+    if (degree > 1) block = var->takeBlock(std::max<int64_t>(layout->block_bytes, 1), device, (void*)stream.stream());
+    if (degree == 1) {
+      std::vector<at::Tensor> prepared = var->takeBuffers(plan, (void*)stream.stream());
+      if ((int)prepared.size() == n_out) buffers = std::move(prepared);
+    }
+    auto newBuffer = [&](int o) {
+      const Slot& sl = layout->slots[(size_t)o * degree];   // (at full size: the kept-row counts cut it later)
+      return at::empty(at::IntArrayRef(sl.sizes, sl.rank), at::TensorOptions().dtype(atDtype(layout->dtype[o])).device(device));
+    };
     for (int o = 0; o < n_out; ++o) {
-      const int32_t dt = layout->dtype[o];
       const int64_t item = layout->item[o];
       char* base;
       if (degree == 1) {
-        const Slot& sl = slot_of[(size_t)o * degree];
-        buffers[o] = at::empty(at::IntArrayRef(sl.sizes, sl.rank), at::TensorOptions().dtype(atDtype(dt)).device(device));
+        if (!buffers[o].defined()) buffers[o] = newBuffer(o);
         base = (char*)buffers[o].data_ptr();
       } else {
         base = (char*)block.data_ptr() + layout->base[o];
@@ -537,7 +576,6 @@ class RegionRunner {
       for (int64_t t = 0; t < degree; ++t)
         ptrs[(size_t)o * degree + t] = base + slot_of[(size_t)o * degree + t].offset_elems * item;
     }
-    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index());
     Workspace ws;
     if (compact_) {
       ws = var->take(fx_plan_scratch_bytes(plan), degree, device, (void*)stream.stream());
@@ -592,21 +630,27 @@ class RegionRunner {
                                  compact_ ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
     clock.tick(HS_LAUNCH);
-    std::vector<std::vector<at::Tensor>> outs(n_out);
-    for (int o = 0; o < n_out; ++o) {
-      if (degree == 1) {
-        outs[o].push_back(std::move(buffers[o]));
-        continue;
+    // The tasks' tensors: views of the block, made while the kernels run.
+    std::vector<at::Tensor> flat;   // [output][task]
+    if (degree > 1) {
+      flat.reserve((size_t)n_out * degree);
+      for (int o = 0; o < n_out; ++o) {
+        const int64_t first_elem = layout->base[o] / layout->item[o];
+        for (int64_t t = 0; t < degree; ++t) {
+          const Slot& sl = slot_of[(size_t)o * degree + t];
+          auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(block.storage()), block.key_set(),
+                                                           c10::scalarTypeToTypeMeta(atDtype(layout->dtype[o])));
+          impl->set_storage_offset(first_elem + sl.offset_elems);
+          impl->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
+          flat.emplace_back(std::move(impl));
+        }
       }
-      outs[o].reserve(degree);
-      for (int64_t t = 0; t < degree; ++t) {
-        const Slot& sl = slot_of[(size_t)o * degree + t];
-        auto impl = c10::make_intrusive<c10::TensorImpl>(c10::TensorImpl::VIEW, c10::Storage(block.storage()), block.key_set(),
-                                                         c10::scalarTypeToTypeMeta(atDtype(layout->dtype[o])));
-        impl->set_storage_offset(layout->base[o] / layout->item[o] + sl.offset_elems);
-        impl->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
-        outs[o].emplace_back(std::move(impl));
-      }
+      // the next call's block is allocated now, while this call's kernels run
+      var->prepareBlock(std::max<int64_t>(layout->block_bytes, 1), device, (void*)stream.stream());
+    } else {
+      std::vector<at::Tensor> next(n_out);
+      for (int o = 0; o < n_out; ++o) next[o] = newBuffer(o);
+      var->prepareBuffers(plan, (void*)stream.stream(), std::move(next));
     }
     clock.tick(HS_VIEWS);
     if (compact_) {
@@ -620,15 +664,24 @@ class RegionRunner {
         for (int64_t t = 0; t < degree; ++t) {
           Slot& sl = slots[(size_t)o * degree + t];
           sl.sizes[0] = tot[t];
-          outs[o][t].unsafeGetTensorImpl()->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
+          at::Tensor& out = degree == 1 ? buffers[o] : flat[(size_t)o * degree + t];
+          out.unsafeGetTensorImpl()->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
         }
       var->give(std::move(ws));
     }
     clock.tick(HS_RESIZE);
     drop(stack, n_stack_);
     for (int o = 0; o < n_out; ++o) {
-      if (is_map_) push(stack, c10::List<at::Tensor>(std::move(outs[o])));
-      else push(stack, std::move(outs[o][0]));
+      if (!is_map_) {
+        push(stack, std::move(buffers[o]));
+        continue;
+      }
+      c10::List<at::Tensor> list;
+      list.reserve(degree);
+      if (degree == 1) list.push_back(std::move(buffers[o]));
+      else
+        for (int64_t t = 0; t < degree; ++t) list.push_back(std::move(flat[(size_t)o * degree + t]));
+      push(stack, std::move(list));
     }
     clock.tick(HS_PUSH);
     if (clock.on) g_host_calls.fetch_add(1, std::memory_order_relaxed);

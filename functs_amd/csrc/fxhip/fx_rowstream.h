@@ -198,6 +198,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
 #pragma unroll
     for (uint32_t k = 0; k < KV; ++k) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
   };
+  const bool teller = chunk + 1u == la.chunks;   // the task's last chunk tells the host the task's total
   uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
   // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
   auto look_back = [&]() {
@@ -270,8 +271,16 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
         if (j * 64u + lane < chunk)
           pw[j] = __hip_atomic_load(la.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    for (uint32_t d = 0; d < la.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
-    request(0);
+    if (wave == 1 && teller) {
+      // The host waits for this wave's word: it looks back before it asks for any rows (its polls
+      // would wait for them: loads return in order), so the task's total leaves as soon as the
+      // counts of the task's chunks are known, not when the first sub-tile has arrived.
+      look_back();
+      request(0);
+    } else {
+      for (uint32_t d = 0; d < la.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
+      request(0);
+    }
   }
 
   uint32_t prefix = 0, before = 0, staged_kept = 0, staged_orow = 0;
@@ -291,7 +300,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     // request would be waited for where the next old line is parked
     asm volatile("" ::: "memory");
     // (wave 1 looks back first where it does: its polls wait for everything it has asked for)
-    const bool looks_back = wave == 1u && s == 0u;
+    const bool looks_back = wave == 1u && s == 0u && !teller;
     if (s + 1u < n_sub && !looks_back) request(s + 1u);
     const uint32_t t_r0 = s * sub_rows, t_rows = min(sub_rows, c_rows - t_r0);
     if (wave == 0) {

@@ -271,7 +271,7 @@ def measure(w, steps, warmup):
     return ms, kern, single
 
 
-def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0):
+def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0, **build_options):
     """Per-call wall time of the same config through functs_amd.jit: the scripted
     program, functionalized, with its regions run by tssa::ParallelFunctor
     (output allocation, launches and the kept-row synchronisation included).
@@ -283,7 +283,7 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0):
     import functs_amd.jit as fj
     from functs_amd.benchmark import PROGRAMS
     import functs_amd.aot as aot
-    fn = fj.build(fj.script(PROGRAMS[name]), list(cpu_args))
+    fn = fj.build(fj.script(PROGRAMS[name]), list(cpu_args), **build_options)
     args = [a.to(dev) if isinstance(a, torch.Tensor) else a for a in cpu_args]
     for _ in range(warmup):
         fn(*args)
@@ -513,6 +513,18 @@ def main():
         ts_us, n_functors, spec_share, sync_us, cold_us, cold_sync_us, host = torchscript_route(
             name, w.cpu_args, dev, args.steps, args.warmup, COLD_BYTES)
         rec["torchscript_route_host_us"] = host
+        rec["torchscript_route_direct_call"] = n_functors == 1   # one functor: called without the TorchScript interpreter
+        if rec["row_compaction"]:
+            # opt-in forms of the same call (functs_amd.jit.build): results that stay the operator's
+            # lists, and results at full size with their counts as a tensor, which wait for nothing
+            options = {"padded_outputs": dict(padded_outputs=True)}
+            if name in ("c3", "c5"):
+                options["lazy_lists"] = dict(lazy_lists=True)
+            for label, kw in options.items():
+                o_us, _, _, o_sync, o_cold, o_cold_sync, _ = torchscript_route(name, w.cpu_args, dev, args.steps, args.warmup, COLD_BYTES, **kw)
+                rec["torchscript_route_latency_us_" + label] = round(o_cold, 2)
+                rec["torchscript_route_drained_latency_us_" + label] = round(o_cold_sync, 2)
+                rec["torchscript_route_latency_us_warm_" + label] = round(o_us, 2)
         rec["torchscript_route_latency_us"] = round(cold_us, 2)
         rec["torchscript_route_drained_latency_us"] = round(cold_sync_us, 2)
         rec["torchscript_route_latency_us_warm"] = round(ts_us, 2)

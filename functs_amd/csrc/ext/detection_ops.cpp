@@ -455,6 +455,41 @@ bool fuseTailsIn(Block* b) {
 
 bool FuseDetectionTail(std::shared_ptr<Graph> graph) { return fuseTailsIn(graph->block()); }
 
+bool PadCompactedResults(std::shared_ptr<Graph> graph) {
+  if (graph->outputs().size() != 1) return false;
+  Node* ret = graph->outputs()[0]->node();
+  if (ret->kind() != c10::prim::TupleConstruct || ret->owningBlock() != graph->block() || ret->output()->uses().size() != 1) return false;
+  bool changed = false;
+  for (auto it = graph->nodes().begin(); it != graph->nodes().end();) {
+    Node* f = *it;
+    ++it;
+    if (f->kind() != sym::ParallelFunctor() || !f->hasAttribute(sym::compact_rows()) || f->i(sym::compact_rows()) == 0 ||
+        f->hasAttribute(sym::padded_outputs()))
+      continue;
+    if (f->i(sym::is_parallel_map()) != 0 && f->i(sym::parallel_degree()) < 1) continue;   // (an empty map has no padded form)
+    bool only_returned = true;
+    for (Value* o : f->outputs())
+      for (const Use& u : o->uses()) only_returned = only_returned && u.user == ret;
+    if (!only_returned) continue;
+    Node* padded = graph->create(sym::ParallelFunctor(), f->inputs(), f->outputs().size() + 1);
+    padded->copyAttributes(*f);
+    padded->i_(sym::padded_outputs(), 1);
+    padded->setSourceRange(f->sourceRange());
+    for (Value* o : padded->outputs()) o->setType(c10::TensorType::get());
+    padded->insertBefore(f);
+    for (size_t k = 0; k < f->outputs().size(); ++k) f->output(k)->replaceAllUsesWith(padded->output(k));
+    ret->addInput(padded->output(f->outputs().size()));
+    f->destroy();
+    changed = true;
+  }
+  if (changed) {
+    std::vector<c10::TypePtr> types;
+    for (Value* v : ret->inputs()) types.push_back(v->type());
+    ret->output()->setType(c10::TupleType::create(std::move(types)));
+  }
+  return changed;
+}
+
 TORCH_LIBRARY(functs, m) {
   m.def("nms(Tensor dets, Tensor scores, float iou_threshold) -> Tensor", nms);
   m.def("batched_nms(Tensor boxes, Tensor scores, Tensor idxs, float iou_threshold=0.45) -> (Tensor, Tensor)", batchedNms);

@@ -15,6 +15,104 @@ namespace py = pybind11;
 using namespace functs;
 using torch::jit::Graph;
 
+namespace {
+// A built graph that is nothing but ONE tssa::ParallelFunctor over the function's arguments (what
+// the pipeline makes of a program that fuses completely) is called without the TorchScript
+// interpreter: the arguments go to the operator's stack, its results come back.  Same operator,
+// same results; what is saved is the executor's per-call work around a single node.
+// A List[Tensor] result that stays the operator's list: elements become Python objects when they
+// are asked for.  A map over many tasks returns hundreds of tensors, and a caller that looks at a
+// few of them (or hands the list on) does not pay for a wrapper per element on every call.
+struct TensorList {
+  c10::List<at::Tensor> list;
+  py::list tolist() const {
+    py::list out(list.size());
+    for (size_t k = 0; k < list.size(); ++k) out[k] = py::reinterpret_steal<py::object>(THPVariable_Wrap(list.get(k)));
+    return out;
+  }
+};
+
+struct DirectFunctor {
+  bool lazy_lists = false;                      // List[Tensor] results come back as TensorList
+  std::shared_ptr<Graph> graph;                 // owns the node
+  mutable std::optional<torch::jit::Operation> op;   // (Operation's call operator is not const)
+  std::vector<int> source;                      // per operator input: graph input number, or -1 - k for constants[k]
+  std::vector<c10::IValue> constants;
+  std::vector<c10::TypePtr> arg_types;          // of the graph inputs
+  std::vector<int> results;                     // per returned value: operator output number
+  size_t n_op_outputs = 0;
+  bool tuple_result = false;
+
+  static std::shared_ptr<DirectFunctor> match(const std::shared_ptr<Graph>& graph) {
+    using namespace torch::jit;
+    Node* functor = nullptr;
+    Node* tuple = nullptr;
+    for (Node* n : graph->nodes()) {
+      if (n->kind() == c10::prim::Constant) continue;
+      if (n->kind() == c10::Symbol::fromQualString("tssa::ParallelFunctor") && !functor) { functor = n; continue; }
+      if (n->kind() == c10::prim::TupleConstruct && functor && !tuple) { tuple = n; continue; }
+      return nullptr;
+    }
+    if (!functor || graph->outputs().size() != 1) return nullptr;
+    auto d = std::make_shared<DirectFunctor>();
+    d->graph = graph;
+    for (Value* in : functor->inputs()) {
+      if (auto c = toIValue(in)) {
+        d->source.push_back(-1 - (int)d->constants.size());
+        d->constants.push_back(*c);
+        continue;
+      }
+      size_t k = 0;
+      while (k < graph->inputs().size() && graph->inputs()[k] != in) ++k;
+      if (k == graph->inputs().size()) return nullptr;
+      d->source.push_back((int)k);
+    }
+    for (Value* in : graph->inputs()) d->arg_types.push_back(in->type());
+    Value* ret = graph->outputs()[0];
+    std::vector<Value*> returned;
+    if (tuple) {
+      if (ret != tuple->output() || tuple->output()->uses().size() != 1) return nullptr;
+      for (Value* v : tuple->inputs()) returned.push_back(v);
+      d->tuple_result = true;
+    } else {
+      returned.push_back(ret);
+    }
+    for (Value* v : returned) {
+      if (v->node() != functor) return nullptr;
+      for (int seen : d->results)
+        if (seen == (int)v->offset()) return nullptr;   // (results are moved out of the stack one by one)
+      d->results.push_back((int)v->offset());
+    }
+    d->n_op_outputs = functor->outputs().size();
+    d->op = functor->getOperation();
+    return d;
+  }
+
+  py::object call(const py::args& args) const {
+    TORCH_CHECK(args.size() == arg_types.size(), "expected ", arg_types.size(), " arguments, got ", args.size());
+    torch::jit::Stack stack;
+    stack.reserve(source.size() + n_op_outputs);
+    for (int s : source) {
+      if (s < 0) stack.push_back(constants[(size_t)(-1 - s)]);
+      else stack.push_back(torch::jit::toIValue(args[(size_t)s], arg_types[(size_t)s]));
+    }
+    {
+      py::gil_scoped_release release;
+      (*op)(stack);
+    }
+    TORCH_CHECK(stack.size() == n_op_outputs, "the operator left ", stack.size(), " values for ", n_op_outputs, " results");
+    auto convert = [this](c10::IValue&& v) -> py::object {
+      if (lazy_lists && v.isTensorList()) return py::cast(TensorList{std::move(v).toTensorList()});
+      return torch::jit::toPyObject(std::move(v));
+    };
+    if (!tuple_result) return convert(std::move(stack[(size_t)results[0]]));
+    py::tuple out(results.size());
+    for (size_t k = 0; k < results.size(); ++k) out[k] = convert(std::move(stack[(size_t)results[k]]));
+    return std::move(out);
+  }
+};
+}  // namespace
+
 PYBIND11_MODULE(_C, m) {
   m.doc() = "MI355X backend of FuncTs/FAIT fused functionalized regions";
   py::class_<TensorSSAMutateInfo, std::shared_ptr<TensorSSAMutateInfo>>(m, "TensorSSAMutateInfo")
@@ -89,6 +187,7 @@ PYBIND11_MODULE(_C, m) {
   m.def("_plan_functors", PlanFunctors);
   m.def("_jit_pass_infer_static_shapes", InferStaticShapes);
   m.def("_jit_pass_fuse_detection_tail", FuseDetectionTail);
+  m.def("_jit_pass_pad_compacted_results", PadCompactedResults);
   m.def("_functor_host_timing", functorHostTiming);
   m.def("_functor_host_times", []() {
     py::dict d;
@@ -135,4 +234,23 @@ PYBIND11_MODULE(_C, m) {
     return h;
   });
   m.def("_fxhip_library", []() { return functs::fxhipLibraryPath(); });
+  py::class_<TensorList>(m, "TensorList")
+      .def("__len__", [](const TensorList& self) { return self.list.size(); })
+      .def("__getitem__",
+           [](const TensorList& self, int64_t k) {
+             const int64_t n = (int64_t)self.list.size();
+             if (k < -n || k >= n) throw py::index_error("TensorList index out of range");
+             return py::reinterpret_steal<py::object>(THPVariable_Wrap(self.list.get((size_t)(k < 0 ? k + n : k))));
+           })
+      .def("__getitem__", [](const TensorList& self, const py::slice& s) -> py::object { return py::object(self.tolist()[s]); })
+      .def("__iter__", [](const TensorList& self) -> py::object { return py::iter(self.tolist()); })
+      .def("tolist", &TensorList::tolist)
+      .def("__repr__", [](const TensorList& self) { return "TensorList(" + std::to_string(self.list.size()) + " tensors)"; });
+  // (a TensorList over given tensors: what a lazy result is, without running a functor)
+  m.def("_tensor_list", [](const std::vector<at::Tensor>& tensors) { return TensorList{c10::List<at::Tensor>(tensors)}; });
+  py::class_<DirectFunctor, std::shared_ptr<DirectFunctor>>(m, "DirectFunctor")
+      .def_readwrite("lazy_lists", &DirectFunctor::lazy_lists)
+      .def("__call__", [](const DirectFunctor& self, const py::args& args) { return self.call(args); });
+  // the direct form of a built graph, or None when the graph is more than one functor
+  m.def("_direct_functor", [](std::shared_ptr<Graph> graph) { return DirectFunctor::match(graph); });
 }

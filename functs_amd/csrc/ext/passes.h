@@ -88,6 +88,15 @@ void setSinkProducers(bool on);
 // (yolov3_bbox.py:104-179, 233-243).  True if the graph changed.
 bool FuseDetectionTail(std::shared_ptr<torch::jit::Graph> graph);
 
+// Opt-in (functs_amd.jit.build(..., padded_outputs=True)): every compacting functor whose results
+// are only returned gets padded_outputs=1, i.e. it returns each result at its full size (a map:
+// one tensor [tasks, rows, ...]) and does NOT wait for the kept-row counts, which it returns as
+// one more tensor (int32 in pinned host memory, written by the kernels) at the end of the
+// function's result tuple, one per such functor.  Rows from counts[task] on hold no values.  For
+// callers that feed the results to further work on the same stream and never need the sizes on
+// the host.  True if the graph changed.
+bool PadCompactedResults(std::shared_ptr<torch::jit::Graph> graph);
+
 // Static types of intermediate values (the reference's InferShape, fait/passes/refine_types.cpp:
 // 420-685, run at fait_pipeline.cpp:47): every operator node whose tensor arguments have complete
 // static types and whose other arguments are constants is run on meta tensors of those types, and

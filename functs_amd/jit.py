@@ -26,23 +26,39 @@ class AotScriptFunction(object):
     only.  Such a function keeps the functionalized script it was built from and builds a graph
     per set of argument shapes, the first one from the example; ``graph`` is that first one."""
 
-    def __init__(self, aot_script_fn, source=None, key=None, **kwargs):
+    def __init__(self, aot_script_fn, source=None, key=None, lazy_lists=False, padded_outputs=False, **kwargs):
         self._aot_script_fn = aot_script_fn
         self._source = source
-        self._variants = {key: aot_script_fn} if source is not None else None
+        self._lazy_lists = lazy_lists
+        self._padded_outputs = padded_outputs
+        self._call = _direct(aot_script_fn, lazy_lists)
+        self._variants = {key: self._call} if source is not None else None
 
     @property
     def graph(self):
         return self._aot_script_fn.graph
 
-    def __call__(self, *args, **kwargs):
+    def __call__(self, *args):
         if self._variants is None:
-            return self._aot_script_fn(*args, **kwargs)
+            return self._call(*args)
         key = _shape_key(args)
         fn = self._variants.get(key)
         if fn is None:
-            fn = self._variants[key] = _compile(self._source, args)[0]
-        return fn(*args, **kwargs)
+            fn = self._variants[key] = _direct(_compile(self._source, args, self._padded_outputs)[0], self._lazy_lists)
+        return fn(*args)
+
+
+def _direct(script_fn, lazy_lists=False):
+    """What a call of a built function runs: a graph that is one tssa::ParallelFunctor over the
+    arguments is called without the TorchScript interpreter (functs_amd._C.DirectFunctor: same
+    operator, same results), any other graph through its ScriptFunction."""
+    direct = _C._direct_functor(script_fn.graph)
+    if direct is None:
+        if lazy_lists:
+            raise ValueError("lazy_lists needs a function that builds into one fused region")
+        return script_fn
+    direct.lazy_lists = lazy_lists
+    return direct
 
 
 def extract_type_hint_from_tensor(input_):
@@ -155,23 +171,37 @@ class GraphedFunction(AotScriptFunction):
         return self._map(out, lambda t: t.clone())
 
 
-def build(fn, example_input: List[object], hip_graph: bool = False) -> AotScriptFunction:
+def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: bool = False,
+          padded_outputs: bool = False) -> AotScriptFunction:
     """Form fused regions in a functionalized script and return the callable
-    (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``."""
+    (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``.
+    ``lazy_lists=True`` (a function that builds into ONE fused region only): List[Tensor] results
+    come back as ``functs_amd._C.TensorList`` - a sequence whose elements become Python tensors when
+    they are read (len, indexing, iteration, ``tolist()``) - instead of Python lists, which cost a
+    wrapper object per element on every call (a map over 80 tasks returns 160 tensors).
+    ``padded_outputs=True``: row-compacting regions whose results the function returns hand them
+    back at full size (a map: one tensor [tasks, rows, ...] per result) without waiting for the
+    kept-row counts, which come as one more tensor at the end of the result tuple (int32, pinned
+    host memory that the kernels write; rows from counts[task] on hold no values): for callers that
+    pass the results on to work on the same stream."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
         raise AttributeError("only a functionalized jit script can be built")
-    aot, specialized = _compile(fn, example_input)
+    aot, specialized = _compile(fn, example_input, padded_outputs)
     source, key = (fn, _shape_key(example_input)) if specialized else (None, None)
-    return GraphedFunction(aot, source, key) if hip_graph else AotScriptFunction(aot, source, key)
+    if hip_graph:
+        return GraphedFunction(aot, source, key)
+    return AotScriptFunction(aot, source, key, lazy_lists=lazy_lists, padded_outputs=padded_outputs)
 
 
-def _compile(fn, example_input):
+def _compile(fn, example_input, padded_outputs=False):
     """(compiled function, whether its graph holds constants of the example's shapes)"""
     g = fn.graph.copy()
     if isinstance(fn, torch.jit.ScriptModule):
         _strip_self(g)
     hints = [extract_type_hint_from_tensor(i) for i in example_input]
     specialized = bool(_C._jit_pass_fait_pipeline(g, hints))
+    if padded_outputs:
+        _C._jit_pass_pad_compacted_results(g)
     return _C._create_function_from_graph("forward", g), specialized
 
 

@@ -179,7 +179,7 @@ def _run_benchmark_programs(names):
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--out", default=SPEC_DIR, help="directory the generated sources go to")
-    ap.add_argument("--programs", default="c1,c2,c3,c4,c5,variants,coverage,stream",
+    ap.add_argument("--programs", default="c1,c2,c3,c4,c5,c5_nms,yolo_head,yolo_head_nms,attention,delta2bbox,variants,coverage,stream",
                     help="what to capture: benchmark programs, variants (other spellings of the detection head), "
                          "coverage, stream")
     ap.add_argument("--plan-only", action="store_true", help="plan the regions without running them: needs no GPU")

@@ -811,8 +811,10 @@ static uint32_t rs_max_sub_rows(const FxRsInfo& ri) {
   return std::min<uint32_t>(FX_RS_SUB, (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S);
 }
 // the window, then the staged outputs (fx_rowstream.h lays them out the same way)
-static uint32_t rs_lds_bytes(const FxRsInfo& ri, const FxRsKernel* k, uint32_t sub) {
-  return (((sub * ri.S + 3u + 3u) >> 2) + 1u) * 16u + (sub * k->stage_row_words + 8u * k->n_staged) * 4u;
+// window, staged outputs, and the chunk's table of side values
+static uint32_t rs_lds_bytes(const FxRsInfo& ri, const FxRsKernel* k, uint32_t sub, uint32_t chunk_rows, bool side) {
+  return (((sub * ri.S + 3u + 3u) >> 2) + 1u) * 16u + (sub * k->stage_row_words + 8u * k->n_staged) * 4u +
+         (side ? chunk_rows * k->side_row_words * 4u : 0u);
 }
 static size_t rs_status_words(const FxRsInfo& ri) {
   const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
@@ -854,35 +856,59 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
     const uint32_t forced_sub = rs_env("FXHIP_RS_SUB_ROWS"), forced_chunk = rs_env("FXHIP_RS_CHUNK_ROWS");
     uint32_t best_sub = 0, best_cr = 0, best_n = 0;
-    for (uint32_t sub = rs_max_sub_rows(ri); sub >= 8u; sub = sub > 8u ? std::max<uint32_t>(8u, sub - 8u) : 0u) {
-      if (forced_sub && sub > forced_sub) continue;
-      int per_cu = 0;
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern->fn, (int)FX_BLOCK, (size_t)rs_lds_bytes(ri, kern, sub)) != hipSuccess || per_cu < 1) {
-        (void)hipGetLastError();
-        continue;
+    bool best_side = false;
+    // with the chunk's table of side values in LDS, and without it (where the table would cost a
+    // workgroup per CU or a sub-tile per chunk, the rows load their side values themselves)
+    for (int with_side = kern->side_row_words != 0 ? 1 : 0; with_side >= 0; --with_side) {
+      for (uint32_t sub = rs_max_sub_rows(ri); sub >= 8u; sub = sub > 8u ? std::max<uint32_t>(8u, sub - 8u) : 0u) {
+        if (forced_sub && sub > forced_sub) continue;
+        // at most the occupancy the kernels are compiled for: a launch that needs a seventh slot per CU
+        // (kernels that happen to stay below 73 registers) is not placed at once and takes 27.4 us
+        // where six per CU take 23.4 us
+        auto slots = [&](uint32_t chunk_rows) {
+          int n = 0;
+          if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern->fn, (int)FX_BLOCK,
+                                                           (size_t)rs_lds_bytes(ri, kern, sub, chunk_rows, with_side != 0)) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+          }
+          return std::min(n, (int)FX_RS_OCC);
+        };
+        auto chunkFor = [&](int per_cu) {
+          const uint32_t resident = (uint32_t)per_cu * (uint32_t)std::max(cus, 1);
+          const uint32_t per_task = std::max<uint32_t>(1u, resident / std::max<uint32_t>(ri.n_tasks, 1u));
+          uint32_t c = (ri.n_rows + per_task - 1) / per_task;
+          c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(c, min_chunk));
+          if (forced_chunk) c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(forced_chunk, min_chunk));
+          return c;
+        };
+        // the table is part of the LDS, and the chunk follows from the number of resident
+        // workgroups: from the largest chunk down until both agree
+        int per_cu = slots(FX_BLOCK);
+        if (per_cu < 1) continue;
+        uint32_t cr = chunkFor(per_cu);
+        for (int round = 0; round < 3; ++round) {
+          const int better = slots(cr);
+          if (better <= per_cu) break;
+          per_cu = better;
+          cr = chunkFor(per_cu);
+        }
+        const uint32_t n = (cr + sub - 1) / sub;
+        if (rs_env("FXHIP_RS_VERBOSE"))
+          fprintf(stderr, "[fxhip] row-stream geometry: side table %d, sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
+                  with_side, sub, rs_lds_bytes(ri, kern, sub, cr, with_side != 0), per_cu, cr, n);
+        if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; best_side = with_side != 0; }
+        if (forced_sub || sub == 8u) break;
       }
-      // at most the occupancy the kernels are compiled for: a launch that needs a seventh slot per CU
-      // (kernels that happen to stay below 73 registers) is not placed at once and takes 27.4 us
-      // where six per CU take 23.4 us
-      per_cu = std::min(per_cu, (int)FX_RS_OCC);
-      const uint32_t resident = (uint32_t)per_cu * (uint32_t)std::max(cus, 1);
-      const uint32_t per_task = std::max<uint32_t>(1u, resident / std::max<uint32_t>(ri.n_tasks, 1u));
-      uint32_t cr = (ri.n_rows + per_task - 1) / per_task;
-      cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(cr, min_chunk));
-      if (forced_chunk) cr = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(forced_chunk, min_chunk));
-      const uint32_t n = (cr + sub - 1) / sub;
-      if (rs_env("FXHIP_RS_VERBOSE"))
-        fprintf(stderr, "[fxhip] row-stream geometry: sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
-                sub, rs_lds_bytes(ri, kern, sub), per_cu, cr, n);
-      if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; }
-      if (forced_sub || sub == 8u) break;
     }
     if (best_sub == 0) return fail(FX_E_LIMIT, "row-stream kernel: no sub-tile size fits the device");
     pl->rs_sub_rows = best_sub;
     pl->rs_chunk_rows = best_cr;
+    pl->rs_side_lds = best_side ? 1u : 0u;
   }
   rl->sub_rows = pl->rs_sub_rows;
   rl->chunk_rows = pl->rs_chunk_rows;
+  rl->side_lds = pl->rs_side_lds;
   rl->chunks = (ri.n_rows + rl->chunk_rows - 1) / rl->chunk_rows;
   const uint32_t cr = rl->chunk_rows;
   // A launch whose first sub-tiles alone are megabytes of requests floods the memory system: there
@@ -895,7 +921,7 @@ static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const Fx
   const uint32_t grid = rl.chunks * rl.n_tasks;
   if (grid == 0) return hipSuccess;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows), stream);
+  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----

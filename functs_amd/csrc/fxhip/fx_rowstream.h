@@ -172,6 +172,10 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
   const uint32_t sub_rows = (c_rows + n_sub0 - 1u) / n_sub0;
   const uint32_t n_sub = (c_rows + sub_rows - 1u) / sub_rows;
   FxRsRt rt{la, task, {}, {}};
+  // What the rows' own code reads from memory besides the window (a few words per row: anchors,
+  // strides ...) is fetched for all rows of the chunk before the first sub-tile, into a table in LDS.
+  const bool SIDE_LDS = P::n_row_cols != 0u && P::n_side != 0u && P::n_side <= FX_RS_MAX_SIDE && la.side_lds != 0u;
+  uint32_t* side = nullptr;
   {
     // staged outputs behind the window, each sub_rows rows and a group of slack
     uint32_t* sp = L + ((((la.sub_rows * S + 3u + 3u) >> 2) + 1u) << 2);
@@ -181,6 +185,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
       rt.ph[k] = 0u;
       if (k < P::n_out && P::stage_rowlen[k] != 0u) sp += la.sub_rows * P::stage_rowlen[k] + 8u;
     }
+    side = sp;   // la.chunk_rows rows of P::n_side words
   }
   // element 0 of this task's rows of the window input
   const FX_AS1 uint32_t* win = (const FX_AS1 uint32_t*)rt.in(0) + (int64_t)la.in_tcoef[0] * task;
@@ -194,9 +199,12 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(a0 & ~(uint64_t)15);
     n_vec = (shift + rows * S + 3u) >> 2;   // <= KV * NT (host)
     // every line is used once; lanes past the end ask for the last line again rather than branch,
-    // so that the requests leave back to back
+    // so that the requests leave back to back; a load of which no lane of the wave has a part is
+    // left out (a branch on a value that all lanes share)
+    const uint32_t n_vec_u = uni(n_vec);
 #pragma unroll
-    for (uint32_t k = 0; k < KV; ++k) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
+    for (uint32_t k = 0; k < KV; ++k)
+      if (k * NT + wave * 64u < n_vec_u) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
   };
   const bool teller = chunk + 1u == la.chunks;   // the task's last chunk tells the host the task's total
   uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
@@ -271,6 +279,15 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
         if (j * 64u + lane < chunk)
           pw[j] = __hip_atomic_load(la.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    if (SIDE_LDS) {
+      // (these waves hold their rows back anyway, and the table is shared by the tasks: cache hits)
+      for (uint32_t r = threadIdx.x - 64u; r < c_rows; r += NT - 64u) {
+        typename P::Side sd;
+        P::template row_side<FxRsRt>(rt, c_r0 + r, sd);
+#pragma unroll
+        for (uint32_t k = 0; k < P::n_side; ++k) side[r * P::n_side + k] = sd.s[k];
+      }
+    }
     if (wave == 1 && teller) {
       // The host waits for this wave's word: it looks back before it asks for any rows (its polls
       // would wait for them: loads return in order), so the task's total leaves as soon as the
@@ -344,7 +361,17 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     // ---- the columns with code of their own: one kept row per lane
     if (P::n_row_cols != 0u && threadIdx.x < n_kept) {
       const uint32_t src = s_rowmap[threadIdx.x];
-      P::template row<FxRsRt>(rt, Wb + src * S, rs0 + src, orow + threadIdx.x, threadIdx.x);
+      // What the row reads besides the window: from the chunk's table in LDS.  (Loaded here, the
+      // words would arrive behind the next sub-tile, which this wave has asked for already: loads
+      // return in order.)
+      typename P::Side sd;
+      if (SIDE_LDS) {
+#pragma unroll
+        for (uint32_t k = 0; k < P::n_side; ++k) sd.s[k] = side[(t_r0 + src) * P::n_side + k];
+      } else {
+        P::template row_side<FxRsRt>(rt, rs0 + src, sd);
+      }
+      P::template row<FxRsRt>(rt, Wb + src * S, sd, rs0 + src, orow + threadIdx.x, threadIdx.x);
     }
     // ---- vector segments: four columns per lane
     fx_rs_segments<P>(typename P::Vecs{}, rt, Wb, s_rowmap, n_kept, rs0, orow, threadIdx.x, NT);
@@ -359,12 +386,13 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
 }
 
 struct FxRsRegistrar {
-  FxRsRegistrar(uint64_t key, const void* fn, uint32_t S, uint32_t stage_row_words, uint32_t n_staged) {
+  FxRsRegistrar(uint64_t key, const void* fn, uint32_t S, uint32_t stage_row_words, uint32_t n_staged, uint32_t side_row_words) {
     FxRsKernel k;
     k.fn = fn;
     k.S = S;
     k.stage_row_words = stage_row_words;
     k.n_staged = n_staged;
+    k.side_row_words = side_row_words;
     fx_rs_register(key, k);
   }
 };
@@ -372,4 +400,5 @@ struct FxRsRegistrar {
 }  // namespace
 
 #define FX_RS_REGISTER(P) \
-  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P>, P::S, P::stage_row_words, P::n_staged);
+  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P>, P::S, P::stage_row_words, P::n_staged, \
+                                           (P::n_row_cols != 0u && P::n_side <= FX_RS_MAX_SIDE) ? P::n_side : 0u);

@@ -24,7 +24,7 @@
 
 #include "fx_bytecode.h"
 
-#define FX_RS_VERSION 2u
+#define FX_RS_VERSION 3u
 #define FX_RS_MAX_IN 8u         // input buffers of a region
 #define FX_RS_MAX_OUT 8u        // outputs
 #define FX_RS_MAX_FIMM 24u      // distinct floating-point constants
@@ -38,6 +38,7 @@
 #define FX_RS_OCC 6              // waves per SIMD the register budget of a generated kernel is set for (80 registers)
 #define FX_RS_VEC_MIN 8u        // shortest run of alike columns that takes the vector form
 #define FX_RS_MAX_UNROLL 64u    // most columns evaluated one by one per row
+#define FX_RS_MAX_SIDE 16u      // most words per row that a chunk keeps in LDS of what its rows read besides the window
 
 // What the analysis of a plan found (host).
 struct FxRsInfo {
@@ -69,7 +70,8 @@ struct FxRsLaunch {
   int32_t in_tcoef[FX_RS_MAX_IN];
   uint32_t out_slot[FX_RS_MAX_OUT], out_tstride[FX_RS_MAX_OUT];
   uint32_t fimm[FX_RS_MAX_FIMM];
-  uint32_t slot_err, pad0;
+  uint32_t slot_err;
+  uint32_t side_lds;            // the chunk keeps a table of its rows' side values in LDS (0: a row loads them when its turn comes)
   uint32_t* status;             // one word per chunk, tagged with the epoch
   uint32_t* totals;             // pinned host memory: kept rows per task
 };
@@ -81,6 +83,7 @@ struct FxRsKernel {
   uint32_t S = 0;               // row length the kernel is generated for
   uint32_t stage_row_words = 0; // elements per kept row that the kernel puts together in LDS before they leave
   uint32_t n_staged = 0;        // outputs that take that route
+  uint32_t side_row_words = 0;  // words per row of the chunk's table of what the rows read besides the window
 };
 void fx_rs_register(uint64_t key, const FxRsKernel& k);
 const FxRsKernel* fx_rs_find(uint64_t key);

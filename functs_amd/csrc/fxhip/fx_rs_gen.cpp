@@ -741,11 +741,15 @@ struct Emitter {
   const Model& m;
   const Graph& g;
   bool window;            // loads of input 0 read the staged row (W) instead of memory
-  std::ostringstream& o;
+  std::ostringstream* out;   // where the code goes (emitSide and emitAll of one emitter may write to different places)
   const char* ind;
   std::vector<char> done;
+  // Loads from memory whose address depends on the row only, in the order in which emitSide
+  // issues them: a row's code in two parts, the loads (which can leave ahead of everything
+  // else the wave asks for) and the rest, which finds their values in sd.s[].
+  std::vector<int> side;
   Emitter(const Model& m_, const Graph& g_, bool window_, std::ostringstream& o_, const char* ind_)
-      : m(m_), g(g_), window(window_), o(o_), ind(ind_), done(g_.nodes.size(), 0) {}
+      : m(m_), g(g_), window(window_), out(&o_), ind(ind_), done(g_.nodes.size(), 0) {}
 
   std::string ref(int id) const {
     if (id == M_TRUE) return "true";
@@ -792,39 +796,50 @@ struct Emitter {
     if (n.kind == K_CONST || n.kind == K_FIMM) return;
     const std::string me = ref(id);
     const char* ty = isBool(n.kind) ? "const bool " : "const uint32_t ";
-    o << ind << ty << me << " = ";
+    (*out) << ind << ty << me << " = ";
     switch (n.kind) {
-      case K_SCAL: o << "rs_scal<" << n.i[1] << ">(rt, " << n.i[0] << ")"; break;
-      case K_AFF: o << lin(n.i[0], n.i[1], n.i[2]); break;
+      case K_SCAL: (*out) << "rs_scal<" << n.i[1] << ">(rt, " << n.i[0] << ")"; break;
+      case K_AFF: (*out) << lin(n.i[0], n.i[1], n.i[2]); break;
       case K_LOAD:
       case K_LOADG: {
         const uint32_t dt = (uint32_t)(n.i[1] & 0xff);
         const int cvt = (int)(n.i[1] >> 8);
         if (fromWindow(n)) {
-          if (n.kind == K_LOADG) o << "W[" << ref(n.a[0]) << " ? (" << winOff(n) << ") : 0]";
-          else o << "W[" << winOff(n) << "]";
+          if (n.kind == K_LOADG) (*out) << "W[" << ref(n.a[0]) << " ? (" << winOff(n) << ") : 0]";
+          else (*out) << "W[" << winOff(n) << "]";
         } else {
-          o << "rs_ld<" << dtName(dt) << ", " << cvt << ">(rt, " << n.i[0] << ", ";
-          if (n.kind == K_LOADG) o << ref(n.a[0]) << " ? " << loadOff(n) << " : 0u";
-          else o << loadOff(n);
-          o << ")";
+          (*out) << "rs_ld<" << dtName(dt) << ", " << cvt << ">(rt, " << n.i[0] << ", ";
+          if (n.kind == K_LOADG) (*out) << ref(n.a[0]) << " ? " << loadOff(n) << " : 0u";
+          else (*out) << loadOff(n);
+          (*out) << ")";
         }
       } break;
       case K_LOADX:
-        o << "rs_ldx<" << dtName((uint32_t)n.i[1]) << ">(rt, " << n.i[0] << ", (uint32_t)((int32_t)" << ref(n.a[0]) << " + " << n.i[2] << "))";
+        (*out) << "rs_ldx<" << dtName((uint32_t)n.i[1]) << ">(rt, " << n.i[0] << ", (uint32_t)((int32_t)" << ref(n.a[0]) << " + " << n.i[2] << "))";
         break;
-      case K_UN: o << "rs_" << opname((uint32_t)n.op) << "(" << ref(n.a[0]) << ")"; break;
-      case K_BIN: o << "rs_" << opname((uint32_t)n.op) << "(" << ref(n.a[0]) << ", " << ref(n.a[1]) << ")"; break;
-      case K_SEL: o << "rs_SEL(" << ref(n.a[0]) << ", " << ref(n.a[1]) << ", " << ref(n.a[2]) << ")"; break;
-      case K_IRANGE: o << "rs_IRANGE(" << ref(n.a[0]) << ", " << n.i[0] << ", " << n.i[1] << ", " << n.i[2] << ")"; break;
-      case K_B2I: o << "(" << ref(n.a[0]) << " ? 1u : 0u)"; break;
-      case K_NZ: o << "(" << ref(n.a[0]) << " != 0u)"; break;
-      case K_INR: o << "rs_INR(" << ref(n.a[0]) << ", " << n.i[0] << "u, " << n.i[1] << ")"; break;
-      case K_BAND: o << "(" << ref(n.a[0]) << " && " << ref(n.a[1]) << ")"; break;
-      case K_BNOT: o << "!" << ref(n.a[0]); break;
-      default: o << "0u"; break;
+      case K_UN: (*out) << "rs_" << opname((uint32_t)n.op) << "(" << ref(n.a[0]) << ")"; break;
+      case K_BIN: (*out) << "rs_" << opname((uint32_t)n.op) << "(" << ref(n.a[0]) << ", " << ref(n.a[1]) << ")"; break;
+      case K_SEL: (*out) << "rs_SEL(" << ref(n.a[0]) << ", " << ref(n.a[1]) << ", " << ref(n.a[2]) << ")"; break;
+      case K_IRANGE: (*out) << "rs_IRANGE(" << ref(n.a[0]) << ", " << n.i[0] << ", " << n.i[1] << ", " << n.i[2] << ")"; break;
+      case K_B2I: (*out) << "(" << ref(n.a[0]) << " ? 1u : 0u)"; break;
+      case K_NZ: (*out) << "(" << ref(n.a[0]) << " != 0u)"; break;
+      case K_INR: (*out) << "rs_INR(" << ref(n.a[0]) << ", " << n.i[0] << "u, " << n.i[1] << ")"; break;
+      case K_BAND: (*out) << "(" << ref(n.a[0]) << " && " << ref(n.a[1]) << ")"; break;
+      case K_BNOT: (*out) << "!" << ref(n.a[0]); break;
+      default: (*out) << "0u"; break;
     }
-    o << ";\n";
+    (*out) << ";\n";
+  }
+
+  // The unconditional loads from memory that `roots` need (merged where they are neighbours), each
+  // into its slot of sd.s[]; returns the number of slots.  emitAll(roots, ...) of the SAME emitter
+  // afterwards takes their values from there.
+  size_t emitSide(const std::vector<int>& roots) {
+    std::vector<char> seen(g.nodes.size(), 0);
+    std::vector<int> order;
+    for (int r : roots) collect(r, seen, order);
+    emitLoads(order, true, /*to_side=*/true);
+    return side.size();
   }
 
   // Everything the values in `roots` need, loads first.  Plain 32-bit loads of neighbouring
@@ -833,11 +848,22 @@ struct Emitter {
     std::vector<char> seen(g.nodes.size(), 0);
     std::vector<int> order;
     for (int r : roots) collect(r, seen, order);
+    if (!side.empty()) {
+      for (size_t k = 0; k < side.size(); ++k) {
+        (*out) << ind << "const uint32_t " << ref(side[k]) << " = sd.s[" << k << "];\n";
+        done[side[k]] = 1;
+      }
+    }
+    emitLoads(order, merge_loads, false);
+    for (int id : order) emitNode(id);
+  }
+
+  void emitLoads(const std::vector<int>& order, bool merge_loads, bool to_side) {
     // loads from memory, merged
     std::vector<int> plain;
     for (int id : order) {
       const Node& n = g.nodes[id];
-      if (n.kind != K_LOAD || fromWindow(n)) continue;
+      if (n.kind != K_LOAD || fromWindow(n) || done[id]) continue;
       const uint32_t dt = (uint32_t)(n.i[1] & 0xff);
       if (merge_loads && (dt == FX_F32 || dt == FX_I32) && (n.i[1] >> 8) == 0 && n.i[4] == 0) plain.push_back(id);
     }
@@ -858,21 +884,41 @@ struct Emitter {
       const size_t w = e - k >= 4 ? 4 : (e - k >= 2 ? 2 : 1);
       if (w > 1) {
         const Node& n0 = g.nodes[plain[k]];
-        o << ind << "uint32_t";
-        for (size_t j = 0; j < w; ++j) o << (j ? ", " : " ") << ref(plain[k + j]);
-        o << ";\n" << ind << "rs_ld" << w << "(rt, " << n0.i[0] << ", " << loadOff(n0);
+        if (!to_side) {
+          (*out) << ind << "uint32_t";
+          for (size_t j = 0; j < w; ++j) (*out) << (j ? ", " : " ") << ref(plain[k + j]);
+          (*out) << ";\n";
+        }
+        (*out) << ind << "rs_ld" << w << "(rt, " << n0.i[0] << ", " << loadOff(n0);
         for (size_t j = 0; j < w; ++j) {
-          o << ", " << ref(plain[k + j]);
+          if (to_side) {
+            (*out) << ", sd.s[" << side.size() << "]";
+            side.push_back(plain[k + j]);
+          } else {
+            (*out) << ", " << ref(plain[k + j]);
+          }
           done[plain[k + j]] = 1;
         }
-        o << ");\n";
+        (*out) << ");\n";
       }
       k += w;
     }
-    // the other loads whose address needs nothing computed, then the rest in order
-    for (int id : order)
-      if (g.nodes[id].kind == K_LOAD) emitNode(id);
-    for (int id : order) emitNode(id);
+    // the other loads whose address needs nothing computed
+    for (int id : order) {
+      const Node& n = g.nodes[id];
+      if (n.kind != K_LOAD || done[id] || fromWindow(n)) continue;
+      if (to_side) {
+        if (n.i[4] != 0) continue;   // (walks along the columns: not a row's load)
+        const uint32_t dt = (uint32_t)(n.i[1] & 0xff);
+        (*out) << ind << "sd.s[" << side.size() << "] = rs_ld<" << dtName(dt) << ", " << (int)(n.i[1] >> 8) << ">(rt, " << n.i[0] << ", " << loadOff(n) << ");\n";
+        side.push_back(id);
+        done[id] = 1;
+      } else {
+        emitNode(id);
+      }
+    }
+    if (to_side)   // (emitAll declares the values again from sd.s[])
+      for (int id : side) done[id] = 0;
   }
 };
 
@@ -939,14 +985,25 @@ std::string emitSource(const Model& m, const std::string& label) {
     << "  // the columns that need code of their own, for one kept row: W is the row in the window,\n"
     << "  // row its index in the task, orow its index among the kept rows of the task, lrow among those\n"
     << "  // of the sub-tile\n"
-    << "  static constexpr uint32_t n_row_cols = " << m.row_cols.size() << ";\n"
-    << "  template <class RT>\n"
-    << "  static FX_RS_FN void row(const RT& rt, const uint32_t* W, uint32_t row, uint32_t orow, uint32_t lrow) {\n"
-    << "    const uint32_t t = 0; (void)t; (void)W; (void)row; (void)orow; (void)lrow;\n";
+    << "  static constexpr uint32_t n_row_cols = " << m.row_cols.size() << ";\n";
   {
-    Emitter em(m, m.g_row, true, o, "    ");
+    // in two parts: what a row reads from memory besides the window (side: its loads can leave
+    // ahead of the next sub-tile's requests, which everything later would queue behind), and the rest
+    std::ostringstream side_body;
+    Emitter em(m, m.g_row, true, side_body, "    ");
     std::vector<int> roots;
     for (const Segment& s : m.row_cols) roots.push_back(s.result);
+    const size_t n_side = em.emitSide(roots);
+    o << "  struct Side { uint32_t s[" << std::max<size_t>(n_side, 1) << "]; };\n"
+      << "  static constexpr uint32_t n_side = " << n_side << ";\n"
+      << "  template <class RT>\n"
+      << "  static FX_RS_FN void row_side(const RT& rt, uint32_t row, Side& sd) {\n"
+      << "    (void)rt; (void)row; (void)sd;\n"
+      << side_body.str() << "  }\n"
+      << "  template <class RT>\n"
+      << "  static FX_RS_FN void row(const RT& rt, const uint32_t* W, const Side& sd, uint32_t row, uint32_t orow, uint32_t lrow) {\n"
+      << "    const uint32_t t = 0; (void)t; (void)W; (void)sd; (void)row; (void)orow; (void)lrow;\n";
+    em.out = &o;
     em.emitAll(roots, true);
     // stores: four neighbouring columns of a plain 32-bit output as one 128-bit store
     for (size_t k = 0; k < m.row_cols.size();) {

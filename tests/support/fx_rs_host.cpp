@@ -205,7 +205,11 @@ void run_policy(const FxRsLaunch& la, const FxDyn* dyn, uint32_t* totals, uint32
         for (auto& st : stage) std::fill(st.begin(), st.end(), 0xdeadbeefu);
         fx_rs_phases<P, 0u, FxRsRt>(rt, orow);
         if (P::n_row_cols != 0u)
-          for (uint32_t r = 0; r < n_kept; ++r) P::template row<FxRsRt>(rt, Wb + rowmap[r] * S, rs0 + rowmap[r], orow + r, r);
+          for (uint32_t r = 0; r < n_kept; ++r) {
+            typename P::Side sd;
+            P::template row_side<FxRsRt>(rt, rs0 + rowmap[r], sd);
+            P::template row<FxRsRt>(rt, Wb + rowmap[r] * S, sd, rs0 + rowmap[r], orow + r, r);
+          }
         for (uint32_t tid = 0; tid < nt; ++tid)
           fx_rs_segments<P, FxRsRt>(typename P::Vecs{}, rt, Wb, rowmap.data(), n_kept, rs0, orow, tid, nt);
         if (P::n_staged != 0u)

@@ -109,7 +109,10 @@ def test_the_generated_row_code_shares_what_the_columns_share():
         src = r.rowstream_source(*_inputs(50, 80, 1))
         row = src[src.index("static FX_RS_FN void row("):src.index("using Vecs")]
         assert row.count("rs_EXP(") == 2 and row.count("rs_SIGMOID(") == 3, (decode, row)
-        assert row.count("rs_ld4(") == 1          # the anchor's four corners: one 128-bit load
+        # what the row reads besides the window is loaded by a part of its own (it leaves ahead of
+        # the next sub-tile's requests): the anchor's four corners as one 128-bit load, the stride
+        side = src[src.index("static FX_RS_FN void row_side("):src.index("static FX_RS_FN void row(")]
+        assert side.count("rs_ld4(") == 1 and side.count("rs_ld<") == 1 and "rs_ld" not in row
         assert "rs_SEL" not in row and "rs_INR" not in row   # every column predicate decided by the generator
 
 

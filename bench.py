@@ -235,14 +235,9 @@ def copy_reference_ms(dev, nbytes, rounds=4):
         _lib.copy_bytes(a, b)
     flush(dev)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(rounds):
-        for a, b in pairs:
-            _lib.copy_bytes(a, b)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / (rounds * n_pairs)
+    # launched back to back by the library, the way the regions' kernels are timed (a Python loop
+    # issues a launch every 5 to 6 us, longer than a small copy runs)
+    return _lib.copy_bytes_timed_sets(pairs, rounds)
 
 
 def measure(w, steps, warmup):

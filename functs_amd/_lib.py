@@ -195,6 +195,8 @@ _sig("fx_lstm_stack", _i, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _i, 
 _sig("fx_set_lstm_spin_limit", None, ctypes.c_uint32)
 _sig("fx_device_count", _i)
 _sig("fx_copy_bytes", _i, _vp, _vp, ctypes.c_size_t, _vp)
+_sig("fx_copy_bytes_timed_sets", _i, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p), _i, ctypes.c_size_t, _i, _vp,
+     ctypes.POINTER(ctypes.c_float))
 
 
 class FxError(RuntimeError):
@@ -207,6 +209,20 @@ def check(rc):
     if rc < 0:
         raise FxError(rc, lib.fx_last_error().decode())
     return rc
+
+
+def copy_bytes_timed_sets(pairs, rounds, stream=None):
+    """Mean milliseconds per launch of the copy kernel over `rounds` passes through the (src, dst)
+    pairs, launched back to back by the library (fx_copy_bytes_timed_sets)."""
+    import torch
+    nbytes = pairs[0][0].numel() * pairs[0][0].element_size()
+    assert all(a.is_cuda and b.is_cuda and a.numel() * a.element_size() == nbytes == b.numel() * b.element_size() for a, b in pairs)
+    src = (ctypes.c_void_p * len(pairs))(*[a.data_ptr() for a, _ in pairs])
+    dst = (ctypes.c_void_p * len(pairs))(*[b.data_ptr() for _, b in pairs])
+    st = torch.cuda.current_stream(pairs[0][0].device).cuda_stream if stream is None else stream
+    ms = ctypes.c_float()
+    check(lib.fx_copy_bytes_timed_sets(src, dst, len(pairs), nbytes, rounds, st, ctypes.byref(ms)))
+    return float(ms.value)
 
 
 def copy_bytes(src, dst, stream=None):

@@ -480,6 +480,12 @@ int fx_sort_nms(const fx_nms_desc* desc, void* stream);
 int fx_device_count(void);
 /* plain 16-byte copy kernel of known size: counter calibration and bandwidth ceiling */
 int fx_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
+/* The same copy timed the way fx_region_run_timed_sets times a region's kernels: `rounds` passes
+ * over n_sets (src, dst) pairs of `bytes` each, launched back to back from here between two events
+ * on the stream; *ms_per_copy is the mean per launch.  (A loop in an interpreted language cannot
+ * issue launches as fast as a small copy runs.) */
+int fx_copy_bytes_timed_sets(const void* const* src, void* const* dst, int n_sets, size_t bytes, int rounds, void* stream,
+                             float* ms_per_copy);
 
 #ifdef __cplusplus
 }

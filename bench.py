@@ -16,13 +16,19 @@ the scripted program whose fused regions run as tssa::ParallelFunctor;
 `compiled_kernels` says whether the regions ran ahead-of-time compiled kernels
 (functs_amd.aot) or the bytecode interpreter (`--interpreter` forces the latter);
 `per_config` repeats the measurement for every benchmark configuration that is
-implemented.  `roofline` prices the dominant kernel against the 8 TB/s
+implemented, each with its CPU baseline, the library's copy kernel on the same
+bytes, the operator's host time by section and, for row compactions (whose default
+is the kernel generated from the region's programs, fx_rs_kernel), the figures of
+the hand-written and the generic kernels and of the opt-in call forms (lazy_lists,
+padded_outputs); `head_variants`: other spellings of the detection head, each on its
+own generated kernel; `c5_nms_tail`: the compaction followed by the detection tail,
+also through the TorchScript route.  `roofline` prices the dominant kernel against the 8 TB/s
 HBM peak with the algorithmic bytes of the call; its duration is measured with
 HIP events on the launch stream around ten back-to-back launches of the kernel
 (mean per launch, `kernel_ms`; the reading of a pair around a single launch,
 which carries about 2 us of the pair itself, is `kernel_ms_single_launch`).
 `cpu_baseline` times the unfused TorchScript CPU path (the oracle) on a bounded
-sample.
+sample (`cpu_baseline_one_thread`: the same on one thread).
 """
 import argparse
 import json

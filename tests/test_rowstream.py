@@ -126,6 +126,12 @@ def test_regions_without_a_row_stream_form_say_why():
     r = configs.build_c3_classes(6)
     info = r.rowstream_info(torch.rand(40, 4), torch.rand(40, 7))
     assert info["ok"] and info["row_elements"] == 4
+    # ... and at the benchmark's size (80 tasks of 8 732 rows) the launch would need more workgroups
+    # than the device holds at once, which the skeleton counts on: the generic kernels keep it
+    r = configs.build_c3_classes(80)
+    big = r.rowstream_info(torch.rand(8732, 4), torch.rand(8732, 81))
+    assert big["ok"] and not big["active"]
+    assert r.rowstream_info(torch.rand(873, 4), torch.rand(873, 81))["active"]
     # a row of which less than half is read
     r = Region()
     x = r.tensor_input(torch.float32, 2)

@@ -182,7 +182,12 @@ std::vector<int64_t> keptCounts(const char* op, const Tensor& n, c10::Device dev
       __builtin_ia32_pause();
       if (clock::now() < next_query) continue;
       if (stream.query()) {
+        // drained and still pending: the launch ran on another stream than the current one, or not at all
         stream.synchronize();
+        if (pending()) {
+          const hipError_t e = hipDeviceSynchronize();
+          TORCH_CHECK(e == hipSuccess, op, ": hipDeviceSynchronize: ", hipGetErrorString(e));
+        }
         TORCH_CHECK(!pending(), op, ": the kept counts of a launch were never written");
         break;
       }

@@ -383,6 +383,7 @@ struct Variant {
   // the output block of the next call of a map, allocated while the last call's kernels ran
   at::Tensor next_block;
   void* next_stream = nullptr;
+  static constexpr int64_t kMaxPrepared = 512ll << 20;
   // likewise the output tensors of the next call of a single task (one per output, at full size)
   std::vector<at::Tensor> next_buffers;
   const fx_plan* next_buffers_plan = nullptr;
@@ -408,6 +409,7 @@ struct Variant {
     return at::empty({bytes}, at::TensorOptions().dtype(at::kByte).device(device));
   }
   void prepareBlock(int64_t bytes, c10::Device device, void* stream) {
+    if (bytes > kMaxPrepared) return;   // (what is prepared stays allocated between calls)
     at::Tensor b = at::empty({bytes}, at::TensorOptions().dtype(at::kByte).device(device));   // on the current stream
     std::lock_guard<std::mutex> lock(mu);
     next_block = std::move(b);
@@ -648,9 +650,13 @@ class RegionRunner {
       // the next call's block is allocated now, while this call's kernels run
       var->prepareBlock(std::max<int64_t>(layout->block_bytes, 1), device, (void*)stream.stream());
     } else {
-      std::vector<at::Tensor> next(n_out);
-      for (int o = 0; o < n_out; ++o) next[o] = newBuffer(o);
-      var->prepareBuffers(plan, (void*)stream.stream(), std::move(next));
+      int64_t bytes = 0;
+      for (int o = 0; o < n_out; ++o) bytes += layout->total[o] * layout->item[o];
+      if (bytes <= Variant::kMaxPrepared) {
+        std::vector<at::Tensor> next(n_out);
+        for (int o = 0; o < n_out; ++o) next[o] = newBuffer(o);
+        var->prepareBuffers(plan, (void*)stream.stream(), std::move(next));
+      }
     }
     clock.tick(HS_VIEWS);
     if (compact_) {

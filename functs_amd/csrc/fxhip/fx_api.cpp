@@ -433,7 +433,7 @@ int fx_plan_head_info(const fx_plan* p, int64_t* out, int cap) {
   out[7] = hi.n_tasks;
   return FX_OK;
 }
-void fx_set_rowstream(int on) { g_rs_mode.store(on ? 1 : 0, std::memory_order_relaxed); }
+void fx_set_rowstream(int on) { g_rs_mode.store(on == 2 ? 2 : (on ? 1 : 0), std::memory_order_relaxed); }
 int fx_rowstream_count(void) { return fx_rs_count(); }
 int fx_plan_rowstream_info(const fx_plan* p, int64_t* out, int cap) {
   if (!p || !out || cap < 8) return fail(FX_E_INVALID, "fx_plan_rowstream_info: out[>=8] required");
@@ -807,8 +807,9 @@ static const FxRsKernel* rs_of(const fx::Plan* pl) {
   // before it): a launch that needs more workgroups than the device holds, even with chunks of
   // FX_BLOCK rows, would spend its time in bounded waits and their fallback, and keeps the generic
   // two passes (80 tasks of 8 732 rows: 26.6 us that way against 7.9 + 15.1 us).
+  // (fx_set_rowstream(2) takes the kernel all the same: its bounded waits end every launch)
   const uint64_t chunks = ((uint64_t)pl->rs.n_rows + FX_BLOCK - 1) / FX_BLOCK;
-  if (chunks * pl->rs.n_tasks > (uint64_t)rs_compute_units() * FX_RS_OCC) return nullptr;
+  if (g_rs_mode.load(std::memory_order_relaxed) != 2 && chunks * pl->rs.n_tasks > (uint64_t)rs_compute_units() * FX_RS_OCC) return nullptr;
   const FxRsKernel* k = fx_rs_find(pl->rs.key);
   return (k && k->S == pl->rs.S) ? k : nullptr;
 }

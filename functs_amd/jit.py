@@ -38,7 +38,11 @@ class AotScriptFunction(object):
     def graph(self):
         return self._aot_script_fn.graph
 
-    def __call__(self, *args):
+    def __call__(self, *args, **kwargs):
+        if kwargs:   # by name: through the ScriptFunction, which knows the argument names
+            if self._variants is not None or self._lazy_lists:
+                raise TypeError("this built function takes positional arguments only")
+            return self._aot_script_fn(*args, **kwargs)
         if self._variants is None:
             return self._call(*args)
         key = _shape_key(args)

@@ -178,7 +178,7 @@ def test_data_dependent_predicates_and_other_dtypes_on_the_cpu():
 
 
 # ---- on the GPU ---------------------------------------------------------------------------------
-def _three_ways(r, *args):
+def _three_ways(r, *args, mode=1):
     """(generated kernel, generic two passes), both on the GPU; the generated kernel must be in use."""
     info = r.rowstream_info(*args)
     assert info["ok"] and info["active"], "no generated kernel linked for key %016x: run python -m functs_amd.aot --plan-only and rebuild" % info["key"]
@@ -191,7 +191,7 @@ def _three_ways(r, *args):
         assert lib.fx_plan_launches(r.plan(arr, n).handle) == 2
         two = run_region("hip", r, *args)
     finally:
-        lib.fx_set_rowstream(1)
+        lib.fx_set_rowstream(mode)
         lib.fx_set_head_kernel(1)
     return one, two
 
@@ -305,8 +305,19 @@ def test_predictions_that_start_at_an_odd_address_and_outputs_of_every_phase():
 @pytest.mark.gpu
 @pytest.mark.parametrize("n,batch", [(100000, None), (60000, 16)])
 def test_launches_beyond_what_the_device_holds_at_once(n, batch):
+    """By default such a launch keeps the two passes (the skeleton counts on all workgroups being
+    resident); forced onto the generated kernel it still ends and gives the same rows: chunks
+    whose predecessors have not started give up their bounded wait and count for themselves."""
     args = _inputs(n, 80, batch or 1, seed=3)
-    one, two = _three_ways(_build("stack", batch), *args)
+    r = _build("stack", batch)
+    info = r.rowstream_info(*args)
+    beyond = -(-n // 256) * (batch or 1) > 256 * 6      # chunks of 256 rows against six workgroups on each of 256 CUs
+    assert info["ok"] and info["active"] == (not beyond)
+    lib.fx_set_rowstream(2)
+    try:
+        one, two = _three_ways(r, *args, mode=2)
+    finally:
+        lib.fx_set_rowstream(1)
     assert_exact(_flat(one), _flat(two), "n=%d batch=%s" % (n, batch))
 
 

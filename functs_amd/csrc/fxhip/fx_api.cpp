@@ -827,8 +827,8 @@ static uint32_t rs_env(const char* name) {   // tuning aids: 0 when not set
   const char* e = getenv(name);
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
 }
-static uint32_t rs_max_sub_rows(const FxRsInfo& ri) {
-  return std::min<uint32_t>(FX_RS_SUB, (FX_RS_KV * FX_BLOCK * 4u - 6u) / ri.S);
+static uint32_t rs_max_sub_rows(const FxRsInfo& ri, uint32_t kv = FX_RS_KV) {
+  return std::min<uint32_t>(FX_RS_SUB, (kv * FX_BLOCK * 4u - 6u) / ri.S);
 }
 // the window, then the staged outputs (fx_rowstream.h lays them out the same way)
 // window, staged outputs, and the chunk's table of side values
@@ -876,55 +876,67 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     const uint32_t min_chunk = std::min<uint32_t>(FX_RS_MIN_CHUNK, std::max<uint32_t>(ri.n_rows, 1u));
     const uint32_t forced_sub = rs_env("FXHIP_RS_SUB_ROWS"), forced_chunk = rs_env("FXHIP_RS_CHUNK_ROWS");
     uint32_t best_sub = 0, best_cr = 0, best_n = 0;
-    bool best_side = false;
-    // with the chunk's table of side values in LDS, and without it (where the table would cost a
-    // workgroup per CU or a sub-tile per chunk, the rows load their side values themselves)
-    for (int with_side = kern->side_row_words != 0 ? 1 : 0; with_side >= 0; --with_side) {
-      for (uint32_t sub = rs_max_sub_rows(ri); sub >= 8u; sub = sub > 8u ? std::max<uint32_t>(8u, sub - 8u) : 0u) {
-        if (forced_sub && sub > forced_sub) continue;
-        // at most the occupancy the kernels are compiled for: a launch that needs a seventh slot per CU
-        // (kernels that happen to stay below 73 registers) is not placed at once and takes 27.4 us
-        // where six per CU take 23.4 us
-        auto slots = [&](uint32_t chunk_rows) {
-          int n = 0;
-          if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern->fn, (int)FX_BLOCK,
-                                                           (size_t)rs_lds_bytes(ri, kern, sub, chunk_rows, with_side != 0)) != hipSuccess) {
-            (void)hipGetLastError();
-            return 0;
+    bool best_side = false, best_lean = false;
+    // The kernel built for five loads per lane and sub-tile first (fewer registers), the one for six
+    // where it saves a sub-tile per chunk; with the chunk's table of side values in LDS, and without
+    // it where the table would cost a workgroup per CU or a sub-tile per chunk (the rows then load
+    // their side values themselves).  Fewest sub-tiles per chunk wins, the first found among equals.
+    const uint32_t forced_loads = rs_env("FXHIP_RS_LOADS");   // tuning aid: FX_RS_KV or FX_RS_KV_LEAN
+    for (int lean = 1; lean >= 0; --lean) {
+      const void* fn = lean ? kern->fn_lean : kern->fn;
+      if (!fn || (forced_loads && forced_loads != (lean ? FX_RS_KV_LEAN : FX_RS_KV))) continue;
+      // (measured on the benchmark's shape: 22.6 against 22.95 us for kernels that store as they
+      // compute; with outputs staged in LDS, where LDS and not registers bounds the occupancy, 25.6 against 24.4)
+      if (lean && kern->n_staged != 0 && !forced_loads) continue;
+      const uint32_t max_sub = rs_max_sub_rows(ri, lean ? FX_RS_KV_LEAN : FX_RS_KV);
+      if (max_sub < 8u) continue;
+      for (int with_side = kern->side_row_words != 0 ? 1 : 0; with_side >= 0; --with_side) {
+        for (uint32_t sub = max_sub; sub >= 8u; sub = sub > 8u ? std::max<uint32_t>(8u, sub - 4u) : 0u) {
+          if (forced_sub && sub > forced_sub) continue;
+          // at most the occupancy the kernels are compiled for: a launch that needs a seventh slot per CU
+          // is not placed at once and takes 27.4 us where six per CU take 23.4 us
+          auto slots = [&](uint32_t chunk_rows) {
+            int n = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, (int)FX_BLOCK,
+                                                             (size_t)rs_lds_bytes(ri, kern, sub, chunk_rows, with_side != 0)) != hipSuccess) {
+              (void)hipGetLastError();
+              return 0;
+            }
+            return std::min(n, (int)FX_RS_OCC);
+          };
+          auto chunkFor = [&](int per_cu) {
+            const uint32_t resident = (uint32_t)per_cu * (uint32_t)std::max(cus, 1);
+            const uint32_t per_task = std::max<uint32_t>(1u, resident / std::max<uint32_t>(ri.n_tasks, 1u));
+            uint32_t c = (ri.n_rows + per_task - 1) / per_task;
+            c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(c, min_chunk));
+            if (forced_chunk) c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(forced_chunk, min_chunk));
+            return c;
+          };
+          // the table is part of the LDS, and the chunk follows from the number of resident
+          // workgroups: from the largest chunk down until both agree
+          int per_cu = slots(FX_BLOCK);
+          if (per_cu < 1) continue;
+          uint32_t cr = chunkFor(per_cu);
+          for (int round = 0; round < 3; ++round) {
+            const int better = slots(cr);
+            if (better <= per_cu) break;
+            per_cu = better;
+            cr = chunkFor(per_cu);
           }
-          return std::min(n, (int)FX_RS_OCC);
-        };
-        auto chunkFor = [&](int per_cu) {
-          const uint32_t resident = (uint32_t)per_cu * (uint32_t)std::max(cus, 1);
-          const uint32_t per_task = std::max<uint32_t>(1u, resident / std::max<uint32_t>(ri.n_tasks, 1u));
-          uint32_t c = (ri.n_rows + per_task - 1) / per_task;
-          c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(c, min_chunk));
-          if (forced_chunk) c = std::min<uint32_t>(FX_BLOCK, std::max<uint32_t>(forced_chunk, min_chunk));
-          return c;
-        };
-        // the table is part of the LDS, and the chunk follows from the number of resident
-        // workgroups: from the largest chunk down until both agree
-        int per_cu = slots(FX_BLOCK);
-        if (per_cu < 1) continue;
-        uint32_t cr = chunkFor(per_cu);
-        for (int round = 0; round < 3; ++round) {
-          const int better = slots(cr);
-          if (better <= per_cu) break;
-          per_cu = better;
-          cr = chunkFor(per_cu);
+          const uint32_t n = (cr + sub - 1) / sub;
+          if (rs_env("FXHIP_RS_VERBOSE"))
+            fprintf(stderr, "[fxhip] row-stream geometry: %u loads, side table %d, sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
+                    lean ? FX_RS_KV_LEAN : FX_RS_KV, with_side, sub, rs_lds_bytes(ri, kern, sub, cr, with_side != 0), per_cu, cr, n);
+          if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; best_side = with_side != 0; best_lean = lean != 0; }
+          if (forced_sub || sub == 8u) break;
         }
-        const uint32_t n = (cr + sub - 1) / sub;
-        if (rs_env("FXHIP_RS_VERBOSE"))
-          fprintf(stderr, "[fxhip] row-stream geometry: side table %d, sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
-                  with_side, sub, rs_lds_bytes(ri, kern, sub, cr, with_side != 0), per_cu, cr, n);
-        if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; best_side = with_side != 0; }
-        if (forced_sub || sub == 8u) break;
       }
     }
     if (best_sub == 0) return fail(FX_E_LIMIT, "row-stream kernel: no sub-tile size fits the device");
     pl->rs_sub_rows = best_sub;
     pl->rs_chunk_rows = best_cr;
     pl->rs_side_lds = best_side ? 1u : 0u;
+    pl->rs_lean = best_lean ? 1u : 0u;
   }
   rl->sub_rows = pl->rs_sub_rows;
   rl->chunk_rows = pl->rs_chunk_rows;
@@ -935,13 +947,16 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
   // the counts get a head start.  A small launch would only lose the time.
   const uint64_t first_bytes = (uint64_t)rl->chunks * ri.n_tasks * std::min<uint32_t>(cr, rl->sub_rows) * ri.S * 4u;
   rl->bulk_delay = first_bytes >= FX_RS_FLOOD_BYTES ? FX_RS_BULK_DELAY : 0u;
+  if (const uint32_t d = rs_env("FXHIP_RS_BULK_DELAY")) rl->bulk_delay = d - 1u;   // tuning aids (value + 1; FXHIP_RS_LATE_TELL=1)
+  rl->late_tell = rs_env("FXHIP_RS_LATE_TELL") ? 1u : 0u;
   return FX_OK;
 }
-static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const FxRsLaunch& rl, const FxDyn* dyn, hipStream_t stream) {
+static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const FxRsLaunch& rl, const FxDyn* dyn, hipStream_t stream,
+                            bool lean) {
   const uint32_t grid = rl.chunks * rl.n_tasks;
   if (grid == 0) return hipSuccess;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
+  return hipLaunchKernel(lean && kern->fn_lean ? kern->fn_lean : kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----
@@ -1110,7 +1125,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
       rl.epoch = epoch + (uint32_t)r;
-      HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn, stream));
+      HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn, stream, pl->rs_lean != 0));
     }
     HIP_OK(mark(1));
     nk = rl.chunks * rl.n_tasks > 0 ? 1 : 0;
@@ -1254,7 +1269,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
       } else if (rsk) {
         rl.epoch = epoch + (uint32_t)(r * n_sets + i);
         rl.totals = totals_host[i];
-        HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn[i], stream));
+        HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn[i], stream, pl->rs_lean != 0));
       } else if (head) {
         hl.epoch = epoch + (uint32_t)(r * n_sets + i);
         hl.totals = totals_host[i];

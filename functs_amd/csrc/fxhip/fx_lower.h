@@ -134,7 +134,7 @@ struct Plan {
   std::vector<Status> head_status;
   uint32_t head_resident = 0;
   uint32_t cmap_resident_wide = 0;   // class-map head kernel: workgroups of its wide form
-  uint32_t rs_side_lds = 0, rs_sub_rows = 0, rs_chunk_rows = 0;   // row-stream kernel: geometry of a launch (chosen at the first one)
+  uint32_t rs_lean = 0, rs_side_lds = 0, rs_sub_rows = 0, rs_chunk_rows = 0;   // row-stream kernel: geometry of a launch (chosen at the first one)
 };
 
 // Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?

@@ -154,9 +154,9 @@ FX_RS_FN void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_
 #include "fx_rs_ops.h"
 namespace {
 
-template <class P>
+template <class P, uint32_t KV>
 __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
-  constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, KV = FX_RS_KV, NSUB = FX_RS_NSUB, S = P::S;
+  constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, NSUB = FX_RS_NSUB, S = P::S;
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];   // the window: sub_rows rows of S elements
   __shared__ uint32_t s_rowmap[FX_RS_SUB];
   __shared__ uint8_t s_keep[FX_BLOCK];
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     for (uint32_t k = 0; k < KV; ++k)
       if (k * NT + wave * 64u < n_vec_u) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
   };
-  const bool teller = chunk + 1u == la.chunks;   // the task's last chunk tells the host the task's total
+  const bool teller = chunk + 1u == la.chunks && la.late_tell == 0u;   // the task's last chunk tells the host the task's total
   uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
   // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
   auto look_back = [&]() {
@@ -386,9 +386,11 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
 }
 
 struct FxRsRegistrar {
-  FxRsRegistrar(uint64_t key, const void* fn, uint32_t S, uint32_t stage_row_words, uint32_t n_staged, uint32_t side_row_words) {
+  FxRsRegistrar(uint64_t key, const void* fn, const void* fn_lean, uint32_t S, uint32_t stage_row_words, uint32_t n_staged,
+                uint32_t side_row_words) {
     FxRsKernel k;
     k.fn = fn;
+    k.fn_lean = fn_lean;
     k.S = S;
     k.stage_row_words = stage_row_words;
     k.n_staged = n_staged;
@@ -400,5 +402,6 @@ struct FxRsRegistrar {
 }  // namespace
 
 #define FX_RS_REGISTER(P) \
-  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P>, P::S, P::stage_row_words, P::n_staged, \
+  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P, FX_RS_KV>,                                \
+                                           (const void*)&fx_rs_kernel<P, FX_RS_KV_LEAN>, P::S, P::stage_row_words, P::n_staged, \
                                            (P::n_row_cols != 0u && P::n_side <= FX_RS_MAX_SIDE) ? P::n_side : 0u);

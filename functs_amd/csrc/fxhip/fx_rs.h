@@ -30,7 +30,9 @@
 #define FX_RS_MAX_FIMM 24u      // distinct floating-point constants
 #define FX_RS_SUB 64u           // most rows of a sub-tile (one ballot)
 #define FX_RS_NSUB 4u           // most sub-tiles of a chunk: a chunk holds at most FX_BLOCK rows
-#define FX_RS_KV 6u             // 128-bit loads per lane that carry a sub-tile
+#define FX_RS_KV 6u             // most 128-bit loads per lane that carry a sub-tile
+#define FX_RS_KV_LEAN 5u        // every kernel is also built for five (four registers less: 70 instead of 77 on the
+                                // benchmark's region, 22.5 against 23.2 us); the host takes it where it costs no sub-tile
 #define FX_RS_STATUS_BITS 9u    // a chunk's count is at most FX_BLOCK
 #define FX_RS_MIN_CHUNK 64u     // fewest rows of a chunk unless a task has fewer
 #define FX_RS_FLOOD_BYTES (8u << 20)   // first sub-tiles of a launch from which on the counts are sent ahead of the rows
@@ -72,6 +74,8 @@ struct FxRsLaunch {
   uint32_t fimm[FX_RS_MAX_FIMM];
   uint32_t slot_err;
   uint32_t side_lds;            // the chunk keeps a table of its rows' side values in LDS (0: a row loads them when its turn comes)
+  uint32_t late_tell;           // tuning aid: the task's last chunk looks back where the others do (the host hears the total later)
+  uint32_t pad0;
   uint32_t* status;             // one word per chunk, tagged with the epoch
   uint32_t* totals;             // pinned host memory: kept rows per task
 };
@@ -79,7 +83,8 @@ static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte
 
 // ---- host side: generated kernels linked into the library ----
 struct FxRsKernel {
-  const void* fn = nullptr;     // fx_rs_kernel<P>
+  const void* fn = nullptr;     // fx_rs_kernel<P, FX_RS_KV>
+  const void* fn_lean = nullptr; // fx_rs_kernel<P, FX_RS_KV_LEAN>
   uint32_t S = 0;               // row length the kernel is generated for
   uint32_t stage_row_words = 0; // elements per kept row that the kernel puts together in LDS before they leave
   uint32_t n_staged = 0;        // outputs that take that route

@@ -162,6 +162,8 @@ _sig("fx_plan_specialized", _i, _vp)
 _sig("fx_plan_spec_source", _i, _vp, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t)
 _sig("fx_set_specialization", None, _i)
 _sig("fx_specialization_count", _i)
+_sig("fx_plan_dense_lean", _i, _vp)
+_sig("fx_set_dense_lean", None, _i)
 _sig("fx_spec_dump_dir", _i, ctypes.c_char_p)
 _sig("fx_spec_dump_what", _i, _i)
 _sig("fx_region_wait_totals", _i, _vp, _vp, _vp)

@@ -26,7 +26,7 @@ struct FxSpecKernels;
 const FxSpecKernels* fx_spec_find(uint64_t hash);
 int fx_spec_count();
 hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
-                           hipStream_t stream, const FxSpecKernels* spec);
+                           hipStream_t stream, const FxSpecKernels* spec, const FxLeanArgs* lean, uint32_t slot_err);
 hipError_t fx_launch_compact_count(const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
                                    hipStream_t stream, const FxSpecKernels* spec);
 hipError_t fx_launch_compact_scatter(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn,
@@ -36,6 +36,7 @@ hipError_t fx_launch_compact_stream(int rank, const uint32_t* sb, const FxLaunch
                                     hipStream_t stream, const FxSpecKernels* spec);
 uint32_t fx_stream_lds_bytes(const FxLaunchInfo& li, bool compiled);
 bool fx_spec_has_stream(const FxSpecKernels* spec);
+bool fx_spec_has_lean(const FxSpecKernels* spec);
 // fx_head.hip
 hipError_t fx_launch_head_stream(const FxHeadLaunch& hl, const FxDyn* dyn, hipStream_t stream);
 hipError_t fx_head_resident(uint32_t lds_bytes, uint32_t* workgroups, uint32_t* per_cu);
@@ -640,6 +641,22 @@ size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
 #define FX_STREAM_LDS_LIMIT 64000u   // 64 KiB less the kernel's static tables
 #define FX_EPOCH_MAX ((1u << 23) - 1u)
 
+// Lean dense kernel (fx_spec.h): on unless switched off (tests compare it with the general kernel).
+static std::atomic<int> g_dense_lean{[] {
+  const char* e = getenv("FXHIP_DENSE_LEAN");
+  return (e && e[0] == '0') ? 0 : 1;
+}()};
+static const FxLeanArgs* lean_of(const fx::Plan* pl) {
+  return g_dense_lean.load(std::memory_order_relaxed) ? &pl->lean : nullptr;
+}
+
+int fx_plan_dense_lean(const fx_plan* p) {
+  if (!p) return 0;
+  const fx::Plan* pl = P(p);
+  return (pl->mode == FX_MODE_DENSE && lean_of(pl) && pl->lean.n_outs != 0 && fx_spec_has_lean(spec_of(pl))) ? 1 : 0;
+}
+void fx_set_dense_lean(int on) { g_dense_lean.store(on ? 1 : 0, std::memory_order_relaxed); }
+
 static FxLaunchInfo launch_info(const fx::Plan* pl) {
   const fx::Region& R = *pl->region;
   FxLaunchInfo li;
@@ -1118,7 +1135,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     HIP_OK(mark(0));
     // persistent workgroups: at most FX_DENSE_WG_PER_CU per CU worth of blocks stride over the units
     for (int r = 0; r < repeat; ++r)
-      HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+      HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn, std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec, lean_of(pl), pl->lean_slot_err));
     HIP_OK(mark(1));
     nk = pl->grid > 0 ? 1 : 0;
   } else if (rsk) {
@@ -1265,7 +1282,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   for (int r = 0; r < rounds; ++r)
     for (int i = 0; i < n_sets; ++i) {
       if (!compact) {
-        HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec));
+        HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec, lean_of(pl), pl->lean_slot_err));
       } else if (rsk) {
         rl.epoch = epoch + (uint32_t)(r * n_sets + i);
         rl.totals = totals_host[i];

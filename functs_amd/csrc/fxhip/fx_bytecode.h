@@ -13,6 +13,7 @@
 // arithmetic of its lowerings (functs/csrc/jit/tensorexpr/nnc_ext.cpp:62-392,
 // fait/fuser/custom_lowering_func.cpp:17-498).
 #pragma once
+#include <stddef.h>
 #include <stdint.h>
 
 #define FX_MAXR 6        // max rank of a region output (root coordinates)
@@ -245,6 +246,47 @@ struct FxHeader {
   uint32_t slot_status;  // streaming compaction: shared pointer slot of the tile status words
   uint32_t pad[1];
 };
+
+// Dense regions with ONE task class of one or two outputs per task (the usual case) whose
+// programs are compiled: the lean dense kernel (fx_dense_lean in fx_spec.h) takes what a
+// workgroup needs in front of its first load from a short argument block, copied out of the
+// descriptor at plan time, and stages the descriptor only if a program reads it.  A kernel start
+// costs a trip to the argument segment per line of it that is read and per level of dependent
+// reads, and about as much again per jump to code that has not been fetched yet, so the block is
+// small, read in one go, and the kernel short; regions that do not fit take the general kernel.
+#define FX_FAST_OUTS 2
+#define FX_LEAN_P 24     // pointers and
+#define FX_LEAN_S 16     // scalars of a region that the lean kernel's argument block holds
+// One output of the region: the fields of FxOut that place a work item, the leading load's
+// affine map, and the two buffers.  160 bytes, laid out so that a kernel for rank <= 3 reads the
+// first 128 only; the records start at a multiple of 64 bytes in the argument segment.
+struct FxLeanOut {
+  uint64_t out_ptr;             // the output's buffer and the leading load's, resolved at launch when
+  uint64_t lead_ptr;            // they do not change with the task (0: look the slot up in p[])
+  uint32_t ptr_slot, lead_slot; // may carry FX_SLOT_TASK
+  uint32_t lead;                // as FxOut::lead
+  uint32_t block_begin, task_stride, unit_items, inner, vd, gpr, gp_magic, gp_shift, n_groups;   // as in FxOut
+  int32_t lead_base, lead_tcoef;
+  int32_t lead_cf[FX_MAXR];
+  uint32_t dms[FX_MAXR - 1][3]; // FxOut::dim, magic, shift of dimensions 1 .. FX_MAXR - 1
+  uint32_t pad;
+};
+struct FxLeanArgs {
+  uint32_t blob_words, n_p, n_s, total_units;   // as in FxLaunchInfo
+  uint32_t n_outs;              // 0: the region does not fit the lean kernel
+  uint32_t bpt;                 // work units per task, and the division by it
+  uint32_t bpt_magic, bpt_shift;
+  uint32_t n_sptr, n_tptr;
+  uint32_t cls_off;             // word offset of the class record in the descriptor
+  uint32_t second_begin;        // first unit of a task that belongs to the second output
+  uint64_t err_ptr;             // the error word of guarded loads (0: none), resolved at launch
+  struct FxLeanOut out[FX_FAST_OUTS];
+  uint64_t p[FX_LEAN_P];        // the first n_p words of FxDyn::p
+  uint32_t s[FX_LEAN_S];        // the first n_s words of FxDyn::s
+};
+#ifdef __cplusplus
+static_assert(sizeof(FxLeanOut) == 160 && offsetof(FxLeanArgs, out) == 56, "the records of FxLeanArgs start on a line of the argument segment (behind the 8-byte descriptor pointer)");
+#endif
 
 // dynamic (per call) arguments, passed by value in the kernarg segment
 struct FxDyn {

@@ -26,6 +26,7 @@
 // fait/tensorexpr/functor_parallization.cpp:93-108) and, for the
 // data-dependent part, the ATen nonzero/index calls the reference leaves
 // unfused (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
+#include <cstring>
 #include "fx_spec.h"
 
 #include <mutex>
@@ -218,6 +219,7 @@ const FxSpecKernels* fx_spec_find(uint64_t hash) {
   return it == spec_table().end() ? nullptr : &it->second;   // entries are never erased
 }
 bool fx_spec_has_stream(const FxSpecKernels* spec) { return spec && spec->stream != nullptr; }
+bool fx_spec_has_lean(const FxSpecKernels* spec) { return spec && spec->lean != nullptr; }
 int fx_spec_count() {
   std::lock_guard<std::mutex> g(spec_mutex());
   return (int)spec_table().size();
@@ -299,8 +301,23 @@ static hipError_t allow_lds(K kernel, uint32_t bytes) {
   } while (0)
 
 hipError_t fx_launch_dense(int rank, const uint32_t* sb, const FxLaunchInfo& li, const FxDyn* dyn, uint32_t grid,
-                           hipStream_t stream, const FxSpecKernels* spec) {
+                           hipStream_t stream, const FxSpecKernels* spec, const FxLeanArgs* lean, uint32_t slot_err) {
   if (grid == 0) return hipSuccess;
+  if (spec && spec->lean && lean && lean->n_outs != 0) {
+    // the lean kernel: a short argument block instead of FxLaunch + FxDyn
+    FxLeanArgs a = *lean;
+    a.err_ptr = slot_err ? dyn->p[slot_err - 1u] : 0;
+    for (uint32_t o = 0; o < a.n_outs; ++o) {
+      FxLeanOut& lo = a.out[o];
+      lo.out_ptr = (lo.ptr_slot & FX_SLOT_TASK) ? 0 : dyn->p[lo.ptr_slot & 0xffffu];
+      lo.lead_ptr = (!lo.lead || (lo.lead_slot & FX_SLOT_TASK)) ? 0 : dyn->p[lo.lead_slot & 0xffffu];
+    }
+    memcpy(a.p, dyn->p, sizeof(uint64_t) * a.n_p);
+    memcpy(a.s, dyn->s, sizeof(uint32_t) * a.n_s);
+    void* args[2] = {(void*)&sb, (void*)&a};
+    return hipLaunchKernel(spec->lean, dim3(grid), dim3(FX_BLOCK), args, spec->lean_stages ? lds_bytes_compiled(li) : 0u,
+                           stream);
+  }
   const FxLaunch la = make_launch(li);
   const uint32_t lds = fx_lds_bytes(li);
   if (spec && spec->dense) return launch_spec(spec->dense, sb, la, dyn, grid, lds_bytes_compiled(li), stream);

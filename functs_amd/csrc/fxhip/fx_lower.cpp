@@ -2254,6 +2254,64 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   hp->off_taskmap = off_taskmap;
   hp->total_words = (uint32_t)blob.size();
 
+  // One class of at most FX_FAST_OUTS outputs of 32-bit elements, none of them reduced over
+  // rows, tasks numbered in order, few enough pointers and scalars: the region fits the lean
+  // dense kernel's argument block (the kernel itself exists only for compiled programs).
+  memset(&P->lean, 0, sizeof(P->lean));
+  if (P->mode == FX_MODE_DENSE && classes.size() == 1 && !classes[0].outs.empty() &&
+      classes[0].outs.size() <= FX_FAST_OUTS && P->grid > 0 &&
+      P->sptr.size() + P->tptr.size() * (size_t)T <= FX_LEAN_P &&
+      P->sscal.size() + P->tscal.size() * (size_t)T <= FX_LEAN_S) {
+    const ClassBuild& cb = classes[0];
+    bool fits = taskmap.size() == (size_t)T;
+    for (size_t i = 0; fits && i < taskmap.size(); ++i) fits = taskmap[i] == (uint32_t)i;
+    for (const FxOut& od : cb.outs)
+      fits = fits && !od.rowwave &&
+             ((od.dtype == FX_F32 && od.vt == FX_VT_F) || (od.dtype == FX_I32 && od.vt == FX_VT_I));
+    if (fits) {
+      FxLeanArgs& f = P->lean;
+      f.blob_words = (uint32_t)blob.size();
+      f.n_p = (uint32_t)(P->sptr.size() + P->tptr.size() * (size_t)T);
+      f.n_s = (uint32_t)(P->sscal.size() + P->tscal.size() * (size_t)T);
+      f.total_units = P->grid;
+      f.n_outs = (uint32_t)cb.outs.size();
+      f.bpt = cb.cls.blocks_per_task;
+      fx_fastdiv_make(f.bpt, &f.bpt_magic, &f.bpt_shift);
+      f.n_sptr = h.n_sptr;
+      f.n_tptr = h.n_tptr;
+      f.cls_off = off_class;
+      f.second_begin = cb.outs.size() > 1 ? cb.outs[1].block_begin : 0xffffffffu;
+      P->lean_slot_err = h.slot_err;
+      for (size_t o = 0; o < cb.outs.size(); ++o) {
+        const FxOut& od = cb.outs[o];
+        FxLeanOut& lo = f.out[o];
+        lo.ptr_slot = od.ptr_slot;
+        lo.lead = od.lead;
+        lo.block_begin = od.block_begin;
+        lo.task_stride = od.task_stride;
+        lo.unit_items = od.unit_items;
+        lo.inner = od.inner;
+        lo.vd = od.vd;
+        lo.gpr = od.gpr;
+        lo.gp_magic = od.gp_magic;
+        lo.gp_shift = od.gp_shift;
+        lo.n_groups = od.n_groups;
+        for (int k = 1; k < FX_MAXR; ++k) {
+          lo.dms[k - 1][0] = od.dim[k];
+          lo.dms[k - 1][1] = od.magic[k];
+          lo.dms[k - 1][2] = od.shift[k];
+        }
+        if (!od.lead) continue;
+        const FxInsn& li = cb.code[od.prog_begin];
+        const FxAffine& af = cb.affs[(size_t)li.b];
+        for (int k = 0; k < FX_MAXR; ++k) lo.lead_cf[k] = fx_aff_coef(&af, k);
+        lo.lead_base = af.base;
+        lo.lead_tcoef = af.tcoef;
+        lo.lead_slot = (uint32_t)li.a;
+      }
+    }
+  }
+
   P->lds_bytes = (uint32_t)((blob.size() + 2 * (P->sptr.size() + P->tptr.size() * (size_t)T) +
                              (P->sscal.size() + P->tscal.size() * (size_t)T) + 4 +
                              (size_t)max_temps * FX_V * FX_BLOCK) * 4);

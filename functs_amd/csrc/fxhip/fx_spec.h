@@ -35,6 +35,8 @@ struct FxSpecKernels {
   const void* scatter = nullptr;  // fx_compact_scatter<R, FxSpec<P>>
   uint32_t scatter_threads = 0;   // workgroup size that kernel is compiled for
   const void* stream = nullptr;   // fx_compact_stream<R, FxSpec<P>>
+  const void* lean = nullptr;     // fx_dense_lean<R, P>: dense regions that fit FxLeanArgs
+  bool lean_stages = false;       // ... and whether it stages the descriptor into LDS (a program reads it)
 };
 void fx_spec_register(uint64_t hash, const FxSpecKernels& k);
 const FxSpecKernels* fx_spec_find(uint64_t hash);
@@ -372,10 +374,225 @@ struct FxSpec {
   }
 };
 
+// ---- the lean dense kernel -------------------------------------------------
+// fx_region_dense serves every dense region and every element type, and compiled for one
+// program it is still tens of kilobytes of code that a workgroup jumps through: on a small
+// region the kernel's time is the start of its workgroups (argument segment, descriptor
+// staging, instruction fetch), not the data.  Regions of one task class with one or two
+// outputs of 32-bit elements and no row reductions (FxLeanArgs, decided at plan time) run this
+// kernel instead: unit, output record, leading load and pointers come from a short argument
+// block through scalar loads, the leading loads of the unit are issued first, and the
+// descriptor is staged into LDS behind them, and only if a program of the region reads it
+// (affine maps of further loads, scalars).  Results are those of fx_region_dense bit for bit:
+// the same item geometry, the same fx_step / fx_pure_step.
+#define FX_AS4 __attribute__((address_space(4)))
+
+template <class P>
+constexpr bool fx_spec_reads_descriptor() {
+  for (int e = 0; e < P::n_entries; ++e)
+    if (P::entries[e].kind == 0 && P::entries[e].pure == 0) return true;
+  return false;
+}
+
+template <class P, int R, int E, class GETCX>
+__device__ __forceinline__ void fx_lean_out(const FX_AS4 uint32_t* od, const uint32_t task, const uint32_t local_block,
+                                            const FX_AS4 uint64_t* gp, const uint32_t tp_off, const uint64_t err,
+                                            GETCX&& get_cx, const uint32_t lane, const uint32_t wave) {
+  constexpr FxSpecEntry en = P::entries[E];
+  static_assert(en.kind == 0, "dense regions have output programs only");
+  constexpr FxInsn LI = P::code[en.begin > 0 ? en.begin - 1 : 0];   // the leading load, if the output has one
+  const bool lead = en.begin > 0 && LI.op == FX_LDA && od[FX_W(FxLeanOut, lead)] != 0;
+  // a buffer that does not change with the task was resolved by the host; else its slot is looked up
+  auto arg_ptr = [&](uint32_t word, uint32_t slot) -> uint64_t {
+    if (slot & FX_SLOT_TASK) return gp[tp_off + (slot & 0xffffu)];
+    return ((uint64_t)od[word + 1] << 32) | od[word];
+  };
+  const uint64_t op = arg_ptr(FX_W(FxLeanOut, out_ptr), od[FX_W(FxLeanOut, ptr_slot)]);
+  FxLead ld;
+#pragma unroll
+  for (int k = 0; k < FX_MAXR; ++k) ld.cf[k] = k < (R > 4 ? FX_MAXR : 4) ? (int32_t)od[FX_W(FxLeanOut, lead_cf) + k] : 0;
+  ld.base = (int32_t)od[FX_W(FxLeanOut, lead_base)] + (int32_t)od[FX_W(FxLeanOut, lead_tcoef)] * (int32_t)task;
+  ld.p = arg_ptr(FX_W(FxLeanOut, lead_ptr), od[FX_W(FxLeanOut, lead_slot)]);
+  ld.err = err;
+  ld.dt = LI.dt;
+  ld.cvt = (LI.flags & FX_F_I2F) != 0;
+  ld.lds = false;
+  ld.win = nullptr;
+  ld.win_base = 0;
+
+  const uint32_t ublock = local_block - od[FX_W(FxLeanOut, block_begin)];
+  const uint32_t obase = od[FX_W(FxLeanOut, task_stride)] * task;
+  uint32_t dk[R], mk[R], sk[R];
+  dk[0] = mk[0] = sk[0] = 0;
+#pragma unroll
+  for (int k = 1; k < R; ++k) {
+    dk[k] = od[FX_W(FxLeanOut, dms) + 3 * (k - 1)];
+    mk[k] = od[FX_W(FxLeanOut, dms) + 3 * (k - 1) + 1];
+    sk[k] = od[FX_W(FxLeanOut, dms) + 3 * (k - 1) + 2];
+  }
+  const uint32_t kmax = od[FX_W(FxLeanOut, unit_items)];   // 1 or FX_K items per wave and unit
+  const uint32_t inner = od[FX_W(FxLeanOut, inner)];
+  const uint32_t vd = od[FX_W(FxLeanOut, vd)];
+  const uint32_t gpr = od[FX_W(FxLeanOut, gpr)];
+  const uint32_t gp_magic = od[FX_W(FxLeanOut, gp_magic)], gp_shift = od[FX_W(FxLeanOut, gp_shift)];
+  const uint32_t n_groups = od[FX_W(FxLeanOut, n_groups)];
+  const uint32_t item0 = ublock * (4u * kmax) + wave * kmax;
+  const uint32_t n_items = (n_groups + 63u) / 64u;
+  const bool have = item0 < n_items;
+
+  // item k of this wave: 64 lane groups of FX_V consecutive elements along the last dimension
+  auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) {
+    const uint32_t g = (item0 + k) * 64u + lane;
+    const bool live = g < n_groups;
+    const uint32_t gg = live ? g : 0u;
+    const uint32_t row = fx_fastdiv(gg, gp_magic, gp_shift);
+    const uint32_t col0 = (gg - row * gpr) * FX_V;
+    M = 0;
+#pragma unroll
+    for (int j = 0; j < FX_V; ++j) {
+      if (live && col0 + j < inner) M |= 1u << j;
+      q.cv[j] = (int32_t)(col0 + j);
+      e[j] = row * inner + col0 + j;
+    }
+    q.vd = vd;
+    q.step = 1;
+    const uint32_t rem = fx_unflatten<R>(row, vd, dk, mk, sk, q.c0);
+    q.c0[0] = vd == 0 ? 0 : (int32_t)rem;
+  };
+
+  uint32_t A[FX_K][FX_V];
+  if (have && lead) {
+#pragma unroll
+    for (uint32_t k = 0; k < FX_K; ++k) {
+      if (k < kmax && item0 + k < n_items) {
+        uint32_t e[FX_V], M;
+        FxCoord<R> q;
+        make_item(k, e, M, q);
+        fx_lead_load<R>(ld, q, M, A[k]);
+      }
+    }
+  }
+  // every wave of the workgroup comes by here, with or without items: the staging has a barrier
+  FxCtx cx = get_cx();
+  if (!have) return;
+  if constexpr (en.pure != 0) {
+#pragma unroll
+    for (uint32_t k = 0; k < FX_K; ++k) {
+      if (k < kmax && item0 + k < n_items) {
+        uint32_t e[FX_V], M;
+        FxCoord<R> q;
+        make_item(k, e, M, q);
+        fx_spec_pure<P, en.begin, en.end, FX_V>(A[k]);
+        fx_store_vec(op, obase, e, M, true, FX_F32, FX_VT_F, A[k]);
+      }
+    }
+  } else {
+    // one copy of the program: the loop stays rolled, the preloaded values are picked by selects
+#pragma unroll 1
+    for (uint32_t k = 0; k < FX_K; ++k) {
+      if (k < kmax && item0 + k < n_items) {
+        uint32_t e[FX_V], M;
+        FxCoord<R> q;
+        make_item(k, e, M, q);
+        uint32_t B[FX_V];
+#pragma unroll
+        for (int j = 0; j < FX_V; ++j) {
+          uint32_t v = A[0][j];
+#pragma unroll
+          for (uint32_t kk = 1; kk < FX_K; ++kk) v = (k == kk) ? A[kk][j] : v;
+          B[j] = lead ? v : 0u;
+        }
+        FxRegs rg;
+        fx_regs_init(rg);
+        FxRegTemps<P::n_temps, fx_spec_n_insn<P>()> ts;
+        fx_spec_range<P, R, en.begin, en.end>(cx, q, ts, M, B, rg);
+        fx_store_vec(op, obase, e, M, true, FX_F32, FX_VT_F, B);
+      }
+    }
+  }
+}
+
+template <int R, class P>
+__global__ __launch_bounds__(FX_BLOCK, 4) void fx_dense_lean(const uint32_t* __restrict__ sb, const FxLeanArgs) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t L[];
+  const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
+  // the argument block is read through the argument segment pointer, never by naming the
+  // parameter: indexing a by-value aggregate dynamically would copy it to per-lane scratch
+  const FX_AS4 uint8_t* ka = (const FX_AS4 uint8_t*)__builtin_amdgcn_kernarg_segment_ptr() + 8;
+  const FX_AS4 uint32_t* aw = (const FX_AS4 uint32_t*)ka;
+  const FX_AS4 uint64_t* gp = (const FX_AS4 uint64_t*)(ka + offsetof(FxLeanArgs, p));
+  const uint32_t total_units = aw[FX_W(FxLeanArgs, total_units)];
+  {
+    // A word of every line of the block that the prologue will read, asked for together with the
+    // first one: the lines then arrive in one trip instead of one trip per level of the reads.
+    constexpr uint32_t LW = 16, N_LINES = (56 + (P::n_entries > 1 ? 2 : 1) * (R > 3 ? 160 : 128)) / 64;
+    uint32_t t[N_LINES];
+#pragma unroll
+    for (uint32_t k = 0; k < N_LINES; ++k) t[k] = aw[(k + 1) * LW - 2];
+#pragma unroll
+    for (uint32_t k = 0; k < N_LINES; ++k) asm volatile("" : : "s"(t[k]));
+  }
+  const uint32_t bpt = aw[FX_W(FxLeanArgs, bpt)];
+  const uint32_t n_sptr = aw[FX_W(FxLeanArgs, n_sptr)], n_tptr = aw[FX_W(FxLeanArgs, n_tptr)];
+  const uint64_t err = ((uint64_t)aw[FX_W(FxLeanArgs, err_ptr) + 1] << 32) | aw[FX_W(FxLeanArgs, err_ptr)];
+  constexpr uint32_t OUT0 = FX_W(FxLeanArgs, out), OUTW = sizeof(FxLeanOut) / 4;
+  bool staged = false;
+  for (uint32_t unit = blockIdx.x; unit < total_units; unit += gridDim.x) {
+    const uint32_t task = fx_fastdiv(unit, aw[FX_W(FxLeanArgs, bpt_magic)], aw[FX_W(FxLeanArgs, bpt_shift)]);
+    const uint32_t local_block = unit - task * bpt;
+    auto get_cx = [&]() -> FxCtx {
+      FxCtx cx{};
+      if constexpr (fx_spec_reads_descriptor<P>()) {
+        const uint32_t blob_words = aw[FX_W(FxLeanArgs, blob_words)];
+        const uint32_t n_p = aw[FX_W(FxLeanArgs, n_p)], n_s = aw[FX_W(FxLeanArgs, n_s)];
+        if (!staged) {
+          // LDS layout of fx_stage: [descriptor][pointers: 2 words each][scalars]
+          const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)sb;
+          fx_u32x4* l4 = (fx_u32x4*)L;
+          for (uint32_t i = threadIdx.x; i < blob_words / 4; i += FX_BLOCK) l4[i] = g4[i];
+          const FX_AS4 uint32_t* gs = (const FX_AS4 uint32_t*)(ka + offsetof(FxLeanArgs, s));
+          uint64_t* lp = (uint64_t*)(L + blob_words);
+          uint32_t* ls = L + blob_words + 2 * n_p;
+          for (uint32_t i = threadIdx.x; i < n_p; i += FX_BLOCK) lp[i] = gp[i];
+          for (uint32_t i = threadIdx.x; i < n_s; i += FX_BLOCK) ls[i] = gs[i];
+          __syncthreads();
+          staged = true;
+        }
+        FxLaunch la;
+        la.blob_words = blob_words;
+        la.n_p = n_p;
+        la.temps_off = (blob_words + 2 * n_p + n_s + 3u) & ~3u;
+        FxWork w;
+        w.cls = L + aw[FX_W(FxLeanArgs, cls_off)];
+        w.task = (int)task;
+        w.local_block = local_block;
+        cx = fx_make_ctx(L, la, w);
+      }
+      return cx;
+    };
+    const uint32_t tp_off = n_sptr + task * n_tptr;
+    if constexpr (P::n_entries > 1) {
+      if (local_block >= aw[FX_W(FxLeanArgs, second_begin)]) {
+        fx_lean_out<P, R, 1>(aw + OUT0 + OUTW, task, local_block, gp, tp_off, err, get_cx, lane, wave);
+        continue;
+      }
+    }
+    fx_lean_out<P, R, 0>(aw + OUT0, task, local_block, gp, tp_off, err, get_cx, lane, wave);
+  }
+}
+
+template <int R, class P>
+const void* fx_spec_lean_kernel() {
+  if constexpr (P::n_entries <= FX_FAST_OUTS) return (const void*)&fx_dense_lean<R, P>;
+  else return nullptr;
+}
+
 struct FxSpecRegistrar {
   FxSpecRegistrar(uint64_t hash, const void* dense, const void* count, const void* scatter, uint32_t scatter_threads,
-                  const void* stream = nullptr) {
+                  const void* stream = nullptr, const void* lean = nullptr, bool lean_stages = false) {
     FxSpecKernels k;
+    k.lean = lean;
+    k.lean_stages = lean_stages;
     k.dense = dense;
     k.count = count;
     k.scatter = scatter;
@@ -387,8 +604,10 @@ struct FxSpecRegistrar {
 
 }  // namespace
 
-#define FX_SPEC_DENSE(P, R) \
-  static FxSpecRegistrar fx_registrar_##P(P::hash, (const void*)&fx_region_dense<R, FxSpec<P>>, nullptr, nullptr, 0);
+// (the lean kernel has compile-time code for at most FX_FAST_OUTS outputs)
+#define FX_SPEC_DENSE(P, R)                                                                                         \
+  static FxSpecRegistrar fx_registrar_##P(P::hash, (const void*)&fx_region_dense<R, FxSpec<P>>, nullptr, nullptr, 0, \
+                                          nullptr, fx_spec_lean_kernel<R, P>(), fx_spec_reads_descriptor<P>());
 #define FX_SPEC_COMPACT(P, R)                                                                    \
   static FxSpecRegistrar fx_registrar_##P(P::hash, nullptr, (const void*)&fx_compact_count<FxSpec<P>>, \
                                           (const void*)&fx_compact_scatter<R, FxSpec<P>>, 64u * FxSpec<P>::kWaves, \

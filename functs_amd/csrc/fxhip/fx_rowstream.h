@@ -211,17 +211,33 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
   // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
   auto look_back = [&]() {
     const uint32_t first = b - chunk;
+    // A lane watches the words of chunks lane, lane + 64, ..., four at a time: what is still
+    // missing of the four is asked for again in one go, so a round of polls costs one trip
+    // however many of the words a lane has.
+    constexpr uint32_t NG = 4u;
     uint32_t part = 0;
     bool ok = true;
-    for (uint32_t i = lane; i < chunk; i += 64u) {
-      uint32_t wv = i < 64u ? pw[0] : (i < 128u ? pw[1] : 0u), polls = 0;
-      while ((wv >> FX_RS_STATUS_BITS) != la.epoch) {
+    for (uint32_t base = 0; base < chunk && ok; base += NG * 64u) {
+      uint32_t wv[NG], polls = 0;
+#pragma unroll
+      for (uint32_t j = 0; j < NG; ++j) wv[j] = (base == 0u && j < 2u) ? pw[j] : 0u;
+      for (;;) {
+        bool missing = false;
+#pragma unroll
+        for (uint32_t j = 0; j < NG; ++j)
+          missing = missing || (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch);
+        if (!missing) break;
         if (polls >= la.spin_limit) { ok = false; break; }
         ++polls;
         __builtin_amdgcn_s_sleep(1);
-        wv = __hip_atomic_load(la.status + first + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (uint32_t j = 0; j < NG; ++j)
+          if (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch)
+            wv[j] = __hip_atomic_load(la.status + first + base + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      part += ok ? (wv & ((1u << FX_RS_STATUS_BITS) - 1u)) : 0u;
+#pragma unroll
+      for (uint32_t j = 0; j < NG; ++j)
+        part += (ok && base + j * 64u + lane < chunk) ? (wv[j] & ((1u << FX_RS_STATUS_BITS) - 1u)) : 0u;
     }
     part = fx_wave_sum(part, lane);
     const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;

@@ -11,7 +11,8 @@ synchronisations, the way the reference times a call (functs/utils/evaluate.py:1
 Prints ONE JSON line.  `value` is the per-call latency of the headline workload
 (c5: ParallelMap over 16 YOLOv3-style images) through the TorchScript route, i.e.
 the scripted program whose fused regions run as tssa::ParallelFunctor;
-`drained_latency_us` is the same call with the device drained after every call;
+`drained_latency_us` is the same call with the device drained after every call
+(`drain_floor_us`: a 256-byte copy kernel drained the same way);
 `region_api_latency_us` is the same regions driven from Python through ctypes;
 `compiled_kernels` says whether the regions ran ahead-of-time compiled kernels
 (functs_amd.aot) or the bytecode interpreter (`--interpreter` forces the latter);
@@ -200,6 +201,23 @@ def flush(dev):
     # drained before anything is timed: launches queued right behind the flush read up to 1.5 us
     # longer each over the first tens of launches (seen on the 4 us kernels of c1)
     torch.cuda.synchronize()
+
+
+def drain_floor_us(dev, n=200):
+    """One small library kernel and a device synchronisation, per round: what draining the device
+    after a call costs whatever the call does (the part of every drained latency that no kernel
+    of this library can take away)."""
+    import torch
+    from functs_amd import _lib
+    x, y = torch.zeros(64, device=dev), torch.zeros(64, device=dev)
+    for _ in range(20):
+        _lib.copy_bytes(x, y)
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        _lib.copy_bytes(x, y)
+        torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e6 / n
 
 
 def recorded_traffic(kernel, workload):
@@ -818,6 +836,7 @@ def main():
                    "route": "functs_amd.jit.script -> build -> tssa::ParallelFunctor (C++ operator over the C ABI)",
                    "compiled_kernels": head["compiled_kernels"] and not args.interpreter,
                    "drained_latency_us": head["torchscript_route_drained_latency_us"],
+                   "drain_floor_us": round(drain_floor_us(dev), 2),
                    "latency_us_warm": head["torchscript_route_latency_us_warm"],
                    "drained_latency_us_warm": head["torchscript_route_drained_latency_us_warm"],
                    "region_api_latency_us": head["latency_us"], "launches_per_call": head["launches_per_call"],

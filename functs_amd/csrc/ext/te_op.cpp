@@ -697,7 +697,8 @@ class RegionRunner {
   // them; nothing runs): `kind` is the first word of fx_plan_head_info when that kernel is in
   // use (0: the generic kernels), `shapes` the shapes of task 0's results.
   void dryRun(const std::vector<c10::IValue>& samples, int64_t* kind, std::vector<std::vector<int64_t>>* shapes,
-              int64_t* rowstream = nullptr, std::string* rowstream_why = nullptr, std::vector<c10::ScalarType>* dtypes = nullptr) {
+              int64_t* rowstream = nullptr, std::string* rowstream_why = nullptr, std::vector<c10::ScalarType>* dtypes = nullptr,
+              int64_t* kernels = nullptr) {
     TORCH_CHECK(samples.size() == n_stack_, "dryRun: argument count");
     int64_t degree = degree_;
     size_t first = 0;
@@ -719,6 +720,10 @@ class RegionRunner {
     int64_t info[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     FX_OK_OR_THROW(fx_plan_head_info(plan, info, 8));
     *kind = info[1] ? info[0] : 0;
+    if (kernels) {   // [0]: compiled kernels are linked for the region's programs, [1]: a dense region on the lean kernel
+      kernels[0] = fx_plan_specialized(plan);
+      kernels[1] = fx_plan_dense_lean(plan);
+    }
     if (rowstream) {
       FX_OK_OR_THROW(fx_plan_rowstream_info(plan, rowstream, 8));
       if (rowstream_why) {
@@ -1711,8 +1716,11 @@ void planIn(Block* b, std::vector<std::string>* report) {
       std::vector<std::vector<int64_t>> shapes;
       std::string why;
       RegionRunner r(n);
-      r.dryRun(samples, &kind, &shapes, rs, &why);
+      int64_t kernels[2] = {0, 0};
+      r.dryRun(samples, &kind, &shapes, rs, &why, nullptr, kernels);
       line << "functor planned: " << shapes.size() << " output(s)";
+      if (!(n->hasAttribute(sym::compact_rows()) && n->i(sym::compact_rows()) != 0))
+        line << (kernels[1] ? ", compiled (lean dense kernel)" : kernels[0] ? ", compiled" : ", interpreted");
       if (n->hasAttribute(sym::compact_rows()) && n->i(sym::compact_rows()) != 0) {
         if (rs[0]) {
           char hx[32];

@@ -63,6 +63,9 @@ def test_the_head_is_two_functors_and_the_second_streams_rows():
     assert "aten::sigmoid" in sub and "aten::cat" in sub and "aten::zeros" in sub   # objectness, scores and their padding sank into the map
     report = aot.plan(fn)
     assert len(report) == 2 and "row-stream key" in report[1], report
+    # the dense part of the head (decode for the whole batch) has compiled programs and fits the
+    # short dense kernel
+    assert "lean dense kernel" in report[0], report
 
 
 @pytest.mark.gpu

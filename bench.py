@@ -21,7 +21,8 @@ implemented, each with its CPU baseline, the library's copy kernel on the same
 bytes, the operator's host time by section and, for row compactions (whose default
 is the kernel generated from the region's programs, fx_rs_kernel), the figures of
 the hand-written and the generic kernels and of the opt-in call forms (lazy_lists,
-padded_outputs); `head_variants`: other spellings of the detection head, each on its
+padded_outputs); `c5_batch64`: four times c5's batch, more chunks than the device holds
+workgroups; `head_variants`: other spellings of the detection head, each on its
 own generated kernel; `c5_nms_tail`: the compaction followed by the detection tail,
 also through the TorchScript route.  `roofline` prices the dominant kernel against the 8 TB/s
 HBM peak with the algorithmic bytes of the call; its duration is measured with
@@ -757,6 +758,43 @@ def main():
             del bound
         return out
 
+    def run_big_batch(batch=64):
+        """The benchmark's region and one of the variants on four times c5's batch: more chunks of
+        256 rows than the device holds workgroups (2 688 against 1 536), so every workgroup of the
+        row-stream kernel takes chunks in turn; the variant also on the generic two passes."""
+        from functs_amd import configs, _lib
+        from functs_amd.benchmark.inputs import INPUTS
+        from functs_amd.region import timed_sets
+        preds, anchors, strides = INPUTS["c5"](0)
+        torch.manual_seed(1)
+        preds = preds.repeat(batch // preds.size(0), 1, 1)
+        preds = preds + 0.01 * torch.randn(preds.shape)
+        out = {"batch": batch}
+        for vname, region_of in (("benchmark", lambda: configs.build_c5(batch)),
+                                 ("stack", lambda: configs.build_head_variant(batch=batch, **configs.HEAD_VARIANTS["stack"]))):
+            for rowstream in ((True, False) if vname == "stack" else (True,)):
+                _lib.lib.fx_set_rowstream(1 if rowstream else 0)
+                _lib.lib.fx_set_head_kernel(1 if rowstream else 0)
+                try:
+                    region = region_of()
+                    bound = [region.bind(preds.clone().to(dev), anchors.to(dev), strides.to(dev)) for _ in range(2)]
+                    for bc in bound:
+                        bc.launch()
+                    res = bound[0].results()
+                    torch.cuda.synchronize()
+                    alg = bound[0].plan.alg_bytes + sum(t.numel() * t.element_size() for o in res for t in (o if isinstance(o, list) else [o]))
+                    flush(dev)
+                    ms = timed_sets(bound, which=-1, rounds=6)
+                    out[vname if rowstream else vname + "_generic"] = {
+                        "kernel": head_kernel_in_use(bound[0].plan), "launches_per_call": bound[0].plan.launches,
+                        "call_kernels_us": round(ms * 1e3, 2), "algorithmic_bytes": alg,
+                        "frac_hbm_peak_call": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                    del bound
+                finally:
+                    _lib.lib.fx_set_rowstream(1)
+                    _lib.lib.fx_set_head_kernel(1)
+        return out
+
     def run_stream():
         """Not one of the five configurations: one big fused elementwise region (sigmoid(2x + 1) on
         [8192, 4096] fp32), the shape on which the dense kernel itself meets the HBM roofline."""
@@ -802,6 +840,10 @@ def main():
             per["head_variants"] = run_variants()
         except Exception as e:
             per["head_variants"] = {"error": str(e)[:200]}
+        try:
+            per["c5_batch64"] = run_big_batch()
+        except Exception as e:
+            per["c5_batch64"] = {"error": str(e)[:200]}
         try:
             per["c4"] = run_c4()
         except Exception as e:

@@ -820,13 +820,17 @@ static const FxRsKernel* rs_of(const fx::Plan* pl) {
   if (pl->mode != FX_MODE_COMPACT || !pl->rs.ok || !g_rs_mode.load(std::memory_order_relaxed) ||
       !g_specialize.load(std::memory_order_relaxed))
     return nullptr;
-  // The skeleton counts on every workgroup being resident at once (a chunk looks back at all chunks
-  // before it): a launch that needs more workgroups than the device holds, even with chunks of
-  // FX_BLOCK rows, would spend its time in bounded waits and their fallback, and keeps the generic
-  // two passes (80 tasks of 8 732 rows: 26.6 us that way against 7.9 + 15.1 us).
-  // (fx_set_rowstream(2) takes the kernel all the same: its bounded waits end every launch)
+  // The workgroups of a launch are persistent: a launch with more chunks than the device holds
+  // workgroups gives every workgroup several chunks in turn.  That pays where the tasks stream
+  // rows of their own (a batch of images: 64 images 90 us against 161 us on the two passes).  A
+  // map of many tasks over the SAME rows (80 classes over 8 732 rows) would stream them once per
+  // task, chunk after chunk, and keeps the generic two passes (27.6 us that way against 22.5 us).
+  // (fx_set_rowstream(2) takes the kernel all the same)
   const uint64_t chunks = ((uint64_t)pl->rs.n_rows + FX_BLOCK - 1) / FX_BLOCK;
-  if (g_rs_mode.load(std::memory_order_relaxed) != 2 && chunks * pl->rs.n_tasks > (uint64_t)rs_compute_units() * FX_RS_OCC) return nullptr;
+  const bool rows_of_their_own = pl->rs.n_tasks <= 1 || pl->rs.in_tcoef[0] != 0;
+  if (g_rs_mode.load(std::memory_order_relaxed) != 2 && !rows_of_their_own &&
+      chunks * pl->rs.n_tasks > (uint64_t)rs_compute_units() * FX_RS_OCC)
+    return nullptr;
   const FxRsKernel* k = fx_rs_find(pl->rs.key);
   return (k && k->S == pl->rs.S) ? k : nullptr;
 }
@@ -894,6 +898,7 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     const uint32_t forced_sub = rs_env("FXHIP_RS_SUB_ROWS"), forced_chunk = rs_env("FXHIP_RS_CHUNK_ROWS");
     uint32_t best_sub = 0, best_cr = 0, best_n = 0;
     bool best_side = false, best_lean = false;
+    int best_per_cu = 0;
     // The kernel built for five loads per lane and sub-tile first (fewer registers), the one for six
     // where it saves a sub-tile per chunk; with the chunk's table of side values in LDS, and without
     // it where the table would cost a workgroup per CU or a sub-tile per chunk (the rows then load
@@ -944,7 +949,7 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
           if (rs_env("FXHIP_RS_VERBOSE"))
             fprintf(stderr, "[fxhip] row-stream geometry: %u loads, side table %d, sub-tile %u rows, %u B of LDS, %d workgroups per CU, chunk %u rows, %u sub-tiles\n",
                     lean ? FX_RS_KV_LEAN : FX_RS_KV, with_side, sub, rs_lds_bytes(ri, kern, sub, cr, with_side != 0), per_cu, cr, n);
-          if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; best_side = with_side != 0; best_lean = lean != 0; }
+          if (best_sub == 0 || n < best_n) { best_sub = sub; best_cr = cr; best_n = n; best_side = with_side != 0; best_lean = lean != 0; best_per_cu = per_cu; }
           if (forced_sub || sub == 8u) break;
         }
       }
@@ -954,6 +959,7 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     pl->rs_chunk_rows = best_cr;
     pl->rs_side_lds = best_side ? 1u : 0u;
     pl->rs_lean = best_lean ? 1u : 0u;
+    pl->rs_grid_cap = (uint32_t)best_per_cu * (uint32_t)std::max(cus, 1);   // workgroups that the device holds at once
   }
   rl->sub_rows = pl->rs_sub_rows;
   rl->chunk_rows = pl->rs_chunk_rows;
@@ -968,9 +974,10 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
   rl->late_tell = rs_env("FXHIP_RS_LATE_TELL") ? 1u : 0u;
   return FX_OK;
 }
+// (persistent workgroups: at most as many as the device holds at once, each takes chunks in turn)
 static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const FxRsLaunch& rl, const FxDyn* dyn, hipStream_t stream,
-                            bool lean) {
-  const uint32_t grid = rl.chunks * rl.n_tasks;
+                            bool lean, uint32_t grid_cap) {
+  const uint32_t grid = std::min<uint32_t>(rl.chunks * rl.n_tasks, std::max<uint32_t>(grid_cap, 1u));
   if (grid == 0) return hipSuccess;
   void* args[2] = {(void*)&rl, (void*)dyn};
   return hipLaunchKernel(lean && kern->fn_lean ? kern->fn_lean : kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
@@ -1142,7 +1149,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     HIP_OK(mark(0));
     for (int r = 0; r < repeat; ++r) {
       rl.epoch = epoch + (uint32_t)r;
-      HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn, stream, pl->rs_lean != 0));
+      HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn, stream, pl->rs_lean != 0, pl->rs_grid_cap));
     }
     HIP_OK(mark(1));
     nk = rl.chunks * rl.n_tasks > 0 ? 1 : 0;
@@ -1286,7 +1293,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
       } else if (rsk) {
         rl.epoch = epoch + (uint32_t)(r * n_sets + i);
         rl.totals = totals_host[i];
-        HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn[i], stream, pl->rs_lean != 0));
+        HIP_OK(rs_launch(rsk, pl->rs, rl, &dyn[i], stream, pl->rs_lean != 0, pl->rs_grid_cap));
       } else if (head) {
         hl.epoch = epoch + (uint32_t)(r * n_sets + i);
         hl.totals = totals_host[i];

@@ -136,7 +136,7 @@ struct Plan {
   uint32_t cmap_resident_wide = 0;   // class-map head kernel: workgroups of its wide form
   FxLeanArgs lean{};           // dense regions that fit the lean kernel: its argument block but for the per-call parts (n_outs 0: none)
   uint32_t lean_slot_err = 0;  // as FxHeader::slot_err
-  uint32_t rs_lean = 0, rs_side_lds = 0, rs_sub_rows = 0, rs_chunk_rows = 0;   // row-stream kernel: geometry of a launch (chosen at the first one)
+  uint32_t rs_lean = 0, rs_side_lds = 0, rs_sub_rows = 0, rs_chunk_rows = 0, rs_grid_cap = 0;   // row-stream kernel: geometry of a launch (chosen at the first one)
 };
 
 // Fills p->head: does the plan compute the decode + score filter of a detection head (fx_head_match.cpp)?

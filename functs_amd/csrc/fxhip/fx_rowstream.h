@@ -163,241 +163,250 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
   __shared__ uint32_t s_wsum[NW];
   __shared__ uint32_t s_prefix, s_ok, s_nk, s_total, s_told;
   const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
-  const uint32_t b = blockIdx.x;
-  const uint32_t task = b / la.chunks, chunk = b - task * la.chunks;
-  const uint32_t c_r0 = chunk * la.chunk_rows;
-  const uint32_t c_rows = min(la.chunk_rows, la.n_rows - c_r0);   // >= 1 (host)
-  // sub-tiles of equal size, at most la.sub_rows rows each
-  const uint32_t n_sub0 = (c_rows + la.sub_rows - 1u) / la.sub_rows;
-  const uint32_t sub_rows = (c_rows + n_sub0 - 1u) / n_sub0;
-  const uint32_t n_sub = (c_rows + sub_rows - 1u) / sub_rows;
-  FxRsRt rt{la, task, {}, {}};
-  // What the rows' own code reads from memory besides the window (a few words per row: anchors,
-  // strides ...) is fetched for all rows of the chunk before the first sub-tile, into a table in LDS.
-  const bool SIDE_LDS = P::n_row_cols != 0u && P::n_side != 0u && P::n_side <= FX_RS_MAX_SIDE && la.side_lds != 0u;
-  uint32_t* side = nullptr;
-  {
-    // staged outputs behind the window, each sub_rows rows and a group of slack
-    uint32_t* sp = L + ((((la.sub_rows * S + 3u + 3u) >> 2) + 1u) << 2);
-#pragma unroll
-    for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) {
-      rt.stg[k] = sp;
-      rt.ph[k] = 0u;
-      if (k < P::n_out && P::stage_rowlen[k] != 0u) sp += la.sub_rows * P::stage_rowlen[k] + 8u;
+  // Persistent workgroups: the launch has as many as the device holds at once, and workgroup w
+  // takes the chunks w, w + gridDim.x, ... of the launch in that order (chunks are numbered task
+  // by task).  A chunk waits for chunks with smaller numbers only, and those are in the hands of
+  // workgroups that are running: no chunk waits for one that has not been started.
+  const uint32_t n_chunks_all = la.chunks * la.n_tasks;
+  for (uint32_t b = blockIdx.x; b < n_chunks_all; b += gridDim.x) {
+    const uint32_t task = b / la.chunks, chunk = b - task * la.chunks;
+    const uint32_t c_r0 = chunk * la.chunk_rows;
+    const uint32_t c_rows = min(la.chunk_rows, la.n_rows - c_r0);   // >= 1 (host)
+    // sub-tiles of equal size, at most la.sub_rows rows each
+    const uint32_t n_sub0 = (c_rows + la.sub_rows - 1u) / la.sub_rows;
+    const uint32_t sub_rows = (c_rows + n_sub0 - 1u) / n_sub0;
+    const uint32_t n_sub = (c_rows + sub_rows - 1u) / sub_rows;
+    FxRsRt rt{la, task, {}, {}};
+    // What the rows' own code reads from memory besides the window (a few words per row: anchors,
+    // strides ...) is fetched for all rows of the chunk before the first sub-tile, into a table in LDS.
+    const bool SIDE_LDS = P::n_row_cols != 0u && P::n_side != 0u && P::n_side <= FX_RS_MAX_SIDE && la.side_lds != 0u;
+    uint32_t* side = nullptr;
+    {
+      // staged outputs behind the window, each sub_rows rows and a group of slack
+      uint32_t* sp = L + ((((la.sub_rows * S + 3u + 3u) >> 2) + 1u) << 2);
+  #pragma unroll
+      for (uint32_t k = 0; k < FX_RS_MAX_OUT; ++k) {
+        rt.stg[k] = sp;
+        rt.ph[k] = 0u;
+        if (k < P::n_out && P::stage_rowlen[k] != 0u) sp += la.sub_rows * P::stage_rowlen[k] + 8u;
+      }
+      side = sp;   // la.chunk_rows rows of P::n_side words
     }
-    side = sp;   // la.chunk_rows rows of P::n_side words
-  }
-  // element 0 of this task's rows of the window input
-  const FX_AS1 uint32_t* win = (const FX_AS1 uint32_t*)rt.in(0) + (int64_t)la.in_tcoef[0] * task;
+    // element 0 of this task's rows of the window input
+    const FX_AS1 uint32_t* win = (const FX_AS1 uint32_t*)rt.in(0) + (int64_t)la.in_tcoef[0] * task;
 
-  fx_u32x4 wr[KV];
-  uint32_t shift = 0, n_vec = 0;
-  auto request = [&](uint32_t s) {
-    const uint32_t r0 = c_r0 + s * sub_rows, rows = min(sub_rows, c_rows - s * sub_rows);
-    const uint64_t a0 = (uint64_t)(win + (size_t)r0 * S);
-    shift = ((uint32_t)a0 & 15u) >> 2;   // elements between the 16-byte line and the first row
-    const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(a0 & ~(uint64_t)15);
-    n_vec = (shift + rows * S + 3u) >> 2;   // <= KV * NT (host)
-    // every line is used once; lanes past the end ask for the last line again rather than branch,
-    // so that the requests leave back to back; a load of which no lane of the wave has a part is
-    // left out (a branch on a value that all lanes share)
-    const uint32_t n_vec_u = uni(n_vec);
-#pragma unroll
-    for (uint32_t k = 0; k < KV; ++k)
-      if (k * NT + wave * 64u < n_vec_u) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
-  };
-  const bool teller = chunk + 1u == la.chunks && la.late_tell == 0u;   // the task's last chunk tells the host the task's total
-  uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
-  // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
-  auto look_back = [&]() {
-    const uint32_t first = b - chunk;
-    // A lane watches the words of chunks lane, lane + 64, ..., four at a time: what is still
-    // missing of the four is asked for again in one go, so a round of polls costs one trip
-    // however many of the words a lane has.
-    constexpr uint32_t NG = 4u;
-    uint32_t part = 0;
-    bool ok = true;
-    for (uint32_t base = 0; base < chunk && ok; base += NG * 64u) {
-      uint32_t wv[NG], polls = 0;
-#pragma unroll
-      for (uint32_t j = 0; j < NG; ++j) wv[j] = (base == 0u && j < 2u) ? pw[j] : 0u;
-      for (;;) {
-        bool missing = false;
-#pragma unroll
+    fx_u32x4 wr[KV];
+    uint32_t shift = 0, n_vec = 0;
+    auto request = [&](uint32_t s) {
+      const uint32_t r0 = c_r0 + s * sub_rows, rows = min(sub_rows, c_rows - s * sub_rows);
+      const uint64_t a0 = (uint64_t)(win + (size_t)r0 * S);
+      shift = ((uint32_t)a0 & 15u) >> 2;   // elements between the 16-byte line and the first row
+      const FX_AS1 fx_u32x4* g4 = (const FX_AS1 fx_u32x4*)(a0 & ~(uint64_t)15);
+      n_vec = (shift + rows * S + 3u) >> 2;   // <= KV * NT (host)
+      // every line is used once; lanes past the end ask for the last line again rather than branch,
+      // so that the requests leave back to back; a load of which no lane of the wave has a part is
+      // left out (a branch on a value that all lanes share)
+      const uint32_t n_vec_u = uni(n_vec);
+  #pragma unroll
+      for (uint32_t k = 0; k < KV; ++k)
+        if (k * NT + wave * 64u < n_vec_u) wr[k] = __builtin_nontemporal_load(&g4[min(threadIdx.x + k * NT, n_vec - 1u)]);
+    };
+    const bool teller = chunk + 1u == la.chunks && la.late_tell == 0u;   // the task's last chunk tells the host the task's total
+    uint32_t pw[2] = {0, 0};   // wave 1: what its first look at the earlier chunks found
+    // One look-back per workgroup (wave 1): the sum of the counts of the earlier chunks of the task.
+    auto look_back = [&]() {
+      const uint32_t first = b - chunk;
+      // A lane watches the words of chunks lane, lane + 64, ..., four at a time: what is still
+      // missing of the four is asked for again in one go, so a round of polls costs one trip
+      // however many of the words a lane has.
+      constexpr uint32_t NG = 4u;
+      uint32_t part = 0;
+      bool ok = true;
+      for (uint32_t base = 0; base < chunk && ok; base += NG * 64u) {
+        uint32_t wv[NG], polls = 0;
+  #pragma unroll
+        for (uint32_t j = 0; j < NG; ++j) wv[j] = (base == 0u && j < 2u) ? pw[j] : 0u;
+        for (;;) {
+          bool missing = false;
+  #pragma unroll
+          for (uint32_t j = 0; j < NG; ++j)
+            missing = missing || (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch);
+          if (!missing) break;
+          if (polls >= la.spin_limit) { ok = false; break; }
+          ++polls;
+          __builtin_amdgcn_s_sleep(1);
+  #pragma unroll
+          for (uint32_t j = 0; j < NG; ++j)
+            if (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch)
+              wv[j] = __hip_atomic_load(la.status + first + base + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+  #pragma unroll
         for (uint32_t j = 0; j < NG; ++j)
-          missing = missing || (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch);
-        if (!missing) break;
-        if (polls >= la.spin_limit) { ok = false; break; }
-        ++polls;
-        __builtin_amdgcn_s_sleep(1);
-#pragma unroll
-        for (uint32_t j = 0; j < NG; ++j)
-          if (base + j * 64u + lane < chunk && (wv[j] >> FX_RS_STATUS_BITS) != la.epoch)
-            wv[j] = __hip_atomic_load(la.status + first + base + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          part += (ok && base + j * 64u + lane < chunk) ? (wv[j] & ((1u << FX_RS_STATUS_BITS) - 1u)) : 0u;
       }
-#pragma unroll
-      for (uint32_t j = 0; j < NG; ++j)
-        part += (ok && base + j * 64u + lane < chunk) ? (wv[j] & ((1u << FX_RS_STATUS_BITS) - 1u)) : 0u;
-    }
-    part = fx_wave_sum(part, lane);
-    const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
-    if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
-    // The task's last chunk tells the host the task's total as soon as it is known: its own
-    // count comes from its status word (wave 0 publishes it right after the gather).  The host
-    // polls the word while the kernel still runs: a system-scope store goes through to host
-    // memory instead of waiting in L2 for the end of the kernel.
-    if (chunk + 1u == la.chunks && all_ok) {
-      uint32_t wv = 0, polls = 0;
-      bool own = true;
-      for (;;) {
-        wv = __hip_atomic_load(la.status + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((wv >> FX_RS_STATUS_BITS) == la.epoch) break;
-        if (polls >= la.spin_limit) { own = false; break; }
-        ++polls;
-        __builtin_amdgcn_s_sleep(1);
+      part = fx_wave_sum(part, lane);
+      const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
+      if (lane == 0) { s_prefix = part; s_ok = all_ok ? 1u : 0u; }
+      // The task's last chunk tells the host the task's total as soon as it is known: its own
+      // count comes from its status word (wave 0 publishes it right after the gather).  The host
+      // polls the word while the kernel still runs: a system-scope store goes through to host
+      // memory instead of waiting in L2 for the end of the kernel.
+      if (chunk + 1u == la.chunks && all_ok) {
+        uint32_t wv = 0, polls = 0;
+        bool own = true;
+        for (;;) {
+          wv = __hip_atomic_load(la.status + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if ((wv >> FX_RS_STATUS_BITS) == la.epoch) break;
+          if (polls >= la.spin_limit) { own = false; break; }
+          ++polls;
+          __builtin_amdgcn_s_sleep(1);
+        }
+        if (own && lane == 0) {
+          __hip_atomic_store(la.totals + task, part + (wv & ((1u << FX_RS_STATUS_BITS) - 1u)), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_SYSTEM);
+          s_told = 1u;
+        }
       }
-      if (own && lane == 0) {
-        __hip_atomic_store(la.totals + task, part + (wv & ((1u << FX_RS_STATUS_BITS) - 1u)), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_SYSTEM);
-        s_told = 1u;
-      }
-    }
-  };
-  // ---- requests: mask of the chunk's rows (wave 0), first look at the earlier chunks (wave 1),
-  // rows of the first sub-tile (everybody).  In a launch that floods the memory system
-  // (la.bulk_delay) the waves that carry no gather hold their requests back for a moment: the
-  // counts, a few bytes per row that every later workgroup of the task waits for, then reach the
-  // memory system ahead of the bulk instead of somewhere in a queue of tens of megabytes.
-  if (wave == 0) {
-    bool keep[NSUB];
-#pragma unroll
-    for (uint32_t j = 0; j < NSUB; ++j) {
-      const uint32_t r = j * 64u + lane;
-      // rows past the chunk evaluate the chunk's last row (a valid address) and are dropped
-      keep[j] = P::template mask<FxRsRt>(rt, c_r0 + min(r, c_rows - 1u)) && r < c_rows;
-    }
-    request(0);
-    uint32_t nk = 0;
-#pragma unroll
-    for (uint32_t j = 0; j < NSUB; ++j) {
-      s_keep[j * 64u + lane] = keep[j] ? 1u : 0u;
-      nk += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(keep[j]));
-    }
-    if (lane == 0) {
-      __hip_atomic_store(la.status + b, (la.epoch << FX_RS_STATUS_BITS) | nk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_total = nk;
-    }
-  } else {
-    if (wave == 1) {
-      if (lane == 0) s_told = 0u;
-#pragma unroll
-      for (uint32_t j = 0; j < 2; ++j)
-        if (j * 64u + lane < chunk)
-          pw[j] = __hip_atomic_load(la.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (SIDE_LDS) {
-      // (these waves hold their rows back anyway, and the table is shared by the tasks: cache hits)
-      for (uint32_t r = threadIdx.x - 64u; r < c_rows; r += NT - 64u) {
-        typename P::Side sd;
-        P::template row_side<FxRsRt>(rt, c_r0 + r, sd);
-#pragma unroll
-        for (uint32_t k = 0; k < P::n_side; ++k) side[r * P::n_side + k] = sd.s[k];
-      }
-    }
-    if (wave == 1 && teller) {
-      // The host waits for this wave's word: it looks back before it asks for any rows (its polls
-      // would wait for them: loads return in order), so the task's total leaves as soon as the
-      // counts of the task's chunks are known, not when the first sub-tile has arrived.
-      look_back();
-      request(0);
-    } else {
-      for (uint32_t d = 0; d < la.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
-      request(0);
-    }
-  }
-
-  uint32_t prefix = 0, before = 0, staged_kept = 0, staged_orow = 0;
-  for (uint32_t s = 0; s < n_sub; ++s) {
-    if (s) __syncthreads();   // the window and the row map of the sub-tile before are no longer read
-    // Outputs that the sub-tile before put together in LDS leave now, as aligned runs, while the
-    // next window is parked: behind the barrier above everything is in place, and the barrier
-    // below keeps this sub-tile's values out of the buffers until everything has left.
-    if (P::n_staged != 0u && s) fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
-    const uint32_t sh = shift;
-#pragma unroll
-    for (uint32_t k = 0; k < KV; ++k) {
-      const uint32_t v = threadIdx.x + k * NT;
-      if (v < n_vec) ((fx_u32x4*)L)[v] = wr[k];
-    }
-    // all of the sub-tile is parked before the next one is asked for: interleaved, every new
-    // request would be waited for where the next old line is parked
-    asm volatile("" ::: "memory");
-    // (wave 1 looks back first where it does: its polls wait for everything it has asked for)
-    const bool looks_back = wave == 1u && s == 0u && !teller;
-    if (s + 1u < n_sub && !looks_back) request(s + 1u);
-    const uint32_t t_r0 = s * sub_rows, t_rows = min(sub_rows, c_rows - t_r0);
+    };
+    // ---- requests: mask of the chunk's rows (wave 0), first look at the earlier chunks (wave 1),
+    // rows of the first sub-tile (everybody).  In a launch that floods the memory system
+    // (la.bulk_delay) the waves that carry no gather hold their requests back for a moment: the
+    // counts, a few bytes per row that every later workgroup of the task waits for, then reach the
+    // memory system ahead of the bulk instead of somewhere in a queue of tens of megabytes.
     if (wave == 0) {
-      const bool keep = lane < t_rows && s_keep[t_r0 + lane] != 0u;
-      const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
-      if (keep) s_rowmap[__popcll(bal & ((1ull << lane) - 1ull))] = lane;
-      if (lane == 0) s_nk = (uint32_t)__popcll(bal);
-    } else if (looks_back) {
-      look_back();
-      if (s + 1u < n_sub) request(s + 1u);
-    }
-    __syncthreads();
-    if (s == 0) {
-      if (uni(s_ok) == 0u) {
-        // an earlier chunk has not reported in time: count the kept rows in front of this chunk
-        // here, from memory
-        uint32_t cnt = 0;
-        for (uint32_t r = threadIdx.x; r < c_r0 + ((NT - c_r0 % NT) % NT); r += NT) {
-          const bool k2 = P::template mask<FxRsRt>(rt, min(r, c_r0 - 1u)) && r < c_r0;
-          cnt += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(k2));
-        }
-        if (lane == 0) s_wsum[wave] = cnt;
-        __syncthreads();
-        if (threadIdx.x == 0) {
-          uint32_t p = 0;
-          for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
-          s_prefix = p;
-        }
-        __syncthreads();
+      bool keep[NSUB];
+  #pragma unroll
+      for (uint32_t j = 0; j < NSUB; ++j) {
+        const uint32_t r = j * 64u + lane;
+        // rows past the chunk evaluate the chunk's last row (a valid address) and are dropped
+        keep[j] = P::template mask<FxRsRt>(rt, c_r0 + min(r, c_rows - 1u)) && r < c_rows;
       }
-      prefix = uni(s_prefix);
-      // (the total of the task, unless wave 1 has told the host already)
-      if (chunk + 1u == la.chunks && threadIdx.x == 0 && s_told == 0u)
-        __hip_atomic_store(la.totals + task, prefix + s_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
-    const uint32_t n_kept = uni(s_nk);
-    const uint32_t* Wb = L + sh;
-    const uint32_t orow = prefix + before;          // first compacted row of this sub-tile
-    const uint32_t rs0 = c_r0 + t_r0;               // first source row of this sub-tile
-    fx_rs_phases<P, 0u>(rt, orow);
-    // ---- the columns with code of their own: one kept row per lane
-    if (P::n_row_cols != 0u && threadIdx.x < n_kept) {
-      const uint32_t src = s_rowmap[threadIdx.x];
-      // What the row reads besides the window: from the chunk's table in LDS.  (Loaded here, the
-      // words would arrive behind the next sub-tile, which this wave has asked for already: loads
-      // return in order.)
-      typename P::Side sd;
+      request(0);
+      uint32_t nk = 0;
+  #pragma unroll
+      for (uint32_t j = 0; j < NSUB; ++j) {
+        s_keep[j * 64u + lane] = keep[j] ? 1u : 0u;
+        nk += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(keep[j]));
+      }
+      if (lane == 0) {
+        __hip_atomic_store(la.status + b, (la.epoch << FX_RS_STATUS_BITS) | nk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_total = nk;
+      }
+    } else {
+      if (wave == 1) {
+        if (lane == 0) s_told = 0u;
+  #pragma unroll
+        for (uint32_t j = 0; j < 2; ++j)
+          if (j * 64u + lane < chunk)
+            pw[j] = __hip_atomic_load(la.status + b - chunk + j * 64u + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       if (SIDE_LDS) {
-#pragma unroll
-        for (uint32_t k = 0; k < P::n_side; ++k) sd.s[k] = side[(t_r0 + src) * P::n_side + k];
-      } else {
-        P::template row_side<FxRsRt>(rt, rs0 + src, sd);
+        // (these waves hold their rows back anyway, and the table is shared by the tasks: cache hits)
+        for (uint32_t r = threadIdx.x - 64u; r < c_rows; r += NT - 64u) {
+          typename P::Side sd;
+          P::template row_side<FxRsRt>(rt, c_r0 + r, sd);
+  #pragma unroll
+          for (uint32_t k = 0; k < P::n_side; ++k) side[r * P::n_side + k] = sd.s[k];
+        }
       }
-      P::template row<FxRsRt>(rt, Wb + src * S, sd, rs0 + src, orow + threadIdx.x, threadIdx.x);
+      if (wave == 1 && teller) {
+        // The host waits for this wave's word: it looks back before it asks for any rows (its polls
+        // would wait for them: loads return in order), so the task's total leaves as soon as the
+        // counts of the task's chunks are known, not when the first sub-tile has arrived.
+        look_back();
+        request(0);
+      } else {
+        if (b == blockIdx.x)   // (the first chunks of the launch start together; later ones are spread out)
+        for (uint32_t d = 0; d < la.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
+        request(0);
+      }
     }
-    // ---- vector segments: four columns per lane
-    fx_rs_segments<P>(typename P::Vecs{}, rt, Wb, s_rowmap, n_kept, rs0, orow, threadIdx.x, NT);
-    staged_kept = n_kept;
-    staged_orow = orow;
-    before += n_kept;
-  }
-  if (P::n_staged != 0u) {
-    __syncthreads();
-    fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
+
+    uint32_t prefix = 0, before = 0, staged_kept = 0, staged_orow = 0;
+    for (uint32_t s = 0; s < n_sub; ++s) {
+      if (s) __syncthreads();   // the window and the row map of the sub-tile before are no longer read
+      // Outputs that the sub-tile before put together in LDS leave now, as aligned runs, while the
+      // next window is parked: behind the barrier above everything is in place, and the barrier
+      // below keeps this sub-tile's values out of the buffers until everything has left.
+      if (P::n_staged != 0u && s) fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
+      const uint32_t sh = shift;
+  #pragma unroll
+      for (uint32_t k = 0; k < KV; ++k) {
+        const uint32_t v = threadIdx.x + k * NT;
+        if (v < n_vec) ((fx_u32x4*)L)[v] = wr[k];
+      }
+      // all of the sub-tile is parked before the next one is asked for: interleaved, every new
+      // request would be waited for where the next old line is parked
+      asm volatile("" ::: "memory");
+      // (wave 1 looks back first where it does: its polls wait for everything it has asked for)
+      const bool looks_back = wave == 1u && s == 0u && !teller;
+      if (s + 1u < n_sub && !looks_back) request(s + 1u);
+      const uint32_t t_r0 = s * sub_rows, t_rows = min(sub_rows, c_rows - t_r0);
+      if (wave == 0) {
+        const bool keep = lane < t_rows && s_keep[t_r0 + lane] != 0u;
+        const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+        if (keep) s_rowmap[__popcll(bal & ((1ull << lane) - 1ull))] = lane;
+        if (lane == 0) s_nk = (uint32_t)__popcll(bal);
+      } else if (looks_back) {
+        look_back();
+        if (s + 1u < n_sub) request(s + 1u);
+      }
+      __syncthreads();
+      if (s == 0) {
+        if (uni(s_ok) == 0u) {
+          // an earlier chunk has not reported in time: count the kept rows in front of this chunk
+          // here, from memory
+          uint32_t cnt = 0;
+          for (uint32_t r = threadIdx.x; r < c_r0 + ((NT - c_r0 % NT) % NT); r += NT) {
+            const bool k2 = P::template mask<FxRsRt>(rt, min(r, c_r0 - 1u)) && r < c_r0;
+            cnt += (uint32_t)__popcll(__builtin_amdgcn_ballot_w64(k2));
+          }
+          if (lane == 0) s_wsum[wave] = cnt;
+          __syncthreads();
+          if (threadIdx.x == 0) {
+            uint32_t p = 0;
+            for (uint32_t k = 0; k < NW; ++k) p += s_wsum[k];
+            s_prefix = p;
+          }
+          __syncthreads();
+        }
+        prefix = uni(s_prefix);
+        // (the total of the task, unless wave 1 has told the host already)
+        if (chunk + 1u == la.chunks && threadIdx.x == 0 && s_told == 0u)
+          __hip_atomic_store(la.totals + task, prefix + s_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      const uint32_t n_kept = uni(s_nk);
+      const uint32_t* Wb = L + sh;
+      const uint32_t orow = prefix + before;          // first compacted row of this sub-tile
+      const uint32_t rs0 = c_r0 + t_r0;               // first source row of this sub-tile
+      fx_rs_phases<P, 0u>(rt, orow);
+      // ---- the columns with code of their own: one kept row per lane
+      if (P::n_row_cols != 0u && threadIdx.x < n_kept) {
+        const uint32_t src = s_rowmap[threadIdx.x];
+        // What the row reads besides the window: from the chunk's table in LDS.  (Loaded here, the
+        // words would arrive behind the next sub-tile, which this wave has asked for already: loads
+        // return in order.)
+        typename P::Side sd;
+        if (SIDE_LDS) {
+  #pragma unroll
+          for (uint32_t k = 0; k < P::n_side; ++k) sd.s[k] = side[(t_r0 + src) * P::n_side + k];
+        } else {
+          P::template row_side<FxRsRt>(rt, rs0 + src, sd);
+        }
+        P::template row<FxRsRt>(rt, Wb + src * S, sd, rs0 + src, orow + threadIdx.x, threadIdx.x);
+      }
+      // ---- vector segments: four columns per lane
+      fx_rs_segments<P>(typename P::Vecs{}, rt, Wb, s_rowmap, n_kept, rs0, orow, threadIdx.x, NT);
+      staged_kept = n_kept;
+      staged_orow = orow;
+      before += n_kept;
+    }
+    if (P::n_staged != 0u) {
+      __syncthreads();
+      fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
+    }
+    // the window, the row map and the tables are written again by the next chunk
+    if (b + gridDim.x < n_chunks_all) __syncthreads();
   }
 }
 

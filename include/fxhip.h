@@ -244,12 +244,12 @@ int fx_plan_head_info(const fx_plan*, int64_t* out, int cap);
  * for it is linked and enabled (fx_region_run uses it), out[2], out[3] = low and high word of its
  * key, out[4] = elements per row of the streamed input, out[5] = rows, out[6] = tasks,
  * out[7] = input buffers.  fx_plan_rowstream_why: what rules the form out (empty when out[0]).
- * The kernel is used for a launch whose workgroups the device holds all at once (the skeleton
- * counts on it: every chunk looks back at the chunks before it); a launch with more chunks than
- * that, even at 256 rows each, keeps the generic two passes (out[1] = 0).
+ * The kernel's workgroups are persistent: a launch has at most as many as the device holds at
+ * once, and each takes chunks of up to 256 rows in turn (a chunk looks back at the chunks before
+ * it, which are done or running).  One kind of launch beyond that size keeps the generic two
+ * passes (out[1] = 0): a map of several tasks that all stream the SAME rows.
  * fx_set_rowstream: process-wide switch, default 1 = on (FXHIP_ROWSTREAM=0: off; also off while
- * fx_set_specialization(0) holds); 2 = on also for launches beyond what the device holds at once
- * (their bounded waits and the fallback behind them end every launch; slower than the two passes). */
+ * fx_set_specialization(0) holds); 2 = on also for that kind of launch (slower than the two passes). */
 int fx_plan_rowstream_info(const fx_plan*, int64_t* out, int cap);
 int fx_plan_rowstream_why(const fx_plan*, char* buf, size_t cap);               /* returns the full length */
 int fx_plan_rowstream_source(const fx_plan*, const char* label, char* buf, size_t cap); /* returns the full length */

@@ -126,8 +126,8 @@ def test_regions_without_a_row_stream_form_say_why():
     r = configs.build_c3_classes(6)
     info = r.rowstream_info(torch.rand(40, 4), torch.rand(40, 7))
     assert info["ok"] and info["row_elements"] == 4
-    # ... and at the benchmark's size (80 tasks of 8 732 rows) the launch would need more workgroups
-    # than the device holds at once, which the skeleton counts on: the generic kernels keep it
+    # ... and at the benchmark's size (80 tasks of 8 732 rows) the launch has more chunks than the
+    # device holds workgroups, and all tasks stream the same rows: the generic kernels keep it
     r = configs.build_c3_classes(80)
     big = r.rowstream_info(torch.rand(8732, 4), torch.rand(8732, 81))
     assert big["ok"] and not big["active"]
@@ -305,20 +305,43 @@ def test_predictions_that_start_at_an_odd_address_and_outputs_of_every_phase():
 @pytest.mark.gpu
 @pytest.mark.parametrize("n,batch", [(100000, None), (60000, 16)])
 def test_launches_beyond_what_the_device_holds_at_once(n, batch):
-    """By default such a launch keeps the two passes (the skeleton counts on all workgroups being
-    resident); forced onto the generated kernel it still ends and gives the same rows: chunks
-    whose predecessors have not started give up their bounded wait and count for themselves."""
+    """The workgroups are persistent: with more chunks than the device holds workgroups (16 x 235
+    chunks of 256 rows against six workgroups on each of 256 CUs) every workgroup takes chunks in
+    turn, and the rows are those of the two passes."""
     args = _inputs(n, 80, batch or 1, seed=3)
     r = _build("stack", batch)
     info = r.rowstream_info(*args)
-    beyond = -(-n // 256) * (batch or 1) > 256 * 6      # chunks of 256 rows against six workgroups on each of 256 CUs
-    assert info["ok"] and info["active"] == (not beyond)
+    assert info["ok"] and info["active"]
+    one, two = _three_ways(r, *args)
+    assert_exact(_flat(one), _flat(two), "n=%d batch=%s" % (n, batch))
+
+
+@pytest.mark.gpu
+def test_one_task_with_more_chunks_than_the_device_holds_workgroups():
+    """450 000 rows are 1 758 chunks of 256 rows for 1 536 workgroups: some take a second chunk."""
+    r = configs.build_row_filter()
+    torch.manual_seed(11)
+    args = [torch.rand(450000, 19) - 0.5, torch.rand(450000, 2) - 0.5]
+    one, two = _three_ways(r, *args)
+    assert_exact(_flat(one), _flat(two), "row filter, 450 000 rows")
+
+
+@pytest.mark.gpu
+def test_a_map_over_the_same_rows_keeps_the_two_passes_beyond_that_size_unless_forced():
+    """80 class tasks over the same 8 732 boxes: by default the generic kernels; forced onto the
+    generated kernel (every workgroup takes chunks in turn) the same rows."""
+    r = configs.build_c3_classes(80)
+    torch.manual_seed(12)
+    args = [torch.rand(8732, 4), torch.rand(8732, 81) * 0.1]
+    assert not r.rowstream_info(*args)["active"]
+    two = run_region("hip", r, *args)
     lib.fx_set_rowstream(2)
     try:
-        one, two = _three_ways(r, *args, mode=2)
+        assert r.rowstream_info(*args)["active"]
+        one = run_region("hip", r, *args)
     finally:
         lib.fx_set_rowstream(1)
-    assert_exact(_flat(one), _flat(two), "n=%d batch=%s" % (n, batch))
+    assert_exact(_flat(one), _flat(two), "class map, 80 tasks")
 
 
 @pytest.mark.gpu

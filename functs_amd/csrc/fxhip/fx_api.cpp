@@ -904,8 +904,11 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     // it where the table would cost a workgroup per CU or a sub-tile per chunk (the rows then load
     // their side values themselves).  Fewest sub-tiles per chunk wins, the first found among equals.
     const uint32_t forced_loads = rs_env("FXHIP_RS_LOADS");   // tuning aid: FX_RS_KV or FX_RS_KV_LEAN
-    for (int lean = 1; lean >= 0; --lean) {
-      const void* fn = lean ? kern->fn_lean : kern->fn;
+    // (a launch with more chunks than the device holds workgroups runs the build with persistent
+    // workgroups, which exists for six loads only)
+    const bool beyond = (uint64_t)((ri.n_rows + FX_BLOCK - 1) / FX_BLOCK) * ri.n_tasks > (uint64_t)std::max(cus, 1) * FX_RS_OCC;
+    for (int lean = beyond ? 0 : 1; lean >= 0; --lean) {
+      const void* fn = beyond ? kern->fn_persist : lean ? kern->fn_lean : kern->fn;
       if (!fn || (forced_loads && forced_loads != (lean ? FX_RS_KV_LEAN : FX_RS_KV))) continue;
       // (measured on the benchmark's shape: 22.6 against 22.95 us for kernels that store as they
       // compute; with outputs staged in LDS, where LDS and not registers bounds the occupancy, 25.6 against 24.4)
@@ -977,10 +980,12 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
 // (persistent workgroups: at most as many as the device holds at once, each takes chunks in turn)
 static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const FxRsLaunch& rl, const FxDyn* dyn, hipStream_t stream,
                             bool lean, uint32_t grid_cap) {
-  const uint32_t grid = std::min<uint32_t>(rl.chunks * rl.n_tasks, std::max<uint32_t>(grid_cap, 1u));
-  if (grid == 0) return hipSuccess;
+  const uint32_t n_chunks = rl.chunks * rl.n_tasks, cap = std::max<uint32_t>(grid_cap, 1u);
+  if (n_chunks == 0) return hipSuccess;
+  const bool persist = n_chunks > cap;
+  const uint32_t grid = persist ? cap : n_chunks;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(lean && kern->fn_lean ? kern->fn_lean : kern->fn, dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
+  return hipLaunchKernel(persist ? kern->fn_persist : (lean && kern->fn_lean ? kern->fn_lean : kern->fn), dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----

@@ -154,7 +154,7 @@ FX_RS_FN void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_
 #include "fx_rs_ops.h"
 namespace {
 
-template <class P, uint32_t KV>
+template <class P, uint32_t KV, bool PERSIST>
 __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
   constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, NSUB = FX_RS_NSUB, S = P::S;
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];   // the window: sub_rows rows of S elements
@@ -163,12 +163,14 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
   __shared__ uint32_t s_wsum[NW];
   __shared__ uint32_t s_prefix, s_ok, s_nk, s_total, s_told;
   const uint32_t lane = threadIdx.x & 63u, wave = uni(threadIdx.x >> 6);
-  // Persistent workgroups: the launch has as many as the device holds at once, and workgroup w
-  // takes the chunks w, w + gridDim.x, ... of the launch in that order (chunks are numbered task
-  // by task).  A chunk waits for chunks with smaller numbers only, and those are in the hands of
-  // workgroups that are running: no chunk waits for one that has not been started.
+  // A launch that fits the device has a workgroup per chunk.  PERSIST: a launch with more chunks
+  // than the device holds workgroups has as many workgroups as it holds, and workgroup w takes
+  // the chunks w, w + gridDim.x, ... in that order (chunks are numbered task by task).  A chunk
+  // waits for chunks with smaller numbers only, and those are in the hands of workgroups that are
+  // running: no chunk waits for one that has not been started.  (A build of its own: the loop
+  // costs registers, which the launches that fit do not pay.)
   const uint32_t n_chunks_all = la.chunks * la.n_tasks;
-  for (uint32_t b = blockIdx.x; b < n_chunks_all; b += gridDim.x) {
+  for (uint32_t b = blockIdx.x;;) {
     const uint32_t task = b / la.chunks, chunk = b - task * la.chunks;
     const uint32_t c_r0 = chunk * la.chunk_rows;
     const uint32_t c_rows = min(la.chunk_rows, la.n_rows - c_r0);   // >= 1 (host)
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
         look_back();
         request(0);
       } else {
-        if (b == blockIdx.x)   // (the first chunks of the launch start together; later ones are spread out)
+        if (!PERSIST || b == blockIdx.x)   // (the first chunks of a launch start together; later ones are spread out)
         for (uint32_t d = 0; d < la.bulk_delay; d += 32u) __builtin_amdgcn_s_sleep(32);
         request(0);
       }
@@ -405,17 +407,23 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
       __syncthreads();
       fx_rs_copy_out<P, 0u>(rt, staged_kept, staged_orow, threadIdx.x, NT);
     }
-    // the window, the row map and the tables are written again by the next chunk
-    if (b + gridDim.x < n_chunks_all) __syncthreads();
+    if constexpr (!PERSIST) {
+      break;
+    } else {
+      b += gridDim.x;
+      if (b >= n_chunks_all) break;
+      __syncthreads();   // the window, the row map and the tables are written again by the next chunk
+    }
   }
 }
 
 struct FxRsRegistrar {
-  FxRsRegistrar(uint64_t key, const void* fn, const void* fn_lean, uint32_t S, uint32_t stage_row_words, uint32_t n_staged,
-                uint32_t side_row_words) {
+  FxRsRegistrar(uint64_t key, const void* fn, const void* fn_lean, const void* fn_persist, uint32_t S, uint32_t stage_row_words,
+                uint32_t n_staged, uint32_t side_row_words) {
     FxRsKernel k;
     k.fn = fn;
     k.fn_lean = fn_lean;
+    k.fn_persist = fn_persist;
     k.S = S;
     k.stage_row_words = stage_row_words;
     k.n_staged = n_staged;
@@ -427,6 +435,7 @@ struct FxRsRegistrar {
 }  // namespace
 
 #define FX_RS_REGISTER(P) \
-  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P, FX_RS_KV>,                                \
-                                           (const void*)&fx_rs_kernel<P, FX_RS_KV_LEAN>, P::S, P::stage_row_words, P::n_staged, \
-                                           (P::n_row_cols != 0u && P::n_side <= FX_RS_MAX_SIDE) ? P::n_side : 0u);
+  static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P, FX_RS_KV, false>,                          \
+                                           (const void*)&fx_rs_kernel<P, FX_RS_KV_LEAN, false>,                             \
+                                           (const void*)&fx_rs_kernel<P, FX_RS_KV, true>, P::S, P::stage_row_words,         \
+                                           P::n_staged, (P::n_row_cols != 0u && P::n_side <= FX_RS_MAX_SIDE) ? P::n_side : 0u);

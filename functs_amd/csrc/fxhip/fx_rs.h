@@ -83,8 +83,9 @@ static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte
 
 // ---- host side: generated kernels linked into the library ----
 struct FxRsKernel {
-  const void* fn = nullptr;     // fx_rs_kernel<P, FX_RS_KV>
-  const void* fn_lean = nullptr; // fx_rs_kernel<P, FX_RS_KV_LEAN>
+  const void* fn = nullptr;     // fx_rs_kernel<P, FX_RS_KV, false>
+  const void* fn_lean = nullptr; // fx_rs_kernel<P, FX_RS_KV_LEAN, false>
+  const void* fn_persist = nullptr; // fx_rs_kernel<P, FX_RS_KV, true>: workgroups that take several chunks in turn
   uint32_t S = 0;               // row length the kernel is generated for
   uint32_t stage_row_words = 0; // elements per kept row that the kernel puts together in LDS before they leave
   uint32_t n_staged = 0;        // outputs that take that route

@@ -127,6 +127,13 @@ def _plan_benchmark_programs(names):
     if "coverage" in names:
         _plan_region(configs.build_column_standardize(), torch.rand(*configs.COLUMN_STANDARDIZE_SHAPE))
         _plan_region(configs.build_row_filter(), *[torch.rand(*sh) - 0.5 for sh in configs.ROW_FILTER_SHAPES])
+        for batch, levels in ((2, configs.GENERATED_ANCHOR_LEVELS), (16, configs.GENERATED_ANCHOR_LEVELS_C5)):
+            # only the row-stream unit of the large instance: its program table is long, and the
+            # generic kernels run it interpreted
+            _lib.lib.fx_spec_dump_what(3 if batch == 2 else 2)
+            _plan_region(configs.build_c5_generated_anchors(batch, levels), torch.empty(batch, sum(f * f * 3 for f, _ in levels), 85),
+                         *[torch.empty(3, 4) for _ in levels])
+        _lib.lib.fx_spec_dump_what(3)
     if "stream" in names:
         r = Region()
         xi = r.tensor_input(torch.float32, 2)

@@ -197,6 +197,12 @@ def _level_anchors(r, base, feat, stride):
     return (base.unsqueeze(0) + shifts.unsqueeze(1)).view(-1, 4)
 
 
+# the small instance of build_c5_generated_anchors that the tests run and kernels are linked for
+GENERATED_ANCHOR_LEVELS = ((3, 32.0), (5, 16.0), (9, 8.0))
+# ... and the benchmark's instance (YOLOv3 at 416 x 416: 10 647 rows)
+GENERATED_ANCHOR_LEVELS_C5 = ((13, 32.0), (26, 16.0), (52, 8.0))
+
+
 def build_c5_generated_anchors(batch, levels):
     """C5 with the anchor / stride tables generated inside the region (arange, repeat, view,
     stack, broadcast add, cat) instead of read from HBM: the step in front of the hot path

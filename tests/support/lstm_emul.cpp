@@ -191,6 +191,9 @@ extern "C" int fx_lstm_emul_give_up(const float* x, const float* wih, const floa
   if (poisoned(-1)) bits |= 8;
   std::fill(ctl.begin(), ctl.end(), 0u);
   std::fill(hbuf.begin(), hbuf.end(), 0ull);
+  // (this launch has every workgroup: it must not give up because the host's threads, more than
+  // it has cores, took long to be scheduled)
+  a.spin_limit = 0x7fffffffu;
   launch(-1);
   if (ctl[FX_LSTM_W_ERR] == 0u) bits |= 16;
   return bits;

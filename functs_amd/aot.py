@@ -24,13 +24,28 @@ Use, for your own model::
         # or, on a GPU:  fn(*example_inputs)   - every region planned while it runs leaves its source
     # then rebuild the library:  python -c "import __graft_entry__ as g; g.build()"
 
+Or at run time, where ``hipcc`` is at hand (the reference's way: code per subgraph when the
+operator is first made): ``functs_amd.jit.build(..., compile_kernels=True)`` or
+``aot.compile_missing(fn)`` plans the function's regions, compiles the units that are not linked
+into small shared objects of their own and loads them; they register with the loaded library
+like the linked ones (row-stream units take seconds and are the default; the general kernels
+instantiated for a region's programs, `tables="dense"` / `"all"`, up to a minute or two).  The objects are kept in ``kernel_cache_dir()`` and
+loaded again by every later process (``load_cached_kernels``, called when the package is
+imported).
+
 ``python -m functs_amd.aot`` does this for the benchmark programs of ``functs_amd.benchmark``
 (both routes: the Region API and the TorchScript operator) and for the other spellings of the
 detection head in ``functs_amd.configs.HEAD_VARIANTS``; with ``--plan-only`` it needs no GPU.
 """
 import argparse
 import contextlib
+import ctypes
+import glob
+import hashlib
 import os
+import shutil
+import subprocess
+import tempfile
 
 from . import _lib
 
@@ -50,6 +65,111 @@ def capture(directory: str = SPEC_DIR, program_tables: bool = True, rowstream: b
     finally:
         _lib.check(_lib.lib.fx_spec_dump_dir(None))
         _lib.lib.fx_spec_dump_what(3)
+
+
+# ---- kernels compiled at run time ---------------------------------------------------------------
+_FXHIP_DIR = os.path.dirname(SPEC_DIR)
+_HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]   # as csrc/fxhip/Makefile
+_loaded = {}   # path -> CDLL (kept: the library calls into them)
+
+
+def _abi_tag() -> str:
+    """Kernels are compiled against the library's headers: a cache per state of those."""
+    h = hashlib.sha1()
+    for f in sorted(glob.glob(os.path.join(_FXHIP_DIR, "*.h"))):
+        with open(f, "rb") as fh:
+            h.update(os.path.basename(f).encode())
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def kernel_cache_dir() -> str:
+    """Where kernels compiled at run time are kept: ``$FUNCTS_AMD_KERNEL_CACHE`` or
+    ``functs_amd/lib/jit``, in a directory per state of the library's headers."""
+    base = os.environ.get("FUNCTS_AMD_KERNEL_CACHE") or os.path.join(os.path.dirname(_lib.LIB_PATH), "jit")
+    return os.path.join(base, _abi_tag())
+
+
+def hipcc_path():
+    """The HIP compiler driver, or None."""
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def _load_kernel_object(path: str) -> None:
+    if path not in _loaded:
+        # its static initialisers hand the kernels to the loaded library (fx_spec_register / fx_rs_register)
+        _loaded[path] = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+def load_cached_kernels() -> int:
+    """Loads every kernel object of kernel_cache_dir(); returns how many are loaded."""
+    d = kernel_cache_dir()
+    if os.path.isdir(d):
+        for path in sorted(glob.glob(os.path.join(d, "fx_*.so"))):
+            try:
+                _load_kernel_object(path)
+            except OSError:
+                pass   # a stale or half-written object: compile_missing writes it again
+    return len(_loaded)
+
+
+def compile_sources(directory: str, verbose: bool = False, tables: str = "none"):
+    """Compiles the generated units of `directory` that have no object in the cache yet into
+    shared objects there and loads them.  Every row-stream unit (``fx_rs_*.hip``: straight-line
+    code, seconds) is compiled; of the program tables (``fx_spec_*.hip``: the general kernels
+    instantiated for a region's programs, up to a minute or two each) none (`tables` = "none",
+    the default: dense regions and two-pass forms keep the interpreter), those of dense regions
+    ("dense") or all ("all").  Returns the names compiled."""
+    cc = hipcc_path()
+    if cc is None:
+        raise RuntimeError("no hipcc found (PATH, $HIPCC, /opt/rocm/bin): generate the sources with aot.capture() and "
+                           "build them into the library instead")
+    out_dir = kernel_cache_dir()
+    os.makedirs(out_dir, exist_ok=True)
+    lib_dir = os.path.dirname(_lib.LIB_PATH)
+    done = []
+    for src in sorted(glob.glob(os.path.join(directory, "fx_*.hip"))):
+        name = os.path.splitext(os.path.basename(src))[0]
+        if name.startswith("fx_spec_"):
+            with open(src) as fh:
+                dense = "FX_SPEC_DENSE" in fh.read()
+            if tables == "none" or (tables == "dense" and not dense):
+                continue
+        obj = os.path.join(out_dir, name + ".so")
+        if not os.path.isfile(obj):
+            tmp = obj + ".%d.tmp" % os.getpid()
+            cmd = [cc] + _HIPCC_FLAGS + ["-shared", "-I", SPEC_DIR, src, "-o", tmp, "-L", lib_dir, "-lfxhip", "-Wl,-rpath," + lib_dir]
+            if verbose:
+                print("[functs_amd.aot] compiling %s" % name, flush=True)
+            res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+            if res.returncode != 0:
+                if os.path.exists(tmp):
+                    os.unlink(tmp)
+                raise RuntimeError("hipcc failed on %s:\n%s" % (src, res.stderr[-2000:]))
+            os.replace(tmp, obj)
+            done.append(name)
+        _load_kernel_object(obj)
+    return done
+
+
+def compile_missing(fn=None, planner=None, verbose: bool = False, tables: str = "none"):
+    """Plans the regions of a built function (or whatever `planner()` plans) for the static types
+    of its example, and compiles and loads the kernels that are not linked in.  Needs no GPU.
+    Returns the names of the units compiled now."""
+    tmp = tempfile.mkdtemp(prefix="functs_amd_src_")
+    try:
+        with capture(tmp):
+            if fn is not None:
+                plan(fn)
+            if planner is not None:
+                planner()
+        return compile_sources(tmp, verbose=verbose, tables=tables)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
 
 
 def linked() -> int:

@@ -176,7 +176,7 @@ class GraphedFunction(AotScriptFunction):
 
 
 def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: bool = False,
-          padded_outputs: bool = False) -> AotScriptFunction:
+          padded_outputs: bool = False, compile_kernels=False) -> AotScriptFunction:
     """Form fused regions in a functionalized script and return the callable
     (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``.
     ``lazy_lists=True`` (a function that builds into ONE fused region only): List[Tensor] results
@@ -187,11 +187,21 @@ def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: 
     back at full size (a map: one tensor [tasks, rows, ...] per result) without waiting for the
     kept-row counts, which come as one more tensor at the end of the result tuple (int32, pinned
     host memory that the kernels write; rows from counts[task] on hold no values): for callers that
-    pass the results on to work on the same stream."""
+    pass the results on to work on the same stream.
+    ``compile_kernels=True``: the row compactions of the built function that have a row-stream
+    form but no kernel linked into the library get theirs now (generated for the example's static
+    types, compiled with hipcc into the kernel cache, a few seconds per region the first time;
+    later processes load them from the cache): where the reference generates and compiles code
+    per subgraph when the operator is made (fait/fuser/graph_builder.cpp:259-712).
+    ``compile_kernels="dense"`` also instantiates the general kernels for the dense regions'
+    programs (a minute or two per region with long programs), ``"all"`` for every region."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
         raise AttributeError("only a functionalized jit script can be built")
     aot, specialized = _compile(fn, example_input, padded_outputs)
     source, key = (fn, _shape_key(example_input)) if specialized else (None, None)
+    if compile_kernels:
+        from . import aot as _aot
+        _aot.compile_missing(aot, tables=compile_kernels if isinstance(compile_kernels, str) else "none")
     if hip_graph:
         return GraphedFunction(aot, source, key)
     return AotScriptFunction(aot, source, key, lazy_lists=lazy_lists, padded_outputs=padded_outputs)

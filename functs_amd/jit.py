@@ -6,6 +6,7 @@ Same entry points as the reference's ``functs.jit`` (functs/jit/_script.py:12-11
 ``shape_infer`` refines the graph's argument types from example inputs.
 """
 import inspect
+import os
 from typing import List, Sequence
 
 import torch
@@ -176,7 +177,7 @@ class GraphedFunction(AotScriptFunction):
 
 
 def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: bool = False,
-          padded_outputs: bool = False, compile_kernels=False) -> AotScriptFunction:
+          padded_outputs: bool = False, compile_kernels=None) -> AotScriptFunction:
     """Form fused regions in a functionalized script and return the callable
     (functs/jit/_script.py:58-73).  ``hip_graph=True`` returns a ``GraphedFunction``.
     ``lazy_lists=True`` (a function that builds into ONE fused region only): List[Tensor] results
@@ -194,11 +195,16 @@ def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: 
     later processes load them from the cache): where the reference generates and compiles code
     per subgraph when the operator is made (fait/fuser/graph_builder.cpp:259-712).
     ``compile_kernels="dense"`` also instantiates the general kernels for the dense regions'
-    programs (a minute or two per region with long programs), ``"all"`` for every region."""
+    programs (a minute or two per region with long programs), ``"all"`` for every region.  Left
+    at None the environment decides: ``FUNCTS_AMD_COMPILE_KERNELS=1`` (or ``dense`` / ``all``)
+    switches it on for code that calls ``build`` the reference's way."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
         raise AttributeError("only a functionalized jit script can be built")
     aot, specialized = _compile(fn, example_input, padded_outputs)
     source, key = (fn, _shape_key(example_input)) if specialized else (None, None)
+    if compile_kernels is None:
+        env = os.environ.get("FUNCTS_AMD_COMPILE_KERNELS", "0").strip().lower()
+        compile_kernels = env if env in ("dense", "all") else env not in ("", "0", "false", "no")
     if compile_kernels:
         from . import aot as _aot
         _aot.compile_missing(aot, tables=compile_kernels if isinstance(compile_kernels, str) else "none")

@@ -126,6 +126,25 @@ def test_build_with_compile_kernels_links_the_row_stream_kernel_of_a_new_program
     assert len([f for f in os.listdir(aot.kernel_cache_dir()) if f.endswith(".so")]) == 1
 
 
+@needs_hipcc
+def test_the_environment_switches_it_on_for_code_that_builds_the_reference_way(tmp_path, monkeypatch):
+    import functs_amd.jit as fj
+    monkeypatch.setenv("FUNCTS_AMD_KERNEL_CACHE", str(tmp_path))
+    pred, anchors, strides = _args(batch=1, n=640, seed=3)
+
+    def other(pred: torch.Tensor, anchors: torch.Tensor, strides: torch.Tensor):
+        obj = pred[0][:, 4].sigmoid()
+        keep = obj * 2.0 >= 1.1
+        return (pred[0].tanh() * strides.unsqueeze(-1))[keep], (anchors[:, 0] + obj)[keep]
+
+    monkeypatch.setenv("FUNCTS_AMD_COMPILE_KERNELS", "0")
+    first = aot.plan(fj.build(fj.script(other), [pred, anchors, strides]))
+    if len(first) != 1 or "row-stream key" not in first[0] or "(kernel linked)" in first[0]:
+        pytest.skip("not a program for this test: %r" % (first,))
+    monkeypatch.setenv("FUNCTS_AMD_COMPILE_KERNELS", "1")
+    assert "(kernel linked)" in aot.plan(fj.build(fj.script(other), [pred, anchors, strides]))[0]
+
+
 @pytest.mark.gpu
 @needs_hipcc
 def test_a_program_built_with_compile_kernels_equals_eager():

@@ -467,6 +467,7 @@ int fx_plan_rowstream_launch(const fx_plan* p, uint32_t chunk_rows, uint32_t sub
   rl.chunk_rows = chunk_rows;
   rl.chunks = (rl.n_rows + chunk_rows - 1) / chunk_rows;
   rl.sub_rows = sub_rows;
+  fx_rs_finish_geometry(&rl);
   memcpy(out, &rl, sizeof(rl));
   return (int)sizeof(rl);
 }
@@ -968,6 +969,7 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
   rl->chunk_rows = pl->rs_chunk_rows;
   rl->side_lds = pl->rs_side_lds;
   rl->chunks = (ri.n_rows + rl->chunk_rows - 1) / rl->chunk_rows;
+  fx_rs_finish_geometry(rl);
   const uint32_t cr = rl->chunk_rows;
   // A launch whose first sub-tiles alone are megabytes of requests floods the memory system: there
   // the counts get a head start.  A small launch would only lose the time.

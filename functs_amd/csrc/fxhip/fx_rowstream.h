@@ -171,13 +171,14 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
   // costs registers, which the launches that fit do not pay.)
   const uint32_t n_chunks_all = la.chunks * la.n_tasks;
   for (uint32_t b = blockIdx.x;;) {
-    const uint32_t task = b / la.chunks, chunk = b - task * la.chunks;
+    const uint32_t task = fx_fastdiv(b, la.chunks_magic, la.chunks_shift), chunk = b - task * la.chunks;
     const uint32_t c_r0 = chunk * la.chunk_rows;
-    const uint32_t c_rows = min(la.chunk_rows, la.n_rows - c_r0);   // >= 1 (host)
-    // sub-tiles of equal size, at most la.sub_rows rows each
-    const uint32_t n_sub0 = (c_rows + la.sub_rows - 1u) / la.sub_rows;
-    const uint32_t sub_rows = (c_rows + n_sub0 - 1u) / n_sub0;
-    const uint32_t n_sub = (c_rows + sub_rows - 1u) / sub_rows;
+    // rows of the chunk (>= 1) and its sub-tiles of equal size, at most la.sub_rows rows each: the
+    // host has divided (fx_rs_finish_geometry)
+    const bool last_chunk = chunk + 1u == la.chunks;
+    const uint32_t c_rows = last_chunk ? la.rows_last : la.chunk_rows;
+    const uint32_t sub_rows = last_chunk ? la.sub_rows_last : la.sub_rows_whole;
+    const uint32_t n_sub = last_chunk ? la.n_sub_last : la.n_sub_whole;
     FxRsRt rt{la, task, {}, {}};
     // What the rows' own code reads from memory besides the window (a few words per row: anchors,
     // strides ...) is fetched for all rows of the chunk before the first sub-tile, into a table in LDS.

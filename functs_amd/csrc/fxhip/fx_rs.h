@@ -76,10 +76,30 @@ struct FxRsLaunch {
   uint32_t side_lds;            // the chunk keeps a table of its rows' side values in LDS (0: a row loads them when its turn comes)
   uint32_t late_tell;           // tuning aid: the task's last chunk looks back where the others do (the host hears the total later)
   uint32_t pad0;
+  // what a workgroup would otherwise divide for: b / chunks by multiplication, and the sub-tiles
+  // (equal in size, at most sub_rows rows) of a whole chunk and of a task's last chunk
+  uint32_t chunks_magic, chunks_shift;
+  uint32_t sub_rows_whole, n_sub_whole;
+  uint32_t rows_last, sub_rows_last, n_sub_last;
+  uint32_t pad1;
   uint32_t* status;             // one word per chunk, tagged with the epoch
   uint32_t* totals;             // pinned host memory: kept rows per task
 };
 static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte boundary");
+// the derived fields of a launch block whose n_rows, chunk_rows, chunks and sub_rows are set
+static inline void fx_rs_finish_geometry(FxRsLaunch* rl) {
+  fx_fastdiv_make(rl->chunks ? rl->chunks : 1u, &rl->chunks_magic, &rl->chunks_shift);
+  auto split = [&](uint32_t rows, uint32_t* sub_rows, uint32_t* n_sub) {
+    const uint32_t cap = rl->sub_rows ? rl->sub_rows : 1u;
+    const uint32_t n0 = rows ? (rows + cap - 1u) / cap : 1u;
+    *sub_rows = rows ? (rows + n0 - 1u) / n0 : 1u;
+    *n_sub = rows ? (rows + *sub_rows - 1u) / *sub_rows : 0u;
+  };
+  const uint32_t whole = rl->chunk_rows;
+  rl->rows_last = rl->chunks ? rl->n_rows - (rl->chunks - 1u) * whole : 0u;
+  split(whole, &rl->sub_rows_whole, &rl->n_sub_whole);
+  split(rl->rows_last, &rl->sub_rows_last, &rl->n_sub_last);
+}
 
 // ---- host side: generated kernels linked into the library ----
 struct FxRsKernel {

@@ -28,8 +28,9 @@ Or at run time, where ``hipcc`` is at hand (the reference's way: code per subgra
 operator is first made): ``functs_amd.jit.build(..., compile_kernels=True)`` or
 ``aot.compile_missing(fn)`` plans the function's regions, compiles the units that are not linked
 into small shared objects of their own and loads them; they register with the loaded library
-like the linked ones (row-stream units take seconds and are the default; the general kernels
-instantiated for a region's programs, `tables="dense"` / `"all"`, up to a minute or two).  The objects are kept in ``kernel_cache_dir()`` and
+like the linked ones (row-stream units take seconds; the general kernels instantiated for a
+region's programs seconds to minutes, so by default only dense regions with short programs get
+them: `tables`).  The objects are kept in ``kernel_cache_dir()`` and
 loaded again by every later process (``load_cached_kernels``, called when the package is
 imported).
 
@@ -43,6 +44,7 @@ import ctypes
 import glob
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import tempfile
@@ -72,6 +74,7 @@ _FXHIP_DIR = os.path.dirname(SPEC_DIR)
 _HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]   # as csrc/fxhip/Makefile
 _loaded = {}   # path -> CDLL (kept: the library calls into them)
+AUTO_TABLE_INSNS = 256   # program tables up to this many instructions are compiled without being asked for (about 20 s)
 
 
 def _abi_tag() -> str:
@@ -117,13 +120,14 @@ def load_cached_kernels() -> int:
     return len(_loaded)
 
 
-def compile_sources(directory: str, verbose: bool = False, tables: str = "none"):
+def compile_sources(directory: str, verbose: bool = False, tables: str = "auto"):
     """Compiles the generated units of `directory` that have no object in the cache yet into
     shared objects there and loads them.  Every row-stream unit (``fx_rs_*.hip``: straight-line
     code, seconds) is compiled; of the program tables (``fx_spec_*.hip``: the general kernels
-    instantiated for a region's programs, up to a minute or two each) none (`tables` = "none",
-    the default: dense regions and two-pass forms keep the interpreter), those of dense regions
-    ("dense") or all ("all").  Returns the names compiled."""
+    instantiated for a region's programs: 5 s for a few instructions, 10 s for fifty, two minutes
+    for 1 500) those of dense regions with at most AUTO_TABLE_INSNS instructions (`tables` =
+    "auto", the default), of all dense regions ("dense"), all ("all") or none ("none").  Regions
+    left out keep the interpreter.  Returns the names compiled."""
     cc = hipcc_path()
     if cc is None:
         raise RuntimeError("no hipcc found (PATH, $HIPCC, /opt/rocm/bin): generate the sources with aot.capture() and "
@@ -136,8 +140,11 @@ def compile_sources(directory: str, verbose: bool = False, tables: str = "none")
         name = os.path.splitext(os.path.basename(src))[0]
         if name.startswith("fx_spec_"):
             with open(src) as fh:
-                dense = "FX_SPEC_DENSE" in fh.read()
-            if tables == "none" or (tables == "dense" and not dense):
+                text = fh.read()
+            dense = "FX_SPEC_DENSE" in text
+            m = re.search(r"FxInsn code\[(\d+)\]", text)
+            n_insn = int(m.group(1)) if m else 1 << 30
+            if tables == "none" or (tables == "dense" and not dense) or (tables == "auto" and not (dense and n_insn <= AUTO_TABLE_INSNS)):
                 continue
         obj = os.path.join(out_dir, name + ".so")
         if not os.path.isfile(obj):
@@ -156,7 +163,7 @@ def compile_sources(directory: str, verbose: bool = False, tables: str = "none")
     return done
 
 
-def compile_missing(fn=None, planner=None, verbose: bool = False, tables: str = "none"):
+def compile_missing(fn=None, planner=None, verbose: bool = False, tables: str = "auto"):
     """Plans the regions of a built function (or whatever `planner()` plans) for the static types
     of its example, and compiles and loads the kernels that are not linked in.  Needs no GPU.
     Returns the names of the units compiled now."""

@@ -189,13 +189,15 @@ def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: 
     kept-row counts, which come as one more tensor at the end of the result tuple (int32, pinned
     host memory that the kernels write; rows from counts[task] on hold no values): for callers that
     pass the results on to work on the same stream.
-    ``compile_kernels=True``: the row compactions of the built function that have a row-stream
-    form but no kernel linked into the library get theirs now (generated for the example's static
-    types, compiled with hipcc into the kernel cache, a few seconds per region the first time;
-    later processes load them from the cache): where the reference generates and compiles code
-    per subgraph when the operator is made (fait/fuser/graph_builder.cpp:259-712).
-    ``compile_kernels="dense"`` also instantiates the general kernels for the dense regions'
-    programs (a minute or two per region with long programs), ``"all"`` for every region.  Left
+    ``compile_kernels=True``: the regions of the built function that have no kernels linked into
+    the library get theirs now: row compactions with a row-stream form their one-launch kernel,
+    dense regions with programs of up to 256 instructions the compiled dense kernels (generated
+    for the example's static types, compiled with hipcc into the kernel cache, 3 to 20 seconds per
+    region the first time; later processes load them from the cache): where the reference
+    generates and compiles code per subgraph when the operator is made
+    (fait/fuser/graph_builder.cpp:259-712).  ``compile_kernels="dense"`` instantiates the general
+    kernels for every dense region's programs (two minutes for 1 500 instructions), ``"all"`` for
+    every region, ``"none"`` for none (row-stream kernels only).  Left
     at None the environment decides: ``FUNCTS_AMD_COMPILE_KERNELS=1`` (or ``dense`` / ``all``)
     switches it on for code that calls ``build`` the reference's way."""
     if not isinstance(fn, (torch.jit.ScriptFunction, torch.jit.ScriptModule)):
@@ -204,10 +206,10 @@ def build(fn, example_input: List[object], hip_graph: bool = False, lazy_lists: 
     source, key = (fn, _shape_key(example_input)) if specialized else (None, None)
     if compile_kernels is None:
         env = os.environ.get("FUNCTS_AMD_COMPILE_KERNELS", "0").strip().lower()
-        compile_kernels = env if env in ("dense", "all") else env not in ("", "0", "false", "no")
+        compile_kernels = env if env in ("dense", "all", "none", "auto") else env not in ("", "0", "false", "no")
     if compile_kernels:
         from . import aot as _aot
-        _aot.compile_missing(aot, tables=compile_kernels if isinstance(compile_kernels, str) else "none")
+        _aot.compile_missing(aot, tables=compile_kernels if isinstance(compile_kernels, str) else "auto")
     if hip_graph:
         return GraphedFunction(aot, source, key)
     return AotScriptFunction(aot, source, key, lazy_lists=lazy_lists, padded_outputs=padded_outputs)

@@ -166,3 +166,44 @@ def test_a_program_built_with_compile_kernels_equals_eager():
     assert_close(got[2].cpu(), want[2], "objectness")
     assert_close(got[1].cpu(), want[1], "class scores")
     assert_boxes_close(got[0].cpu(), want[0], "boxes")
+
+
+@needs_hipcc
+def test_a_dense_region_with_a_short_program_gets_compiled_kernels_too(tmp_path, monkeypatch):
+    import functs_amd.jit as fj
+    monkeypatch.setenv("FUNCTS_AMD_KERNEL_CACHE", str(tmp_path))
+
+    def short(x: torch.Tensor, y: torch.Tensor):
+        z = x.clone()
+        z[:, 1:3] = (y[:, 1:3] * 1.5 - x[:, 1:3]).tanh()
+        return z.relu() + y
+
+    ex = [torch.rand(300, 40), torch.rand(300, 40)]
+    first = aot.plan(fj.build(fj.script(short), ex))
+    if len(first) != 1 or "interpreted" not in first[0]:
+        pytest.skip("not a program for this test: %r" % (first,))
+    after = aot.plan(fj.build(fj.script(short), ex, compile_kernels=True))
+    assert "compiled" in after[0], after
+
+
+@pytest.mark.gpu
+@needs_hipcc
+def test_a_dense_program_built_with_compile_kernels_equals_eager_and_the_interpreter():
+    import functs_amd.jit as fj
+    dev = torch.device("cuda:0")
+
+    def short(x: torch.Tensor, y: torch.Tensor):
+        z = x.clone()
+        z[:, 2:5] = (y[:, 2:5] * 0.75 - x[:, 2:5]).tanh()
+        return z.relu() + y
+
+    torch.manual_seed(8)
+    ex = [torch.randn(1000, 33), torch.randn(1000, 33)]
+    want = short(*ex)
+    dex = [t.to(dev) for t in ex]
+    interpreted = fj.build(fj.script(short), dex, compile_kernels=False)(*dex).cpu()
+    fn = fj.build(fj.script(short), dex, compile_kernels=True)
+    assert "compiled" in aot.plan(fn)[0], aot.plan(fn)
+    got = fn(*dex).cpu()
+    assert torch.equal(got, interpreted)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-6)

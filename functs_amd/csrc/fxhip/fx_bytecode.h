@@ -268,8 +268,9 @@ struct FxLeanOut {
   uint32_t block_begin, task_stride, unit_items, inner, vd, gpr, gp_magic, gp_shift, n_groups;   // as in FxOut
   int32_t lead_base, lead_tcoef;
   int32_t lead_cf[FX_MAXR];
+  uint32_t rowseg;              // 0, or as FxOut::rowseg of an output whose items are whole rows (FxOut::rowwave); then
+                                // n_groups holds the number of rows
   uint32_t dms[FX_MAXR - 1][3]; // FxOut::dim, magic, shift of dimensions 1 .. FX_MAXR - 1
-  uint32_t pad;
 };
 struct FxLeanArgs {
   uint32_t blob_words, n_p, n_s, total_units;   // as in FxLaunchInfo

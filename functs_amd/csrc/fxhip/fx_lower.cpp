@@ -2254,8 +2254,8 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   hp->off_taskmap = off_taskmap;
   hp->total_words = (uint32_t)blob.size();
 
-  // One class of at most FX_FAST_OUTS outputs of 32-bit elements, none of them reduced over
-  // rows, tasks numbered in order, few enough pointers and scalars: the region fits the lean
+  // One class of at most FX_FAST_OUTS outputs of 32-bit elements, tasks numbered in order, few
+  // enough pointers and scalars: the region fits the lean
   // dense kernel's argument block (the kernel itself exists only for compiled programs).
   memset(&P->lean, 0, sizeof(P->lean));
   if (P->mode == FX_MODE_DENSE && classes.size() == 1 && !classes[0].outs.empty() &&
@@ -2266,8 +2266,7 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
     bool fits = taskmap.size() == (size_t)T;
     for (size_t i = 0; fits && i < taskmap.size(); ++i) fits = taskmap[i] == (uint32_t)i;
     for (const FxOut& od : cb.outs)
-      fits = fits && !od.rowwave &&
-             ((od.dtype == FX_F32 && od.vt == FX_VT_F) || (od.dtype == FX_I32 && od.vt == FX_VT_I));
+      fits = fits && ((od.dtype == FX_F32 && od.vt == FX_VT_F) || (od.dtype == FX_I32 && od.vt == FX_VT_I));
     if (fits) {
       FxLeanArgs& f = P->lean;
       f.blob_words = (uint32_t)blob.size();
@@ -2295,7 +2294,8 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
         lo.gpr = od.gpr;
         lo.gp_magic = od.gp_magic;
         lo.gp_shift = od.gp_shift;
-        lo.n_groups = od.n_groups;
+        lo.n_groups = od.rowwave ? (od.inner ? od.numel / od.inner : 0u) : od.n_groups;
+        lo.rowseg = od.rowwave ? od.rowseg : 0u;
         for (int k = 1; k < FX_MAXR; ++k) {
           lo.dms[k - 1][0] = od.dim[k];
           lo.dms[k - 1][1] = od.magic[k];

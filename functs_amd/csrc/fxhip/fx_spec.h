@@ -379,7 +379,7 @@ struct FxSpec {
 // program it is still tens of kilobytes of code that a workgroup jumps through: on a small
 // region the kernel's time is the start of its workgroups (argument segment, descriptor
 // staging, instruction fetch), not the data.  Regions of one task class with one or two
-// outputs of 32-bit elements and no row reductions (FxLeanArgs, decided at plan time) run this
+// outputs of 32-bit elements (FxLeanArgs, decided at plan time) run this
 // kernel instead: unit, output record, leading load and pointers come from a short argument
 // block through scalar loads, the leading loads of the unit are issued first, and the
 // descriptor is staged into LDS behind them, and only if a program of the region reads it
@@ -435,18 +435,33 @@ __device__ __forceinline__ void fx_lean_out(const FX_AS4 uint32_t* od, const uin
   const uint32_t vd = od[FX_W(FxLeanOut, vd)];
   const uint32_t gpr = od[FX_W(FxLeanOut, gpr)];
   const uint32_t gp_magic = od[FX_W(FxLeanOut, gp_magic)], gp_shift = od[FX_W(FxLeanOut, gp_shift)];
-  const uint32_t n_groups = od[FX_W(FxLeanOut, n_groups)];
+  const uint32_t n_groups = od[FX_W(FxLeanOut, n_groups)];   // (rows, for an output whose items are whole rows)
   const uint32_t item0 = ublock * (4u * kmax) + wave * kmax;
-  const uint32_t n_items = (n_groups + 63u) / 64u;
+  // An output that is reduced over its rows (FX_WMAX / FX_WSUM) takes one row per segment of
+  // rowseg lanes, so that the wave-wide reductions see exactly the elements of that row.
+  const uint32_t rowseg = od[FX_W(FxLeanOut, rowseg)];
+  const uint32_t segsh = 31u - (uint32_t)__builtin_clz(rowseg | 1u);
+  const uint32_t rows_per_item = 64u >> segsh;
+  const uint32_t n_items = rowseg ? (n_groups + rows_per_item - 1u) / rows_per_item : (n_groups + 63u) / 64u;
   const bool have = item0 < n_items;
 
   // item k of this wave: 64 lane groups of FX_V consecutive elements along the last dimension
   auto make_item = [&](uint32_t k, uint32_t (&e)[FX_V], uint32_t& M, FxCoord<R>& q) {
-    const uint32_t g = (item0 + k) * 64u + lane;
-    const bool live = g < n_groups;
-    const uint32_t gg = live ? g : 0u;
-    const uint32_t row = fx_fastdiv(gg, gp_magic, gp_shift);
-    const uint32_t col0 = (gg - row * gpr) * FX_V;
+    uint32_t row, col0;
+    bool live;
+    if (rowseg) {
+      const uint32_t seg = lane >> segsh;
+      row = (item0 + k) * rows_per_item + seg;
+      col0 = (lane - seg * rowseg) * FX_V;
+      live = row < n_groups;
+      if (!live) row = 0;
+    } else {
+      const uint32_t g = (item0 + k) * 64u + lane;
+      live = g < n_groups;
+      const uint32_t gg = live ? g : 0u;
+      row = fx_fastdiv(gg, gp_magic, gp_shift);
+      col0 = (gg - row * gpr) * FX_V;
+    }
     M = 0;
 #pragma unroll
     for (int j = 0; j < FX_V; ++j) {
@@ -475,6 +490,7 @@ __device__ __forceinline__ void fx_lean_out(const FX_AS4 uint32_t* od, const uin
   // every wave of the workgroup comes by here, with or without items: the staging has a barrier
   FxCtx cx = get_cx();
   if (!have) return;
+  cx.wseg = rowseg ? rowseg : 64u;
   if constexpr (en.pure != 0) {
 #pragma unroll
     for (uint32_t k = 0; k < FX_K; ++k) {

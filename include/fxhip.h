@@ -276,8 +276,8 @@ int fx_plan_spec_source(const fx_plan*, const char* label, char* buf, size_t cap
 void fx_set_specialization(int on);             /* process-wide switch, default on (FXHIP_SPECIALIZE=0: off) */
 int fx_specialization_count(void);              /* specialised regions linked into the library */
 void fx_launch_stats(uint64_t* total, uint64_t* specialised); /* region kernel launches of this process so far */
-/* Dense regions of one task class with one or two outputs of 32-bit elements and no reduction
- * over rows are run by a short kernel of their own when their programs are compiled: it takes
+/* Dense regions of one task class with one or two outputs of 32-bit elements are run by a short
+ * kernel of their own when their programs are compiled: it takes
  * what a workgroup needs in front of its first load from a small argument block and stages the
  * descriptor only if a program reads it (on a region of a few MB the start of the workgroups is
  * what a launch costs).  Same results as the general kernel, bit for bit.

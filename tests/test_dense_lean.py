@@ -5,8 +5,9 @@ their own when their programs are compiled (fx_dense_lean, the counterpart of th
 one-element-per-thread launch of fait/tensorexpr/cuda_codegen_tssa.cpp:1167-1306).  It has to
 give the general kernel's results bit for bit: same item geometry, same instruction steps.
 The programs here are ones whose compiled kernels are linked into the library: the collapsed
-get_started loop (examples/get_started.py:10-15) and an elementwise chain, at shapes that end
-inside a lane group, inside an item, inside a unit and at both unit sizes."""
+get_started loop (examples/get_started.py:10-15), an elementwise chain (at shapes that end
+inside a lane group, inside an item, inside a unit and at both unit sizes), SSD's decode + softmax
+and a region with reduction loops."""
 import pytest
 import torch
 
@@ -88,6 +89,46 @@ def test_partial_loop_keeps_the_other_rows(lean_switch):
     want[:123] += 1
     assert torch.equal(lean, general)
     assert torch.equal(lean, want)
+
+
+@gpu
+@pytest.mark.parametrize("rows,classes", [(8732, 81), (100, 81), (7, 81), (513, 21)])
+def test_rows_that_are_reduced_on_the_lean_kernel(rows, classes, lean_switch):
+    """SSD's decode + softmax (functs/benchmark/ai_model/ssd/ssd_bbox.py:121-154, 163-170): the
+    scores take one row per segment of a wave and are reduced inside it; two outputs."""
+    dev = torch.device("cuda:0")
+    torch.manual_seed(rows)
+    loc = torch.randn(1, rows, 4, device=dev)
+    conf = torch.randn(1, rows, classes, device=dev) * 3
+    priors = torch.rand(rows, 4, device=dev)
+    r = configs.build_c3_decode()
+    bc = r.bind(loc, conf, priors)
+    if not r.specialized(loc, conf, priors):
+        pytest.skip("no compiled kernels linked for this number of classes")
+    assert _lean(bc)
+    bc.launch()
+    lean = [t.clone() for t in bc.results()]
+    _lib.lib.fx_set_dense_lean(0)
+    general = r(loc, conf, priors)
+    torch.cuda.synchronize()
+    assert torch.equal(lean[0], general[0]) and torch.equal(lean[1], general[1])
+    torch.testing.assert_close(lean[1], conf[0].softmax(-1), rtol=1e-5, atol=1e-7)
+
+
+@gpu
+def test_reduction_loops_and_a_row_softmax_on_the_lean_kernel(lean_switch):
+    dev = torch.device("cuda:0")
+    torch.manual_seed(4)
+    x = torch.randn(*configs.COLUMN_STANDARDIZE_SHAPE, device=dev)
+    r = configs.build_column_standardize()
+    bc = r.bind(x)
+    assert _lean(bc)
+    bc.launch()
+    lean = [t.clone() for t in bc.results()]
+    _lib.lib.fx_set_dense_lean(0)
+    general = r(x)
+    torch.cuda.synchronize()
+    assert torch.equal(lean[0], general[0]) and torch.equal(lean[1], general[1])
 
 
 @gpu

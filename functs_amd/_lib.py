@@ -195,6 +195,7 @@ _sig("fx_lstm_stack_fits", ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_in
 _sig("fx_lstm_stack_workspace_bytes", ctypes.c_size_t, _i, _i, _i)
 _sig("fx_lstm_stack", _i, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _fp, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp)
 _sig("fx_set_lstm_spin_limit", None, ctypes.c_uint32)
+_sig("fx_set_totals_spin_us", None, ctypes.c_uint32)
 _sig("fx_device_count", _i)
 _sig("fx_copy_bytes", _i, _vp, _vp, ctypes.c_size_t, _vp)
 _sig("fx_copy_bytes_timed_sets", _i, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p), _i, ctypes.c_size_t, _i, _vp,

@@ -269,6 +269,7 @@ static std::atomic<uint32_t> g_stream_spin{[] {
   const char* e = getenv("FXHIP_STREAM_SPIN");
   return e ? (uint32_t)strtoul(e, nullptr, 10) : 4000u;
 }()};
+static std::atomic<uint32_t> g_totals_spin_us{2000u};   // microseconds that fx_region_wait_totals polls from the host before it blocks in the stream
 static std::atomic<uint32_t> g_lstm_spin{1000000u};   // polls of a wait of fx_lstm_stack before it is given up
 static std::mutex g_dump_mu;
 static std::string g_dump_dir;
@@ -1336,11 +1337,14 @@ int fx_region_wait_totals(const fx_plan* plan, const uint32_t* totals_host, void
   const volatile uint32_t* tot = totals_host;
   const int T = pl->region->degree;
   // The count of a task is stored by its last tile early in the second pass, through
-  // host-coherent memory: it is usually here well before the kernel has finished.  If the
-  // stream has drained without all of them showing up (memory that the host does not see
-  // until then), a synchronisation settles it.
+  // host-coherent memory: it is usually here well before the kernel has finished, and the
+  // host looks for it from its own core.  Counts that take longer than the polling budget
+  // (a stream with other work queued ahead of the launch, memory that the host does not see
+  // until the stream has drained) are waited for in the runtime's stream synchronisation,
+  // which does not keep a core busy for that long.
   using clock = std::chrono::steady_clock;
   const clock::time_point t0 = clock::now();
+  const clock::duration budget = std::chrono::microseconds(g_totals_spin_us.load(std::memory_order_relaxed));
   clock::time_point next_query = t0 + std::chrono::microseconds(50);
   for (;;) {
     bool all = true;
@@ -1349,12 +1353,13 @@ int fx_region_wait_totals(const fx_plan* plan, const uint32_t* totals_host, void
       std::atomic_thread_fence(std::memory_order_acquire);
       return FX_OK;
     }
-    __builtin_ia32_pause();
     const clock::time_point now = clock::now();
+    if (now - t0 >= budget) break;
+    __builtin_ia32_pause();
     if (now >= next_query) {
       // the runtime is asked rarely: a query takes its locks and slows the launches of other threads
       const hipError_t q = hipStreamQuery(stream);
-      if (q == hipSuccess || now - t0 > std::chrono::seconds(10)) break;
+      if (q == hipSuccess) break;
       if (q != hipErrorNotReady) HIP_OK(q);
       next_query = now + std::chrono::microseconds(50);
     }
@@ -1482,6 +1487,7 @@ int fx_lstm_stack(const float* x, const float* wih, const float* whh, const floa
   g_spec_launches.fetch_add(1, std::memory_order_relaxed);
   return FX_OK;
 }
+void fx_set_totals_spin_us(uint32_t us) { g_totals_spin_us.store(us, std::memory_order_relaxed); }
 void fx_set_lstm_spin_limit(uint32_t polls) { g_lstm_spin.store(polls, std::memory_order_relaxed); }
 
 // ---- detection tail (fx_nms.hip) ----

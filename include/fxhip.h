@@ -303,11 +303,14 @@ int fx_region_run(fx_region*, const fx_plan*, const fx_arg* args, int n_args, vo
 /* Returns once every task's kept-row count of the last fx_region_run on `stream` with this
  * totals_host is readable.  The counts are stored early in the second pass, so this usually
  * returns while the kernels still run: the caller can size its output views and go on; the
- * outputs themselves are valid in stream order, like after any asynchronous launch.  Falls
- * back to synchronising the stream.  Where ATen's nonzero / masked index synchronise
+ * outputs themselves are valid in stream order, like after any asynchronous launch.  The
+ * calling thread polls the pinned words for at most fx_set_totals_spin_us microseconds (default
+ * 2000; 0: not at all) and then blocks in a synchronisation of the stream, so a launch queued
+ * behind long work does not keep a core busy.  Where ATen's nonzero / masked index synchronise
  * (the reference leaves x[mask] to them, convert_to_tensorssa.cpp:422-443). */
 #define FX_TOTAL_PENDING 0xffffffffu
 int fx_region_wait_totals(const fx_plan*, const uint32_t* totals_host, void* stream);
+void fx_set_totals_spin_us(uint32_t microseconds);
 
 /* fx_region_run with a HIP event pair around every kernel on `stream`; waits for
  * the last event and returns the duration of each launch in milliseconds

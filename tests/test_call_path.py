@@ -97,6 +97,26 @@ def test_the_direct_call_returns_what_the_interpreter_returns(name, small):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name,small", [("c2", dict(grids=[4, 6, 8])), ("c5", dict(grids=[4, 6, 8], batch=5)), ("c3", dict(n_priors=500, n_cls=9))])
+def test_kept_row_counts_waited_for_in_the_stream_give_the_same_results(name, small):
+    """With a polling budget of 0 the operator does not look for the counts from the host at all:
+    it blocks in the stream's synchronisation and finds them afterwards."""
+    from functs_amd import _lib
+    args = INPUTS[name](4, **small)
+    fn = fj.build(fj.script(PROGRAMS[name]), list(args))
+    gargs = _cuda(args)
+    print("counts from the drained stream", name, flush=True)
+    ref = [t.clone() for t in _flat(fn(*gargs))]
+    _lib.lib.fx_set_totals_spin_us(0)
+    try:
+        got = [_flat(fn(*gargs)) for _ in range(3)]
+    finally:
+        _lib.lib.fx_set_totals_spin_us(2000)
+    for g in got:
+        assert len(g) == len(ref) and all(x.shape == y.shape and torch.equal(x, y) for x, y in zip(g, ref))
+
+
+@pytest.mark.gpu
 def test_lazy_lists_hold_the_same_tensors():
     args = INPUTS["c5"](2, grids=[4, 6, 8], batch=5)
     plain = fj.build(fj.script(PROGRAMS["c5"]), list(args))

@@ -171,6 +171,9 @@ _sig("fx_launch_stats", None, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ct
 _sig("fx_region_marshal", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,
      ctypes.c_size_t)
 _sig("fx_dyn_bytes", ctypes.c_size_t)
+_sig("fx_plan_table_sizes", _i, _vp, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(_i))
+_sig("fx_region_marshal_tables", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp,
+     ctypes.POINTER(ctypes.c_uint64), ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint32), ctypes.c_size_t)
 _sig("fx_region_run", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp)
 _sig("fx_region_run_timed", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,
      ctypes.POINTER(ctypes.c_float), _i, _ip)

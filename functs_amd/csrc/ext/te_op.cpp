@@ -579,8 +579,9 @@ class RegionRunner {
         ptrs[(size_t)o * degree + t] = base + slot_of[(size_t)o * degree + t].offset_elems * item;
     }
     Workspace ws;
-    if (compact_) {
-      ws = var->take(fx_plan_scratch_bytes(plan), degree, device, (void*)stream.stream());
+    const size_t scratch_bytes = fx_plan_scratch_bytes(plan);   // (a dense map of very many tasks keeps its tables there)
+    if (compact_ || scratch_bytes > 0) {
+      ws = var->take(scratch_bytes, degree, device, (void*)stream.stream());
       ws.stream = (void*)stream.stream();
     }
     checkAsyncError();
@@ -629,8 +630,9 @@ class RegionRunner {
       return;
     }
     FX_OK_OR_THROW(fx_region_run(var->region, plan, args.data(), (int)args.size(), ptrs.data(),
-                                 compact_ ? ws.scratch.data_ptr() : nullptr,
+                                 ws.scratch.defined() ? ws.scratch.data_ptr() : nullptr,
                                  compact_ ? (uint32_t*)ws.totals.data_ptr() : nullptr, (void*)stream.stream()));
+    if (!compact_ && ws.scratch.defined()) var->give(std::move(ws));   // (the next borrower is ordered behind this launch)
     clock.tick(HS_LAUNCH);
     // The tasks' tensors: views of the block, made while the kernels run.
     std::vector<at::Tensor> flat;   // [output][task]

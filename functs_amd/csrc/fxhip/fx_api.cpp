@@ -39,6 +39,7 @@ bool fx_spec_has_stream(const FxSpecKernels* spec);
 bool fx_spec_has_lean(const FxSpecKernels* spec);
 // fx_head.hip
 hipError_t fx_launch_head_stream(const FxHeadLaunch& hl, const FxDyn* dyn, hipStream_t stream);
+hipError_t fx_upload_words(const uint64_t* words, size_t n_words, void* dst, hipStream_t stream);
 hipError_t fx_head_resident(uint32_t lds_bytes, uint32_t* workgroups, uint32_t* per_cu);
 uint32_t fx_head_lds_bytes(const FxHeadLaunch& hl);
 // fx_cmap.hip
@@ -576,8 +577,15 @@ int fx_async_error_take(int mask) {
 // `safe`: a device address that can always be read.  Kernels clamp the address of
 // an element that is not live to element 0 of its buffer, so a tensor without
 // elements (whose pointer may be null) is given this address instead.
+static int fill_tables(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
+                       uint32_t* totals_host, const void* safe, uint64_t* p_out, uint32_t* s_out, const void* status);
 static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
                     uint32_t* totals_host, const void* safe, FxDyn* dyn, const void* status = nullptr) {
+  if (pl->wide) return fail(FX_E_LIMIT, "the tables of this plan do not fit the kernel argument block (a map of many tasks): fx_region_run uploads them");
+  return fill_tables(pl, args, out_ptrs, scratch, totals_host, safe, dyn->p, dyn->s, status);
+}
+static int fill_tables(const fx::Plan* pl, const fx_arg* args, void* const* out_ptrs, void* scratch,
+                       uint32_t* totals_host, const void* safe, uint64_t* p_out, uint32_t* s_out, const void* status) {
   const fx::Region& R = *pl->region;
   const int T = R.degree;
   auto ptr_of = [&](const fx::PtrSrc& s, int task) -> uint64_t {
@@ -615,12 +623,12 @@ static int fill_dyn(const fx::Plan* pl, const fx_arg* args, void* const* out_ptr
     return u;
   };
   size_t np = pl->sptr.size(), ntp = pl->tptr.size(), ns = pl->sscal.size(), nts = pl->tscal.size();
-  for (size_t i = 0; i < np; ++i) dyn->p[i] = ptr_of(pl->sptr[i], 0);
+  for (size_t i = 0; i < np; ++i) p_out[i] = ptr_of(pl->sptr[i], 0);
   for (int t = 0; t < T; ++t)
-    for (size_t i = 0; i < ntp; ++i) dyn->p[np + t * ntp + i] = ptr_of(pl->tptr[i], t);
-  for (size_t i = 0; i < ns; ++i) dyn->s[i] = scal_of(pl->sscal[i], 0);
+    for (size_t i = 0; i < ntp; ++i) p_out[np + t * ntp + i] = ptr_of(pl->tptr[i], t);
+  for (size_t i = 0; i < ns; ++i) s_out[i] = scal_of(pl->sscal[i], 0);
   for (int t = 0; t < T; ++t)
-    for (size_t i = 0; i < nts; ++i) dyn->s[ns + t * nts + i] = scal_of(pl->tscal[i], t);
+    for (size_t i = 0; i < nts; ++i) s_out[ns + t * nts + i] = scal_of(pl->tscal[i], t);
   if (scalar_overflow) return fail(FX_E_LIMIT, "an integer scalar argument is outside 32 bits (integer arithmetic in regions is 32-bit)");
   if (pl->uses_guard && safe && !err_word(true)) return fail(FX_E_HIP, "no pinned memory for the error word");
   return FX_OK;
@@ -638,6 +646,29 @@ int fx_region_marshal(fx_region* reg, const fx_plan* plan, const fx_arg* args, i
 }
 
 size_t fx_dyn_bytes(void) { return sizeof(FxDyn); }
+
+int fx_plan_table_sizes(const fx_plan* plan, size_t* n_pointers, size_t* n_scalars, int* uploaded) {
+  if (!plan) return fail(FX_E_INVALID, "null argument");
+  const fx::Plan* pl = P(plan);
+  const size_t T = (size_t)pl->region->degree;
+  if (n_pointers) *n_pointers = pl->sptr.size() + pl->tptr.size() * T;
+  if (n_scalars) *n_scalars = pl->sscal.size() + pl->tscal.size() * T;
+  if (uploaded) *uploaded = pl->wide ? 1 : 0;
+  return FX_OK;
+}
+
+int fx_region_marshal_tables(fx_region* reg, const fx_plan* plan, const fx_arg* args, int n_args, void* const* out_ptrs,
+                             void* scratch, uint32_t* totals_host, uint64_t* pointers, size_t pointer_cap,
+                             uint32_t* scalars, size_t scalar_cap) {
+  if (!reg || !plan || !out_ptrs || !pointers || !scalars) return fail(FX_E_INVALID, "null argument");
+  const fx::Plan* pl = P(plan);
+  if (pl->region != &reg->r) return fail(FX_E_INVALID, "plan does not belong to this region");
+  if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
+  size_t np = 0, ns = 0;
+  fx_plan_table_sizes(plan, &np, &ns, nullptr);
+  if (pointer_cap < np || scalar_cap < ns) return fail(FX_E_INVALID, "tables too small (fx_plan_table_sizes)");
+  return fill_tables(pl, args, out_ptrs, scratch, totals_host, nullptr, pointers, scalars, nullptr);
+}
 
 // ---- streaming compaction: per-stream status words ----
 #define FX_STREAM_LDS_LIMIT 64000u   // 64 KiB less the kernel's static tables
@@ -1124,8 +1155,21 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     if (!status) streaming = false;
   }
   FxDyn dyn;
-  rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn, status);
-  if (rc != FX_OK) return rc;
+  if (pl->wide) {
+    // a map of many tasks: the tables go to the end of the caller's scratch memory, in stream
+    // order ahead of the kernels that stage them from there
+    if (!scratch) return fail(FX_E_INVALID, "this plan keeps its tables in scratch memory (fx_plan_scratch_bytes): scratch is null");
+    std::vector<uint64_t> words(pl->wide_bytes / 8, 0);
+    rc = fill_tables(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, words.data(), (uint32_t*)(words.data() + li.n_p), status);
+    if (rc != FX_OK) return rc;
+    void* table = (char*)scratch + pl->wide_off;
+    HIP_OK(fx_upload_words(words.data(), (size_t)li.n_p + ((size_t)li.n_s + 1) / 2, table, stream));
+    li.wide = (uint64_t)(uintptr_t)table;
+    memset(&dyn, 0, sizeof dyn);
+  } else {
+    rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn, status);
+    if (rc != FX_OK) return rc;
+  }
   const uint32_t* sb = (const uint32_t*)pl->dev_blob;
   if (pl->mode == FX_MODE_COMPACT) {
     // Tasks without rows launch no tile: their total is published here.  The others hold a
@@ -1223,6 +1267,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
   const bool compact = pl->mode == FX_MODE_COMPACT;
   if (compact && (!scratch || !totals_host)) return fail(FX_E_INVALID, "compacting region needs scratch and totals per set");
+  if (pl->wide) return fail(FX_E_LIMIT, "fx_region_run_timed_sets: not for a plan whose tables are uploaded (a map of many tasks)");
   hipStream_t stream = (hipStream_t)stream_;
   // one untimed call per set: uploads the descriptor, leaves every set's scratch valid
   for (int i = 0; i < n_sets; ++i) {

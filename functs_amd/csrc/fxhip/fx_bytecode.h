@@ -27,6 +27,8 @@
 #define FX_MASK_DEPTH 16 // nesting depth of predicated regions (4 bits each in a u64)
 #define FX_DYN_P 320     // 8-byte dynamic words passed by value (pointers)
 #define FX_DYN_S 176     // 4-byte dynamic words passed by value (scalars)
+#define FX_WIDE_P 4096   // most pointers of a call whose tables travel through device memory (maps of many tasks)
+#define FX_WIDE_S 4096   // most scalars of such a call
 #define FX_MAX_TPTR 32   // per-task pointers staged in LDS
 #define FX_MAX_TSCAL 32  // per-task scalars staged in LDS
 #define FX_MAGIC 0x46585231u  // "FXR1"
@@ -167,6 +169,7 @@ struct FxLaunchInfo {
   uint32_t side_slot[2], side_stride[2];
   int32_t side_tcoef[2], side_lo[2];
   uint32_t side_span[2], side_words[2];
+  uint64_t wide;        // device address of the call's uploaded tables, or 0 (see FxLaunch)
 };
 
 #define FX_SLOT_TASK 0x40000000  // buffer/scalar slot lives in the per-task table

@@ -1059,6 +1059,7 @@ __device__ __forceinline__ void fx_rows_batch(const FxCtx& cx, const FxLead& ld,
 // ---- workgroup prologue ----------------------------------------------------
 // LDS layout (words): [blob][pointers: 2 words each][scalars][pad][temps]
 struct FxLaunch {
+  uint64_t wide;        // 0, or the device address of the call's tables (n_p pointers, then n_s scalars) where the argument block is too small for them
   uint32_t blob_words;  // multiple of 4
   uint32_t n_p;         // pointers in use in FxDyn::p
   uint32_t n_s;         // scalars in use in FxDyn::s
@@ -1103,6 +1104,10 @@ __device__ __forceinline__ void fx_stage(uint32_t* L, const uint32_t* __restrict
   const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
   const uint64_t* gp = (const uint64_t*)(ka + FX_KERNARG_DYN_OFF);
   const uint32_t* gs = (const uint32_t*)(ka + FX_KERNARG_DYN_OFF + 8 * FX_DYN_P);
+  if (la.wide != 0) {   // a map of many tasks: the tables were uploaded ahead of this launch
+    gp = (const uint64_t*)la.wide;
+    gs = (const uint32_t*)(gp + la.n_p);
+  }
   uint64_t* lp = (uint64_t*)(L + la.blob_words);
   uint32_t* ls = L + la.blob_words + 2 * la.n_p;
   for (uint32_t i = threadIdx.x; i < la.n_p; i += NT) lp[i] = gp[i];

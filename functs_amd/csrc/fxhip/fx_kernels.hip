@@ -26,6 +26,7 @@
 // fait/tensorexpr/functor_parallization.cpp:93-108) and, for the
 // data-dependent part, the ATen nonzero/index calls the reference leaves
 // unfused (functs/csrc/jit/passes/convert_to_tensorssa.cpp:422-443).
+#include <algorithm>
 #include <cstring>
 #include "fx_spec.h"
 
@@ -232,8 +233,34 @@ static hipError_t launch_spec(const void* fn, const uint32_t* sb, const FxLaunch
   return hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds, stream);
 }
 
+// The tables of a call that the kernel argument block cannot hold (a map of many tasks) travel
+// to device memory in pieces: each launch carries one piece by value and stores it.  In stream
+// order like the kernels that read the tables, nothing for the host to keep alive, and a
+// captured graph replays it.
+__global__ __launch_bounds__(FX_BLOCK) void fx_store_words(const FxDyn piece, uint64_t* dst, uint32_t n_words) {
+  (void)piece;   // read through the argument segment: indexing a by-value aggregate would copy it to per-lane memory
+  const uint64_t* src = (const uint64_t*)((const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr());
+  for (uint32_t i = threadIdx.x; i < n_words; i += FX_BLOCK) dst[i] = src[i];
+}
+hipError_t fx_upload_words(const uint64_t* words, size_t n_words, void* dst, hipStream_t stream) {
+  static_assert(sizeof(FxDyn) % 8 == 0, "pieces are whole 8-byte words");
+  const size_t per = sizeof(FxDyn) / 8;
+  FxDyn piece;
+  memset(&piece, 0, sizeof piece);
+  for (size_t at = 0; at < n_words; at += per) {
+    const uint32_t n = (uint32_t)std::min(per, n_words - at);
+    memcpy(&piece, words + at, (size_t)n * 8);
+    uint64_t* d = (uint64_t*)dst + at;
+    void* args[3] = {(void*)&piece, (void*)&d, (void*)&n};
+    const hipError_t e = hipLaunchKernel((const void*)&fx_store_words, dim3(1), dim3(FX_BLOCK), args, 0, stream);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 static FxLaunch make_launch(const FxLaunchInfo& li) {
   FxLaunch la;
+  la.wide = li.wide;
   la.blob_words = li.blob_words;
   la.n_p = li.n_p;
   la.n_s = li.n_s;

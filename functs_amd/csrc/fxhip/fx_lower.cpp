@@ -2169,10 +2169,11 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
   P->tscal = slots.tscal;
   FX_CHECK(P->tptr.size() <= FX_MAX_TPTR, FX_E_LIMIT, "more than " << FX_MAX_TPTR << " per-task tensors");
   FX_CHECK(P->tscal.size() <= FX_MAX_TSCAL, FX_E_LIMIT, "more than " << FX_MAX_TSCAL << " per-task scalars");
-  FX_CHECK(P->sptr.size() + P->tptr.size() * (size_t)T <= FX_DYN_P, FX_E_LIMIT,
-           "tasks x per-task tensors exceeds " << FX_DYN_P << " pointer slots");
-  FX_CHECK(P->sscal.size() + P->tscal.size() * (size_t)T <= FX_DYN_S, FX_E_LIMIT,
-           "tasks x per-task scalars exceeds " << FX_DYN_S << " scalar slots");
+  const size_t n_ptrs = P->sptr.size() + P->tptr.size() * (size_t)T, n_scals = P->sscal.size() + P->tscal.size() * (size_t)T;
+  FX_CHECK(n_ptrs <= FX_WIDE_P, FX_E_LIMIT, "tasks x per-task tensors exceeds " << FX_WIDE_P << " pointer slots");
+  FX_CHECK(n_scals <= FX_WIDE_S, FX_E_LIMIT, "tasks x per-task scalars exceeds " << FX_WIDE_S << " scalar slots");
+  P->wide = n_ptrs > FX_DYN_P || n_scals > FX_DYN_S;
+  if (P->wide) P->stream.ok = false;   // (the one-launch forms read their tables from the kernel arguments)
 
   // scratch: flags [T][max_rows] bytes, counts [T][max_rowtiles] u32
   if (P->mode == FX_MODE_COMPACT) {
@@ -2184,6 +2185,11 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
     P->launches = 2;
   } else {
     P->launches = gb > 0 ? 1 : 0;
+  }
+  if (P->wide) {
+    P->wide_off = P->scratch_bytes;
+    P->wide_bytes = (n_ptrs * 8 + n_scals * 4 + 255) & ~(size_t)255;
+    P->scratch_bytes += P->wide_bytes;
   }
 
   // algorithmic bytes: every referenced input once + dense outputs once
@@ -2357,9 +2363,13 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
     }
   }
   P->spec_key = spec_hash(*P);
-  match_head(P.get());
-  match_classmap(P.get());
-  rs_analyze(P.get());
+  if (!P->wide) {
+    match_head(P.get());
+    match_classmap(P.get());
+    rs_analyze(P.get());
+  } else {
+    P->rs.why = "more per-task buffers than the kernel argument block holds: the tables are uploaded and the general kernels read them";
+  }
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;

@@ -105,6 +105,12 @@ struct Plan {
   uint32_t grid = 0;           // dense grid, or scatter grid in compaction mode
   uint32_t grid_count = 0;     // compaction pass 1
   uint32_t lds_bytes = 0;
+  // A call with more pointers or scalars than the kernel argument block holds (a map of many
+  // tasks): the tables are written to device memory at wide_off of the caller's scratch by small
+  // upload launches ahead of the kernels, which stage them from there.  Such a plan runs the
+  // general kernels only.
+  bool wide = false;
+  size_t wide_off = 0, wide_bytes = 0;
   bool needs_compiled = false;   // the interpreter's temporaries exceed the LDS of a workgroup
   StreamInfo stream;
   FxHeadInfo head;               // the plan is the decode + score filter of a detection head (fx_head.h)

@@ -355,7 +355,7 @@ class BoundCall:
                 ptrs[o * T + t] = ten.data_ptr()
             self.outs.append(row)
         self.ptrs = ptrs
-        self.scratch = torch.empty(max(plan.scratch_bytes, 1), dtype=torch.uint8, device=dev) if plan.compact else None
+        self.scratch = torch.empty(max(plan.scratch_bytes, 1), dtype=torch.uint8, device=dev) if (plan.compact or plan.scratch_bytes > 0) else None
         self.totals = torch.zeros(T, dtype=torch.int32).pin_memory() if plan.compact else None
         self._stream = None
 

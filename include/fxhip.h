@@ -348,6 +348,19 @@ int fx_region_run_timed_sets(fx_region*, const fx_plan*, int n_sets, const fx_ar
 int fx_region_marshal(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
                       void* scratch, uint32_t* totals_host, void* dyn_out, size_t dyn_cap);
 size_t fx_dyn_bytes(void);
+/* A map of many tasks can have more pointers and scalars than that block holds (320 and 176):
+ * up to 4096 of each, fx_region_run then writes the two tables to the end of the caller's scratch
+ * memory (fx_plan_scratch_bytes counts them, also for a region that does not compact) with small
+ * launches ahead of the kernels, which read them from there; such a plan runs the general
+ * kernels (the one-launch forms and the short dense kernel read the argument block), and
+ * fx_region_marshal refuses it.  The reference passes every task's buffers as kernel arguments
+ * and clones the body per task (functor_parallization.cpp:12-111): its limit is the compiler's.
+ * fx_plan_table_sizes: entries of the two tables, and whether the plan uploads them.
+ * fx_region_marshal_tables: the tables themselves, for any plan (host only; tests). */
+int fx_plan_table_sizes(const fx_plan*, size_t* n_pointers, size_t* n_scalars, int* uploaded);
+int fx_region_marshal_tables(fx_region*, const fx_plan*, const fx_arg* args, int n_args, void* const* out_ptrs,
+                             void* scratch, uint32_t* totals_host, uint64_t* pointers, size_t pointer_cap,
+                             uint32_t* scalars, size_t scalar_cap);
 
 /* int64 in regions.  Programs that only MOVE int64 data (select / slice / index / where / cat /
  * *_rev / row compaction ...) are exact for every value: they travel as two 32-bit words.

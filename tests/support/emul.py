@@ -39,11 +39,15 @@ def lstm_emul():
 
 
 def _load():
-    if not os.path.exists(_SO):
+    sources = [os.path.join(_HERE, "fx_emul.cpp"), os.path.join(_HERE, "..", "..", "functs_amd", "csrc", "fxhip", "fx_bytecode.h")]
+    if not os.path.exists(_SO) or any(os.path.exists(s) and os.path.getmtime(s) > os.path.getmtime(_SO) for s in sources):
         build()
     so = ctypes.CDLL(_SO)
     so.fx_emul_run.restype = ctypes.c_int
     so.fx_emul_run.argtypes = [ctypes.POINTER(ctypes.c_uint32), ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+    so.fx_emul_run_tables.restype = ctypes.c_int
+    so.fx_emul_run_tables.argtypes = [ctypes.POINTER(ctypes.c_uint32), ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint64),
+                                      ctypes.POINTER(ctypes.c_uint32), ctypes.c_void_p]
     return so
 
 
@@ -69,12 +73,21 @@ def run(region, *args):
         outs.append(row)
     scratch = torch.zeros(max(p.scratch_bytes, 1), dtype=torch.uint8)
     totals = torch.zeros(T, dtype=torch.int32)
-    dyn = ctypes.create_string_buffer(lib.fx_dyn_bytes())
-    check(lib.fx_region_marshal(region._h, p.handle, arr, n, ptrs, scratch.data_ptr(), totals.data_ptr(), dyn, len(dyn)))
     words = ctypes.POINTER(ctypes.c_uint32)()
     nw = ctypes.c_size_t()
     check(lib.fx_plan_blob(p.handle, ctypes.byref(words), ctypes.byref(nw)))
-    rc = _so.fx_emul_run(words, nw.value, dyn, totals.data_ptr())
+    n_p, n_s, uploaded = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_int()
+    check(lib.fx_plan_table_sizes(p.handle, ctypes.byref(n_p), ctypes.byref(n_s), ctypes.byref(uploaded)))
+    if uploaded.value:
+        # a map of many tasks: the tables at their full length (on the device they are uploaded)
+        tp, ts = (ctypes.c_uint64 * max(n_p.value, 1))(), (ctypes.c_uint32 * max(n_s.value, 1))()
+        check(lib.fx_region_marshal_tables(region._h, p.handle, arr, n, ptrs, scratch.data_ptr(), totals.data_ptr(),
+                                           tp, len(tp), ts, len(ts)))
+        rc = _so.fx_emul_run_tables(words, nw.value, tp, ts, totals.data_ptr())
+    else:
+        dyn = ctypes.create_string_buffer(lib.fx_dyn_bytes())
+        check(lib.fx_region_marshal(region._h, p.handle, arr, n, ptrs, scratch.data_ptr(), totals.data_ptr(), dyn, len(dyn)))
+        rc = _so.fx_emul_run(words, nw.value, dyn, totals.data_ptr())
     assert rc == 0
     if p.compact:
         tl = totals.tolist()

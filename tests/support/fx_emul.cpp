@@ -289,9 +289,15 @@ void decompose(const FxOut& od, uint32_t e, int32_t* c) {
 
 }  // namespace
 
+extern "C" int fx_emul_run_tables(const uint32_t* sb, size_t n_words, const uint64_t* pointers, const uint32_t* scalars, uint32_t* totals);
 extern "C" int fx_emul_run(const uint32_t* sb, size_t n_words, const void* dyn_, uint32_t* totals) {
-  (void)n_words;
   const FxDyn* dyn = (const FxDyn*)dyn_;
+  return fx_emul_run_tables(sb, n_words, dyn->p, dyn->s, totals);
+}
+// the same with the two tables at any length (a map of more tasks than the by-value block holds)
+extern "C" int fx_emul_run_tables(const uint32_t* sb, size_t n_words, const uint64_t* pointers, const uint32_t* scalars, uint32_t* totals) {
+  (void)n_words;
+  struct { const uint64_t* p; const uint32_t* s; } tables = {pointers, scalars}, *dyn = &tables;
   const FxHeader* h = (const FxHeader*)sb;
   if (h->magic != FX_MAGIC) return -1;
   const FxClass* cls = (const FxClass*)(sb + h->off_class);

@@ -360,6 +360,22 @@ def test_c5_torchscript_gpu(grids, batch):
 
 
 @pytest.mark.gpu
+def test_c5_torchscript_gpu_more_images_than_the_argument_block_has_pointers_for():
+    """130 images x 3 results = 390 per-task buffers: the pointer table is uploaded ahead of the
+    kernels (the general count + scatter pair), and the results are those of the oracle."""
+    args = oc.c5_inputs(2, SMALL_GRIDS, 130)
+    rb, rc, ro = oc.run("c5", *args)
+    f = _built("c5", args)
+    print("c5 with 130 images", flush=True)
+    for _ in range(2):   # (the second call reuses the borrowed scratch with its table)
+        gb, gc, go = _cpu(f(*_cuda(args)))
+        assert len(gb) == 130
+        assert_boxes_close(gb, list(rb), "c5 boxes")
+        assert_close(gc, list(rc), "c5 cls")
+        assert_close(go, list(ro), "c5 obj")
+
+
+@pytest.mark.gpu
 def test_c5_torchscript_gpu_new_batch_size_same_function():
     """parallel_degree is taken from the trip count at run time."""
     args3 = oc.c5_inputs(0, SMALL_GRIDS, 3)

@@ -860,11 +860,12 @@ static const FxRsKernel* rs_of(const fx::Plan* pl) {
   // task, chunk after chunk, and keeps the generic two passes (27.6 us that way against 22.5 us).
   // (fx_set_rowstream(2) takes the kernel all the same)
   const uint64_t chunks = ((uint64_t)pl->rs.n_rows + FX_BLOCK - 1) / FX_BLOCK;
-  const bool rows_of_their_own = pl->rs.n_tasks <= 1 || pl->rs.in_tcoef[0] != 0;
+  const bool rows_of_their_own = pl->rs.n_tasks <= 1 || pl->rs.in_tcoef[0] != 0 || (pl->rs.in_slot[0] & FX_SLOT_TASK) != 0;
   if (g_rs_mode.load(std::memory_order_relaxed) != 2 && !rows_of_their_own &&
       chunks * pl->rs.n_tasks > (uint64_t)rs_compute_units() * FX_RS_OCC)
     return nullptr;
   const FxRsKernel* k = fx_rs_find(pl->rs.key);
+  if (k && pl->wide && !k->fn_wide) return nullptr;
   return (k && k->S == pl->rs.S) ? k : nullptr;
 }
 // Geometry of a launch.  Rows of a sub-tile: at most FX_RS_SUB and what FX_RS_KV 128-bit loads per
@@ -939,9 +940,11 @@ static int rs_launch_info(fx::Plan* pl, const FxRsKernel* kern, FxRsLaunch* rl) 
     const uint32_t forced_loads = rs_env("FXHIP_RS_LOADS");   // tuning aid: FX_RS_KV or FX_RS_KV_LEAN
     // (a launch with more chunks than the device holds workgroups runs the build with persistent
     // workgroups, which exists for six loads only)
-    const bool beyond = (uint64_t)((ri.n_rows + FX_BLOCK - 1) / FX_BLOCK) * ri.n_tasks > (uint64_t)std::max(cus, 1) * FX_RS_OCC;
+    // (and a map whose tables are uploaded runs the build that reads them from device memory:
+    // persistent workgroups as well, a map of that many tasks seldom fits the device)
+    const bool beyond = pl->wide || (uint64_t)((ri.n_rows + FX_BLOCK - 1) / FX_BLOCK) * ri.n_tasks > (uint64_t)std::max(cus, 1) * FX_RS_OCC;
     for (int lean = beyond ? 0 : 1; lean >= 0; --lean) {
-      const void* fn = beyond ? kern->fn_persist : lean ? kern->fn_lean : kern->fn;
+      const void* fn = pl->wide ? kern->fn_wide : beyond ? kern->fn_persist : lean ? kern->fn_lean : kern->fn;
       if (!fn || (forced_loads && forced_loads != (lean ? FX_RS_KV_LEAN : FX_RS_KV))) continue;
       // (measured on the benchmark's shape: 22.6 against 22.95 us for kernels that store as they
       // compute; with outputs staged in LDS, where LDS and not registers bounds the occupancy, 25.6 against 24.4)
@@ -1019,7 +1022,8 @@ static hipError_t rs_launch(const FxRsKernel* kern, const FxRsInfo& ri, const Fx
   const bool persist = n_chunks > cap;
   const uint32_t grid = persist ? cap : n_chunks;
   void* args[2] = {(void*)&rl, (void*)dyn};
-  return hipLaunchKernel(persist ? kern->fn_persist : (lean && kern->fn_lean ? kern->fn_lean : kern->fn), dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
+  if (rl.wide != 0 && !kern->fn_wide) return hipErrorInvalidDeviceFunction;   // (rs_of has looked)
+  return hipLaunchKernel(rl.wide != 0 ? kern->fn_wide : persist ? kern->fn_persist : (lean && kern->fn_lean ? kern->fn_lean : kern->fn), dim3(grid), dim3(FX_BLOCK), args, rs_lds_bytes(ri, kern, rl.sub_rows, rl.chunk_rows, rl.side_lds != 0), stream);
 }
 
 // ---- class-map head kernel (fx_cmap.h): geometry of a launch ----
@@ -1165,6 +1169,7 @@ static int run_impl(fx_region* reg, const fx_plan* plan, const fx_arg* args, int
     void* table = (char*)scratch + pl->wide_off;
     HIP_OK(fx_upload_words(words.data(), (size_t)li.n_p + ((size_t)li.n_s + 1) / 2, table, stream));
     li.wide = (uint64_t)(uintptr_t)table;
+    rl.wide = li.wide;
     memset(&dyn, 0, sizeof dyn);
   } else {
     rc = fill_dyn(pl, args, out_ptrs, scratch, totals_host, pl->dev_blob, &dyn, status);

@@ -2363,13 +2363,11 @@ static const Plan* plan_region_once(Region& R, const fx_arg* args, int n_args) {
     }
   }
   P->spec_key = spec_hash(*P);
-  if (!P->wide) {
+  if (!P->wide) {   // (the hand-written kernels read their tables from the kernel arguments)
     match_head(P.get());
     match_classmap(P.get());
-    rs_analyze(P.get());
-  } else {
-    P->rs.why = "more per-task buffers than the kernel argument block holds: the tables are uploaded and the general kernels read them";
   }
+  rs_analyze(P.get());
   const Plan* res = P.get();
   R.plans[key] = std::move(P);
   return res;

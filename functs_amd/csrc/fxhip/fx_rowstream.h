@@ -49,16 +49,20 @@ struct FxRsRt {
   uint32_t task;
   uint32_t* stg[FX_RS_MAX_OUT];   // LDS: where a staged output's kept rows of the sub-tile are put together
   uint32_t ph[FX_RS_MAX_OUT];     // and the phase of the run in memory (first element's index mod 4)
+  // the call's tables: the FxDyn block behind the launch block in the argument segment, or (the
+  // build for maps of many tasks) where the launch block says they were uploaded
+  bool wide;
   FX_RS_FN const uint32_t* staged(int k) const { return stg[k]; }
   FX_RS_FN uint64_t ptr(uint32_t slot) const {
     const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
-    const uint64_t* gp = (const uint64_t*)(ka + sizeof(FxRsLaunch));
+    const uint64_t* gp = wide ? (const uint64_t*)la.wide : (const uint64_t*)(ka + sizeof(FxRsLaunch));
     const uint32_t pi = (slot & FX_SLOT_TASK) ? la.n_sptr + task * la.n_tptr + (slot & 0xffffu) : (slot & 0xffffu);
     return gp[pi];
   }
   FX_RS_FN uint32_t scal(int32_t slot) const {
     const uint8_t* ka = (const uint8_t*)__builtin_amdgcn_kernarg_segment_ptr();
-    const uint32_t* gs = (const uint32_t*)(ka + sizeof(FxRsLaunch) + offsetof(FxDyn, s));
+    const uint32_t* gs = wide ? (const uint32_t*)((const uint64_t*)la.wide + la.n_sptr + la.n_tasks * la.n_tptr)
+                              : (const uint32_t*)(ka + sizeof(FxRsLaunch) + offsetof(FxDyn, s));
     const uint32_t si = ((uint32_t)slot & FX_SLOT_TASK) ? la.n_sscal + task * la.n_tscal + ((uint32_t)slot & 0xffffu) : ((uint32_t)slot & 0xffffu);
     return gs[si];
   }
@@ -154,7 +158,7 @@ FX_RS_FN void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_
 #include "fx_rs_ops.h"
 namespace {
 
-template <class P, uint32_t KV, bool PERSIST>
+template <class P, uint32_t KV, bool PERSIST, bool WIDE = false>
 __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
   constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, NSUB = FX_RS_NSUB, S = P::S;
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];   // the window: sub_rows rows of S elements
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
     const uint32_t c_rows = last_chunk ? la.rows_last : la.chunk_rows;
     const uint32_t sub_rows = last_chunk ? la.sub_rows_last : la.sub_rows_whole;
     const uint32_t n_sub = last_chunk ? la.n_sub_last : la.n_sub_whole;
-    FxRsRt rt{la, task, {}, {}};
+    FxRsRt rt{la, task, {}, {}, WIDE};
     // What the rows' own code reads from memory besides the window (a few words per row: anchors,
     // strides ...) is fetched for all rows of the chunk before the first sub-tile, into a table in LDS.
     const bool SIDE_LDS = P::n_row_cols != 0u && P::n_side != 0u && P::n_side <= FX_RS_MAX_SIDE && la.side_lds != 0u;
@@ -419,12 +423,13 @@ __global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLa
 }
 
 struct FxRsRegistrar {
-  FxRsRegistrar(uint64_t key, const void* fn, const void* fn_lean, const void* fn_persist, uint32_t S, uint32_t stage_row_words,
-                uint32_t n_staged, uint32_t side_row_words) {
+  FxRsRegistrar(uint64_t key, const void* fn, const void* fn_lean, const void* fn_persist, const void* fn_wide, uint32_t S,
+                uint32_t stage_row_words, uint32_t n_staged, uint32_t side_row_words) {
     FxRsKernel k;
     k.fn = fn;
     k.fn_lean = fn_lean;
     k.fn_persist = fn_persist;
+    k.fn_wide = fn_wide;
     k.S = S;
     k.stage_row_words = stage_row_words;
     k.n_staged = n_staged;
@@ -438,5 +443,6 @@ struct FxRsRegistrar {
 #define FX_RS_REGISTER(P) \
   static FxRsRegistrar fx_rs_registrar_##P(P::key, (const void*)&fx_rs_kernel<P, FX_RS_KV, false>,                          \
                                            (const void*)&fx_rs_kernel<P, FX_RS_KV_LEAN, false>,                             \
-                                           (const void*)&fx_rs_kernel<P, FX_RS_KV, true>, P::S, P::stage_row_words,         \
+                                           (const void*)&fx_rs_kernel<P, FX_RS_KV, true>,                                   \
+                                           (const void*)&fx_rs_kernel<P, FX_RS_KV, true, true>, P::S, P::stage_row_words,   \
                                            P::n_staged, (P::n_row_cols != 0u && P::n_side <= FX_RS_MAX_SIDE) ? P::n_side : 0u);

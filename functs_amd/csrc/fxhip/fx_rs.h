@@ -84,6 +84,7 @@ struct FxRsLaunch {
   uint32_t pad1;
   uint32_t* status;             // one word per chunk, tagged with the epoch
   uint32_t* totals;             // pinned host memory: kept rows per task
+  uint64_t wide;                // 0, or the device address of the call's tables (pointers, then scalars) where the FxDyn block is too small for them
 };
 static_assert(sizeof(FxRsLaunch) % 8 == 0, "the FxDyn block follows at an 8-byte boundary");
 // the derived fields of a launch block whose n_rows, chunk_rows, chunks and sub_rows are set
@@ -106,6 +107,7 @@ struct FxRsKernel {
   const void* fn = nullptr;     // fx_rs_kernel<P, FX_RS_KV, false>
   const void* fn_lean = nullptr; // fx_rs_kernel<P, FX_RS_KV_LEAN, false>
   const void* fn_persist = nullptr; // fx_rs_kernel<P, FX_RS_KV, true>: workgroups that take several chunks in turn
+  const void* fn_wide = nullptr;    // fx_rs_kernel<P, FX_RS_KV, true, true>: the same, reading the call's tables from device memory (FxRsLaunch::wide)
   uint32_t S = 0;               // row length the kernel is generated for
   uint32_t stage_row_words = 0; // elements per kept row that the kernel puts together in LDS before they leave
   uint32_t n_staged = 0;        // outputs that take that route

@@ -352,7 +352,8 @@ size_t fx_dyn_bytes(void);
  * up to 4096 of each, fx_region_run then writes the two tables to the end of the caller's scratch
  * memory (fx_plan_scratch_bytes counts them, also for a region that does not compact) with small
  * launches ahead of the kernels, which read them from there; such a plan runs the general
- * kernels (the one-launch forms and the short dense kernel read the argument block), and
+ * kernels or the build of its generated row-stream kernel that reads device memory (the
+ * hand-written one-launch kernels and the short dense kernel read the argument block), and
  * fx_region_marshal refuses it.  The reference passes every task's buffers as kernel arguments
  * and clones the body per task (functor_parallization.cpp:12-111): its limit is the compiler's.
  * fx_plan_table_sizes: entries of the two tables, and whether the plan uploads them.

@@ -362,13 +362,17 @@ def test_c5_torchscript_gpu(grids, batch):
 @pytest.mark.gpu
 def test_c5_torchscript_gpu_more_images_than_the_argument_block_has_pointers_for():
     """130 images x 3 results = 390 per-task buffers: the pointer table is uploaded ahead of the
-    kernels (the general count + scatter pair), and the results are those of the oracle."""
+    kernel (the build of the generated row-stream kernel that reads its tables from device memory:
+    still one launch), and the results are those of the oracle."""
+    import functs_amd.aot as aot
     args = oc.c5_inputs(2, SMALL_GRIDS, 130)
     rb, rc, ro = oc.run("c5", *args)
     f = _built("c5", args)
     print("c5 with 130 images", flush=True)
     for _ in range(2):   # (the second call reuses the borrowed scratch with its table)
+        l0, _s = aot.launch_stats()
         gb, gc, go = _cpu(f(*_cuda(args)))
+        assert aot.launch_stats()[0] - l0 == 1
         assert len(gb) == 130
         assert_boxes_close(gb, list(rb), "c5 boxes")
         assert_close(gc, list(rc), "c5 cls")

@@ -9,7 +9,7 @@ TorchScript interpreter computes for it (every reference test is differential
 against it: test/test_basic.py:50-52, test/test_immut_tensorexpr.py:22,
 fait/testing/test_lowering.cpp:221, fait/fait.cpp:74-77).
 
-The programs imitate, at the shapes BASELINE.json names:
+The programs imitate, at the shapes of the five benchmark configurations:
   c1  examples/get_started.py:10-15 (verbatim)
   c2  functs/benchmark/ai_model/yolov3/yolov3_bbox.py:12-23, 206-243
       (sigmoid_ slice assign, objectness / class sigmoid, box decode written

@@ -1,7 +1,7 @@
 """Parity of the five benchmark configurations with the oracle (stock
 TorchScript on the CPU, oracle/configs.py) on the same seeded inputs.
 
-Reduced shapes run on the emulator and on the GPU; BASELINE.json's full shapes
+Reduced shapes run on the emulator and on the GPU; the benchmark configurations' full shapes
 run on the GPU only.  Bars: bit-exact for select/slice/assign/compaction
 results (c1, kept-row sets and row order everywhere), 1e-5 relative for fp32
 elementwise math (sigmoid/exp/softmax/box decode).
@@ -140,7 +140,7 @@ def test_c3_zero_loc_closed_form(backend):
 
 
 # ---------------------------------------------------------------------------
-# BASELINE.json's full shapes (GPU only)
+# the benchmark configurations' full shapes (GPU only)
 # ---------------------------------------------------------------------------
 
 

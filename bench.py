@@ -22,7 +22,8 @@ bytes, the operator's host time by section and, for row compactions (whose defau
 is the kernel generated from the region's programs, fx_rs_kernel), the figures of
 the hand-written and the generic kernels and of the opt-in call forms (lazy_lists,
 padded_outputs); `c5_batch64`: four times c5's batch, more chunks than the device holds
-workgroups; `head_variants`: other spellings of the detection head, each on its
+workgroups; `c5_batch128`: eight times, more per-task buffers than the kernel arguments hold
+(the pointer table is uploaded ahead of the kernel); `head_variants`: other spellings of the detection head, each on its
 own generated kernel; `c5_nms_tail`: the compaction followed by the detection tail,
 also through the TorchScript route.  `roofline` prices the dominant kernel against the 8 TB/s
 HBM peak with the algorithmic bytes of the call; its duration is measured with
@@ -784,7 +785,7 @@ def main():
                     torch.cuda.synchronize()
                     alg = bound[0].plan.alg_bytes + sum(t.numel() * t.element_size() for o in res for t in (o if isinstance(o, list) else [o]))
                     flush(dev)
-                    ms = timed_sets(bound, which=-1, rounds=6)
+                    ms = timed_sets(bound, which=-1, rounds=6 if batch <= 64 else 3)
                     out[vname if rowstream else vname + "_generic"] = {
                         "kernel": head_kernel_in_use(bound[0].plan), "launches_per_call": bound[0].plan.launches,
                         "call_kernels_us": round(ms * 1e3, 2), "algorithmic_bytes": alg,
@@ -840,10 +841,11 @@ def main():
             per["head_variants"] = run_variants()
         except Exception as e:
             per["head_variants"] = {"error": str(e)[:200]}
-        try:
-            per["c5_batch64"] = run_big_batch()
-        except Exception as e:
-            per["c5_batch64"] = {"error": str(e)[:200]}
+        for batch in (64, 128):
+            try:
+                per["c5_batch%d" % batch] = run_big_batch(batch)
+            except Exception as e:
+                per["c5_batch%d" % batch] = {"error": str(e)[:200]}
         try:
             per["c4"] = run_c4()
         except Exception as e:

@@ -1272,11 +1272,13 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   if (n_args != pl->n_args) return fail(FX_E_INVALID, "argument count differs from the plan");
   const bool compact = pl->mode == FX_MODE_COMPACT;
   if (compact && (!scratch || !totals_host)) return fail(FX_E_INVALID, "compacting region needs scratch and totals per set");
-  if (pl->wide) return fail(FX_E_LIMIT, "fx_region_run_timed_sets: not for a plan whose tables are uploaded (a map of many tasks)");
+  // (a plan whose tables are uploaded keeps them in every set's scratch memory, dense or not)
+  const bool with_scratch = compact || pl->wide;
+  if (pl->wide && !scratch) return fail(FX_E_INVALID, "this plan keeps its tables in scratch memory (fx_plan_scratch_bytes): scratch per set");
   hipStream_t stream = (hipStream_t)stream_;
   // one untimed call per set: uploads the descriptor, leaves every set's scratch valid
   for (int i = 0; i < n_sets; ++i) {
-    const int rc = run_impl(reg, plan, args[i], n_args, out_ptrs[i], compact ? scratch[i] : nullptr,
+    const int rc = run_impl(reg, plan, args[i], n_args, out_ptrs[i], with_scratch ? scratch[i] : nullptr,
                             compact ? totals_host[i] : nullptr, stream_, nullptr, 0, nullptr);
     if (rc != FX_OK) return rc;
   }
@@ -1334,6 +1336,7 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   std::vector<FxDyn> dyn((size_t)n_sets);
   for (int i = 0; i < n_sets; ++i) {
     memset(&dyn[i], 0, sizeof(FxDyn));
+    if (pl->wide) continue;   // (the untimed call above has left the set's tables in its scratch memory)
     const int rc = fill_dyn(pl, args[i], out_ptrs[i], compact ? scratch[i] : nullptr, compact ? totals_host[i] : nullptr,
                             pl->dev_blob, &dyn[i], status);
     if (rc != FX_OK) return rc;
@@ -1346,6 +1349,10 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   HIP_OK(hipEventRecord(e0, stream));
   for (int r = 0; r < rounds; ++r)
     for (int i = 0; i < n_sets; ++i) {
+      if (pl->wide) {
+        li.wide = (uint64_t)(uintptr_t)((char*)scratch[i] + pl->wide_off);
+        rl.wide = li.wide;
+      }
       if (!compact) {
         HIP_OK(fx_launch_dense(pl->max_rank, sb, li, &dyn[i], std::min<uint32_t>(pl->grid, 256u * FX_DENSE_WG_PER_CU), stream, spec, lean_of(pl), pl->lean_slot_err));
       } else if (rsk) {

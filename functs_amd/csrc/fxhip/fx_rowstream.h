@@ -158,8 +158,10 @@ FX_RS_FN void rs_st4_at(const FxRsRt& rt, int k, uint32_t e, uint32_t a, uint32_
 #include "fx_rs_ops.h"
 namespace {
 
+// (WIDE, the build that reads the call's tables from device memory, is compiled for one workgroup
+// per CU less: at the others' occupancy it spills, 194 against 182 us for the head on 128 images)
 template <class P, uint32_t KV, bool PERSIST, bool WIDE = false>
-__global__ __launch_bounds__(FX_BLOCK, FX_RS_OCC) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
+__global__ __launch_bounds__(FX_BLOCK, (WIDE ? FX_RS_OCC - 1u : FX_RS_OCC)) void fx_rs_kernel(const FxRsLaunch la, const FxDyn) {
   constexpr uint32_t NT = FX_BLOCK, NW = NT / 64u, NSUB = FX_RS_NSUB, S = P::S;
   extern __shared__ __attribute__((aligned(16))) uint32_t L[];   // the window: sub_rows rows of S elements
   __shared__ uint32_t s_rowmap[FX_RS_SUB];

@@ -305,7 +305,8 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0, **build_
     (output allocation, launches and the kept-row synchronisation included).
     With cold_bytes, consecutive calls rotate over copies of the inputs and the outputs of
     the last calls are kept alive, so that the allocator hands out other blocks: the calls
-    then work on memory that the caches do not hold (returned beside the warm figures)."""
+    then work on memory that the caches do not hold (returned beside the warm figures).
+    Every figure is the median over regions_for(steps) timed regions of exactly `steps` calls."""
     import collections
     import torch
     import functs_amd.jit as fj
@@ -313,23 +314,35 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0, **build_
     import functs_amd.aot as aot
     fn = fj.build(fj.script(PROGRAMS[name]), list(cpu_args), **build_options)
     args = [a.to(dev) if isinstance(a, torch.Tensor) else a for a in cpu_args]
-    for _ in range(warmup):
+    n_regions = regions_for(steps)
+
+    def regions(call, k, drained=False):
+        """Median time per call over n_regions timed regions of exactly k calls each, every region
+        between two device synchronisations (drained: a synchronisation after every call)."""
+        per_call = []
+        for _ in range(n_regions):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(k):
+                call(i)
+                if drained:
+                    torch.cuda.synchronize()
+            torch.cuda.synchronize()
+            per_call.append((time.perf_counter() - t0) * 1e6 / k)
+        per_call.sort()
+        return per_call[len(per_call) // 2]
+
+    # the calls that settle the process (first launches load the kernels' code, the allocators
+    # grow their pools) are not part of the warm-up the caller asks for
+    for _ in range(max(warmup, SETTLE_CALLS)):
         fn(*args)
     torch.cuda.synchronize()
     l0, s0 = aot.launch_stats()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn(*args)
-    torch.cuda.synchronize()
-    us = (time.perf_counter() - t0) * 1e6 / steps
+    us = regions(lambda i: fn(*args), steps)
     l1, s1 = aot.launch_stats()
     # the same call with the device drained after every call: issue to completion of one call
     n_sync = max(steps // 4, 5)
-    t0 = time.perf_counter()
-    for _ in range(n_sync):
-        fn(*args)
-        torch.cuda.synchronize()
-    sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
+    sync_us = regions(lambda i: fn(*args), n_sync, drained=True)
     n_functors = str(fn.graph).count("= tssa::ParallelFunctor")
     cold_us = cold_sync_us = None
     if cold_bytes:
@@ -337,21 +350,15 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0, **build_
         n_sets = min(MAX_SETS, max(4, -(-cold_bytes // max(2 * in_bytes, 1))))
         sets = [[a.clone() if isinstance(a, torch.Tensor) else a for a in args] for _ in range(n_sets)]
         ring = collections.deque(maxlen=n_sets)
-        for i in range(max(warmup, n_sets)):
+        # (the ring of kept results has to fill and the allocator to hand out a block for the call
+        # after it before the calls run as they do in the long run)
+        for i in range(max(warmup, n_sets + 2, SETTLE_CALLS)):
             ring.append(fn(*sets[i % n_sets]))
         torch.cuda.synchronize()
         flush(dev)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            ring.append(fn(*sets[i % n_sets]))
-        torch.cuda.synchronize()
-        cold_us = (time.perf_counter() - t0) * 1e6 / steps
-        t0 = time.perf_counter()
-        for i in range(n_sync):
-            ring.append(fn(*sets[i % n_sets]))
-            torch.cuda.synchronize()
-        cold_sync_us = (time.perf_counter() - t0) * 1e6 / n_sync
+        cold_us = regions(lambda i: ring.append(fn(*sets[i % n_sets])), steps)
+        cold_sync_us = regions(lambda i: ring.append(fn(*sets[i % n_sets])), n_sync, drained=True)
     # host time of the operator by section (mean microseconds per operator call), warm calls
     from functs_amd import _C
     _C._functor_host_timing(True)
@@ -361,6 +368,16 @@ def torchscript_route(name, cpu_args, dev, steps, warmup, cold_bytes=0, **build_
     host = {k: round(v, 2) for k, v in _C._functor_host_times().items()}
     _C._functor_host_timing(False)
     return us, n_functors, (s1 - s0) / max(l1 - l0, 1), sync_us, cold_us, cold_sync_us, host
+
+
+SETTLE_CALLS = 24      # untimed calls of a freshly built function before its first timed region
+TIMED_CALLS = 200      # calls a figure rests on: a region of K calls is repeated until about this many have run
+
+
+def regions_for(steps):
+    """How many timed regions of `steps` calls a figure is the median of (an odd number)."""
+    n = max(1, -(-TIMED_CALLS // max(steps, 1)))
+    return min(n | 1, 15)
 
 
 def set_kernels(rowstream, head):
@@ -865,11 +882,12 @@ def main():
     out = {
         "metric": "per-call latency",
         "value": head["torchscript_route_latency_us"],
-        "value_kind": "back-to-back: K calls between two device synchronisations, consecutive calls on rotated copies of the inputs and on fresh output blocks (cold caches); drained_latency_us: the device drained after every call; *_warm: every call on the same buffers",
+        "value_kind": "back-to-back: K calls between two device synchronisations, consecutive calls on rotated copies of the inputs and on fresh output blocks (cold caches); the median of timed_regions such regions of exactly K calls each (about 200 calls in all), after the W warm-up calls and the calls that settle a freshly built function (kernel code loaded, allocator pools grown); drained_latency_us: the device drained after every call; *_warm: every call on the same buffers",
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "timed_regions": regions_for(args.steps),
         "ms_per_step": round(head["torchscript_route_latency_us"] / 1e3, 5),
         "higher_is_better": False,
         "scaling": "weak",

@@ -167,6 +167,7 @@ _sig("fx_set_dense_lean", None, _i)
 _sig("fx_spec_dump_dir", _i, ctypes.c_char_p)
 _sig("fx_spec_dump_what", _i, _i)
 _sig("fx_region_wait_totals", _i, _vp, _vp, _vp)
+_sig("fx_region_poll_totals", _i, _vp, _vp, ctypes.c_uint32)
 _sig("fx_launch_stats", None, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64))
 _sig("fx_region_marshal", _i, _vp, _vp, ctypes.POINTER(FxArg), _i, ctypes.POINTER(_vp), _vp, _vp, _vp,
      ctypes.c_size_t)

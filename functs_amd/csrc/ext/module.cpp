@@ -32,6 +32,32 @@ struct TensorList {
   }
 };
 
+// The hook of a direct call (passes.h): the caller keeps the interpreter's lock through the
+// operator, so the Python lists of a map's results can be made while the kernels run; the lock is
+// given up only around a wait that outlasts the operator's short poll.
+struct DirectCallHook final : functs::EarlyResultsHook {
+  std::vector<py::object> lists;   // per operator output: its Python list, made early
+  PyThreadState* saved = nullptr;
+  void tensorsReady(size_t n_lists, int64_t degree, const at::Tensor* flat) override {
+    lists.clear();
+    lists.reserve(n_lists);
+    for (size_t o = 0; o < n_lists; ++o) {
+      py::list l((size_t)degree);
+      for (int64_t t = 0; t < degree; ++t) {
+        PyObject* item = THPVariable_Wrap(flat[o * (size_t)degree + (size_t)t]);
+        if (!item) throw py::error_already_set();
+        PyList_SET_ITEM(l.ptr(), (Py_ssize_t)t, item);
+      }
+      lists.push_back(std::move(l));
+    }
+  }
+  void beforeBlocking() override { saved = PyEval_SaveThread(); }
+  void afterBlocking() override {
+    if (saved) PyEval_RestoreThread(saved);
+    saved = nullptr;
+  }
+};
+
 struct DirectFunctor {
   bool lazy_lists = false;                      // List[Tensor] results come back as TensorList
   std::shared_ptr<Graph> graph;                 // owns the node
@@ -96,18 +122,27 @@ struct DirectFunctor {
       if (s < 0) stack.push_back(constants[(size_t)(-1 - s)]);
       else stack.push_back(torch::jit::toIValue(args[(size_t)s], arg_types[(size_t)s]));
     }
-    {
+    DirectCallHook hook;
+    if (lazy_lists) {
       py::gil_scoped_release release;
+      (*op)(stack);
+    } else {
+      struct Installed {
+        explicit Installed(functs::EarlyResultsHook* h) { functs::setEarlyResultsHook(h); }
+        ~Installed() { functs::setEarlyResultsHook(nullptr); }
+      } installed(&hook);
       (*op)(stack);
     }
     TORCH_CHECK(stack.size() == n_op_outputs, "the operator left ", stack.size(), " values for ", n_op_outputs, " results");
-    auto convert = [this](c10::IValue&& v) -> py::object {
+    auto convert = [this, &hook](c10::IValue&& v, size_t output) -> py::object {
       if (lazy_lists && v.isTensorList()) return py::cast(TensorList{std::move(v).toTensorList()});
+      // (the list made while the kernels ran holds the very tensors of the operator's list)
+      if (output < hook.lists.size() && v.isTensorList()) return std::move(hook.lists[output]);
       return torch::jit::toPyObject(std::move(v));
     };
-    if (!tuple_result) return convert(std::move(stack[(size_t)results[0]]));
+    if (!tuple_result) return convert(std::move(stack[(size_t)results[0]]), (size_t)results[0]);
     py::tuple out(results.size());
-    for (size_t k = 0; k < results.size(); ++k) out[k] = convert(std::move(stack[(size_t)results[k]]));
+    for (size_t k = 0; k < results.size(); ++k) out[k] = convert(std::move(stack[(size_t)results[k]]), (size_t)results[k]);
     return std::move(out);
   }
 };

@@ -116,6 +116,19 @@ std::vector<std::string> PlanFunctors(std::shared_ptr<torch::jit::Graph> graph);
 // Host time of tssa::ParallelFunctor by section (flatten, plan, alloc, launch, views, wait_counts,
 // resize, push): switching on clears the sums; the read gives "calls" and the mean microseconds per
 // operator call of every section.
+// A caller of tssa::ParallelFunctor that holds the Python interpreter's lock through the call
+// (functs_amd._C.DirectFunctor) installs one of these for its thread: the operator hands over the
+// tensors of a map's list results as soon as they exist - views of the output block, made while
+// the kernels run, their first dimension still at full size and cut in place once the kept-row
+// counts are known - so that the wrapper objects of a call's results are made in the kernels'
+// shadow and not behind the wait; and it tells before it blocks for longer than a short poll.
+struct EarlyResultsHook {
+  virtual ~EarlyResultsHook() = default;
+  virtual void tensorsReady(size_t n_lists, int64_t degree, const at::Tensor* flat /* [list][task] */) = 0;
+  virtual void beforeBlocking() = 0;
+  virtual void afterBlocking() = 0;
+};
+void setEarlyResultsHook(EarlyResultsHook* hook);   // of the calling thread; nullptr removes it
 void functorHostTiming(bool on);
 std::vector<std::pair<std::string, double>> functorHostTimes();
 

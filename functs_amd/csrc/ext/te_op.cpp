@@ -358,6 +358,14 @@ struct HostClock {
   }
 };
 
+thread_local EarlyResultsHook* t_early_hook = nullptr;
+// between beforeBlocking and afterBlocking of the hook, also when an error leaves the scope
+struct BlockingScope {
+  EarlyResultsHook* hook;
+  explicit BlockingScope(EarlyResultsHook* h) : hook(h) { if (hook) hook->beforeBlocking(); }
+  ~BlockingScope() { if (hook) hook->afterBlocking(); }
+};
+
 // device scratch and the pinned landing zone of the kept-row counts; a call
 // borrows one and hands it back, so concurrent calls never share
 struct Workspace {
@@ -661,11 +669,22 @@ class RegionRunner {
       }
     }
     clock.tick(HS_VIEWS);
+    EarlyResultsHook* const hook = t_early_hook;
+    if (hook && is_map_ && degree > 1 && compact_) hook->tensorsReady((size_t)n_out, degree, flat.data());
     if (compact_) {
       // The kept-row counts decide the output shapes.  ATen's nonzero / masked index
       // synchronise the stream for that; here the counts arrive through pinned memory early
       // in the second pass, and the outputs are valid in stream order.
-      FX_OK_OR_THROW(fx_region_wait_totals(plan, (const uint32_t*)ws.totals.data_ptr(), (void*)stream.stream()));
+      // (a caller that holds the interpreter's lock: a short poll first, and word before the long wait)
+      int ready = 0;
+      if (hook) {
+        ready = fx_region_poll_totals(plan, (const uint32_t*)ws.totals.data_ptr(), 200u);
+        FX_OK_OR_THROW(ready < 0 ? ready : 0);
+      }
+      if (!ready) {
+        BlockingScope scope(hook);
+        FX_OK_OR_THROW(fx_region_wait_totals(plan, (const uint32_t*)ws.totals.data_ptr(), (void*)stream.stream()));
+      }
       clock.tick(HS_WAIT);
       const int32_t* tot = ws.totals.data_ptr<int32_t>();
       for (int o = 0; o < n_out; ++o)
@@ -1746,6 +1765,8 @@ std::vector<std::string> PlanFunctors(std::shared_ptr<Graph> graph) {
   planIn(graph->block(), &report);
   return report;
 }
+
+void setEarlyResultsHook(EarlyResultsHook* hook) { t_early_hook = hook; }
 
 void functorHostTiming(bool on) {
   if (on) {

@@ -1386,6 +1386,27 @@ int fx_region_run_timed_sets(fx_region* reg, const fx_plan* plan, int n_sets, co
   return FX_OK;
 }
 
+int fx_region_poll_totals(const fx_plan* plan, const uint32_t* totals_host, uint32_t spin_us) {
+  if (!plan || !totals_host) return fail(FX_E_INVALID, "null argument");
+  const fx::Plan* pl = P(plan);
+  if (pl->mode != FX_MODE_COMPACT) return fail(FX_E_INVALID, "not a compacting region");
+  const volatile uint32_t* tot = totals_host;
+  const int T = pl->region->degree;
+  using clock = std::chrono::steady_clock;
+  const clock::time_point t0 = clock::now();
+  const clock::duration budget = std::chrono::microseconds(spin_us);
+  for (;;) {
+    bool all = true;
+    for (int t = 0; t < T; ++t) all = all && tot[t] != FX_TOTAL_PENDING;
+    if (all) {
+      std::atomic_thread_fence(std::memory_order_acquire);
+      return 1;
+    }
+    if (clock::now() - t0 >= budget) return 0;
+    __builtin_ia32_pause();
+  }
+}
+
 int fx_region_wait_totals(const fx_plan* plan, const uint32_t* totals_host, void* stream_) {
   if (!plan || !totals_host) return fail(FX_E_INVALID, "null argument");
   const fx::Plan* pl = P(plan);

@@ -311,6 +311,10 @@ int fx_region_run(fx_region*, const fx_plan*, const fx_arg* args, int n_args, vo
 #define FX_TOTAL_PENDING 0xffffffffu
 int fx_region_wait_totals(const fx_plan*, const uint32_t* totals_host, void* stream);
 void fx_set_totals_spin_us(uint32_t microseconds);
+/* The polling part alone: 1 as soon as every count is readable, 0 when they are not after
+ * spin_us microseconds (nothing blocks, no call into the runtime), negative on error.  For a
+ * caller that holds a lock it must give up before it may block (the Python interpreter's). */
+int fx_region_poll_totals(const fx_plan*, const uint32_t* totals_host, uint32_t spin_us);
 
 /* fx_region_run with a HIP event pair around every kernel on `stream`; waits for
  * the last event and returns the duration of each launch in milliseconds

@@ -117,6 +117,39 @@ def test_kept_row_counts_waited_for_in_the_stream_give_the_same_results(name, sm
 
 
 @pytest.mark.gpu
+def test_calls_from_two_threads_on_their_own_streams():
+    """The direct call keeps the interpreter's lock while it polls for the kept-row counts and makes
+    the result lists: two threads calling the same built function get their own results."""
+    import threading
+    args_a, args_b = INPUTS["c5"](11, grids=[4, 6, 8], batch=5), INPUTS["c5"](12, grids=[4, 6, 8], batch=5)
+    fn = fj.build(fj.script(PROGRAMS["c5"]), list(args_a))
+    ga, gb = _cuda(args_a), _cuda(args_b)
+    ref_a, ref_b = [t.clone() for t in _flat(fn(*ga))], [t.clone() for t in _flat(fn(*gb))]
+    torch.cuda.synchronize()
+    print("two threads", flush=True)
+    bad = []
+
+    def work(gargs, ref, tag):
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.default_stream())
+        with torch.cuda.stream(stream):
+            for k in range(100):
+                got = _flat(fn(*gargs))
+                stream.synchronize()
+                if len(got) != len(ref) or not all(x.shape == y.shape and torch.equal(x, y) for x, y in zip(got, ref)):
+                    bad.append((tag, k))
+                    return
+
+    threads = [threading.Thread(target=work, args=(ga, ref_a, "a")), threading.Thread(target=work, args=(gb, ref_b, "b"))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads)
+    assert not bad, bad
+
+
+@pytest.mark.gpu
 def test_lazy_lists_hold_the_same_tensors():
     args = INPUTS["c5"](2, grids=[4, 6, 8], batch=5)
     plain = fj.build(fj.script(PROGRAMS["c5"]), list(args))

@@ -358,6 +358,28 @@ struct HostClock {
   }
 };
 
+// The key of a call's argument kinds (which variant of the region serves it), put together per
+// call: a string with the few appends it needs (a stream costs a locale and an allocation a call).
+struct Signature {
+  std::string s;
+  Signature() { s.reserve(96); }
+  Signature& operator<<(const char* t) { s.append(t); return *this; }
+  Signature& operator<<(long long v) {
+    char buf[24];
+    int n = 0;
+    unsigned long long u = v < 0 ? 0ull - (unsigned long long)v : (unsigned long long)v;
+    do { buf[n++] = (char)('0' + u % 10); u /= 10; } while (u);
+    if (v < 0) s.push_back('-');
+    while (n) s.push_back(buf[--n]);
+    return *this;
+  }
+  Signature& operator<<(long v) { return *this << (long long)v; }
+  Signature& operator<<(int v) { return *this << (long long)v; }
+  Signature& operator<<(unsigned v) { return *this << (long long)v; }
+  Signature& operator<<(unsigned long v) { return *this << (long long)v; }
+  const std::string& str() const { return s; }
+};
+
 thread_local EarlyResultsHook* t_early_hook = nullptr;
 // between beforeBlocking and afterBlocking of the hook, also when an error leaves the scope
 struct BlockingScope {
@@ -494,7 +516,12 @@ class RegionRunner {
     HostClock clock;
     // flatten arguments
     std::vector<fx_arg> args;
-    std::ostringstream sig;
+    {   // one entry per shared argument and per task of a per-task one (more only for list-valued scalars)
+      size_t n_par = 0;
+      if (is_map_) for (int64_t p : is_par_) n_par += p != 0;
+      args.reserve(n_args_ + n_par * (size_t)std::max<int64_t>(degree, 1));
+    }
+    Signature sig;
     c10::Device device(c10::kCPU);
     bool have_device = false;
     flatten(inputs, first, degree, /*dry=*/false, args, sig, device, have_device);
@@ -730,7 +757,7 @@ class RegionRunner {
     if (!is_map_) degree = 1;
     TORCH_CHECK(degree >= 1, "dryRun: empty map");
     std::vector<fx_arg> args;
-    std::ostringstream sig;
+    Signature sig;
     c10::Device device(c10::kCPU);
     bool have_device = false;
     flatten(samples, first, degree, /*dry=*/true, args, sig, device, have_device);
@@ -777,7 +804,7 @@ class RegionRunner {
   // of scalars as their elements) and the signature that selects the region variant.  `dry`:
   // tensors stand for their types only (no device, no pointer).
   void flatten(at::ArrayRef<c10::IValue> inputs, size_t first, int64_t degree, bool dry, std::vector<fx_arg>& args,
-               std::ostringstream& sig, c10::Device& device, bool& have_device) {
+               Signature& sig, c10::Device& device, bool& have_device) {
     sig << degree;
     auto addTensor = [&](const at::Tensor& t) {
       TORCH_CHECK(dry || t.is_cuda(), "tssa::ParallelFunctor runs on the GPU only; got a ", t.device(), " tensor");

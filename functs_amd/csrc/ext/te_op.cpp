@@ -583,9 +583,7 @@ class RegionRunner {
     }
     clock.tick(HS_PLAN);
     typedef OutSlot Slot;
-    std::vector<Slot> slots;   // a copy only where the kept-row counts change the sizes
-    if (compact_) slots = layout->slots;
-    const Slot* slot_of = compact_ ? slots.data() : layout->slots.data();
+    const Slot* slot_of = layout->slots.data();   // (full sizes; the kept-row counts replace dimension 0 below)
     // A map: ONE allocation for all outputs of all tasks (an allocation costs about a
     // microsecond of host time); a single task: one tensor per output.
     std::vector<at::Tensor> buffers(n_out);
@@ -716,10 +714,12 @@ class RegionRunner {
       const int32_t* tot = ws.totals.data_ptr<int32_t>();
       for (int o = 0; o < n_out; ++o)
         for (int64_t t = 0; t < degree; ++t) {
-          Slot& sl = slots[(size_t)o * degree + t];
-          sl.sizes[0] = tot[t];
+          const Slot& sl = slot_of[(size_t)o * degree + t];
+          int64_t sizes[FX_ARG_MAX_RANK];
+          std::copy(sl.sizes, sl.sizes + sl.rank, sizes);
+          sizes[0] = tot[t];
           at::Tensor& out = degree == 1 ? buffers[o] : flat[(size_t)o * degree + t];
-          out.unsafeGetTensorImpl()->set_sizes_contiguous(at::IntArrayRef(sl.sizes, sl.rank));
+          out.unsafeGetTensorImpl()->set_sizes_contiguous(at::IntArrayRef(sizes, sl.rank));
         }
       var->give(std::move(ws));
     }

@@ -111,3 +111,31 @@ def test_region_without_gpu_fails_loudly():
     r.finalize()
     with pytest.raises(_lib.FxError):
         r(torch.rand(4))  # CPU tensors: no fallback path
+
+
+def test_polling_for_the_kept_row_counts_never_blocks():
+    """fx_region_poll_totals looks at the pinned words only: 0 while a task's count is pending
+    (after the time it was given), 1 once every count is there; not for regions that keep all rows."""
+    import time
+    r = Region(parallel_degree=3, is_parallel_map=True)
+    x = r.tensor_input(torch.float32, 2, per_task=True)
+    r.compact_rows(x.select(1, 0) > 0.5)
+    r.output(x * 2.0)
+    r.finalize()
+    xs = [torch.rand(10 + k, 4) for k in range(3)]
+    arr, n, keep = r._flatten((xs,))
+    p = r.plan(arr, n)
+    pending = 0xFFFFFFFF
+    totals = (ctypes.c_uint32 * 3)(5, pending, 7)
+    t0 = time.perf_counter()
+    assert lib.fx_region_poll_totals(p.handle, totals, 2000) == 0
+    assert 0.0015 < time.perf_counter() - t0 < 0.5
+    assert lib.fx_region_poll_totals(p.handle, totals, 0) == 0
+    totals[1] = 0
+    assert lib.fx_region_poll_totals(p.handle, totals, 0) == 1
+    dense = Region()
+    d = dense.tensor_input(torch.float32, 2)
+    dense.output(d + 1.0)
+    dense.finalize()
+    arr, n, keep = dense._flatten((torch.rand(4, 4),))
+    assert lib.fx_region_poll_totals(dense.plan(arr, n).handle, totals, 0) < 0

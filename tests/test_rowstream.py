@@ -376,3 +376,51 @@ def test_a_captured_call_takes_the_two_passes_and_replays_follow_their_inputs():
         for t in range(2):
             assert tot[t] == want[t][2].shape[0]
             assert_close(bc.outs[2][t][:tot[t]].cpu(), want[t][2], "replay seed %d image %d" % (seed, t))
+
+
+def _list_input_head(batch):
+    """The head over a LIST of images: every task's prediction matrix is a tensor of its own."""
+    from functs_amd import Region
+    r = Region(parallel_degree=batch, is_parallel_map=True)
+    p = r.tensor_input(torch.float32, 2, per_task=True)
+    anchors = r.tensor_input(torch.float32, 2)
+    strides = r.tensor_input(torch.float32, 1)
+    pxy, pwh = p.slice(1, 0, 2).sigmoid(), p.slice(1, 2, 4)
+    obj, cls = p.select(1, 4).sigmoid(), p.slice(1, 5, None).sigmoid()
+    xy = (anchors.slice(1, 0, 2) + anchors.slice(1, 2, None)) * 0.5 + (pxy - 0.5) * strides.unsqueeze(-1)
+    wh = (anchors.slice(1, 2, None) - anchors.slice(1, 0, 2)) * 0.5 * pwh.exp()
+    r.compact_rows(obj >= 0.3)
+    r.output(r.cat([xy - wh, xy + wh], 1))
+    r.output(cls)
+    r.output(obj)
+    return r.finalize()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch,n", [(4, 900), (40, 10647)])
+def test_a_map_over_a_list_of_images_streams_each_image_once(batch, n):
+    """Per-task window pointers (the kernel is the linked one of the `cat` spelling: where a task's
+    rows lie is an argument of the launch); the larger case has more chunks than the device holds
+    workgroups (1 680 of 256 rows), which a map over rows of its own takes in turn."""
+    r = _list_input_head(batch)
+    g = torch.Generator().manual_seed(9)
+    pred = torch.randn(batch, n, 85, generator=g)
+    anchors = torch.rand(n, 4, generator=g) * 100
+    strides = torch.full((n,), 8.0)
+    images = [pred[t].clone() for t in range(batch)]
+    dev = torch.device("cuda:0")
+    dargs = [[im.to(dev) for im in images], anchors.to(dev), strides.to(dev)]
+    assert r.rowstream_info(*dargs)["active"]
+    print("list of", batch, "images", flush=True)
+    arr, cnt, _ = r._flatten(dargs)
+    assert lib.fx_plan_launches(r.plan(arr, cnt).handle) == 1
+    one = [[t.cpu() for t in o] for o in r(*dargs)]
+    torch.cuda.synchronize()
+    lib.fx_set_rowstream(0)
+    try:
+        two = [[t.cpu() for t in o] for o in r(*dargs)]
+        torch.cuda.synchronize()
+    finally:
+        lib.fx_set_rowstream(1)
+    assert_exact(one, two, "list of images: one launch vs two passes")
+    assert [o.shape[0] for o in one[0]] == [int((torch.sigmoid(im[:, 4]) >= 0.3).sum()) for im in images]

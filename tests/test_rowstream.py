@@ -397,11 +397,13 @@ def _list_input_head(batch):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("batch,n", [(4, 900), (40, 10647)])
+@pytest.mark.parametrize("batch,n", [(4, 900), (40, 10647), (130, 900)])
 def test_a_map_over_a_list_of_images_streams_each_image_once(batch, n):
     """Per-task window pointers (the kernel is the linked one of the `cat` spelling: where a task's
-    rows lie is an argument of the launch); the larger case has more chunks than the device holds
-    workgroups (1 680 of 256 rows), which a map over rows of its own takes in turn."""
+    rows lie is an argument of the launch); the second case has more chunks than the device holds
+    workgroups (1 680 of 256 rows), which a map over rows of its own takes in turn; the third
+    more per-task buffers (520) than the kernel arguments hold: the build that reads the uploaded
+    table."""
     r = _list_input_head(batch)
     g = torch.Generator().manual_seed(9)
     pred = torch.randn(batch, n, 85, generator=g)
